@@ -1,0 +1,428 @@
+// Spatial batch normalisation: training forward, backward and inference.
+// Replaces cudnnBatchNormalizationForwardTraining / Backward / ForwardInference as called at
+// cuda/source/dopt/cuda/nnet/cudnn7.d:608-610, :632-634, :650-652, including the reference's
+// packed output layouts (core/source/dopt/core/ops/nnet.d:222-235).
+//
+// Three launches per op, all deterministic (no atomics):
+//   1. partial: block (channel, slice) accumulates shifted moments of its share of the channel
+//      (shift K = first element of the channel, so that E[(x-K)^2] - E[x-K]^2 does not cancel);
+//   2. finalize: one thread per channel folds the slices in float64, derives mean / 1/std and the
+//      small per-channel outputs, and writes a per-channel coefficient table;
+//   3. apply: a flat 128-bit streaming pass over the tensor using the table.
+#include "common.h"
+
+namespace {
+
+using namespace dopt;
+
+constexpr int kBlock = 256;
+constexpr int kUnroll = 4;
+constexpr int kMaxSlices = 64;
+
+struct Coef {  // one per channel, 16 bytes
+    float mean;  // batch (or running) mean
+    float a;     // scale * rstd
+    float b;     // bias
+    float d;     // train/infer: rstd (informational)
+};
+struct CoefG {   // grad: a = scale * rstd, b = dbias / m, d = dscale / m
+    float mean, rstd, a, b, d;
+    float pad[3];
+};
+
+__device__ inline float wave_sum(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+    return v;
+}
+
+// Sums four per-thread values over the block; results valid in thread 0.
+__device__ inline void block_sum(float (&v)[4], float (*part)[kBlock / 64])
+{
+    constexpr int kN = 4;
+#pragma unroll
+    for (int k = 0; k < kN; k++) {
+        v[k] = wave_sum(v[k]);
+        if ((threadIdx.x & 63) == 0) part[k][threadIdx.x >> 6] = v[k];
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int k = 0; k < kN; k++) {
+            float r = 0.0f;
+#pragma unroll
+            for (int w = 0; w < kBlock / 64; w++) r += part[k][w];
+            v[k] = r;
+        }
+    }
+}
+
+// Moments of x (and of dy, dy*(x-K) when kGrad) for block (c, s): images n = s, s+S, ...
+// kFlat: for small `inner` the block walks (n, i) pairs with a flat index instead of rows.
+template <bool kGrad, bool kFlat>
+__global__ __launch_bounds__(kBlock) void bn_partial_k(size_t N, size_t C, size_t inner, size_t S, const float *x,
+                                                        const float *dy, float *partial)
+{
+    __shared__ float part[4][kBlock / 64];
+    const size_t c = blockIdx.x % C, s = blockIdx.x / C;
+    const float K = x[c * inner];
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (kFlat) {
+        const size_t per = N * inner;
+        for (size_t j = threadIdx.x; j < per; j += kBlock) {
+            size_t n = j / inner, i = j % inner;
+            size_t e = (n * C + c) * inner + i;
+            float v = x[e] - K;
+            acc[0] += v;
+            acc[1] += v * v;
+            if (kGrad) {
+                float g = dy[e];
+                acc[2] += g;
+                acc[3] += g * v;
+            }
+        }
+    } else {
+        // inner % 4 == 0 and 16-byte aligned rows (checked on the host)
+        const size_t inner4 = inner >> 2;
+        for (size_t n = s; n < N; n += S) {
+            const float4 *row = (const float4 *)(x + (n * C + c) * inner);
+            const float4 *grow = (const float4 *)(dy + (n * C + c) * inner);
+            for (size_t i = threadIdx.x; i < inner4; i += kBlock) {
+                float4 q = row[i];
+                float v0 = q.x - K, v1 = q.y - K, v2 = q.z - K, v3 = q.w - K;
+                acc[0] += (v0 + v1) + (v2 + v3);
+                acc[1] += (v0 * v0 + v1 * v1) + (v2 * v2 + v3 * v3);
+                if (kGrad) {
+                    float4 g = grow[i];
+                    acc[2] += (g.x + g.y) + (g.z + g.w);
+                    acc[3] += (g.x * v0 + g.y * v1) + (g.z * v2 + g.w * v3);
+                }
+            }
+        }
+    }
+    block_sum(acc, part);
+    if (threadIdx.x == 0) {
+        float *p = partial + (c * S + s) * 4;
+        p[0] = acc[0];
+        p[1] = acc[1];
+        if (kGrad) {
+            p[2] = acc[2];
+            p[3] = acc[3];
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void bn_train_finalize_k(size_t N, size_t C, size_t inner, size_t S,
+                                                               double factor, double eps, const float *x,
+                                                               const float *partial, const float *scale,
+                                                               const float *bias, const float *run_mean,
+                                                               const float *run_var, Coef *coef, float *new_mean,
+                                                               float *new_var)
+{
+    size_t c = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (c >= C) return;
+    double m = (double)N * (double)inner;
+    double s1 = 0.0, s2 = 0.0;
+    for (size_t s = 0; s < S; s++) {
+        s1 += (double)partial[(c * S + s) * 4 + 0];
+        s2 += (double)partial[(c * S + s) * 4 + 1];
+    }
+    double K = (double)x[c * inner];
+    double d1 = s1 / m;
+    double mean = K + d1;
+    double var = s2 / m - d1 * d1;  // biased
+    if (var < 0.0) var = 0.0;
+    double rstd = 1.0 / sqrt(var + eps);
+    Coef k;
+    k.mean = (float)mean;
+    k.a = (float)((double)scale[c] * rstd);
+    k.b = bias[c];
+    k.d = (float)rstd;
+    coef[c] = k;
+    double unbiased = m > 1.0 ? var * m / (m - 1.0) : var;
+    new_mean[c] = (float)((1.0 - factor) * (double)run_mean[c] + factor * mean);
+    new_var[c] = (float)((1.0 - factor) * (double)run_var[c] + factor * unbiased);
+}
+
+__global__ __launch_bounds__(kBlock) void bn_infer_prepare_k(size_t C, double eps, const float *scale,
+                                                              const float *bias, const float *mean, const float *var,
+                                                              Coef *coef)
+{
+    size_t c = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (c >= C) return;
+    double rstd = 1.0 / sqrt((double)var[c] + eps);
+    Coef k;
+    k.mean = mean[c];
+    k.a = (float)((double)scale[c] * rstd);
+    k.b = bias[c];
+    k.d = (float)rstd;
+    coef[c] = k;
+}
+
+__global__ __launch_bounds__(kBlock) void bn_grad_finalize_k(size_t N, size_t C, size_t inner, size_t S, double eps,
+                                                              const float *x, const float *partial,
+                                                              const float *scale, CoefG *coef, float *dscale,
+                                                              float *dbias)
+{
+    size_t c = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (c >= C) return;
+    double m = (double)N * (double)inner;
+    double s1 = 0.0, s2 = 0.0, g1 = 0.0, g2 = 0.0;
+    for (size_t s = 0; s < S; s++) {
+        const float *p = partial + (c * S + s) * 4;
+        s1 += (double)p[0];
+        s2 += (double)p[1];
+        g1 += (double)p[2];
+        g2 += (double)p[3];
+    }
+    double K = (double)x[c * inner];
+    double d1 = s1 / m;
+    double mean = K + d1;
+    double var = s2 / m - d1 * d1;
+    if (var < 0.0) var = 0.0;
+    double rstd = 1.0 / sqrt(var + eps);
+    double db = g1;                          // sum dy
+    double ds = rstd * (g2 - d1 * g1);       // sum dy * xhat,  xhat = (x - mean) * rstd
+    CoefG k;
+    k.mean = (float)mean;
+    k.rstd = (float)rstd;
+    k.a = (float)((double)scale[c] * rstd);
+    k.b = (float)(db / m);
+    k.d = (float)(ds / m);
+    k.pad[0] = k.pad[1] = k.pad[2] = 0.0f;
+    coef[c] = k;
+    dscale[c] = (float)ds;
+    dbias[c] = (float)db;
+}
+
+// y = a * (x - mean) + b
+template <typename IdxT, bool kVec>
+__global__ __launch_bounds__(kBlock) void bn_apply_k(IdxT total, IdxT C, IdxT inner, const float *x, const Coef *coef,
+                                                      float *y)
+{
+    if (kVec) {
+        const IdxT n4 = total >> 2, inner4 = inner >> 2;
+        const float4 *x4 = (const float4 *)x;
+        float4 *y4 = (float4 *)y;
+        for (IdxT base = (IdxT)blockIdx.x * (kBlock * kUnroll); base < n4;
+             base += (IdxT)gridDim.x * (kBlock * kUnroll)) {
+            float4 v[kUnroll];
+            Coef k[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+                IdxT i = base + (IdxT)u * kBlock + threadIdx.x;
+                if (i < n4) {
+                    v[u] = x4[i];
+                    k[u] = coef[(i / inner4) % C];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+                IdxT i = base + (IdxT)u * kBlock + threadIdx.x;
+                if (i < n4) {
+                    float4 r;
+                    r.x = k[u].a * (v[u].x - k[u].mean) + k[u].b;
+                    r.y = k[u].a * (v[u].y - k[u].mean) + k[u].b;
+                    r.z = k[u].a * (v[u].z - k[u].mean) + k[u].b;
+                    r.w = k[u].a * (v[u].w - k[u].mean) + k[u].b;
+                    y4[i] = r;
+                }
+            }
+        }
+    } else {
+        for (IdxT i = (IdxT)blockIdx.x * kBlock + threadIdx.x; i < total; i += (IdxT)gridDim.x * kBlock) {
+            Coef k = coef[(i / inner) % C];
+            y[i] = k.a * (x[i] - k.mean) + k.b;
+        }
+    }
+}
+
+// dx = a * (dy - b - xhat * d),  xhat = (x - mean) * rstd
+__device__ inline float bn_dx(const CoefG &k, float dy, float x)
+{
+    float xhat = (x - k.mean) * k.rstd;
+    return k.a * ((dy - k.b) - xhat * k.d);
+}
+
+template <typename IdxT, bool kVec>
+__global__ __launch_bounds__(kBlock) void bn_grad_apply_k(IdxT total, IdxT C, IdxT inner, const float *dy,
+                                                           const float *x, const CoefG *coef, float *dx)
+{
+    if (kVec) {
+        const IdxT n4 = total >> 2, inner4 = inner >> 2;
+        const float4 *x4 = (const float4 *)x;
+        const float4 *g4 = (const float4 *)dy;
+        float4 *o4 = (float4 *)dx;
+        for (IdxT base = (IdxT)blockIdx.x * (kBlock * kUnroll); base < n4;
+             base += (IdxT)gridDim.x * (kBlock * kUnroll)) {
+            float4 v[kUnroll], g[kUnroll];
+            IdxT ch[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+                IdxT i = base + (IdxT)u * kBlock + threadIdx.x;
+                if (i < n4) {
+                    v[u] = x4[i];
+                    g[u] = g4[i];
+                    ch[u] = (i / inner4) % C;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+                IdxT i = base + (IdxT)u * kBlock + threadIdx.x;
+                if (i < n4) {
+                    CoefG k = coef[ch[u]];
+                    o4[i] = make_float4(bn_dx(k, g[u].x, v[u].x), bn_dx(k, g[u].y, v[u].y), bn_dx(k, g[u].z, v[u].z),
+                                        bn_dx(k, g[u].w, v[u].w));
+                }
+            }
+        }
+    } else {
+        for (IdxT i = (IdxT)blockIdx.x * kBlock + threadIdx.x; i < total; i += (IdxT)gridDim.x * kBlock) {
+            CoefG k = coef[(i / inner) % C];
+            dx[i] = bn_dx(k, dy[i], x[i]);
+        }
+    }
+}
+
+size_t pick_slices(size_t N, size_t C)
+{
+    size_t S = ceil_div((size_t)num_cus() * 8, C);
+    if (S > N) S = N;
+    if (S > kMaxSlices) S = kMaxSlices;
+    return S < 1 ? 1 : S;
+}
+
+unsigned apply_grid(size_t total, bool vec)
+{
+    size_t blocks = vec ? ceil_div(total / 4, (size_t)kBlock * kUnroll) : ceil_div(total, (size_t)kBlock);
+    size_t cap = (size_t)num_cus() * 8;
+    return (unsigned)(blocks < 1 ? 1 : (blocks > cap ? cap : blocks));
+}
+
+template <bool kGrad>
+int launch_partial(size_t N, size_t C, size_t inner, const float *x, const float *dy, float *partial, size_t *S_out)
+{
+    bool rows = inner >= 256 && (inner & 3) == 0 && aligned16(x) && (!kGrad || aligned16(dy));
+    size_t S = rows ? pick_slices(N, C) : 1;
+    *S_out = S;
+    if (rows)
+        hipLaunchKernelGGL((bn_partial_k<kGrad, false>), dim3((unsigned)(C * S)), dim3(kBlock), 0, stream(), N, C, inner,
+                           S, x, dy, partial);
+    else
+        hipLaunchKernelGGL((bn_partial_k<kGrad, true>), dim3((unsigned)C), dim3(kBlock), 0, stream(), N, C, inner, S, x,
+                           dy, partial);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+int launch_apply(size_t total, size_t C, size_t inner, const float *x, const Coef *coef, float *y)
+{
+    bool vec = (inner & 3) == 0 && aligned16(x) && aligned16(y);
+    unsigned grid = apply_grid(total, vec);
+    bool small = total < 0x7fffffffull;
+    if (small) {
+        if (vec)
+            hipLaunchKernelGGL((bn_apply_k<unsigned, true>), dim3(grid), dim3(kBlock), 0, stream(), (unsigned)total,
+                               (unsigned)C, (unsigned)inner, x, coef, y);
+        else
+            hipLaunchKernelGGL((bn_apply_k<unsigned, false>), dim3(grid), dim3(kBlock), 0, stream(), (unsigned)total,
+                               (unsigned)C, (unsigned)inner, x, coef, y);
+    } else {
+        if (vec)
+            hipLaunchKernelGGL((bn_apply_k<size_t, true>), dim3(grid), dim3(kBlock), 0, stream(), total, C, inner, x,
+                               coef, y);
+        else
+            hipLaunchKernelGGL((bn_apply_k<size_t, false>), dim3(grid), dim3(kBlock), 0, stream(), total, C, inner, x,
+                               coef, y);
+    }
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int dopt_hip_bn_train(size_t N, size_t C, size_t inner, double momentum, const float *x, const float *scale,
+                      const float *bias, const float *run_mean, const float *run_var, float *packed)
+{
+    size_t total = N * C * inner;
+    DOPT_REQUIRE(total > 0, "dopt_hip_bn_train: empty input");
+    DOPT_REQUIRE(x && scale && bias && run_mean && run_var && packed, "dopt_hip_bn_train: null argument");
+    DOPT_REQUIRE(C <= 0x7fffffffu / kMaxSlices, "dopt_hip_bn_train: too many channels");
+    DOPT_ENSURE_INIT();
+    // workspace: [partials C*S*4 floats | coefficient table C * 16 bytes]
+    size_t part_bytes = C * kMaxSlices * 4 * sizeof(float);
+    char *ws = (char *)workspace(part_bytes + C * sizeof(Coef));
+    if (!ws) return DOPT_HIP_ERR_OOM;
+    float *partial = (float *)ws;
+    Coef *coef = (Coef *)(ws + part_bytes);
+    size_t S;
+    if (int rc = launch_partial<false>(N, C, inner, x, nullptr, partial, &S)) return rc;
+    double factor = 1.0 - momentum;    // cudnn7.d:592
+    double eps = (double)1e-5f;        // cudnn7.d:610
+    hipLaunchKernelGGL(bn_train_finalize_k, dim3((unsigned)ceil_div(C, (size_t)kBlock)), dim3(kBlock), 0, stream(), N,
+                       C, inner, S, factor, eps, x, partial, scale, bias, run_mean, run_var, coef, packed + total,
+                       packed + total + C);
+    DOPT_LAUNCH_CHECK();
+    return launch_apply(total, C, inner, x, coef, packed);
+}
+
+int dopt_hip_bn_grad(size_t N, size_t C, size_t inner, const float *dy, const float *x, const float *scale,
+                     float *packed)
+{
+    size_t total = N * C * inner;
+    DOPT_REQUIRE(total > 0, "dopt_hip_bn_grad: empty input");
+    DOPT_REQUIRE(dy && x && scale && packed, "dopt_hip_bn_grad: null argument");
+    DOPT_REQUIRE(C <= 0x7fffffffu / kMaxSlices, "dopt_hip_bn_grad: too many channels");
+    DOPT_ENSURE_INIT();
+    size_t part_bytes = C * kMaxSlices * 4 * sizeof(float);
+    char *ws = (char *)workspace(part_bytes + C * sizeof(CoefG));
+    if (!ws) return DOPT_HIP_ERR_OOM;
+    float *partial = (float *)ws;
+    CoefG *coef = (CoefG *)(ws + part_bytes);
+    size_t S;
+    if (int rc = launch_partial<true>(N, C, inner, x, dy, partial, &S)) return rc;
+    double eps = (double)1e-5f;  // cudnn7.d:634
+    hipLaunchKernelGGL(bn_grad_finalize_k, dim3((unsigned)ceil_div(C, (size_t)kBlock)), dim3(kBlock), 0, stream(), N, C,
+                       inner, S, eps, x, partial, scale, coef, packed + total, packed + total + C);
+    DOPT_LAUNCH_CHECK();
+    bool vec = (inner & 3) == 0 && aligned16(x) && aligned16(dy) && aligned16(packed);
+    unsigned grid = apply_grid(total, vec);
+    bool small = total < 0x7fffffffull;
+    if (small) {
+        if (vec)
+            hipLaunchKernelGGL((bn_grad_apply_k<unsigned, true>), dim3(grid), dim3(kBlock), 0, stream(), (unsigned)total,
+                               (unsigned)C, (unsigned)inner, dy, x, coef, packed);
+        else
+            hipLaunchKernelGGL((bn_grad_apply_k<unsigned, false>), dim3(grid), dim3(kBlock), 0, stream(),
+                               (unsigned)total, (unsigned)C, (unsigned)inner, dy, x, coef, packed);
+    } else {
+        if (vec)
+            hipLaunchKernelGGL((bn_grad_apply_k<size_t, true>), dim3(grid), dim3(kBlock), 0, stream(), total, C, inner,
+                               dy, x, coef, packed);
+        else
+            hipLaunchKernelGGL((bn_grad_apply_k<size_t, false>), dim3(grid), dim3(kBlock), 0, stream(), total, C, inner,
+                               dy, x, coef, packed);
+    }
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_bn_infer(size_t N, size_t C, size_t inner, const float *x, const float *scale, const float *bias,
+                      const float *mean, const float *var, float *y)
+{
+    size_t total = N * C * inner;
+    if (total == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(x && scale && bias && mean && var && y, "dopt_hip_bn_infer: null argument");
+    DOPT_ENSURE_INIT();
+    Coef *coef = (Coef *)workspace(C * sizeof(Coef));
+    if (!coef) return DOPT_HIP_ERR_OOM;
+    hipLaunchKernelGGL(bn_infer_prepare_k, dim3((unsigned)ceil_div(C, (size_t)kBlock)), dim3(kBlock), 0, stream(), C,
+                       1e-5 /* cudnn7.d:652 */, scale, bias, mean, var, coef);
+    DOPT_LAUNCH_CHECK();
+    return launch_apply(total, C, inner, x, coef, y);
+}
+
+}  // extern "C"

@@ -1,0 +1,66 @@
+// Internal helpers shared by every translation unit of libdopthip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+
+#include "../../include/dopt_hip.h"
+
+namespace dopt {
+
+// Records the message returned by dopt_hip_last_error() and hands back `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+void clear_error();
+
+// The library stream (created by dopt_hip_init; lazily initialises device 0 otherwise).
+hipStream_t stream();
+bool ensure_init();
+
+// Process-wide scratch memory, grown on demand (the analogue of the single conv workspace at
+// cuda/nnet/cudnn7.d:111).  Valid until the next call that asks for more; all users enqueue on
+// the one library stream, so consecutive users never overlap.
+void *workspace(size_t bytes);
+
+// Number of compute units of the active device (256 on MI355X); used to size grids.
+int num_cus();
+
+inline size_t ceil_div(size_t a, size_t b) { return (a + b - 1) / b; }
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// hipRTC: compile `source` (once per distinct `key`) and return the named kernel.
+int rtc_get(const std::string &key, const std::string &source, const char *kernel_name, hipFunction_t *fn);
+int rtc_compile_only(const std::string &source, const char *arch, std::string *log);
+int rtc_launch(hipFunction_t fn, unsigned grid, unsigned block, void **args);
+
+}  // namespace dopt
+
+#define DOPT_HIP_CHECK(expr)                                                                       \
+    do {                                                                                           \
+        hipError_t e_ = (expr);                                                                    \
+        if (e_ != hipSuccess)                                                                      \
+            return ::dopt::fail(DOPT_HIP_ERR_RUNTIME, "%s:%d: %s failed: %s", __FILE__, __LINE__,  \
+                                #expr, hipGetErrorString(e_));                                     \
+    } while (0)
+
+#define DOPT_LAUNCH_CHECK()                                                                        \
+    do {                                                                                           \
+        hipError_t e_ = hipGetLastError();                                                         \
+        if (e_ != hipSuccess)                                                                      \
+            return ::dopt::fail(DOPT_HIP_ERR_RUNTIME, "%s:%d: kernel launch failed: %s", __FILE__, \
+                                __LINE__, hipGetErrorString(e_));                                  \
+    } while (0)
+
+#define DOPT_REQUIRE(cond, ...)                                                                    \
+    do {                                                                                           \
+        if (!(cond)) return ::dopt::fail(DOPT_HIP_ERR_INVALID, __VA_ARGS__);                       \
+    } while (0)
+
+#define DOPT_ENSURE_INIT()                                                                         \
+    do {                                                                                           \
+        if (!::dopt::ensure_init()) return DOPT_HIP_ERR_RUNTIME;                                   \
+    } while (0)

@@ -1,0 +1,267 @@
+// Layout ops on 4-byte elements: slice, pad, repeat, rank-2 transpose.
+// Replaces cuda/source/dopt/cuda/basic.d (host recursion issuing one cuMemcpy per innermost row
+// for slice/pad, a per-axis byte-granular NVRTC kernel with temporaries for repeat, cublasSgeam
+// for transpose) with one bandwidth-bound kernel per op.
+#include "common.h"
+
+namespace {
+
+using namespace dopt;
+
+constexpr int kMaxRank = 8;
+constexpr int kBlock = 256;
+
+struct NdDesc {
+    int rank;
+    size_t out_shape[kMaxRank];
+    size_t in_shape[kMaxRank];
+    size_t in_stride[kMaxRank];
+    size_t offset[kMaxRank];  // slice: start, pad: before
+};
+
+unsigned grid_for(size_t n)
+{
+    size_t blocks = ceil_div(n, (size_t)kBlock);
+    size_t cap = (size_t)num_cus() * 16;
+    return (unsigned)(blocks < 1 ? 1 : (blocks > cap ? cap : blocks));
+}
+
+// out[idx] = in[(coord + start) . in_stride]
+__global__ __launch_bounds__(kBlock) void slice_nd(NdDesc d, size_t total, const uint32_t *in, uint32_t *out)
+{
+    for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < total; idx += (size_t)gridDim.x * kBlock) {
+        size_t rem = idx, src = 0;
+#pragma unroll
+        for (int i = kMaxRank - 1; i >= 0; i--) {
+            if (i < d.rank) {
+                size_t c = rem % d.out_shape[i];
+                rem /= d.out_shape[i];
+                src += (c + d.offset[i]) * d.in_stride[i];
+            }
+        }
+        out[idx] = in[src];
+    }
+}
+
+// out[idx] = coord - before inside the input ? in[...] : 0   (every output element is written)
+__global__ __launch_bounds__(kBlock) void pad_nd(NdDesc d, size_t total, const uint32_t *in, uint32_t *out)
+{
+    for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < total; idx += (size_t)gridDim.x * kBlock) {
+        size_t rem = idx, src = 0;
+        bool inside = true;
+#pragma unroll
+        for (int i = kMaxRank - 1; i >= 0; i--) {
+            if (i < d.rank) {
+                size_t c = rem % d.out_shape[i];
+                rem /= d.out_shape[i];
+                size_t ic = c - d.offset[i];  // wraps to a huge value when c < before
+                inside = inside && (ic < d.in_shape[i]);
+                src += ic * d.in_stride[i];
+            }
+        }
+        out[idx] = inside ? in[src] : 0u;
+    }
+}
+
+// out[coord] = in[coord mod in_shape]
+__global__ __launch_bounds__(kBlock) void repeat_nd(NdDesc d, size_t total, const uint32_t *in, uint32_t *out)
+{
+    for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < total; idx += (size_t)gridDim.x * kBlock) {
+        size_t rem = idx, src = 0;
+#pragma unroll
+        for (int i = kMaxRank - 1; i >= 0; i--) {
+            if (i < d.rank) {
+                size_t c = rem % d.out_shape[i];
+                rem /= d.out_shape[i];
+                src += (c % d.in_shape[i]) * d.in_stride[i];
+            }
+        }
+        out[idx] = in[src];
+    }
+}
+
+// Contiguous copy, 128-bit when both ends are 16-byte aligned.
+__global__ __launch_bounds__(kBlock) void copy_vec4(size_t n4, const uint4 *in, uint4 *out)
+{
+    for (size_t base = (size_t)blockIdx.x * (kBlock * 4); base < n4; base += (size_t)gridDim.x * (kBlock * 4)) {
+        uint4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            size_t i = base + (size_t)u * kBlock + threadIdx.x;
+            if (i < n4) v[u] = in[i];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            size_t i = base + (size_t)u * kBlock + threadIdx.x;
+            if (i < n4) out[i] = v[u];
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void copy_scalar(size_t n, const uint32_t *in, uint32_t *out)
+{
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) out[i] = in[i];
+}
+
+// [rows, cols] -> [cols, rows] through a 64x64 LDS tile (padded to 65 to stay conflict-free).
+__global__ __launch_bounds__(kBlock) void transpose_tile(size_t rows, size_t cols, const uint32_t *in, uint32_t *out)
+{
+    __shared__ uint32_t tile[64][65];
+    const size_t tiles_x = (cols + 63) / 64;
+    const size_t bx = blockIdx.x % tiles_x, by = blockIdx.x / tiles_x;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 x 4
+    const size_t c = bx * 64 + tx;
+#pragma unroll
+    for (int k = 0; k < 16; k++) {
+        size_t r = by * 64 + ty + 4 * k;
+        if (r < rows && c < cols) tile[ty + 4 * k][tx] = in[r * cols + c];
+    }
+    __syncthreads();
+    const size_t orow_base = bx * 64, ocol = by * 64 + tx;  // out is [cols, rows]
+#pragma unroll
+    for (int k = 0; k < 16; k++) {
+        size_t orow = orow_base + ty + 4 * k;
+        if (orow < cols && ocol < rows) out[orow * rows + ocol] = tile[tx][ty + 4 * k];
+    }
+}
+
+int copy_contiguous(const uint32_t *in, uint32_t *out, size_t n)
+{
+    if (n == 0) return DOPT_HIP_OK;
+    if (aligned16(in) && aligned16(out) && n >= 4) {
+        size_t n4 = n / 4;
+        size_t blocks = ceil_div(n4, (size_t)kBlock * 4);
+        size_t cap = (size_t)num_cus() * 8;
+        hipLaunchKernelGGL(copy_vec4, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(kBlock), 0, stream(), n4,
+                           (const uint4 *)in, (uint4 *)out);
+        DOPT_LAUNCH_CHECK();
+        size_t tail = n - n4 * 4;
+        if (tail) {
+            hipLaunchKernelGGL(copy_scalar, dim3(1), dim3(kBlock), 0, stream(), tail, in + n4 * 4, out + n4 * 4);
+            DOPT_LAUNCH_CHECK();
+        }
+        return DOPT_HIP_OK;
+    }
+    hipLaunchKernelGGL(copy_scalar, dim3(grid_for(n)), dim3(kBlock), 0, stream(), n, in, out);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+size_t volume(const size_t *shape, int rank)
+{
+    size_t v = 1;
+    for (int i = 0; i < rank; i++) v *= shape[i];
+    return v;
+}
+
+void fill_strides(NdDesc &d)
+{
+    size_t s = 1;
+    for (int i = d.rank - 1; i >= 0; i--) {
+        d.in_stride[i] = s;
+        s *= d.in_shape[i];
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int dopt_hip_slice(int rank, const size_t *in_shape, const size_t *out_shape, const size_t *start,
+                   const void *in, void *out)
+{
+    DOPT_REQUIRE(rank >= 0 && rank <= kMaxRank, "dopt_hip_slice: rank %d not supported (max %d)", rank, kMaxRank);
+    DOPT_REQUIRE(in && out && (rank == 0 || (in_shape && out_shape && start)), "dopt_hip_slice: null argument");
+    for (int i = 0; i < rank; i++)
+        DOPT_REQUIRE(start[i] + out_shape[i] <= in_shape[i] && out_shape[i] > 0,
+                     "dopt_hip_slice: axis %d: [%zu, %zu) outside extent %zu", i, start[i], start[i] + out_shape[i],
+                     in_shape[i]);
+    DOPT_ENSURE_INIT();
+    size_t total = volume(out_shape, rank);
+    // A slice that only cuts the outermost axis (BN's rank-1 unpacking, row blocks) is one
+    // contiguous run.
+    bool contiguous = true;
+    for (int i = 1; i < rank; i++) contiguous = contiguous && start[i] == 0 && out_shape[i] == in_shape[i];
+    if (contiguous) {
+        size_t inner = rank > 0 ? volume(in_shape + 1, rank - 1) : 1;
+        size_t off = rank > 0 ? start[0] * inner : 0;
+        return copy_contiguous((const uint32_t *)in + off, (uint32_t *)out, total);
+    }
+    NdDesc d{};
+    d.rank = rank;
+    for (int i = 0; i < rank; i++) {
+        d.out_shape[i] = out_shape[i];
+        d.in_shape[i] = in_shape[i];
+        d.offset[i] = start[i];
+    }
+    fill_strides(d);
+    hipLaunchKernelGGL(slice_nd, dim3(grid_for(total)), dim3(kBlock), 0, stream(), d, total, (const uint32_t *)in,
+                       (uint32_t *)out);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_pad(int rank, const size_t *in_shape, const size_t *out_shape, const size_t *before,
+                 const void *in, void *out)
+{
+    DOPT_REQUIRE(rank >= 0 && rank <= kMaxRank, "dopt_hip_pad: rank %d not supported (max %d)", rank, kMaxRank);
+    DOPT_REQUIRE(in && out && (rank == 0 || (in_shape && out_shape && before)), "dopt_hip_pad: null argument");
+    for (int i = 0; i < rank; i++)
+        DOPT_REQUIRE(before[i] + in_shape[i] <= out_shape[i], "dopt_hip_pad: axis %d: input does not fit the output", i);
+    DOPT_ENSURE_INIT();
+    size_t total = volume(out_shape, rank);
+    if (total == 0) return DOPT_HIP_OK;
+    if (rank == 0) return copy_contiguous((const uint32_t *)in, (uint32_t *)out, 1);
+    NdDesc d{};
+    d.rank = rank;
+    for (int i = 0; i < rank; i++) {
+        d.out_shape[i] = out_shape[i];
+        d.in_shape[i] = in_shape[i];
+        d.offset[i] = before[i];
+    }
+    fill_strides(d);
+    hipLaunchKernelGGL(pad_nd, dim3(grid_for(total)), dim3(kBlock), 0, stream(), d, total, (const uint32_t *)in,
+                       (uint32_t *)out);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_repeat(int rank, const size_t *in_shape, const size_t *reps, const void *in, void *out)
+{
+    DOPT_REQUIRE(rank >= 0 && rank <= kMaxRank, "dopt_hip_repeat: rank %d not supported (max %d)", rank, kMaxRank);
+    DOPT_REQUIRE(in && out && (rank == 0 || (in_shape && reps)), "dopt_hip_repeat: null argument");
+    DOPT_ENSURE_INIT();
+    NdDesc d{};
+    d.rank = rank;
+    bool identity = true;
+    for (int i = 0; i < rank; i++) {
+        DOPT_REQUIRE(reps[i] > 0, "dopt_hip_repeat: repetitions must be positive");
+        d.in_shape[i] = in_shape[i];
+        d.out_shape[i] = in_shape[i] * reps[i];
+        identity = identity && reps[i] == 1;
+    }
+    size_t total = volume(d.out_shape, rank);
+    if (total == 0) return DOPT_HIP_OK;
+    if (identity) return copy_contiguous((const uint32_t *)in, (uint32_t *)out, total);  // cuda/basic.d:168-172
+    fill_strides(d);
+    hipLaunchKernelGGL(repeat_nd, dim3(grid_for(total)), dim3(kBlock), 0, stream(), d, total, (const uint32_t *)in,
+                       (uint32_t *)out);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_transpose2d(size_t rows, size_t cols, const void *in, void *out)
+{
+    if (rows * cols == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(in && out, "dopt_hip_transpose2d: null argument");
+    DOPT_ENSURE_INIT();
+    if (rows == 1 || cols == 1) return copy_contiguous((const uint32_t *)in, (uint32_t *)out, rows * cols);
+    size_t tiles = ceil_div(cols, 64) * ceil_div(rows, 64);
+    DOPT_REQUIRE(tiles <= 0x7fffffffu, "dopt_hip_transpose2d: matrix too large");
+    hipLaunchKernelGGL(transpose_tile, dim3((unsigned)tiles), dim3(kBlock), 0, stream(), rows, cols,
+                       (const uint32_t *)in, (uint32_t *)out);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,456 @@
+// Bandwidth-bound NN ops (fp32, NCHW): relu, addBias, maxpool, softmax and their gradients.
+// Each replaces one cuDNN call of cuda/source/dopt/cuda/nnet/cudnn7.d (cited per entry point in
+// include/dopt_hip.h) with a single streaming kernel: every input is read once and every
+// output written once, with 128-bit accesses wherever the shapes allow.
+#include <cfloat>
+
+#include "common.h"
+
+namespace {
+
+using namespace dopt;
+
+constexpr int kBlock = 256;
+constexpr int kUnroll = 4;
+
+unsigned stream_grid(size_t n4)
+{
+    size_t blocks = ceil_div(n4, (size_t)kBlock * kUnroll);
+    size_t cap = (size_t)num_cus() * 8;
+    return (unsigned)(blocks < 1 ? 1 : (blocks > cap ? cap : blocks));
+}
+
+unsigned flat_grid(size_t n)
+{
+    size_t blocks = ceil_div(n, (size_t)kBlock);
+    size_t cap = (size_t)num_cus() * 16;
+    return (unsigned)(blocks < 1 ? 1 : (blocks > cap ? cap : blocks));
+}
+
+// NaN propagates (CUDNN_PROPAGATE_NAN): NaN < 0 is false, so x passes through.
+__device__ inline float relu1(float x) { return x < 0.0f ? 0.0f : x; }
+__device__ inline float relu_grad1(float dy, float x) { return x > 0.0f ? dy : 0.0f; }
+
+// ---------------------------------------------------------------------------------- relu
+template <bool kVec>
+__global__ __launch_bounds__(kBlock) void relu_fwd_k(size_t n, const float *x, float *y)
+{
+    if (kVec) {
+        const size_t n4 = n >> 2;
+        const float4 *x4 = (const float4 *)x;
+        float4 *y4 = (float4 *)y;
+        for (size_t base = (size_t)blockIdx.x * (kBlock * kUnroll); base < n4;
+             base += (size_t)gridDim.x * (kBlock * kUnroll)) {
+            float4 v[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+                size_t i = base + (size_t)u * kBlock + threadIdx.x;
+                if (i < n4) v[u] = x4[i];
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+                size_t i = base + (size_t)u * kBlock + threadIdx.x;
+                if (i < n4) y4[i] = make_float4(relu1(v[u].x), relu1(v[u].y), relu1(v[u].z), relu1(v[u].w));
+            }
+        }
+        if (blockIdx.x == 0) {
+            size_t i = (n4 << 2) + threadIdx.x;
+            if (i < n) y[i] = relu1(x[i]);
+        }
+    } else {
+        for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock)
+            y[i] = relu1(x[i]);
+    }
+}
+
+template <bool kVec>
+__global__ __launch_bounds__(kBlock) void relu_bwd_k(size_t n, const float *dy, const float *x, float *dx)
+{
+    if (kVec) {
+        const size_t n4 = n >> 2;
+        const float4 *g4 = (const float4 *)dy;
+        const float4 *x4 = (const float4 *)x;
+        float4 *o4 = (float4 *)dx;
+        for (size_t base = (size_t)blockIdx.x * (kBlock * kUnroll); base < n4;
+             base += (size_t)gridDim.x * (kBlock * kUnroll)) {
+            float4 g[kUnroll], v[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+                size_t i = base + (size_t)u * kBlock + threadIdx.x;
+                if (i < n4) {
+                    g[u] = g4[i];
+                    v[u] = x4[i];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+                size_t i = base + (size_t)u * kBlock + threadIdx.x;
+                if (i < n4)
+                    o4[i] = make_float4(relu_grad1(g[u].x, v[u].x), relu_grad1(g[u].y, v[u].y),
+                                        relu_grad1(g[u].z, v[u].z), relu_grad1(g[u].w, v[u].w));
+            }
+        }
+        if (blockIdx.x == 0) {
+            size_t i = (n4 << 2) + threadIdx.x;
+            if (i < n) dx[i] = relu_grad1(dy[i], x[i]);
+        }
+    } else {
+        for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock)
+            dx[i] = relu_grad1(dy[i], x[i]);
+    }
+}
+
+// ---------------------------------------------------------------------------------- bias
+// y[n,c,i] = x[n,c,i] + b[c].  kVec needs inner % 4 == 0 so that a float4 stays inside one channel.
+template <bool kVec>
+__global__ __launch_bounds__(kBlock) void bias_fwd_k(size_t total, size_t C, size_t inner, const float *x,
+                                                      const float *b, float *y)
+{
+    if (kVec) {
+        const size_t n4 = total >> 2, inner4 = inner >> 2;
+        const float4 *x4 = (const float4 *)x;
+        float4 *y4 = (float4 *)y;
+        for (size_t base = (size_t)blockIdx.x * (kBlock * kUnroll); base < n4;
+             base += (size_t)gridDim.x * (kBlock * kUnroll)) {
+            float4 v[kUnroll];
+            float bb[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+                size_t i = base + (size_t)u * kBlock + threadIdx.x;
+                if (i < n4) {
+                    v[u] = x4[i];
+                    bb[u] = b[(i / inner4) % C];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+                size_t i = base + (size_t)u * kBlock + threadIdx.x;
+                if (i < n4) y4[i] = make_float4(v[u].x + bb[u], v[u].y + bb[u], v[u].z + bb[u], v[u].w + bb[u]);
+            }
+        }
+    } else {
+        for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (size_t)gridDim.x * kBlock)
+            y[i] = x[i] + b[(i / inner) % C];
+    }
+}
+
+__device__ inline float block_sum(float v, float *part)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float r = 0.0f;
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int w = 0; w < kBlock / 64; w++) r += part[w];
+    }
+    __syncthreads();
+    return r;  // valid in thread 0
+}
+
+// Stage 1 of db[c] = sum_{n,i} dy[n,c,i]: block (c, s) sums images n = s, s+S, ... of channel c.
+__global__ __launch_bounds__(kBlock) void bias_bwd_partial_k(size_t N, size_t C, size_t inner, size_t S,
+                                                              const float *dy, float *partial)
+{
+    __shared__ float part[kBlock / 64];
+    const size_t c = blockIdx.x % C, s = blockIdx.x / C;
+    float acc = 0.0f;
+    for (size_t n = s; n < N; n += S) {
+        const float *row = dy + (n * C + c) * inner;
+        for (size_t i = threadIdx.x; i < inner; i += kBlock) acc += row[i];
+    }
+    float r = block_sum(acc, part);
+    if (threadIdx.x == 0) partial[c * S + s] = r;
+}
+
+// Variant for small `inner` (dense layers, tiny feature maps): thread t walks (n, i) pairs of channel c.
+__global__ __launch_bounds__(kBlock) void bias_bwd_flat_k(size_t N, size_t C, size_t inner, const float *dy,
+                                                           float *db)
+{
+    __shared__ float part[kBlock / 64];
+    const size_t c = blockIdx.x;
+    const size_t per = N * inner;
+    float acc = 0.0f;
+    for (size_t j = threadIdx.x; j < per; j += kBlock) {
+        size_t n = j / inner, i = j % inner;
+        acc += dy[(n * C + c) * inner + i];
+    }
+    float r = block_sum(acc, part);
+    if (threadIdx.x == 0) db[c] = r;
+}
+
+// Stage 2: fixed-order sum of the S partials of each channel (deterministic, no atomics).
+__global__ __launch_bounds__(kBlock) void bias_bwd_final_k(size_t C, size_t S, const float *partial, float *db)
+{
+    size_t c = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (c >= C) return;
+    float acc = 0.0f;
+    for (size_t s = 0; s < S; s++) acc += partial[c * S + s];
+    db[c] = acc;
+}
+
+// ---------------------------------------------------------------------------------- maxpool
+// std.algorithm.max(acc, v) = acc < v ? v : acc, starting from -float.max (cpu/nnet.d:103-113).
+__device__ inline float dmax(float acc, float v) { return acc < v ? v : acc; }
+
+// 2x2 windows, W % 4 == 0, 16-byte aligned: one thread makes two adjacent outputs from two float4 rows.
+__global__ __launch_bounds__(kBlock) void maxpool2x2_fwd_k(size_t maps, size_t H, size_t W, const float *x, float *y)
+{
+    const size_t P = H >> 1, Q2 = W >> 2;  // output rows, output column PAIRS
+    const size_t total = maps * P * Q2;
+    for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < total; idx += (size_t)gridDim.x * kBlock) {
+        size_t q2 = idx % Q2, t = idx / Q2;
+        size_t p = t % P, m = t / P;
+        const float4 *r0 = (const float4 *)(x + (m * H + 2 * p) * W) + q2;
+        const float4 *r1 = (const float4 *)(x + (m * H + 2 * p + 1) * W) + q2;
+        float4 a = *r0, b = *r1;
+        float o0 = dmax(dmax(dmax(dmax(-FLT_MAX, a.x), a.y), b.x), b.y);
+        float o1 = dmax(dmax(dmax(dmax(-FLT_MAX, a.z), a.w), b.z), b.w);
+        ((float2 *)(y + (m * P + p) * (W >> 1)))[q2] = make_float2(o0, o1);
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void maxpool_fwd_k(size_t maps, size_t H, size_t W, size_t ph, size_t pw,
+                                                         const float *x, float *y)
+{
+    const size_t P = H / ph, Q = W / pw;
+    const size_t total = maps * P * Q;
+    for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < total; idx += (size_t)gridDim.x * kBlock) {
+        size_t q = idx % Q, t = idx / Q;
+        size_t p = t % P, m = t / P;
+        const float *img = x + m * H * W;
+        float acc = -FLT_MAX;
+        for (size_t j = 0; j < ph; j++)
+            for (size_t i = 0; i < pw; i++) acc = dmax(acc, img[(p * ph + j) * W + q * pw + i]);
+        y[idx] = acc;
+    }
+}
+
+// Gradient goes to the first maximum of the window in row-major order (strict '>' keeps the earlier one).
+__device__ inline void route2x2(float a, float b, float c, float d, float g, float &oa, float &ob, float &oc,
+                                float &od)
+{
+    int best = 0;
+    float bv = a;
+    if (b > bv) { bv = b; best = 1; }
+    if (c > bv) { bv = c; best = 2; }
+    if (d > bv) { bv = d; best = 3; }
+    oa = best == 0 ? g : 0.0f;
+    ob = best == 1 ? g : 0.0f;
+    oc = best == 2 ? g : 0.0f;
+    od = best == 3 ? g : 0.0f;
+}
+
+// 2x2, H even, W % 4 == 0, aligned: a thread owns two adjacent windows = a float4 of each of two rows.
+__global__ __launch_bounds__(kBlock) void maxpool2x2_bwd_k(size_t maps, size_t H, size_t W, const float *dy,
+                                                            const float *x, float *dx)
+{
+    const size_t P = H >> 1, Q2 = W >> 2;
+    const size_t total = maps * P * Q2;
+    for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < total; idx += (size_t)gridDim.x * kBlock) {
+        size_t q2 = idx % Q2, t = idx / Q2;
+        size_t p = t % P, m = t / P;
+        size_t row0 = (m * H + 2 * p) * W, row1 = row0 + W;
+        float4 a = ((const float4 *)(x + row0))[q2], b = ((const float4 *)(x + row1))[q2];
+        float2 g = ((const float2 *)(dy + (m * P + p) * (W >> 1)))[q2];
+        float4 oa, ob;
+        route2x2(a.x, a.y, b.x, b.y, g.x, oa.x, oa.y, ob.x, ob.y);
+        route2x2(a.z, a.w, b.z, b.w, g.y, oa.z, oa.w, ob.z, ob.w);
+        ((float4 *)(dx + row0))[q2] = oa;
+        ((float4 *)(dx + row1))[q2] = ob;
+    }
+}
+
+// General windows: one thread per INPUT element; rows/columns beyond the last full window get 0.
+__global__ __launch_bounds__(kBlock) void maxpool_bwd_k(size_t maps, size_t H, size_t W, size_t ph, size_t pw,
+                                                         const float *dy, const float *x, float *dx)
+{
+    const size_t P = H / ph, Q = W / pw;
+    const size_t total = maps * H * W;
+    for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < total; idx += (size_t)gridDim.x * kBlock) {
+        size_t w = idx % W, t = idx / W;
+        size_t h = t % H, m = t / H;
+        size_t p = h / ph, q = w / pw;
+        float out = 0.0f;
+        if (p < P && q < Q) {
+            const float *img = x + m * H * W;
+            size_t best = (p * ph) * W + q * pw;
+            float bv = img[best];
+            for (size_t j = 0; j < ph; j++)
+                for (size_t i = 0; i < pw; i++) {
+                    size_t e = (p * ph + j) * W + q * pw + i;
+                    float v = img[e];
+                    if (v > bv) { bv = v; best = e; }
+                }
+            if (best == h * W + w) out = dy[(m * P + p) * Q + q];
+        }
+        dx[idx] = out;
+    }
+}
+
+// ---------------------------------------------------------------------------------- softmax
+// One thread per (n, i) lane, channel loop in the order of cpu/nnet.d:129-166: max, exp and
+// running fp32 sum, divide.
+__global__ __launch_bounds__(kBlock) void softmax_fwd_k(size_t N, size_t C, size_t inner, const float *x, float *y)
+{
+    const size_t total = N * inner;
+    for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < total; idx += (size_t)gridDim.x * kBlock) {
+        size_t n = idx / inner, i = idx % inner;
+        const float *px = x + n * C * inner + i;
+        float *py = y + n * C * inner + i;
+        float m = -FLT_MAX;
+        for (size_t c = 0; c < C; c++) m = dmax(m, px[c * inner]);
+        float s = 0.0f;
+        for (size_t c = 0; c < C; c++) {
+            float pot = expf(px[c * inner] - m);
+            s += pot;
+            py[c * inner] = pot;
+        }
+        for (size_t c = 0; c < C; c++) py[c * inner] = py[c * inner] / s;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void softmax_bwd_k(size_t N, size_t C, size_t inner, const float *dy,
+                                                         const float *y, float *dx)
+{
+    const size_t total = N * inner;
+    for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < total; idx += (size_t)gridDim.x * kBlock) {
+        size_t n = idx / inner, i = idx % inner;
+        size_t base = n * C * inner + i;
+        float dot = 0.0f;
+        for (size_t c = 0; c < C; c++) dot += dy[base + c * inner] * y[base + c * inner];
+        for (size_t c = 0; c < C; c++) dx[base + c * inner] = y[base + c * inner] * (dy[base + c * inner] - dot);
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int dopt_hip_relu_fwd(size_t n, const float *x, float *y)
+{
+    if (n == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(x && y, "dopt_hip_relu_fwd: null argument");
+    DOPT_ENSURE_INIT();
+    if (aligned16(x) && aligned16(y))
+        hipLaunchKernelGGL(relu_fwd_k<true>, dim3(stream_grid(n / 4)), dim3(kBlock), 0, stream(), n, x, y);
+    else
+        hipLaunchKernelGGL(relu_fwd_k<false>, dim3(flat_grid(n)), dim3(kBlock), 0, stream(), n, x, y);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_relu_bwd(size_t n, const float *dy, const float *x, float *dx)
+{
+    if (n == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(dy && x && dx, "dopt_hip_relu_bwd: null argument");
+    DOPT_ENSURE_INIT();
+    if (aligned16(dy) && aligned16(x) && aligned16(dx))
+        hipLaunchKernelGGL(relu_bwd_k<true>, dim3(stream_grid(n / 4)), dim3(kBlock), 0, stream(), n, dy, x, dx);
+    else
+        hipLaunchKernelGGL(relu_bwd_k<false>, dim3(flat_grid(n)), dim3(kBlock), 0, stream(), n, dy, x, dx);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_bias_fwd(size_t N, size_t C, size_t inner, const float *x, const float *b, float *y)
+{
+    size_t total = N * C * inner;
+    if (total == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(x && b && y, "dopt_hip_bias_fwd: null argument");
+    DOPT_ENSURE_INIT();
+    if ((inner & 3) == 0 && aligned16(x) && aligned16(y))
+        hipLaunchKernelGGL(bias_fwd_k<true>, dim3(stream_grid(total / 4)), dim3(kBlock), 0, stream(), total, C, inner,
+                           x, b, y);
+    else
+        hipLaunchKernelGGL(bias_fwd_k<false>, dim3(flat_grid(total)), dim3(kBlock), 0, stream(), total, C, inner, x,
+                           b, y);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_bias_bwd(size_t N, size_t C, size_t inner, const float *dy, float *db)
+{
+    if (C == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(db && (N * inner == 0 || dy), "dopt_hip_bias_bwd: null argument");
+    DOPT_ENSURE_INIT();
+    if (N * inner == 0) return dopt_hip_memset(db, 0, C * sizeof(float));
+    DOPT_REQUIRE(C <= 0x7fffffffu / 64, "dopt_hip_bias_bwd: too many channels");
+    if (inner < 256) {
+        hipLaunchKernelGGL(bias_bwd_flat_k, dim3((unsigned)C), dim3(kBlock), 0, stream(), N, C, inner, dy, db);
+        DOPT_LAUNCH_CHECK();
+        return DOPT_HIP_OK;
+    }
+    // Enough (channel, image-slice) blocks to fill the machine; partials are then summed in a fixed order.
+    size_t S = ceil_div((size_t)num_cus() * 8, C);
+    if (S > N) S = N;
+    if (S > 64) S = 64;
+    if (S < 1) S = 1;
+    float *partial = (float *)workspace(C * S * sizeof(float));
+    if (!partial) return DOPT_HIP_ERR_OOM;
+    hipLaunchKernelGGL(bias_bwd_partial_k, dim3((unsigned)(C * S)), dim3(kBlock), 0, stream(), N, C, inner, S, dy,
+                       partial);
+    DOPT_LAUNCH_CHECK();
+    hipLaunchKernelGGL(bias_bwd_final_k, dim3((unsigned)ceil_div(C, (size_t)kBlock)), dim3(kBlock), 0, stream(), C, S,
+                       partial, db);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_maxpool_fwd(size_t N, size_t C, size_t H, size_t W, size_t ph, size_t pw, const float *x, float *y)
+{
+    DOPT_REQUIRE(ph > 0 && pw > 0, "dopt_hip_maxpool_fwd: pool dims must be positive");
+    size_t maps = N * C, P = H / ph, Q = W / pw;
+    if (maps * P * Q == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(x && y, "dopt_hip_maxpool_fwd: null argument");
+    DOPT_ENSURE_INIT();
+    if (ph == 2 && pw == 2 && (H & 1) == 0 && (W & 3) == 0 && aligned16(x) && aligned16(y))
+        hipLaunchKernelGGL(maxpool2x2_fwd_k, dim3(flat_grid(maps * P * (W / 4))), dim3(kBlock), 0, stream(), maps, H, W,
+                           x, y);
+    else
+        hipLaunchKernelGGL(maxpool_fwd_k, dim3(flat_grid(maps * P * Q)), dim3(kBlock), 0, stream(), maps, H, W, ph, pw,
+                           x, y);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_maxpool_bwd(size_t N, size_t C, size_t H, size_t W, size_t ph, size_t pw, const float *dy,
+                         const float *x, float *dx)
+{
+    DOPT_REQUIRE(ph > 0 && pw > 0, "dopt_hip_maxpool_bwd: pool dims must be positive");
+    size_t maps = N * C;
+    if (maps * H * W == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(x && dx && ((H / ph) * (W / pw) == 0 || dy), "dopt_hip_maxpool_bwd: null argument");
+    DOPT_ENSURE_INIT();
+    if (ph == 2 && pw == 2 && (H & 1) == 0 && (W & 3) == 0 && aligned16(x) && aligned16(dx) && aligned16(dy))
+        hipLaunchKernelGGL(maxpool2x2_bwd_k, dim3(flat_grid(maps * (H / 2) * (W / 4))), dim3(kBlock), 0, stream(), maps,
+                           H, W, dy, x, dx);
+    else
+        hipLaunchKernelGGL(maxpool_bwd_k, dim3(flat_grid(maps * H * W)), dim3(kBlock), 0, stream(), maps, H, W, ph, pw,
+                           dy, x, dx);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_softmax_fwd(size_t N, size_t C, size_t inner, const float *x, float *y)
+{
+    if (N * C * inner == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(x && y, "dopt_hip_softmax_fwd: null argument");
+    DOPT_ENSURE_INIT();
+    hipLaunchKernelGGL(softmax_fwd_k, dim3(flat_grid(N * inner)), dim3(kBlock), 0, stream(), N, C, inner, x, y);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_softmax_bwd(size_t N, size_t C, size_t inner, const float *dy, const float *y, float *dx)
+{
+    if (N * C * inner == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(dy && y && dx, "dopt_hip_softmax_bwd: null argument");
+    DOPT_ENSURE_INIT();
+    hipLaunchKernelGGL(softmax_bwd_k, dim3(flat_grid(N * inner)), dim3(kBlock), 0, stream(), N, C, inner, dy, y, dx);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,465 @@
+// Pointwise and reduction ops: gfx950 HIP source templates instantiated per (op, dtype) through
+// hipRTC.  Replaces the NVRTC string generator of cuda/source/dopt/cuda/math.d:129-205 (one
+// scalar element per thread, device sync after each launch) with 128-bit vector loads, four
+// independent loads in flight per lane and no host synchronisation.  Semantics follow the CPU
+// evaluator, cpu/source/dopt/cpu/math.d:312-437 (pointwise), :90-247 (sum / maxElement) and
+// :249-310 (argmin).
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "common.h"
+
+namespace {
+
+using namespace dopt;
+
+struct OpInfo {
+    const char *name;
+    int arity;
+    const char *expr_f32;
+    const char *expr_i32;
+};
+
+// `a`, `b` are the operands of type T.  Integer arithmetic wraps (D semantics); every integer
+// unary op except neg goes through float and truncates back (cpu/math.d:418).
+const OpInfo kOps[] = {
+    {"add", 2, "a + b", "(int)((unsigned)a + (unsigned)b)"},
+    {"sub", 2, "a - b", "(int)((unsigned)a - (unsigned)b)"},
+    {"mul", 2, "a * b", "(int)((unsigned)a * (unsigned)b)"},
+    {"div", 2, "a / b", "a / b"},
+    {"lt", 2, "(T)(a < b)", "(T)(a < b)"},
+    {"lte", 2, "(T)(a <= b)", "(T)(a <= b)"},
+    {"gt", 2, "(T)(a > b)", "(T)(a > b)"},
+    {"gte", 2, "(T)(a >= b)", "(T)(a >= b)"},
+    {"eq", 2, "(T)(a == b)", "(T)(a == b)"},
+    {"neq", 2, "(T)(a != b)", "(T)(a != b)"},
+    {"max", 2, "(a < b ? b : a)", "(a < b ? b : a)"},
+    {"min", 2, "(a < b ? a : b)", "(a < b ? a : b)"},
+    {"pow", 2, "powf(a, b)", "dopt_ipow(a, b)"},
+    {"atan2", 2, "atan2f(a, b)", "(int)atan2f((float)a, (float)b)"},
+    {"neg", 1, "-a", "(int)(0u - (unsigned)a)"},
+    {"abs", 1, "fabsf(a)", "(int)fabsf((float)a)"},
+    {"sgn", 1, "(T)((a > 0) - (a < 0))", "(int)(float)(((float)a > 0) - ((float)a < 0))"},
+    {"exp", 1, "expf(a)", "(int)expf((float)a)"},
+    {"log", 1, "logf(a)", "(int)logf((float)a)"},
+    {"sqrt", 1, "sqrtf(a)", "(int)sqrtf((float)a)"},
+    {"sin", 1, "sinf(a)", "(int)sinf((float)a)"},
+    {"cos", 1, "cosf(a)", "(int)cosf((float)a)"},
+    {"tan", 1, "tanf(a)", "(int)tanf((float)a)"},
+    {"asin", 1, "asinf(a)", "(int)asinf((float)a)"},
+    {"acos", 1, "acosf(a)", "(int)acosf((float)a)"},
+    {"atan", 1, "atanf(a)", "(int)atanf((float)a)"},
+    {"sinh", 1, "sinhf(a)", "(int)sinhf((float)a)"},
+    {"cosh", 1, "coshf(a)", "(int)coshf((float)a)"},
+    {"tanh", 1, "tanhf(a)", "(int)tanhf((float)a)"},
+    {"asinh", 1, "asinhf(a)", "(int)asinhf((float)a)"},
+    {"acosh", 1, "acoshf(a)", "(int)acoshf((float)a)"},
+    {"atanh", 1, "atanhf(a)", "(int)atanhf((float)a)"},
+};
+
+const OpInfo *find_op(const char *name)
+{
+    for (const OpInfo &o : kOps)
+        if (!strcmp(o.name, name)) return &o;
+    return nullptr;
+}
+
+const char *kPointwiseBody = R"SRC(
+typedef T T4 __attribute__((ext_vector_type(4)));
+#define UNROLL 4
+#define BLOCK 256
+
+// std.math.pow(int, int): exponentiation by squaring with wrapping multiplies.
+__device__ inline int dopt_ipow(int x, int n)
+{
+    if (n < 0) {
+        if (x == 1) return 1;
+        if (x == -1) return (n & 1) ? -1 : 1;
+        return 0;
+    }
+    unsigned p = 1u, v = (unsigned)x, m = (unsigned)n;
+    while (m) {
+        if (m & 1u) p *= v;
+        m >>= 1;
+        v *= v;
+    }
+    return (int)p;
+}
+
+__device__ inline T dopt_op(T a, T b) { return (T)(OPEXPR); }
+
+// 16-byte aligned operands: each lane keeps UNROLL independent 128-bit loads per operand in flight.
+extern "C" __global__ __launch_bounds__(BLOCK) void pw_vec(size_t n, const T *a, const T *b, T *o)
+{
+    const size_t n4 = n >> 2;
+    const T4 *a4 = (const T4 *)a;
+    const T4 *b4 = (const T4 *)b;
+    T4 *o4 = (T4 *)o;
+    for (size_t base = (size_t)blockIdx.x * (BLOCK * UNROLL); base < n4;
+         base += (size_t)gridDim.x * (BLOCK * UNROLL)) {
+        T4 x[UNROLL], y[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            size_t i = base + (size_t)u * BLOCK + threadIdx.x;
+            if (i < n4) {
+                x[u] = a4[i];
+#if ARITY == 2
+                y[u] = b4[i];
+#else
+                y[u] = x[u];
+#endif
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            size_t i = base + (size_t)u * BLOCK + threadIdx.x;
+            if (i < n4) {
+                T4 r;
+                r.x = dopt_op(x[u].x, y[u].x);
+                r.y = dopt_op(x[u].y, y[u].y);
+                r.z = dopt_op(x[u].z, y[u].z);
+                r.w = dopt_op(x[u].w, y[u].w);
+                o4[i] = r;
+            }
+        }
+    }
+    if (blockIdx.x == 0) {
+        size_t i = (n4 << 2) + threadIdx.x;
+        if (i < n) {
+#if ARITY == 2
+            o[i] = dopt_op(a[i], b[i]);
+#else
+            o[i] = dopt_op(a[i], a[i]);
+#endif
+        }
+    }
+}
+
+// Any alignment.
+extern "C" __global__ __launch_bounds__(BLOCK) void pw_scalar(size_t n, const T *a, const T *b, T *o)
+{
+    for (size_t i = (size_t)blockIdx.x * BLOCK + threadIdx.x; i < n; i += (size_t)gridDim.x * BLOCK) {
+#if ARITY == 2
+        o[i] = dopt_op(a[i], b[i]);
+#else
+        o[i] = dopt_op(a[i], a[i]);
+#endif
+    }
+}
+)SRC";
+
+std::string pointwise_source(const OpInfo &op, int dtype)
+{
+    std::string s;
+    s += dtype == DOPT_HIP_F32 ? "typedef float T;\n" : "typedef int T;\n";
+    s += "#define ARITY " + std::to_string(op.arity) + "\n";
+    s += std::string("#define OPEXPR ") + (dtype == DOPT_HIP_F32 ? op.expr_f32 : op.expr_i32) + "\n";
+    s += kPointwiseBody;
+    return s;
+}
+
+// ------------------------------------------------------------------------------ reductions
+
+const char *kReduceBody = R"SRC(
+#define BLOCK 256
+
+__device__ inline T combine(T a, T b) { return (T)(COMBINE); }
+
+__device__ inline T wave_reduce(T v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        T o = __shfl_down(v, off, 64);
+        v = combine(v, o);
+    }
+    return v;
+}
+
+__device__ inline T block_reduce(T v)
+{
+    __shared__ T part[BLOCK / 64];
+    v = wave_reduce(v);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = v;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int w = 1; w < BLOCK / 64; w++) v = combine(v, part[w]);
+    }
+    return v;  // valid in thread 0
+}
+
+// Contiguous rows: block (row o, chunk c) reduces in[o*R + c*chunk ... ) into out[o*nchunks + c].
+extern "C" __global__ __launch_bounds__(BLOCK) void red_rows(const T *in, T *out, size_t R, size_t chunk,
+                                                              size_t nchunks)
+{
+    const size_t o = blockIdx.x / nchunks, c = blockIdx.x % nchunks;
+    const size_t start = c * chunk;
+    size_t end = start + chunk;
+    if (end > R) end = R;
+    const T *row = in + o * R;
+    T acc0 = (T)(IDENT), acc1 = (T)(IDENT), acc2 = (T)(IDENT), acc3 = (T)(IDENT);
+    size_t i = start + threadIdx.x;
+    for (; i + 3 * BLOCK < end; i += 4 * BLOCK) {
+        T v0 = row[i], v1 = row[i + BLOCK], v2 = row[i + 2 * BLOCK], v3 = row[i + 3 * BLOCK];
+        acc0 = combine(acc0, v0);
+        acc1 = combine(acc1, v1);
+        acc2 = combine(acc2, v2);
+        acc3 = combine(acc3, v3);
+    }
+    for (; i < end; i += BLOCK) acc0 = combine(acc0, row[i]);
+    T acc = combine(combine(acc0, acc1), combine(acc2, acc3));
+    acc = block_reduce(acc);
+    if (threadIdx.x == 0) out[blockIdx.x] = acc;
+}
+
+// Strided lanes: thread (o, j) folds in[(o*R + r)*inner + j] over r, coalesced across j.
+extern "C" __global__ __launch_bounds__(BLOCK) void red_cols(const T *in, T *out, size_t outer, size_t R,
+                                                              size_t inner)
+{
+    const size_t total = outer * inner;
+    for (size_t idx = (size_t)blockIdx.x * BLOCK + threadIdx.x; idx < total; idx += (size_t)gridDim.x * BLOCK) {
+        const size_t o = idx / inner, j = idx % inner;
+        const T *p = in + o * R * inner + j;
+        T acc = (T)(IDENT);
+        for (size_t r = 0; r < R; r++) acc = combine(acc, p[r * inner]);
+        out[idx] = acc;
+    }
+}
+)SRC";
+
+const char *kArgminBody = R"SRC(
+#define BLOCK 256
+// Thread (o, j) scans the axis with a strict '<' against the type's maximum: the first minimum
+// wins and a lane that never fires keeps index 0 (cpu/math.d:281-296).
+extern "C" __global__ __launch_bounds__(BLOCK) void argmin_k(const T *in, int *out, size_t outer, size_t A,
+                                                              size_t vol)
+{
+    const size_t total = outer * vol;
+    for (size_t idx = (size_t)blockIdx.x * BLOCK + threadIdx.x; idx < total; idx += (size_t)gridDim.x * BLOCK) {
+        const size_t o = idx / vol, j = idx % vol;
+        const T *p = in + o * A * vol + j;
+        T best = (T)(TMAX);
+        int bi = 0;
+        for (size_t i = 0; i < A; i++) {
+            T v = p[i * vol];
+            if (v < best) {
+                best = v;
+                bi = (int)i;
+            }
+        }
+        out[idx] = bi;
+    }
+}
+)SRC";
+
+std::string reduce_source(bool is_sum, int dtype)
+{
+    std::string s;
+    bool f = dtype == DOPT_HIP_F32;
+    s += f ? "typedef float T;\n" : "typedef int T;\n";
+    if (is_sum) {
+        s += f ? "#define COMBINE a + b\n" : "#define COMBINE (int)((unsigned)a + (unsigned)b)\n";
+        s += "#define IDENT 0\n";
+    } else {
+        s += "#define COMBINE (a < b ? b : a)\n";
+        // identity -T.max (cpu/math.d:186): int32 starts at -INT_MAX, not INT_MIN
+        s += f ? "#define IDENT -3.402823466e+38f\n" : "#define IDENT -2147483647\n";
+    }
+    s += kReduceBody;
+    return s;
+}
+
+std::string argmin_source(int dtype)
+{
+    std::string s;
+    s += dtype == DOPT_HIP_F32 ? "typedef float T;\n#define TMAX 3.402823466e+38f\n"
+                               : "typedef int T;\n#define TMAX 2147483647\n";
+    s += kArgminBody;
+    return s;
+}
+
+unsigned grid_for(size_t work_items_per_block_unit, size_t units)
+{
+    size_t blocks = ceil_div(units, work_items_per_block_unit);
+    size_t cap = (size_t)num_cus() * 8;
+    if (blocks > cap) blocks = cap;
+    if (blocks < 1) blocks = 1;
+    return (unsigned)blocks;
+}
+
+int check_dtype(int dtype)
+{
+    if (dtype != DOPT_HIP_F32 && dtype != DOPT_HIP_I32)
+        return fail(DOPT_HIP_ERR_UNSUPPORTED, "Element type not supported.");
+    return DOPT_HIP_OK;
+}
+
+// One (outer, R, inner) reduction pass on the device.
+int reduce_pass(hipFunction_t rows, hipFunction_t cols, const void *in, void *out, size_t outer, size_t R,
+                size_t inner, size_t esize)
+{
+    if (outer * inner == 0) return DOPT_HIP_OK;
+    if (inner > 1 || R <= 64) {
+        unsigned grid = grid_for(256, outer * inner);
+        void *args[] = {(void *)&in, (void *)&out, (void *)&outer, (void *)&R, (void *)&inner};
+        return rtc_launch(cols, grid, 256, args);
+    }
+    // contiguous rows
+    size_t nchunks = 1;
+    if (outer < 1024) {
+        size_t want = ceil_div((size_t)num_cus() * 4, outer);
+        size_t maxc = ceil_div(R, (size_t)256 * 16);
+        nchunks = want < maxc ? want : maxc;
+        if (nchunks < 1) nchunks = 1;
+    }
+    size_t chunk = ceil_div(R, nchunks);
+    chunk = (chunk + 255) / 256 * 256;
+    nchunks = ceil_div(R, chunk);
+    if (nchunks == 1) {
+        void *args[] = {(void *)&in, (void *)&out, (void *)&R, (void *)&chunk, (void *)&nchunks};
+        return rtc_launch(rows, (unsigned)outer, 256, args);
+    }
+    void *partial = nullptr;
+    int rc = dopt_hip_malloc(&partial, outer * nchunks * esize);
+    if (rc) return rc;
+    {
+        void *args[] = {(void *)&in, (void *)&partial, (void *)&R, (void *)&chunk, (void *)&nchunks};
+        rc = rtc_launch(rows, (unsigned)(outer * nchunks), 256, args);
+    }
+    if (!rc) {
+        size_t one = 1, r2 = nchunks, chunk2 = (nchunks + 255) / 256 * 256;
+        const void *pin = partial;
+        void *args[] = {(void *)&pin, (void *)&out, (void *)&r2, (void *)&chunk2, (void *)&one};
+        rc = rtc_launch(rows, (unsigned)outer, 256, args);
+    }
+    dopt_hip_free(partial);  // stream-ordered: the next user of this block is enqueued after us
+    return rc;
+}
+
+}  // namespace
+
+extern "C" {
+
+int dopt_hip_pointwise(const char *op, int dtype, size_t n, const void *a, const void *b, void *out)
+{
+    DOPT_REQUIRE(op != nullptr, "dopt_hip_pointwise: op is null");
+    const OpInfo *info = find_op(op);
+    if (!info) return fail(DOPT_HIP_ERR_UNSUPPORTED, "dopt_hip_pointwise: unknown operation '%s'", op);
+    if (int rc = check_dtype(dtype)) return rc;
+    DOPT_REQUIRE((info->arity == 2) == (b != nullptr), "dopt_hip_pointwise: '%s' takes %d operand(s)", op,
+                 info->arity);
+    if (n == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(a && out, "dopt_hip_pointwise: null operand");
+    DOPT_ENSURE_INIT();
+    bool vec = aligned16(a) && aligned16(out) && (!b || aligned16(b));
+    const char *kname = vec ? "pw_vec" : "pw_scalar";
+    std::string key = std::string("pw:") + op + (dtype == DOPT_HIP_F32 ? ":f32:" : ":i32:") + kname;
+    hipFunction_t fn;
+    if (int rc = rtc_get(key, pointwise_source(*info, dtype), kname, &fn)) return rc;
+    const void *bb = b ? b : a;
+    unsigned grid = vec ? grid_for(256 * 4, ceil_div(n, 4)) : grid_for(256, n);
+    void *args[] = {(void *)&n, (void *)&a, (void *)&bb, (void *)&out};
+    return rtc_launch(fn, grid, 256, args);
+}
+
+int dopt_hip_reduce(const char *op, int dtype, const size_t *shape, int rank, const size_t *axes, int naxes,
+                    const void *in, void *out)
+{
+    DOPT_REQUIRE(op && shape && axes && in && out, "dopt_hip_reduce: null argument");
+    bool is_sum = !strcmp(op, "sum");
+    if (!is_sum && strcmp(op, "maxElement"))
+        return fail(DOPT_HIP_ERR_UNSUPPORTED, "dopt_hip_reduce: unknown reduction '%s'", op);
+    if (int rc = check_dtype(dtype)) return rc;
+    DOPT_REQUIRE(rank >= 1 && rank <= 16 && naxes >= 1 && naxes <= rank, "dopt_hip_reduce: bad rank/axes count");
+    bool reduced[16] = {false};
+    for (int i = 0; i < naxes; i++) {
+        DOPT_REQUIRE(axes[i] < (size_t)rank && !reduced[axes[i]], "dopt_hip_reduce: axes must be distinct and < rank");
+        reduced[axes[i]] = true;
+    }
+    size_t cur[16];
+    size_t vol = 1;
+    for (int i = 0; i < rank; i++) {
+        cur[i] = shape[i];
+        vol *= shape[i];
+    }
+    if (vol == 0) return DOPT_HIP_OK;
+    DOPT_ENSURE_INIT();
+    std::string key = std::string("red:") + op + (dtype == DOPT_HIP_F32 ? ":f32" : ":i32");
+    std::string src = reduce_source(is_sum, dtype);
+    hipFunction_t rows, cols;
+    if (int rc = rtc_get(key + ":rows", src, "red_rows", &rows)) return rc;
+    if (int rc = rtc_get(key + ":cols", src, "red_cols", &cols)) return rc;
+
+    // Runs of adjacent reduced axes collapse into one (outer, R, inner) pass each, last run first.
+    // The result is independent of the order in which axes are folded up to fp32 rounding.
+    std::vector<std::pair<int, int>> runs;
+    for (int i = 0; i < rank;) {
+        if (!reduced[i]) { i++; continue; }
+        int j = i;
+        while (j + 1 < rank && reduced[j + 1]) j++;
+        runs.push_back({i, j});
+        i = j + 1;
+    }
+    const void *src_ptr = in;
+    void *tmp_prev = nullptr;
+    int rc = DOPT_HIP_OK;
+    for (int ri = (int)runs.size() - 1; ri >= 0 && !rc; ri--) {
+        int a0 = runs[ri].first, a1 = runs[ri].second;
+        size_t outer = 1, R = 1, inner = 1;
+        for (int i = 0; i < a0; i++) outer *= cur[i];
+        for (int i = a0; i <= a1; i++) R *= cur[i];
+        for (int i = a1 + 1; i < rank; i++) inner *= cur[i];
+        void *dst = out;
+        void *tmp = nullptr;
+        if (ri > 0) {
+            rc = dopt_hip_malloc(&tmp, outer * inner * 4);
+            if (rc) break;
+            dst = tmp;
+        }
+        rc = reduce_pass(rows, cols, src_ptr, dst, outer, R, inner, 4);
+        if (tmp_prev) dopt_hip_free(tmp_prev);
+        tmp_prev = tmp;
+        src_ptr = dst;
+        for (int i = a0; i <= a1; i++) cur[i] = 1;
+    }
+    if (tmp_prev) dopt_hip_free(tmp_prev);
+    return rc;
+}
+
+int dopt_hip_argmin(int dtype, const size_t *shape, int rank, size_t axis, const void *in, int32_t *out)
+{
+    DOPT_REQUIRE(shape && in && out, "dopt_hip_argmin: null argument");
+    if (int rc = check_dtype(dtype)) return rc;
+    DOPT_REQUIRE(rank >= 1 && rank <= 16 && axis < (size_t)rank, "dopt_hip_argmin: axis must be < rank");
+    size_t outer = 1, A = shape[axis], vol = 1;
+    for (size_t i = 0; i < axis; i++) outer *= shape[i];
+    for (int i = (int)axis + 1; i < rank; i++) vol *= shape[i];
+    if (outer * vol == 0) return DOPT_HIP_OK;
+    DOPT_ENSURE_INIT();
+    hipFunction_t fn;
+    std::string key = std::string("argmin") + (dtype == DOPT_HIP_F32 ? ":f32" : ":i32");
+    if (int rc = rtc_get(key, argmin_source(dtype), "argmin_k", &fn)) return rc;
+    unsigned grid = grid_for(256, outer * vol);
+    void *args[] = {(void *)&in, (void *)&out, (void *)&outer, (void *)&A, (void *)&vol};
+    return rtc_launch(fn, grid, 256, args);
+}
+
+int dopt_hip_rtc_compile_only(const char *op, int dtype, const char *arch)
+{
+    DOPT_REQUIRE(op && arch, "dopt_hip_rtc_compile_only: null argument");
+    if (int rc = check_dtype(dtype)) return rc;
+    std::string src;
+    if (!strcmp(op, "sum") || !strcmp(op, "maxElement")) {
+        src = reduce_source(!strcmp(op, "sum"), dtype);
+    } else if (!strcmp(op, "argmin")) {
+        src = argmin_source(dtype);
+    } else {
+        const OpInfo *info = find_op(op);
+        if (!info) return fail(DOPT_HIP_ERR_UNSUPPORTED, "dopt_hip_rtc_compile_only: unknown operation '%s'", op);
+        src = pointwise_source(*info, dtype);
+    }
+    return rtc_compile_only(src, arch, nullptr);
+}
+
+}  // extern "C"

@@ -1,0 +1,331 @@
+"""Thin numpy-facing wrappers over the C ABI: a device `Tensor` (pooled HIP buffer + shape +
+dtype) and one function per kernel entry point.  Shapes follow the reference's op judges
+(core/source/dopt/core/ops/{basic,math,nnet}.d); all arithmetic happens in libdopthip.so.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import capi
+
+_DT = {np.dtype(np.float32): capi.F32, np.dtype(np.int32): capi.I32}
+
+
+def _vol(shape):
+    v = 1
+    for s in shape:
+        v *= int(s)
+    return v
+
+
+class Tensor:
+    """A dense row-major device tensor owning a pooled buffer (the HIPBuffer of this backend)."""
+
+    def __init__(self, shape, dtype=np.float32, _ptr=None, _owner=None):
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = np.dtype(dtype)
+        if self.dtype not in _DT:
+            raise capi.HipError(3, "Element type not supported.")
+        self.nbytes = _vol(self.shape) * 4
+        self._owner = _owner
+        if _ptr is not None:
+            self.ptr = _ptr
+        else:
+            p = C.c_void_p()
+            capi.check(capi.load().dopt_hip_malloc(C.byref(p), self.nbytes))
+            self.ptr = p.value or 0
+
+    @property
+    def size(self):
+        return _vol(self.shape)
+
+    @property
+    def code(self):
+        return _DT[self.dtype]
+
+    def set(self, array):
+        a = np.ascontiguousarray(array, dtype=self.dtype)
+        if a.nbytes != self.nbytes:
+            raise capi.HipError(1, "input buffer is the wrong length.")
+        capi.check(capi.load().dopt_hip_copy_h2d(self.ptr, a.ctypes.data, a.nbytes))
+        return self
+
+    def numpy(self):
+        out = np.empty(self.shape, self.dtype)
+        capi.check(capi.load().dopt_hip_copy_d2h(out.ctypes.data, self.ptr, self.nbytes))
+        return out
+
+    def reshape(self, shape):
+        """Aliases the same buffer (the reference's `reshape` has no kernel either)."""
+        if _vol(shape) != self.size:
+            raise ValueError("reshape changes the volume")
+        return Tensor(shape, self.dtype, _ptr=self.ptr, _owner=self)
+
+    def view(self, offset, shape):
+        """Sub-buffer starting `offset` elements in (packed batch-norm outputs)."""
+        if offset + _vol(shape) > self.size:
+            raise ValueError("view out of range")
+        return Tensor(shape, self.dtype, _ptr=self.ptr + 4 * offset, _owner=self)
+
+    def free(self):
+        if self._owner is None and self.ptr:
+            capi.load().dopt_hip_free(self.ptr)
+        self.ptr = 0
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def tensor(array, dtype=None):
+    a = np.ascontiguousarray(array, dtype=dtype)
+    if a.dtype == np.float64:
+        a = a.astype(np.float32)
+    if a.dtype == np.int64:
+        a = a.astype(np.int32)
+    return Tensor(a.shape, a.dtype).set(a)
+
+
+def sync():
+    capi.check(capi.load().dopt_hip_sync())
+
+
+# ------------------------------------------------------------------------------- pointwise
+
+def pointwise(op, a, b=None):
+    out = Tensor(a.shape, a.dtype)
+    if b is not None and (b.shape != a.shape or b.dtype != a.dtype):
+        raise capi.HipError(1, "pointwise operands must have the same type")
+    capi.check(capi.load().dopt_hip_pointwise(op.encode(), a.code, a.size, a.ptr, b.ptr if b is not None else None,
+                                              out.ptr))
+    return out
+
+
+def _reduce(name, a, axes):
+    axes = list(range(len(a.shape))) if not axes else [int(x) for x in axes]
+    oshape = [s for i, s in enumerate(a.shape) if i not in axes]
+    out = Tensor(oshape, a.dtype)
+    capi.check(capi.load().dopt_hip_reduce(name, a.code, capi.sizes(a.shape), len(a.shape), capi.sizes(axes),
+                                           len(axes), a.ptr, out.ptr))
+    return out
+
+
+def sum(a, axes=None):  # noqa: A001 - reference op name
+    return _reduce(b"sum", a, axes)
+
+
+def max_element(a, axes=None):
+    return _reduce(b"maxElement", a, axes)
+
+
+def argmin(a, axis):
+    oshape = list(a.shape)
+    oshape[axis] = 1
+    out = Tensor(oshape, np.int32)
+    capi.check(capi.load().dopt_hip_argmin(a.code, capi.sizes(a.shape), len(a.shape), axis, a.ptr, out.ptr))
+    return out
+
+
+# ------------------------------------------------------------------------------- layout
+
+def slice(a, start, stop):  # noqa: A001
+    oshape = [e - s for s, e in zip(start, stop)]
+    out = Tensor(oshape, a.dtype)
+    capi.check(capi.load().dopt_hip_slice(len(a.shape), capi.sizes(a.shape), capi.sizes(oshape), capi.sizes(start),
+                                          a.ptr, out.ptr))
+    return out
+
+
+def pad(a, before, after):
+    oshape = [b + s + e for b, s, e in zip(before, a.shape, after)]
+    out = Tensor(oshape, a.dtype)
+    capi.check(capi.load().dopt_hip_pad(len(a.shape), capi.sizes(a.shape), capi.sizes(oshape), capi.sizes(before),
+                                        a.ptr, out.ptr))
+    return out
+
+
+def repeat(a, reps):
+    oshape = [s * r for s, r in zip(a.shape, reps)]
+    out = Tensor(oshape, a.dtype)
+    capi.check(capi.load().dopt_hip_repeat(len(a.shape), capi.sizes(a.shape), capi.sizes(reps), a.ptr, out.ptr))
+    return out
+
+
+def transpose(a):
+    rows, cols = a.shape
+    out = Tensor((cols, rows), a.dtype)
+    capi.check(capi.load().dopt_hip_transpose2d(rows, cols, a.ptr, out.ptr))
+    return out
+
+
+# ------------------------------------------------------------------------------- dense / conv
+
+def matmul(a, b):
+    if a.dtype != np.float32 or b.dtype != np.float32:
+        raise capi.HipError(3, "Element type not supported.")
+    M, K = a.shape
+    K2, N = b.shape
+    if K != K2:
+        raise capi.HipError(1, "matmul: inner dimensions differ")
+    out = Tensor((M, N))
+    capi.check(capi.load().dopt_hip_sgemm(M, N, K, a.ptr, b.ptr, out.ptr))
+    return out
+
+
+def conv_desc(xshape, wshape, padding=(0, 0), stride=(1, 1)):
+    N, Cc, H, W = xshape
+    K, C2, R, S = wshape
+    if Cc != C2:
+        raise capi.HipError(1, "convolution: channel counts differ")
+    return capi.ConvDesc(N, Cc, H, W, K, R, S, padding[0], padding[1], stride[0], stride[1])
+
+
+def conv_out_shape(d):
+    return (d.N, d.K, (d.H + 2 * d.padH - d.R) // d.strideH + 1, (d.W + 2 * d.padW - d.S) // d.strideW + 1)
+
+
+def convolution(x, w, padding=(0, 0), stride=(1, 1)):
+    d = conv_desc(x.shape, w.shape, padding, stride)
+    y = Tensor(conv_out_shape(d))
+    capi.check(capi.load().dopt_hip_conv_fwd(C.byref(d), x.ptr, w.ptr, y.ptr))
+    return y
+
+
+def conv_bwd_data(dy, w, xshape, padding=(0, 0), stride=(1, 1)):
+    d = conv_desc(xshape, w.shape, padding, stride)
+    if tuple(dy.shape) != conv_out_shape(d):
+        raise capi.HipError(1, "convolutionFeaturesGrad: gradient shape does not match")
+    dx = Tensor(xshape)
+    capi.check(capi.load().dopt_hip_conv_bwd_data(C.byref(d), dy.ptr, w.ptr, dx.ptr))
+    return dx
+
+
+def conv_bwd_filter(dy, x, wshape, padding=(0, 0), stride=(1, 1)):
+    d = conv_desc(x.shape, wshape, padding, stride)
+    if tuple(dy.shape) != conv_out_shape(d):
+        raise capi.HipError(1, "convolutionFiltersGrad: gradient shape does not match")
+    dw = Tensor(wshape)
+    capi.check(capi.load().dopt_hip_conv_bwd_filter(C.byref(d), dy.ptr, x.ptr, dw.ptr))
+    return dw
+
+
+# ------------------------------------------------------------------------------- NN ops
+
+def _nci(shape):
+    inner = _vol(shape[2:]) if len(shape) > 2 else 1
+    return shape[0], shape[1], inner
+
+
+def maxpool(x, dims):
+    N, Cc, H, W = x.shape
+    y = Tensor((N, Cc, H // dims[0], W // dims[1]))
+    capi.check(capi.load().dopt_hip_maxpool_fwd(N, Cc, H, W, dims[0], dims[1], x.ptr, y.ptr))
+    return y
+
+
+def maxpool_grad(dy, x, dims):
+    N, Cc, H, W = x.shape
+    dx = Tensor(x.shape)
+    capi.check(capi.load().dopt_hip_maxpool_bwd(N, Cc, H, W, dims[0], dims[1], dy.ptr, x.ptr, dx.ptr))
+    return dx
+
+
+def softmax(x):
+    y = Tensor(x.shape)
+    capi.check(capi.load().dopt_hip_softmax_fwd(*_nci(x.shape), x.ptr, y.ptr))
+    return y
+
+
+def softmax_grad(dy, y):
+    dx = Tensor(y.shape)
+    capi.check(capi.load().dopt_hip_softmax_bwd(*_nci(y.shape), dy.ptr, y.ptr, dx.ptr))
+    return dx
+
+
+def relu(x):
+    y = Tensor(x.shape)
+    capi.check(capi.load().dopt_hip_relu_fwd(x.size, x.ptr, y.ptr))
+    return y
+
+
+def relu_grad(dy, x):
+    dx = Tensor(x.shape)
+    capi.check(capi.load().dopt_hip_relu_bwd(x.size, dy.ptr, x.ptr, dx.ptr))
+    return dx
+
+
+def add_bias(x, b):
+    y = Tensor(x.shape)
+    capi.check(capi.load().dopt_hip_bias_fwd(*_nci(x.shape), x.ptr, b.ptr, y.ptr))
+    return y
+
+
+def add_bias_grad(dy):
+    db = Tensor((dy.shape[1],))
+    capi.check(capi.load().dopt_hip_bias_bwd(*_nci(dy.shape), dy.ptr, db.ptr))
+    return db
+
+
+def bn_train(x, scale, bias, run_mean, run_var, momentum):
+    N, Cc, inner = _nci(x.shape)
+    packed = Tensor((x.size + 2 * Cc,))
+    capi.check(capi.load().dopt_hip_bn_train(N, Cc, inner, float(momentum), x.ptr, scale.ptr, bias.ptr, run_mean.ptr,
+                                             run_var.ptr, packed.ptr))
+    return packed
+
+
+def bn_grad(dy, x, scale):
+    N, Cc, inner = _nci(x.shape)
+    packed = Tensor((x.size + 2 * Cc,))
+    capi.check(capi.load().dopt_hip_bn_grad(N, Cc, inner, dy.ptr, x.ptr, scale.ptr, packed.ptr))
+    return packed
+
+
+def bn_infer(x, scale, bias, mean, var):
+    y = Tensor(x.shape)
+    capi.check(capi.load().dopt_hip_bn_infer(*_nci(x.shape), x.ptr, scale.ptr, bias.ptr, mean.ptr, var.ptr, y.ptr))
+    return y
+
+
+# ------------------------------------------------------------------------------- optimizers
+
+class FusedOptimizer:
+    """Multi-tensor in-place updater over fixed parameter / gradient / state tensors."""
+
+    def __init__(self, params, grads, m, v=None, vhat=None, skip=None):
+        n = len(params)
+        refs = (capi.TensorRef * max(n, 1))()
+        for i in range(n):
+            refs[i] = capi.TensorRef(params[i].ptr, grads[i].ptr, m[i].ptr, v[i].ptr if v else None,
+                                     vhat[i].ptr if vhat else None, params[i].size,
+                                     1 if (skip and skip[i]) else 0)
+        self._keep = (params, grads, m, v, vhat)
+        h = C.c_void_p()
+        capi.check(capi.load().dopt_hip_optim_create(n, refs, C.byref(h)))
+        self._h = h
+        self.b1 = C.c_float(1.0)   # online/adam.d:44-45: b1, b2 start at 1
+        self.b2 = C.c_float(1.0)
+
+    def sgd(self, lr=0.01, mu=0.0, nesterov=False):
+        capi.check(capi.load().dopt_hip_sgd_step(self._h, lr, mu, int(nesterov)))
+
+    def adam(self, alpha=1e-3, beta1=0.9, beta2=0.999, eps=1e-8):
+        capi.check(capi.load().dopt_hip_adam_step(self._h, alpha, beta1, beta2, eps, C.byref(self.b1),
+                                                  C.byref(self.b2)))
+
+    def amsgrad(self, alpha=1e-3, beta1=0.9, beta2=0.999, eps=1e-8):
+        capi.check(capi.load().dopt_hip_amsgrad_step(self._h, alpha, beta1, beta2, eps, C.byref(self.b1),
+                                                     C.byref(self.b2)))
+
+    def close(self):
+        if self._h:
+            capi.load().dopt_hip_optim_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

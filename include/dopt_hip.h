@@ -1,0 +1,226 @@
+/*
+ * dopt_hip.h -- C ABI of libdopthip.so, the MI355X (gfx950) kernel library behind dopt's
+ * device-backend plugin interface.
+ *
+ * This is the surface a `dopt.hip` D package binds with `extern(C)`: each entry point
+ * replaces one device call site of the reference's CUDA backend (cited per function as
+ * file:line under the reference's root).  Conventions:
+ *   - every function returns 0 on success; non-zero is an error code from dopt_hip_status and
+ *     dopt_hip_last_error() then holds the message the D wrapper passes to `enforce`;
+ *   - all tensor pointers are DEVICE pointers unless the name says host; tensors are dense,
+ *     row-major (NCHW / KCRS for images and filters); sizes count elements, not bytes;
+ *   - everything is enqueued on one library-owned HIP stream and returns without waiting;
+ *     dopt_hip_copy_d2h and dopt_hip_sync are the synchronisation points (the reference
+ *     synchronises after nearly every launch, but callers only rely on ordering and on a
+ *     device-to-host read seeing finished data);
+ *   - single host thread per process, like the reference's registries.
+ */
+#ifndef DOPT_HIP_H
+#define DOPT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    DOPT_HIP_OK = 0,
+    DOPT_HIP_ERR_INVALID = 1,     /* argument the reference would `enforce` against */
+    DOPT_HIP_ERR_RUNTIME = 2,     /* a HIP runtime call failed */
+    DOPT_HIP_ERR_UNSUPPORTED = 3, /* "Element type not supported." / unknown op name */
+    DOPT_HIP_ERR_OOM = 4,         /* "CUDA memory allocation failed" analogue */
+    DOPT_HIP_ERR_RTC = 5          /* run-time compilation failed (log in last_error) */
+} dopt_hip_status;
+
+/* element types of core/source/dopt/core/types.d:5-14 that the backend supports
+   (cuda/package.d:511-525) */
+typedef enum { DOPT_HIP_F32 = 0, DOPT_HIP_I32 = 1 } dopt_hip_dtype;
+
+/* ---------------------------------------------------------------------------------------
+ * Runtime: device, stream, pooled buffers, copies.
+ * ------------------------------------------------------------------------------------- */
+
+/* cuda/package.d:36-63 (cuInit / cuCtxCreate on device 0).  Idempotent. */
+int dopt_hip_init(int device);
+/* Frees the pool, the workspace, cached RTC modules and the stream. */
+int dopt_hip_shutdown(void);
+/* Message of the last failing call on this thread ("" if none). */
+const char *dopt_hip_last_error(void);
+
+/* CUDABuffer.create, cuda/package.d:134-156: device allocation, zero-filled.  Served from a
+   size-class pool over hipMalloc instead of one cuMemAlloc + GC.collect() per buffer.
+   bytes == 0 yields *ptr == NULL and success (package.d:144-147). */
+int dopt_hip_malloc(void **ptr, size_t bytes);
+/* CUDABuffer.destroy, cuda/package.d:161-164: returns the block to the pool. */
+int dopt_hip_free(void *ptr);
+/* Releases every cached (free) block back to the driver. */
+int dopt_hip_pool_trim(void);
+/* live = bytes handed out, cached = bytes parked in the pool, device_allocs = hipMalloc calls so far. */
+int dopt_hip_pool_stats(size_t *live_bytes, size_t *cached_bytes, size_t *device_allocs);
+
+/* cuMemsetD8 (cuda/package.d:152,245; cuda/basic.d:135) */
+int dopt_hip_memset(void *dst, int byte_value, size_t bytes);
+/* CUDABuffer.set(void[]) -> cuMemcpyHtoD, cuda/package.d:172-176 */
+int dopt_hip_copy_h2d(void *dst, const void *host_src, size_t bytes);
+/* CUDABuffer.get -> cuMemcpyDtoH, cuda/package.d:207-211.  Waits for all queued work. */
+int dopt_hip_copy_d2h(void *host_dst, const void *src, size_t bytes);
+/* CUDABuffer.set(DeviceBuffer) -> cuMemcpyDtoD, cuda/package.d:187-190 */
+int dopt_hip_copy_d2d(void *dst, const void *src, size_t bytes);
+/* cuCtxSynchronize (cuda/nvrtc.d:111,123; cudnn7.d:157 ...) */
+int dopt_hip_sync(void);
+/* The hipStream_t every entry point enqueues on (for callers that record their own events). */
+void *dopt_hip_stream(void);
+
+/* Event pairs on the library stream: the device-time replacement for the host StopWatch of
+   CUDAPlan.profiler (cuda/package.d:265,410-415). */
+int dopt_hip_event_create(void **event);
+int dopt_hip_event_record(void *event);
+int dopt_hip_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for `stop` */
+int dopt_hip_event_destroy(void *event);
+
+/* ---------------------------------------------------------------------------------------
+ * Pointwise and reductions: hipRTC-instantiated gfx950 templates (replace the NVRTC generator,
+ * cuda/nvrtc.d:29-132 and cuda/math.d:129-205).  Compiled once per (op, dtype), cached.
+ * ------------------------------------------------------------------------------------- */
+
+/* cuda/math.d:89-127 with CPU-evaluator semantics (cpu/math.d:312-437).
+   Binary: add sub mul div lt lte gt gte eq neq max min pow atan2  (b != NULL)
+   Unary : neg abs sgn exp log sqrt sin cos tan asin acos atan sinh cosh tanh asinh acosh atanh
+           (b == NULL).  The reference's CUDA backend sends everything after sqrt to a host
+           round trip (cuda/package.d:81-119); here they run on the device. */
+int dopt_hip_pointwise(const char *op, int dtype, size_t n, const void *a, const void *b_or_null, void *out);
+
+/* `sum` / `maxElement` (op = "sum" | "maxElement"): cpu/math.d:90-247, reached in the reference through
+   the host fallback cuda/package.d:81-119.  Reduces `axes` (distinct, each < rank) of a dense
+   tensor; out has the reduced axes removed (core/ops/math.d:162-175). */
+int dopt_hip_reduce(const char *op, int dtype, const size_t *shape, int rank,
+                    const size_t *axes, int naxes, const void *in, void *out);
+/* `argmin`: cpu/math.d:249-310.  int32 output with the reduced axis kept as size 1
+   (core/ops/math.d:185-191); the first minimum wins; a lane with no element below the
+   type's maximum yields index 0. */
+int dopt_hip_argmin(int dtype, const size_t *shape, int rank, size_t axis, const void *in, int32_t *out);
+
+/* Compiles the template for (op, dtype) for `arch` (e.g. "gfx950") without loading it: lets a
+   machine with no GPU check that every template builds.  op may also be "sum", "maxElement", "argmin". */
+int dopt_hip_rtc_compile_only(const char *op, int dtype, const char *arch);
+
+/* ---------------------------------------------------------------------------------------
+ * Layout ops on 4-byte elements (cuda/basic.d hard-codes size = 4 at :40,:95).
+ * ------------------------------------------------------------------------------------- */
+
+/* `slice`: cuda/basic.d:31-84 (one cuMemcpy per innermost row there; one kernel here). */
+int dopt_hip_slice(int rank, const size_t *in_shape, const size_t *out_shape, const size_t *start,
+                   const void *in, void *out);
+/* `pad`: cuda/basic.d:86-141 (memset + row copies there; one kernel writing every element here). */
+int dopt_hip_pad(int rank, const size_t *in_shape, const size_t *out_shape, const size_t *before,
+                 const void *in, void *out);
+/* `repeat`: cuda/basic.d:143-217; tiling order pinned by core/ops/basic.d:336-356. */
+int dopt_hip_repeat(int rank, const size_t *in_shape, const size_t *reps, const void *in, void *out);
+/* `transpose` of a rank-2 tensor [rows, cols] -> [cols, rows]: cublasSgeam at cuda/basic.d:237-238. */
+int dopt_hip_transpose2d(size_t rows, size_t cols, const void *in, void *out);
+
+/* ---------------------------------------------------------------------------------------
+ * Dense and convolution (fp32 MFMA).
+ * ------------------------------------------------------------------------------------- */
+
+/* `matmul`: cublasSgemm_v2 at cuda/math.d:234-235.  Row-major C[M,N] = A[M,K] * B[K,N],
+   alpha = 1, beta = 0, no transposes.  K == 1 (broadcast outer product), N == 1 and M == 1
+   (matrix-vector) take bandwidth-bound paths: the reference routes scalar broadcasts and
+   row/column sums through matmul (core/ops/basic.d:370-381, core/ops/math.d:257-279). */
+int dopt_hip_sgemm(size_t M, size_t N, size_t K, const float *A, const float *B, float *C);
+
+typedef struct {
+    size_t N, C, H, W;       /* features [N,C,H,W] */
+    size_t K, R, S;          /* filters  [K,C,R,S] */
+    size_t padH, padW, strideH, strideW;
+} dopt_hip_conv_desc;
+
+/* `convolution`: cudnnConvolutionForward at cudnn7.d:154, CUDNN_CONVOLUTION mode (:87): a TRUE
+   convolution, y[n,k,p,q] = sum x[n,c,p*sy-ph+r,q*sx-pw+s] * w[k,c,R-1-r,S-1-s]. */
+int dopt_hip_conv_fwd(const dopt_hip_conv_desc *d, const float *x, const float *w, float *y);
+/* `convolutionFeaturesGrad` (also convolutionTranspose): cudnnConvolutionBackwardData, cudnn7.d:199. */
+int dopt_hip_conv_bwd_data(const dopt_hip_conv_desc *d, const float *dy, const float *w, float *dx);
+/* `convolutionFiltersGrad`: cudnnConvolutionBackwardFilter, cudnn7.d:244. */
+int dopt_hip_conv_bwd_filter(const dopt_hip_conv_desc *d, const float *dy, const float *x, float *dw);
+
+/* ---------------------------------------------------------------------------------------
+ * Bandwidth-bound NN ops (fp32, NCHW; `inner` = product of the dims after the channel dim).
+ * ------------------------------------------------------------------------------------- */
+
+/* `maxpool`: cudnnPoolingForward, cudnn7.d:303; window = stride = (ph, pw), no padding,
+   output dims floor(H/ph) x floor(W/pw) (core/ops/nnet.d:97-107). */
+int dopt_hip_maxpool_fwd(size_t N, size_t C, size_t H, size_t W, size_t ph, size_t pw, const float *x, float *y);
+/* `maxpoolGrad`: cudnnPoolingBackward, cudnn7.d:328.  The reference passes (dy, y, x); y is
+   recomputed from x here, so it is not an argument.  Ties go to the first maximum of the
+   window in row-major order. */
+int dopt_hip_maxpool_bwd(size_t N, size_t C, size_t H, size_t W, size_t ph, size_t pw,
+                         const float *dy, const float *x, float *dx);
+/* `softmax` over dim 1 of [N, C, inner]: cudnnSoftmaxForward ACCURATE/CHANNEL, cudnn7.d:364;
+   arithmetic order of cpu/nnet.d:129-166. */
+int dopt_hip_softmax_fwd(size_t N, size_t C, size_t inner, const float *x, float *y);
+/* `softmaxGrad`: cudnnSoftmaxBackward, cudnn7.d:397; dx = y * (dy - sum_c dy*y). */
+int dopt_hip_softmax_bwd(size_t N, size_t C, size_t inner, const float *dy, const float *y, float *dx);
+/* `relu`: cudnnActivationForward RELU / PROPAGATE_NAN, cudnn7.d:433. */
+int dopt_hip_relu_fwd(size_t n, const float *x, float *y);
+/* `reluGrad`: cudnnActivationBackward, cudnn7.d:471; dx = x > 0 ? dy : 0 (y is not needed). */
+int dopt_hip_relu_bwd(size_t n, const float *dy, const float *x, float *dx);
+/* `addBias`: cuMemcpy + cudnnAddTensor, cudnn7.d:502-507; y = x + b[c] in one pass. */
+int dopt_hip_bias_fwd(size_t N, size_t C, size_t inner, const float *x, const float *b, float *y);
+/* `addBiasGrad`: cudnnConvolutionBackwardBias, cudnn7.d:539-540; db[c] = sum_{n,i} dy.  The
+   reference passes beta = 1 and so accumulates into its output buffer across executions;
+   this computes the plain sum (beta = 0), identical on the first execution. */
+int dopt_hip_bias_bwd(size_t N, size_t C, size_t inner, const float *dy, float *db);
+
+/* `batchNormTrain`: cudnnBatchNormalizationForwardTraining (spatial), cudnn7.d:608-610.
+   packed = [ y (N*C*inner) | newRunMean (C) | newRunVar (C) ] as core/ops/nnet.d:222-225;
+   momentum is the op attribute (running = momentum*running + (1-momentum)*batch; the running
+   variance takes the unbiased batch estimate); eps = 1e-5f. */
+int dopt_hip_bn_train(size_t N, size_t C, size_t inner, double momentum, const float *x,
+                      const float *scale, const float *bias, const float *run_mean,
+                      const float *run_var, float *packed);
+/* `batchNormGrad`: cudnnBatchNormalizationBackward, cudnn7.d:632-634.
+   packed = [ dx | dscale (C) | dbias (C) ] as core/ops/nnet.d:232-235; batch statistics are
+   recomputed from x as the reference does (it saves none). */
+int dopt_hip_bn_grad(size_t N, size_t C, size_t inner, const float *dy, const float *x,
+                     const float *scale, float *packed);
+/* `batchNormInference`: cudnnBatchNormalizationForwardInference, cudnn7.d:650-652; eps = 1e-5. */
+int dopt_hip_bn_infer(size_t N, size_t C, size_t inner, const float *x, const float *scale,
+                      const float *bias, const float *mean, const float *var, float *y);
+
+/* ---------------------------------------------------------------------------------------
+ * Fused multi-tensor optimizer updates.  The reference has no such kernels: dopt.online
+ * builds each rule as a graph of pointwise ops with GEMM broadcasts
+ * (online/source/dopt/online/{sgd,adam,amsgrad}.d).  These kernels restate those graphs with
+ * one fp32 rounding per graph node and no FMA contraction, in place, one launch for all
+ * tensors.
+ * ------------------------------------------------------------------------------------- */
+
+typedef struct {
+    float *w;        /* parameter, updated in place unless skip_w */
+    const float *g;  /* gradient */
+    float *m;        /* momentum buffer (SGD) / first moment (ADAM, AMSGrad), in place */
+    float *v;        /* second moment (ADAM, AMSGrad), in place; NULL for SGD */
+    float *vhat;     /* running max (AMSGrad), in place; NULL otherwise */
+    size_t n;        /* element count */
+    int skip_w;      /* 1: a projection replaces the new value (online/adam.d:66-72), leave w alone */
+} dopt_hip_tensor_ref;
+
+/* Builds the device-side chunk table for a fixed set of tensors; reuse it every step. */
+int dopt_hip_optim_create(int ntensors, const dopt_hip_tensor_ref *refs, void **handle);
+int dopt_hip_optim_destroy(void *handle);
+/* online/sgd.d:44-63.  mom' = mom*mu (+|-) lr*g;  w' = w - mom'  (Nesterov: (w + mu*mom') - lr*g). */
+int dopt_hip_sgd_step(void *handle, float lr, float mu, int nesterov);
+/* online/adam.d:44-63.  *b1, *b2 (host) are the persisted running products beta^t; they are
+   advanced here exactly as the graph does (nb = b*beta) and eta is derived from them on the
+   host in fp32: eta = (alpha*sqrt(1-nb2))/(1-nb1). */
+int dopt_hip_adam_step(void *handle, float alpha, float beta1, float beta2, float eps, float *b1, float *b2);
+/* online/amsgrad.d:52-69: ADAM's m', v', w' (w' uses v', as the reference does) plus
+   vhat' = max(vhat, OLD v). */
+int dopt_hip_amsgrad_step(void *handle, float alpha, float beta1, float beta2, float eps, float *b1, float *b2);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DOPT_HIP_H */

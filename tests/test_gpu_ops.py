@@ -1,0 +1,419 @@
+"""Parity of every kernel entry point of libdopthip.so (through the C ABI) against the CPU oracle.
+
+Tolerances are the ones the project states: bit-exact for integer, index and layout work and
+for single-rounding fp32 arithmetic; <= 2 ulp for fp32 transcendentals; rtol 1e-4 / atol 1e-5
+for GEMM, convolution and reductions (atol scaled by sqrt(reduction length) where the summed
+terms are O(1) random numbers, since the sum itself then has that magnitude).
+"""
+import numpy as np
+import pytest
+
+import oracle as O
+from util import assert_close, ulp_diff
+
+pytestmark = pytest.mark.gpu
+
+ops = pytest.importorskip("dopt_amd.ops")
+T = ops.tensor
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+# ----------------------------------------------------------------------------- runtime
+def test_buffer_roundtrip_zero_fill_and_pool_reuse():
+    from dopt_amd import capi
+    import ctypes as C
+    lib = capi.load()
+    a = rng(0).standard_normal(100003).astype(np.float32)
+    t = T(a)
+    assert np.array_equal(t.numpy(), a)
+    z = ops.Tensor((4097,), np.int32)
+    assert not z.numpy().any()                      # CUDABuffer.create zero-fills
+    with pytest.raises(capi.HipError):
+        z.set(np.zeros(5, np.int32))                # "input buffer is the wrong length."
+    allocs0 = C.c_size_t()
+    lib.dopt_hip_pool_stats(None, None, C.byref(allocs0))
+    ptr = z.ptr
+    z.free()
+    z2 = ops.Tensor((4097,), np.int32)
+    allocs1 = C.c_size_t()
+    lib.dopt_hip_pool_stats(None, None, C.byref(allocs1))
+    assert z2.ptr == ptr and allocs1.value == allocs0.value   # served from the pool
+    assert not z2.numpy().any()
+
+
+# ----------------------------------------------------------------------------- pointwise
+@pytest.mark.parametrize("n", [1, 3, 4, 1023, 4096, 100003, 1 << 20])
+def test_pointwise_f32_exact(n):
+    r = rng(n)
+    a = (r.standard_normal(n) * 5).astype(np.float32)
+    b = (r.standard_normal(n) * 3).astype(np.float32)
+    b[::13] = a[::13]
+    ta, tb = T(a), T(b)
+    for op in ["add", "sub", "mul", "div", "lt", "lte", "gt", "gte", "eq", "neq", "max", "min"]:
+        assert np.array_equal(ops.pointwise(op, ta, tb).numpy(), O.pointwise(op, a, b)), op
+    for op in ["neg", "abs", "sgn"]:
+        assert np.array_equal(ops.pointwise(op, ta).numpy(), O.pointwise(op, a)), op
+    pa = np.abs(a)
+    assert np.array_equal(ops.pointwise("sqrt", T(pa)).numpy(), O.pointwise("sqrt", pa))
+
+
+def test_pointwise_f32_transcendentals_within_2ulp():
+    r = rng(5)
+    n = 200001
+    x = (r.standard_normal(n) * 4).astype(np.float32)
+    p = (np.abs(x) + 1e-3).astype(np.float32)
+    e = r.standard_normal(n).astype(np.float32)
+    small = (r.uniform(-0.99, 0.99, n)).astype(np.float32)
+    cases = [("exp", x, None), ("log", p, None), ("pow", p, e), ("sin", x, None), ("cos", x, None),
+             ("tanh", x, None), ("atan", x, None), ("atan2", x, e), ("asin", small, None), ("sinh", x, None)]
+    for op, a, b in cases:
+        got = ops.pointwise(op, T(a), T(b) if b is not None else None).numpy()
+        want = O.pointwise(op, a, b)
+        assert ulp_diff(got, want).max() <= 2, (op, ulp_diff(got, want).max())
+
+
+def test_pointwise_unaligned_views_take_the_scalar_path():
+    a = rng(1).standard_normal(1001).astype(np.float32)
+    b = rng(2).standard_normal(1001).astype(np.float32)
+    ta, tb = T(a), T(b)
+    va, vb = ta.view(1, (1000,)), tb.view(1, (1000,))
+    assert np.array_equal(ops.pointwise("mul", va, vb).numpy(), a[1:] * b[1:])
+
+
+def test_pointwise_i32():
+    r = rng(3)
+    n = 10007
+    a = r.integers(-1000, 1000, n).astype(np.int32)
+    b = (r.integers(1, 50, n) * r.choice([-1, 1], n)).astype(np.int32)
+    ta, tb = T(a), T(b)
+    for op in ["add", "sub", "mul", "div", "lt", "lte", "gt", "gte", "eq", "neq", "max", "min"]:
+        got = ops.pointwise(op, ta, tb)
+        assert got.dtype == np.int32
+        assert np.array_equal(got.numpy(), O.pointwise(op, a, b)), op
+    for op in ["neg", "abs", "sgn"]:
+        assert np.array_equal(ops.pointwise(op, ta).numpy(), O.pointwise(op, a)), op
+    base, ex = r.integers(-6, 7, n).astype(np.int32), r.integers(0, 8, n).astype(np.int32)
+    assert np.array_equal(ops.pointwise("pow", T(base), T(ex)).numpy(), O.pointwise("pow", base, ex))
+    pos = np.abs(a)
+    assert np.array_equal(ops.pointwise("sqrt", T(pos)).numpy(), O.pointwise("sqrt", pos))
+    big = np.array([2**31 - 1, -2**31], np.int32)
+    one = np.array([1, -1], np.int32)
+    assert np.array_equal(ops.pointwise("add", T(big), T(one)).numpy(), O.pointwise("add", big, one))
+
+
+def test_pointwise_rejects_bad_arity_and_names():
+    from dopt_amd import capi
+    a = T(np.ones(4, np.float32))
+    with pytest.raises(capi.HipError):
+        ops.pointwise("add", a)
+    with pytest.raises(capi.HipError):
+        ops.pointwise("bogus", a, a)
+
+
+# ----------------------------------------------------------------------------- reductions
+@pytest.mark.parametrize("shape,axes", [
+    ((128, 10), None), ((100, 10), None), ((7,), None), ((3, 4, 5), (1,)), ((3, 4, 5), (0, 2)),
+    ((2, 3, 4, 5), (1, 2)), ((2, 3, 4, 5), (3,)), ((2, 3, 4, 5), (0,)), ((640, 640, 3, 3), None),
+    ((5, 70000), (1,)), ((2048, 33), (1,)), ((4, 6), (0,)),
+])
+def test_sum_and_max(shape, axes):
+    r = rng(11)
+    x = r.standard_normal(shape).astype(np.float32)
+    red = int(np.prod([shape[a] for a in (axes or range(len(shape)))]))
+    got = ops.sum(T(x), axes).numpy()
+    want64 = x.astype(np.float64).sum(axis=tuple(axes) if axes else None)
+    assert got.shape == np.asarray(want64).shape
+    assert_close(got, want64, "sum", scale=np.sqrt(red))
+    if red <= 4096:  # the reference's own fp32 left-fold is itself within tolerance of the device result
+        assert_close(got, O.sum(x, axes), "sum vs reference order", scale=np.sqrt(red))
+    assert np.array_equal(ops.max_element(T(x), axes).numpy(), O.max_element(x, axes))
+    xi = r.integers(-1000, 1000, shape).astype(np.int32)
+    assert np.array_equal(ops.sum(T(xi), axes).numpy(), O.sum(xi, axes))
+    assert np.array_equal(ops.max_element(T(xi), axes).numpy(), O.max_element(xi, axes))
+
+
+def test_max_identity_is_minus_type_max():
+    x = np.full((3, 5), -2**31, np.int32)
+    assert np.array_equal(ops.max_element(T(x), (1,)).numpy(), O.max_element(x, (1,)))
+
+
+@pytest.mark.parametrize("shape,axis", [((5,), 0), ((2, 3), 1), ((2, 3), 0), ((4, 5, 6), 1), ((3, 1000), 1),
+                                        ((1000, 3), 0)])
+def test_argmin(shape, axis):
+    r = rng(12)
+    x = r.integers(-5, 5, shape).astype(np.float32)   # many ties: first minimum must win
+    got = ops.argmin(T(x), axis)
+    assert got.dtype == np.int32
+    assert np.array_equal(got.numpy(), O.argmin(x, axis))
+    xi = r.integers(-5, 5, shape).astype(np.int32)
+    assert np.array_equal(ops.argmin(T(xi), axis).numpy(), O.argmin(xi, axis))
+
+
+def test_argmin_all_max_lane_gives_zero():
+    x = np.full((2, 4), np.finfo(np.float32).max, np.float32)
+    assert np.array_equal(ops.argmin(T(x), 1).numpy(), O.argmin(x, 1))
+
+
+# ----------------------------------------------------------------------------- layout
+@pytest.mark.parametrize("shape", [(7,), (4, 6), (3, 4, 5), (2, 3, 4, 5), (33, 65), (8388608 // 64 + 128,)])
+def test_slice_pad_repeat(shape):
+    r = rng(21)
+    x = r.integers(-1000, 1000, shape).astype(np.int32)
+    tx = T(x)
+    for _ in range(3):
+        start = [int(r.integers(0, s)) for s in shape]
+        stop = [int(r.integers(a + 1, s + 1)) for a, s in zip(start, shape)]
+        assert np.array_equal(ops.slice(tx, start, stop).numpy(), O.slice(x, start, stop))
+        before = [int(r.integers(0, 3)) for _ in shape]
+        after = [int(r.integers(0, 3)) for _ in shape]
+        assert np.array_equal(ops.pad(tx, before, after).numpy(), O.pad(x, before, after))
+    if x.size < 5000:
+        reps = [int(r.integers(1, 4)) for _ in shape]
+        assert np.array_equal(ops.repeat(tx, reps).numpy(), O.repeat(x, reps))
+    # leading-axis slices are the batch-norm unpacking pattern (core/ops/nnet.d:484-488)
+    cut = shape[0] // 2
+    start, stop = [cut] + [0] * (len(shape) - 1), list(shape)
+    assert np.array_equal(ops.slice(tx, start, stop).numpy(), x[cut:])
+
+
+def test_slice_rejects_out_of_range():
+    from dopt_amd import capi
+    with pytest.raises(capi.HipError):
+        ops.slice(T(np.zeros((3, 3), np.float32)), [1, 1], [4, 3])
+
+
+@pytest.mark.parametrize("rows,cols", [(2, 2), (1, 9), (9, 1), (5, 9), (64, 64), (65, 130), (512, 512), (10, 784),
+                                       (1000, 3)])
+def test_transpose(rows, cols):
+    x = rng(22).standard_normal((rows, cols)).astype(np.float32)
+    assert np.array_equal(ops.transpose(T(x)).numpy(), O.transpose(x))
+
+
+# ----------------------------------------------------------------------------- matmul
+MM_SHAPES = [
+    (2, 2, 1), (100, 10, 784), (784, 10, 100), (100, 10, 1), (1000, 1, 1), (100, 1, 10),      # config 1
+    (256, 512, 784), (256, 512, 512), (256, 10, 512), (784, 512, 256), (256, 784, 512),        # config 2
+    (128, 512, 512), (128, 10, 512), (128, 512, 1), (1, 512, 128), (512, 512, 128),            # VGG head
+    (81920, 1, 64), (2359296, 1, 1),                                                           # WRN mean pool, scalar broadcast
+    (7, 5, 3), (33, 65, 129), (130, 258, 70), (64, 256, 16), (65, 3, 200), (1, 17, 40), (19, 1, 23), (300, 300, 300),
+]
+
+
+@pytest.mark.parametrize("M,N,K", MM_SHAPES)
+def test_matmul(M, N, K):
+    r = rng(M * 31 + N * 7 + K)
+    a = r.standard_normal((M, K)).astype(np.float32)
+    b = r.standard_normal((K, N)).astype(np.float32)
+    got = ops.matmul(T(a), T(b)).numpy()
+    if K == 1:
+        assert np.array_equal(got, a * b.reshape(1, N))      # a single rounding: exact
+        return
+    want = O.matmul(a, b, f64=True) if M * N * K < 5e8 else (a.astype(np.float64) @ b.astype(np.float64))
+    assert_close(got, want, "matmul %dx%dx%d" % (M, N, K), scale=np.sqrt(K))
+
+
+def test_matmul_broadcast_by_ones_is_exact():
+    # core/ops/basic.d:370-381: repeat(n) = ones[n,1] . x[1,vol]; scalars broadcast the same way
+    x = rng(31).standard_normal((1, 513)).astype(np.float32)
+    ones = np.ones((77, 1), np.float32)
+    assert np.array_equal(ops.matmul(T(ones), T(x)).numpy(), np.repeat(x, 77, axis=0))
+    s = np.array([[0.001]], np.float32)
+    col = np.ones((100003, 1), np.float32)
+    assert np.array_equal(ops.matmul(T(col), T(s)).numpy(), np.full((100003, 1), s[0, 0], np.float32))
+
+
+def test_matmul_rejects_int():
+    from dopt_amd import capi
+    with pytest.raises(capi.HipError):
+        ops.matmul(T(np.ones((2, 2), np.int32)), T(np.ones((2, 2), np.int32)))
+
+
+# ----------------------------------------------------------------------------- convolution
+CONV_CASES = [  # N, C, H, W, K, R, S, pad, stride
+    (2, 3, 8, 8, 4, 3, 3, (1, 1), (1, 1)),
+    (1, 2, 7, 9, 3, 3, 3, (0, 0), (1, 1)),
+    (2, 2, 9, 8, 3, 3, 3, (1, 1), (2, 2)),
+    (1, 3, 6, 6, 2, 1, 1, (0, 0), (2, 2)),
+    (1, 1, 5, 7, 2, 2, 3, (1, 2), (1, 2)),
+    (3, 16, 8, 8, 32, 3, 3, (1, 1), (1, 1)),
+    (2, 20, 6, 6, 70, 3, 3, (1, 1), (1, 1)),      # channel counts that are not tile multiples
+    (4, 3, 32, 32, 64, 3, 3, (1, 1), (1, 1)),     # VGG conv1 shape at batch 4
+    (2, 64, 32, 32, 64, 3, 3, (1, 1), (1, 1)),    # VGG conv2
+    (2, 64, 16, 16, 128, 3, 3, (1, 1), (1, 1)),   # VGG conv3
+    (8, 256, 4, 4, 512, 3, 3, (1, 1), (1, 1)),    # VGG conv8: split reduction
+    (16, 512, 2, 2, 512, 3, 3, (1, 1), (1, 1)),   # VGG conv11-13
+    (2, 16, 32, 32, 160, 1, 1, (0, 0), (1, 1)),   # WRN 1x1 shortcut
+    (2, 160, 32, 32, 320, 3, 3, (1, 1), (2, 2)),  # WRN stage entry, stride 2
+    (2, 160, 32, 32, 320, 1, 1, (0, 0), (2, 2)),  # WRN strided shortcut
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_convolution_all_three(case):
+    N, C, H, W, K, R, S, pad, st = case
+    r = rng(hash(case) % 1000)
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+    w = (r.standard_normal((K, C, R, S)) * np.sqrt(2.0 / (C * R * S))).astype(np.float32)
+    y_ref = O.convolution(x, w, pad, st)
+    y = ops.convolution(T(x), T(w), pad, st)
+    assert y.shape == y_ref.shape
+    assert_close(y.numpy(), y_ref, "conv fwd", scale=1.0)
+    dy = r.standard_normal(y_ref.shape).astype(np.float32)
+    dx = ops.conv_bwd_data(T(dy), T(w), x.shape, pad, st).numpy()
+    assert_close(dx, O.conv_bwd_data(dy, w, x.shape, pad, st), "conv bwd-data", scale=1.0)
+    dw = ops.conv_bwd_filter(T(dy), T(x), w.shape, pad, st).numpy()
+    npix = N * y_ref.shape[2] * y_ref.shape[3]
+    assert_close(dw, O.conv_bwd_filter(dy, x, w.shape, pad, st), "conv bwd-filter", scale=np.sqrt(npix))
+
+
+def test_convolution_matches_reference_cpu_kernel_on_same_shapes():
+    # the reference CPU kernel (fp32, its own loop order) is a valid oracle when out dims == in dims
+    r = rng(41)
+    x = r.standard_normal((2, 8, 8, 8)).astype(np.float32)
+    w = r.standard_normal((4, 8, 3, 3)).astype(np.float32)
+    got = ops.convolution(T(x), T(w), (1, 1), (1, 1)).numpy()
+    assert_close(got, O.convolution(x, w, (1, 1), (1, 1), f64=False), "conv vs cpu kernel", scale=np.sqrt(72))
+
+
+# ----------------------------------------------------------------------------- pooling / softmax / relu / bias
+@pytest.mark.parametrize("shape,dims", [((1, 1, 4, 4), (2, 2)), ((2, 3, 6, 9), (2, 3)), ((2, 3, 5, 5), (2, 2)),
+                                        ((4, 64, 32, 32), (2, 2)), ((4, 512, 2, 2), (2, 2)), ((2, 3, 8, 6), (2, 2)),
+                                        ((2, 2, 8, 8), (4, 2))])
+def test_maxpool_and_grad(shape, dims):
+    r = rng(51)
+    x = r.integers(-3, 4, shape).astype(np.float32)    # ties everywhere: the tie rule is exercised
+    y_ref = O.maxpool(x, dims)
+    assert np.array_equal(ops.maxpool(T(x), dims).numpy(), y_ref)
+    dy = r.standard_normal(y_ref.shape).astype(np.float32)
+    assert np.array_equal(ops.maxpool_grad(T(dy), T(x), dims).numpy(), O.maxpool_grad(dy, x, dims))
+
+
+@pytest.mark.parametrize("shape", [(1, 5), (128, 10), (256, 10), (4, 7, 3), (3, 5, 2, 2)])
+def test_softmax_and_grad(shape):
+    r = rng(52)
+    x = (r.standard_normal(shape) * 3).astype(np.float32)
+    got = ops.softmax(T(x)).numpy()
+    assert ulp_diff(got, O.softmax(x)).max() <= 4          # same loop order; expf differs by <= 2 ulp
+    assert_close(got, O.softmax(x, f64=True), "softmax")
+    y = O.softmax(x, f64=True)
+    dy = r.standard_normal(shape).astype(np.float32)
+    assert_close(ops.softmax_grad(T(dy), T(y)).numpy(), O.softmax_grad(dy, y), "softmax grad")
+
+
+@pytest.mark.parametrize("n", [1, 5, 4096, 100003])
+def test_relu(n):
+    r = rng(53)
+    x = r.standard_normal(n).astype(np.float32)
+    x[::7] = 0.0
+    if n > 2:
+        x[2] = np.nan
+    dy = r.standard_normal(n).astype(np.float32)
+    got = ops.relu(T(x)).numpy()
+    assert ulp_diff(got, O.relu(x)).max() == 0
+    assert np.array_equal(ops.relu_grad(T(dy), T(x)).numpy(), O.relu_grad(dy, x))
+
+
+@pytest.mark.parametrize("shape", [(4, 64, 32, 32), (3, 5, 4, 2), (6, 5), (128, 512, 2, 2), (2, 7, 3, 3),
+                                   (64, 256, 8, 8)])
+def test_bias(shape):
+    r = rng(54)
+    x = r.standard_normal(shape).astype(np.float32)
+    b = r.standard_normal(shape[1]).astype(np.float32)
+    assert np.array_equal(ops.add_bias(T(x), T(b)).numpy(), O.add_bias(x, b))
+    red = x.size // shape[1]
+    assert_close(ops.add_bias_grad(T(x)).numpy(), O.add_bias_grad(x), "bias grad", scale=np.sqrt(red))
+
+
+# ----------------------------------------------------------------------------- batch norm
+@pytest.mark.parametrize("shape", [(4, 3, 5, 5), (8, 6), (2, 4, 3, 1), (8, 64, 32, 32), (128, 512, 2, 2), (3, 2),
+                                   (16, 16, 16, 16)])
+def test_batchnorm_train_grad_infer(shape):
+    r = rng(61)
+    C = shape[1]
+    x = (r.standard_normal(shape) * 2 + 3).astype(np.float32)    # mean well away from 0
+    gamma = r.standard_normal(C).astype(np.float32)
+    beta = r.standard_normal(C).astype(np.float32)
+    rm = r.standard_normal(C).astype(np.float32)
+    rv = (r.random(C) + 0.5).astype(np.float32)
+    dy = r.standard_normal(shape).astype(np.float32)
+    mom = float(np.float32(0.9))
+    vol = x.size
+    m = vol // C
+    got = ops.bn_train(T(x), T(gamma), T(beta), T(rm), T(rv), mom).numpy()
+    want = O.bn_train(x, gamma, beta, rm, rv, mom)
+    assert got.shape == (vol + 2 * C,)
+    assert_close(got[:vol], want[:vol], "bn y")
+    assert_close(got[vol:], want[vol:], "bn running stats")
+    g = ops.bn_grad(T(dy), T(x), T(gamma)).numpy()
+    gw = O.bn_grad(dy, x, gamma)
+    assert_close(g[:vol], gw[:vol], "bn dx")
+    assert_close(g[vol:], gw[vol:], "bn dscale/dbias", scale=np.sqrt(m))
+    assert_close(ops.bn_infer(T(x), T(gamma), T(beta), T(rm), T(rv)).numpy(), O.bn_infer(x, gamma, beta, rm, rv),
+                 "bn infer")
+
+
+def test_batchnorm_large_mean_small_variance():
+    # E[x^2] - E[x]^2 would lose everything here; the shifted moments must not
+    r = rng(62)
+    x = (1000.0 + r.standard_normal((64, 8, 16, 16)) * 0.01).astype(np.float32)
+    ones, zeros = np.ones(8, np.float32), np.zeros(8, np.float32)
+    got = ops.bn_train(T(x), T(ones), T(zeros), T(zeros), T(ones), 0.9).numpy()
+    want = O.bn_train(x, ones, zeros, zeros, ones, 0.9)
+    assert_close(got[:x.size], want[:x.size], "bn y, ill-conditioned", rtol=2e-3, atol=2e-3)
+    assert_close(got[x.size + 8:], want[x.size + 8:], "running var", rtol=1e-3)
+
+
+# ----------------------------------------------------------------------------- optimizers
+def _opt_state(r, sizes):
+    w = [r.standard_normal(n).astype(np.float32) for n in sizes]
+    g = [(r.standard_normal(n) * 0.1).astype(np.float32) for n in sizes]
+    m = [(r.standard_normal(n) * 0.1).astype(np.float32) for n in sizes]
+    v = [np.abs(r.standard_normal(n) * 0.01).astype(np.float32) for n in sizes]
+    vh = [np.abs(r.standard_normal(n) * 0.01).astype(np.float32) for n in sizes]
+    return w, g, m, v, vh
+
+
+OPT_SIZES = [1, 3, 4096, 4097, 10, 100003, 8192, 512]
+
+
+@pytest.mark.parametrize("nesterov", [False, True])
+def test_fused_sgd_is_bit_exact(nesterov):
+    w, g, m, _, _ = _opt_state(rng(71), OPT_SIZES)
+    tw, tg, tm = [T(a) for a in w], [T(a) for a in g], [T(a) for a in m]
+    opt = ops.FusedOptimizer(tw, tg, tm)
+    for step in range(2):
+        opt.sgd(0.01, 0.9, nesterov)
+        for i in range(len(w)):
+            w[i], m[i] = O.sgd_step(w[i], g[i], m[i], 0.01, 0.9, nesterov)
+    for i in range(len(w)):
+        assert np.array_equal(tw[i].numpy(), w[i]) and np.array_equal(tm[i].numpy(), m[i]), i
+
+
+@pytest.mark.parametrize("rule", ["adam", "amsgrad"])
+def test_fused_adam_amsgrad_are_bit_exact(rule):
+    w, g, m, v, vh = _opt_state(rng(72), OPT_SIZES)
+    skip = [False] * len(w)
+    skip[2] = True                                   # a projected parameter: w untouched, moments still updated
+    w2_before = w[2].copy()
+    tw, tg, tm, tv, tvh = ([T(a) for a in lst] for lst in (w, g, m, v, vh))
+    opt = ops.FusedOptimizer(tw, tg, tm, tv, tvh if rule == "amsgrad" else None, skip)
+    b1 = b2 = 1.0
+    for step in range(3):
+        getattr(opt, rule)(1e-3, 0.9, 0.999, 1e-8)
+        b1, b2, eta = O.adam_scalars(1e-3, 0.9, 0.999, b1, b2)
+        for i in range(len(w)):
+            if rule == "adam":
+                w[i], m[i], v[i] = O.adam_step(w[i], g[i], m[i], v[i], eta)
+            else:
+                w[i], m[i], v[i], vh[i] = O.amsgrad_step(w[i], g[i], m[i], v[i], vh[i], eta)
+    assert opt.b1.value == np.float32(b1) and opt.b2.value == np.float32(b2)
+    for i in range(len(w)):
+        want_w = w2_before if skip[i] else w[i]
+        assert np.array_equal(tw[i].numpy(), want_w), ("w", i)
+        assert np.array_equal(tm[i].numpy(), m[i]), ("m", i)
+        assert np.array_equal(tv[i].numpy(), v[i]), ("v", i)
+        if rule == "amsgrad":
+            assert np.array_equal(tvh[i].numpy(), vh[i]), ("vhat", i)

@@ -1,0 +1,31 @@
+import numpy as np
+
+
+def ulp_diff(a, b):
+    """Distance in units in the last place between two float32 arrays (NaN pairs count as 0)."""
+    a = np.asarray(a, np.float32)
+    b = np.asarray(b, np.float32)
+    both_nan = np.isnan(a) & np.isnan(b)
+    ai = a.view(np.int32).astype(np.int64)
+    bi = b.view(np.int32).astype(np.int64)
+    ai = np.where(ai < 0, -(ai & 0x7FFFFFFF), ai)
+    bi = np.where(bi < 0, -(bi & 0x7FFFFFFF), bi)
+    d = np.abs(ai - bi)
+    return np.where(both_nan, 0, d)
+
+
+# north_star tolerances
+GEMM_RTOL, GEMM_ATOL = 1e-4, 1e-5
+
+
+def assert_close(got, want, what="", rtol=GEMM_RTOL, atol=GEMM_ATOL, scale=None):
+    """|got - want| <= atol*scale + rtol*|want|.  `scale` rescales atol for reductions whose terms
+    are far from O(1) (a length-n dot product of N(0,1) terms has magnitude sqrt(n))."""
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    tol = atol * (scale if scale else 1.0) + rtol * np.abs(want)
+    bad = np.abs(got - want) > tol
+    if bad.any():
+        i = np.argmax(np.abs(got - want) - tol)
+        raise AssertionError("%s: %d/%d outside tolerance; worst at %d: got %r want %r" %
+                             (what, bad.sum(), bad.size, i, got.ravel()[i], want.ravel()[i]))
