@@ -1,0 +1,181 @@
+#!/usr/bin/env python3
+"""Headline benchmark: one full training step (forward + backward + SGD update) of the VGG-16-style
+CIFAR-shape network with batch norm at batch 128 in fp32, on one MI355X, through HIPPlan and the
+kernel library.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--unfused] [--no-views] [--no-cpu]
+
+A step is one execution of the update plan on device-resident synthetic inputs (inputs are in
+HBM before the timed region starts).  After the timed region the same step is run again with
+per-kernel HIP events (on the library's stream) to measure the convolution kernels against the
+fp32 MFMA roofline, and the reference's CPU convolution (this repository's C restatement of it)
+is timed on the host cores as the reported CPU baseline.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+BATCH = 128
+MFMA_FP32_PEAK_TFLOPS = 157.3
+HBM_PEAK_GBS = 8000.0
+
+# (C, K, H) of the 13 VGG-16 3x3 pad-1 convolutions on a 32x32 input
+VGG_CONVS = [(3, 64, 32), (64, 64, 32), (64, 128, 16), (128, 128, 16), (128, 256, 8), (256, 256, 8), (256, 256, 8),
+             (256, 512, 4), (512, 512, 4), (512, 512, 4), (512, 512, 2), (512, 512, 2), (512, 512, 2)]
+
+
+def conv_flops(n, c, k, h):
+    return 2.0 * n * k * c * 9 * h * h
+
+
+def build_step(batch, fused, views, timing, seed=0):
+    from dopt_amd import core, nnet, online, ops
+    rng = np.random.default_rng(seed)
+    features = core.float32([batch, 3, 32, 32])
+    labels = core.float32([batch, 10])
+    init = nnet.Init(seed + 1)
+    preds = nnet.softmax(nnet.dense(nnet.vgg16(features, [512, 512], init), 10, init))
+    net = nnet.DAGNetwork([features], [preds])
+    loss = nnet.crossEntropy(preds.trainOutput, labels) + net.paramLoss
+    flags = (core.PLAN_VIEWS if views else 0) | (core.PLAN_TIMING if timing else 0)
+    if fused:
+        updater = online.fused_sgd([loss, preds.trainOutput], net.params, net.paramProj, 0.01, 0.0, flags=flags)
+    else:
+        updater = online.sgd([loss, preds.trainOutput], net.params, net.paramProj, flags=flags)
+    x = rng.standard_normal((batch, 3, 32, 32)).astype(np.float32)
+    y = np.zeros((batch, 10), np.float32)
+    y[np.arange(batch), rng.integers(0, 10, batch)] = 1.0
+    args = {features: ops.tensor(x), labels: ops.tensor(y)}   # resident in HBM before timing starts
+    return updater, args, net
+
+
+def cpu_baseline(seconds_budget=20.0):
+    """The reference's CPU convolution kernel (cpu/source/dopt/cpu/nnet.d:20-87, single-threaded
+    direct loops; the reference CPU backend has no backward or batch-norm kernels at all) over the
+    13 VGG layers at a small batch, expressed as images/s of conv-forward alone."""
+    import oracle as O
+    rng = np.random.default_rng(0)
+    b = 1
+    t_total = 0.0
+    # calibrate on batch 1, then spend the remaining budget on one larger batch
+    for attempt in range(2):
+        t0 = time.perf_counter()
+        for (c, k, h) in VGG_CONVS:
+            x = rng.standard_normal((b, c, h, h)).astype(np.float32)
+            w = rng.standard_normal((k, c, 3, 3)).astype(np.float32)
+            O.convolution(x, w, (1, 1), (1, 1), f64=False)
+        t_total = time.perf_counter() - t0
+        if attempt == 0:
+            nb = int(max(1, min(32, (seconds_budget - t_total) / max(t_total, 1e-3))))
+            if nb == b:
+                break
+            b = nb
+    return {"value": round(b / t_total, 3), "unit": "images/s", "cores": 1, "kind": "port",
+            "sample": "conv-forward only: the 13 VGG-16 3x3 convolutions at batch %d through the C restatement of "
+                      "the reference's single-threaded CPU kernel (%.1f s); the reference CPU backend implements no "
+                      "backward, bias, ReLU or batch-norm kernels, so a full CPU training step does not exist" % (
+                          b, t_total)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--unfused", action="store_true", help="run the reference's op-graph SGD instead of the fused kernel")
+    ap.add_argument("--no-views", action="store_true", help="disable the copy-eliding plan rewrites")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-kernel-timing", action="store_true", help="skip the per-kernel event pass")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build drives one GPU per process and implements no collectives; run with --gpus 1")
+
+    from dopt_amd import capi, ops
+    capi.check(capi.load().dopt_hip_init(0))
+    fused, views = not a.unfused, not a.no_views
+
+    updater, args, net = build_step(BATCH, fused, views, timing=False)
+    for _ in range(a.warmup):
+        updater.step_async(args)
+    ops.sync()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        updater.step_async(args)
+    ops.sync()
+    elapsed = time.perf_counter() - t0
+    loss = float(updater._out_bufs[0].numpy())
+    ms_per_step = elapsed / a.steps * 1e3
+    stats = updater.plan.stats()
+
+    result = {
+        "metric": "train images/sec, VGG-16 CIFAR-shape fp32 b128",
+        "value": round(BATCH / (elapsed / a.steps), 2),
+        "unit": "images/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "config 4: VGG-16 + batch norm, input [128,3,32,32], FC 512-512-10, softmax "
+                               "cross-entropy, one forward + backward + SGD(lr 0.01) step",
+                   "global_batch": BATCH, "optimizer": "fused multi-tensor SGD" if fused else "op-graph SGD",
+                   "plan_rewrites": "views" if views else "none",
+                   "kernels_per_step": stats["kernels"] + (1 if fused else 0),
+                   "plan_buffer_MB": round(stats["buffer_bytes"] / 2**20, 1),
+                   "parameters": int(sum(p.volume for p in net.params)), "loss_after": round(loss, 5)},
+    }
+    if not np.isfinite(loss):
+        sys.exit("bench.py: the loss is not finite (%r)" % loss)
+
+    if not a.no_kernel_timing:
+        # Same step, every kernel object bracketed by hipEvents on the library stream.
+        del updater
+        tup, targs, _ = build_step(BATCH, fused, views, timing=True)
+        for _ in range(2):
+            tup.step_async(targs)
+        ops.sync()
+        before = tup.plan.profile()
+        nsteps = max(3, min(a.steps, 10))
+        for _ in range(nsteps):
+            tup.step_async(targs)
+        ops.sync()
+        after = tup.plan.profile()
+        per_step = {k: ((after[k][0] - before.get(k, (0, 0))[0]) / nsteps, (after[k][1] - before.get(k, (0, 0))[1]) // nsteps)
+                    for k in after}
+        fwd = sum(conv_flops(BATCH, c, k, h) for c, k, h in VGG_CONVS)
+        bwd_data = fwd - conv_flops(BATCH, *VGG_CONVS[0])   # the first layer's input needs no gradient
+        gather_us = per_step["convolution"][0] + per_step["convolutionFeaturesGrad"][0]
+        gather_launches = per_step["convolution"][1] + per_step["convolutionFeaturesGrad"][1]
+        gather_tflops = (fwd + bwd_data) / (gather_us * 1e-6) / 1e12
+        wgrad_tflops = fwd / (per_step["convolutionFiltersGrad"][0] * 1e-6) / 1e12
+        result["roofline"] = {
+            "kernel": "conv_gather_k (implicit-GEMM convolution forward + backward-data)",
+            "bound": "mfma", "achieved": round(gather_tflops, 2), "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(gather_tflops / MFMA_FP32_PEAK_TFLOPS, 4), "traffic": None,
+            "launches_per_step": int(gather_launches),
+            "flops_per_launch": round((fwd + bwd_data) / gather_launches, 1),
+            "avg_launch_us": round(gather_us / gather_launches, 2),
+        }
+        result["kernels"] = {
+            "conv_wgrad_k": {"achieved_TFLOPs": round(wgrad_tflops, 2),
+                             "frac_of_mfma_peak": round(wgrad_tflops / MFMA_FP32_PEAK_TFLOPS, 4),
+                             "us_per_step": round(per_step["convolutionFiltersGrad"][0], 1)},
+            "device_us_per_step_by_op": {k: round(v[0], 1) for k, v in sorted(per_step.items(), key=lambda kv: -kv[1][0])},
+            "device_us_per_step_total": round(sum(v[0] for v in per_step.values()), 1),
+        }
+        del tup
+
+    if not a.no_cpu:
+        result["cpu_baseline"] = cpu_baseline()
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

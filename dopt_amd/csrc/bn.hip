@@ -23,11 +23,11 @@ struct Coef {  // one per channel, 16 bytes
     float mean;  // batch (or running) mean
     float a;     // scale * rstd
     float b;     // bias
-    float d;     // train/infer: rstd (informational)
+    float mean_lo;  // mean - (float)mean: keeps x - mean accurate when |mean| >> std
 };
 struct CoefG {   // grad: a = scale * rstd, b = dbias / m, d = dscale / m
-    float mean, rstd, a, b, d;
-    float pad[3];
+    float mean, rstd, a, b, d, mean_lo;
+    float pad[2];
 };
 
 __device__ inline float wave_sum(float v)
@@ -138,7 +138,7 @@ __global__ __launch_bounds__(kBlock) void bn_train_finalize_k(size_t N, size_t C
     k.mean = (float)mean;
     k.a = (float)((double)scale[c] * rstd);
     k.b = bias[c];
-    k.d = (float)rstd;
+    k.mean_lo = (float)(mean - (double)k.mean);
     coef[c] = k;
     double unbiased = m > 1.0 ? var * m / (m - 1.0) : var;
     new_mean[c] = (float)((1.0 - factor) * (double)run_mean[c] + factor * mean);
@@ -156,7 +156,7 @@ __global__ __launch_bounds__(kBlock) void bn_infer_prepare_k(size_t C, double ep
     k.mean = mean[c];
     k.a = (float)((double)scale[c] * rstd);
     k.b = bias[c];
-    k.d = (float)rstd;
+    k.mean_lo = 0.0f;
     coef[c] = k;
 }
 
@@ -190,13 +190,14 @@ __global__ __launch_bounds__(kBlock) void bn_grad_finalize_k(size_t N, size_t C,
     k.a = (float)((double)scale[c] * rstd);
     k.b = (float)(db / m);
     k.d = (float)(ds / m);
-    k.pad[0] = k.pad[1] = k.pad[2] = 0.0f;
+    k.mean_lo = (float)(mean - (double)k.mean);
+    k.pad[0] = k.pad[1] = 0.0f;
     coef[c] = k;
     dscale[c] = (float)ds;
     dbias[c] = (float)db;
 }
 
-// y = a * (x - mean) + b
+// y = a * ((x - mean) - mean_lo) + b
 template <typename IdxT, bool kVec>
 __global__ __launch_bounds__(kBlock) void bn_apply_k(IdxT total, IdxT C, IdxT inner, const float *x, const Coef *coef,
                                                       float *y)
@@ -222,10 +223,10 @@ __global__ __launch_bounds__(kBlock) void bn_apply_k(IdxT total, IdxT C, IdxT in
                 IdxT i = base + (IdxT)u * kBlock + threadIdx.x;
                 if (i < n4) {
                     float4 r;
-                    r.x = k[u].a * (v[u].x - k[u].mean) + k[u].b;
-                    r.y = k[u].a * (v[u].y - k[u].mean) + k[u].b;
-                    r.z = k[u].a * (v[u].z - k[u].mean) + k[u].b;
-                    r.w = k[u].a * (v[u].w - k[u].mean) + k[u].b;
+                    r.x = k[u].a * ((v[u].x - k[u].mean) - k[u].mean_lo) + k[u].b;
+                    r.y = k[u].a * ((v[u].y - k[u].mean) - k[u].mean_lo) + k[u].b;
+                    r.z = k[u].a * ((v[u].z - k[u].mean) - k[u].mean_lo) + k[u].b;
+                    r.w = k[u].a * ((v[u].w - k[u].mean) - k[u].mean_lo) + k[u].b;
                     y4[i] = r;
                 }
             }
@@ -233,7 +234,7 @@ __global__ __launch_bounds__(kBlock) void bn_apply_k(IdxT total, IdxT C, IdxT in
     } else {
         for (IdxT i = (IdxT)blockIdx.x * kBlock + threadIdx.x; i < total; i += (IdxT)gridDim.x * kBlock) {
             Coef k = coef[(i / inner) % C];
-            y[i] = k.a * (x[i] - k.mean) + k.b;
+            y[i] = k.a * ((x[i] - k.mean) - k.mean_lo) + k.b;
         }
     }
 }
@@ -241,7 +242,7 @@ __global__ __launch_bounds__(kBlock) void bn_apply_k(IdxT total, IdxT C, IdxT in
 // dx = a * (dy - b - xhat * d),  xhat = (x - mean) * rstd
 __device__ inline float bn_dx(const CoefG &k, float dy, float x)
 {
-    float xhat = (x - k.mean) * k.rstd;
+    float xhat = ((x - k.mean) - k.mean_lo) * k.rstd;
     return k.a * ((dy - k.b) - xhat * k.d);
 }
 

@@ -1,0 +1,912 @@
+// HIPBuffer, the kernel registry, the built-in kernel objects and HIPPlan: the host side of the
+// backend, mirroring cuda/source/dopt/cuda/package.d (registry :479-507, CUDABuffer :124-251,
+// CUDAPlan :261-433) and the kernel classes of cuda/source/dopt/cuda/{math,basic}.d and
+// cuda/source/dopt/cuda/nnet/cudnn7.d.  Every kernel object pulls shapes and attributes off its
+// Operation in its constructor and makes exactly one call into the kernel library in execute().
+//
+// Differences from the reference that keep results identical:
+//   - no device synchronisation after each kernel (one in-order stream);
+//   - a host argument is uploaded once per execution, not once per consumer (package.d:373-381);
+//   - buffers come from the pool, with no GC.collect() per allocation (package.d:141);
+//   - an operation without a registered kernel is an error instead of a silent host round trip
+//     (package.d:81-119): sum, maxElement, argmin and the trigonometric ops have device kernels;
+//   - optional rewrites (DOPT_HIP_PLAN_VIEWS) replace copies by aliases.
+#include "plan.h"
+
+#include <algorithm>
+#include <cstring>
+#include <functional>
+#include <set>
+
+#include "../../include/dopt_hip_plan.h"
+
+namespace dopt {
+
+Graph::~Graph()
+{
+    for (Operation &o : ops)
+        if (o.value) dopt_hip_free(o.value);
+}
+
+// ------------------------------------------------------------------------------- HIPBuffer
+
+std::unique_ptr<HIPBuffer> HIPBuffer::create(size_t numBytes)
+{
+    std::unique_ptr<HIPBuffer> b(new HIPBuffer());
+    if (numBytes == 0) return b;  // package.d:144-147
+    if (dopt_hip_malloc(&b->mPtr, numBytes) != DOPT_HIP_OK) return nullptr;
+    b->mNumBytes = numBytes;
+    return b;
+}
+
+HIPBuffer::~HIPBuffer()
+{
+    if (mPtr) dopt_hip_free(mPtr);
+}
+
+int HIPBuffer::set(const void *host, size_t bytes)
+{
+    if (bytes != mNumBytes) return fail(DOPT_HIP_ERR_INVALID, "input buffer is the wrong length.");
+    return dopt_hip_copy_h2d(mPtr, host, bytes);
+}
+
+int HIPBuffer::set(const HIPBuffer &other)
+{
+    if (other.mNumBytes != mNumBytes) return fail(DOPT_HIP_ERR_INVALID, "Mismatch in buffer size");
+    return dopt_hip_copy_d2d(mPtr, other.mPtr, mNumBytes);
+}
+
+int HIPBuffer::get(void *host, size_t bytes) const
+{
+    if (bytes != mNumBytes) return fail(DOPT_HIP_ERR_INVALID, "output buffer is the wrong length.");
+    return dopt_hip_copy_d2h(host, mPtr, bytes);
+}
+
+// ------------------------------------------------------------------------------- registry
+
+namespace {
+
+std::unordered_map<std::string, HIPKernelCtr> &kernelCtrs()
+{
+    static std::unordered_map<std::string, HIPKernelCtr> m;
+    return m;
+}
+
+using ExecFn = std::function<int(const std::vector<const void *> &, void *)>;
+
+class FnKernel : public HIPKernel {
+public:
+    explicit FnKernel(ExecFn fn) : mFn(std::move(fn)) {}
+    int execute(const std::vector<const void *> &inputs, const std::vector<size_t> &, void *output, size_t) override
+    {
+        return mFn(inputs, output);
+    }
+
+private:
+    ExecFn mFn;
+};
+
+std::unique_ptr<HIPKernel> make(ExecFn fn) { return std::unique_ptr<HIPKernel>(new FnKernel(std::move(fn))); }
+
+const std::vector<size_t> *sizes_attr(const Operation &op, const char *key)
+{
+    auto it = op.sizeAttrs.find(key);
+    if (it == op.sizeAttrs.end()) {
+        fail(DOPT_HIP_ERR_INVALID, "operation '%s' has no attribute '%s'", op.opType.c_str(), key);
+        return nullptr;
+    }
+    return &it->second;
+}
+
+bool need_deps(const Operation &op, size_t n)
+{
+    if (op.deps.size() == n) return true;
+    fail(DOPT_HIP_ERR_INVALID, "operation '%s' expects %zu dependencies, has %zu", op.opType.c_str(), n,
+         op.deps.size());
+    return false;
+}
+
+bool need_f32(const Operation &op)
+{
+    if (op.dtype == DOPT_HIP_F32) return true;
+    fail(DOPT_HIP_ERR_UNSUPPORTED, "Element type not supported.");  // cuda/math.d:237-240
+    return false;
+}
+
+// [N, C, prod(rest)] view used by the cuDNN descriptors (cudnn7.d:339-348, 416-418, 488-492)
+void nci(const std::vector<size_t> &shape, size_t *N, size_t *C, size_t *inner)
+{
+    *N = shape.size() > 0 ? shape[0] : 1;
+    *C = shape.size() > 1 ? shape[1] : 1;
+    *inner = 1;
+    for (size_t i = 2; i < shape.size(); i++) *inner *= shape[i];
+}
+
+dopt_hip_conv_desc conv_desc(const std::vector<size_t> &x, const std::vector<size_t> &w, const std::vector<size_t> &pad,
+                             const std::vector<size_t> &stride)
+{
+    dopt_hip_conv_desc d{};
+    d.N = x[0]; d.C = x[1]; d.H = x[2]; d.W = x[3];
+    d.K = w[0]; d.R = w[2]; d.S = w[3];
+    d.padH = pad[0]; d.padW = pad[1]; d.strideH = stride[0]; d.strideW = stride[1];
+    return d;
+}
+
+bool rank4(const std::vector<size_t> &s, const char *what)
+{
+    if (s.size() == 4) return true;
+    fail(DOPT_HIP_ERR_INVALID, "%s must have rank 4", what);
+    return false;
+}
+
+std::unique_ptr<HIPKernel> pointwiseCtr(const Graph &g, int id)
+{
+    const Operation &op = g.ops[id];
+    std::string name = op.opType;
+    const size_t n = op.volume();
+    const int dtype = op.dtype;
+    const size_t arity = op.deps.size();
+    if (arity != 1 && arity != 2) {
+        fail(DOPT_HIP_ERR_INVALID, "pointwise operation '%s' with %zu dependencies", name.c_str(), arity);
+        return nullptr;
+    }
+    return make([=](const std::vector<const void *> &in, void *out) {
+        return dopt_hip_pointwise(name.c_str(), dtype, n, in[0], arity == 2 ? in[1] : nullptr, out);
+    });
+}
+
+void registerBuiltinsOnce()
+{
+    auto &R = kernelCtrs();
+    // cuda/math.d:89-92 plus the ops the reference leaves to its host fallback (core/ops/math.d:75-76)
+    for (const char *name : {"add", "sub", "mul", "div", "lt", "lte", "gt", "gte", "eq", "neq", "max", "min", "pow",
+                             "atan2", "neg", "abs", "sgn", "exp", "log", "sqrt", "sin", "cos", "tan", "asin", "acos",
+                             "atan", "sinh", "cosh", "tanh", "asinh", "acosh", "atanh"})
+        R[name] = pointwiseCtr;
+
+    // cuda/math.d:214-247
+    R["matmul"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];
+        if (!need_deps(op, 2) || !need_f32(op)) return nullptr;
+        const auto &a = g.ops[op.deps[0]].shape, &b = g.ops[op.deps[1]].shape;
+        if (a.size() != 2 || b.size() != 2 || a[1] != b[0]) {
+            fail(DOPT_HIP_ERR_INVALID, "matmul: operands must be rank 2 with matching inner dimension");
+            return nullptr;
+        }
+        const size_t M = a[0], K = a[1], N = b[1];
+        return make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_sgemm(M, N, K, (const float *)in[0], (const float *)in[1], (float *)out);
+        });
+    };
+
+    // cpu/math.d:90-247 (host fallback in the reference)
+    for (const char *name : {"sum", "maxElement"})
+        R[name] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+            const Operation &op = g.ops[id];
+            if (!need_deps(op, 1)) return nullptr;
+            const auto *axes = sizes_attr(op, "axes");
+            if (!axes) return nullptr;
+            std::vector<size_t> shape = g.ops[op.deps[0]].shape, ax = *axes;
+            std::string name = op.opType;
+            const int dtype = op.dtype;
+            return make([=](const std::vector<const void *> &in, void *out) {
+                return dopt_hip_reduce(name.c_str(), dtype, shape.data(), (int)shape.size(), ax.data(), (int)ax.size(),
+                                       in[0], out);
+            });
+        };
+    R["argmin"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];
+        if (!need_deps(op, 1)) return nullptr;
+        const auto *axis = sizes_attr(op, "axis");
+        if (!axis || axis->size() != 1) return nullptr;
+        std::vector<size_t> shape = g.ops[op.deps[0]].shape;
+        const size_t ax = (*axis)[0];
+        const int dtype = g.ops[op.deps[0]].dtype;
+        return make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_argmin(dtype, shape.data(), (int)shape.size(), ax, in[0], (int32_t *)out);
+        });
+    };
+
+    // cuda/basic.d:31-247
+    R["slice"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];
+        if (!need_deps(op, 1)) return nullptr;
+        const auto *start = sizes_attr(op, "start");
+        if (!start) return nullptr;
+        std::vector<size_t> in = g.ops[op.deps[0]].shape, out = op.shape, st = *start;
+        return make([=](const std::vector<const void *> &i, void *o) {
+            return dopt_hip_slice((int)in.size(), in.data(), out.data(), st.data(), i[0], o);
+        });
+    };
+    R["pad"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];
+        if (!need_deps(op, 1)) return nullptr;
+        const auto *before = sizes_attr(op, "before");
+        if (!before) return nullptr;
+        std::vector<size_t> in = g.ops[op.deps[0]].shape, out = op.shape, bf = *before;
+        return make([=](const std::vector<const void *> &i, void *o) {
+            return dopt_hip_pad((int)in.size(), in.data(), out.data(), bf.data(), i[0], o);
+        });
+    };
+    R["repeat"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];
+        if (!need_deps(op, 1)) return nullptr;
+        const auto *reps = sizes_attr(op, "repetitions");
+        if (!reps) return nullptr;
+        std::vector<size_t> in = g.ops[op.deps[0]].shape, rp = *reps;
+        return make([=](const std::vector<const void *> &i, void *o) {
+            return dopt_hip_repeat((int)in.size(), in.data(), rp.data(), i[0], o);
+        });
+    };
+    R["transpose"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];
+        if (!need_deps(op, 1)) return nullptr;
+        const auto *order = sizes_attr(op, "order");
+        if (!order) return nullptr;
+        const auto &in = g.ops[op.deps[0]].shape;
+        if (in.size() > 2) {
+            fail(DOPT_HIP_ERR_UNSUPPORTED, "transpose is only implemented for rank <= 2");  // cpu/basic.d:120
+            return nullptr;
+        }
+        const bool swap = in.size() == 2 && (*order)[0] == 1;
+        const size_t rows = in.size() == 2 ? in[0] : 1, cols = in.size() == 2 ? in[1] : op.volume();
+        const size_t bytes = op.bytes();
+        return make([=](const std::vector<const void *> &i, void *o) {
+            if (!swap) return dopt_hip_copy_d2d(o, i[0], bytes);
+            return dopt_hip_transpose2d(rows, cols, i[0], o);
+        });
+    };
+
+    // cuda/nnet/cudnn7.d:113-249
+    R["convolution"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];
+        if (!need_deps(op, 2) || !need_f32(op)) return nullptr;
+        const auto *pad = sizes_attr(op, "padding"), *stride = sizes_attr(op, "stride");
+        const auto &x = g.ops[op.deps[0]].shape, &w = g.ops[op.deps[1]].shape;
+        if (!pad || !stride || !rank4(x, "convolution features") || !rank4(w, "convolution filters")) return nullptr;
+        dopt_hip_conv_desc d = conv_desc(x, w, *pad, *stride);
+        return make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_conv_fwd(&d, (const float *)in[0], (const float *)in[1], (float *)out);
+        });
+    };
+    R["convolutionFeaturesGrad"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];  // deps [parentGrad, filters]; output = features shape (cudnn7.d:167-169)
+        if (!need_deps(op, 2) || !need_f32(op)) return nullptr;
+        const auto *pad = sizes_attr(op, "padding"), *stride = sizes_attr(op, "stride");
+        const auto &w = g.ops[op.deps[1]].shape;
+        if (!pad || !stride || !rank4(op.shape, "convolutionFeaturesGrad output") || !rank4(w, "filters")) return nullptr;
+        dopt_hip_conv_desc d = conv_desc(op.shape, w, *pad, *stride);
+        return make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_conv_bwd_data(&d, (const float *)in[0], (const float *)in[1], (float *)out);
+        });
+    };
+    R["convolutionFiltersGrad"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];  // deps [parentGrad, features]; output = filters shape (cudnn7.d:212-214)
+        if (!need_deps(op, 2) || !need_f32(op)) return nullptr;
+        const auto *pad = sizes_attr(op, "padding"), *stride = sizes_attr(op, "stride");
+        const auto &x = g.ops[op.deps[1]].shape;
+        if (!pad || !stride || !rank4(x, "features") || !rank4(op.shape, "convolutionFiltersGrad output")) return nullptr;
+        dopt_hip_conv_desc d = conv_desc(x, op.shape, *pad, *stride);
+        return make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_conv_bwd_filter(&d, (const float *)in[0], (const float *)in[1], (float *)out);
+        });
+    };
+
+    // cudnn7.d:251-333
+    R["maxpool"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];
+        if (!need_deps(op, 1) || !need_f32(op)) return nullptr;
+        const auto *dims = sizes_attr(op, "dims");
+        const auto &x = g.ops[op.deps[0]].shape;
+        if (!dims || dims->size() != 2 || !rank4(x, "maxpool features")) return nullptr;
+        const size_t N = x[0], C = x[1], H = x[2], W = x[3], ph = (*dims)[0], pw = (*dims)[1];
+        return make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_maxpool_fwd(N, C, H, W, ph, pw, (const float *)in[0], (float *)out);
+        });
+    };
+    R["maxpoolGrad"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];  // deps [parentGrad, y, x] (core/ops/nnet.d:402-407)
+        if (!need_deps(op, 3) || !need_f32(op)) return nullptr;
+        const auto *dims = sizes_attr(op, "dims");
+        const auto &x = g.ops[op.deps[2]].shape;
+        if (!dims || dims->size() != 2 || !rank4(x, "maxpoolGrad features")) return nullptr;
+        const size_t N = x[0], C = x[1], H = x[2], W = x[3], ph = (*dims)[0], pw = (*dims)[1];
+        return make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_maxpool_bwd(N, C, H, W, ph, pw, (const float *)in[0], (const float *)in[2], (float *)out);
+        });
+    };
+
+    // cudnn7.d:335-404
+    R["softmax"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];
+        if (!need_deps(op, 1) || !need_f32(op)) return nullptr;
+        size_t N, C, inner;
+        nci(op.shape, &N, &C, &inner);
+        return make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_softmax_fwd(N, C, inner, (const float *)in[0], (float *)out);
+        });
+    };
+    R["softmaxGrad"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];  // deps [parentGrad, y]
+        if (!need_deps(op, 2) || !need_f32(op)) return nullptr;
+        size_t N, C, inner;
+        nci(op.shape, &N, &C, &inner);
+        return make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_softmax_bwd(N, C, inner, (const float *)in[0], (const float *)in[1], (float *)out);
+        });
+    };
+
+    // cudnn7.d:406-478
+    R["relu"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];
+        if (!need_deps(op, 1) || !need_f32(op)) return nullptr;
+        const size_t n = op.volume();
+        return make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_relu_fwd(n, (const float *)in[0], (float *)out);
+        });
+    };
+    R["reluGrad"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];  // deps [parentGrad, y, x]
+        if (!need_deps(op, 3) || !need_f32(op)) return nullptr;
+        const size_t n = op.volume();
+        return make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_relu_bwd(n, (const float *)in[0], (const float *)in[2], (float *)out);
+        });
+    };
+
+    // cudnn7.d:480-545
+    R["addBias"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];
+        if (!need_deps(op, 2) || !need_f32(op)) return nullptr;
+        size_t N, C, inner;
+        nci(op.shape, &N, &C, &inner);
+        return make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_bias_fwd(N, C, inner, (const float *)in[0], (const float *)in[1], (float *)out);
+        });
+    };
+    R["addBiasGrad"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];
+        if (!need_deps(op, 1) || !need_f32(op)) return nullptr;
+        size_t N, C, inner;
+        nci(g.ops[op.deps[0]].shape, &N, &C, &inner);
+        return make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_bias_bwd(N, C, inner, (const float *)in[0], (float *)out);
+        });
+    };
+
+    // cudnn7.d:547-654
+    R["batchNormTrain"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];  // deps [x, scale, bias, mean, var]
+        if (!need_deps(op, 5) || !need_f32(op)) return nullptr;
+        auto it = op.doubleAttrs.find("momentum");
+        if (it == op.doubleAttrs.end()) {
+            fail(DOPT_HIP_ERR_INVALID, "batchNormTrain has no 'momentum' attribute");
+            return nullptr;
+        }
+        const double momentum = it->second;
+        size_t N, C, inner;
+        nci(g.ops[op.deps[0]].shape, &N, &C, &inner);
+        return make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_bn_train(N, C, inner, momentum, (const float *)in[0], (const float *)in[1],
+                                     (const float *)in[2], (const float *)in[3], (const float *)in[4], (float *)out);
+        });
+    };
+    R["batchNormGrad"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];  // deps [parentGrad, x, scale]
+        if (!need_deps(op, 3) || !need_f32(op)) return nullptr;
+        size_t N, C, inner;
+        nci(g.ops[op.deps[1]].shape, &N, &C, &inner);
+        return make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_bn_grad(N, C, inner, (const float *)in[0], (const float *)in[1], (const float *)in[2],
+                                    (float *)out);
+        });
+    };
+    R["batchNormInference"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];  // deps [x, scale, bias, mean, var]
+        if (!need_deps(op, 5) || !need_f32(op)) return nullptr;
+        size_t N, C, inner;
+        nci(op.shape, &N, &C, &inner);
+        return make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_bn_infer(N, C, inner, (const float *)in[0], (const float *)in[1], (const float *)in[2],
+                                     (const float *)in[3], (const float *)in[4], (float *)out);
+        });
+    };
+}
+
+bool is_leaf(const Operation &op) { return op.opType == "variable" || op.opType == "constant"; }
+
+}  // namespace
+
+void registerBuiltinKernels()
+{
+    static bool done = false;
+    if (done) return;
+    done = true;
+    registerBuiltinsOnce();
+}
+
+int registerHIPKernel(const std::string &opName, HIPKernelCtr ctr)
+{
+    registerBuiltinKernels();
+    auto &R = kernelCtrs();
+    if (R.find(opName) != R.end())
+        return fail(DOPT_HIP_ERR_INVALID, "A HIPKernelCtr is already registered for the operation '%s'", opName.c_str());
+    R[opName] = std::move(ctr);
+    return DOPT_HIP_OK;
+}
+
+void deregisterHIPKernel(const std::string &opName)
+{
+    registerBuiltinKernels();
+    kernelCtrs().erase(opName);
+}
+
+std::vector<std::string> listHIPOperations()
+{
+    registerBuiltinKernels();
+    std::vector<std::string> names;
+    for (auto &kv : kernelCtrs()) names.push_back(kv.first);
+    std::sort(names.begin(), names.end());
+    names.push_back("variable");
+    names.push_back("reshape");
+    return names;
+}
+
+// ------------------------------------------------------------------------------- HIPPlan
+
+namespace {
+
+struct Alias {
+    int source = -1;     // op whose buffer is aliased
+    size_t offset = 0;   // bytes
+};
+
+void toposort(const Graph &g, int op, std::vector<char> &seen, std::vector<int> &order)
+{
+    // iterative depth-first walk, dependencies first (core/ops/package.d:284-311)
+    std::vector<std::pair<int, size_t>> stack{{op, 0}};
+    if (seen[op]) return;
+    seen[op] = 1;
+    while (!stack.empty()) {
+        auto &top = stack.back();
+        const Operation &o = g.ops[top.first];
+        if (top.second < o.deps.size()) {
+            int d = o.deps[top.second++];
+            if (!seen[d]) {
+                seen[d] = 1;
+                stack.push_back({d, 0});
+            }
+        } else {
+            order.push_back(top.first);
+            stack.pop_back();
+        }
+    }
+}
+
+}  // namespace
+
+int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flags, std::unique_ptr<HIPPlan> *out)
+{
+    registerBuiltinKernels();
+    if (!ensure_init()) return DOPT_HIP_ERR_RUNTIME;
+    const Graph &g = *graph;
+    const int nops = (int)g.ops.size();
+    for (int o : outputs)
+        if (o < 0 || o >= nops) return fail(DOPT_HIP_ERR_INVALID, "plan output %d is not an operation of the graph", o);
+
+    std::unique_ptr<HIPPlan> p(new HIPPlan());
+    p->mGraph = graph;
+    p->mFlags = flags;
+    p->mOutputs = outputs;
+    std::vector<char> seen((size_t)nops, 0);
+    for (int o : outputs) toposort(g, o, seen, p->mOps);
+
+    // aliases: reshape always (package.d:295-299); contiguous slices and slice-of-pad under VIEWS
+    std::vector<Alias> alias((size_t)nops);
+    for (int id : p->mOps) {
+        const Operation &op = g.ops[id];
+        if (op.opType == "reshape") {
+            if (op.deps.size() != 1) return fail(DOPT_HIP_ERR_INVALID, "reshape expects one dependency");
+            alias[id].source = op.deps[0];
+        } else if ((flags & DOPT_HIP_PLAN_VIEWS) && op.opType == "slice" && op.deps.size() == 1) {
+            const Operation &src = g.ops[op.deps[0]];
+            auto st = op.sizeAttrs.find("start");
+            if (st == op.sizeAttrs.end() || st->second.size() != src.rank() || op.rank() != src.rank()) continue;
+            const std::vector<size_t> &start = st->second;
+            // slice(pad(x)) selecting exactly x
+            if (src.opType == "pad" && src.deps.size() == 1) {
+                auto bf = src.sizeAttrs.find("before");
+                if (bf != src.sizeAttrs.end() && bf->second == start && g.ops[src.deps[0]].shape == op.shape) {
+                    alias[id].source = src.deps[0];
+                    continue;
+                }
+            }
+            bool contiguous = true;
+            for (size_t i = 1; i < src.rank(); i++) contiguous = contiguous && start[i] == 0 && op.shape[i] == src.shape[i];
+            if (contiguous && src.rank() > 0) {
+                size_t inner = 1;
+                for (size_t i = 1; i < src.rank(); i++) inner *= src.shape[i];
+                alias[id].source = op.deps[0];
+                alias[id].offset = start[0] * inner * 4;
+            }
+        }
+    }
+
+    // operations whose results are actually consumed (everything, unless VIEWS created dead copies)
+    std::vector<char> needed((size_t)nops, 0);
+    {
+        std::vector<int> work(outputs.begin(), outputs.end());
+        while (!work.empty()) {
+            int id = work.back();
+            work.pop_back();
+            if (needed[id]) continue;
+            needed[id] = 1;
+            if (alias[id].source >= 0) work.push_back(alias[id].source);
+            else for (int d : g.ops[id].deps) work.push_back(d);
+        }
+    }
+
+    // kernels and buffers
+    for (int id : p->mOps) {
+        if (!needed[id]) continue;
+        const Operation &op = g.ops[id];
+        if (is_leaf(op)) {
+            if (!op.value && op.bytes() > 0)
+                return fail(DOPT_HIP_ERR_INVALID, "%s %d has no value buffer", op.opType.c_str(), id);
+            p->mResults[id] = op.value;
+            continue;
+        }
+        if (alias[id].source >= 0) continue;  // resolved per execution
+        auto it = kernelCtrs().find(op.opType);
+        if (it == kernelCtrs().end())
+            return fail(DOPT_HIP_ERR_UNSUPPORTED, "Could not construct a HIP kernel for operation of type '%s'",
+                        op.opType.c_str());
+        clear_error();
+        std::unique_ptr<HIPKernel> k = it->second(g, id);
+        if (!k) {
+            std::string why = dopt_hip_last_error();
+            return fail(DOPT_HIP_ERR_INVALID, "Could not construct a HIP kernel for operation of type '%s': %s",
+                        op.opType.c_str(), why.empty() ? "constructor returned null" : why.c_str());
+        }
+        void *buf = nullptr;
+        if (int rc = dopt_hip_malloc(&buf, op.bytes())) return rc;
+        if (buf) p->mOwned.push_back(buf);
+        p->mBufferBytes += op.bytes();
+        p->mResults[id] = buf;
+        Step s;
+        s.op = id;
+        s.kernel = std::move(k);
+        s.inputs.resize(op.deps.size());
+        s.inputBytes.resize(op.deps.size());
+        for (size_t i = 0; i < op.deps.size(); i++) s.inputBytes[i] = g.ops[op.deps[i]].bytes();
+        p->mSteps.push_back(std::move(s));
+    }
+    // remember aliases for the per-execution resolve pass
+    for (int id : p->mOps)
+        if (needed[id] && alias[id].source >= 0) p->mResults[id] = nullptr;
+    p->mAliasSource.assign((size_t)nops, -1);
+    p->mAliasOffset.assign((size_t)nops, 0);
+    for (int id : p->mOps)
+        if (needed[id] && alias[id].source >= 0) {
+            p->mAliasSource[id] = alias[id].source;
+            p->mAliasOffset[id] = alias[id].offset;
+        }
+    p->mNeeded = needed;
+    if (flags & DOPT_HIP_PLAN_TIMING) {
+        p->mEvents.resize(p->mSteps.size());
+        for (auto &ev : p->mEvents) {
+            DOPT_HIP_CHECK(hipEventCreate(&ev.first));
+            DOPT_HIP_CHECK(hipEventCreate(&ev.second));
+        }
+    }
+    // Resolve aliases once against the variables' own values so that result() is meaningful before
+    // the first execution (an alias of a variable that is later passed as an argument moves with it).
+    if (int rc = p->resolve(0, nullptr, nullptr, nullptr)) return rc;
+    *out = std::move(p);
+    return DOPT_HIP_OK;
+}
+
+HIPPlan::~HIPPlan() { cleanup(); }
+
+void HIPPlan::cleanup()
+{
+    if (mClean) return;
+    for (void *b : mOwned) dopt_hip_free(b);
+    mOwned.clear();
+    for (auto &kv : mArgStaging) dopt_hip_free(kv.second);
+    mArgStaging.clear();
+    for (auto &ev : mEvents) {
+        (void)hipEventDestroy(ev.first);
+        (void)hipEventDestroy(ev.second);
+    }
+    mEvents.clear();
+    mClean = true;
+}
+
+int HIPPlan::resolve(int nargs, const int *argOps, const void *const *argPtrs, const int *argOnHost)
+{
+    const Graph &g = *mGraph;
+    // variables: argument buffer if given, else the variable's own value (package.d:367-401)
+    for (int id : mOps)
+        if (mNeeded[id] && is_leaf(g.ops[id])) mResults[id] = g.ops[id].value;
+    for (int a = 0; a < nargs; a++) {
+        const int id = argOps[a];
+        if (id < 0 || id >= (int)g.ops.size() || g.ops[id].opType != "variable")
+            return fail(DOPT_HIP_ERR_INVALID,
+                        "All assignments in args must be for Operations with an opType of 'variable'");
+        if (!mNeeded[id]) continue;
+        if (argOnHost && argOnHost[a]) {
+            void *&stage = mArgStaging[id];
+            if (!stage)
+                if (int rc = dopt_hip_malloc(&stage, g.ops[id].bytes())) return rc;
+            if (int rc = dopt_hip_copy_h2d(stage, argPtrs[a], g.ops[id].bytes())) return rc;  // once per execution
+            mResults[id] = stage;
+        } else {
+            mResults[id] = const_cast<void *>(argPtrs[a]);
+        }
+    }
+    for (int id : mOps)
+        if (mNeeded[id] && mAliasSource[id] >= 0)
+            mResults[id] = (char *)mResults[mAliasSource[id]] + mAliasOffset[id];
+    for (Step &s : mSteps) {
+        const Operation &op = g.ops[s.op];
+        for (size_t i = 0; i < op.deps.size(); i++) s.inputs[i] = mResults[op.deps[i]];
+    }
+    return DOPT_HIP_OK;
+}
+
+int HIPPlan::execute(int nargs, const int *argOps, const void *const *argPtrs, const int *argOnHost, int nrets,
+                     void *const *rets)
+{
+    if (mClean) return fail(DOPT_HIP_ERR_INVALID, "plan was cleaned up");
+    if (nrets > (int)mOutputs.size()) return fail(DOPT_HIP_ERR_INVALID, "more return buffers than plan outputs");
+    if (int rc = resolve(nargs, argOps, argPtrs, argOnHost)) return rc;
+    const bool timing = !mEvents.empty();
+    for (size_t i = 0; i < mSteps.size(); i++) {
+        Step &s = mSteps[i];
+        if (timing) DOPT_HIP_CHECK(hipEventRecord(mEvents[i].first, stream()));
+        if (int rc = s.kernel->execute(s.inputs, s.inputBytes, mResults[s.op], mGraph->ops[s.op].bytes())) return rc;
+        if (timing) DOPT_HIP_CHECK(hipEventRecord(mEvents[i].second, stream()));
+    }
+    if (timing) {
+        DOPT_HIP_CHECK(hipStreamSynchronize(stream()));
+        for (size_t i = 0; i < mSteps.size(); i++) {
+            float ms = 0.0f;
+            DOPT_HIP_CHECK(hipEventElapsedTime(&ms, mEvents[i].first, mEvents[i].second));
+            auto &slot = profiler[mGraph->ops[mSteps[i].op].opType];
+            slot.first += (double)ms * 1000.0;
+            slot.second += 1;
+        }
+    }
+    for (int i = 0; i < nrets; i++) {
+        if (!rets[i]) continue;
+        const int o = mOutputs[(size_t)i];
+        if (int rc = dopt_hip_copy_d2d(rets[i], mResults[o], mGraph->ops[o].bytes())) return rc;  // package.d:419-422
+    }
+    return DOPT_HIP_OK;
+}
+
+int HIPPlan::result(int op, void **ptr, size_t *bytes) const
+{
+    auto it = mResults.find(op);
+    if (it == mResults.end()) return fail(DOPT_HIP_ERR_INVALID, "operation %d is not part of this plan", op);
+    if (ptr) *ptr = it->second;
+    if (bytes) *bytes = mGraph->ops[op].bytes();
+    return DOPT_HIP_OK;
+}
+
+std::string HIPPlan::profile()
+{
+    std::string s;
+    char line[256];
+    for (auto &kv : profiler) {
+        snprintf(line, sizeof(line), "%s %.1f %zu\n", kv.first.c_str(), kv.second.first, kv.second.second);
+        s += line;
+    }
+    return s;
+}
+
+}  // namespace dopt
+
+// ------------------------------------------------------------------------------- C ABI
+
+using namespace dopt;
+
+namespace {
+
+int copy_text(const std::string &s, char *buf, size_t buf_bytes, size_t *needed)
+{
+    if (needed) *needed = s.size() + 1;
+    if (buf && buf_bytes > 0) {
+        size_t n = s.size() < buf_bytes - 1 ? s.size() : buf_bytes - 1;
+        memcpy(buf, s.data(), n);
+        buf[n] = '\0';
+    }
+    return DOPT_HIP_OK;
+}
+
+class CKernel : public HIPKernel {
+public:
+    explicit CKernel(dopt_hip_kernel k) : mK(k) {}
+    ~CKernel() override
+    {
+        if (mK.destroy) mK.destroy(mK.self);
+    }
+    int execute(const std::vector<const void *> &inputs, const std::vector<size_t> &inputBytes, void *output,
+                size_t outputBytes) override
+    {
+        return mK.execute(mK.self, (int)inputs.size(), inputs.data(), inputBytes.data(), output, outputBytes);
+    }
+
+private:
+    dopt_hip_kernel mK;
+};
+
+bool valid_op(Graph *g, int op) { return g && op >= 0 && op < (int)g->ops.size(); }
+
+}  // namespace
+
+extern "C" {
+
+int dopt_hip_graph_create(void **graph)
+{
+    DOPT_REQUIRE(graph != nullptr, "dopt_hip_graph_create: graph is null");
+    *graph = new Graph();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_graph_destroy(void *graph)
+{
+    delete (Graph *)graph;
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_graph_add_op(void *graph, const char *op_type, int dtype, int rank, const size_t *shape, int ndeps,
+                          const int *deps, int *op_id)
+{
+    Graph *g = (Graph *)graph;
+    DOPT_REQUIRE(g && op_type && op_id, "dopt_hip_graph_add_op: null argument");
+    DOPT_REQUIRE(rank >= 0 && rank <= 8 && (rank == 0 || shape), "dopt_hip_graph_add_op: rank must be 0..8");
+    DOPT_REQUIRE(ndeps >= 0 && (ndeps == 0 || deps), "dopt_hip_graph_add_op: bad dependency list");
+    if (dtype != DOPT_HIP_F32 && dtype != DOPT_HIP_I32)
+        return fail(DOPT_HIP_ERR_UNSUPPORTED, "Element type not supported.");
+    Operation op;
+    op.opType = op_type;
+    op.dtype = dtype;
+    op.shape.assign(shape, shape + rank);
+    for (int i = 0; i < ndeps; i++) {
+        DOPT_REQUIRE(deps[i] >= 0 && deps[i] < (int)g->ops.size(), "dopt_hip_graph_add_op: dependency %d does not exist",
+                     deps[i]);
+        op.deps.push_back(deps[i]);
+    }
+    if (is_leaf(op)) {
+        DOPT_REQUIRE(ndeps == 0, "%s takes no dependencies", op_type);
+        if (int rc = dopt_hip_malloc(&op.value, op.bytes())) return rc;  // defaultVarAllocator
+    }
+    g->ops.push_back(std::move(op));
+    *op_id = (int)g->ops.size() - 1;
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_graph_set_attr_sizes(void *graph, int op, const char *key, const size_t *values, int n)
+{
+    Graph *g = (Graph *)graph;
+    DOPT_REQUIRE(valid_op(g, op) && key && n >= 0 && (n == 0 || values), "dopt_hip_graph_set_attr_sizes: bad argument");
+    g->ops[op].sizeAttrs[key].assign(values, values + n);
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_graph_set_attr_double(void *graph, int op, const char *key, double value)
+{
+    Graph *g = (Graph *)graph;
+    DOPT_REQUIRE(valid_op(g, op) && key, "dopt_hip_graph_set_attr_double: bad argument");
+    g->ops[op].doubleAttrs[key] = value;
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_graph_value(void *graph, int op, void **device_ptr, size_t *bytes)
+{
+    Graph *g = (Graph *)graph;
+    DOPT_REQUIRE(valid_op(g, op), "dopt_hip_graph_value: no such operation");
+    DOPT_REQUIRE(is_leaf(g->ops[op]), "dopt_hip_graph_value: only variables and constants have a value");
+    if (device_ptr) *device_ptr = g->ops[op].value;
+    if (bytes) *bytes = g->ops[op].bytes();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_graph_op_type(void *graph, int op, const char **op_type, int *dtype, int *rank, size_t *shape8, int *ndeps)
+{
+    Graph *g = (Graph *)graph;
+    DOPT_REQUIRE(valid_op(g, op), "dopt_hip_graph_op_type: no such operation");
+    const Operation &o = g->ops[op];
+    if (op_type) *op_type = o.opType.c_str();
+    if (dtype) *dtype = o.dtype;
+    if (rank) *rank = (int)o.rank();
+    if (shape8)
+        for (size_t i = 0; i < o.rank() && i < 8; i++) shape8[i] = o.shape[i];
+    if (ndeps) *ndeps = (int)o.deps.size();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_graph_op_dep(void *graph, int op, int index, int *dep)
+{
+    Graph *g = (Graph *)graph;
+    DOPT_REQUIRE(valid_op(g, op) && dep && index >= 0 && index < (int)g->ops[op].deps.size(),
+                 "dopt_hip_graph_op_dep: bad argument");
+    *dep = g->ops[op].deps[(size_t)index];
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_register_kernel(const char *op_name, dopt_hip_kernel_ctor ctor, void *user)
+{
+    DOPT_REQUIRE(op_name && ctor, "dopt_hip_register_kernel: null argument");
+    return registerHIPKernel(op_name, [ctor, user](const Graph &g, int op) -> std::unique_ptr<HIPKernel> {
+        dopt_hip_kernel k{};
+        if (ctor((void *)&g, op, user, &k) != 0 || !k.execute) {
+            if (!*dopt_hip_last_error()) fail(DOPT_HIP_ERR_INVALID, "kernel constructor refused the operation");
+            return nullptr;
+        }
+        return std::unique_ptr<HIPKernel>(new CKernel(k));
+    });
+}
+
+int dopt_hip_deregister_kernel(const char *op_name)
+{
+    DOPT_REQUIRE(op_name != nullptr, "dopt_hip_deregister_kernel: null argument");
+    deregisterHIPKernel(op_name);
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_list_operations(char *buf, size_t buf_bytes, size_t *needed)
+{
+    std::string s;
+    for (const std::string &n : listHIPOperations()) s += n + "\n";
+    return copy_text(s, buf, buf_bytes, needed);
+}
+
+int dopt_hip_plan_create(void *graph, int noutputs, const int *outputs, unsigned flags, void **plan)
+{
+    DOPT_REQUIRE(graph && plan && noutputs >= 0 && (noutputs == 0 || outputs), "dopt_hip_plan_create: bad argument");
+    *plan = nullptr;
+    std::unique_ptr<HIPPlan> p;
+    if (int rc = HIPPlan::create((Graph *)graph, std::vector<int>(outputs, outputs + noutputs), flags, &p)) return rc;
+    *plan = p.release();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_plan_execute(void *plan, int nargs, const int *arg_ops, const void *const *arg_ptrs, const int *arg_on_host,
+                          int nrets, void *const *rets)
+{
+    DOPT_REQUIRE(plan != nullptr, "dopt_hip_plan_execute: plan is null");
+    DOPT_REQUIRE(nargs >= 0 && (nargs == 0 || (arg_ops && arg_ptrs)) && nrets >= 0 && (nrets == 0 || rets),
+                 "dopt_hip_plan_execute: bad argument");
+    return ((HIPPlan *)plan)->execute(nargs, arg_ops, arg_ptrs, arg_on_host, nrets, rets);
+}
+
+int dopt_hip_plan_result(void *plan, int op, void **device_ptr, size_t *bytes)
+{
+    DOPT_REQUIRE(plan != nullptr, "dopt_hip_plan_result: plan is null");
+    return ((HIPPlan *)plan)->result(op, device_ptr, bytes);
+}
+
+int dopt_hip_plan_stats(void *plan, size_t *kernels, size_t *buffer_bytes)
+{
+    DOPT_REQUIRE(plan != nullptr, "dopt_hip_plan_stats: plan is null");
+    if (kernels) *kernels = ((HIPPlan *)plan)->kernelCount();
+    if (buffer_bytes) *buffer_bytes = ((HIPPlan *)plan)->bufferBytes();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_plan_profile(void *plan, char *buf, size_t buf_bytes, size_t *needed)
+{
+    DOPT_REQUIRE(plan != nullptr, "dopt_hip_plan_profile: plan is null");
+    return copy_text(((HIPPlan *)plan)->profile(), buf, buf_bytes, needed);
+}
+
+int dopt_hip_plan_destroy(void *plan)
+{
+    delete (HIPPlan *)plan;
+    return DOPT_HIP_OK;
+}
+
+}  // extern "C"

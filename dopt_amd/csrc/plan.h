@@ -1,0 +1,114 @@
+// Host-side mirror of the reference's backend plugin interface
+// (cuda/source/dopt/cuda/package.d), with HIP in place of CUDA in every name.
+#pragma once
+
+#include <functional>
+#include <map>
+#include <memory>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "common.h"
+
+namespace dopt {
+
+// What a kernel constructor can read off an Operation (core/ops/package.d:52-251).
+struct Operation {
+    std::string opType;
+    std::vector<int> deps;
+    std::map<std::string, std::vector<size_t>> sizeAttrs;   // attributes["..."].get!(size_t[]) / size_t
+    std::map<std::string, double> doubleAttrs;              // attributes["..."].get!double
+    int dtype = DOPT_HIP_F32;
+    std::vector<size_t> shape;
+    void *value = nullptr;  // variable / constant: its HIPBuffer
+    size_t volume() const
+    {
+        size_t v = 1;
+        for (size_t s : shape) v *= s;
+        return v;
+    }
+    size_t bytes() const { return volume() * 4; }
+    size_t rank() const { return shape.size(); }
+};
+
+struct Graph {
+    std::vector<Operation> ops;
+    ~Graph();
+};
+
+// class CUDABuffer (cuda/package.d:124-251) over the pooled allocator.
+class HIPBuffer {
+public:
+    static std::unique_ptr<HIPBuffer> create(size_t numBytes);  // zero-filled; 0 bytes -> empty buffer
+    ~HIPBuffer();
+    int set(const void *host, size_t bytes);       // "input buffer is the wrong length."
+    int set(const HIPBuffer &other);               // "Mismatch in buffer size"
+    int get(void *host, size_t bytes) const;       // "output buffer is the wrong length."
+    size_t numBytes() const { return mNumBytes; }
+    void *ptr() const { return mPtr; }
+
+private:
+    HIPBuffer() = default;
+    size_t mNumBytes = 0;
+    void *mPtr = nullptr;
+};
+
+// interface CUDAKernel (cuda/package.d:68-79)
+class HIPKernel {
+public:
+    virtual ~HIPKernel() = default;
+    // inputs[i] is the buffer of op.deps[i]; output is preallocated by the plan.
+    virtual int execute(const std::vector<const void *> &inputs, const std::vector<size_t> &inputBytes, void *output,
+                        size_t outputBytes) = 0;
+};
+
+// alias CUDAKernelCtr = CUDAKernel delegate(Operation op) (cuda/package.d:25).  A constructor
+// reports failure by returning null after calling dopt::fail().
+using HIPKernelCtr = std::function<std::unique_ptr<HIPKernel>(const Graph &graph, int op)>;
+
+int registerHIPKernel(const std::string &opName, HIPKernelCtr ctr);   // throws-equivalent if present
+void deregisterHIPKernel(const std::string &opName);
+std::vector<std::string> listHIPOperations();
+void registerBuiltinKernels();  // idempotent
+
+// class CUDAPlan (cuda/package.d:261-433)
+class HIPPlan {
+public:
+    static int create(Graph *graph, const std::vector<int> &outputs, unsigned flags, std::unique_ptr<HIPPlan> *out);
+    ~HIPPlan();
+    void cleanup();
+    int execute(int nargs, const int *argOps, const void *const *argPtrs, const int *argOnHost, int nrets,
+                void *const *rets);
+    int result(int op, void **ptr, size_t *bytes) const;
+    size_t kernelCount() const { return mSteps.size(); }
+    size_t bufferBytes() const { return mBufferBytes; }
+    std::string profile();
+    std::map<std::string, std::pair<double, size_t>> profiler;  // opType -> (microseconds, executions)
+
+private:
+    HIPPlan() = default;
+    struct Step {
+        int op;
+        std::unique_ptr<HIPKernel> kernel;
+        std::vector<const void *> inputs;
+        std::vector<size_t> inputBytes;
+    };
+    Graph *mGraph = nullptr;
+    unsigned mFlags = 0;
+    std::vector<int> mOutputs;
+    std::vector<int> mOps;                       // topological order
+    std::vector<Step> mSteps;                    // kernels to run, in order
+    std::unordered_map<int, void *> mResults;    // op -> buffer
+    std::vector<void *> mOwned;                  // buffers to free in cleanup
+    std::unordered_map<int, void *> mArgStaging; // variable op -> plan-owned device copy for host args
+    std::vector<int> mAliasSource;               // per op: the op whose buffer it aliases, or -1
+    std::vector<size_t> mAliasOffset;            // per op: byte offset into the aliased buffer
+    std::vector<char> mNeeded;                   // per op: its result is consumed
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> mEvents;
+    size_t mBufferBytes = 0;
+    bool mClean = false;
+    int resolve(int nargs, const int *argOps, const void *const *argPtrs, const int *argOnHost);
+};
+
+}  // namespace dopt

@@ -1,0 +1,263 @@
+"""The backend behind its plugin boundary: graphs built with the reference's op constructors,
+executed by HIPPlan through the C ABI.  Replays every known-answer test the reference holds
+(they all go through `evaluate`), the registry contract, plan semantics, and the optimizers
+(op-graph form vs fused kernels vs the oracle)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle as O
+from util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+core = pytest.importorskip("dopt_amd.core")
+from dopt_amd import capi, nnet, online, ops  # noqa: E402
+from dopt_amd.core import (evaluate, float32, float32Constant, grad, int32)  # noqa: E402
+
+
+def _f(shape, vals):
+    return float32(shape, np.array(vals, np.float32))
+
+
+# ----------------------------------------------------------------------------- reference KATs through evaluate()
+def test_kat_slice_pad_reshape_transpose_repeat(kats):
+    k = kats["slice"]
+    out = evaluate(core.slice(int32(k["shape"], k["input"]), k["start"], k["stop"]))
+    assert out.dtype == np.int32 and out.ravel().tolist() == k["expected"]
+    k = kats["pad"]
+    assert evaluate(core.pad(int32(k["shape"], k["input"]), k["before"], k["after"])).ravel().tolist() == k["expected"]
+    k = kats["reshape"]
+    r1 = _f(k["shape"], k["input"]).reshape(k["newShape"])
+    assert r1.shape == tuple(k["newShape"]) and evaluate(r1).ravel().tolist() == k["expected"]
+    k = kats["transpose"]
+    assert evaluate(core.transpose(_f(k["shape"], k["input"]), k["order"])).ravel().tolist() == k["expected"]
+    for name in ("repeat_1x1", "repeat_2x2"):
+        k = kats[name]
+        got = evaluate(core.repeat(_f(k["shape"], k["input"]), k["repetitions"]))
+        assert got.ravel().tolist() == [float(v) for v in k["expected"]]
+    k = kats["repeat_scalar_count"]
+    assert evaluate(core.repeat(_f(k["shape"], k["input"]), k["repetitions"])).ravel().tolist() == k["expected"]
+
+
+def test_kat_matmul_sum_argmin_max(kats):
+    k = kats["matmul"]
+    assert evaluate(core.matmul(_f(k["a_shape"], k["a"]), _f(k["b_shape"], k["b"]))).ravel().tolist() == k["expected"]
+    for c in kats["sum"]["cases"]:
+        assert evaluate(core.sum(_f(c["shape"], c["input"]), c["axes"])).ravel().tolist() == c["expected"]
+    for c in kats["argmin"]["cases"]:
+        out = evaluate(core.argmin(_f(c["shape"], c["input"]), c["axis"]))
+        assert out.dtype == np.int32 and out.ravel().tolist() == c["expected"]
+    for c in kats["maxElement"]["cases"]:
+        assert evaluate(core.maxElement(_f(c["shape"], c["input"]), c["axes"])).ravel().tolist() == c["expected"]
+
+
+def test_kat_convolution_maxpool_softmax(kats):
+    k = kats["convolution"]
+    y = evaluate(core.convolution(_f(k["features_shape"], k["features"]), _f(k["filters_shape"], k["filters"])))
+    assert y.ravel().tolist() == [float(v) for v in k["expected"]]       # pins the filter flip
+    k = kats["maxpool"]
+    assert evaluate(core.maxpool(_f(k["shape"], k["input"]), k["dims"])).ravel().tolist() == \
+        [float(np.float32(v)) for v in k["expected"]]
+    k = kats["softmax"]
+    assert np.allclose(evaluate(core.softmax(_f(k["shape"], k["input"]))).ravel(), k["expected"], rtol=k["rel"],
+                       atol=k["abs"])
+
+
+def test_kat_grads_and_scalar_plan(kats):
+    x = float32()
+    y = x * x
+    r = np.float32(-63.21875)
+    g = evaluate(grad(y, [x]), {x: np.array([r])})[0]
+    assert g[()] == r + r                                                 # grads/package.d:113-129
+    k = kats["slice_grad"]
+    a, b = _f(k["shape"], k["a"]), _f(k["shape"], k["b"])
+    c = core.slice(a * b, k["start"], k["stop"])
+    assert evaluate(grad(c, [a]))[0].ravel().tolist() == [float(v) for v in k["expected"]]
+    k = kats["scalar_plan"]
+    assert evaluate(_f([], [k["a"]]) * _f([], [k["b"]]) + _f([], [k["c"]]))[()] == k["expected"]
+
+
+def test_kat_batchnorm_running_mean_with_adam(kats):
+    # nnet/layers/batchnorm.d:158-177, through the op-graph ADAM and the projections
+    k = kats["batchnorm_running_mean"]
+    x = _f(k["shape"], k["x"])
+    layers = nnet.batchNorm(nnet.dataSource(x))
+    net = nnet.DAGNetwork([x], [layers])
+    trloss = core.sum(layers.trainOutput)
+    updater = online.adam([trloss], net.params, net.paramProj)
+    for _ in range(200):                      # 0.9^200 ~ 7e-10: converged far below the 1e-2 tolerance
+        updater.step_async(None)
+    mean = layers.params[2].symbol.value
+    assert np.allclose(mean, k["expected_running_mean"], rtol=k["rel"], atol=k["abs"])
+
+
+# ----------------------------------------------------------------------------- registry (cuda/package.d:479-507)
+def test_registry_contract():
+    names = core.list_operations()
+    for n in ["add", "matmul", "convolution", "convolutionFeaturesGrad", "convolutionFiltersGrad", "maxpool",
+              "maxpoolGrad", "softmax", "softmaxGrad", "relu", "reluGrad", "addBias", "addBiasGrad", "batchNormTrain",
+              "batchNormGrad", "batchNormInference", "slice", "pad", "repeat", "transpose", "sum", "maxElement",
+              "argmin", "variable", "reshape"]:
+        assert n in names, n
+    lib = core._lib()
+    CTOR = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p)
+    ctor = CTOR(lambda g, op, user, out: 1)
+    rc = lib.dopt_hip_register_kernel(b"add", C.cast(ctor, C.c_void_p), None)
+    assert rc == 1 and b"already registered" in lib.dopt_hip_last_error()
+    # deregister then the op cannot be planned; re-registering a refusing constructor also fails loudly
+    assert lib.dopt_hip_deregister_kernel(b"atanh") == 0
+    assert "atanh" not in core.list_operations()
+    with pytest.raises(capi.HipError, match="Could not construct a HIP kernel"):
+        evaluate(core.atanh(_f([2], [0.5, -0.5])))
+    assert lib.dopt_hip_register_kernel(b"atanh", C.cast(ctor, C.c_void_p), None) == 0
+    with pytest.raises(capi.HipError, match="Could not construct a HIP kernel"):
+        evaluate(core.atanh(_f([2], [0.5, -0.5])))
+    lib.dopt_hip_deregister_kernel(b"atanh")
+
+
+def test_custom_kernel_through_the_registry():
+    lib = core._lib()
+
+    class Kernel(C.Structure):
+        _fields_ = [("self", C.c_void_p), ("execute", C.c_void_p), ("destroy", C.c_void_p)]
+
+    EXEC = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int, C.POINTER(C.c_void_p), C.POINTER(C.c_size_t), C.c_void_p,
+                       C.c_size_t)
+    CTOR = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.POINTER(Kernel))
+    calls = []
+
+    def execute(self, nin, inputs, nbytes, out, out_bytes):
+        calls.append((nin, nbytes[0], out_bytes))
+        # an "atanh" that is really a device-to-device copy of its input
+        return capi.load().dopt_hip_copy_d2d(out, inputs[0], out_bytes)
+    exec_c = EXEC(execute)
+
+    def ctor(graph, op, user, out):
+        out[0].self = None
+        out[0].execute = C.cast(exec_c, C.c_void_p)
+        out[0].destroy = None
+        return 0
+    ctor_c = CTOR(ctor)
+    lib.dopt_hip_deregister_kernel(b"atanh")
+    assert lib.dopt_hip_register_kernel(b"atanh", C.cast(ctor_c, C.c_void_p), None) == 0
+    try:
+        got = evaluate(core.atanh(_f([3], [5, -7, 0])))
+        assert got.tolist() == [5.0, -7.0, 0.0] and calls == [(1, 12, 12)]
+    finally:
+        lib.dopt_hip_deregister_kernel(b"atanh")
+
+
+# ----------------------------------------------------------------------------- plan semantics
+def test_plan_args_must_be_variables_and_sizes_must_match():
+    a = _f([2], [1, 2])
+    y = a + a
+    plan = core.compile([y])
+    with pytest.raises(capi.HipError, match="opType of 'variable'"):
+        plan.execute({y: np.zeros(2, np.float32)})
+    with pytest.raises(capi.HipError):
+        plan.execute({a: np.zeros(3, np.float32)})
+    assert plan.execute({a: np.array([3, 4], np.float32)})[0].tolist() == [6.0, 8.0]
+    assert plan.execute()[0].tolist() == [2.0, 4.0]          # falls back to the variable's own value
+    plan.cleanup()
+
+
+def test_plan_views_do_not_change_results():
+    r = np.random.default_rng(3)
+    x = float32([4, 6, 5, 5], r.standard_normal((4, 6, 5, 5)).astype(np.float32))
+    gamma = float32([1, 6, 1, 1], np.ones(6, np.float32))
+    beta, mean = float32([6]), float32([6])
+    var = float32([6], np.ones(6, np.float32))
+    y, nm, nv = core.batchNormTrain(x, gamma, beta, mean, var, 0.9)
+    loss = core.sum(core.relu(y) * core.relu(y))
+    outs = [loss, nm, nv] + grad(loss, [x, gamma, beta])
+    plain = core.compile(outs)
+    views = core.compile(outs, core.PLAN_VIEWS)
+    assert views.stats()["kernels"] < plain.stats()["kernels"]
+    for a, b in zip(plain.execute(), views.execute()):
+        assert np.array_equal(a, b)
+    plain.cleanup()
+    views.cleanup()
+
+
+# ----------------------------------------------------------------------------- optimizers
+def _toy_problem(seed):
+    r = np.random.default_rng(seed)
+    x = float32([16, 12], r.standard_normal((16, 12)).astype(np.float32))
+    t = float32([16, 5], r.standard_normal((16, 5)).astype(np.float32))
+    w = float32([12, 5], (r.standard_normal((12, 5)) * 0.3).astype(np.float32))
+    b = float32([5], r.standard_normal(5).astype(np.float32))
+    pred = core.matmul(x, w) + core.repeat(b, 16)
+    loss = nnet.squaredError(pred, t)
+    return loss, [w, b]
+
+
+@pytest.mark.parametrize("rule", ["sgd", "nesterov", "adam", "amsgrad"])
+def test_fused_updaters_match_the_op_graph_form_bit_for_bit(rule):
+    loss_a, wrt_a = _toy_problem(5)
+    loss_b, wrt_b = _toy_problem(5)
+    if rule in ("sgd", "nesterov"):
+        nest = rule == "nesterov"
+        ua = online.sgd([loss_a], wrt_a, None, _f([], [0.05]), _f([], [0.9]), nest)
+        ub = online.fused_sgd([loss_b], wrt_b, None, 0.05, 0.9, nest)
+    else:
+        ua = getattr(online, rule)([loss_a], wrt_a, None, _f([], [0.01]))
+        ub = getattr(online, "fused_" + rule)([loss_b], wrt_b, None, 0.01)
+    for step in range(5):
+        la, lb = ua()[0], ub()[0]
+        assert la == lb, (step, la, lb)
+        for pa, pb in zip(wrt_a, wrt_b):
+            assert np.array_equal(pa.value, pb.value), (rule, step)
+    if rule in ("adam", "amsgrad"):
+        assert np.array_equal(ua.means[0].value, ub.state["m"][0].numpy())
+        assert np.array_equal(ua.vars[1].value, ub.state["v"][1].numpy())
+        assert ua.b1.value[()] == np.float32(ub.opt.b1.value) and ua.b2.value[()] == np.float32(ub.opt.b2.value)
+    if rule == "amsgrad":
+        assert np.array_equal(ua.varhats[0].value, ub.state["vhat"][0].numpy())
+
+
+@pytest.mark.parametrize("rule", ["sgd", "adam", "amsgrad"])
+def test_fit_line_scenario(rule):
+    # online/{sgd,adam,amsgrad}.d unittests: y = 3x + 2, one sample per step (the reference only prints m, c)
+    r = np.random.default_rng(7)
+    xs = r.uniform(-10, 10, 100).astype(np.float32)
+    ys = np.float32(3) * xs + np.float32(2)
+    x, m, c, y = float32(), float32(), float32(), float32()
+    yhat = m * x + c
+    obj = (yhat - y) * (yhat - y)
+    if rule == "sgd":
+        up, steps = online.sgd([obj], [m, c], None, _f([], [0.001]), _f([], [0.9])), 300
+    else:
+        up, steps = getattr(online, rule)([obj], [m, c], None, _f([], [0.1])), 1500
+    for i in range(steps):
+        up.step_async({x: xs[i % 100:i % 100 + 1], y: ys[i % 100:i % 100 + 1]})
+    assert abs(m.value[()] - 3) < 0.1 and abs(c.value[()] - 2) < 0.5, (m.value, c.value)
+
+
+# ----------------------------------------------------------------------------- config 1: softmax regression step
+def test_config1_softmax_regression_step_matches_the_oracle():
+    # examples/mnistlogit.d:39-47: softmax built by hand from matmul/maxElement/exp/sum/repeat/div, SGD lr 0.1
+    r0, r1 = np.random.default_rng(0), np.random.default_rng(1)
+    X = r0.random((100, 784)).astype(np.float32)
+    lab = r1.integers(0, 10, 100)
+    Y = np.zeros((100, 10), np.float32)
+    Y[np.arange(100), lab] = 1
+    feats, labels = float32([100, 784]), float32([100, 10])
+    W, b = float32([784, 10]), float32([10])
+    linear = core.matmul(feats, W) + core.repeat(b, 100)
+    numer = core.exp(linear - core.maxElement(linear))
+    denom = core.repeat(core.sum(numer, [1]).reshape([100, 1]), [1, 10])
+    preds = numer / denom
+    loss = nnet.crossEntropy(preds, labels)
+    up = online.sgd([loss, preds], [W, b], None, _f([], [0.1]))
+    loss0, p0 = up({feats: X, labels: Y})
+    # zero weights: uniform predictions, loss = -log(0.1 + 1e-6)
+    assert np.allclose(p0, 0.1, rtol=1e-6)
+    assert_close(loss0, -np.log(0.1 + 1e-6), "initial loss")
+    # oracle step: dL/dlinear = (softmax - Y)/100 for the composed graph; W' = W - 0.1 * X^T dlin
+    dlin = (np.full((100, 10), 0.1) - Y) / 100.0 * (0.1 / (0.1 + 1e-6))
+    assert_close(W.value, -0.1 * (X.astype(np.float64).T @ dlin), "W after one step", scale=0.01)
+    assert_close(b.value, -0.1 * dlin.sum(axis=0), "b after one step", scale=0.01)
+    loss1, _ = up({feats: X, labels: Y})
+    assert loss1 < loss0
