@@ -26,14 +26,26 @@ __device__ inline void mma_slab(const float *As, const float *Bs, int a_off, int
     const int kh = lane >> 5, l32 = lane & 31;
     const float *ap = As + kh * LDA + a_off + l32;
     const float *bp = Bs + kh * LDB + b_off + l32;
+    // software pipelined: the fragments of step ks+1 are requested from LDS before the four
+    // MFMAs of step ks are issued, so the LDS latency hides behind 256 cycles of matrix work
+    float a0 = ap[0], a1 = ap[32], b0 = bp[0], b1 = bp[32];
 #pragma unroll
     for (int ks = 0; ks < BK / 2; ++ks) {
-        float a0 = ap[(2 * ks) * LDA], a1 = ap[(2 * ks) * LDA + 32];
-        float b0 = bp[(2 * ks) * LDB], b1 = bp[(2 * ks) * LDB + 32];
+        float na0 = 0.f, na1 = 0.f, nb0 = 0.f, nb1 = 0.f;
+        if (ks + 1 < BK / 2) {
+            na0 = ap[(2 * ks + 2) * LDA];
+            na1 = ap[(2 * ks + 2) * LDA + 32];
+            nb0 = bp[(2 * ks + 2) * LDB];
+            nb1 = bp[(2 * ks + 2) * LDB + 32];
+        }
         acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
         acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
         acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
         acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+        a0 = na0;
+        a1 = na1;
+        b0 = nb0;
+        b1 = nb1;
     }
 }
 
@@ -62,5 +74,33 @@ __device__ inline bool xcd_remap(unsigned bid, unsigned total, unsigned *logical
 }
 
 inline unsigned xcd_grid(unsigned total) { return ((total + 7u) / 8u) * 8u; }
+
+// Buffer-resource loads: the hardware range check returns 0 for an offset at or past the end of
+// the buffer, so a masked element is loaded from kOobOffset instead of being branched around.
+// That keeps the gather loops branch-free (one basic block the scheduler can interleave with the
+// MFMAs) and the address arithmetic 32-bit.  Valid byte offsets must stay below 2^31.
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+constexpr unsigned kOobOffset = 0x80000000u;
+
+__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void *base, size_t bytes)
+{
+    const size_t clamped = bytes < 0x7fffffffu ? bytes : 0x7fffffffu;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)clamped, 0x00020000);
+}
+
+// voffset: per-lane byte offset (VGPR); soffset: wave-uniform byte offset (SGPR).
+__device__ inline float buffer_load_f32(__amdgpu_buffer_rsrc_t r, unsigned voffset, unsigned soffset)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)voffset, (int)soffset, 0));
+}
+
+__device__ inline float4 buffer_load_f32x4(__amdgpu_buffer_rsrc_t r, unsigned voffset, unsigned soffset)
+{
+    // Keep the builtin's own vector type: converting it to an ext_vector_type first makes the
+    // compiler load a single dword and splat it.
+    auto v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voffset, (int)soffset, 0);
+    static_assert(sizeof(v) == sizeof(float4), "b128 load must yield 16 bytes");
+    return __builtin_bit_cast(float4, v);
+}
 
 }  // namespace dopt

@@ -19,7 +19,7 @@ struct Gemm {
     const float *A, *B;
     float *C;  // or `splits` partial copies
     int M, N, K;
-    int mtiles, ntiles, slabs_total, slabs_per_split;
+    int mtiles, ntiles, slabs_total, slabs_per_split, splits;
     size_t out_elems;
 };
 
@@ -33,11 +33,15 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_k(Gemm p)
     __shared__ float As[2][BK * LDA];
     __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB];
 
+    // 1-D grid over (split, tile), tile fastest: the blocks an XCD receives work on neighbouring
+    // tiles of the same slice of the reduction, whatever the ratio of tiles to splits
     unsigned L;
-    if (!xcd_remap(blockIdx.x, (unsigned)(p.mtiles * p.ntiles), &L)) return;
-    const int mt = (int)(L % (unsigned)p.mtiles), nt = (int)(L / (unsigned)p.mtiles);
+    const unsigned tiles = (unsigned)(p.mtiles * p.ntiles);
+    if (!xcd_remap(blockIdx.x, tiles * (unsigned)p.splits, &L)) return;
+    const int split = (int)(L / tiles);
+    const unsigned tile = L - (unsigned)split * tiles;
+    const int mt = (int)(tile % (unsigned)p.mtiles), nt = (int)(tile / (unsigned)p.mtiles);
     const int m0 = mt * BM, n0 = nt * BN;
-    const int split = blockIdx.y;
     const int slab_begin = split * p.slabs_per_split;
     const int slab_end = min(slab_begin + p.slabs_per_split, p.slabs_total);
 
@@ -238,6 +242,7 @@ int dopt_hip_sgemm(size_t M, size_t N, size_t K, const float *A, const float *B,
     if (splits < 1) splits = 1;
     g.slabs_per_split = (g.slabs_total + splits - 1) / splits;
     splits = (g.slabs_total + g.slabs_per_split - 1) / g.slabs_per_split;
+    g.splits = splits;
     float *partial = nullptr;
     if (splits > 1) {
         partial = (float *)workspace((size_t)splits * g.out_elems * sizeof(float));
@@ -245,7 +250,7 @@ int dopt_hip_sgemm(size_t M, size_t N, size_t K, const float *A, const float *B,
     }
     g.C = splits > 1 ? partial : C;
     const bool vecB = (N % 4 == 0) && aligned16(B);
-    dim3 grid(xcd_grid((unsigned)tiles), (unsigned)splits);
+    dim3 grid(xcd_grid((unsigned)(tiles * splits)));
     if (big) {
         if (vecB) hipLaunchKernelGGL((sgemm_k<128, true>), grid, dim3(kGemmThreads), 0, stream(), g);
         else hipLaunchKernelGGL((sgemm_k<128, false>), grid, dim3(kGemmThreads), 0, stream(), g);
