@@ -12,17 +12,18 @@
 // GEMM view: M = output channels of the op, columns = output pixels (n,oh,ow), reduction =
 // (tap, ci) with ci padded to a multiple of 16 so that a 16-deep slab has ONE tap: the input
 // offset and the bounds mask are then uniform over the slab, and a lane's loads for successive
-// channels are one add apart.  Wp is the filter re-packed once per call into [tap*ci][m]
-// (m contiguous), so the A tile goes global -> LDS with 128-bit accesses; the pack costs two
-// passes over the filter, < 2 % of the layer's MFMA time for every VGG layer.
+// channels differ by a wave-uniform offset.  Wp is the filter re-packed once per call into
+// [tap*ci][m] (m contiguous), so the A tile goes global -> LDS with 128-bit accesses.
 //
-// Backward-filter is a GEMM with M = K (output channels), columns = (c,r',s') in filter memory
-// order, reduction = output pixels (n,p,q); both operands are gathered with lanes along the
-// pixel index (contiguous in memory).
+// Backward-filter is a GEMM with M = K (output channels), columns = (r', s', c) tap-major with c
+// padded to 16, reduction = output pixels (n,p,q); both operands are gathered with lanes along
+// the pixel index (contiguous in memory).  A second kernel sums the reduction splits and permutes
+// the columns back to [K][C][R][S].
 //
-// Layers with few output tiles (small spatial extent, or the short-and-wide filter gradients)
-// split the reduction over blockIdx.y; partial tiles go to the workspace and are summed in a
-// fixed order by a second kernel -- no float atomics, so results are reproducible.
+// All gathers go through buffer-resource loads whose range check supplies the zero padding, so
+// the inner loops are branch-free.  Layers with few output tiles split the reduction; partial
+// tiles go to the workspace and are summed in a fixed order -- no float atomics, so results are
+// reproducible.
 #include "common.h"
 #include "mfma_core.h"
 
@@ -31,6 +32,8 @@ namespace {
 using namespace dopt;
 
 constexpr int BK = 16;
+
+// ------------------------------------------------------------------------------------ gather
 
 struct GatherConv {
     const float *in;   // gathered operand [N, Cin, IH, IW]
@@ -43,14 +46,15 @@ struct GatherConv {
     size_t out_elems, in_bytes, wp_bytes;
 };
 
-template <int BM, bool kBwd>
-__global__ __launch_bounds__(kGemmThreads, 2) void conv_gather_k(GatherConv p)
+// kMode: 0 = forward, 1 = backward-data with unit stride (no divisions), 2 = backward-data, any stride
+template <class T, int kMode>
+__global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_gather_k(GatherConv p)
 {
-    constexpr int BN = BM == 128 ? 128 : 256, WN = BM == 128 ? 2 : 4;
-    constexpr int LDA = BM + 4, LDB = BN + 4;
-    constexpr int NA = BM * BK / 4 / kGemmThreads;  // float4 loads of A per thread
-    constexpr int RSTEP = kGemmThreads / BN;        // reduction rows covered by one pass of B loads
-    constexpr int NB = BK / RSTEP;                  // scalar loads of B per thread
+    constexpr int BM = T::BM, BN = T::BN, LDA = T::LDA, LDB = T::LDB, THREADS = T::THREADS;
+    constexpr int NA = BM * BK / 4 / THREADS;  // float4 loads of A per thread
+    constexpr int RSTEP = THREADS / BN;        // reduction rows covered by one pass of B loads
+    constexpr int NB = BK / RSTEP;             // scalar loads of B per thread
+    static_assert(NA >= 1 && NB >= 1 && RSTEP >= 1, "tile too small for the thread count");
     __shared__ __attribute__((aligned(16))) float As[2][BK * LDA];
     __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB];
 
@@ -67,7 +71,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void conv_gather_k(GatherConv p)
     const int slab_end = min(slab_begin + p.slabs_per_split, p.slabs_total);
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-    const int wm = w / WN, wn = w % WN;
+    const int wm = w / T::WN, wn = w % T::WN;
 
     const __amdgpu_buffer_rsrc_t rin = make_rsrc(p.in, p.in_bytes);
     const __amdgpu_buffer_rsrc_t rwp = make_rsrc(p.wp, p.wp_bytes);
@@ -77,7 +81,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void conv_gather_k(GatherConv p)
     int a_lds[NA];
 #pragma unroll
     for (int i = 0; i < NA; i++) {
-        const int f = tid + kGemmThreads * i;
+        const int f = tid + THREADS * i;
         const int row = f / (BM / 4), gm = m0 + (f % (BM / 4)) * 4;
         a_voff[i] = gm < p.Mp ? (unsigned)(row * p.Mp + gm) * 4u : kOobOffset;
         a_lds[i] = row * LDA + (f % (BM / 4)) * 4;
@@ -86,18 +90,14 @@ __global__ __launch_bounds__(kGemmThreads, 2) void conv_gather_k(GatherConv p)
     // B: the output pixel this thread gathers for
     const int bcol = tid % BN, brow0 = tid / BN;
     const int pix = n0 + bcol;
-    const bool pix_ok = pix < p.ncols;
+    const int pix_oob = p.ncols - 1 - pix;  // negative past the last pixel
     const int OHW = p.OH * p.OW;
-    int n_img = 0, oh = 0, ow = 0;
-    if (pix_ok) {
-        n_img = pix / OHW;
-        int pq = pix - n_img * OHW;
-        oh = pq / p.OW;
-        ow = pq - oh * p.OW;
-    }
+    const int n_img = pix / OHW, pq = pix - n_img * OHW;
+    const int oh = pq / p.OW, ow = pq - oh * p.OW;
     const int chan_stride = p.IH * p.IW;
     const int pix_base = (n_img * p.Cin + brow0) * chan_stride;  // element offset of (n, channel brow0, 0, 0)
     const int row_limit = p.Cin - brow0;                          // rows with ci0 + RSTEP*i >= row_limit are padding
+    const bool c_full = p.CinPad == p.Cin;
 
     // running position in the (tap, channel) reduction, advanced slab by slab without divisions
     int kk0 = slab_begin * BK;
@@ -111,24 +111,27 @@ __global__ __launch_bounds__(kGemmThreads, 2) void conv_gather_k(GatherConv p)
         const unsigned a_soff = (unsigned)(kk0 * p.Mp) * 4u;
 #pragma unroll
         for (int i = 0; i < NA; i++) areg[i] = buffer_load_f32x4(rwp, a_voff[i], a_soff);
-        int ih, iw;
-        bool ok = pix_ok;
-        if (!kBwd) {
+        int ih, iw, bad = pix_oob;
+        if (kMode == 0) {
             ih = oh * p.strideH - p.padH + (p.R - 1 - tr);
             iw = ow * p.strideW - p.padW + (p.S - 1 - ts);
+        } else if (kMode == 1) {
+            ih = oh + p.padH - (p.R - 1 - tr);
+            iw = ow + p.padW - (p.S - 1 - ts);
         } else {
             // out = dx[.., h, w]; in = dy[.., ph, qw] with h = ph*stride - pad + r, r = R-1-tr
             const int nh = oh + p.padH - (p.R - 1 - tr), nw = ow + p.padW - (p.S - 1 - ts);
             ih = nh / p.strideH;
             iw = nw / p.strideW;
-            ok = ok && nh >= 0 && nw >= 0 && ih * p.strideH == nh && iw * p.strideW == nw;
+            // negative numerators, and numerators that are not multiples of the stride, hit no input
+            bad |= nh | nw | -(int)(ih * p.strideH != nh) | -(int)(iw * p.strideW != nw);
         }
-        ok = ok && (unsigned)ih < (unsigned)p.IH && (unsigned)iw < (unsigned)p.IW;
-        const unsigned b_voff = ok ? (unsigned)(pix_base + ih * p.IW + iw) * 4u : kOobOffset;
+        bad |= ih | (p.IH - 1 - ih) | iw | (p.IW - 1 - iw);  // sign bit set: outside the input
+        const unsigned b_voff = bad < 0 ? kOobOffset : (unsigned)(pix_base + ih * p.IW + iw) * 4u;
 #pragma unroll
         for (int i = 0; i < NB; i++) {
             const int ci = ci0 + RSTEP * i;  // wave-uniform
-            const unsigned voff = (p.CinPad == p.Cin || ci < row_limit) ? b_voff : kOobOffset;
+            const unsigned voff = (c_full || ci < row_limit) ? b_voff : kOobOffset;
             breg[i] = buffer_load_f32(rin, voff, (unsigned)(ci * chan_stride) * 4u);
         }
         kk0 += BK;
@@ -148,38 +151,40 @@ __global__ __launch_bounds__(kGemmThreads, 2) void conv_gather_k(GatherConv p)
         for (int i = 0; i < NB; i++) Bs[buf][(brow0 + RSTEP * i) * LDB + bcol] = breg[i];
     };
 
-    v16f acc[2][2];
+    v16f acc[T::MI][T::NI];
     zero_acc(acc);
     load();
     store(0);
     __syncthreads();
     int cur = 0;
-    // steady state: no branches inside, so loads, MFMAs and LDS stores of one iteration form one block
+    // steady state: no data-dependent branches inside
     for (int slab = slab_begin; slab < slab_end - 1; ++slab) {
         load();
-        mma_slab<BK, LDA, LDB>(As[cur], Bs[cur], wm * 64, wn * 64, acc, lane);
+        mma_slab<BK, LDA, LDB>(As[cur], Bs[cur], wm * (BM / T::WM), wn * (BN / T::WN), acc, lane);
         store(cur ^ 1);
         __syncthreads();
         cur ^= 1;
     }
-    mma_slab<BK, LDA, LDB>(As[cur], Bs[cur], wm * 64, wn * 64, acc, lane);
+    mma_slab<BK, LDA, LDB>(As[cur], Bs[cur], wm * (BM / T::WM), wn * (BN / T::WN), acc, lane);
 
     float *outp = p.out + (size_t)split * p.out_elems;
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+    for (int j = 0; j < T::NI; j++) {
+        const int col = n0 + wn * (BN / T::WN) + j * 32 + (lane & 31);
         if (col >= p.ncols) continue;
         const int n2 = col / OHW, pq2 = col - n2 * OHW;
         float *base = outp + (size_t)n2 * p.Mout * OHW + pq2;
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int i = 0; i < T::MI; i++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int m = m0 + wm * 64 + i * 32 + acc_row(v, lane);
+                const int m = m0 + wm * (BM / T::WM) + i * 32 + acc_row(v, lane);
                 if (m < p.Mout) base[(size_t)m * OHW] = acc[i][j][v];
             }
     }
 }
+
+// ------------------------------------------------------------------------------------ backward-filter
 
 struct FilterGrad {
     const float *dy;  // [N, K, P, Q]
@@ -194,23 +199,19 @@ struct FilterGrad {
     size_t out_elems, dy_bytes, x_bytes;
 };
 
-// Backward-filter.  GEMM columns are ordered tap-major, (r', s', c) with c padded to Cp, so that the
-// 16-column groups a thread loads share one filter tap: the input displacement and the bounds test
-// are then per group, not per element, and successive channels differ by a wave-uniform offset.
-// TPT = number of column groups of a tile that may belong to different taps (BN / gcd(BN, Cp)).
-// The partial tiles are summed over the splits and permuted back to [K][C][R][S] by wgrad_reduce_k.
-template <int BM, int TPT>
-__global__ __launch_bounds__(kGemmThreads, 2) void conv_wgrad_k(FilterGrad p)
+// TPT = number of column groups of a tile that may belong to different taps (BN / gcd(BN, Cp)):
+// the input displacement and the bounds test are per group, not per element.
+template <class T, int TPT>
+__global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_wgrad_k(FilterGrad p)
 {
-    constexpr int BN = BM == 128 ? 128 : 256, WN = BM == 128 ? 2 : 4;
-    constexpr int LDA = BM + 4, LDB = BN + 4;
-    constexpr int NA = BM / 16, NB = BN / 16;  // scalar loads per thread: lanes run along the pixel index
+    constexpr int BM = T::BM, BN = T::BN, LDA = T::LDA, LDB = T::LDB;
+    static_assert(T::THREADS == 256, "lanes run along 16 pixels, 16 rows per pass");
+    constexpr int NA = BM / 16, NB = BN / 16;  // scalar loads per thread
     constexpr int GSZ = NB / TPT;              // loads per tap group
+    static_assert(GSZ * TPT == NB, "TPT must divide the loads per thread");
     __shared__ float As[2][BK * LDA];
     __shared__ float Bs[2][BK * LDB];
 
-    // 1-D grid over (split, tile), tile fastest: the blocks an XCD receives work on neighbouring
-    // tiles of the same slice of the reduction, whatever the ratio of tiles to splits
     unsigned L;
     const unsigned tiles = (unsigned)(p.mtiles * p.ntiles);
     if (!xcd_remap(blockIdx.x, tiles * (unsigned)p.splits, &L)) return;
@@ -222,7 +223,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void conv_wgrad_k(FilterGrad p)
     const int slab_end = min(slab_begin + p.slabs_per_split, p.slabs_total);
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-    const int wm = w / WN, wn = w % WN;
+    const int wm = w / T::WN, wn = w % T::WN;
     const int kl = tid & 15, r0 = tid >> 4;  // reduction row inside the slab; first tile row/column
     const int PQ = p.P * p.Q, HW = p.H * p.W;
 
@@ -293,7 +294,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void conv_wgrad_k(FilterGrad p)
         for (int i = 0; i < NB; i++) Bs[buf][kl * LDB + r0 + 16 * i] = breg[i];
     };
 
-    v16f acc[2][2];
+    v16f acc[T::MI][T::NI];
     zero_acc(acc);
     load(slab_begin);
     store(0);
@@ -301,63 +302,82 @@ __global__ __launch_bounds__(kGemmThreads, 2) void conv_wgrad_k(FilterGrad p)
     int cur = 0;
     for (int slab = slab_begin; slab < slab_end - 1; ++slab) {
         load(slab + 1);
-        mma_slab<BK, LDA, LDB>(As[cur], Bs[cur], wm * 64, wn * 64, acc, lane);
+        mma_slab<BK, LDA, LDB>(As[cur], Bs[cur], wm * (BM / T::WM), wn * (BN / T::WN), acc, lane);
         store(cur ^ 1);
         __syncthreads();
         cur ^= 1;
     }
-    mma_slab<BK, LDA, LDB>(As[cur], Bs[cur], wm * 64, wn * 64, acc, lane);
+    mma_slab<BK, LDA, LDB>(As[cur], Bs[cur], wm * (BM / T::WM), wn * (BN / T::WN), acc, lane);
 
     float *outp = p.out + (size_t)split * p.out_elems;
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+    for (int j = 0; j < T::NI; j++) {
+        const int col = n0 + wn * (BN / T::WN) + j * 32 + (lane & 31);
         if (col >= p.ncols) continue;
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int i = 0; i < T::MI; i++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int m = m0 + wm * 64 + i * 32 + acc_row(v, lane);
+                const int m = m0 + wm * (BM / T::WM) + i * 32 + acc_row(v, lane);
                 if (m < p.K) outp[(size_t)m * p.ncols + col] = acc[i][j][v];
             }
     }
 }
 
-// dw[k][c][tap] = sum_s partial[s][k][tap*Cp + c], summed in a fixed order (reproducible).  Block
-// (k, 16-channel chunk) reads tap rows coalesced, stages them in LDS and writes its 16*taps outputs
-// contiguously.  Eight independent partial sums per element keep eight loads in flight: the split
-// count reaches the hundreds for the wide early layers and a single dependent chain would be
-// latency-bound.
-__global__ __launch_bounds__(256) void wgrad_reduce_k(int K, int C, int Cp, int taps, int splits, size_t split_stride,
-                                                       const float *partial, float *dw)
+// dw[k][c][tap] = sum_s partial[s][k][tap*Cp + c], summed in a fixed order (reproducible).
+// Block (k, chunk of `ch` channels): 64 element lanes x 4 split lanes.  Wavefront sl folds the
+// splits s = sl, sl+4, ... of every element with four independent chains (the split count reaches
+// the hundreds for the wide early layers, one dependent chain per element would be latency
+// bound); the four wavefront sums are then added in order, and the chunk is written out
+// contiguously in [c][tap] order.
+__global__ __launch_bounds__(256) void wgrad_reduce_k(int K, int C, int Cp, int taps, int ch, int splits,
+                                                       size_t split_stride, const float *partial, float *dw)
 {
-    extern __shared__ float stage[];  // [16][taps]
-    const int k = blockIdx.x, c0 = blockIdx.y * 16;
-    const int nc = min(16, C - c0);
+    extern __shared__ float lds[];  // part[4][ch*taps] then stage[ch*taps]
+    const int k = blockIdx.x, c0 = blockIdx.y * ch;
+    const int nc = min(ch, C - c0);
+    const int nelem = nc * taps, cap = ch * taps;
+    float *part = lds, *stage = lds + 4 * cap;
+    const int el = threadIdx.x & 63, sl = threadIdx.x >> 6;
     const float *src = partial + (size_t)k * taps * Cp + c0;
-    for (int i = threadIdx.x; i < nc * taps; i += 256) {
+    for (int i = el; i < nelem; i += 64) {
         const int t = i / nc, c = i - t * nc;
         const float *q = src + (size_t)t * Cp + c;
-        float a[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        int sp = 0;
-        for (; sp + 8 <= splits; sp += 8) {
-#pragma unroll
-            for (int u = 0; u < 8; u++) a[u] += q[(size_t)(sp + u) * split_stride];
+        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+        int sp = sl;
+        for (; sp + 12 < splits; sp += 16) {
+            a0 += q[(size_t)sp * split_stride];
+            a1 += q[(size_t)(sp + 4) * split_stride];
+            a2 += q[(size_t)(sp + 8) * split_stride];
+            a3 += q[(size_t)(sp + 12) * split_stride];
         }
-        for (int u = 0; sp < splits; sp++, u++) a[u] += q[(size_t)sp * split_stride];
-        stage[c * taps + t] = ((a[0] + a[1]) + (a[2] + a[3])) + ((a[4] + a[5]) + (a[6] + a[7]));
+        for (; sp < splits; sp += 4) a0 += q[(size_t)sp * split_stride];
+        part[sl * cap + i] = (a0 + a1) + (a2 + a3);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < nelem; i += 256) {
+        const int t = i / nc, c = i - t * nc;
+        stage[c * taps + t] = (part[i] + part[cap + i]) + (part[2 * cap + i] + part[3 * cap + i]);
     }
     __syncthreads();
     float *dst = dw + ((size_t)k * C + c0) * taps;
-    for (int i = threadIdx.x; i < nc * taps; i += 256) dst[i] = stage[i];
+    for (int i = threadIdx.x; i < nelem; i += 256) dst[i] = stage[i];
 }
 
+// ------------------------------------------------------------------------------------ helpers
+
 // out[i] = sum_s partial[s][i], s ascending.
-__global__ __launch_bounds__(256) void splitk_reduce_k(size_t n, int splits, const float *partial, float *out)
+__global__ __launch_bounds__(256) void splitk_reduce_k(size_t n4, int splits, const float4 *partial, float4 *out)
 {
-    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
-        float acc = partial[i];
-        for (int s = 1; s < splits; s++) acc += partial[(size_t)s * n + i];
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (size_t)gridDim.x * 256) {
+        float4 acc = partial[i];
+        for (int s = 1; s < splits; s++) {
+            const float4 v = partial[(size_t)s * n4 + i];
+            acc.x += v.x;
+            acc.y += v.y;
+            acc.z += v.z;
+            acc.w += v.w;
+        }
         out[i] = acc;
     }
 }
@@ -404,10 +424,11 @@ __global__ __launch_bounds__(256) void pack_bwd_k(int K, int C, int taps, int KP
 
 int round_up(int v, int to) { return (v + to - 1) / to * to; }
 
-int pick_splits(int tiles, int slabs_total, int cap = 64)
+// Reduction splits so that about `blocks_wanted` workgroups exist, at least 4 slabs each.
+int pick_splits(int tiles, int slabs_total, int blocks_wanted, int cap)
 {
-    int want = (2 * num_cus() + tiles - 1) / tiles;      // aim at two workgroups per CU
-    int max_by_depth = slabs_total / 4 > 0 ? slabs_total / 4 : 1;  // keep >= 4 slabs per split
+    int want = (blocks_wanted + tiles - 1) / tiles;
+    int max_by_depth = slabs_total / 4 > 0 ? slabs_total / 4 : 1;
     int s = want < max_by_depth ? want : max_by_depth;
     if (s > cap) s = cap;
     return s < 1 ? 1 : s;
@@ -427,6 +448,23 @@ int check_desc(const dopt_hip_conv_desc *d, size_t *P, size_t *Q, const char *wh
                  "%s: tensors of 2^29 elements or more are not supported", who);
     return DOPT_HIP_OK;
 }
+
+int launch_splitk_reduce(size_t elems, int splits, const float *partial, float *out)
+{
+    // float4 passes: the caller only splits when elems % 4 == 0, and the partial copies start on
+    // 256-byte boundaries of the workspace; `out` comes from the pool or is checked by the caller
+    const size_t n4 = elems / 4;
+    size_t blocks = ceil_div(n4, (size_t)256);
+    size_t cap = (size_t)num_cus() * 8;
+    hipLaunchKernelGGL(splitk_reduce_k, dim3((unsigned)(blocks > cap ? cap : (blocks < 1 ? 1 : blocks))), dim3(256), 0,
+                       stream(), n4, splits, (const float4 *)partial, (float4 *)out);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+using GatherWide = Tile<64, 256, 1, 4>;     // few output channels, many pixels
+using GatherSquare = Tile<128, 128, 2, 2>;  // enough tiles for two workgroups per CU
+using GatherDeep = Tile<128, 128, 2, 4>;    // few tiles: 8 wavefronts per workgroup, one workgroup per CU
 
 // Shared host driver of forward (kBwd = false) and backward-data (kBwd = true).
 template <bool kBwd>
@@ -453,12 +491,24 @@ int run_gather(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in,
     g.ncols = g.N * g.OH * g.OW;
     g.slabs_total = taps * g.CinPad / BK;
     g.out_elems = (size_t)g.ncols * g.Mout;
-    const bool big = g.Mout > 64;
-    const int BM = big ? 128 : 64, BN = big ? 128 : 256;
+
+    // tile shape: wide tiles for <= 64 output channels; otherwise 128x128, with 8 wavefronts per
+    // workgroup when there are too few tiles to give every CU two 4-wavefront workgroups
+    enum { kWide, kSquare, kDeep } shape;
+    int BM, BN, blocks_wanted;
+    if (g.Mout <= 64) {
+        shape = kWide; BM = 64; BN = 256; blocks_wanted = 2 * num_cus();
+    } else {
+        BM = 128; BN = 128;
+        const int t = ((g.Mout + 127) / 128) * ((g.ncols + 127) / 128);
+        if (t >= 2 * num_cus()) { shape = kSquare; blocks_wanted = 2 * num_cus(); }
+        else { shape = kDeep; blocks_wanted = num_cus(); }
+    }
     g.mtiles = (g.Mout + BM - 1) / BM;
     g.ntiles = (g.ncols + BN - 1) / BN;
     const int tiles = g.mtiles * g.ntiles;
-    int splits = pick_splits(tiles, g.slabs_total);
+    int splits = pick_splits(tiles, g.slabs_total, blocks_wanted, 64);
+    if (g.out_elems % 4 != 0 || !aligned16(out)) splits = 1;  // the split reduction works on float4
     g.slabs_per_split = (g.slabs_total + splits - 1) / splits;
     splits = (g.slabs_total + g.slabs_per_split - 1) / g.slabs_per_split;  // no empty split
     g.splits = splits;
@@ -490,20 +540,24 @@ int run_gather(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in,
     g.wp_bytes = wp_elems * sizeof(float);
     g.out = splits > 1 ? partial : out;
     dim3 grid(xcd_grid((unsigned)(tiles * splits)));
-    if (big)
-        hipLaunchKernelGGL((conv_gather_k<128, kBwd>), grid, dim3(kGemmThreads), 0, stream(), g);
-    else
-        hipLaunchKernelGGL((conv_gather_k<64, kBwd>), grid, dim3(kGemmThreads), 0, stream(), g);
+    const int mode = !kBwd ? 0 : (g.strideH == 1 && g.strideW == 1 ? 1 : 2);
+#define DOPT_GATHER(TILE)                                                                                      \
+    do {                                                                                                       \
+        if (mode == 0) hipLaunchKernelGGL((conv_gather_k<TILE, 0>), grid, dim3(TILE::THREADS), 0, stream(), g); \
+        else if (mode == 1) hipLaunchKernelGGL((conv_gather_k<TILE, 1>), grid, dim3(TILE::THREADS), 0, stream(), g); \
+        else hipLaunchKernelGGL((conv_gather_k<TILE, 2>), grid, dim3(TILE::THREADS), 0, stream(), g);          \
+    } while (0)
+    if (shape == kWide) DOPT_GATHER(GatherWide);
+    else if (shape == kSquare) DOPT_GATHER(GatherSquare);
+    else DOPT_GATHER(GatherDeep);
+#undef DOPT_GATHER
     DOPT_LAUNCH_CHECK();
-    if (splits > 1) {
-        size_t blocks = ceil_div(g.out_elems, (size_t)256);
-        size_t cap = (size_t)num_cus() * 8;
-        hipLaunchKernelGGL(splitk_reduce_k, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0, stream(),
-                           g.out_elems, splits, partial, out);
-        DOPT_LAUNCH_CHECK();
-    }
+    if (splits > 1) return launch_splitk_reduce(g.out_elems, splits, partial, out);
     return DOPT_HIP_OK;
 }
+
+using WgradSquare = Tile<128, 128, 2, 2>;
+using WgradNarrow = Tile<64, 128, 1, 4>;  // K <= 64
 
 }  // namespace
 
@@ -548,12 +602,12 @@ int dopt_hip_conv_bwd_filter(const dopt_hip_conv_desc *d, const float *dy, const
     f.x_bytes = (size_t)f.N * f.C * f.H * f.W * sizeof(float);
     f.slabs_total = (f.npix + BK - 1) / BK;
     const bool big = f.K > 64;
-    const int BM = big ? 128 : 64, BN = big ? 128 : 256;
+    const int BM = big ? 128 : 64, BN = 128;
     f.mtiles = (f.K + BM - 1) / BM;
     f.ntiles = (f.ncols + BN - 1) / BN;
     const int tiles = f.mtiles * f.ntiles;
     // filter gradients are short and wide (small output, long pixel reduction): allow deep splits
-    int splits = pick_splits(tiles, f.slabs_total, 512);
+    int splits = pick_splits(tiles, f.slabs_total, 2 * num_cus(), 512);
     f.slabs_per_split = (f.slabs_total + splits - 1) / splits;
     splits = (f.slabs_total + f.slabs_per_split - 1) / f.slabs_per_split;
     f.splits = splits;
@@ -563,26 +617,27 @@ int dopt_hip_conv_bwd_filter(const dopt_hip_conv_desc *d, const float *dy, const
     // column groups of one tile that can fall on different taps
     int gw = BN;
     while (f.Cp % gw != 0) gw /= 2;  // largest power-of-two divisor of Cp not above BN (>= 16)
-    int tpt = BN / gw;
-    if (tpt > 4) tpt = BN / 16;      // instantiated: 1, 2, 4 and one group per load
+    const int tpt = BN / gw;         // 1, 2, 4 or 8
     dim3 grid(xcd_grid((unsigned)(tiles * splits)));
-#define DOPT_WGRAD(BMV, TPTV) hipLaunchKernelGGL((conv_wgrad_k<BMV, TPTV>), grid, dim3(kGemmThreads), 0, stream(), f)
+#define DOPT_WGRAD(TILE, TPTV) hipLaunchKernelGGL((conv_wgrad_k<TILE, TPTV>), grid, dim3(TILE::THREADS), 0, stream(), f)
     if (big) {
-        if (tpt == 1) DOPT_WGRAD(128, 1);
-        else if (tpt == 2) DOPT_WGRAD(128, 2);
-        else if (tpt == 4) DOPT_WGRAD(128, 4);
-        else DOPT_WGRAD(128, 8);
+        if (tpt == 1) DOPT_WGRAD(WgradSquare, 1);
+        else if (tpt == 2) DOPT_WGRAD(WgradSquare, 2);
+        else if (tpt == 4) DOPT_WGRAD(WgradSquare, 4);
+        else DOPT_WGRAD(WgradSquare, 8);
     } else {
-        if (tpt == 1) DOPT_WGRAD(64, 1);
-        else if (tpt == 2) DOPT_WGRAD(64, 2);
-        else if (tpt == 4) DOPT_WGRAD(64, 4);
-        else DOPT_WGRAD(64, 16);
+        if (tpt == 1) DOPT_WGRAD(WgradNarrow, 1);
+        else if (tpt == 2) DOPT_WGRAD(WgradNarrow, 2);
+        else if (tpt == 4) DOPT_WGRAD(WgradNarrow, 4);
+        else DOPT_WGRAD(WgradNarrow, 8);
     }
 #undef DOPT_WGRAD
     DOPT_LAUNCH_CHECK();
-    dim3 rgrid((unsigned)f.K, (unsigned)((f.C + 15) / 16));
-    hipLaunchKernelGGL(wgrad_reduce_k, rgrid, dim3(256), (size_t)16 * taps * sizeof(float), stream(), f.K, f.C, f.Cp,
-                       taps, splits, f.out_elems, partial, dw);
+    // 64-channel chunks when that still leaves >= 1024 workgroups and the LDS staging stays small
+    const int ch = ((size_t)f.K * ((f.C + 63) / 64) >= 1024 && taps <= 16) ? 64 : 16;
+    dim3 rgrid((unsigned)f.K, (unsigned)((f.C + ch - 1) / ch));
+    hipLaunchKernelGGL(wgrad_reduce_k, rgrid, dim3(256), (size_t)5 * ch * taps * sizeof(float), stream(), f.K, f.C,
+                       f.Cp, taps, ch, splits, f.out_elems, partial, dw);
     DOPT_LAUNCH_CHECK();
     return DOPT_HIP_OK;
 }

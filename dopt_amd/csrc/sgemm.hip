@@ -14,6 +14,7 @@ namespace {
 using namespace dopt;
 
 constexpr int BK = 16;
+constexpr int kGemmThreads = 256;
 
 struct Gemm {
     const float *A, *B;
