@@ -157,3 +157,36 @@ def vgg(features, extractor_sizes, dense_sizes, init, batchnorm=True):   # nnet/
 
 def vgg16(features, dense_sizes=(4096, 4096), init=None, batchnorm=True):
     return vgg(features, VGG16_SIZES, dense_sizes, init or Init(0), batchnorm)
+
+
+def _wrn_block(in_layer, u, n, s, init, weight_decay):   # nnet/models/wrn.d:104-200
+    res = None
+    for _ in range(n):
+        res = relu(batchNorm(in_layer))
+        res = conv2D(res, u, [3, 3], init, padding=(1, 1), stride=(s, s), use_bias=False, weight_decay=weight_decay)
+        res = relu(batchNorm(res))
+        res = conv2D(res, u, [3, 3], init, padding=(1, 1), use_bias=False, weight_decay=weight_decay)
+        shortcut = in_layer
+        if in_layer.output.shape[1] != res.output.shape[1]:
+            # 1x1 projection taken from the block INPUT (before its batch norm), no padding
+            shortcut = conv2D(in_layer, u, [1, 1], init, stride=(s, s), use_bias=False, weight_decay=weight_decay)
+        res = Layer([res, shortcut], res.output + shortcut.output, res.trainOutput + shortcut.trainOutput, [])
+        in_layer, s = res, 1
+    return res
+
+
+def meanPool(inp):   # nnet/models/wrn.d:202-219: a row sum (rewritten to a GEMV by `sum`) times 1/(H*W)
+    def impl(x):
+        n, c, hw = x.shape[0], x.shape[1], x.shape[2] * x.shape[3]
+        return core.sum(x.reshape([n * c, hw]), [1]).reshape([n, c]) * (1.0 / hw)
+    return Layer([inp], impl(inp.output), impl(inp.trainOutput), [])
+
+
+def wideResNet(features, depth, width, init=None, weight_decay=0.0001, stride=(1, 2, 2), base=16):
+    """nnet/models/wrn.d:56-102 with the default options (no dropout, no norm constraints)."""
+    init = init or Init(0)
+    n = (depth - 4) // 6
+    pred = conv2D(dataSource(features), base, [3, 3], init, padding=(1, 1), use_bias=False, weight_decay=weight_decay)
+    for mult, s in zip((1, 2, 4), stride):
+        pred = _wrn_block(pred, base * mult * width, n, s, init, weight_decay)
+    return meanPool(relu(batchNorm(pred)))

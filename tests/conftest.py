@@ -11,6 +11,13 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+    # Load what is built; build only when nothing is there (hipcc cross-compiles without a GPU).
+    # A missing library is an error, never a reason to skip or to fall back.
+    from dopt_amd import build as hip_build
+    if not os.path.exists(hip_build.LIB_PATH):
+        hip_build.build()
+    import oracle
+    oracle.build()          # no-op when liboracle.so exists
 
 
 @pytest.fixture(scope="session")

@@ -12,7 +12,7 @@ from util import assert_close
 
 pytestmark = pytest.mark.gpu
 
-core = pytest.importorskip("dopt_amd.core")
+from dopt_amd import core
 from dopt_amd import capi, nnet, online, ops  # noqa: E402
 from dopt_amd.core import (evaluate, float32, float32Constant, grad, int32)  # noqa: E402
 

@@ -13,7 +13,7 @@ from util import assert_close, ulp_diff
 
 pytestmark = pytest.mark.gpu
 
-ops = pytest.importorskip("dopt_amd.ops")
+from dopt_amd import ops
 T = ops.tensor
 
 
