@@ -1,0 +1,123 @@
+"""Per-kernel throughput of the bandwidth-bound entry points against the HBM roofline.
+
+    python -m dopt_amd.kernel_bench [--iters 50] [--json]
+
+Each row times one C-ABI entry point at a shape taken from the benchmark configurations (the
+VGG-16 b128 activations, the 16M-parameter fused update) with HIP events on the library's stream
+and reports ALGORITHMIC bytes / time: every tensor counted once per kernel, whatever the kernel
+really moves (a two-pass batch norm reads its input twice but is charged 8 B/element).
+"""
+import argparse
+import ctypes as C
+import json
+
+import numpy as np
+
+from . import capi, ops, workloads
+
+HBM_PEAK = 8.0e12
+
+
+def _time(fn, iters, warm=5):
+    lib = capi.load()
+    ev = [C.c_void_p(), C.c_void_p()]
+    for e in ev:
+        capi.check(lib.dopt_hip_event_create(C.byref(e)))
+    for _ in range(warm):
+        fn()
+    capi.check(lib.dopt_hip_event_record(ev[0]))
+    for _ in range(iters):
+        fn()
+    capi.check(lib.dopt_hip_event_record(ev[1]))
+    ms = C.c_float()
+    capi.check(lib.dopt_hip_event_elapsed_ms(ev[0], ev[1], C.byref(ms)))
+    for e in ev:
+        lib.dopt_hip_event_destroy(e)
+    return ms.value * 1e-3 / iters
+
+
+def _rand(shape, seed=0):
+    return ops.tensor(np.random.default_rng(seed).standard_normal(shape, dtype=np.float32))
+
+
+def cases():
+    """(name, shape text, algorithmic bytes, callable) per row.  Every callable writes into an output
+    tensor allocated once, before the timed loop, so a row times the kernels of one entry point only."""
+    rows, keep = [], []
+
+    def add(name, shape, nbytes, fn):
+        o = fn(None)                                         # the first call allocates the output ...
+        keep.append(o)
+        rows.append((name, shape, nbytes, lambda: fn(o)))   # ... every later call reuses it
+
+    act = (128, 64, 32, 32)                      # the largest VGG activation: 8.39 M elements, 33.5 MB
+    n = int(np.prod(act))
+    x, dy = _rand(act, 1), _rand(act, 2)
+    fa, fb = x.reshape((n,)), dy.reshape((n,))
+    add("pointwise add", "%d" % n, 12 * n, lambda o: ops.pointwise("add", fa, fb, out=o))
+    add("pointwise mul", "%d" % n, 12 * n, lambda o: ops.pointwise("mul", fa, fb, out=o))
+    add("pointwise abs", "%d" % n, 8 * n, lambda o: ops.pointwise("abs", fa, out=o))
+    add("pointwise exp", "%d" % n, 8 * n, lambda o: ops.pointwise("exp", fa, out=o))
+    add("relu", str(act), 8 * n, lambda o: ops.relu(x, out=o))
+    add("reluGrad", str(act), 12 * n, lambda o: ops.relu_grad(dy, x, out=o))
+    bias = _rand((64,), 3)
+    add("addBias", str(act), 8 * n, lambda o: ops.add_bias(x, bias, out=o))
+    add("addBiasGrad", str(act), 4 * n, lambda o: ops.add_bias_grad(dy, out=o))
+    add("maxpool 2x2", str(act), 5 * n, lambda o: ops.maxpool(x, (2, 2), out=o))
+    pdy = _rand((128, 64, 16, 16), 4)
+    add("maxpoolGrad 2x2", str(act), 9 * n, lambda o: ops.maxpool_grad(pdy, x, (2, 2), out=o))
+    g, b, rm, rv = (_rand((64,), 5 + i) for i in range(4))
+    rv.set(np.abs(rv.numpy()) + 0.5)
+    add("batchNormTrain", str(act), 8 * n, lambda o: ops.bn_train(x, g, b, rm, rv, 0.9, out=o))
+    add("batchNormGrad", str(act), 12 * n, lambda o: ops.bn_grad(dy, x, g, out=o))
+    add("batchNormInference", str(act), 8 * n, lambda o: ops.bn_infer(x, g, b, rm, rv, out=o))
+    add("sum (all axes)", str(act), 4 * n, lambda o: ops.sum(x, out=o))
+    add("sum axes [0,2,3]", str(act), 4 * n, lambda o: ops.sum(x, [0, 2, 3], out=o))
+    add("maxElement (all axes)", str(act), 4 * n, lambda o: ops.max_element(x, out=o))
+    m2 = x.reshape((4096, 2048))
+    add("transpose", "(4096, 2048)", 8 * n, lambda o: ops.transpose(m2, out=o))
+    add("argmin axis 1", "(4096, 2048)", 4 * n, lambda o: ops.argmin(m2, 1, out=o))
+    sm = _rand((65536, 128), 9)
+    add("softmax", "(65536, 128)", 8 * sm.size, lambda o: ops.softmax(sm, out=o))
+    add("slice (contiguous)", "%d -> %d" % (n, n - 128), 8 * (n - 128), lambda o: ops.slice(fa, [0], [n - 128], out=o))
+    add("slice (4-d interior)", "%s -> (128, 64, 30, 30)" % (act,), 8 * 128 * 64 * 900,
+        lambda o: ops.slice(x, [0, 0, 1, 1], [128, 64, 31, 31], out=o))
+    add("pad (1-d tail)", "%d + 128" % n, 8 * n, lambda o: ops.pad(fa, [0], [128], out=o))
+    add("repeat", "%s x [1,1,2,2]" % (act,), 20 * n, lambda o: ops.repeat(x, [1, 1, 2, 2], out=o))
+
+    # the fused multi-tensor updates over the 16 777 216-parameter, 40-tensor workload
+    st = workloads.adam16m_state(0)
+    tw, tg, tm, tv, tvh = ([ops.tensor(s[k]) for s in st] for k in ("w", "g", "m", "v", "vhat"))
+    total = workloads.ADAM16M_TOTAL
+    sgd = ops.FusedOptimizer(tw, tg, tm)
+    adam = ops.FusedOptimizer(tw, tg, tm, tv)
+    ams = ops.FusedOptimizer(tw, tg, tm, tv, tvh)
+    rows.append(("fused SGD (40 tensors)", "%d" % total, 20 * total, lambda: sgd.sgd(0.01, 0.9, False)))
+    rows.append(("fused ADAM (40 tensors)", "%d" % total, 28 * total, lambda: adam.adam(1e-3, 0.9, 0.999, 1e-8)))
+    rows.append(("fused AMSGrad (40 tensors)", "%d" % total, 36 * total, lambda: ams.amsgrad(1e-3, 0.9, 0.999, 1e-8)))
+    keep.extend([x, dy, bias, pdy, g, b, rm, rv, sm, tw, tg, tm, tv, tvh, sgd, adam, ams])
+    return rows, keep
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--iters", type=int, default=50)
+    ap.add_argument("--json", action="store_true")
+    args = ap.parse_args()
+    out = []
+    rows, keep = cases()
+    for name, shape, nbytes, fn in rows:
+        sec = _time(fn, args.iters)
+        out.append({"kernel": name, "shape": shape, "us": sec * 1e6, "GB/s": nbytes / sec / 1e9,
+                    "frac_of_8TB/s": nbytes / sec / HBM_PEAK})
+    ops.sync()
+    if args.json:
+        print(json.dumps(out))
+        return
+    print("%-28s %-40s %10s %10s %8s" % ("kernel", "shape", "us", "GB/s", "of peak"))
+    for r in out:
+        print("%-28s %-40s %10.1f %10.0f %7.1f%%" % (r["kernel"], r["shape"], r["us"], r["GB/s"], 100 * r["frac_of_8TB/s"]))
+
+
+if __name__ == "__main__":
+    main()

@@ -92,10 +92,20 @@ def sync():
     capi.check(capi.load().dopt_hip_sync())
 
 
+def _out(out, shape, dtype=np.float32):
+    """The result tensor: a fresh zero-filled pooled buffer, or the caller's (a kernel's `execute`
+    is handed its output buffer by the plan, cuda/package.d:68-79)."""
+    if out is None:
+        return Tensor(shape, dtype)
+    if _vol(out.shape) != _vol(shape) or out.dtype != np.dtype(dtype):
+        raise capi.HipError(1, "output buffer has the wrong size or type")
+    return out
+
+
 # ------------------------------------------------------------------------------- pointwise
 
-def pointwise(op, a, b=None):
-    out = Tensor(a.shape, a.dtype)
+def pointwise(op, a, b=None, out=None):
+    out = _out(out, a.shape, a.dtype)
     if b is not None and (b.shape != a.shape or b.dtype != a.dtype):
         raise capi.HipError(1, "pointwise operands must have the same type")
     capi.check(capi.load().dopt_hip_pointwise(op.encode(), a.code, a.size, a.ptr, b.ptr if b is not None else None,
@@ -103,73 +113,73 @@ def pointwise(op, a, b=None):
     return out
 
 
-def _reduce(name, a, axes):
+def _reduce(name, a, axes, out=None):
     axes = list(range(len(a.shape))) if not axes else [int(x) for x in axes]
     oshape = [s for i, s in enumerate(a.shape) if i not in axes]
-    out = Tensor(oshape, a.dtype)
+    out = _out(out, oshape, a.dtype)
     capi.check(capi.load().dopt_hip_reduce(name, a.code, capi.sizes(a.shape), len(a.shape), capi.sizes(axes),
                                            len(axes), a.ptr, out.ptr))
     return out
 
 
-def sum(a, axes=None):  # noqa: A001 - reference op name
-    return _reduce(b"sum", a, axes)
+def sum(a, axes=None, out=None):  # noqa: A001 - reference op name
+    return _reduce(b"sum", a, axes, out)
 
 
-def max_element(a, axes=None):
-    return _reduce(b"maxElement", a, axes)
+def max_element(a, axes=None, out=None):
+    return _reduce(b"maxElement", a, axes, out)
 
 
-def argmin(a, axis):
+def argmin(a, axis, out=None):
     oshape = list(a.shape)
     oshape[axis] = 1
-    out = Tensor(oshape, np.int32)
+    out = _out(out, oshape, np.int32)
     capi.check(capi.load().dopt_hip_argmin(a.code, capi.sizes(a.shape), len(a.shape), axis, a.ptr, out.ptr))
     return out
 
 
 # ------------------------------------------------------------------------------- layout
 
-def slice(a, start, stop):  # noqa: A001
+def slice(a, start, stop, out=None):  # noqa: A001
     oshape = [e - s for s, e in zip(start, stop)]
-    out = Tensor(oshape, a.dtype)
+    out = _out(out, oshape, a.dtype)
     capi.check(capi.load().dopt_hip_slice(len(a.shape), capi.sizes(a.shape), capi.sizes(oshape), capi.sizes(start),
                                           a.ptr, out.ptr))
     return out
 
 
-def pad(a, before, after):
+def pad(a, before, after, out=None):
     oshape = [b + s + e for b, s, e in zip(before, a.shape, after)]
-    out = Tensor(oshape, a.dtype)
+    out = _out(out, oshape, a.dtype)
     capi.check(capi.load().dopt_hip_pad(len(a.shape), capi.sizes(a.shape), capi.sizes(oshape), capi.sizes(before),
                                         a.ptr, out.ptr))
     return out
 
 
-def repeat(a, reps):
+def repeat(a, reps, out=None):
     oshape = [s * r for s, r in zip(a.shape, reps)]
-    out = Tensor(oshape, a.dtype)
+    out = _out(out, oshape, a.dtype)
     capi.check(capi.load().dopt_hip_repeat(len(a.shape), capi.sizes(a.shape), capi.sizes(reps), a.ptr, out.ptr))
     return out
 
 
-def transpose(a):
+def transpose(a, out=None):
     rows, cols = a.shape
-    out = Tensor((cols, rows), a.dtype)
+    out = _out(out, (cols, rows), a.dtype)
     capi.check(capi.load().dopt_hip_transpose2d(rows, cols, a.ptr, out.ptr))
     return out
 
 
 # ------------------------------------------------------------------------------- dense / conv
 
-def matmul(a, b):
+def matmul(a, b, out=None):
     if a.dtype != np.float32 or b.dtype != np.float32:
         raise capi.HipError(3, "Element type not supported.")
     M, K = a.shape
     K2, N = b.shape
     if K != K2:
         raise capi.HipError(1, "matmul: inner dimensions differ")
-    out = Tensor((M, N))
+    out = _out(out, (M, N))
     capi.check(capi.load().dopt_hip_sgemm(M, N, K, a.ptr, b.ptr, out.ptr))
     return out
 
@@ -186,27 +196,27 @@ def conv_out_shape(d):
     return (d.N, d.K, (d.H + 2 * d.padH - d.R) // d.strideH + 1, (d.W + 2 * d.padW - d.S) // d.strideW + 1)
 
 
-def convolution(x, w, padding=(0, 0), stride=(1, 1)):
+def convolution(x, w, padding=(0, 0), stride=(1, 1), out=None):
     d = conv_desc(x.shape, w.shape, padding, stride)
-    y = Tensor(conv_out_shape(d))
+    y = _out(out, conv_out_shape(d))
     capi.check(capi.load().dopt_hip_conv_fwd(C.byref(d), x.ptr, w.ptr, y.ptr))
     return y
 
 
-def conv_bwd_data(dy, w, xshape, padding=(0, 0), stride=(1, 1)):
+def conv_bwd_data(dy, w, xshape, padding=(0, 0), stride=(1, 1), out=None):
     d = conv_desc(xshape, w.shape, padding, stride)
     if tuple(dy.shape) != conv_out_shape(d):
         raise capi.HipError(1, "convolutionFeaturesGrad: gradient shape does not match")
-    dx = Tensor(xshape)
+    dx = _out(out, xshape)
     capi.check(capi.load().dopt_hip_conv_bwd_data(C.byref(d), dy.ptr, w.ptr, dx.ptr))
     return dx
 
 
-def conv_bwd_filter(dy, x, wshape, padding=(0, 0), stride=(1, 1)):
+def conv_bwd_filter(dy, x, wshape, padding=(0, 0), stride=(1, 1), out=None):
     d = conv_desc(x.shape, wshape, padding, stride)
     if tuple(dy.shape) != conv_out_shape(d):
         raise capi.HipError(1, "convolutionFiltersGrad: gradient shape does not match")
-    dw = Tensor(wshape)
+    dw = _out(out, wshape)
     capi.check(capi.load().dopt_hip_conv_bwd_filter(C.byref(d), dy.ptr, x.ptr, dw.ptr))
     return dw
 
@@ -218,73 +228,73 @@ def _nci(shape):
     return shape[0], shape[1], inner
 
 
-def maxpool(x, dims):
+def maxpool(x, dims, out=None):
     N, Cc, H, W = x.shape
-    y = Tensor((N, Cc, H // dims[0], W // dims[1]))
+    y = _out(out, (N, Cc, H // dims[0], W // dims[1]))
     capi.check(capi.load().dopt_hip_maxpool_fwd(N, Cc, H, W, dims[0], dims[1], x.ptr, y.ptr))
     return y
 
 
-def maxpool_grad(dy, x, dims):
+def maxpool_grad(dy, x, dims, out=None):
     N, Cc, H, W = x.shape
-    dx = Tensor(x.shape)
+    dx = _out(out, x.shape)
     capi.check(capi.load().dopt_hip_maxpool_bwd(N, Cc, H, W, dims[0], dims[1], dy.ptr, x.ptr, dx.ptr))
     return dx
 
 
-def softmax(x):
-    y = Tensor(x.shape)
+def softmax(x, out=None):
+    y = _out(out, x.shape)
     capi.check(capi.load().dopt_hip_softmax_fwd(*_nci(x.shape), x.ptr, y.ptr))
     return y
 
 
-def softmax_grad(dy, y):
-    dx = Tensor(y.shape)
+def softmax_grad(dy, y, out=None):
+    dx = _out(out, y.shape)
     capi.check(capi.load().dopt_hip_softmax_bwd(*_nci(y.shape), dy.ptr, y.ptr, dx.ptr))
     return dx
 
 
-def relu(x):
-    y = Tensor(x.shape)
+def relu(x, out=None):
+    y = _out(out, x.shape)
     capi.check(capi.load().dopt_hip_relu_fwd(x.size, x.ptr, y.ptr))
     return y
 
 
-def relu_grad(dy, x):
-    dx = Tensor(x.shape)
+def relu_grad(dy, x, out=None):
+    dx = _out(out, x.shape)
     capi.check(capi.load().dopt_hip_relu_bwd(x.size, dy.ptr, x.ptr, dx.ptr))
     return dx
 
 
-def add_bias(x, b):
-    y = Tensor(x.shape)
+def add_bias(x, b, out=None):
+    y = _out(out, x.shape)
     capi.check(capi.load().dopt_hip_bias_fwd(*_nci(x.shape), x.ptr, b.ptr, y.ptr))
     return y
 
 
-def add_bias_grad(dy):
-    db = Tensor((dy.shape[1],))
+def add_bias_grad(dy, out=None):
+    db = _out(out, (dy.shape[1],))
     capi.check(capi.load().dopt_hip_bias_bwd(*_nci(dy.shape), dy.ptr, db.ptr))
     return db
 
 
-def bn_train(x, scale, bias, run_mean, run_var, momentum):
+def bn_train(x, scale, bias, run_mean, run_var, momentum, out=None):
     N, Cc, inner = _nci(x.shape)
-    packed = Tensor((x.size + 2 * Cc,))
+    packed = _out(out, (x.size + 2 * Cc,))
     capi.check(capi.load().dopt_hip_bn_train(N, Cc, inner, float(momentum), x.ptr, scale.ptr, bias.ptr, run_mean.ptr,
                                              run_var.ptr, packed.ptr))
     return packed
 
 
-def bn_grad(dy, x, scale):
+def bn_grad(dy, x, scale, out=None):
     N, Cc, inner = _nci(x.shape)
-    packed = Tensor((x.size + 2 * Cc,))
+    packed = _out(out, (x.size + 2 * Cc,))
     capi.check(capi.load().dopt_hip_bn_grad(N, Cc, inner, dy.ptr, x.ptr, scale.ptr, packed.ptr))
     return packed
 
 
-def bn_infer(x, scale, bias, mean, var):
-    y = Tensor(x.shape)
+def bn_infer(x, scale, bias, mean, var, out=None):
+    y = _out(out, x.shape)
     capi.check(capi.load().dopt_hip_bn_infer(*_nci(x.shape), x.ptr, scale.ptr, bias.ptr, mean.ptr, var.ptr, y.ptr))
     return y
 
