@@ -155,7 +155,7 @@ def main():
         gather_tflops = (fwd + bwd_data) / (gather_us * 1e-6) / 1e12
         wgrad_tflops = fwd / (per_step["convolutionFiltersGrad"][0] * 1e-6) / 1e12
         result["roofline"] = {
-            "kernel": "conv_gather_k (implicit-GEMM convolution forward + backward-data)",
+            "kernel": "conv_patch_k (3x3 implicit-GEMM convolution forward + backward-data, incl. filter pack and split reduction)",
             "bound": "mfma", "achieved": round(gather_tflops, 2), "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": round(gather_tflops / MFMA_FP32_PEAK_TFLOPS, 4), "traffic": None,
             "launches_per_step": int(gather_launches),

@@ -184,6 +184,239 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_gather_k(Ga
     }
 }
 
+// ------------------------------------------------------------------------------------ patch (3x3, unit stride)
+//
+// Forward and backward-data of 3x3 unit-stride convolutions.  The gathered operand is not
+// re-fetched per filter tap: for a chunk of 16 input channels the block loads the input patch
+// under its pixel tile ONCE -- the tile's rows plus a one-pixel halo, zero-filled outside the
+// image by the buffer range check -- and the nine taps read it at nine offsets.  LDS holds the
+// patch position-major, Bp[pos][16 channels (+4 pad)], and the filter slab of one tap row-major,
+// As[m][16 channels (+4 pad)], so that a lane's operands for a whole 16-channel slab are two
+// 128-bit LDS reads per 32-wide fragment: lane half kh (= lane / 32) multiplies channels
+// kh*8 .. kh*8+7 of the chunk over the slab's eight matrix steps (the same channel permutation on
+// both operands, so every channel is counted once).  Per 32 matrix instructions a wavefront
+// issues 8 fragment reads, 1-2 filter loads and stores and ~5 patch loads and stores.
+
+struct PatchConv {
+    const float *in;   // gathered operand [N, Cin, IH, IW]
+    const float *wp;   // packed filter [chunks][9][Mp][16]
+    float *out;        // [N, Mout, OH, OW], or `splits` partial copies of it
+    int N, Cin, IH, IW, Mout, OH, OW;
+    int PT, PL;        // input row / column of patch position (0,0) is (oh0 - PT, -PL)
+    int flip;          // 1: tap (tr,ts) reads patch offset (2-tr, 2-ts); 0: (tr, ts)
+    int nimg, rows;    // images per pixel tile; output rows of each image in the tile
+    int PR, PC, psz;   // patch rows and columns per image; patch positions per tile = nimg*PR*PC
+    unsigned magic_psz, magic_img, magic_pc;  // floor(2^32/d)+1 for d = psz, PR*PC, PC (exact for x*d < 2^32)
+    int Mp;            // rows of one packed filter slab (Mout rounded up to the tile height)
+    int ncols, mtiles, ntiles, chunks_total, chunks_per_split, splits;
+    size_t out_elems, in_bytes, wp_bytes;
+};
+
+__device__ inline unsigned fast_div(unsigned x, unsigned magic) { return __umulhi(x, magic); }
+
+template <class T, int NPMAX, bool kCFull>
+__global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_patch_k(PatchConv p)
+{
+    constexpr int BM = T::BM, BN = T::BN, THREADS = T::THREADS, MI = T::MI, NI = T::NI;
+    constexpr int TAPS = 9, CH = 16, LDP = 20;
+    constexpr int NA = BM * CH / 4 / THREADS;  // float4 of the filter slab per thread
+    static_assert(NA >= 1, "tile too small for the thread count");
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int pstride = (p.psz + 1) * LDP;  // one spare position absorbs the stores of unused slots
+    float *const As0 = lds;                  // [2][BM * LDP]
+    float *const Bp0 = lds + 2 * BM * LDP;   // [2][pstride]
+
+    unsigned L;
+    const unsigned tiles = (unsigned)(p.mtiles * p.ntiles);
+    if (!xcd_remap(blockIdx.x, tiles * (unsigned)p.splits, &L)) return;
+    const int split = (int)(L / tiles);
+    const unsigned tile = L - (unsigned)split * tiles;
+    const int mt = (int)(tile % (unsigned)p.mtiles), nt = (int)(tile / (unsigned)p.mtiles);
+    const int m0 = mt * BM, n0 = nt * BN;
+    const int cb = split * p.chunks_per_split;
+    const int ce = min(cb + p.chunks_per_split, p.chunks_total);
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int wm = w / T::WN, wn = w % T::WN;
+    const int kh = lane >> 5, l32 = lane & 31;
+    const int OHW = p.OH * p.OW;
+    const int chan_stride = p.IH * p.IW;
+
+    const __amdgpu_buffer_rsrc_t rin = make_rsrc(p.in, p.in_bytes);
+    const __amdgpu_buffer_rsrc_t rwp = make_rsrc(p.wp, p.wp_bytes);
+
+    // ---- patch slots of this thread: element e = i*THREADS + tid -> (channel e / psz, position e % psz)
+    const int n_first = n0 / OHW, oh0 = (n0 - n_first * OHW) / p.OW;
+    unsigned p_voff[NPMAX];  // byte offset of the element inside channel chunk 0, or kOobOffset
+    int p_lds[NPMAX];        // byte offset inside a patch buffer
+    int p_chan[NPMAX];       // channel inside the chunk (only read when the last chunk is ragged)
+#pragma unroll
+    for (int i = 0; i < NPMAX; i++) {
+        const unsigned e = (unsigned)(i * THREADS + tid);
+        const unsigned c = fast_div(e, p.magic_psz);
+        const unsigned pos = e - c * (unsigned)p.psz;
+        const unsigned img = fast_div(pos, p.magic_img);
+        const unsigned rem = pos - img * (unsigned)(p.PR * p.PC);
+        const unsigned pr = fast_div(rem, p.magic_pc);
+        const unsigned pc = rem - pr * (unsigned)p.PC;
+        const int n = n_first + (int)img, ih = oh0 + (int)pr - p.PT, iw = (int)pc - p.PL;
+        const int bad = (CH - 1 - (int)c) | (p.N - 1 - n) | ih | (p.IH - 1 - ih) | iw | (p.IW - 1 - iw);
+        p_voff[i] = bad < 0 ? kOobOffset : (unsigned)(((n * p.Cin + (int)c) * p.IH + ih) * p.IW + iw) * 4u;
+        p_lds[i] = c < (unsigned)CH ? (int)(pos * LDP + c) * 4 : (p.psz * LDP + (tid & 15)) * 4;
+        p_chan[i] = (int)c;
+    }
+    float preg[NPMAX];
+    auto patch_load = [&](int i, int chunk) {
+        unsigned voff = p_voff[i];
+        if (!kCFull) voff = chunk * CH + p_chan[i] < p.Cin ? voff : kOobOffset;
+        preg[i] = buffer_load_f32(rin, voff, (unsigned)(chunk * CH * chan_stride) * 4u);
+    };
+    auto patch_store = [&](int i, float *buf) { *(float *)((char *)buf + p_lds[i]) = preg[i]; };
+
+    // ---- filter slab slots: float4 f = ii*THREADS + tid -> (row f / 4, channel quad f % 4)
+    unsigned a_voff[NA];
+    int a_lds[NA];
+#pragma unroll
+    for (int ii = 0; ii < NA; ii++) {
+        const int f = ii * THREADS + tid;
+        a_voff[ii] = (unsigned)((m0 + f / 4) * CH + (f % 4) * 4) * 4u;  // m0 + row < Mp always
+        a_lds[ii] = (f / 4) * LDP + (f % 4) * 4;
+    }
+    float4 areg[NA];
+    const unsigned slab_bytes = (unsigned)p.Mp * CH * 4u;
+    auto a_load = [&](int sidx) {
+#pragma unroll
+        for (int ii = 0; ii < NA; ii++) areg[ii] = buffer_load_f32x4(rwp, a_voff[ii], (unsigned)sidx * slab_bytes);
+    };
+    auto a_store = [&](float *buf) {
+#pragma unroll
+        for (int ii = 0; ii < NA; ii++) *(float4 *)&buf[a_lds[ii]] = areg[ii];
+    };
+
+    // ---- fragment addresses
+    const float *a_frag = As0 + (wm * (BM / T::WM) + l32) * LDP + kh * 8;
+    int b_frag[NI];  // float offset inside a patch buffer of this lane's pixel, tap offset (0,0)
+#pragma unroll
+    for (int j = 0; j < NI; j++) {
+        const int q = wn * (BN / T::WN) + j * 32 + l32;  // pixel inside the tile
+        const int img = q / (p.rows * p.OW), r = q / p.OW - img * p.rows, col = q % p.OW;
+        b_frag[j] = ((img * p.PR + r) * p.PC + col) * LDP + kh * 8;
+    }
+
+    v16f acc[MI][NI];
+    zero_acc(acc);
+
+    // prologue: the first patch and the first filter slab
+#pragma unroll
+    for (int i = 0; i < NPMAX; i++) patch_load(i, cb);
+    a_load(cb * TAPS);
+#pragma unroll
+    for (int i = 0; i < NPMAX; i++) patch_store(i, Bp0);
+    a_store(As0);
+    __syncthreads();
+
+    int acur = 0, pcur = 0;
+    int sidx = cb * TAPS;  // filter slab being multiplied
+    // loads of the next patch are issued during taps 0..3 of a chunk, its LDS stores during taps 5..8
+    constexpr int PER = (NPMAX + 3) / 4;
+    for (int chunk = cb; chunk < ce; ++chunk) {
+        float *const bp_cur = Bp0 + pcur * pstride;
+        float *const bp_nxt = Bp0 + (pcur ^ 1) * pstride;
+        static_for<0, TAPS>([&](auto ttag) {
+            constexpr int t = decltype(ttag)::value;
+            constexpr int tr = t / 3, ts = t % 3;
+            const int tapoff = (p.flip ? (2 - tr) * p.PC + (2 - ts) : tr * p.PC + ts) * LDP;
+            const float *ap = a_frag + acur * (BM * LDP);
+            float *const as_nxt = As0 + (acur ^ 1) * (BM * LDP);
+            float4 fa[MI][2], fb[NI][2];
+#pragma unroll
+            for (int i = 0; i < MI; i++) {
+                fa[i][0] = *(const float4 *)(ap + i * 32 * LDP);
+                fa[i][1] = *(const float4 *)(ap + i * 32 * LDP + 4);
+            }
+#pragma unroll
+            for (int j = 0; j < NI; j++) {
+                fb[j][0] = *(const float4 *)(bp_cur + b_frag[j] + tapoff);
+                fb[j][1] = *(const float4 *)(bp_cur + b_frag[j] + tapoff + 4);
+            }
+            static_for<0, 8>([&](auto stag) {
+                constexpr int ks = decltype(stag)::value;
+                // side work of this step
+                if constexpr (ks == 0) a_load(sidx + 1);
+                if constexpr (ks == 7) a_store(as_nxt);
+                if constexpr (t < 4 && ks >= 1 && ks <= 6) {
+                    // PER loads of tap t, dealt over steps 1..6
+                    constexpr int first = t * PER + (ks - 1) * ((PER + 5) / 6);
+                    constexpr int last = first + (PER + 5) / 6;
+#pragma unroll
+                    for (int i = first; i < last; i++)
+                        if (i < (t + 1) * PER && i < NPMAX) patch_load(i, chunk + 1);
+                }
+                if constexpr (t >= 5 && ks >= 1 && ks <= 6) {
+                    constexpr int first = (t - 5) * PER + (ks - 1) * ((PER + 5) / 6);
+                    constexpr int last = first + (PER + 5) / 6;
+#pragma unroll
+                    for (int i = first; i < last; i++)
+                        if (i < (t - 4) * PER && i < NPMAX) patch_store(i, bp_nxt);
+                }
+#pragma unroll
+                for (int i = 0; i < MI; i++)
+#pragma unroll
+                    for (int j = 0; j < NI; j++) {
+                        const float4 av = fa[i][ks / 4], bv = fb[j][ks / 4];
+                        const float a = ks % 4 == 0 ? av.x : ks % 4 == 1 ? av.y : ks % 4 == 2 ? av.z : av.w;
+                        const float b = ks % 4 == 0 ? bv.x : ks % 4 == 1 ? bv.y : ks % 4 == 2 ? bv.z : bv.w;
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[i][j], 0, 0, 0);
+                    }
+#pragma unroll
+                for (int g = 0; g < MI * NI; g++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x216, 2, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            __syncthreads();
+            acur ^= 1;
+            ++sidx;
+        });
+        pcur ^= 1;
+    }
+
+    float *outp = p.out + (size_t)split * p.out_elems;
+#pragma unroll
+    for (int j = 0; j < NI; j++) {
+        const int col = n0 + wn * (BN / T::WN) + j * 32 + l32;
+        if (col >= p.ncols) continue;
+        const int n2 = col / OHW, pq2 = col - n2 * OHW;
+        float *base = outp + (size_t)n2 * p.Mout * OHW + pq2;
+#pragma unroll
+        for (int i = 0; i < MI; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int m = m0 + wm * (BM / T::WM) + i * 32 + acc_row(v, lane);
+                if (m < p.Mout) base[(size_t)m * OHW] = acc[i][j][v];
+            }
+    }
+}
+
+// Packed filter of the patch kernel: wp[((chunk*9 + tap)*Mp + m)*16 + j] = w[m*sm + (chunk*16+j)*sc + tap]
+// (zero where m >= M or the channel is past the end).  Forward: m = output channel k (sm = C*9,
+// sc = 9); backward-data: m = input channel c (sm = 9, sc = C*9), reduction over k.
+__global__ __launch_bounds__(256) void pack_patch_k(int M, int Cred, int Mp, int chunks, size_t sm, size_t sc,
+                                                     const float *w, float *wp)
+{
+    const size_t total = (size_t)chunks * 9 * Mp * 16;
+    for (size_t o = (size_t)blockIdx.x * 256 + threadIdx.x; o < total; o += (size_t)gridDim.x * 256) {
+        const int j = (int)(o & 15);
+        size_t r = o >> 4;
+        const int m = (int)(r % (size_t)Mp);
+        r /= (size_t)Mp;
+        const int tap = (int)(r % 9), chunk = (int)(r / 9);
+        const int c = chunk * 16 + j;
+        wp[o] = (m < M && c < Cred) ? w[(size_t)m * sm + (size_t)c * sc + tap] : 0.0f;
+    }
+}
+
 // ------------------------------------------------------------------------------------ backward-filter
 
 struct FilterGrad {
@@ -466,10 +699,126 @@ using GatherWide = Tile<64, 256, 1, 4>;     // few output channels, many pixels
 using GatherSquare = Tile<128, 128, 2, 2>;  // enough tiles for two workgroups per CU
 using GatherDeep = Tile<128, 128, 2, 4>;    // few tiles: 8 wavefronts per workgroup, one workgroup per CU
 
+unsigned div_magic(unsigned d) { return (unsigned)((((unsigned long long)1 << 32) / d) + 1); }
+
+template <class T, int NPMAX>
+int launch_patch(const PatchConv &pc, bool c_full, dim3 grid, size_t lds_bytes)
+{
+    // above 64 KB of dynamic LDS a kernel has to be told once
+    static bool raised[2] = {false, false};
+    if (!raised[c_full]) {
+        const void *fn = c_full ? (const void *)conv_patch_k<T, NPMAX, true> : (const void *)conv_patch_k<T, NPMAX, false>;
+        DOPT_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        raised[c_full] = true;
+    }
+    if (c_full) hipLaunchKernelGGL((conv_patch_k<T, NPMAX, true>), grid, dim3(T::THREADS), lds_bytes, stream(), pc);
+    else hipLaunchKernelGGL((conv_patch_k<T, NPMAX, false>), grid, dim3(T::THREADS), lds_bytes, stream(), pc);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+// 3x3 unit-stride layers whose pixel tiles are whole rows of one image or whole images.
+// Returns DOPT_HIP_OK with *done = false when the layer does not fit this path.
+template <bool kBwd>
+int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, const float *w, float *out, bool *done)
+{
+    *done = false;
+    if (d->R != 3 || d->S != 3 || d->strideH != 1 || d->strideW != 1 || d->padH > 2 || d->padW > 2) return DOPT_HIP_OK;
+    PatchConv pc{};
+    pc.N = (int)d->N;
+    if (!kBwd) {
+        pc.Cin = (int)d->C; pc.IH = (int)d->H; pc.IW = (int)d->W;
+        pc.Mout = (int)d->K; pc.OH = (int)P; pc.OW = (int)Q;
+        pc.PT = (int)d->padH; pc.PL = (int)d->padW; pc.flip = 1;
+    } else {
+        pc.Cin = (int)d->K; pc.IH = (int)P; pc.IW = (int)Q;
+        pc.Mout = (int)d->C; pc.OH = (int)d->H; pc.OW = (int)d->W;
+        pc.PT = 2 - (int)d->padH; pc.PL = 2 - (int)d->padW; pc.flip = 0;
+    }
+    pc.ncols = pc.N * pc.OH * pc.OW;
+    enum { kWide, kSquare, kDeep } shape;
+    int BM, BN, blocks_wanted, npmax, threads;
+    if (pc.Mout <= 64) {
+        shape = kWide; BM = 64; BN = 256; blocks_wanted = 2 * num_cus(); npmax = 24; threads = 256;
+    } else {
+        BM = 128; BN = 128;
+        const int t = ((pc.Mout + 127) / 128) * ((pc.ncols + 127) / 128);
+        if (t >= 2 * num_cus()) { shape = kSquare; blocks_wanted = 2 * num_cus(); npmax = 16; threads = 256; }
+        else { shape = kDeep; blocks_wanted = num_cus(); npmax = 16; threads = 512; }
+    }
+    // pixel tile = `rows` full rows of one image, or `nimg` whole images
+    if (BN % pc.OW != 0) return DOPT_HIP_OK;
+    const int tile_rows = BN / pc.OW;
+    if (tile_rows <= pc.OH) {
+        if (pc.OH % tile_rows != 0) return DOPT_HIP_OK;
+        pc.nimg = 1; pc.rows = tile_rows;
+    } else {
+        if (tile_rows % pc.OH != 0) return DOPT_HIP_OK;
+        pc.nimg = tile_rows / pc.OH; pc.rows = pc.OH;
+    }
+    pc.PR = pc.rows + 2; pc.PC = pc.OW + 2;
+    pc.psz = pc.nimg * pc.PR * pc.PC;
+    if ((size_t)pc.psz * 16 > (size_t)npmax * threads) return DOPT_HIP_OK;
+    const size_t lds_bytes = ((size_t)2 * BM * 20 + (size_t)2 * (pc.psz + 1) * 20) * sizeof(float);
+    if (lds_bytes > 160 * 1024) return DOPT_HIP_OK;
+    pc.magic_psz = div_magic((unsigned)pc.psz);
+    pc.magic_img = div_magic((unsigned)(pc.PR * pc.PC));
+    pc.magic_pc = div_magic((unsigned)pc.PC);
+    pc.mtiles = (pc.Mout + BM - 1) / BM;
+    pc.ntiles = (pc.ncols + BN - 1) / BN;
+    pc.Mp = pc.mtiles * BM;
+    pc.chunks_total = (pc.Cin + 15) / 16;
+    pc.out_elems = (size_t)pc.ncols * pc.Mout;
+    const int tiles = pc.mtiles * pc.ntiles;
+    int splits = (blocks_wanted + tiles - 1) / tiles;
+    if (splits > pc.chunks_total) splits = pc.chunks_total;
+    if (splits > 64) splits = 64;
+    if (pc.out_elems % 4 != 0 || !aligned16(out)) splits = 1;
+    pc.chunks_per_split = (pc.chunks_total + splits - 1) / splits;
+    splits = (pc.chunks_total + pc.chunks_per_split - 1) / pc.chunks_per_split;
+    pc.splits = splits;
+
+    const size_t wp_elems = (size_t)pc.chunks_total * 9 * pc.Mp * 16;
+    const size_t wp_bytes = (wp_elems * sizeof(float) + 255) / 256 * 256;
+    const size_t part_bytes = splits > 1 ? (size_t)splits * pc.out_elems * sizeof(float) : 0;
+    char *ws = (char *)workspace(wp_bytes + part_bytes);
+    if (!ws) return DOPT_HIP_ERR_OOM;
+    float *wp = (float *)ws;
+    float *partial = (float *)(ws + wp_bytes);
+    {
+        const size_t blocks = ceil_div(wp_elems, (size_t)256);
+        const size_t cap = (size_t)num_cus() * 16;
+        const size_t C9 = (size_t)d->C * 9;
+        hipLaunchKernelGGL(pack_patch_k, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0, stream(), pc.Mout,
+                           pc.Cin, pc.Mp, pc.chunks_total, kBwd ? (size_t)9 : C9, kBwd ? C9 : (size_t)9, w, wp);
+        DOPT_LAUNCH_CHECK();
+    }
+    pc.in = in;
+    pc.wp = wp;
+    pc.in_bytes = (size_t)pc.N * pc.Cin * pc.IH * pc.IW * sizeof(float);
+    pc.wp_bytes = wp_elems * sizeof(float);
+    pc.out = splits > 1 ? partial : out;
+    const dim3 grid(xcd_grid((unsigned)(tiles * splits)));
+    const bool c_full = pc.Cin % 16 == 0;
+    int rc;
+    if (shape == kWide) rc = launch_patch<GatherWide, 24>(pc, c_full, grid, lds_bytes);
+    else if (shape == kSquare) rc = launch_patch<GatherSquare, 16>(pc, c_full, grid, lds_bytes);
+    else rc = launch_patch<GatherDeep, 16>(pc, c_full, grid, lds_bytes);
+    if (rc) return rc;
+    *done = true;
+    if (splits > 1) return launch_splitk_reduce(pc.out_elems, splits, partial, out);
+    return DOPT_HIP_OK;
+}
+
 // Shared host driver of forward (kBwd = false) and backward-data (kBwd = true).
 template <bool kBwd>
 int run_gather(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, const float *w, float *out)
 {
+    {
+        bool done = false;
+        if (int rc = run_patch<kBwd>(d, P, Q, in, w, out, &done)) return rc;
+        if (done) return DOPT_HIP_OK;
+    }
     GatherConv g{};
     const int taps = (int)(d->R * d->S);
     g.N = (int)d->N;

@@ -57,6 +57,23 @@ __device__ inline void mma_slab(const float *As, const float *Bs, int a_off, int
     }
 }
 
+
+// Compile-time loop: f(StepTag<I>{}) for I = 0 .. N-1, so that the body can use I in constant
+// expressions (register-array indices, `if constexpr`).
+template <int I>
+struct StepTag {
+    static constexpr int value = I;
+};
+
+template <int I, int N, class F>
+__device__ inline void static_for(F &&f)
+{
+    if constexpr (I < N) {
+        f(StepTag<I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
 template <int MI, int NI>
 __device__ inline void zero_acc(v16f (&acc)[MI][NI])
 {

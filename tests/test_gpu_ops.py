@@ -252,6 +252,17 @@ CONV_CASES = [  # N, C, H, W, K, R, S, pad, stride
     (2, 16, 32, 32, 160, 1, 1, (0, 0), (1, 1)),   # WRN 1x1 shortcut
     (2, 160, 32, 32, 320, 3, 3, (1, 1), (2, 2)),  # WRN stage entry, stride 2
     (2, 160, 32, 32, 320, 1, 1, (0, 0), (2, 2)),  # WRN strided shortcut
+    # 3x3 unit-stride layers take the patch kernel: tiles of several whole images with a ragged
+    # last tile, no padding / full padding (output smaller / larger than the input), channel counts
+    # that are not multiples of 16, row counts that do not divide the tile (falls back to the gather)
+    (5, 32, 4, 4, 130, 3, 3, (1, 1), (1, 1)),
+    (3, 20, 8, 8, 70, 3, 3, (1, 1), (1, 1)),
+    (2, 16, 10, 10, 40, 3, 3, (0, 0), (1, 1)),
+    (2, 16, 6, 6, 24, 3, 3, (2, 2), (1, 1)),
+    (2, 24, 16, 16, 64, 3, 3, (1, 0), (1, 1)),
+    (1, 16, 12, 8, 32, 3, 3, (1, 1), (1, 1)),
+    (3, 48, 2, 2, 200, 3, 3, (1, 1), (1, 1)),
+    (130, 16, 2, 2, 16, 3, 3, (1, 1), (1, 1)),
 ]
 
 
