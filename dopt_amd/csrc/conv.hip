@@ -597,6 +597,191 @@ __global__ __launch_bounds__(256) void wgrad_reduce_k(int K, int C, int Cp, int 
     for (int i = threadIdx.x; i < nelem; i += 256) dst[i] = stage[i];
 }
 
+// ------------------------------------------------------------------------------------ backward-filter, 3x3 patch
+//
+// Filter gradient of 3x3, unit-stride, pad-1 convolutions:
+//   dw[k][c][2-r][2-s] = sum over (n, p, q) of dy[n][k][p][q] * x[n][c][p-1+r][q-1+s].
+// The reduction runs over pixels.  A block owns BM output channels x BC input channels x all nine
+// taps and walks the pixels in chunks of 64 (G = 64/W full rows of one image).  Per chunk it
+// stages dy[BM][64] and ONE halo patch x[BC][G+2][W(+halo)] in LDS; the nine taps read that patch
+// at nine offsets, so x is fetched once, not nine times.  The twelve wavefronts are
+// (32 rows of k) x (32 channels) x (tap row r): a wavefront keeps the three taps s = 0..2 of its
+// tap row in three 32x32 accumulators.  A lane's operands for a 16-pixel slab are pixels
+// kh*8 .. kh*8+7 of the slab (kh = lane / 32): two 128-bit reads of dy, and for x a 10-wide
+// window (two aligned 128-bit reads and the two edge columns) that serves all three taps by
+// register selection.  Per 24 matrix instructions a wavefront issues 6 LDS reads.
+
+struct WgradPatch {
+    const float *dy;  // [N, K, H, W]
+    const float *x;   // [N, C, H, W]
+    float *out;       // `splits` partial copies of [K][9 * Cp] (tap-major columns)
+    int N, C, K, H, W;
+    int G, bands;         // output rows per chunk (G*W = 64); bands = H / G chunks per image
+    int ppitch, cstride;  // patch row pitch W+8 (pixel q at column q+4); floats per channel
+    int quads_row;        // W / 4
+    int Cp, ncols;
+    int mtiles, ctiles, chunks_total, chunks_per_split, splits;
+    size_t out_elems, dy_bytes, x_bytes;
+};
+
+template <int WM, int WC>
+__global__ __launch_bounds__(768, 1) void conv_wgrad_patch_k(WgradPatch p)
+{
+    constexpr int BM = 32 * WM, BC = 32 * WC, THREADS = 768, NPIX = 64, APITCH = NPIX + 4;
+    constexpr int NAQ = (BM * NPIX / 4 + THREADS - 1) / THREADS;  // float4 slots of dy per thread
+    constexpr int NBQ = WC == 1 ? 2 : 3;                          // float4 slots of x per thread (host checks)
+    static_assert(WM * WC == 4, "twelve wavefronts: 4 (row, channel) groups x 3 tap rows");
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int bsize = BC * p.cstride;
+    float *const A0 = lds;                     // [2][BM * APITCH]
+    float *const B0 = lds + 2 * BM * APITCH;   // [2][bsize]
+    float *const dummy = B0 + 2 * bsize;       // 4 floats absorbing the stores of unused slots
+
+    unsigned L;
+    const unsigned tiles = (unsigned)(p.mtiles * p.ctiles);
+    if (!xcd_remap(blockIdx.x, tiles * (unsigned)p.splits, &L)) return;
+    const int split = (int)(L / tiles);
+    const unsigned tile = L - (unsigned)split * tiles;
+    const int mt = (int)(tile % (unsigned)p.mtiles), ct = (int)(tile / (unsigned)p.mtiles);
+    const int k0 = mt * BM, c0 = ct * BC;
+    const int cb = split * p.chunks_per_split;
+    const int ce = min(cb + p.chunks_per_split, p.chunks_total);
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int kh = lane >> 5, l32 = lane & 31;
+    const int dr = w % 3, grp = w / 3;
+    const int wm = grp / WC, wc = grp % WC;
+    const int HW = p.H * p.W;
+
+    const __amdgpu_buffer_rsrc_t rdy = make_rsrc(p.dy, p.dy_bytes);
+    const __amdgpu_buffer_rsrc_t rx = make_rsrc(p.x, p.x_bytes);
+
+    // ---- load slots
+    unsigned a_voff[NAQ];
+    int a_lds[NAQ];
+#pragma unroll
+    for (int i = 0; i < NAQ; i++) {
+        const int a = i * THREADS + tid;
+        const int row = a / 16, quad = a % 16;
+        const bool ok = a < BM * 16 && k0 + row < p.K;
+        a_voff[i] = ok ? (unsigned)((k0 + row) * HW + quad * 4) * 4u : kOobOffset;
+        a_lds[i] = a < BM * 16 ? row * APITCH + quad * 4 : -1;
+    }
+    unsigned b_voff[NBQ];
+    int b_lds[NBQ], b_edge[NBQ];  // b_edge: 1 = top halo row, 2 = bottom halo row
+    const int quads_ch = (p.G + 2) * p.quads_row;
+#pragma unroll
+    for (int i = 0; i < NBQ; i++) {
+        const int b = i * THREADS + tid;
+        const int c = b / quads_ch, rem = b - c * quads_ch;
+        const int pr = rem / p.quads_row, quad = rem - pr * p.quads_row;
+        const bool ok = c < BC && c0 + c < p.C;
+        // row p0 - 1 + pr of channel c0 + c; p0 and the image are added per chunk
+        b_voff[i] = ok ? (unsigned)(((c0 + c) * p.H + pr) * p.W + quad * 4) * 4u : kOobOffset;
+        b_lds[i] = c < BC ? c * p.cstride + pr * p.ppitch + 4 + quad * 4 : -1;
+        b_edge[i] = pr == 0 ? 1 : (pr == p.G + 1 ? 2 : 0);
+    }
+    float4 areg[NAQ], breg[NBQ];
+    int n_img = cb / p.bands, band = cb - n_img * p.bands;  // position of the chunk being FETCHED
+    auto fetch = [&]() {
+        const int p0 = band * p.G;
+        const unsigned a_soff = (unsigned)(n_img * p.K * HW + p0 * p.W) * 4u;
+#pragma unroll
+        for (int i = 0; i < NAQ; i++) areg[i] = buffer_load_f32x4(rdy, a_voff[i], a_soff);
+        // x row p0 - 1 + pr.  Offsets handed to a buffer load must not go negative: the "- 1" row is
+        // taken off the wave-uniform part, except for the very first chunk of the tensor, where it is
+        // taken off the per-lane part (whose top halo row, the only one it could underflow, is masked)
+        const int kill = (band == 0 ? 1 : 0) | (band == p.bands - 1 ? 2 : 0);
+        const bool first = n_img == 0 && band == 0;
+        const unsigned roww = (unsigned)p.W * 4u;
+        const unsigned b_soff = (unsigned)(n_img * p.C * HW + p0 * p.W) * 4u - (first ? 0u : roww);
+#pragma unroll
+        for (int i = 0; i < NBQ; i++) {
+            const bool dead = (b_edge[i] & kill) != 0 || b_voff[i] == kOobOffset;
+            breg[i] = buffer_load_f32x4(rx, dead ? kOobOffset : b_voff[i] - (first ? roww : 0u), b_soff);
+        }
+        if (++band == p.bands) {
+            band = 0;
+            ++n_img;
+        }
+    };
+    auto stash = [&](int buf) {
+        float *A = A0 + buf * (BM * APITCH), *B = B0 + buf * bsize;
+#pragma unroll
+        for (int i = 0; i < NAQ; i++) *(float4 *)(a_lds[i] >= 0 ? A + a_lds[i] : dummy) = areg[i];
+#pragma unroll
+        for (int i = 0; i < NBQ; i++) *(float4 *)(b_lds[i] >= 0 ? B + b_lds[i] : dummy) = breg[i];
+    };
+
+    // ---- fragment addresses: slab s covers the 8-pixel runs 2s (kh = 0) and 2s+1 (kh = 1) of the chunk
+    const int a_frag = (wm * 32 + l32) * APITCH + kh * 8;
+    int b_frag[4];
+    const int runs_row = p.W / 8;
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        const int u = 2 * s + kh, rho = u / runs_row, q0 = (u - rho * runs_row) * 8;
+        b_frag[s] = ((wc * 32 + l32) * p.cstride + (rho + dr) * p.ppitch + q0) / 4 + 1;  // float4 index of pixel q0
+    }
+
+    // the halo columns are never written again: clear both patch buffers once
+    for (int i = tid; i < 2 * bsize; i += THREADS) B0[i] = 0.0f;
+    __syncthreads();
+
+    v16f acc[3];
+#pragma unroll
+    for (int t = 0; t < 3; t++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[t][v] = 0.0f;
+
+    fetch();
+    stash(0);
+    __syncthreads();
+    int cur = 0;
+    for (int chunk = cb; chunk < ce; ++chunk) {
+        const float *A = A0 + cur * (BM * APITCH) + a_frag;
+        // float4 indexing keeps the 16-byte alignment of the patch reads visible to the compiler
+        const float4 *B = (const float4 *)B0 + cur * (bsize / 4);
+        static_for<0, 4>([&](auto stag) {
+            constexpr int s = decltype(stag)::value;
+            if constexpr (s == 0) fetch();  // the chunk after this one (past the end: harmless, see below)
+            const float4 a_lo = *(const float4 *)(A + s * 16), a_hi = *(const float4 *)(A + s * 16 + 4);
+            // two aligned quads and the two edge columns.  The edge reads are volatile so that the
+            // compiler does not fuse all ten floats into one run starting at the unaligned edge (it
+            // would then read the run as five 2-dword pieces).
+            const float4 *bq = B + b_frag[s];
+            const float4 b_lo = bq[0], b_hi = bq[1];
+            typedef __attribute__((address_space(3))) float lds_float_t;
+            const volatile lds_float_t *be = (const volatile lds_float_t *)bq;
+            const float e_lo = be[-1], e_hi = be[8];
+            const float a8[8] = {a_lo.x, a_lo.y, a_lo.z, a_lo.w, a_hi.x, a_hi.y, a_hi.z, a_hi.w};
+            const float win[10] = {e_lo, b_lo.x, b_lo.y, b_lo.z, b_lo.w, b_hi.x, b_hi.y, b_hi.z, b_hi.w, e_hi};
+#pragma unroll
+            for (int ks = 0; ks < 8; ks++)
+#pragma unroll
+                for (int ds = 0; ds < 3; ds++)
+                    acc[ds] = __builtin_amdgcn_mfma_f32_32x32x2f32(a8[ks], win[ks + ds], acc[ds], 0, 0, 0);
+            if constexpr (s == 3) stash(cur ^ 1);
+        });
+        __syncthreads();
+        cur ^= 1;
+    }
+
+    // partial[k][t * Cp + c] with t = (2 - dr) * 3 + (2 - ds)
+    float *outp = p.out + (size_t)split * p.out_elems;
+    const int c = c0 + wc * 32 + l32;
+    if (c < p.C) {
+#pragma unroll
+        for (int ds = 0; ds < 3; ds++) {
+            const int t = (2 - dr) * 3 + (2 - ds);
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int k = k0 + wm * 32 + acc_row(v, lane);
+                if (k < p.K) outp[(size_t)k * p.ncols + t * p.Cp + c] = acc[ds][v];
+            }
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------ helpers
 
 // out[i] = sum_s partial[s][i], s ascending.
@@ -905,6 +1090,80 @@ int run_gather(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in,
     return DOPT_HIP_OK;
 }
 
+template <int WM, int WC>
+int launch_wgrad_patch(const WgradPatch &wp, dim3 grid, size_t lds_bytes)
+{
+    static bool raised = false;
+    if (!raised) {
+        DOPT_HIP_CHECK(hipFuncSetAttribute((const void *)conv_wgrad_patch_k<WM, WC>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        raised = true;
+    }
+    hipLaunchKernelGGL((conv_wgrad_patch_k<WM, WC>), grid, dim3(768), lds_bytes, stream(), wp);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+int launch_wgrad_reduce(int K, int C, int Cp, int taps, int splits, size_t out_elems, const float *partial, float *dw)
+{
+    // 64-channel chunks when that still leaves >= 1024 workgroups and the LDS staging stays small
+    const int ch = ((size_t)K * ((C + 63) / 64) >= 1024 && taps <= 16) ? 64 : 16;
+    dim3 rgrid((unsigned)K, (unsigned)((C + ch - 1) / ch));
+    hipLaunchKernelGGL(wgrad_reduce_k, rgrid, dim3(256), (size_t)5 * ch * taps * sizeof(float), stream(), K, C, Cp, taps,
+                       ch, splits, out_elems, partial, dw);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+// 3x3, unit stride, pad 1, rows of 8 / 16 / 32 / 64 pixels.  *done = false: not this path.
+int run_wgrad_patch(const dopt_hip_conv_desc *d, const float *dy, const float *x, float *dw, bool *done)
+{
+    *done = false;
+    if (d->R != 3 || d->S != 3 || d->strideH != 1 || d->strideW != 1 || d->padH != 1 || d->padW != 1) return DOPT_HIP_OK;
+    const int W = (int)d->W, H = (int)d->H;
+    if (W != 8 && W != 16 && W != 32 && W != 64) return DOPT_HIP_OK;
+    if (d->C < 16) return DOPT_HIP_OK;  // a 32-channel fragment would be mostly padding
+    WgradPatch wp{};
+    wp.G = 64 / W;
+    if (H % wp.G != 0) return DOPT_HIP_OK;
+    const bool tall = d->K >= 128;  // 128 rows x 32 channels, else 64 x 64
+    if (!tall && W == 64) return DOPT_HIP_OK;
+    const int BM = tall ? 128 : 64, BC = tall ? 32 : 64;
+    wp.dy = dy; wp.x = x;
+    wp.N = (int)d->N; wp.C = (int)d->C; wp.K = (int)d->K; wp.H = H; wp.W = W;
+    wp.bands = H / wp.G;
+    wp.ppitch = W + 8;
+    wp.quads_row = W / 4;
+    int cs = (wp.G + 2) * wp.ppitch;
+    while (cs % 8 != 4) cs += 4;  // 128-bit reads by 32 channels at this stride touch every LDS bank once
+    wp.cstride = cs;
+    wp.Cp = round_up(wp.C, 16);
+    wp.ncols = 9 * wp.Cp;
+    wp.mtiles = (wp.K + BM - 1) / BM;
+    wp.ctiles = (wp.C + BC - 1) / BC;
+    wp.chunks_total = wp.N * wp.bands;
+    wp.out_elems = (size_t)wp.K * wp.ncols;
+    wp.dy_bytes = (size_t)wp.N * wp.K * H * W * sizeof(float);
+    wp.x_bytes = (size_t)wp.N * wp.C * H * W * sizeof(float);
+    const int tiles = wp.mtiles * wp.ctiles;
+    int splits = (num_cus() + tiles - 1) / tiles;
+    const int max_by_depth = wp.chunks_total / 4 > 0 ? wp.chunks_total / 4 : 1;
+    if (splits > max_by_depth) splits = max_by_depth;
+    if (splits > 512) splits = 512;
+    wp.chunks_per_split = (wp.chunks_total + splits - 1) / splits;
+    splits = (wp.chunks_total + wp.chunks_per_split - 1) / wp.chunks_per_split;
+    wp.splits = splits;
+    float *partial = (float *)workspace((size_t)splits * wp.out_elems * sizeof(float));
+    if (!partial) return DOPT_HIP_ERR_OOM;
+    wp.out = partial;
+    const size_t lds_bytes = ((size_t)2 * BM * 68 + (size_t)2 * BC * wp.cstride + 4) * sizeof(float);
+    if (lds_bytes > 160 * 1024) return DOPT_HIP_OK;
+    const dim3 grid(xcd_grid((unsigned)(tiles * splits)));
+    if (int rc = tall ? launch_wgrad_patch<4, 1>(wp, grid, lds_bytes) : launch_wgrad_patch<2, 2>(wp, grid, lds_bytes)) return rc;
+    *done = true;
+    return launch_wgrad_reduce(wp.K, wp.C, wp.Cp, 9, splits, wp.out_elems, partial, dw);
+}
+
 using WgradSquare = Tile<128, 128, 2, 2>;
 using WgradNarrow = Tile<64, 128, 1, 4>;  // K <= 64
 
@@ -936,6 +1195,11 @@ int dopt_hip_conv_bwd_filter(const dopt_hip_conv_desc *d, const float *dy, const
     if (int rc = check_desc(d, &P, &Q, "dopt_hip_conv_bwd_filter")) return rc;
     DOPT_REQUIRE(dy && x && dw, "dopt_hip_conv_bwd_filter: null argument");
     DOPT_ENSURE_INIT();
+    {
+        bool done = false;
+        if (int rc = run_wgrad_patch(d, dy, x, dw, &done)) return rc;
+        if (done) return DOPT_HIP_OK;
+    }
     FilterGrad f{};
     f.dy = dy;
     f.x = x;
@@ -982,13 +1246,7 @@ int dopt_hip_conv_bwd_filter(const dopt_hip_conv_desc *d, const float *dy, const
     }
 #undef DOPT_WGRAD
     DOPT_LAUNCH_CHECK();
-    // 64-channel chunks when that still leaves >= 1024 workgroups and the LDS staging stays small
-    const int ch = ((size_t)f.K * ((f.C + 63) / 64) >= 1024 && taps <= 16) ? 64 : 16;
-    dim3 rgrid((unsigned)f.K, (unsigned)((f.C + ch - 1) / ch));
-    hipLaunchKernelGGL(wgrad_reduce_k, rgrid, dim3(256), (size_t)5 * ch * taps * sizeof(float), stream(), f.K, f.C,
-                       f.Cp, taps, ch, splits, f.out_elems, partial, dw);
-    DOPT_LAUNCH_CHECK();
-    return DOPT_HIP_OK;
+    return launch_wgrad_reduce(f.K, f.C, f.Cp, taps, splits, f.out_elems, partial, dw);
 }
 
 }  // extern "C"

@@ -263,6 +263,13 @@ CONV_CASES = [  # N, C, H, W, K, R, S, pad, stride
     (1, 16, 12, 8, 32, 3, 3, (1, 1), (1, 1)),
     (3, 48, 2, 2, 200, 3, 3, (1, 1), (1, 1)),
     (130, 16, 2, 2, 16, 3, 3, (1, 1), (1, 1)),
+    # filter-gradient patch kernel: rows of 8 / 16 / 32 / 64 pixels, both block shapes (K >= 128 or
+    # not), channel counts off the 32-channel fragment, several bands per image, one-image batches
+    (3, 40, 8, 8, 136, 3, 3, (1, 1), (1, 1)),
+    (2, 70, 16, 16, 48, 3, 3, (1, 1), (1, 1)),
+    (1, 33, 32, 32, 130, 3, 3, (1, 1), (1, 1)),
+    (1, 16, 4, 64, 128, 3, 3, (1, 1), (1, 1)),
+    (5, 96, 16, 8, 64, 3, 3, (1, 1), (1, 1)),
 ]
 
 
