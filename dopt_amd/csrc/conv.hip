@@ -602,34 +602,47 @@ __global__ __launch_bounds__(256) void wgrad_reduce_k(int K, int C, int Cp, int 
 // Filter gradient of 3x3, unit-stride, pad-1 convolutions:
 //   dw[k][c][2-r][2-s] = sum over (n, p, q) of dy[n][k][p][q] * x[n][c][p-1+r][q-1+s].
 // The reduction runs over pixels.  A block owns BM output channels x BC input channels x all nine
-// taps and walks the pixels in chunks of 64 (G = 64/W full rows of one image).  Per chunk it
-// stages dy[BM][64] and ONE halo patch x[BC][G+2][W(+halo)] in LDS; the nine taps read that patch
-// at nine offsets, so x is fetched once, not nine times.  The twelve wavefronts are
-// (32 rows of k) x (32 channels) x (tap row r): a wavefront keeps the three taps s = 0..2 of its
-// tap row in three 32x32 accumulators.  A lane's operands for a 16-pixel slab are pixels
-// kh*8 .. kh*8+7 of the slab (kh = lane / 32): two 128-bit reads of dy, and for x a 10-wide
-// window (two aligned 128-bit reads and the two edge columns) that serves all three taps by
-// register selection.  Per 24 matrix instructions a wavefront issues 6 LDS reads.
+// taps and walks the pixels in chunks of 64.  Per chunk it stages dy[BM][64] and ONE zero-haloed
+// patch of x for its BC channels in LDS; the nine taps read that patch at nine offsets, so x is
+// fetched once, not nine times.  The twelve wavefronts are (32 rows of k) x (32 channels) x
+// (tap row r): a wavefront keeps the three taps s = 0..2 of its tap row in three 32x32
+// accumulators.  A lane's operands for a 16-pixel slab are pixels kh*8 .. kh*8+7 of the slab
+// (kh = lane / 32): two 128-bit reads of dy, and for x a window that serves all three taps by
+// register selection.
+//
+// Geometry of a 64-pixel chunk (kGeo):
+//   0  rows of 8, 16, 32 or 64 pixels: G = 64/W full rows of one image.  Patch rows have pitch W+8
+//      with pixel q at column q+4, so interior quads are 16-byte aligned; a lane's window is two
+//      aligned quads plus the two edge columns.  The halo rows above and below are fetched (or
+//      masked at the image border); the halo columns are cleared once and never written.
+//   1  4x4 images: four whole images.  Same column layout (pitch 12); a lane's 8 pixels are two
+//      rows, each one aligned quad plus two edge columns.  All halo cells stay zero.
+//   2  2x2 images: sixteen whole images, each a 4x4 cell block with the image in the middle; a
+//      lane's 8 pixels are two images, and one aligned quad per (image, row) holds every column
+//      the three taps need.
 
 struct WgradPatch {
     const float *dy;  // [N, K, H, W]
     const float *x;   // [N, C, H, W]
     float *out;       // `splits` partial copies of [K][9 * Cp] (tap-major columns)
     int N, C, K, H, W;
-    int G, bands;         // output rows per chunk (G*W = 64); bands = H / G chunks per image
-    int ppitch, cstride;  // patch row pitch W+8 (pixel q at column q+4); floats per channel
-    int quads_row;        // W / 4
+    int G, bands;         // geometry 0: output rows per chunk (G*W = 64), chunks per image; else 1
+    int imgs;             // images per chunk (1, 4 or 16)
+    int ppitch, cstride;  // patch row pitch; floats per channel (128-bit reads by 32 channels hit every bank once)
+    int quads_row;        // W / 4 (geometry 0)
     int Cp, ncols;
     int mtiles, ctiles, chunks_total, chunks_per_split, splits;
     size_t out_elems, dy_bytes, x_bytes;
 };
 
-template <int WM, int WC>
+template <int WM, int WC, int kGeo>
 __global__ __launch_bounds__(768, 1) void conv_wgrad_patch_k(WgradPatch p)
 {
     constexpr int BM = 32 * WM, BC = 32 * WC, THREADS = 768, NPIX = 64, APITCH = NPIX + 4;
     constexpr int NAQ = (BM * NPIX / 4 + THREADS - 1) / THREADS;  // float4 slots of dy per thread
-    constexpr int NBQ = WC == 1 ? 2 : 3;                          // float4 slots of x per thread (host checks)
+    // float4 slots of x per thread: geometry 0 up to 32*4*8 (W = 32) or 32*3*16 (W = 64) quads per 32
+    // channels; geometries 1, 2 have 16 quads per channel
+    constexpr int NBQ = kGeo == 0 ? (WC == 1 ? 2 : 3) : (BC * 16 + THREADS - 1) / THREADS;
     static_assert(WM * WC == 4, "twelve wavefronts: 4 (row, channel) groups x 3 tap rows");
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int bsize = BC * p.cstride;
@@ -656,53 +669,79 @@ __global__ __launch_bounds__(768, 1) void conv_wgrad_patch_k(WgradPatch p)
     const __amdgpu_buffer_rsrc_t rdy = make_rsrc(p.dy, p.dy_bytes);
     const __amdgpu_buffer_rsrc_t rx = make_rsrc(p.x, p.x_bytes);
 
-    // ---- load slots
+    // ---- load slots.  dy: quad `quad` of row `row` is pixels 4*quad .. 4*quad+3 of the chunk, which
+    // lie in image quad / qpi of the chunk (qpi = quads of one image inside a chunk).
     unsigned a_voff[NAQ];
     int a_lds[NAQ];
+    const int qpi = kGeo == 0 ? 16 : HW / 4;
 #pragma unroll
     for (int i = 0; i < NAQ; i++) {
         const int a = i * THREADS + tid;
         const int row = a / 16, quad = a % 16;
+        const int j = quad / qpi, wq = quad - j * qpi;
         const bool ok = a < BM * 16 && k0 + row < p.K;
-        a_voff[i] = ok ? (unsigned)((k0 + row) * HW + quad * 4) * 4u : kOobOffset;
+        a_voff[i] = ok ? (unsigned)((j * p.K + k0 + row) * HW + wq * 4) * 4u : kOobOffset;
         a_lds[i] = a < BM * 16 ? row * APITCH + quad * 4 : -1;
     }
     unsigned b_voff[NBQ];
-    int b_lds[NBQ], b_edge[NBQ];  // b_edge: 1 = top halo row, 2 = bottom halo row
-    const int quads_ch = (p.G + 2) * p.quads_row;
+    int b_lds[NBQ], b_edge[NBQ];  // b_edge (geometry 0): 1 = top halo row, 2 = bottom halo row
 #pragma unroll
     for (int i = 0; i < NBQ; i++) {
         const int b = i * THREADS + tid;
-        const int c = b / quads_ch, rem = b - c * quads_ch;
-        const int pr = rem / p.quads_row, quad = rem - pr * p.quads_row;
-        const bool ok = c < BC && c0 + c < p.C;
-        // row p0 - 1 + pr of channel c0 + c; p0 and the image are added per chunk
-        b_voff[i] = ok ? (unsigned)(((c0 + c) * p.H + pr) * p.W + quad * 4) * 4u : kOobOffset;
-        b_lds[i] = c < BC ? c * p.cstride + pr * p.ppitch + 4 + quad * 4 : -1;
-        b_edge[i] = pr == 0 ? 1 : (pr == p.G + 1 ? 2 : 0);
+        if (kGeo == 0) {
+            const int quads_ch = (p.G + 2) * p.quads_row;
+            const int c = b / quads_ch, rem = b - c * quads_ch;
+            const int pr = rem / p.quads_row, quad = rem - pr * p.quads_row;
+            const bool ok = c < BC && c0 + c < p.C;
+            // row p0 - 1 + pr of channel c0 + c; p0 and the image are added per chunk
+            b_voff[i] = ok ? (unsigned)(((c0 + c) * p.H + pr) * p.W + quad * 4) * 4u : kOobOffset;
+            b_lds[i] = c < BC ? c * p.cstride + pr * p.ppitch + 4 + quad * 4 : -1;
+            b_edge[i] = pr == 0 ? 1 : (pr == p.G + 1 ? 2 : 0);
+        } else if (kGeo == 1) {
+            const int c = b / 16, j = (b / 4) % 4, row = b % 4;  // image j of the chunk, image row `row`
+            const bool ok = c < BC && c0 + c < p.C;
+            b_voff[i] = ok ? (unsigned)((j * p.C + c0 + c) * 16 + row * 4) * 4u : kOobOffset;
+            b_lds[i] = c < BC ? c * p.cstride + j * 72 + (row + 1) * 12 + 4 : -1;
+            b_edge[i] = 0;
+        } else {
+            const int c = b / 16, j = b % 16;  // the whole 2x2 image j is one quad
+            const bool ok = c < BC && c0 + c < p.C;
+            b_voff[i] = ok ? (unsigned)((j * p.C + c0 + c) * 4) * 4u : kOobOffset;
+            b_lds[i] = c < BC ? c * p.cstride + j * 16 + 5 : -1;  // cell (1,1) of the 4x4 block
+            b_edge[i] = 0;
+        }
     }
     float4 areg[NAQ], breg[NBQ];
-    int n_img = cb / p.bands, band = cb - n_img * p.bands;  // position of the chunk being FETCHED
+    // position of the chunk being FETCHED: first image and, for geometry 0, the band of rows
+    int n_img = kGeo == 0 ? cb / p.bands : cb * p.imgs, band = kGeo == 0 ? cb - n_img * p.bands : 0;
     auto fetch = [&]() {
         const int p0 = band * p.G;
         const unsigned a_soff = (unsigned)(n_img * p.K * HW + p0 * p.W) * 4u;
 #pragma unroll
         for (int i = 0; i < NAQ; i++) areg[i] = buffer_load_f32x4(rdy, a_voff[i], a_soff);
-        // x row p0 - 1 + pr.  Offsets handed to a buffer load must not go negative: the "- 1" row is
-        // taken off the wave-uniform part, except for the very first chunk of the tensor, where it is
-        // taken off the per-lane part (whose top halo row, the only one it could underflow, is masked)
-        const int kill = (band == 0 ? 1 : 0) | (band == p.bands - 1 ? 2 : 0);
-        const bool first = n_img == 0 && band == 0;
-        const unsigned roww = (unsigned)p.W * 4u;
-        const unsigned b_soff = (unsigned)(n_img * p.C * HW + p0 * p.W) * 4u - (first ? 0u : roww);
+        if (kGeo == 0) {
+            // x row p0 - 1 + pr.  Offsets handed to a buffer load must not go negative: the "- 1" row
+            // is taken off the wave-uniform part, except for the very first chunk of the tensor, where
+            // it is taken off the per-lane part (whose top halo row, the only one it could underflow,
+            // is masked)
+            const int kill = (band == 0 ? 1 : 0) | (band == p.bands - 1 ? 2 : 0);
+            const bool first = n_img == 0 && band == 0;
+            const unsigned roww = (unsigned)p.W * 4u;
+            const unsigned b_soff = (unsigned)(n_img * p.C * HW + p0 * p.W) * 4u - (first ? 0u : roww);
 #pragma unroll
-        for (int i = 0; i < NBQ; i++) {
-            const bool dead = (b_edge[i] & kill) != 0 || b_voff[i] == kOobOffset;
-            breg[i] = buffer_load_f32x4(rx, dead ? kOobOffset : b_voff[i] - (first ? roww : 0u), b_soff);
-        }
-        if (++band == p.bands) {
-            band = 0;
-            ++n_img;
+            for (int i = 0; i < NBQ; i++) {
+                const bool dead = (b_edge[i] & kill) != 0 || b_voff[i] == kOobOffset;
+                breg[i] = buffer_load_f32x4(rx, dead ? kOobOffset : b_voff[i] - (first ? roww : 0u), b_soff);
+            }
+            if (++band == p.bands) {
+                band = 0;
+                ++n_img;
+            }
+        } else {
+            const unsigned b_soff = (unsigned)(n_img * p.C * HW) * 4u;
+#pragma unroll
+            for (int i = 0; i < NBQ; i++) breg[i] = buffer_load_f32x4(rx, b_voff[i], b_soff);
+            n_img += p.imgs;
         }
     };
     auto stash = [&](int buf) {
@@ -710,20 +749,39 @@ __global__ __launch_bounds__(768, 1) void conv_wgrad_patch_k(WgradPatch p)
 #pragma unroll
         for (int i = 0; i < NAQ; i++) *(float4 *)(a_lds[i] >= 0 ? A + a_lds[i] : dummy) = areg[i];
 #pragma unroll
-        for (int i = 0; i < NBQ; i++) *(float4 *)(b_lds[i] >= 0 ? B + b_lds[i] : dummy) = breg[i];
+        for (int i = 0; i < NBQ; i++) {
+            if (kGeo != 2) {
+                *(float4 *)(b_lds[i] >= 0 ? B + b_lds[i] : dummy) = breg[i];
+            } else {
+                float *q = b_lds[i] >= 0 ? B + b_lds[i] : dummy;  // rows 1 and 2 of the cell block, columns 1..2
+                const int down = b_lds[i] >= 0 ? 4 : 0;
+                q[0] = breg[i].x;
+                q[1] = breg[i].y;
+                q[down] = breg[i].z;
+                q[down + 1] = breg[i].w;
+            }
+        }
     };
 
-    // ---- fragment addresses: slab s covers the 8-pixel runs 2s (kh = 0) and 2s+1 (kh = 1) of the chunk
+    // ---- fragment addresses
     const int a_frag = (wm * 32 + l32) * APITCH + kh * 8;
-    int b_frag[4];
-    const int runs_row = p.W / 8;
+    int b_frag[4];  // float4 index inside a patch buffer, per slab
+    const int chan = (wc * 32 + l32) * p.cstride;
 #pragma unroll
     for (int s = 0; s < 4; s++) {
-        const int u = 2 * s + kh, rho = u / runs_row, q0 = (u - rho * runs_row) * 8;
-        b_frag[s] = ((wc * 32 + l32) * p.cstride + (rho + dr) * p.ppitch + q0) / 4 + 1;  // float4 index of pixel q0
+        if (kGeo == 0) {
+            // slab s covers the 8-pixel runs 2s (kh = 0) and 2s+1 (kh = 1) of the chunk
+            const int runs_row = p.W / 8;
+            const int u = 2 * s + kh, rho = u / runs_row, q0 = (u - rho * runs_row) * 8;
+            b_frag[s] = (chan + (rho + dr) * p.ppitch + q0) / 4 + 1;  // quad of pixel q0
+        } else if (kGeo == 1) {
+            b_frag[s] = (chan + s * 72 + (2 * kh + dr) * 12) / 4 + 1;  // image s, image rows 2kh and 2kh+1
+        } else {
+            b_frag[s] = (chan + (4 * s + 2 * kh) * 16 + dr * 4) / 4;   // images 4s+2kh and 4s+2kh+1
+        }
     }
 
-    // the halo columns are never written again: clear both patch buffers once
+    // halo cells are never written again: clear both patch buffers once
     for (int i = tid; i < 2 * bsize; i += THREADS) B0[i] = 0.0f;
     __syncthreads();
 
@@ -737,29 +795,53 @@ __global__ __launch_bounds__(768, 1) void conv_wgrad_patch_k(WgradPatch p)
     stash(0);
     __syncthreads();
     int cur = 0;
+    typedef __attribute__((address_space(3))) float lds_float_t;
+    // Fetching runs one chunk ahead and also past the end of this block's range: those loads are
+    // range-checked and their data lands in the LDS buffer that is not read again.
     for (int chunk = cb; chunk < ce; ++chunk) {
         const float *A = A0 + cur * (BM * APITCH) + a_frag;
         // float4 indexing keeps the 16-byte alignment of the patch reads visible to the compiler
         const float4 *B = (const float4 *)B0 + cur * (bsize / 4);
         static_for<0, 4>([&](auto stag) {
             constexpr int s = decltype(stag)::value;
-            if constexpr (s == 0) fetch();  // the chunk after this one (past the end: harmless, see below)
+            if constexpr (s == 0) fetch();
             const float4 a_lo = *(const float4 *)(A + s * 16), a_hi = *(const float4 *)(A + s * 16 + 4);
-            // two aligned quads and the two edge columns.  The edge reads are volatile so that the
-            // compiler does not fuse all ten floats into one run starting at the unaligned edge (it
-            // would then read the run as five 2-dword pieces).
-            const float4 *bq = B + b_frag[s];
-            const float4 b_lo = bq[0], b_hi = bq[1];
-            typedef __attribute__((address_space(3))) float lds_float_t;
-            const volatile lds_float_t *be = (const volatile lds_float_t *)bq;
-            const float e_lo = be[-1], e_hi = be[8];
             const float a8[8] = {a_lo.x, a_lo.y, a_lo.z, a_lo.w, a_hi.x, a_hi.y, a_hi.z, a_hi.w};
-            const float win[10] = {e_lo, b_lo.x, b_lo.y, b_lo.z, b_lo.w, b_hi.x, b_hi.y, b_hi.z, b_hi.w, e_hi};
+            const float4 *bq = B + b_frag[s];
+            // The edge-column reads are volatile so that the compiler does not fuse a whole window
+            // into one run starting at the unaligned edge (it would then read it in 2-dword pieces).
+            const volatile lds_float_t *be = (const volatile lds_float_t *)bq;
+            if constexpr (kGeo == 0) {
+                const float4 b_lo = bq[0], b_hi = bq[1];
+                const float e_lo = be[-1], e_hi = be[8];
+                const float win[10] = {e_lo, b_lo.x, b_lo.y, b_lo.z, b_lo.w, b_hi.x, b_hi.y, b_hi.z, b_hi.w, e_hi};
 #pragma unroll
-            for (int ks = 0; ks < 8; ks++)
+                for (int ks = 0; ks < 8; ks++)
 #pragma unroll
-                for (int ds = 0; ds < 3; ds++)
-                    acc[ds] = __builtin_amdgcn_mfma_f32_32x32x2f32(a8[ks], win[ks + ds], acc[ds], 0, 0, 0);
+                    for (int ds = 0; ds < 3; ds++)
+                        acc[ds] = __builtin_amdgcn_mfma_f32_32x32x2f32(a8[ks], win[ks + ds], acc[ds], 0, 0, 0);
+            } else if constexpr (kGeo == 1) {
+                const float4 r0 = bq[0], r1 = bq[3];  // the next patch row is 12 floats on
+                const float w0[6] = {be[-1], r0.x, r0.y, r0.z, r0.w, be[4]};
+                const float w1[6] = {be[11], r1.x, r1.y, r1.z, r1.w, be[16]};
+#pragma unroll
+                for (int ks = 0; ks < 8; ks++)
+#pragma unroll
+                    for (int ds = 0; ds < 3; ds++)
+                        acc[ds] = __builtin_amdgcn_mfma_f32_32x32x2f32(a8[ks], ks < 4 ? w0[ks + ds] : w1[ks - 4 + ds],
+                                                                       acc[ds], 0, 0, 0);
+            } else {
+                // (image, row) quads: image 0 rows 0, 1 then image 1 rows 0, 1; pixel (row, col) of tap
+                // column ds reads element col + ds of the quad of patch row row + dr
+                const float4 q00 = bq[0], q01 = bq[1], q10 = bq[4], q11 = bq[5];
+                const float win[4][4] = {{q00.x, q00.y, q00.z, q00.w}, {q01.x, q01.y, q01.z, q01.w},
+                                         {q10.x, q10.y, q10.z, q10.w}, {q11.x, q11.y, q11.z, q11.w}};
+#pragma unroll
+                for (int ks = 0; ks < 8; ks++)
+#pragma unroll
+                    for (int ds = 0; ds < 3; ds++)
+                        acc[ds] = __builtin_amdgcn_mfma_f32_32x32x2f32(a8[ks], win[ks / 2][(ks & 1) + ds], acc[ds], 0, 0, 0);
+            }
             if constexpr (s == 3) stash(cur ^ 1);
         });
         __syncthreads();
@@ -1090,16 +1172,16 @@ int run_gather(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in,
     return DOPT_HIP_OK;
 }
 
-template <int WM, int WC>
+template <int WM, int WC, int kGeo>
 int launch_wgrad_patch(const WgradPatch &wp, dim3 grid, size_t lds_bytes)
 {
     static bool raised = false;
     if (!raised) {
-        DOPT_HIP_CHECK(hipFuncSetAttribute((const void *)conv_wgrad_patch_k<WM, WC>,
+        DOPT_HIP_CHECK(hipFuncSetAttribute((const void *)conv_wgrad_patch_k<WM, WC, kGeo>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         raised = true;
     }
-    hipLaunchKernelGGL((conv_wgrad_patch_k<WM, WC>), grid, dim3(768), lds_bytes, stream(), wp);
+    hipLaunchKernelGGL((conv_wgrad_patch_k<WM, WC, kGeo>), grid, dim3(768), lds_bytes, stream(), wp);
     DOPT_LAUNCH_CHECK();
     return DOPT_HIP_OK;
 }
@@ -1115,51 +1197,72 @@ int launch_wgrad_reduce(int K, int C, int Cp, int taps, int splits, size_t out_e
     return DOPT_HIP_OK;
 }
 
-// 3x3, unit stride, pad 1, rows of 8 / 16 / 32 / 64 pixels.  *done = false: not this path.
+// 3x3, unit stride, pad 1; rows of 8 / 16 / 32 / 64 pixels, or 4x4 or 2x2 images.  *done = false: not this path.
 int run_wgrad_patch(const dopt_hip_conv_desc *d, const float *dy, const float *x, float *dw, bool *done)
 {
     *done = false;
     if (d->R != 3 || d->S != 3 || d->strideH != 1 || d->strideW != 1 || d->padH != 1 || d->padW != 1) return DOPT_HIP_OK;
-    const int W = (int)d->W, H = (int)d->H;
-    if (W != 8 && W != 16 && W != 32 && W != 64) return DOPT_HIP_OK;
     if (d->C < 16) return DOPT_HIP_OK;  // a 32-channel fragment would be mostly padding
+    const int W = (int)d->W, H = (int)d->H;
     WgradPatch wp{};
-    wp.G = 64 / W;
-    if (H % wp.G != 0) return DOPT_HIP_OK;
+    int geo;
+    if (W == 8 || W == 16 || W == 32 || W == 64) {
+        geo = 0;
+        wp.G = 64 / W;
+        if (H % wp.G != 0) return DOPT_HIP_OK;
+        wp.bands = H / wp.G;
+        wp.imgs = 1;
+        wp.ppitch = W + 8;
+        wp.cstride = (wp.G + 2) * wp.ppitch;
+        wp.chunks_total = (int)d->N * wp.bands;
+    } else if ((W == 4 && H == 4) || (W == 2 && H == 2)) {
+        geo = W == 4 ? 1 : 2;
+        wp.G = H;
+        wp.bands = 1;
+        wp.imgs = 64 / (H * W);
+        if (d->N % wp.imgs != 0) return DOPT_HIP_OK;
+        wp.ppitch = geo == 1 ? 12 : 4;
+        wp.cstride = geo == 1 ? 4 * 72 : 16 * 16;
+        wp.chunks_total = (int)d->N / wp.imgs;
+    } else {
+        return DOPT_HIP_OK;
+    }
+    while (wp.cstride % 8 != 4) wp.cstride += 4;  // 128-bit reads by 32 channels at this stride touch every LDS bank once
     const bool tall = d->K >= 128;  // 128 rows x 32 channels, else 64 x 64
     if (!tall && W == 64) return DOPT_HIP_OK;
     const int BM = tall ? 128 : 64, BC = tall ? 32 : 64;
     wp.dy = dy; wp.x = x;
     wp.N = (int)d->N; wp.C = (int)d->C; wp.K = (int)d->K; wp.H = H; wp.W = W;
-    wp.bands = H / wp.G;
-    wp.ppitch = W + 8;
     wp.quads_row = W / 4;
-    int cs = (wp.G + 2) * wp.ppitch;
-    while (cs % 8 != 4) cs += 4;  // 128-bit reads by 32 channels at this stride touch every LDS bank once
-    wp.cstride = cs;
     wp.Cp = round_up(wp.C, 16);
     wp.ncols = 9 * wp.Cp;
     wp.mtiles = (wp.K + BM - 1) / BM;
     wp.ctiles = (wp.C + BC - 1) / BC;
-    wp.chunks_total = wp.N * wp.bands;
     wp.out_elems = (size_t)wp.K * wp.ncols;
     wp.dy_bytes = (size_t)wp.N * wp.K * H * W * sizeof(float);
     wp.x_bytes = (size_t)wp.N * wp.C * H * W * sizeof(float);
     const int tiles = wp.mtiles * wp.ctiles;
     int splits = (num_cus() + tiles - 1) / tiles;
-    const int max_by_depth = wp.chunks_total / 4 > 0 ? wp.chunks_total / 4 : 1;
+    const int max_by_depth = wp.chunks_total / 2 > 0 ? wp.chunks_total / 2 : 1;  // two chunks amortise the set-up
     if (splits > max_by_depth) splits = max_by_depth;
     if (splits > 512) splits = 512;
     wp.chunks_per_split = (wp.chunks_total + splits - 1) / splits;
     splits = (wp.chunks_total + wp.chunks_per_split - 1) / wp.chunks_per_split;
     wp.splits = splits;
+    const size_t lds_bytes = ((size_t)2 * BM * 68 + (size_t)2 * BC * wp.cstride + 4) * sizeof(float);
+    if (lds_bytes > 160 * 1024) return DOPT_HIP_OK;
     float *partial = (float *)workspace((size_t)splits * wp.out_elems * sizeof(float));
     if (!partial) return DOPT_HIP_ERR_OOM;
     wp.out = partial;
-    const size_t lds_bytes = ((size_t)2 * BM * 68 + (size_t)2 * BC * wp.cstride + 4) * sizeof(float);
-    if (lds_bytes > 160 * 1024) return DOPT_HIP_OK;
     const dim3 grid(xcd_grid((unsigned)(tiles * splits)));
-    if (int rc = tall ? launch_wgrad_patch<4, 1>(wp, grid, lds_bytes) : launch_wgrad_patch<2, 2>(wp, grid, lds_bytes)) return rc;
+    int rc;
+    if (tall) rc = geo == 0 ? launch_wgrad_patch<4, 1, 0>(wp, grid, lds_bytes)
+                 : geo == 1 ? launch_wgrad_patch<4, 1, 1>(wp, grid, lds_bytes)
+                            : launch_wgrad_patch<4, 1, 2>(wp, grid, lds_bytes);
+    else rc = geo == 0 ? launch_wgrad_patch<2, 2, 0>(wp, grid, lds_bytes)
+            : geo == 1 ? launch_wgrad_patch<2, 2, 1>(wp, grid, lds_bytes)
+                       : launch_wgrad_patch<2, 2, 2>(wp, grid, lds_bytes);
+    if (rc) return rc;
     *done = true;
     return launch_wgrad_reduce(wp.K, wp.C, wp.Cp, 9, splits, wp.out_elems, partial, dw);
 }

@@ -270,6 +270,11 @@ CONV_CASES = [  # N, C, H, W, K, R, S, pad, stride
     (1, 33, 32, 32, 130, 3, 3, (1, 1), (1, 1)),
     (1, 16, 4, 64, 128, 3, 3, (1, 1), (1, 1)),
     (5, 96, 16, 8, 64, 3, 3, (1, 1), (1, 1)),
+    (8, 40, 4, 4, 136, 3, 3, (1, 1), (1, 1)),     # 4x4 images, four per chunk
+    (12, 64, 4, 4, 64, 3, 3, (1, 1), (1, 1)),
+    (32, 48, 2, 2, 130, 3, 3, (1, 1), (1, 1)),    # 2x2 images, sixteen per chunk
+    (16, 70, 2, 2, 32, 3, 3, (1, 1), (1, 1)),
+    (6, 32, 4, 4, 128, 3, 3, (1, 1), (1, 1)),     # batch not a multiple of the chunk: generic kernel
 ]
 
 
