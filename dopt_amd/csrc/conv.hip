@@ -402,18 +402,52 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_patch_k(Pat
 // Packed filter of the patch kernel: wp[((chunk*9 + tap)*Mp + m)*16 + j] = w[m*sm + (chunk*16+j)*sc + tap]
 // (zero where m >= M or the channel is past the end).  Forward: m = output channel k (sm = C*9,
 // sc = 9); backward-data: m = input channel c (sm = 9, sc = C*9), reduction over k.
-__global__ __launch_bounds__(256) void pack_patch_k(int M, int Cred, int Mp, int chunks, size_t sm, size_t sc,
-                                                     const float *w, float *wp)
+// A block transposes 16 rows of one chunk through LDS.  Its source is 16 contiguous runs of 144
+// floats (forward: one per row, its 16 channels x 9 taps; backward: one per reduction channel,
+// its 16 rows x 9 taps), copied to LDS as they lie -- all nine loads of a thread in flight at
+// once; the scattered side of the transposition is the LDS read, whose strides spread the lanes
+// over the banks.
+template <bool kBwd>
+__global__ __launch_bounds__(256) void pack_patch_k(int M, int Cred, int Mp, size_t sm, size_t sc, const float *w,
+                                                     float *wp)
 {
-    const size_t total = (size_t)chunks * 9 * Mp * 16;
-    for (size_t o = (size_t)blockIdx.x * 256 + threadIdx.x; o < total; o += (size_t)gridDim.x * 256) {
-        const int j = (int)(o & 15);
-        size_t r = o >> 4;
-        const int m = (int)(r % (size_t)Mp);
-        r /= (size_t)Mp;
-        const int tap = (int)(r % 9), chunk = (int)(r / 9);
-        const int c = chunk * 16 + j;
-        wp[o] = (m < M && c < Cred) ? w[(size_t)m * sm + (size_t)c * sc + tap] : 0.0f;
+    constexpr int PITCH = kBwd ? 148 : 145;  // floats between runs in LDS
+    __shared__ float stage[16 * PITCH];
+    const int chunk = blockIdx.y, m0 = blockIdx.x * 16;
+    float v[9];
+#pragma unroll
+    for (int i = 0; i < 9; i++) {
+        const int f = i * 256 + threadIdx.x;
+        const int run = f / 144, r = f - run * 144;
+        bool ok;
+        size_t src;
+        if (!kBwd) {  // run = row m0 + run, r = (channel, tap)
+            ok = m0 + run < M && chunk * 16 + r / 9 < Cred;
+            src = (size_t)(m0 + run) * sm + (size_t)chunk * 16 * sc + r;
+        } else {      // run = reduction channel chunk*16 + run, r = (row, tap)
+            ok = chunk * 16 + run < Cred && m0 + r / 9 < M;
+            src = (size_t)(chunk * 16 + run) * sc + (size_t)m0 * sm + r;
+        }
+        v[i] = ok ? w[src] : 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < 9; i++) {
+        const int f = i * 256 + threadIdx.x;
+        stage[(f / 144) * PITCH + f % 144] = v[i];
+    }
+    __syncthreads();
+    // one float4 (four channels of one row and tap) per thread and pass
+    for (int o = threadIdx.x; o < 9 * 16 * 4; o += 256) {
+        const int j4 = o & 3, ml = (o >> 2) & 15, tap = o >> 6;
+        float4 q;
+        if (!kBwd) {
+            const float *s = stage + ml * PITCH + (j4 * 4) * 9 + tap;
+            q = make_float4(s[0], s[9], s[18], s[27]);
+        } else {
+            const float *s = stage + (j4 * 4) * PITCH + ml * 9 + tap;
+            q = make_float4(s[0], s[PITCH], s[2 * PITCH], s[3 * PITCH]);
+        }
+        *(float4 *)&wp[(((size_t)chunk * 9 + tap) * Mp + m0 + ml) * 16 + j4 * 4] = q;
     }
 }
 
@@ -1053,11 +1087,12 @@ int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, 
     float *wp = (float *)ws;
     float *partial = (float *)(ws + wp_bytes);
     {
-        const size_t blocks = ceil_div(wp_elems, (size_t)256);
-        const size_t cap = (size_t)num_cus() * 16;
         const size_t C9 = (size_t)d->C * 9;
-        hipLaunchKernelGGL(pack_patch_k, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0, stream(), pc.Mout,
-                           pc.Cin, pc.Mp, pc.chunks_total, kBwd ? (size_t)9 : C9, kBwd ? C9 : (size_t)9, w, wp);
+        const dim3 pgrid((unsigned)(pc.Mp / 16), (unsigned)pc.chunks_total);
+        if (!kBwd) hipLaunchKernelGGL(pack_patch_k<false>, pgrid, dim3(256), 0, stream(), pc.Mout, pc.Cin, pc.Mp, C9,
+                                      (size_t)9, w, wp);
+        else hipLaunchKernelGGL(pack_patch_k<true>, pgrid, dim3(256), 0, stream(), pc.Mout, pc.Cin, pc.Mp, (size_t)9, C9,
+                                w, wp);
         DOPT_LAUNCH_CHECK();
     }
     pc.in = in;
