@@ -3,7 +3,8 @@
 // cuda/source/dopt/cuda/nnet/cudnn7.d:608-610, :632-634, :650-652, including the reference's
 // packed output layouts (core/source/dopt/core/ops/nnet.d:222-235).
 //
-// Three launches per op, all deterministic (no atomics):
+// Channels of up to 32768 values take the channel-resident path (one launch, one read of the
+// inputs; see bn_resident_k).  Larger channels take three launches, all deterministic (no atomics):
 //   1. partial: block (channel, slice) accumulates shifted moments of its share of the channel
 //      (shift K = first element of the channel, so that E[(x-K)^2] - E[x-K]^2 does not cancel);
 //   2. finalize: one thread per channel folds the slices in float64, derives mean / 1/std and the
@@ -286,6 +287,148 @@ __global__ __launch_bounds__(kBlock) void bn_grad_apply_k(IdxT total, IdxT C, Id
     }
 }
 
+// ---- channel-resident path -------------------------------------------------------------------
+// One block per channel for tensors whose channel (N * inner values) fits the block's registers:
+// x (and dy) are read ONCE, held in registers between the statistics and the output pass, and
+// the op is one launch instead of three.  Statistics are exact two-pass (mean, then centred
+// squares), reduced across the block in float64.
+constexpr int kResQuads = 8;  // float4 per thread
+
+__device__ inline double wave_sum_d(double v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+    return v;
+}
+
+// Sums kN per-thread values over the block (up to 16 wavefronts); every thread gets the totals.
+template <int kN>
+__device__ inline void block_allsum_d(double (&v)[kN], double (*part)[16], double *total)
+{
+    const int wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+#pragma unroll
+    for (int k = 0; k < kN; k++) {
+        v[k] = wave_sum_d(v[k]);
+        if ((threadIdx.x & 63) == 0) part[k][wave] = v[k];
+    }
+    __syncthreads();
+    if (threadIdx.x < kN) {
+        double r = 0.0;
+        for (int w = 0; w < nw; w++) r += part[threadIdx.x][w];
+        total[threadIdx.x] = r;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kN; k++) v[k] = total[k];
+    __syncthreads();
+}
+
+template <bool kGrad>
+__global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, unsigned inner4, double factor, double eps,
+                                                       const float *x, const float *dy, const float *scale,
+                                                       const float *bias, const float *run_mean, const float *run_var,
+                                                       float *out, float *out1, float *out2)
+{
+    __shared__ double part[3][16];
+    __shared__ double total[3];
+    const unsigned c = blockIdx.x, T = blockDim.x, E4 = N * inner4;
+    const float4 *x4 = (const float4 *)x, *g4 = (const float4 *)dy;
+    float4 xv[kResQuads], gv[kResQuads];
+    unsigned idx[kResQuads];
+#pragma unroll
+    for (int i = 0; i < kResQuads; i++) {
+        const unsigned q = i * T + threadIdx.x;
+        const unsigned n = q / inner4, r = q - n * inner4;
+        idx[i] = q < E4 ? (n * C + c) * inner4 + r : 0xffffffffu;
+        xv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        gv[i] = xv[i];
+        if (q < E4) {
+            xv[i] = x4[idx[i]];
+            if (kGrad) gv[i] = g4[idx[i]];
+        }
+    }
+    const double m = 4.0 * (double)E4;
+    double red1[1] = {0.0};
+    {
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < kResQuads; i++) s += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);  // absent quads are zero
+        red1[0] = (double)s;
+    }
+    block_allsum_d<1>(red1, part, total);
+    const double mean = red1[0] / m;
+    const float mean_hi = (float)mean, mean_lo = (float)(mean - (double)mean_hi);
+    double red3[3] = {0.0, 0.0, 0.0};
+    {
+        float ss = 0.f, g1 = 0.f, g2 = 0.f;
+#pragma unroll
+        for (int i = 0; i < kResQuads; i++) {
+            if (idx[i] == 0xffffffffu) continue;
+            const float d0 = (xv[i].x - mean_hi) - mean_lo, d1 = (xv[i].y - mean_hi) - mean_lo;
+            const float d2 = (xv[i].z - mean_hi) - mean_lo, d3 = (xv[i].w - mean_hi) - mean_lo;
+            ss += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+            if (kGrad) {
+                g1 += (gv[i].x + gv[i].y) + (gv[i].z + gv[i].w);
+                g2 += (gv[i].x * d0 + gv[i].y * d1) + (gv[i].z * d2 + gv[i].w * d3);
+            }
+        }
+        red3[0] = (double)ss;
+        red3[1] = (double)g1;
+        red3[2] = (double)g2;
+    }
+    block_allsum_d<3>(red3, part, total);
+    const double var = red3[0] / m;  // biased
+    const double rstd = 1.0 / sqrt(var + eps);
+    float4 *o4 = (float4 *)out;
+    if (!kGrad) {
+        const float a = (float)((double)scale[c] * rstd), b = bias[c];
+#pragma unroll
+        for (int i = 0; i < kResQuads; i++) {
+            if (idx[i] == 0xffffffffu) continue;
+            float4 r;
+            r.x = a * ((xv[i].x - mean_hi) - mean_lo) + b;
+            r.y = a * ((xv[i].y - mean_hi) - mean_lo) + b;
+            r.z = a * ((xv[i].z - mean_hi) - mean_lo) + b;
+            r.w = a * ((xv[i].w - mean_hi) - mean_lo) + b;
+            o4[idx[i]] = r;
+        }
+        if (threadIdx.x == 0) {
+            const double unbiased = m > 1.0 ? var * m / (m - 1.0) : var;
+            out1[c] = (float)((1.0 - factor) * (double)run_mean[c] + factor * mean);
+            out2[c] = (float)((1.0 - factor) * (double)run_var[c] + factor * unbiased);
+        }
+    } else {
+        const double db = red3[1], ds = rstd * red3[2];  // sum dy, sum dy * xhat
+        CoefG k;
+        k.mean = mean_hi;
+        k.mean_lo = mean_lo;
+        k.rstd = (float)rstd;
+        k.a = (float)((double)scale[c] * rstd);
+        k.b = (float)(db / m);
+        k.d = (float)(ds / m);
+#pragma unroll
+        for (int i = 0; i < kResQuads; i++) {
+            if (idx[i] == 0xffffffffu) continue;
+            o4[idx[i]] = make_float4(bn_dx(k, gv[i].x, xv[i].x), bn_dx(k, gv[i].y, xv[i].y), bn_dx(k, gv[i].z, xv[i].z),
+                                     bn_dx(k, gv[i].w, xv[i].w));
+        }
+        if (threadIdx.x == 0) {
+            out1[c] = (float)ds;
+            out2[c] = (float)db;
+        }
+    }
+}
+
+// Threads for the resident path, or 0 when the channel does not fit (or is not 128-bit addressable).
+unsigned resident_threads(size_t N, size_t C, size_t inner, const void *a, const void *b, const void *o)
+{
+    if ((inner & 3) != 0 || !aligned16(a) || (b && !aligned16(b)) || !aligned16(o)) return 0;
+    const size_t E4 = N * (inner / 4);
+    if (E4 == 0 || E4 > (size_t)kResQuads * 1024 || N * C * (inner / 4) >= 0xffffffffull) return 0;
+    size_t T = (ceil_div(E4, (size_t)kResQuads) + 63) / 64 * 64;
+    return (unsigned)(T < 64 ? 64 : T);
+}
+
 size_t pick_slices(size_t N, size_t C)
 {
     size_t S = ceil_div((size_t)num_cus() * 8, C);
@@ -353,6 +496,15 @@ int dopt_hip_bn_train(size_t N, size_t C, size_t inner, double momentum, const f
     DOPT_REQUIRE(x && scale && bias && run_mean && run_var && packed, "dopt_hip_bn_train: null argument");
     DOPT_REQUIRE(C <= 0x7fffffffu / kMaxSlices, "dopt_hip_bn_train: too many channels");
     DOPT_ENSURE_INIT();
+    double factor = 1.0 - momentum;    // cudnn7.d:592
+    double eps = (double)1e-5f;        // cudnn7.d:610
+    if (unsigned T = resident_threads(N, C, inner, x, nullptr, packed)) {
+        hipLaunchKernelGGL(bn_resident_k<false>, dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N, (unsigned)C,
+                           (unsigned)(inner / 4), factor, eps, x, (const float *)nullptr, scale, bias, run_mean, run_var,
+                           packed, packed + total, packed + total + C);
+        DOPT_LAUNCH_CHECK();
+        return DOPT_HIP_OK;
+    }
     // workspace: [partials C*S*4 floats | coefficient table C * 16 bytes]
     size_t part_bytes = C * kMaxSlices * 4 * sizeof(float);
     char *ws = (char *)workspace(part_bytes + C * sizeof(Coef));
@@ -361,8 +513,6 @@ int dopt_hip_bn_train(size_t N, size_t C, size_t inner, double momentum, const f
     Coef *coef = (Coef *)(ws + part_bytes);
     size_t S;
     if (int rc = launch_partial<false>(N, C, inner, x, nullptr, partial, &S)) return rc;
-    double factor = 1.0 - momentum;    // cudnn7.d:592
-    double eps = (double)1e-5f;        // cudnn7.d:610
     hipLaunchKernelGGL(bn_train_finalize_k, dim3((unsigned)ceil_div(C, (size_t)kBlock)), dim3(kBlock), 0, stream(), N,
                        C, inner, S, factor, eps, x, partial, scale, bias, run_mean, run_var, coef, packed + total,
                        packed + total + C);
@@ -378,6 +528,14 @@ int dopt_hip_bn_grad(size_t N, size_t C, size_t inner, const float *dy, const fl
     DOPT_REQUIRE(dy && x && scale && packed, "dopt_hip_bn_grad: null argument");
     DOPT_REQUIRE(C <= 0x7fffffffu / kMaxSlices, "dopt_hip_bn_grad: too many channels");
     DOPT_ENSURE_INIT();
+    double eps = (double)1e-5f;  // cudnn7.d:634
+    if (unsigned T = resident_threads(N, C, inner, x, dy, packed)) {
+        hipLaunchKernelGGL(bn_resident_k<true>, dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N, (unsigned)C,
+                           (unsigned)(inner / 4), 0.0, eps, x, dy, scale, (const float *)nullptr, (const float *)nullptr,
+                           (const float *)nullptr, packed, packed + total, packed + total + C);
+        DOPT_LAUNCH_CHECK();
+        return DOPT_HIP_OK;
+    }
     size_t part_bytes = C * kMaxSlices * 4 * sizeof(float);
     char *ws = (char *)workspace(part_bytes + C * sizeof(CoefG));
     if (!ws) return DOPT_HIP_ERR_OOM;
@@ -385,7 +543,6 @@ int dopt_hip_bn_grad(size_t N, size_t C, size_t inner, const float *dy, const fl
     CoefG *coef = (CoefG *)(ws + part_bytes);
     size_t S;
     if (int rc = launch_partial<true>(N, C, inner, x, dy, partial, &S)) return rc;
-    double eps = (double)1e-5f;  // cudnn7.d:634
     hipLaunchKernelGGL(bn_grad_finalize_k, dim3((unsigned)ceil_div(C, (size_t)kBlock)), dim3(kBlock), 0, stream(), N, C,
                        inner, S, eps, x, partial, scale, coef, packed + total, packed + total + C);
     DOPT_LAUNCH_CHECK();

@@ -356,7 +356,10 @@ def test_bias(shape):
 
 # ----------------------------------------------------------------------------- batch norm
 @pytest.mark.parametrize("shape", [(4, 3, 5, 5), (8, 6), (2, 4, 3, 1), (8, 64, 32, 32), (128, 512, 2, 2), (3, 2),
-                                   (16, 16, 16, 16)])
+                                   (16, 16, 16, 16),
+                                   (40, 4, 32, 32),     # channel too large for the register-resident path
+                                   (128, 8, 16, 16),    # the largest channel that path takes (1024 threads)
+                                   (5, 7, 4, 3)])       # ragged tail in the resident path
 def test_batchnorm_train_grad_infer(shape):
     r = rng(61)
     C = shape[1]
