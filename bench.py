@@ -3,7 +3,7 @@
 CIFAR-shape network with batch norm at batch 128 in fp32, on one MI355X, through HIPPlan and the
 kernel library.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--unfused] [--no-views] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--unfused] [--no-views] [--no-fuse] [--no-cpu]
 
 A step is one execution of the update plan on device-resident synthetic inputs (inputs are in
 HBM before the timed region starts).  After the timed region the same step is run again with
@@ -35,7 +35,7 @@ def conv_flops(n, c, k, h):
     return 2.0 * n * k * c * 9 * h * h
 
 
-def build_step(batch, fused, views, timing, seed=0):
+def build_step(batch, fused, views, timing, seed=0, fuse=True):
     from dopt_amd import core, nnet, online, ops
     rng = np.random.default_rng(seed)
     features = core.float32([batch, 3, 32, 32])
@@ -45,6 +45,7 @@ def build_step(batch, fused, views, timing, seed=0):
     net = nnet.DAGNetwork([features], [preds])
     loss = nnet.crossEntropy(preds.trainOutput, labels) + net.paramLoss
     flags = (core.PLAN_VIEWS if views else 0) | (core.PLAN_TIMING if timing else 0)
+    flags |= core.PLAN_FUSE if (fuse and views) else 0
     if fused:
         updater = online.fused_sgd([loss, preds.trainOutput], net.params, net.paramProj, 0.01, 0.0, flags=flags)
     else:
@@ -91,6 +92,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--unfused", action="store_true", help="run the reference's op-graph SGD instead of the fused kernel")
     ap.add_argument("--no-views", action="store_true", help="disable the copy-eliding plan rewrites")
+    ap.add_argument("--no-fuse", action="store_true", help="run every operation as its own kernel")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-kernel-timing", action="store_true", help="skip the per-kernel event pass")
     a = ap.parse_args()
@@ -99,9 +101,9 @@ def main():
 
     from dopt_amd import capi, ops
     capi.check(capi.load().dopt_hip_init(0))
-    fused, views = not a.unfused, not a.no_views
+    fused, views, fuse = not a.unfused, not a.no_views, not a.no_fuse
 
-    updater, args, net = build_step(BATCH, fused, views, timing=False)
+    updater, args, net = build_step(BATCH, fused, views, timing=False, fuse=fuse)
     for _ in range(a.warmup):
         updater.step_async(args)
     ops.sync()
@@ -125,7 +127,7 @@ def main():
         "config": {"workload": "config 4: VGG-16 + batch norm, input [128,3,32,32], FC 512-512-10, softmax "
                                "cross-entropy, one forward + backward + SGD(lr 0.01) step",
                    "global_batch": BATCH, "optimizer": "fused multi-tensor SGD" if fused else "op-graph SGD",
-                   "plan_rewrites": "views" if views else "none",
+                   "plan_rewrites": ("views+fuse" if fuse else "views") if views else "none",
                    "kernels_per_step": stats["kernels"] + (1 if fused else 0),
                    "plan_buffer_MB": round(stats["buffer_bytes"] / 2**20, 1),
                    "parameters": int(sum(p.volume for p in net.params)), "loss_after": round(loss, 5)},
@@ -136,7 +138,7 @@ def main():
     if not a.no_kernel_timing:
         # Same step, every kernel object bracketed by hipEvents on the library stream.
         del updater
-        tup, targs, _ = build_step(BATCH, fused, views, timing=True)
+        tup, targs, _ = build_step(BATCH, fused, views, timing=True, fuse=fuse)
         for _ in range(2):
             tup.step_async(targs)
         ops.sync()
@@ -150,8 +152,9 @@ def main():
                     for k in after}
         fwd = sum(conv_flops(BATCH, c, k, h) for c, k, h in VGG_CONVS)
         bwd_data = fwd - conv_flops(BATCH, *VGG_CONVS[0])   # the first layer's input needs no gradient
-        gather_us = per_step["convolution"][0] + per_step["convolutionFeaturesGrad"][0]
-        gather_launches = per_step["convolution"][1] + per_step["convolutionFeaturesGrad"][1]
+        conv_keys = [k for k in ("convolution", "convolution+addBias", "convolutionFeaturesGrad") if k in per_step]
+        gather_us = sum(per_step[k][0] for k in conv_keys)
+        gather_launches = sum(per_step[k][1] for k in conv_keys)
         gather_tflops = (fwd + bwd_data) / (gather_us * 1e-6) / 1e12
         wgrad_tflops = fwd / (per_step["convolutionFiltersGrad"][0] * 1e-6) / 1e12
         result["roofline"] = {

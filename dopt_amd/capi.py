@@ -60,6 +60,7 @@ PROTOTYPES = {
     "dopt_hip_transpose2d": [_sz, _sz, _vp, _vp],
     "dopt_hip_sgemm": [_sz, _sz, _sz, _vp, _vp, _vp],
     "dopt_hip_conv_fwd": [C.POINTER(ConvDesc), _vp, _vp, _vp],
+    "dopt_hip_conv_fwd_bias": [C.POINTER(ConvDesc), _vp, _vp, _vp, _vp],
     "dopt_hip_conv_bwd_data": [C.POINTER(ConvDesc), _vp, _vp, _vp],
     "dopt_hip_conv_bwd_filter": [C.POINTER(ConvDesc), _vp, _vp, _vp],
     "dopt_hip_maxpool_fwd": [_sz, _sz, _sz, _sz, _sz, _sz, _vp, _vp],
@@ -71,7 +72,9 @@ PROTOTYPES = {
     "dopt_hip_bias_fwd": [_sz, _sz, _sz, _vp, _vp, _vp],
     "dopt_hip_bias_bwd": [_sz, _sz, _sz, _vp, _vp],
     "dopt_hip_bn_train": [_sz, _sz, _sz, _d, _vp, _vp, _vp, _vp, _vp, _vp],
+    "dopt_hip_bn_train_relu": [_sz, _sz, _sz, _d, _vp, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_bn_grad": [_sz, _sz, _sz, _vp, _vp, _vp, _vp],
+    "dopt_hip_bn_grad_relu": [_sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_bn_infer": [_sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_optim_create": [_i, C.POINTER(TensorRef), C.POINTER(_vp)],
     "dopt_hip_optim_destroy": [_vp],

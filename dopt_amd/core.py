@@ -684,6 +684,7 @@ def grad(objective, wrt):
 
 PLAN_VIEWS = 1
 PLAN_TIMING = 2
+PLAN_FUSE = 4
 
 
 class Plan:

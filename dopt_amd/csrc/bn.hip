@@ -38,6 +38,15 @@ __device__ inline float wave_sum(float v)
     return v;
 }
 
+// Fused ReLU: forward clamps the normalised value; backward drops the gradient where the ReLU
+// output y is not positive (the same tests as the stand-alone relu / reluGrad kernels).
+__device__ inline float relu1(float v) { return v < 0.0f ? 0.0f : v; }
+__device__ inline float masked(float g, float y) { return y > 0.0f ? g : 0.0f; }
+__device__ inline float4 masked4(float4 g, float4 y)
+{
+    return make_float4(masked(g.x, y.x), masked(g.y, y.y), masked(g.z, y.z), masked(g.w, y.w));
+}
+
 // Sums four per-thread values over the block; results valid in thread 0.
 __device__ inline void block_sum(float (&v)[4], float (*part)[kBlock / 64])
 {
@@ -63,7 +72,7 @@ __device__ inline void block_sum(float (&v)[4], float (*part)[kBlock / 64])
 // kFlat: for small `inner` the block walks (n, i) pairs with a flat index instead of rows.
 template <bool kGrad, bool kFlat>
 __global__ __launch_bounds__(kBlock) void bn_partial_k(size_t N, size_t C, size_t inner, size_t S, const float *x,
-                                                        const float *dy, float *partial)
+                                                        const float *dy, const float *ymask, float *partial)
 {
     __shared__ float part[4][kBlock / 64];
     const size_t c = blockIdx.x % C, s = blockIdx.x / C;
@@ -79,6 +88,7 @@ __global__ __launch_bounds__(kBlock) void bn_partial_k(size_t N, size_t C, size_
             acc[1] += v * v;
             if (kGrad) {
                 float g = dy[e];
+                if (ymask) g = masked(g, ymask[e]);
                 acc[2] += g;
                 acc[3] += g * v;
             }
@@ -89,6 +99,7 @@ __global__ __launch_bounds__(kBlock) void bn_partial_k(size_t N, size_t C, size_
         for (size_t n = s; n < N; n += S) {
             const float4 *row = (const float4 *)(x + (n * C + c) * inner);
             const float4 *grow = (const float4 *)(dy + (n * C + c) * inner);
+            const float4 *mrow = (const float4 *)(ymask + (n * C + c) * inner);
             for (size_t i = threadIdx.x; i < inner4; i += kBlock) {
                 float4 q = row[i];
                 float v0 = q.x - K, v1 = q.y - K, v2 = q.z - K, v3 = q.w - K;
@@ -96,6 +107,7 @@ __global__ __launch_bounds__(kBlock) void bn_partial_k(size_t N, size_t C, size_
                 acc[1] += (v0 * v0 + v1 * v1) + (v2 * v2 + v3 * v3);
                 if (kGrad) {
                     float4 g = grow[i];
+                    if (ymask) g = masked4(g, mrow[i]);
                     acc[2] += (g.x + g.y) + (g.z + g.w);
                     acc[3] += (g.x * v0 + g.y * v1) + (g.z * v2 + g.w * v3);
                 }
@@ -201,7 +213,7 @@ __global__ __launch_bounds__(kBlock) void bn_grad_finalize_k(size_t N, size_t C,
 // y = a * ((x - mean) - mean_lo) + b
 template <typename IdxT, bool kVec>
 __global__ __launch_bounds__(kBlock) void bn_apply_k(IdxT total, IdxT C, IdxT inner, const float *x, const Coef *coef,
-                                                      float *y)
+                                                      float *y, int relu)
 {
     if (kVec) {
         const IdxT n4 = total >> 2, inner4 = inner >> 2;
@@ -228,6 +240,7 @@ __global__ __launch_bounds__(kBlock) void bn_apply_k(IdxT total, IdxT C, IdxT in
                     r.y = k[u].a * ((v[u].y - k[u].mean) - k[u].mean_lo) + k[u].b;
                     r.z = k[u].a * ((v[u].z - k[u].mean) - k[u].mean_lo) + k[u].b;
                     r.w = k[u].a * ((v[u].w - k[u].mean) - k[u].mean_lo) + k[u].b;
+                    if (relu) r = make_float4(relu1(r.x), relu1(r.y), relu1(r.z), relu1(r.w));
                     y4[i] = r;
                 }
             }
@@ -235,7 +248,8 @@ __global__ __launch_bounds__(kBlock) void bn_apply_k(IdxT total, IdxT C, IdxT in
     } else {
         for (IdxT i = (IdxT)blockIdx.x * kBlock + threadIdx.x; i < total; i += (IdxT)gridDim.x * kBlock) {
             Coef k = coef[(i / inner) % C];
-            y[i] = k.a * ((x[i] - k.mean) - k.mean_lo) + k.b;
+            const float r = k.a * ((x[i] - k.mean) - k.mean_lo) + k.b;
+            y[i] = relu ? relu1(r) : r;
         }
     }
 }
@@ -249,7 +263,8 @@ __device__ inline float bn_dx(const CoefG &k, float dy, float x)
 
 template <typename IdxT, bool kVec>
 __global__ __launch_bounds__(kBlock) void bn_grad_apply_k(IdxT total, IdxT C, IdxT inner, const float *dy,
-                                                           const float *x, const CoefG *coef, float *dx)
+                                                           const float *ymask, const float *x, const CoefG *coef,
+                                                           float *dx)
 {
     if (kVec) {
         const IdxT n4 = total >> 2, inner4 = inner >> 2;
@@ -266,6 +281,7 @@ __global__ __launch_bounds__(kBlock) void bn_grad_apply_k(IdxT total, IdxT C, Id
                 if (i < n4) {
                     v[u] = x4[i];
                     g[u] = g4[i];
+                    if (ymask) g[u] = masked4(g[u], ((const float4 *)ymask)[i]);
                     ch[u] = (i / inner4) % C;
                 }
             }
@@ -282,7 +298,7 @@ __global__ __launch_bounds__(kBlock) void bn_grad_apply_k(IdxT total, IdxT C, Id
     } else {
         for (IdxT i = (IdxT)blockIdx.x * kBlock + threadIdx.x; i < total; i += (IdxT)gridDim.x * kBlock) {
             CoefG k = coef[(i / inner) % C];
-            dx[i] = bn_dx(k, dy[i], x[i]);
+            dx[i] = bn_dx(k, ymask ? masked(dy[i], ymask[i]) : dy[i], x[i]);
         }
     }
 }
@@ -327,7 +343,7 @@ template <bool kGrad>
 __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, unsigned inner4, double factor, double eps,
                                                        const float *x, const float *dy, const float *scale,
                                                        const float *bias, const float *run_mean, const float *run_var,
-                                                       float *out, float *out1, float *out2)
+                                                       const float *ymask, int relu, float *out, float *out1, float *out2)
 {
     __shared__ double part[3][16];
     __shared__ double total[3];
@@ -344,7 +360,10 @@ __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, un
         gv[i] = xv[i];
         if (q < E4) {
             xv[i] = x4[idx[i]];
-            if (kGrad) gv[i] = g4[idx[i]];
+            if (kGrad) {
+                gv[i] = g4[idx[i]];
+                if (ymask) gv[i] = masked4(gv[i], ((const float4 *)ymask)[idx[i]]);
+            }
         }
     }
     const double m = 4.0 * (double)E4;
@@ -390,6 +409,7 @@ __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, un
             r.y = a * ((xv[i].y - mean_hi) - mean_lo) + b;
             r.z = a * ((xv[i].z - mean_hi) - mean_lo) + b;
             r.w = a * ((xv[i].w - mean_hi) - mean_lo) + b;
+            if (relu) r = make_float4(relu1(r.x), relu1(r.y), relu1(r.z), relu1(r.w));
             o4[idx[i]] = r;
         }
         if (threadIdx.x == 0) {
@@ -445,22 +465,24 @@ unsigned apply_grid(size_t total, bool vec)
 }
 
 template <bool kGrad>
-int launch_partial(size_t N, size_t C, size_t inner, const float *x, const float *dy, float *partial, size_t *S_out)
+int launch_partial(size_t N, size_t C, size_t inner, const float *x, const float *dy, const float *ymask,
+                   float *partial, size_t *S_out)
 {
-    bool rows = inner >= 256 && (inner & 3) == 0 && aligned16(x) && (!kGrad || aligned16(dy));
+    bool rows = inner >= 256 && (inner & 3) == 0 && aligned16(x) && (!kGrad || aligned16(dy)) &&
+                (!ymask || aligned16(ymask));
     size_t S = rows ? pick_slices(N, C) : 1;
     *S_out = S;
     if (rows)
         hipLaunchKernelGGL((bn_partial_k<kGrad, false>), dim3((unsigned)(C * S)), dim3(kBlock), 0, stream(), N, C, inner,
-                           S, x, dy, partial);
+                           S, x, dy, ymask, partial);
     else
         hipLaunchKernelGGL((bn_partial_k<kGrad, true>), dim3((unsigned)C), dim3(kBlock), 0, stream(), N, C, inner, S, x,
-                           dy, partial);
+                           dy, ymask, partial);
     DOPT_LAUNCH_CHECK();
     return DOPT_HIP_OK;
 }
 
-int launch_apply(size_t total, size_t C, size_t inner, const float *x, const Coef *coef, float *y)
+int launch_apply(size_t total, size_t C, size_t inner, const float *x, const Coef *coef, float *y, int relu)
 {
     bool vec = (inner & 3) == 0 && aligned16(x) && aligned16(y);
     unsigned grid = apply_grid(total, vec);
@@ -468,17 +490,101 @@ int launch_apply(size_t total, size_t C, size_t inner, const float *x, const Coe
     if (small) {
         if (vec)
             hipLaunchKernelGGL((bn_apply_k<unsigned, true>), dim3(grid), dim3(kBlock), 0, stream(), (unsigned)total,
-                               (unsigned)C, (unsigned)inner, x, coef, y);
+                               (unsigned)C, (unsigned)inner, x, coef, y, relu);
         else
             hipLaunchKernelGGL((bn_apply_k<unsigned, false>), dim3(grid), dim3(kBlock), 0, stream(), (unsigned)total,
-                               (unsigned)C, (unsigned)inner, x, coef, y);
+                               (unsigned)C, (unsigned)inner, x, coef, y, relu);
     } else {
         if (vec)
             hipLaunchKernelGGL((bn_apply_k<size_t, true>), dim3(grid), dim3(kBlock), 0, stream(), total, C, inner, x,
-                               coef, y);
+                               coef, y, relu);
         else
             hipLaunchKernelGGL((bn_apply_k<size_t, false>), dim3(grid), dim3(kBlock), 0, stream(), total, C, inner, x,
-                               coef, y);
+                               coef, y, relu);
+    }
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+int bn_train_impl(size_t N, size_t C, size_t inner, double momentum, const float *x, const float *scale,
+                  const float *bias, const float *run_mean, const float *run_var, float *packed, int relu,
+                  const char *who)
+{
+    size_t total = N * C * inner;
+    DOPT_REQUIRE(total > 0, "%s: empty input", who);
+    DOPT_REQUIRE(x && scale && bias && run_mean && run_var && packed, "%s: null argument", who);
+    DOPT_REQUIRE(C <= 0x7fffffffu / kMaxSlices, "%s: too many channels", who);
+    DOPT_ENSURE_INIT();
+    double factor = 1.0 - momentum;    // cudnn7.d:592
+    double eps = (double)1e-5f;        // cudnn7.d:610
+    if (unsigned T = resident_threads(N, C, inner, x, nullptr, packed)) {
+        hipLaunchKernelGGL(bn_resident_k<false>, dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N, (unsigned)C,
+                           (unsigned)(inner / 4), factor, eps, x, (const float *)nullptr, scale, bias, run_mean, run_var,
+                           (const float *)nullptr, relu, packed, packed + total, packed + total + C);
+        DOPT_LAUNCH_CHECK();
+        return DOPT_HIP_OK;
+    }
+    // workspace: [partials C*S*4 floats | coefficient table C * 16 bytes]
+    size_t part_bytes = C * kMaxSlices * 4 * sizeof(float);
+    char *ws = (char *)workspace(part_bytes + C * sizeof(Coef));
+    if (!ws) return DOPT_HIP_ERR_OOM;
+    float *partial = (float *)ws;
+    Coef *coef = (Coef *)(ws + part_bytes);
+    size_t S;
+    if (int rc = launch_partial<false>(N, C, inner, x, nullptr, nullptr, partial, &S)) return rc;
+    hipLaunchKernelGGL(bn_train_finalize_k, dim3((unsigned)ceil_div(C, (size_t)kBlock)), dim3(kBlock), 0, stream(), N,
+                       C, inner, S, factor, eps, x, partial, scale, bias, run_mean, run_var, coef, packed + total,
+                       packed + total + C);
+    DOPT_LAUNCH_CHECK();
+    return launch_apply(total, C, inner, x, coef, packed, relu);
+}
+
+int bn_grad_impl(size_t N, size_t C, size_t inner, const float *dy, const float *ymask, const float *x,
+                 const float *scale, float *packed, const char *who)
+{
+    size_t total = N * C * inner;
+    DOPT_REQUIRE(total > 0, "%s: empty input", who);
+    DOPT_REQUIRE(dy && x && scale && packed, "%s: null argument", who);
+    DOPT_REQUIRE(C <= 0x7fffffffu / kMaxSlices, "%s: too many channels", who);
+    DOPT_ENSURE_INIT();
+    double eps = (double)1e-5f;  // cudnn7.d:634
+    if (unsigned T = resident_threads(N, C, inner, x, dy, packed)) {
+        if (!ymask || aligned16(ymask)) {
+            hipLaunchKernelGGL(bn_resident_k<true>, dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N, (unsigned)C,
+                               (unsigned)(inner / 4), 0.0, eps, x, dy, scale, (const float *)nullptr,
+                               (const float *)nullptr, (const float *)nullptr, ymask, 0, packed, packed + total,
+                               packed + total + C);
+            DOPT_LAUNCH_CHECK();
+            return DOPT_HIP_OK;
+        }
+    }
+    size_t part_bytes = C * kMaxSlices * 4 * sizeof(float);
+    char *ws = (char *)workspace(part_bytes + C * sizeof(CoefG));
+    if (!ws) return DOPT_HIP_ERR_OOM;
+    float *partial = (float *)ws;
+    CoefG *coef = (CoefG *)(ws + part_bytes);
+    size_t S;
+    if (int rc = launch_partial<true>(N, C, inner, x, dy, ymask, partial, &S)) return rc;
+    hipLaunchKernelGGL(bn_grad_finalize_k, dim3((unsigned)ceil_div(C, (size_t)kBlock)), dim3(kBlock), 0, stream(), N, C,
+                       inner, S, eps, x, partial, scale, coef, packed + total, packed + total + C);
+    DOPT_LAUNCH_CHECK();
+    bool vec = (inner & 3) == 0 && aligned16(x) && aligned16(dy) && aligned16(packed) && (!ymask || aligned16(ymask));
+    unsigned grid = apply_grid(total, vec);
+    bool small = total < 0x7fffffffull;
+    if (small) {
+        if (vec)
+            hipLaunchKernelGGL((bn_grad_apply_k<unsigned, true>), dim3(grid), dim3(kBlock), 0, stream(), (unsigned)total,
+                               (unsigned)C, (unsigned)inner, dy, ymask, x, coef, packed);
+        else
+            hipLaunchKernelGGL((bn_grad_apply_k<unsigned, false>), dim3(grid), dim3(kBlock), 0, stream(),
+                               (unsigned)total, (unsigned)C, (unsigned)inner, dy, ymask, x, coef, packed);
+    } else {
+        if (vec)
+            hipLaunchKernelGGL((bn_grad_apply_k<size_t, true>), dim3(grid), dim3(kBlock), 0, stream(), total, C, inner,
+                               dy, ymask, x, coef, packed);
+        else
+            hipLaunchKernelGGL((bn_grad_apply_k<size_t, false>), dim3(grid), dim3(kBlock), 0, stream(), total, C, inner,
+                               dy, ymask, x, coef, packed);
     }
     DOPT_LAUNCH_CHECK();
     return DOPT_HIP_OK;
@@ -491,81 +597,26 @@ extern "C" {
 int dopt_hip_bn_train(size_t N, size_t C, size_t inner, double momentum, const float *x, const float *scale,
                       const float *bias, const float *run_mean, const float *run_var, float *packed)
 {
-    size_t total = N * C * inner;
-    DOPT_REQUIRE(total > 0, "dopt_hip_bn_train: empty input");
-    DOPT_REQUIRE(x && scale && bias && run_mean && run_var && packed, "dopt_hip_bn_train: null argument");
-    DOPT_REQUIRE(C <= 0x7fffffffu / kMaxSlices, "dopt_hip_bn_train: too many channels");
-    DOPT_ENSURE_INIT();
-    double factor = 1.0 - momentum;    // cudnn7.d:592
-    double eps = (double)1e-5f;        // cudnn7.d:610
-    if (unsigned T = resident_threads(N, C, inner, x, nullptr, packed)) {
-        hipLaunchKernelGGL(bn_resident_k<false>, dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N, (unsigned)C,
-                           (unsigned)(inner / 4), factor, eps, x, (const float *)nullptr, scale, bias, run_mean, run_var,
-                           packed, packed + total, packed + total + C);
-        DOPT_LAUNCH_CHECK();
-        return DOPT_HIP_OK;
-    }
-    // workspace: [partials C*S*4 floats | coefficient table C * 16 bytes]
-    size_t part_bytes = C * kMaxSlices * 4 * sizeof(float);
-    char *ws = (char *)workspace(part_bytes + C * sizeof(Coef));
-    if (!ws) return DOPT_HIP_ERR_OOM;
-    float *partial = (float *)ws;
-    Coef *coef = (Coef *)(ws + part_bytes);
-    size_t S;
-    if (int rc = launch_partial<false>(N, C, inner, x, nullptr, partial, &S)) return rc;
-    hipLaunchKernelGGL(bn_train_finalize_k, dim3((unsigned)ceil_div(C, (size_t)kBlock)), dim3(kBlock), 0, stream(), N,
-                       C, inner, S, factor, eps, x, partial, scale, bias, run_mean, run_var, coef, packed + total,
-                       packed + total + C);
-    DOPT_LAUNCH_CHECK();
-    return launch_apply(total, C, inner, x, coef, packed);
+    return bn_train_impl(N, C, inner, momentum, x, scale, bias, run_mean, run_var, packed, 0, "dopt_hip_bn_train");
+}
+
+int dopt_hip_bn_train_relu(size_t N, size_t C, size_t inner, double momentum, const float *x, const float *scale,
+                           const float *bias, const float *run_mean, const float *run_var, float *packed)
+{
+    return bn_train_impl(N, C, inner, momentum, x, scale, bias, run_mean, run_var, packed, 1, "dopt_hip_bn_train_relu");
 }
 
 int dopt_hip_bn_grad(size_t N, size_t C, size_t inner, const float *dy, const float *x, const float *scale,
                      float *packed)
 {
-    size_t total = N * C * inner;
-    DOPT_REQUIRE(total > 0, "dopt_hip_bn_grad: empty input");
-    DOPT_REQUIRE(dy && x && scale && packed, "dopt_hip_bn_grad: null argument");
-    DOPT_REQUIRE(C <= 0x7fffffffu / kMaxSlices, "dopt_hip_bn_grad: too many channels");
-    DOPT_ENSURE_INIT();
-    double eps = (double)1e-5f;  // cudnn7.d:634
-    if (unsigned T = resident_threads(N, C, inner, x, dy, packed)) {
-        hipLaunchKernelGGL(bn_resident_k<true>, dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N, (unsigned)C,
-                           (unsigned)(inner / 4), 0.0, eps, x, dy, scale, (const float *)nullptr, (const float *)nullptr,
-                           (const float *)nullptr, packed, packed + total, packed + total + C);
-        DOPT_LAUNCH_CHECK();
-        return DOPT_HIP_OK;
-    }
-    size_t part_bytes = C * kMaxSlices * 4 * sizeof(float);
-    char *ws = (char *)workspace(part_bytes + C * sizeof(CoefG));
-    if (!ws) return DOPT_HIP_ERR_OOM;
-    float *partial = (float *)ws;
-    CoefG *coef = (CoefG *)(ws + part_bytes);
-    size_t S;
-    if (int rc = launch_partial<true>(N, C, inner, x, dy, partial, &S)) return rc;
-    hipLaunchKernelGGL(bn_grad_finalize_k, dim3((unsigned)ceil_div(C, (size_t)kBlock)), dim3(kBlock), 0, stream(), N, C,
-                       inner, S, eps, x, partial, scale, coef, packed + total, packed + total + C);
-    DOPT_LAUNCH_CHECK();
-    bool vec = (inner & 3) == 0 && aligned16(x) && aligned16(dy) && aligned16(packed);
-    unsigned grid = apply_grid(total, vec);
-    bool small = total < 0x7fffffffull;
-    if (small) {
-        if (vec)
-            hipLaunchKernelGGL((bn_grad_apply_k<unsigned, true>), dim3(grid), dim3(kBlock), 0, stream(), (unsigned)total,
-                               (unsigned)C, (unsigned)inner, dy, x, coef, packed);
-        else
-            hipLaunchKernelGGL((bn_grad_apply_k<unsigned, false>), dim3(grid), dim3(kBlock), 0, stream(),
-                               (unsigned)total, (unsigned)C, (unsigned)inner, dy, x, coef, packed);
-    } else {
-        if (vec)
-            hipLaunchKernelGGL((bn_grad_apply_k<size_t, true>), dim3(grid), dim3(kBlock), 0, stream(), total, C, inner,
-                               dy, x, coef, packed);
-        else
-            hipLaunchKernelGGL((bn_grad_apply_k<size_t, false>), dim3(grid), dim3(kBlock), 0, stream(), total, C, inner,
-                               dy, x, coef, packed);
-    }
-    DOPT_LAUNCH_CHECK();
-    return DOPT_HIP_OK;
+    return bn_grad_impl(N, C, inner, dy, nullptr, x, scale, packed, "dopt_hip_bn_grad");
+}
+
+int dopt_hip_bn_grad_relu(size_t N, size_t C, size_t inner, const float *dy, const float *y, const float *x,
+                          const float *scale, float *packed)
+{
+    DOPT_REQUIRE(y != nullptr, "dopt_hip_bn_grad_relu: null argument");
+    return bn_grad_impl(N, C, inner, dy, y, x, scale, packed, "dopt_hip_bn_grad_relu");
 }
 
 int dopt_hip_bn_infer(size_t N, size_t C, size_t inner, const float *x, const float *scale, const float *bias,
@@ -580,7 +631,7 @@ int dopt_hip_bn_infer(size_t N, size_t C, size_t inner, const float *x, const fl
     hipLaunchKernelGGL(bn_infer_prepare_k, dim3((unsigned)ceil_div(C, (size_t)kBlock)), dim3(kBlock), 0, stream(), C,
                        1e-5 /* cudnn7.d:652 */, scale, bias, mean, var, coef);
     DOPT_LAUNCH_CHECK();
-    return launch_apply(total, C, inner, x, coef, y);
+    return launch_apply(total, C, inner, x, coef, y, 0);
 }
 
 }  // extern "C"

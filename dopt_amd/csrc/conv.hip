@@ -201,6 +201,7 @@ struct PatchConv {
     const float *in;   // gathered operand [N, Cin, IH, IW]
     const float *wp;   // packed filter [chunks][9][Mp][16]
     float *out;        // [N, Mout, OH, OW], or `splits` partial copies of it
+    const float *bias; // optional [Mout], added to the finished sums (by the split reduction when there is one)
     int N, Cin, IH, IW, Mout, OH, OW;
     int PT, PL;        // input row / column of patch position (0,0) is (oh0 - PT, -PL)
     int flip;          // 1: tap (tr,ts) reads patch offset (2-tr, 2-ts); 0: (tr, ts)
@@ -383,6 +384,7 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_patch_k(Pat
     }
 
     float *outp = p.out + (size_t)split * p.out_elems;
+    const bool add_bias = p.bias != nullptr && p.splits == 1;
 #pragma unroll
     for (int j = 0; j < NI; j++) {
         const int col = n0 + wn * (BN / T::WN) + j * 32 + l32;
@@ -394,7 +396,7 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_patch_k(Pat
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int m = m0 + wm * (BM / T::WM) + i * 32 + acc_row(v, lane);
-                if (m < p.Mout) base[(size_t)m * OHW] = acc[i][j][v];
+                if (m < p.Mout) base[(size_t)m * OHW] = add_bias ? acc[i][j][v] + p.bias[m] : acc[i][j][v];
             }
     }
 }
@@ -900,8 +902,10 @@ __global__ __launch_bounds__(768, 1) void conv_wgrad_patch_k(WgradPatch p)
 
 // ------------------------------------------------------------------------------------ helpers
 
-// out[i] = sum_s partial[s][i], s ascending.
-__global__ __launch_bounds__(256) void splitk_reduce_k(size_t n4, int splits, const float4 *partial, float4 *out)
+// out[i] = sum_s partial[s][i], s ascending; plus bias[channel of i] when a bias is given
+// (channel = (i / inner) % C for an [N, C, inner] output).
+__global__ __launch_bounds__(256) void splitk_reduce_k(size_t n4, int splits, const float4 *partial, float4 *out,
+                                                        const float *bias, unsigned C, unsigned inner)
 {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (size_t)gridDim.x * 256) {
         float4 acc = partial[i];
@@ -911,6 +915,13 @@ __global__ __launch_bounds__(256) void splitk_reduce_k(size_t n4, int splits, co
             acc.y += v.y;
             acc.z += v.z;
             acc.w += v.w;
+        }
+        if (bias) {
+            const size_t e = i * 4;
+            acc.x += bias[(e / inner) % C];
+            acc.y += bias[((e + 1) / inner) % C];
+            acc.z += bias[((e + 2) / inner) % C];
+            acc.w += bias[((e + 3) / inner) % C];
         }
         out[i] = acc;
     }
@@ -983,7 +994,8 @@ int check_desc(const dopt_hip_conv_desc *d, size_t *P, size_t *Q, const char *wh
     return DOPT_HIP_OK;
 }
 
-int launch_splitk_reduce(size_t elems, int splits, const float *partial, float *out)
+int launch_splitk_reduce(size_t elems, int splits, const float *partial, float *out, const float *bias = nullptr,
+                         unsigned C = 1, unsigned inner = 1)
 {
     // float4 passes: the caller only splits when elems % 4 == 0, and the partial copies start on
     // 256-byte boundaries of the workspace; `out` comes from the pool or is checked by the caller
@@ -991,7 +1003,7 @@ int launch_splitk_reduce(size_t elems, int splits, const float *partial, float *
     size_t blocks = ceil_div(n4, (size_t)256);
     size_t cap = (size_t)num_cus() * 8;
     hipLaunchKernelGGL(splitk_reduce_k, dim3((unsigned)(blocks > cap ? cap : (blocks < 1 ? 1 : blocks))), dim3(256), 0,
-                       stream(), n4, splits, (const float4 *)partial, (float4 *)out);
+                       stream(), n4, splits, (const float4 *)partial, (float4 *)out, bias, C, inner);
     DOPT_LAUNCH_CHECK();
     return DOPT_HIP_OK;
 }
@@ -1021,7 +1033,8 @@ int launch_patch(const PatchConv &pc, bool c_full, dim3 grid, size_t lds_bytes)
 // 3x3 unit-stride layers whose pixel tiles are whole rows of one image or whole images.
 // Returns DOPT_HIP_OK with *done = false when the layer does not fit this path.
 template <bool kBwd>
-int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, const float *w, float *out, bool *done)
+int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, const float *w, const float *bias,
+              float *out, bool *done)
 {
     *done = false;
     if (d->R != 3 || d->S != 3 || d->strideH != 1 || d->strideW != 1 || d->padH > 2 || d->padW > 2) return DOPT_HIP_OK;
@@ -1097,6 +1110,7 @@ int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, 
     }
     pc.in = in;
     pc.wp = wp;
+    pc.bias = bias;
     pc.in_bytes = (size_t)pc.N * pc.Cin * pc.IH * pc.IW * sizeof(float);
     pc.wp_bytes = wp_elems * sizeof(float);
     pc.out = splits > 1 ? partial : out;
@@ -1108,18 +1122,24 @@ int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, 
     else rc = launch_patch<GatherDeep, 16>(pc, c_full, grid, lds_bytes);
     if (rc) return rc;
     *done = true;
-    if (splits > 1) return launch_splitk_reduce(pc.out_elems, splits, partial, out);
+    if (splits > 1)
+        return launch_splitk_reduce(pc.out_elems, splits, partial, out, bias, (unsigned)pc.Mout, (unsigned)(pc.OH * pc.OW));
     return DOPT_HIP_OK;
 }
 
 // Shared host driver of forward (kBwd = false) and backward-data (kBwd = true).
 template <bool kBwd>
-int run_gather(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, const float *w, float *out)
+int run_gather(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, const float *w, float *out,
+               const float *bias = nullptr)
 {
     {
         bool done = false;
-        if (int rc = run_patch<kBwd>(d, P, Q, in, w, out, &done)) return rc;
+        if (int rc = run_patch<kBwd>(d, P, Q, in, w, bias, out, &done)) return rc;
         if (done) return DOPT_HIP_OK;
+    }
+    if (bias) {  // the generic kernel has no fused bias: add it in place afterwards
+        if (int rc = run_gather<kBwd>(d, P, Q, in, w, out, nullptr)) return rc;
+        return dopt_hip_bias_fwd(d->N, kBwd ? d->C : d->K, kBwd ? d->H * d->W : P * Q, out, bias, out);
     }
     GatherConv g{};
     const int taps = (int)(d->R * d->S);
@@ -1316,6 +1336,15 @@ int dopt_hip_conv_fwd(const dopt_hip_conv_desc *d, const float *x, const float *
     DOPT_REQUIRE(x && w && y, "dopt_hip_conv_fwd: null argument");
     DOPT_ENSURE_INIT();
     return run_gather<false>(d, P, Q, x, w, y);
+}
+
+int dopt_hip_conv_fwd_bias(const dopt_hip_conv_desc *d, const float *x, const float *w, const float *bias, float *y)
+{
+    size_t P, Q;
+    if (int rc = check_desc(d, &P, &Q, "dopt_hip_conv_fwd_bias")) return rc;
+    DOPT_REQUIRE(x && w && bias && y, "dopt_hip_conv_fwd_bias: null argument");
+    DOPT_ENSURE_INIT();
+    return run_gather<false>(d, P, Q, x, w, y, bias);
 }
 
 int dopt_hip_conv_bwd_data(const dopt_hip_conv_desc *d, const float *dy, const float *w, float *dx)

@@ -483,6 +483,49 @@ void toposort(const Graph &g, int op, std::vector<char> &seen, std::vector<int> 
     }
 }
 
+
+// Kernels of fused pairs (see HIPPlan::create).  `id` is the later operation of the pair, whose
+// buffer receives the result.
+std::unique_ptr<HIPKernel> make_fused(const Graph &g, int id, int kind, std::string *label)
+{
+    const Operation &op = g.ops[id];
+    if (kind == 1) {  // addBias(convolution(x, w), b): inputs [x, w, b]
+        const Operation &cv = g.ops[op.deps[0]];
+        const auto *pad = sizes_attr(cv, "padding"), *stride = sizes_attr(cv, "stride");
+        const auto &x = g.ops[cv.deps[0]].shape, &w = g.ops[cv.deps[1]].shape;
+        if (!pad || !stride || !rank4(x, "convolution features") || !rank4(w, "convolution filters")) return nullptr;
+        dopt_hip_conv_desc d = conv_desc(x, w, *pad, *stride);
+        *label = "convolution+addBias";
+        return make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_conv_fwd_bias(&d, (const float *)in[0], (const float *)in[1], (const float *)in[2],
+                                          (float *)out);
+        });
+    }
+    if (kind == 2) {  // batchNormTrain whose y part is only read through relu: inputs as batchNormTrain
+        auto it = op.doubleAttrs.find("momentum");
+        if (it == op.doubleAttrs.end()) {
+            fail(DOPT_HIP_ERR_INVALID, "batchNormTrain has no 'momentum' attribute");
+            return nullptr;
+        }
+        const double momentum = it->second;
+        size_t N, C, inner;
+        nci(g.ops[op.deps[0]].shape, &N, &C, &inner);
+        *label = "batchNormTrain+relu";
+        return make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_bn_train_relu(N, C, inner, momentum, (const float *)in[0], (const float *)in[1],
+                                          (const float *)in[2], (const float *)in[3], (const float *)in[4], (float *)out);
+        });
+    }
+    // batchNormGrad(reluGrad(dy, y, .), x, scale): inputs [dy, y, x, scale]
+    size_t N, C, inner;
+    nci(g.ops[op.deps[1]].shape, &N, &C, &inner);
+    *label = "reluGrad+batchNormGrad";
+    return make([=](const std::vector<const void *> &in, void *out) {
+        return dopt_hip_bn_grad_relu(N, C, inner, (const float *)in[0], (const float *)in[1], (const float *)in[2],
+                                     (const float *)in[3], (float *)out);
+    });
+}
+
 }  // namespace
 
 int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flags, std::unique_ptr<HIPPlan> *out)
@@ -532,7 +575,93 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         }
     }
 
-    // operations whose results are actually consumed (everything, unless VIEWS created dead copies)
+    // Fusion (DOPT_HIP_PLAN_FUSE): a pair of operations runs as one kernel when the value between
+    // them has no other reader.  inputsOf[id] lists the operations whose buffers feed id's kernel
+    // (its deps, unless fused); fusedKind[id] names the fused kernel.
+    std::vector<std::vector<int>> inputsOf((size_t)nops);
+    std::vector<int> fusedKind((size_t)nops, 0);  // 1 conv+bias, 2 bn+relu, 3 relugrad+bngrad
+    for (int id : p->mOps) inputsOf[id] = g.ops[id].deps;
+    if (flags & DOPT_HIP_PLAN_FUSE) {
+        auto root = [&](int id, size_t *off) {
+            size_t o = 0;
+            while (alias[id].source >= 0) {
+                o += alias[id].offset;
+                id = alias[id].source;
+            }
+            *off = o;
+            return id;
+        };
+        // readers are counted among the operations that are live after the alias rewrites
+        std::vector<char> live((size_t)nops, 0);
+        {
+            std::vector<int> work(outputs.begin(), outputs.end());
+            while (!work.empty()) {
+                int id = work.back();
+                work.pop_back();
+                if (live[id]) continue;
+                live[id] = 1;
+                if (alias[id].source >= 0) work.push_back(alias[id].source);
+                else for (int d : g.ops[id].deps) work.push_back(d);
+            }
+        }
+        struct Use { int op; int slot; size_t off; };
+        std::vector<std::vector<Use>> uses((size_t)nops);
+        for (int id : p->mOps) {
+            if (!live[id] || alias[id].source >= 0) continue;
+            const Operation &op = g.ops[id];
+            for (size_t j = 0; j < op.deps.size(); j++) {
+                size_t off;
+                const int r = root(op.deps[j], &off);
+                uses[r].push_back({id, (int)j, off});
+            }
+        }
+        // byte offsets at which plan outputs (or aliases of them) expose a buffer
+        std::vector<std::vector<size_t>> exposed((size_t)nops);
+        for (int o : outputs) {
+            size_t off;
+            const int r = root(o, &off);
+            exposed[r].push_back(off);
+        }
+        auto isOutput = [&](int id) { return !exposed[id].empty(); };
+        for (int id : p->mOps) {
+            const Operation &op = g.ops[id];
+            if (alias[id].source >= 0) continue;
+            if (op.opType == "addBias" && op.deps.size() == 2) {
+                const int c = op.deps[0];
+                if (g.ops[c].opType == "convolution" && g.ops[c].deps.size() == 2 && alias[c].source < 0 && !isOutput(c) &&
+                    uses[c].size() == 1 && g.ops[c].dtype == DOPT_HIP_F32) {
+                    fusedKind[id] = 1;
+                    inputsOf[id] = {g.ops[c].deps[0], g.ops[c].deps[1], op.deps[1]};
+                }
+            } else if (op.opType == "relu" && op.deps.size() == 1) {
+                size_t off;
+                const int b = root(op.deps[0], &off);
+                const Operation &bn = g.ops[b];
+                if (bn.opType != "batchNormTrain" || bn.deps.size() != 5 || off != 0 || fusedKind[b] ||
+                    op.volume() != g.ops[bn.deps[0]].volume())
+                    continue;
+                bool ok = true;  // the y part may only feed this relu and the x operand of reluGrad (a sign test)
+                for (size_t e : exposed[b]) ok = ok && e >= op.bytes();  // outputs may expose the statistics only
+                for (const Use &u : uses[b])
+                    if (u.off == 0 && !(u.op == id || (g.ops[u.op].opType == "reluGrad" && u.slot == 2))) ok = false;
+                if (!ok) continue;
+                fusedKind[b] = 2;
+                alias[id].source = b;  // the relu output IS the y part now
+                alias[id].offset = 0;
+            } else if (op.opType == "batchNormGrad" && op.deps.size() == 3) {
+                size_t off;
+                const int rg = root(op.deps[0], &off);
+                const Operation &rgo = g.ops[rg];
+                if (rgo.opType == "reluGrad" && rgo.deps.size() == 3 && off == 0 && alias[rg].source < 0 &&
+                    !isOutput(rg) && uses[rg].size() == 1 && rgo.volume() == g.ops[op.deps[1]].volume()) {
+                    fusedKind[id] = 3;
+                    inputsOf[id] = {rgo.deps[0], rgo.deps[1], op.deps[1], op.deps[2]};
+                }
+            }
+        }
+    }
+
+    // operations whose results are actually consumed (everything, unless rewrites created dead ones)
     std::vector<char> needed((size_t)nops, 0);
     {
         std::vector<int> work(outputs.begin(), outputs.end());
@@ -542,7 +671,7 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
             if (needed[id]) continue;
             needed[id] = 1;
             if (alias[id].source >= 0) work.push_back(alias[id].source);
-            else for (int d : g.ops[id].deps) work.push_back(d);
+            else for (int d : inputsOf[id]) work.push_back(d);
         }
     }
 
@@ -557,12 +686,18 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
             continue;
         }
         if (alias[id].source >= 0) continue;  // resolved per execution
-        auto it = kernelCtrs().find(op.opType);
-        if (it == kernelCtrs().end())
-            return fail(DOPT_HIP_ERR_UNSUPPORTED, "Could not construct a HIP kernel for operation of type '%s'",
-                        op.opType.c_str());
-        clear_error();
-        std::unique_ptr<HIPKernel> k = it->second(g, id);
+        std::unique_ptr<HIPKernel> k;
+        std::string label = op.opType;
+        if (fusedKind[id]) {
+            k = make_fused(g, id, fusedKind[id], &label);
+        } else {
+            auto it = kernelCtrs().find(op.opType);
+            if (it == kernelCtrs().end())
+                return fail(DOPT_HIP_ERR_UNSUPPORTED, "Could not construct a HIP kernel for operation of type '%s'",
+                            op.opType.c_str());
+            clear_error();
+            k = it->second(g, id);
+        }
         if (!k) {
             std::string why = dopt_hip_last_error();
             return fail(DOPT_HIP_ERR_INVALID, "Could not construct a HIP kernel for operation of type '%s': %s",
@@ -575,10 +710,12 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         p->mResults[id] = buf;
         Step s;
         s.op = id;
+        s.label = label;
+        s.inputOps = inputsOf[id];
         s.kernel = std::move(k);
-        s.inputs.resize(op.deps.size());
-        s.inputBytes.resize(op.deps.size());
-        for (size_t i = 0; i < op.deps.size(); i++) s.inputBytes[i] = g.ops[op.deps[i]].bytes();
+        s.inputs.resize(s.inputOps.size());
+        s.inputBytes.resize(s.inputOps.size());
+        for (size_t i = 0; i < s.inputOps.size(); i++) s.inputBytes[i] = g.ops[s.inputOps[i]].bytes();
         p->mSteps.push_back(std::move(s));
     }
     // remember aliases for the per-execution resolve pass
@@ -648,10 +785,8 @@ int HIPPlan::resolve(int nargs, const int *argOps, const void *const *argPtrs, c
     for (int id : mOps)
         if (mNeeded[id] && mAliasSource[id] >= 0)
             mResults[id] = (char *)mResults[mAliasSource[id]] + mAliasOffset[id];
-    for (Step &s : mSteps) {
-        const Operation &op = g.ops[s.op];
-        for (size_t i = 0; i < op.deps.size(); i++) s.inputs[i] = mResults[op.deps[i]];
-    }
+    for (Step &s : mSteps)
+        for (size_t i = 0; i < s.inputOps.size(); i++) s.inputs[i] = mResults[s.inputOps[i]];
     return DOPT_HIP_OK;
 }
 
@@ -673,7 +808,7 @@ int HIPPlan::execute(int nargs, const int *argOps, const void *const *argPtrs, c
         for (size_t i = 0; i < mSteps.size(); i++) {
             float ms = 0.0f;
             DOPT_HIP_CHECK(hipEventElapsedTime(&ms, mEvents[i].first, mEvents[i].second));
-            auto &slot = profiler[mGraph->ops[mSteps[i].op].opType];
+            auto &slot = profiler[mSteps[i].label];
             slot.first += (double)ms * 1000.0;
             slot.second += 1;
         }

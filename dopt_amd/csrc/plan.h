@@ -90,6 +90,8 @@ private:
     HIPPlan() = default;
     struct Step {
         int op;
+        std::string label;                       // profiler key: the opType, or "a+b" for a fused pair
+        std::vector<int> inputOps;               // operations whose buffers are the kernel's inputs
         std::unique_ptr<HIPKernel> kernel;
         std::vector<const void *> inputs;
         std::vector<size_t> inputBytes;

@@ -203,6 +203,14 @@ def convolution(x, w, padding=(0, 0), stride=(1, 1), out=None):
     return y
 
 
+def convolution_bias(x, w, bias, padding=(0, 0), stride=(1, 1), out=None):
+    """addBias(convolution(x, w), bias) in one pass."""
+    d = conv_desc(x.shape, w.shape, padding, stride)
+    y = _out(out, conv_out_shape(d))
+    capi.check(capi.load().dopt_hip_conv_fwd_bias(C.byref(d), x.ptr, w.ptr, bias.ptr, y.ptr))
+    return y
+
+
 def conv_bwd_data(dy, w, xshape, padding=(0, 0), stride=(1, 1), out=None):
     d = conv_desc(xshape, w.shape, padding, stride)
     if tuple(dy.shape) != conv_out_shape(d):
@@ -283,6 +291,23 @@ def bn_train(x, scale, bias, run_mean, run_var, momentum, out=None):
     packed = _out(out, (x.size + 2 * Cc,))
     capi.check(capi.load().dopt_hip_bn_train(N, Cc, inner, float(momentum), x.ptr, scale.ptr, bias.ptr, run_mean.ptr,
                                              run_var.ptr, packed.ptr))
+    return packed
+
+
+def bn_train_relu(x, scale, bias, run_mean, run_var, momentum, out=None):
+    """batchNormTrain whose y part already went through relu."""
+    N, Cc, inner = _nci(x.shape)
+    packed = _out(out, (x.size + 2 * Cc,))
+    capi.check(capi.load().dopt_hip_bn_train_relu(N, Cc, inner, float(momentum), x.ptr, scale.ptr, bias.ptr,
+                                                  run_mean.ptr, run_var.ptr, packed.ptr))
+    return packed
+
+
+def bn_grad_relu(dy, y, x, scale, out=None):
+    """batchNormGrad(reluGrad(dy, y, .), x, scale): y is the relu output."""
+    N, Cc, inner = _nci(x.shape)
+    packed = _out(out, (x.size + 2 * Cc,))
+    capi.check(capi.load().dopt_hip_bn_grad_relu(N, Cc, inner, dy.ptr, y.ptr, x.ptr, scale.ptr, packed.ptr))
     return packed
 
 

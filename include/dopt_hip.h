@@ -140,6 +140,11 @@ typedef struct {
 /* `convolution`: cudnnConvolutionForward at cudnn7.d:154, CUDNN_CONVOLUTION mode (:87): a TRUE
    convolution, y[n,k,p,q] = sum x[n,c,p*sy-ph+r,q*sx-pw+s] * w[k,c,R-1-r,S-1-s]. */
 int dopt_hip_conv_fwd(const dopt_hip_conv_desc *d, const float *x, const float *w, float *y);
+/* `addBias(convolution(x, w), bias)` in one pass: the two reference kernels (cudnn7.d:154 then
+   cudnnAddTensor at cudnn7.d:507) with the bias added where the sums are finished.  Same
+   values as the two calls; used by plans compiled with DOPT_HIP_PLAN_FUSE. */
+int dopt_hip_conv_fwd_bias(const dopt_hip_conv_desc *d, const float *x, const float *w,
+                           const float *bias, float *y);
 /* `convolutionFeaturesGrad` (also convolutionTranspose): cudnnConvolutionBackwardData, cudnn7.d:199. */
 int dopt_hip_conv_bwd_data(const dopt_hip_conv_desc *d, const float *dy, const float *w, float *dx);
 /* `convolutionFiltersGrad`: cudnnConvolutionBackwardFilter, cudnn7.d:244. */
@@ -185,6 +190,18 @@ int dopt_hip_bn_train(size_t N, size_t C, size_t inner, double momentum, const f
    recomputed from x as the reference does (it saves none). */
 int dopt_hip_bn_grad(size_t N, size_t C, size_t inner, const float *dy, const float *x,
                      const float *scale, float *packed);
+/* Fused forms used by plans compiled with DOPT_HIP_PLAN_FUSE; each gives the values of the two
+   reference kernels it stands for.
+   bn_train_relu: `relu(batchNormTrain(...).y)`: cudnn7.d:608-610 then cudnnActivationForward
+   (cudnn7.d:433); the y part of `packed` holds the ReLU output.
+   bn_grad_relu: `batchNormGrad(reluGrad(dy, y, .), x, scale)`: cudnnActivationBackward
+   (cudnn7.d:471) then cudnn7.d:632-634; dy is dropped where the ReLU output y is not
+   positive. */
+int dopt_hip_bn_train_relu(size_t N, size_t C, size_t inner, double momentum, const float *x,
+                           const float *scale, const float *bias, const float *run_mean,
+                           const float *run_var, float *packed);
+int dopt_hip_bn_grad_relu(size_t N, size_t C, size_t inner, const float *dy, const float *y,
+                          const float *x, const float *scale, float *packed);
 /* `batchNormInference`: cudnnBatchNormalizationForwardInference, cudnn7.d:650-652; eps = 1e-5. */
 int dopt_hip_bn_infer(size_t N, size_t C, size_t inner, const float *x, const float *scale,
                       const float *bias, const float *mean, const float *var, float *y);

@@ -71,7 +71,10 @@ enum {
     /* Result-preserving rewrites applied when the plan is constructed: */
     DOPT_HIP_PLAN_VIEWS = 1,  /* contiguous slices alias their input; slice(pad(x)) that undoes the
                                  pad aliases x; operations left without a consumer are dropped */
-    DOPT_HIP_PLAN_TIMING = 2  /* bracket every kernel with HIP events (CUDAPlan.profiler) */
+    DOPT_HIP_PLAN_TIMING = 2, /* bracket every kernel with HIP events (CUDAPlan.profiler) */
+    DOPT_HIP_PLAN_FUSE = 4    /* with VIEWS: run adjacent operations as one kernel where the middle value
+                                 has no other reader -- addBias(convolution), relu(batchNormTrain.y) and
+                                 batchNormGrad(reluGrad) -- with the values of the separate kernels */
 };
 
 /* new CUDAPlan(outputs) (cuda/package.d:267-312): topological sort, one kernel object per

@@ -261,3 +261,54 @@ def test_config1_softmax_regression_step_matches_the_oracle():
     assert_close(b.value, -0.1 * dlin.sum(axis=0), "b after one step", scale=0.01)
     loss1, _ = up({feats: X, labels: Y})
     assert loss1 < loss0
+
+
+# ----------------------------------------------------------------------------- fused kernels
+def test_fused_entry_points_equal_the_separate_kernels():
+    r = np.random.default_rng(80)
+    for shape, wshape in [((4, 16, 8, 8), (40, 16, 3, 3)), ((2, 8, 32, 32), (16, 8, 3, 3)), ((3, 6, 5, 7), (4, 6, 3, 3)),
+                          ((64, 32, 2, 2), (48, 32, 3, 3))]:
+        x = ops.tensor(r.standard_normal(shape).astype(np.float32))
+        w = ops.tensor(r.standard_normal(wshape).astype(np.float32))
+        b = ops.tensor(r.standard_normal(wshape[0]).astype(np.float32))
+        want = ops.add_bias(ops.convolution(x, w, (1, 1)), b).numpy()
+        got = ops.convolution_bias(x, w, b, (1, 1)).numpy()
+        assert np.array_equal(got, want), shape
+    for shape in [(8, 6, 4, 4), (40, 4, 32, 32), (16, 5, 3, 3), (128, 32, 2, 2)]:
+        c = shape[1]
+        x = ops.tensor((r.standard_normal(shape) + 0.5).astype(np.float32))
+        g, bb, rm = (ops.tensor(r.standard_normal(c).astype(np.float32)) for _ in range(3))
+        rv = ops.tensor((r.random(c) + 0.5).astype(np.float32))
+        dy = ops.tensor(r.standard_normal(shape).astype(np.float32))
+        n = x.size
+        plain = ops.bn_train(x, g, bb, rm, rv, 0.9)
+        y = ops.relu(plain.view(0, shape))
+        fused = ops.bn_train_relu(x, g, bb, rm, rv, 0.9)
+        assert np.array_equal(fused.numpy()[:n], y.numpy().reshape(-1)), shape
+        assert np.array_equal(fused.numpy()[n:], plain.numpy()[n:]), shape
+        want = ops.bn_grad(ops.relu_grad(dy, plain.view(0, shape)), x, g).numpy()
+        got = ops.bn_grad_relu(dy, y, x, g).numpy()
+        assert np.array_equal(got, want), shape
+
+
+def test_plan_fusion_does_not_change_results():
+    r = np.random.default_rng(81)
+    X = r.standard_normal((8, 3, 8, 8)).astype(np.float32)
+    Y = np.zeros((8, 10), np.float32)
+    Y[np.arange(8), r.integers(0, 10, 8)] = 1
+    results, kernels = [], []
+    for flags in (0, core.PLAN_VIEWS, core.PLAN_VIEWS | core.PLAN_FUSE):
+        feats, labels = float32([8, 3, 8, 8]), float32([8, 10])
+        init = nnet.Init(82)
+        body = nnet.vgg(feats, [16, 16, -1, 32, -1], [24], init)
+        preds = nnet.softmax(nnet.dense(body, 10, init))
+        net = nnet.DAGNetwork([feats], [preds])
+        loss = nnet.crossEntropy(preds.trainOutput, labels) + net.paramLoss
+        grads = core.grad(loss, net.params)
+        plan = core.compile([loss, preds.trainOutput] + grads + [net.paramProj[p](p) for p in net.paramProj], flags)
+        results.append(plan.execute({feats: X, labels: Y}))
+        kernels.append(plan.stats()["kernels"])
+    for a, b, c in zip(*results):
+        assert np.array_equal(a, b) and np.array_equal(a, c)
+    # three conv blocks: each loses addBias, relu and reluGrad as separate kernels
+    assert kernels[2] == kernels[1] - 9, kernels
