@@ -633,6 +633,49 @@ __global__ __launch_bounds__(256) void wgrad_reduce_k(int K, int C, int Cp, int 
     for (int i = threadIdx.x; i < nelem; i += 256) dst[i] = stage[i];
 }
 
+// out[i] = sum over s of partial[s * stride + i], in a fixed order: split lane sl of a block folds
+// the splits s = sl, sl + SL, ... (four independent chains, then ((a0+a1)+(a2+a3))), and the SL
+// lane sums are added in lane order.  256 threads = (256 / SL) float4 columns x SL split lanes; SL
+// is chosen by the host so that small outputs with hundreds of splits still fill the machine.
+template <int SL>
+__global__ __launch_bounds__(256) void split_sum_k(size_t n4, int splits, size_t stride4, const float4 *partial,
+                                                    float4 *out)
+{
+    constexpr int EL = 256 / SL;
+    __shared__ float4 part[SL][EL];
+    const int el = threadIdx.x % EL, sl = threadIdx.x / EL;
+    const size_t i = (size_t)blockIdx.x * EL + el;
+    float4 a0 = make_float4(0.f, 0.f, 0.f, 0.f), a1 = a0, a2 = a0, a3 = a0;
+    if (i < n4) {
+        const float4 *q = partial + i;
+        int sp = sl;
+        for (; sp + 3 * SL < splits; sp += 4 * SL) {
+            const float4 v0 = q[(size_t)sp * stride4], v1 = q[(size_t)(sp + SL) * stride4];
+            const float4 v2 = q[(size_t)(sp + 2 * SL) * stride4], v3 = q[(size_t)(sp + 3 * SL) * stride4];
+            a0.x += v0.x; a0.y += v0.y; a0.z += v0.z; a0.w += v0.w;
+            a1.x += v1.x; a1.y += v1.y; a1.z += v1.z; a1.w += v1.w;
+            a2.x += v2.x; a2.y += v2.y; a2.z += v2.z; a2.w += v2.w;
+            a3.x += v3.x; a3.y += v3.y; a3.z += v3.z; a3.w += v3.w;
+        }
+        for (; sp < splits; sp += SL) {
+            const float4 v0 = q[(size_t)sp * stride4];
+            a0.x += v0.x; a0.y += v0.y; a0.z += v0.z; a0.w += v0.w;
+        }
+    }
+    part[sl][el] = make_float4((a0.x + a1.x) + (a2.x + a3.x), (a0.y + a1.y) + (a2.y + a3.y),
+                               (a0.z + a1.z) + (a2.z + a3.z), (a0.w + a1.w) + (a2.w + a3.w));
+    __syncthreads();
+    if (sl == 0 && i < n4) {
+        float4 r = part[0][el];
+#pragma unroll
+        for (int k = 1; k < SL; k++) {
+            const float4 v = part[k][el];
+            r.x += v.x; r.y += v.y; r.z += v.z; r.w += v.w;
+        }
+        out[i] = r;
+    }
+}
+
 // ------------------------------------------------------------------------------------ backward-filter, 3x3 patch
 //
 // Filter gradient of 3x3, unit-stride, pad-1 convolutions:
@@ -660,15 +703,15 @@ __global__ __launch_bounds__(256) void wgrad_reduce_k(int K, int C, int Cp, int 
 struct WgradPatch {
     const float *dy;  // [N, K, H, W]
     const float *x;   // [N, C, H, W]
-    float *out;       // `splits` partial copies of [K][9 * Cp] (tap-major columns)
+    float *out;       // dw [K][C][3][3], or `splits` partial copies of it `split_stride` floats apart
+    size_t split_stride;
     int N, C, K, H, W;
     int G, bands;         // geometry 0: output rows per chunk (G*W = 64), chunks per image; else 1
     int imgs;             // images per chunk (1, 4 or 16)
     int ppitch, cstride;  // patch row pitch; floats per channel (128-bit reads by 32 channels hit every bank once)
     int quads_row;        // W / 4 (geometry 0)
-    int Cp, ncols;
     int mtiles, ctiles, chunks_total, chunks_per_split, splits;
-    size_t out_elems, dy_bytes, x_bytes;
+    size_t dy_bytes, x_bytes;
 };
 
 template <int WM, int WC, int kGeo>
@@ -884,19 +927,31 @@ __global__ __launch_bounds__(768, 1) void conv_wgrad_patch_k(WgradPatch p)
         cur ^= 1;
     }
 
-    // partial[k][t * Cp + c] with t = (2 - dr) * 3 + (2 - ds)
-    float *outp = p.out + (size_t)split * p.out_elems;
-    const int c = c0 + wc * 32 + l32;
-    if (c < p.C) {
+    // Epilogue: the accumulators leave through LDS so that every output row -- the BC*9 values
+    // [c][tap] of one k, contiguous in dw's own layout -- is written as one run.  One group of 32
+    // rows (the wavefronts with the same wm) is staged per pass.  out = dw itself when there is one
+    // split, else this split's partial copy (same layout, summed afterwards in split order).
+    __syncthreads();  // all fragment reads of the last chunk are done: LDS is free
+    constexpr int RP = BC * 9 + 1;  // staging row pitch (odd: the 4-row stride between lane halves spreads over banks)
+    float *outp = p.out + (size_t)split * p.split_stride;
+    const int ncv = min(BC, p.C - c0) * 9;  // valid floats of a staged row
+    for (int g = 0; g < WM; g++) {
+        if (wm == g) {
 #pragma unroll
-        for (int ds = 0; ds < 3; ds++) {
-            const int t = (2 - dr) * 3 + (2 - ds);
+            for (int ds = 0; ds < 3; ds++) {
+                const int t = (2 - dr) * 3 + (2 - ds);
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int k = k0 + wm * 32 + acc_row(v, lane);
-                if (k < p.K) outp[(size_t)k * p.ncols + t * p.Cp + c] = acc[ds][v];
+                for (int v = 0; v < 16; v++) lds[acc_row(v, lane) * RP + (wc * 32 + l32) * 9 + t] = acc[ds][v];
             }
         }
+        __syncthreads();
+        for (int r = w; r < 32; r += 12) {  // one wavefront per row
+            const int k = k0 + g * 32 + r;
+            if (k >= p.K) continue;
+            float *dst = outp + ((size_t)k * p.C + c0) * 9;
+            for (int j = lane; j < ncv; j += 64) dst[j] = lds[r * RP + j];
+        }
+        __syncthreads();
     }
 }
 
@@ -1289,26 +1344,31 @@ int run_wgrad_patch(const dopt_hip_conv_desc *d, const float *dy, const float *x
     wp.dy = dy; wp.x = x;
     wp.N = (int)d->N; wp.C = (int)d->C; wp.K = (int)d->K; wp.H = H; wp.W = W;
     wp.quads_row = W / 4;
-    wp.Cp = round_up(wp.C, 16);
-    wp.ncols = 9 * wp.Cp;
     wp.mtiles = (wp.K + BM - 1) / BM;
     wp.ctiles = (wp.C + BC - 1) / BC;
-    wp.out_elems = (size_t)wp.K * wp.ncols;
     wp.dy_bytes = (size_t)wp.N * wp.K * H * W * sizeof(float);
     wp.x_bytes = (size_t)wp.N * wp.C * H * W * sizeof(float);
+    const size_t out_elems = (size_t)wp.K * wp.C * 9;
     const int tiles = wp.mtiles * wp.ctiles;
     int splits = (num_cus() + tiles - 1) / tiles;
     const int max_by_depth = wp.chunks_total / 2 > 0 ? wp.chunks_total / 2 : 1;  // two chunks amortise the set-up
     if (splits > max_by_depth) splits = max_by_depth;
     if (splits > 512) splits = 512;
+    if (out_elems % 4 != 0 || !aligned16(dw)) splits = 1;  // the split sum works on float4
     wp.chunks_per_split = (wp.chunks_total + splits - 1) / splits;
     splits = (wp.chunks_total + wp.chunks_per_split - 1) / wp.chunks_per_split;
     wp.splits = splits;
-    const size_t lds_bytes = ((size_t)2 * BM * 68 + (size_t)2 * BC * wp.cstride + 4) * sizeof(float);
+    const size_t lds_main = ((size_t)2 * BM * 68 + (size_t)2 * BC * wp.cstride + 4) * sizeof(float);
+    const size_t lds_epi = (size_t)32 * (BC * 9 + 1) * sizeof(float);
+    const size_t lds_bytes = lds_main > lds_epi ? lds_main : lds_epi;
     if (lds_bytes > 160 * 1024) return DOPT_HIP_OK;
-    float *partial = (float *)workspace((size_t)splits * wp.out_elems * sizeof(float));
-    if (!partial) return DOPT_HIP_ERR_OOM;
-    wp.out = partial;
+    float *partial = nullptr;
+    if (splits > 1) {
+        partial = (float *)workspace((size_t)splits * out_elems * sizeof(float));
+        if (!partial) return DOPT_HIP_ERR_OOM;
+    }
+    wp.out = splits > 1 ? partial : dw;
+    wp.split_stride = out_elems;
     const dim3 grid(xcd_grid((unsigned)(tiles * splits)));
     int rc;
     if (tall) rc = geo == 0 ? launch_wgrad_patch<4, 1, 0>(wp, grid, lds_bytes)
@@ -1319,7 +1379,18 @@ int run_wgrad_patch(const dopt_hip_conv_desc *d, const float *dy, const float *x
                        : launch_wgrad_patch<2, 2, 2>(wp, grid, lds_bytes);
     if (rc) return rc;
     *done = true;
-    return launch_wgrad_reduce(wp.K, wp.C, wp.Cp, 9, splits, wp.out_elems, partial, dw);
+    if (splits > 1) {
+        // enough blocks for small filters with hundreds of splits: more split lanes per block
+        const size_t n4 = out_elems / 4;
+        if (n4 >= (size_t)64 * 512)
+            hipLaunchKernelGGL(split_sum_k<4>, dim3((unsigned)ceil_div(n4, (size_t)64)), dim3(256), 0, stream(), n4, splits,
+                               n4, (const float4 *)partial, (float4 *)dw);
+        else
+            hipLaunchKernelGGL(split_sum_k<16>, dim3((unsigned)ceil_div(n4, (size_t)16)), dim3(256), 0, stream(), n4, splits,
+                               n4, (const float4 *)partial, (float4 *)dw);
+        DOPT_LAUNCH_CHECK();
+    }
+    return DOPT_HIP_OK;
 }
 
 using WgradSquare = Tile<128, 128, 2, 2>;
