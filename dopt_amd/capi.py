@@ -75,6 +75,7 @@ PROTOTYPES = {
     "dopt_hip_bn_train_relu": [_sz, _sz, _sz, _d, _vp, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_bn_grad": [_sz, _sz, _sz, _vp, _vp, _vp, _vp],
     "dopt_hip_bn_grad_relu": [_sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp],
+    "dopt_hip_bn_grad_fused": [_sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_bn_infer": [_sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_optim_create": [_i, C.POINTER(TensorRef), C.POINTER(_vp)],
     "dopt_hip_optim_destroy": [_vp],

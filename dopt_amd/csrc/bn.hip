@@ -343,7 +343,8 @@ template <bool kGrad>
 __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, unsigned inner4, double factor, double eps,
                                                        const float *x, const float *dy, const float *scale,
                                                        const float *bias, const float *run_mean, const float *run_var,
-                                                       const float *ymask, int relu, float *out, float *out1, float *out2)
+                                                       const float *ymask, int relu, float *out, float *out1, float *out2,
+                                                       float *dx_sum)
 {
     __shared__ double part[3][16];
     __shared__ double total[3];
@@ -426,15 +427,23 @@ __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, un
         k.a = (float)((double)scale[c] * rstd);
         k.b = (float)(db / m);
         k.d = (float)(ds / m);
+        float sdx = 0.f;
 #pragma unroll
         for (int i = 0; i < kResQuads; i++) {
             if (idx[i] == 0xffffffffu) continue;
-            o4[idx[i]] = make_float4(bn_dx(k, gv[i].x, xv[i].x), bn_dx(k, gv[i].y, xv[i].y), bn_dx(k, gv[i].z, xv[i].z),
-                                     bn_dx(k, gv[i].w, xv[i].w));
+            const float4 r = make_float4(bn_dx(k, gv[i].x, xv[i].x), bn_dx(k, gv[i].y, xv[i].y),
+                                         bn_dx(k, gv[i].z, xv[i].z), bn_dx(k, gv[i].w, xv[i].w));
+            o4[idx[i]] = r;
+            sdx += (r.x + r.y) + (r.z + r.w);
         }
         if (threadIdx.x == 0) {
             out1[c] = (float)ds;
             out2[c] = (float)db;
+        }
+        if (dx_sum) {  // the per-channel sum of dx: the bias gradient of an addBias feeding this batch norm
+            double red[1] = {(double)sdx};
+            block_allsum_d<1>(red, part, total);
+            if (threadIdx.x == 0) dx_sum[c] = (float)red[0];
         }
     }
 }
@@ -520,7 +529,7 @@ int bn_train_impl(size_t N, size_t C, size_t inner, double momentum, const float
     if (unsigned T = resident_threads(N, C, inner, x, nullptr, packed)) {
         hipLaunchKernelGGL(bn_resident_k<false>, dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N, (unsigned)C,
                            (unsigned)(inner / 4), factor, eps, x, (const float *)nullptr, scale, bias, run_mean, run_var,
-                           (const float *)nullptr, relu, packed, packed + total, packed + total + C);
+                           (const float *)nullptr, relu, packed, packed + total, packed + total + C, (float *)nullptr);
         DOPT_LAUNCH_CHECK();
         return DOPT_HIP_OK;
     }
@@ -540,7 +549,7 @@ int bn_train_impl(size_t N, size_t C, size_t inner, double momentum, const float
 }
 
 int bn_grad_impl(size_t N, size_t C, size_t inner, const float *dy, const float *ymask, const float *x,
-                 const float *scale, float *packed, const char *who)
+                 const float *scale, float *packed, float *dx_sum, const char *who)
 {
     size_t total = N * C * inner;
     DOPT_REQUIRE(total > 0, "%s: empty input", who);
@@ -553,7 +562,7 @@ int bn_grad_impl(size_t N, size_t C, size_t inner, const float *dy, const float 
             hipLaunchKernelGGL(bn_resident_k<true>, dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N, (unsigned)C,
                                (unsigned)(inner / 4), 0.0, eps, x, dy, scale, (const float *)nullptr,
                                (const float *)nullptr, (const float *)nullptr, ymask, 0, packed, packed + total,
-                               packed + total + C);
+                               packed + total + C, dx_sum);
             DOPT_LAUNCH_CHECK();
             return DOPT_HIP_OK;
         }
@@ -587,6 +596,7 @@ int bn_grad_impl(size_t N, size_t C, size_t inner, const float *dy, const float 
                                dy, ymask, x, coef, packed);
     }
     DOPT_LAUNCH_CHECK();
+    if (dx_sum) return dopt_hip_bias_bwd(N, C, inner, packed, dx_sum);  // large channels: a pass of its own
     return DOPT_HIP_OK;
 }
 
@@ -609,14 +619,20 @@ int dopt_hip_bn_train_relu(size_t N, size_t C, size_t inner, double momentum, co
 int dopt_hip_bn_grad(size_t N, size_t C, size_t inner, const float *dy, const float *x, const float *scale,
                      float *packed)
 {
-    return bn_grad_impl(N, C, inner, dy, nullptr, x, scale, packed, "dopt_hip_bn_grad");
+    return bn_grad_impl(N, C, inner, dy, nullptr, x, scale, packed, nullptr, "dopt_hip_bn_grad");
 }
 
 int dopt_hip_bn_grad_relu(size_t N, size_t C, size_t inner, const float *dy, const float *y, const float *x,
                           const float *scale, float *packed)
 {
     DOPT_REQUIRE(y != nullptr, "dopt_hip_bn_grad_relu: null argument");
-    return bn_grad_impl(N, C, inner, dy, y, x, scale, packed, "dopt_hip_bn_grad_relu");
+    return bn_grad_impl(N, C, inner, dy, y, x, scale, packed, nullptr, "dopt_hip_bn_grad_relu");
+}
+
+int dopt_hip_bn_grad_fused(size_t N, size_t C, size_t inner, const float *dy, const float *y, const float *x,
+                           const float *scale, float *packed, float *dx_sum)
+{
+    return bn_grad_impl(N, C, inner, dy, y, x, scale, packed, dx_sum, "dopt_hip_bn_grad_fused");
 }
 
 int dopt_hip_bn_infer(size_t N, size_t C, size_t inner, const float *x, const float *scale, const float *bias,

@@ -486,7 +486,7 @@ void toposort(const Graph &g, int op, std::vector<char> &seen, std::vector<int> 
 
 // Kernels of fused pairs (see HIPPlan::create).  `id` is the later operation of the pair, whose
 // buffer receives the result.
-std::unique_ptr<HIPKernel> make_fused(const Graph &g, int id, int kind, std::string *label)
+std::unique_ptr<HIPKernel> make_fused(const Graph &g, int id, int kind, void *extra, std::string *label)
 {
     const Operation &op = g.ops[id];
     if (kind == 1) {  // addBias(convolution(x, w), b): inputs [x, w, b]
@@ -516,13 +516,16 @@ std::unique_ptr<HIPKernel> make_fused(const Graph &g, int id, int kind, std::str
                                           (const float *)in[2], (const float *)in[3], (const float *)in[4], (float *)out);
         });
     }
-    // batchNormGrad(reluGrad(dy, y, .), x, scale): inputs [dy, y, x, scale]
+    // batchNormGrad, with reluGrad folded in (kind 3: inputs [dy, y, x, scale]; else [dy, x, scale])
+    // and/or the bias gradient of the preceding addBias written to `extra`
     size_t N, C, inner;
     nci(g.ops[op.deps[1]].shape, &N, &C, &inner);
-    *label = "reluGrad+batchNormGrad";
+    const bool relu = kind == 3;
+    *label = std::string(relu ? "reluGrad+" : "") + "batchNormGrad" + (extra ? "+addBiasGrad" : "");
     return make([=](const std::vector<const void *> &in, void *out) {
-        return dopt_hip_bn_grad_relu(N, C, inner, (const float *)in[0], (const float *)in[1], (const float *)in[2],
-                                     (const float *)in[3], (float *)out);
+        const float *dy = (const float *)in[0], *y = relu ? (const float *)in[1] : nullptr;
+        const float *x = (const float *)in[relu ? 2 : 1], *scale = (const float *)in[relu ? 3 : 2];
+        return dopt_hip_bn_grad_fused(N, C, inner, dy, y, x, scale, (float *)out, (float *)extra);
     });
 }
 
@@ -661,6 +664,29 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         }
     }
 
+    // addBiasGrad(dx of a batchNormGrad): the batch-norm kernel writes the bias gradient too.  The
+    // addBiasGrad operation keeps its buffer but gets no kernel of its own.
+    std::vector<int> biasGradOf((size_t)nops, -1);  // batchNormGrad op -> the addBiasGrad op it serves
+    std::vector<char> absorbed((size_t)nops, 0);
+    if (flags & DOPT_HIP_PLAN_FUSE) {
+        for (int id : p->mOps) {
+            const Operation &op = g.ops[id];
+            if (op.opType != "addBiasGrad" || op.deps.size() != 1 || alias[id].source >= 0) continue;
+            size_t off = 0;
+            int r = op.deps[0];
+            while (alias[r].source >= 0) {
+                off += alias[r].offset;
+                r = alias[r].source;
+            }
+            const Operation &bg = g.ops[r];
+            if (bg.opType != "batchNormGrad" || bg.deps.size() != 3 || off != 0 || biasGradOf[r] >= 0) continue;
+            const Operation &x = g.ops[bg.deps[1]];
+            if (x.rank() < 2 || op.volume() != x.shape[1] || g.ops[op.deps[0]].volume() != x.volume()) continue;
+            biasGradOf[r] = id;
+            absorbed[id] = 1;
+        }
+    }
+
     // operations whose results are actually consumed (everything, unless rewrites created dead ones)
     std::vector<char> needed((size_t)nops, 0);
     {
@@ -675,6 +701,16 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         }
     }
 
+    // buffers first: a fused kernel may write into the buffer of a later operation
+    for (int id : p->mOps) {
+        if (!needed[id] || is_leaf(g.ops[id]) || alias[id].source >= 0) continue;
+        void *buf = nullptr;
+        if (int rc = dopt_hip_malloc(&buf, g.ops[id].bytes())) return rc;
+        if (buf) p->mOwned.push_back(buf);
+        p->mBufferBytes += g.ops[id].bytes();
+        p->mResults[id] = buf;
+    }
+
     // kernels and buffers
     for (int id : p->mOps) {
         if (!needed[id]) continue;
@@ -686,10 +722,12 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
             continue;
         }
         if (alias[id].source >= 0) continue;  // resolved per execution
+        if (absorbed[id]) continue;           // written by the batchNormGrad kernel it follows
         std::unique_ptr<HIPKernel> k;
         std::string label = op.opType;
-        if (fusedKind[id]) {
-            k = make_fused(g, id, fusedKind[id], &label);
+        void *extra = biasGradOf[id] >= 0 && needed[biasGradOf[id]] ? p->mResults[biasGradOf[id]] : nullptr;
+        if (fusedKind[id] || extra) {
+            k = make_fused(g, id, fusedKind[id], extra, &label);
         } else {
             auto it = kernelCtrs().find(op.opType);
             if (it == kernelCtrs().end())
@@ -703,11 +741,6 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
             return fail(DOPT_HIP_ERR_INVALID, "Could not construct a HIP kernel for operation of type '%s': %s",
                         op.opType.c_str(), why.empty() ? "constructor returned null" : why.c_str());
         }
-        void *buf = nullptr;
-        if (int rc = dopt_hip_malloc(&buf, op.bytes())) return rc;
-        if (buf) p->mOwned.push_back(buf);
-        p->mBufferBytes += op.bytes();
-        p->mResults[id] = buf;
         Step s;
         s.op = id;
         s.label = label;

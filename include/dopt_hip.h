@@ -202,6 +202,13 @@ int dopt_hip_bn_train_relu(size_t N, size_t C, size_t inner, double momentum, co
                            const float *run_var, float *packed);
 int dopt_hip_bn_grad_relu(size_t N, size_t C, size_t inner, const float *dy, const float *y,
                           const float *x, const float *scale, float *packed);
+/* bn_grad_fused: batchNormGrad with either neighbour folded in.  y (optional) is the ReLU output
+   as in bn_grad_relu; dx_sum (optional, C floats) receives the per-channel sum of dx, which is
+   `addBiasGrad(dx)` (cudnnConvolutionBackwardBias, cudnn7.d:539) when the batch norm's
+   input came from addBias.  dx_sum is summed in a different order than the stand-alone kernel
+   sums it (same value up to fp32 rounding). */
+int dopt_hip_bn_grad_fused(size_t N, size_t C, size_t inner, const float *dy, const float *y,
+                           const float *x, const float *scale, float *packed, float *dx_sum);
 /* `batchNormInference`: cudnnBatchNormalizationForwardInference, cudnn7.d:650-652; eps = 1e-5. */
 int dopt_hip_bn_infer(size_t N, size_t C, size_t inner, const float *x, const float *scale,
                       const float *bias, const float *mean, const float *var, float *y);

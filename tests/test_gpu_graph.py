@@ -308,7 +308,15 @@ def test_plan_fusion_does_not_change_results():
         plan = core.compile([loss, preds.trainOutput] + grads + [net.paramProj[p](p) for p in net.paramProj], flags)
         results.append(plan.execute({feats: X, labels: Y}))
         kernels.append(plan.stats()["kernels"])
+    differing = 0
     for a, b, c in zip(*results):
-        assert np.array_equal(a, b) and np.array_equal(a, c)
-    # three conv blocks: each loses addBias, relu and reluGrad as separate kernels
-    assert kernels[2] == kernels[1] - 9, kernels
+        assert np.array_equal(a, b)
+        if not np.array_equal(a, c):
+            # only the bias gradient of a convolution feeding a batch norm may differ: the fused kernel
+            # sums dx in another order.  Its exact value is 0 (a bias before a batch norm has no effect),
+            # so both are rounding noise of the dx sum.
+            assert a.ndim == 1 and np.allclose(a, c, rtol=0, atol=2e-5), (a, c)
+            differing += 1
+    assert differing <= 3
+    # three conv blocks: each loses addBias, relu, reluGrad and addBiasGrad as separate kernels
+    assert kernels[2] == kernels[1] - 12, kernels
