@@ -45,6 +45,7 @@ PROTOTYPES = {
     "dopt_hip_copy_h2d": [_vp, _vp, _sz],
     "dopt_hip_copy_d2h": [_vp, _vp, _sz],
     "dopt_hip_copy_d2d": [_vp, _vp, _sz],
+    "dopt_hip_copy_d2d_batch": [C.c_int, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_sz)],
     "dopt_hip_sync": [],
     "dopt_hip_event_create": [C.POINTER(_vp)],
     "dopt_hip_event_record": [_vp],
@@ -59,6 +60,7 @@ PROTOTYPES = {
     "dopt_hip_repeat": [_i, _szp, _szp, _vp, _vp],
     "dopt_hip_transpose2d": [_sz, _sz, _vp, _vp],
     "dopt_hip_sgemm": [_sz, _sz, _sz, _vp, _vp, _vp],
+    "dopt_hip_sgemm_t": [C.c_int, C.c_int, _sz, _sz, _sz, _vp, _vp, _vp],
     "dopt_hip_conv_fwd": [C.POINTER(ConvDesc), _vp, _vp, _vp],
     "dopt_hip_conv_fwd_bias": [C.POINTER(ConvDesc), _vp, _vp, _vp, _vp],
     "dopt_hip_conv_bwd_data": [C.POINTER(ConvDesc), _vp, _vp, _vp],

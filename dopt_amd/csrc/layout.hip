@@ -163,6 +163,22 @@ void fill_strides(NdDesc &d)
     }
 }
 
+// ---- many small device-to-device copies in one launch -----------------------------------------
+constexpr int kBatchCopies = 48;
+struct CopyBatch {  // passed by value: no table to upload
+    const void *src[kBatchCopies];
+    void *dst[kBatchCopies];
+    unsigned words[kBatchCopies];  // 4-byte words
+};
+
+__global__ __launch_bounds__(256) void copy_batch_k(CopyBatch b)
+{
+    const unsigned *s = (const unsigned *)b.src[blockIdx.x];
+    unsigned *d = (unsigned *)b.dst[blockIdx.x];
+    const unsigned n = b.words[blockIdx.x];
+    for (unsigned i = threadIdx.x; i < n; i += 256) d[i] = s[i];
+}
+
 }  // namespace
 
 extern "C" {
@@ -262,6 +278,47 @@ int dopt_hip_transpose2d(size_t rows, size_t cols, const void *in, void *out)
                        (const uint32_t *)in, (uint32_t *)out);
     DOPT_LAUNCH_CHECK();
     return DOPT_HIP_OK;
+}
+
+int dopt_hip_copy_d2d_batch(int n, void *const *dst, const void *const *src, const size_t *bytes)
+{
+    DOPT_REQUIRE(n == 0 || (dst && src && bytes), "dopt_hip_copy_d2d_batch: null argument");
+    DOPT_ENSURE_INIT();
+    CopyBatch b;
+    int filled = 0;
+    auto flush = [&]() -> int {
+        if (filled == 0) return DOPT_HIP_OK;
+        hipLaunchKernelGGL(copy_batch_k, dim3((unsigned)filled), dim3(256), 0, stream(), b);
+        DOPT_LAUNCH_CHECK();
+        filled = 0;
+        return DOPT_HIP_OK;
+    };
+    for (int i = 0; i < n; i++) {
+        if (bytes[i] == 0) continue;
+        DOPT_REQUIRE(dst[i] && src[i], "dopt_hip_copy_d2d_batch: null pointer");
+        const bool small = bytes[i] <= 65536 && bytes[i] % 4 == 0 &&
+                           (reinterpret_cast<uintptr_t>(dst[i]) & 3u) == 0 && (reinterpret_cast<uintptr_t>(src[i]) & 3u) == 0;
+        if (!small) {
+            if (int rc = dopt_hip_copy_d2d(dst[i], src[i], bytes[i])) return rc;
+            continue;
+        }
+        // copies of one launch run side by side: a copy that reads or rewrites what an earlier one
+        // of the batch writes starts a new launch
+        for (int j = 0; j < filled; j++) {
+            const char *d0 = (const char *)b.dst[j], *d1 = d0 + (size_t)b.words[j] * 4;
+            const char *s0 = (const char *)src[i], *t0 = (const char *)dst[i];
+            if ((s0 < d1 && s0 + bytes[i] > d0) || (t0 < d1 && t0 + bytes[i] > d0)) {
+                if (int rc = flush()) return rc;
+                break;
+            }
+        }
+        b.src[filled] = src[i];
+        b.dst[filled] = dst[i];
+        b.words[filled] = (unsigned)(bytes[i] / 4);
+        if (++filled == kBatchCopies)
+            if (int rc = flush()) return rc;
+    }
+    return flush();
 }
 
 }  // extern "C"

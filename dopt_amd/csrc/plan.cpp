@@ -582,7 +582,9 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
     // them has no other reader.  inputsOf[id] lists the operations whose buffers feed id's kernel
     // (its deps, unless fused); fusedKind[id] names the fused kernel.
     std::vector<std::vector<int>> inputsOf((size_t)nops);
-    std::vector<int> fusedKind((size_t)nops, 0);  // 1 conv+bias, 2 bn+relu, 3 relugrad+bngrad
+    std::vector<int> fusedKind((size_t)nops, 0);  // 1 conv+bias, 2 bn+relu, 3 relugrad+bngrad, 6 matmul with transposes
+    std::vector<std::unique_ptr<HIPKernel>> prebuilt((size_t)nops);
+    std::vector<std::string> prebuiltLabel((size_t)nops);
     for (int id : p->mOps) inputsOf[id] = g.ops[id].deps;
     if (flags & DOPT_HIP_PLAN_FUSE) {
         auto root = [&](int id, size_t *off) {
@@ -662,6 +664,64 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
                 }
             }
         }
+
+        // matmul reads a transposed operand in place instead of a copy made by `transpose`, and
+        // transpose(matmul(A, B)) is computed as matmul(B^T, A^T); the transposes left without a
+        // reader drop out.
+        auto is_swap = [&](int t) {
+            const Operation &o = g.ops[t];
+            if (o.opType != "transpose" || o.deps.size() != 1 || o.rank() != 2 || alias[t].source >= 0) return false;
+            auto it = o.sizeAttrs.find("order");
+            return it != o.sizeAttrs.end() && it->second.size() == 2 && it->second[0] == 1 && it->second[1] == 0 &&
+                   o.dtype == DOPT_HIP_F32;
+        };
+        auto through = [&](int id, bool *flip) {  // the matrix behind a chain of 2-d transposes
+            *flip = false;
+            while (is_swap(id)) {
+                id = g.ops[id].deps[0];
+                *flip = !*flip;
+            }
+            return id;
+        };
+        auto plain_matmul = [&](int m) {
+            const Operation &o = g.ops[m];
+            return o.opType == "matmul" && o.deps.size() == 2 && o.rank() == 2 && o.dtype == DOPT_HIP_F32 &&
+                   alias[m].source < 0;
+        };
+        for (int id : p->mOps) {
+            if (!live[id]) continue;
+            int mm = id;
+            bool outT = false;  // compute the transpose of the product
+            if (is_swap(id) && plain_matmul(g.ops[id].deps[0]) && uses[g.ops[id].deps[0]].size() == 1 &&
+                !isOutput(g.ops[id].deps[0])) {
+                mm = g.ops[id].deps[0];
+                outT = true;
+            } else if (!plain_matmul(id)) {
+                continue;
+            }
+            if (!outT && fusedKind[id]) continue;
+            bool tA, tB;
+            int a = through(g.ops[mm].deps[0], &tA), b = through(g.ops[mm].deps[1], &tB);
+            if (!outT && a == g.ops[mm].deps[0] && b == g.ops[mm].deps[1]) continue;  // nothing to fold
+            if (!outT && uses[mm].size() == 1 && is_swap(uses[mm][0].op) && !isOutput(mm)) continue;  // folded into its transpose
+            size_t M = g.ops[mm].shape[0], N = g.ops[mm].shape[1];
+            const Operation &ao = g.ops[g.ops[mm].deps[0]];
+            size_t K = ao.shape[1];
+            if (outT) {  // (A B)^T = B^T A^T
+                std::swap(a, b);
+                const bool na = !tB, nb = !tA;
+                tA = na;
+                tB = nb;
+                std::swap(M, N);
+            }
+            fusedKind[id] = 6;
+            inputsOf[id] = {a, b};
+            const int ta = tA, tb = tB;
+            prebuilt[id] = make([=](const std::vector<const void *> &in, void *out) {
+                return dopt_hip_sgemm_t(ta, tb, M, N, K, (const float *)in[0], (const float *)in[1], (float *)out);
+            });
+            prebuiltLabel[id] = outT ? "matmul+transpose" : "matmul";
+        }
     }
 
     // addBiasGrad(dx of a batchNormGrad): the batch-norm kernel writes the bias gradient too.  The
@@ -726,7 +786,10 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         std::unique_ptr<HIPKernel> k;
         std::string label = op.opType;
         void *extra = biasGradOf[id] >= 0 && needed[biasGradOf[id]] ? p->mResults[biasGradOf[id]] : nullptr;
-        if (fusedKind[id] || extra) {
+        if (prebuilt[id]) {
+            k = std::move(prebuilt[id]);
+            label = prebuiltLabel[id];
+        } else if (fusedKind[id] || extra) {
             k = make_fused(g, id, fusedKind[id], extra, &label);
         } else {
             auto it = kernelCtrs().find(op.opType);
@@ -846,12 +909,18 @@ int HIPPlan::execute(int nargs, const int *argOps, const void *const *argPtrs, c
             slot.second += 1;
         }
     }
+    // package.d:419-422: the outputs go to the caller's buffers
+    mRetDst.clear();
+    mRetSrc.clear();
+    mRetBytes.clear();
     for (int i = 0; i < nrets; i++) {
         if (!rets[i]) continue;
         const int o = mOutputs[(size_t)i];
-        if (int rc = dopt_hip_copy_d2d(rets[i], mResults[o], mGraph->ops[o].bytes())) return rc;  // package.d:419-422
+        mRetDst.push_back(rets[i]);
+        mRetSrc.push_back(mResults[o]);
+        mRetBytes.push_back(mGraph->ops[o].bytes());
     }
-    return DOPT_HIP_OK;
+    return dopt_hip_copy_d2d_batch((int)mRetDst.size(), mRetDst.data(), mRetSrc.data(), mRetBytes.data());
 }
 
 int HIPPlan::result(int op, void **ptr, size_t *bytes) const

@@ -110,6 +110,9 @@ private:
     std::vector<std::pair<hipEvent_t, hipEvent_t>> mEvents;
     size_t mBufferBytes = 0;
     bool mClean = false;
+    std::vector<void *> mRetDst;                 // scratch of execute(): the return copies
+    std::vector<const void *> mRetSrc;
+    std::vector<size_t> mRetBytes;
     int resolve(int nargs, const int *argOps, const void *const *argPtrs, const int *argOnHost);
 };
 

@@ -20,18 +20,91 @@ struct Gemm {
     const float *A, *B;
     float *C;  // or `splits` partial copies
     int M, N, K;
+    int lda, ldb;  // row pitch of A and B as stored
     int mtiles, ntiles, slabs_total, slabs_per_split, splits;
     size_t out_elems;
 };
 
-template <int BM, bool kVecB>
+// An operand tile is BR rows (of M or of N) by BK reduction steps, staged k-major in LDS:
+// Xs[k][r].  In memory the operand is either "k-contiguous" -- element (r, k) at X[r*ld + k],
+// which is A as given or B transposed -- or "r-contiguous" -- element (r, k) at X[k*ld + r],
+// which is B as given or A transposed.
+//   k-contiguous: 16 lanes run along k, 16 row groups; the LDS store does the transposition.
+//   r-contiguous: float4 along r, copied straight into the k-major tile.
+template <int BR>
+struct KContig {
+    static constexpr int N = BR / 16;
+    float reg[N];
+    __device__ void load(const float *X, int ld, int r_base, int r_max, int kk0, int k_max, int tid)
+    {
+        const int kl = tid & 15, r0 = tid >> 4;
+        const bool kok = kk0 + kl < k_max;
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const int r = r_base + r0 + 16 * i;
+            reg[i] = (kok && r < r_max) ? X[(size_t)r * ld + kk0 + kl] : 0.0f;
+        }
+    }
+    __device__ void store(float *Xs, int LD, int tid) const
+    {
+        const int kl = tid & 15, r0 = tid >> 4;
+#pragma unroll
+        for (int i = 0; i < N; i++) Xs[kl * LD + r0 + 16 * i] = reg[i];
+    }
+};
+
+template <int BR, bool kVec>
+struct RContig {
+    static constexpr int N = BR * BK / 4 / kGemmThreads;
+    float4 reg[N];
+    __device__ void load(const float *X, int ld, int r_base, int r_max, int kk0, int k_max, int tid)
+    {
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const int f = tid + kGemmThreads * i;
+            const int row = f / (BR / 4), gr = r_base + (f % (BR / 4)) * 4;
+            const int kk = kk0 + row;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (kk < k_max) {
+                const float *src = X + (size_t)kk * ld + gr;
+                if (kVec) {
+                    if (gr < r_max) v = *(const float4 *)src;  // r_max % 4 == 0: a float4 never straddles the edge
+                } else {
+                    if (gr + 0 < r_max) v.x = src[0];
+                    if (gr + 1 < r_max) v.y = src[1];
+                    if (gr + 2 < r_max) v.z = src[2];
+                    if (gr + 3 < r_max) v.w = src[3];
+                }
+            }
+            reg[i] = v;
+        }
+    }
+    __device__ void store(float *Xs, int LD, int tid) const
+    {
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const int f = tid + kGemmThreads * i;
+            *(float4 *)&Xs[(f / (BR / 4)) * LD + (f % (BR / 4)) * 4] = reg[i];
+        }
+    }
+};
+
+template <bool kCond, class T, class F>
+struct Pick {
+    using type = T;
+};
+template <class T, class F>
+struct Pick<false, T, F> {
+    using type = F;
+};
+
+// C = op(A) * op(B).  kTA: A is stored [K][M]; kTB: B is stored [N][K].
+template <int BM, bool kTA, bool kTB, bool kVec>
 __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_k(Gemm p)
 {
     constexpr int BN = BM == 128 ? 128 : 256, WN = BM == 128 ? 2 : 4;
     constexpr int LDA = BM + 4, LDB = BN + 4;
-    constexpr int NA = BM / 16;                     // A: lanes run along k (contiguous in memory)
-    constexpr int NB4 = BN * BK / 4 / kGemmThreads; // B: float4 along n
-    __shared__ float As[2][BK * LDA];
+    __shared__ __attribute__((aligned(16))) float As[2][BK * LDA];
     __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB];
 
     // 1-D grid over (split, tile), tile fastest: the blocks an XCD receives work on neighbouring
@@ -48,46 +121,16 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_k(Gemm p)
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int wm = w / WN, wn = w % WN;
-    const int kl = tid & 15, r0 = tid >> 4;
 
-    float areg[NA];
-    float4 breg[NB4];
+    typename Pick<kTA, RContig<BM, kVec>, KContig<BM>>::type la;
+    typename Pick<kTB, KContig<BN>, RContig<BN, kVec>>::type lb;
     auto load = [&](int slab) {
-        const int kk0 = slab * BK;
-        const bool kok = kk0 + kl < p.K;
-#pragma unroll
-        for (int i = 0; i < NA; i++) {
-            const int m = m0 + r0 + 16 * i;
-            areg[i] = (kok && m < p.M) ? p.A[(size_t)m * p.K + kk0 + kl] : 0.0f;
-        }
-#pragma unroll
-        for (int i = 0; i < NB4; i++) {
-            const int f = tid + kGemmThreads * i;
-            const int row = f / (BN / 4), gn = n0 + (f % (BN / 4)) * 4;
-            const int kk = kk0 + row;
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (kk < p.K) {
-                const float *src = p.B + (size_t)kk * p.N + gn;
-                if (kVecB) {
-                    if (gn < p.N) v = *(const float4 *)src;  // N % 4 == 0: a float4 never straddles the edge
-                } else {
-                    if (gn + 0 < p.N) v.x = src[0];
-                    if (gn + 1 < p.N) v.y = src[1];
-                    if (gn + 2 < p.N) v.z = src[2];
-                    if (gn + 3 < p.N) v.w = src[3];
-                }
-            }
-            breg[i] = v;
-        }
+        la.load(p.A, p.lda, m0, p.M, slab * BK, p.K, tid);
+        lb.load(p.B, p.ldb, n0, p.N, slab * BK, p.K, tid);
     };
     auto store = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < NA; i++) As[buf][kl * LDA + r0 + 16 * i] = areg[i];
-#pragma unroll
-        for (int i = 0; i < NB4; i++) {
-            const int f = tid + kGemmThreads * i;
-            *(float4 *)&Bs[buf][(f / (BN / 4)) * LDB + (f % (BN / 4)) * 4] = breg[i];
-        }
+        la.store(As[buf], LDA, tid);
+        lb.store(Bs[buf], LDB, tid);
     };
 
     v16f acc[2][2];
@@ -179,7 +222,9 @@ unsigned flat_grid(size_t n)
 
 extern "C" {
 
-int dopt_hip_sgemm(size_t M, size_t N, size_t K, const float *A, const float *B, float *C)
+// C[M,N] = op(A) * op(B) with op(X) = X or its transpose: transA means A is stored [K][M], transB
+// means B is stored [N][K].
+int dopt_hip_sgemm_t(int transA, int transB, size_t M, size_t N, size_t K, const float *A, const float *B, float *C)
 {
     if (M * N == 0) return DOPT_HIP_OK;
     DOPT_REQUIRE(C != nullptr, "dopt_hip_sgemm: C is null");
@@ -190,18 +235,25 @@ int dopt_hip_sgemm(size_t M, size_t N, size_t K, const float *A, const float *B,
                      M * N < ((size_t)1 << 40),
                  "dopt_hip_sgemm: dimensions too large");
 
-    if (K == 1) {
+    if (K == 1) {  // vectors: a transposed vector is the same memory
         hipLaunchKernelGGL(outer_k, dim3(flat_grid(M * N)), dim3(256), 0, stream(), M, N, A, B, C);
         DOPT_LAUNCH_CHECK();
         return DOPT_HIP_OK;
     }
-    if (N == 1) {
-        hipLaunchKernelGGL(gemv_rows_k, dim3((unsigned)ceil_div(M, (size_t)4)), dim3(256), 0, stream(), M, K, A, B, C);
+    // matrix-vector products: `rows` reads the matrix row by row (k contiguous), `cols` column-wise
+    const bool mv_rows = (N == 1 && !transA) || (M == 1 && transB);
+    const bool mv_cols = (M == 1 && !transB) || (N == 1 && transA);
+    if (mv_rows) {
+        const size_t R = N == 1 ? M : N;
+        const float *mat = N == 1 ? A : B, *vec = N == 1 ? B : A;
+        hipLaunchKernelGGL(gemv_rows_k, dim3((unsigned)ceil_div(R, (size_t)4)), dim3(256), 0, stream(), R, K, mat, vec, C);
         DOPT_LAUNCH_CHECK();
         return DOPT_HIP_OK;
     }
-    if (M == 1) {
-        size_t nblocks = ceil_div(N, (size_t)256);
+    if (mv_cols) {
+        const size_t R = M == 1 ? N : M;
+        const float *mat = M == 1 ? B : A, *vec = M == 1 ? A : B;
+        size_t nblocks = ceil_div(R, (size_t)256);
         size_t slices = ceil_div((size_t)num_cus() * 2, nblocks);
         if (slices > ceil_div(K, (size_t)32)) slices = ceil_div(K, (size_t)32);
         if (slices > 64) slices = 64;
@@ -210,14 +262,14 @@ int dopt_hip_sgemm(size_t M, size_t N, size_t K, const float *A, const float *B,
         slices = ceil_div(K, kslice);
         float *partial = C;
         if (slices > 1) {
-            partial = (float *)workspace(slices * N * sizeof(float));
+            partial = (float *)workspace(slices * R * sizeof(float));
             if (!partial) return DOPT_HIP_ERR_OOM;
         }
-        hipLaunchKernelGGL(gemv_cols_k, dim3((unsigned)nblocks, (unsigned)slices), dim3(256), 0, stream(), K, N, kslice,
-                           A, B, partial);
+        hipLaunchKernelGGL(gemv_cols_k, dim3((unsigned)nblocks, (unsigned)slices), dim3(256), 0, stream(), K, R, kslice,
+                           vec, mat, partial);
         DOPT_LAUNCH_CHECK();
         if (slices > 1) {
-            hipLaunchKernelGGL(splitk_reduce_k, dim3(flat_grid(N)), dim3(256), 0, stream(), N, (int)slices, partial, C);
+            hipLaunchKernelGGL(splitk_reduce_k, dim3(flat_grid(R)), dim3(256), 0, stream(), R, (int)slices, partial, C);
             DOPT_LAUNCH_CHECK();
         }
         return DOPT_HIP_OK;
@@ -229,6 +281,8 @@ int dopt_hip_sgemm(size_t M, size_t N, size_t K, const float *A, const float *B,
     g.M = (int)M;
     g.N = (int)N;
     g.K = (int)K;
+    g.lda = (int)(transA ? M : K);
+    g.ldb = (int)(transB ? K : N);
     g.out_elems = M * N;
     g.slabs_total = (int)ceil_div(K, (size_t)BK);
     const bool big = M > 64;
@@ -250,15 +304,25 @@ int dopt_hip_sgemm(size_t M, size_t N, size_t K, const float *A, const float *B,
         if (!partial) return DOPT_HIP_ERR_OOM;
     }
     g.C = splits > 1 ? partial : C;
-    const bool vecB = (N % 4 == 0) && aligned16(B);
+    // 128-bit loads for the operands stored with M (or N) contiguous
+    const bool vec = (!transA || (M % 4 == 0 && aligned16(A))) && (transB || (N % 4 == 0 && aligned16(B)));
     dim3 grid(xcd_grid((unsigned)(tiles * splits)));
-    if (big) {
-        if (vecB) hipLaunchKernelGGL((sgemm_k<128, true>), grid, dim3(kGemmThreads), 0, stream(), g);
-        else hipLaunchKernelGGL((sgemm_k<128, false>), grid, dim3(kGemmThreads), 0, stream(), g);
-    } else {
-        if (vecB) hipLaunchKernelGGL((sgemm_k<64, true>), grid, dim3(kGemmThreads), 0, stream(), g);
-        else hipLaunchKernelGGL((sgemm_k<64, false>), grid, dim3(kGemmThreads), 0, stream(), g);
-    }
+#define DOPT_SGEMM(BMV, TA, TB)                                                                               \
+    do {                                                                                                      \
+        if (vec) hipLaunchKernelGGL((sgemm_k<BMV, TA, TB, true>), grid, dim3(kGemmThreads), 0, stream(), g);   \
+        else hipLaunchKernelGGL((sgemm_k<BMV, TA, TB, false>), grid, dim3(kGemmThreads), 0, stream(), g);      \
+    } while (0)
+#define DOPT_SGEMM_T(BMV)                                   \
+    do {                                                    \
+        if (!transA && !transB) DOPT_SGEMM(BMV, false, false); \
+        else if (!transA) DOPT_SGEMM(BMV, false, true);     \
+        else if (!transB) DOPT_SGEMM(BMV, true, false);     \
+        else DOPT_SGEMM(BMV, true, true);                   \
+    } while (0)
+    if (big) DOPT_SGEMM_T(128);
+    else DOPT_SGEMM_T(64);
+#undef DOPT_SGEMM_T
+#undef DOPT_SGEMM
     DOPT_LAUNCH_CHECK();
     if (splits > 1) {
         hipLaunchKernelGGL(splitk_reduce_k, dim3(flat_grid(g.out_elems)), dim3(256), 0, stream(), g.out_elems, splits,
@@ -266,6 +330,11 @@ int dopt_hip_sgemm(size_t M, size_t N, size_t K, const float *A, const float *B,
         DOPT_LAUNCH_CHECK();
     }
     return DOPT_HIP_OK;
+}
+
+int dopt_hip_sgemm(size_t M, size_t N, size_t K, const float *A, const float *B, float *C)
+{
+    return dopt_hip_sgemm_t(0, 0, M, N, K, A, B, C);
 }
 
 }  // extern "C"

@@ -184,6 +184,17 @@ def matmul(a, b, out=None):
     return out
 
 
+def matmul_t(a, b, trans_a=False, trans_b=False, out=None):
+    """op(a) . op(b): trans_a / trans_b read the operand transposed (a stored [K, M], b stored [N, K])."""
+    K, M = (a.shape if trans_a else a.shape[::-1])
+    N, K2 = (b.shape if trans_b else b.shape[::-1])
+    if K != K2:
+        raise capi.HipError(1, "matmul: inner dimensions differ")
+    out = _out(out, (M, N))
+    capi.check(capi.load().dopt_hip_sgemm_t(int(trans_a), int(trans_b), M, N, K, a.ptr, b.ptr, out.ptr))
+    return out
+
+
 def conv_desc(xshape, wshape, padding=(0, 0), stride=(1, 1)):
     N, Cc, H, W = xshape
     K, C2, R, S = wshape

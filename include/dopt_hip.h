@@ -68,6 +68,10 @@ int dopt_hip_copy_h2d(void *dst, const void *host_src, size_t bytes);
 int dopt_hip_copy_d2h(void *host_dst, const void *src, size_t bytes);
 /* CUDABuffer.set(DeviceBuffer) -> cuMemcpyDtoD, cuda/package.d:187-190 */
 int dopt_hip_copy_d2d(void *dst, const void *src, size_t bytes);
+/* n device-to-device copies, in order; copies of at most 64 KiB share kernel launches.  Stands
+   for the loop of cuMemcpy calls that hands a plan's outputs to the caller's buffers
+   (cuda/package.d:419-422): most of them are a few hundred bytes of batch-norm statistics. */
+int dopt_hip_copy_d2d_batch(int n, void *const *dst, const void *const *src, const size_t *bytes);
 /* cuCtxSynchronize (cuda/nvrtc.d:111,123; cudnn7.d:157 ...) */
 int dopt_hip_sync(void);
 /* The hipStream_t every entry point enqueues on (for callers that record their own events). */
@@ -130,6 +134,12 @@ int dopt_hip_transpose2d(size_t rows, size_t cols, const void *in, void *out);
    (matrix-vector) take bandwidth-bound paths: the reference routes scalar broadcasts and
    row/column sums through matmul (core/ops/basic.d:370-381, core/ops/math.d:257-279). */
 int dopt_hip_sgemm(size_t M, size_t N, size_t K, const float *A, const float *B, float *C);
+/* The same product with either operand read transposed, as cublasSgemm's op(A)/op(B) arguments
+   allow (cuda/math.d:234-235 always passes CUBLAS_OP_N): transA != 0 means A is stored [K][M],
+   transB != 0 means B is stored [N][K].  Plans compiled with DOPT_HIP_PLAN_FUSE use it to skip
+   the `transpose` kernels that only feed a matmul. */
+int dopt_hip_sgemm_t(int transA, int transB, size_t M, size_t N, size_t K, const float *A,
+                     const float *B, float *C);
 
 typedef struct {
     size_t N, C, H, W;       /* features [N,C,H,W] */

@@ -318,5 +318,6 @@ def test_plan_fusion_does_not_change_results():
             assert a.ndim == 1 and np.allclose(a, c, rtol=0, atol=2e-5), (a, c)
             differing += 1
     assert differing <= 3
-    # three conv blocks: each loses addBias, relu, reluGrad and addBiasGrad as separate kernels
-    assert kernels[2] == kernels[1] - 12, kernels
+    # three conv blocks each lose addBias, relu, reluGrad and addBiasGrad as separate kernels, and the
+    # two dense layers lose their transposes
+    assert kernels[2] <= kernels[1] - 12 - 8, kernels

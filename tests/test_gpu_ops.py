@@ -447,3 +447,45 @@ def test_fused_adam_amsgrad_are_bit_exact(rule):
         assert np.array_equal(tv[i].numpy(), v[i]), ("v", i)
         if rule == "amsgrad":
             assert np.array_equal(tvh[i].numpy(), vh[i]), ("vhat", i)
+
+
+def test_batched_device_copies():
+    import ctypes as C
+    from dopt_amd import capi
+    lib = capi.load()
+    r = rng(90)
+    sizes = [1, 3, 64, 512, 16384, 20000, 7, 100] * 8          # more than one launch's worth; one above 64 KiB
+    src = [T(r.standard_normal(n).astype(np.float32)) for n in sizes]
+    dst = [ops.Tensor((n,)) for n in sizes]
+    n = len(sizes)
+    d = (C.c_void_p * n)(*[t.ptr for t in dst])
+    s = (C.c_void_p * n)(*[t.ptr for t in src])
+    b = (C.c_size_t * n)(*[4 * k for k in sizes])
+    capi.check(lib.dopt_hip_copy_d2d_batch(n, d, s, b))
+    for a, c in zip(src, dst):
+        assert np.array_equal(a.numpy(), c.numpy())
+    # a chain a -> b -> c inside one call keeps its order
+    a, bb, c = T(np.arange(8, dtype=np.float32)), ops.Tensor((8,)), ops.Tensor((8,))
+    d = (C.c_void_p * 2)(bb.ptr, c.ptr)
+    s = (C.c_void_p * 2)(a.ptr, bb.ptr)
+    b = (C.c_size_t * 2)(32, 32)
+    capi.check(lib.dopt_hip_copy_d2d_batch(2, d, s, b))
+    assert np.array_equal(c.numpy(), np.arange(8, dtype=np.float32))
+
+
+@pytest.mark.parametrize("shape", [(128, 512, 512), (70, 33, 129), (130, 10, 512), (1, 300, 77), (200, 1, 64), (5, 7, 1),
+                                   (256, 256, 40), (64, 260, 96)])
+@pytest.mark.parametrize("ta,tb", [(False, True), (True, False), (True, True)])
+def test_sgemm_transposed_operands(shape, ta, tb):
+    M, N, K = shape
+    r = rng(M * 7 + N * 3 + K)
+    a = r.standard_normal((M, K)).astype(np.float32)
+    b = r.standard_normal((K, N)).astype(np.float32)
+    want = O.matmul(a, b, f64=True)
+    got = ops.matmul_t(T(np.ascontiguousarray(a.T) if ta else a), T(np.ascontiguousarray(b.T) if tb else b), ta, tb)
+    assert got.shape == (M, N)
+    assert_close(got.numpy(), want, "sgemm_t", scale=np.sqrt(K))
+    # on the matrix-core path it is the product of the transposed copies to the last bit (the
+    # matrix-vector kernels sum in a different order when the matrix is read the other way)
+    if min(M, N, K) > 1:
+        assert np.array_equal(got.numpy(), ops.matmul(T(a), T(b)).numpy())
