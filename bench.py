@@ -157,10 +157,23 @@ def main():
         gather_launches = sum(per_step[k][1] for k in conv_keys)
         gather_tflops = (fwd + bwd_data) / (gather_us * 1e-6) / 1e12
         wgrad_tflops = fwd / (per_step["convolutionFiltersGrad"][0] * 1e-6) / 1e12
+        # HBM bytes per launch of the same kernel, as measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+        # (calibrated against a plain copy); the summary of those runs is kept under profiles/
+        traffic = None
+        tpath = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "conv_kernels_vgg16_b128_hbm_traffic.txt")
+        if os.path.exists(tpath):
+            for line in open(tpath):
+                if line.startswith("traffic_bytes_per_launch conv_patch_k"):
+                    traffic = int(line.split()[-1])
+        conv_bytes = 0   # algorithmic: input and output once, filter once
+        for i, (c, k, h) in enumerate(VGG_CONVS):
+            one = 4 * (BATCH * c * h * h + BATCH * k * h * h + k * c * 9)
+            conv_bytes += one * (1 if i == 0 else 2)
         result["roofline"] = {
             "kernel": "conv_patch_k (3x3 implicit-GEMM convolution forward + backward-data, incl. filter pack and split reduction)",
             "bound": "mfma", "achieved": round(gather_tflops, 2), "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(gather_tflops / MFMA_FP32_PEAK_TFLOPS, 4), "traffic": None,
+            "frac": round(gather_tflops / MFMA_FP32_PEAK_TFLOPS, 4), "traffic": traffic,
+            "algorithmic_bytes_per_launch": int(conv_bytes / gather_launches),
             "launches_per_step": int(gather_launches),
             "flops_per_launch": round((fwd + bwd_data) / gather_launches, 1),
             "avg_launch_us": round(gather_us / gather_launches, 2),
