@@ -311,6 +311,50 @@ __global__ __launch_bounds__(kBlock) void softmax_fwd_k(size_t N, size_t C, size
     }
 }
 
+// Rows of at least 64 contiguous channels (inner == 1): one wavefront per row, lanes stride along
+// the channels, maximum / sum / dot product folded with wavefront shuffles.  Sums are tree-ordered
+// here (the lane-per-row kernels sum in channel order).
+__device__ inline float wave_allsum(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+__global__ __launch_bounds__(kBlock) void softmax_rows_fwd_k(size_t N, size_t C, const float *x, float *y)
+{
+    const size_t row = (size_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+    if (row >= N) return;
+    const int lane = threadIdx.x & 63;
+    const float *px = x + row * C;
+    float *py = y + row * C;
+    float m = -FLT_MAX;
+    for (size_t c = lane; c < C; c += 64) m = dmax(m, px[c]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = dmax(m, __shfl_xor(m, off, 64));
+    float s = 0.0f;
+    for (size_t c = lane; c < C; c += 64) {
+        const float pot = expf(px[c] - m);
+        s += pot;
+        py[c] = pot;
+    }
+    s = wave_allsum(s);
+    for (size_t c = lane; c < C; c += 64) py[c] = py[c] / s;
+}
+
+__global__ __launch_bounds__(kBlock) void softmax_rows_bwd_k(size_t N, size_t C, const float *dy, const float *y,
+                                                              float *dx)
+{
+    const size_t row = (size_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+    if (row >= N) return;
+    const int lane = threadIdx.x & 63;
+    const size_t base = row * C;
+    float dot = 0.0f;
+    for (size_t c = lane; c < C; c += 64) dot += dy[base + c] * y[base + c];
+    dot = wave_allsum(dot);
+    for (size_t c = lane; c < C; c += 64) dx[base + c] = y[base + c] * (dy[base + c] - dot);
+}
+
 __global__ __launch_bounds__(kBlock) void softmax_bwd_k(size_t N, size_t C, size_t inner, const float *dy,
                                                          const float *y, float *dx)
 {
@@ -438,7 +482,11 @@ int dopt_hip_softmax_fwd(size_t N, size_t C, size_t inner, const float *x, float
     if (N * C * inner == 0) return DOPT_HIP_OK;
     DOPT_REQUIRE(x && y, "dopt_hip_softmax_fwd: null argument");
     DOPT_ENSURE_INIT();
-    hipLaunchKernelGGL(softmax_fwd_k, dim3(flat_grid(N * inner)), dim3(kBlock), 0, stream(), N, C, inner, x, y);
+    if (inner == 1 && C >= 64)
+        hipLaunchKernelGGL(softmax_rows_fwd_k, dim3((unsigned)ceil_div(N, (size_t)(kBlock / 64))), dim3(kBlock), 0, stream(),
+                           N, C, x, y);
+    else
+        hipLaunchKernelGGL(softmax_fwd_k, dim3(flat_grid(N * inner)), dim3(kBlock), 0, stream(), N, C, inner, x, y);
     DOPT_LAUNCH_CHECK();
     return DOPT_HIP_OK;
 }
@@ -448,7 +496,11 @@ int dopt_hip_softmax_bwd(size_t N, size_t C, size_t inner, const float *dy, cons
     if (N * C * inner == 0) return DOPT_HIP_OK;
     DOPT_REQUIRE(dy && y && dx, "dopt_hip_softmax_bwd: null argument");
     DOPT_ENSURE_INIT();
-    hipLaunchKernelGGL(softmax_bwd_k, dim3(flat_grid(N * inner)), dim3(kBlock), 0, stream(), N, C, inner, dy, y, dx);
+    if (inner == 1 && C >= 64)
+        hipLaunchKernelGGL(softmax_rows_bwd_k, dim3((unsigned)ceil_div(N, (size_t)(kBlock / 64))), dim3(kBlock), 0, stream(),
+                           N, C, dy, y, dx);
+    else
+        hipLaunchKernelGGL(softmax_bwd_k, dim3(flat_grid(N * inner)), dim3(kBlock), 0, stream(), N, C, inner, dy, y, dx);
     DOPT_LAUNCH_CHECK();
     return DOPT_HIP_OK;
 }

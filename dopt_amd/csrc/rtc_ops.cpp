@@ -213,7 +213,37 @@ extern "C" __global__ __launch_bounds__(BLOCK) void red_rows(const T *in, T *out
     if (threadIdx.x == 0) out[blockIdx.x] = acc;
 }
 
-// Strided lanes: thread (o, j) folds in[(o*R + r)*inner + j] over r, coalesced across j.
+// The same with 128-bit loads: R and chunk are multiples of 4 and `in` is 16-byte aligned.
+extern "C" __global__ __launch_bounds__(BLOCK) void red_rows4(const T *in, T *out, size_t R, size_t chunk,
+                                                               size_t nchunks)
+{
+    const size_t o = blockIdx.x / nchunks, c = blockIdx.x % nchunks;
+    const size_t start = c * chunk;
+    size_t end = start + chunk;
+    if (end > R) end = R;
+    const T4 *row = (const T4 *)(in + o * R);
+    const size_t q0 = start / 4, q1 = end / 4;
+    T acc0 = (T)(IDENT), acc1 = (T)(IDENT), acc2 = (T)(IDENT), acc3 = (T)(IDENT);
+    size_t i = q0 + threadIdx.x;
+    for (; i + 3 * BLOCK < q1; i += 4 * BLOCK) {
+        T4 v0 = row[i], v1 = row[i + BLOCK], v2 = row[i + 2 * BLOCK], v3 = row[i + 3 * BLOCK];
+        acc0 = combine(acc0, combine(combine(v0.x, v0.y), combine(v0.z, v0.w)));
+        acc1 = combine(acc1, combine(combine(v1.x, v1.y), combine(v1.z, v1.w)));
+        acc2 = combine(acc2, combine(combine(v2.x, v2.y), combine(v2.z, v2.w)));
+        acc3 = combine(acc3, combine(combine(v3.x, v3.y), combine(v3.z, v3.w)));
+    }
+    for (; i < q1; i += BLOCK) {
+        T4 v0 = row[i];
+        acc0 = combine(acc0, combine(combine(v0.x, v0.y), combine(v0.z, v0.w)));
+    }
+    T acc = combine(combine(acc0, acc1), combine(acc2, acc3));
+    acc = block_reduce(acc);
+    if (threadIdx.x == 0) out[blockIdx.x] = acc;
+}
+
+// Strided lanes: thread (o, j) folds in[(o*R + r)*inner + j] over r in ascending r (the order of
+// the reference's vector adds), coalesced across j.  Eight loads are in flight per lane; the
+// adds stay sequential.
 extern "C" __global__ __launch_bounds__(BLOCK) void red_cols(const T *in, T *out, size_t outer, size_t R,
                                                               size_t inner)
 {
@@ -222,7 +252,15 @@ extern "C" __global__ __launch_bounds__(BLOCK) void red_cols(const T *in, T *out
         const size_t o = idx / inner, j = idx % inner;
         const T *p = in + o * R * inner + j;
         T acc = (T)(IDENT);
-        for (size_t r = 0; r < R; r++) acc = combine(acc, p[r * inner]);
+        size_t r = 0;
+        for (; r + 8 <= R; r += 8) {
+            T v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) v[u] = p[(r + u) * inner];
+#pragma unroll
+            for (int u = 0; u < 8; u++) acc = combine(acc, v[u]);
+        }
+        for (; r < R; r++) acc = combine(acc, p[r * inner]);
         out[idx] = acc;
     }
 }
@@ -251,13 +289,43 @@ extern "C" __global__ __launch_bounds__(BLOCK) void argmin_k(const T *in, int *o
         out[idx] = bi;
     }
 }
+
+// Innermost axis (vol == 1): one wavefront per row, lanes stride along the row.  Each lane keeps
+// the first minimum of its own elements; lanes are then merged preferring the smaller value and,
+// on equal values, the smaller index -- the first minimum of the row, as the scan above finds it.
+extern "C" __global__ __launch_bounds__(BLOCK) void argmin_rows_k(const T *in, int *out, size_t rows, size_t A)
+{
+    const size_t row = (size_t)blockIdx.x * (BLOCK / 64) + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int lane = threadIdx.x & 63;
+    const T *p = in + row * A;
+    T best = (T)(TMAX);
+    int bi = 0x7fffffff;  // "never fired"
+    for (size_t i = lane; i < A; i += 64) {
+        T v = p[i];
+        if (v < best) {
+            best = v;
+            bi = (int)i;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        T ov = __shfl_down(best, off, 64);
+        int oi = __shfl_down(bi, off, 64);
+        if (ov < best || (ov == best && oi < bi)) {
+            best = ov;
+            bi = oi;
+        }
+    }
+    if (lane == 0) out[row] = bi == 0x7fffffff ? 0 : bi;
+}
 )SRC";
 
 std::string reduce_source(bool is_sum, int dtype)
 {
     std::string s;
     bool f = dtype == DOPT_HIP_F32;
-    s += f ? "typedef float T;\n" : "typedef int T;\n";
+    s += f ? "typedef float T;\ntypedef float4 T4;\n" : "typedef int T;\ntypedef int4 T4;\n";
     if (is_sum) {
         s += f ? "#define COMBINE a + b\n" : "#define COMBINE (int)((unsigned)a + (unsigned)b)\n";
         s += "#define IDENT 0\n";
@@ -296,8 +364,8 @@ int check_dtype(int dtype)
 }
 
 // One (outer, R, inner) reduction pass on the device.
-int reduce_pass(hipFunction_t rows, hipFunction_t cols, const void *in, void *out, size_t outer, size_t R,
-                size_t inner, size_t esize)
+int reduce_pass(hipFunction_t rows, hipFunction_t rows4, hipFunction_t cols, const void *in, void *out, size_t outer,
+                size_t R, size_t inner, size_t esize)
 {
     if (outer * inner == 0) return DOPT_HIP_OK;
     if (inner > 1 || R <= 64) {
@@ -314,27 +382,24 @@ int reduce_pass(hipFunction_t rows, hipFunction_t cols, const void *in, void *ou
         if (nchunks < 1) nchunks = 1;
     }
     size_t chunk = ceil_div(R, nchunks);
-    chunk = (chunk + 255) / 256 * 256;
+    chunk = (chunk + 1023) / 1024 * 1024;
     nchunks = ceil_div(R, chunk);
+    hipFunction_t first = (R % 4 == 0 && aligned16(in)) ? rows4 : rows;
     if (nchunks == 1) {
         void *args[] = {(void *)&in, (void *)&out, (void *)&R, (void *)&chunk, (void *)&nchunks};
-        return rtc_launch(rows, (unsigned)outer, 256, args);
+        return rtc_launch(first, (unsigned)outer, 256, args);
     }
-    void *partial = nullptr;
-    int rc = dopt_hip_malloc(&partial, outer * nchunks * esize);
-    if (rc) return rc;
+    // the partial results live in the process-wide scratch (one in-order stream: no reuse hazard)
+    void *partial = workspace(outer * nchunks * esize);
+    if (!partial) return DOPT_HIP_ERR_OOM;
     {
         void *args[] = {(void *)&in, (void *)&partial, (void *)&R, (void *)&chunk, (void *)&nchunks};
-        rc = rtc_launch(rows, (unsigned)(outer * nchunks), 256, args);
+        if (int rc = rtc_launch(first, (unsigned)(outer * nchunks), 256, args)) return rc;
     }
-    if (!rc) {
-        size_t one = 1, r2 = nchunks, chunk2 = (nchunks + 255) / 256 * 256;
-        const void *pin = partial;
-        void *args[] = {(void *)&pin, (void *)&out, (void *)&r2, (void *)&chunk2, (void *)&one};
-        rc = rtc_launch(rows, (unsigned)outer, 256, args);
-    }
-    dopt_hip_free(partial);  // stream-ordered: the next user of this block is enqueued after us
-    return rc;
+    size_t one = 1, r2 = nchunks, chunk2 = (nchunks + 255) / 256 * 256;
+    const void *pin = partial;
+    void *args[] = {(void *)&pin, (void *)&out, (void *)&r2, (void *)&chunk2, (void *)&one};
+    return rtc_launch(rows, (unsigned)outer, 256, args);
 }
 
 }  // namespace
@@ -387,8 +452,9 @@ int dopt_hip_reduce(const char *op, int dtype, const size_t *shape, int rank, co
     DOPT_ENSURE_INIT();
     std::string key = std::string("red:") + op + (dtype == DOPT_HIP_F32 ? ":f32" : ":i32");
     std::string src = reduce_source(is_sum, dtype);
-    hipFunction_t rows, cols;
+    hipFunction_t rows, rows4, cols;
     if (int rc = rtc_get(key + ":rows", src, "red_rows", &rows)) return rc;
+    if (int rc = rtc_get(key + ":rows4", src, "red_rows4", &rows4)) return rc;
     if (int rc = rtc_get(key + ":cols", src, "red_cols", &cols)) return rc;
 
     // Runs of adjacent reduced axes collapse into one (outer, R, inner) pass each, last run first.
@@ -417,7 +483,7 @@ int dopt_hip_reduce(const char *op, int dtype, const size_t *shape, int rank, co
             if (rc) break;
             dst = tmp;
         }
-        rc = reduce_pass(rows, cols, src_ptr, dst, outer, R, inner, 4);
+        rc = reduce_pass(rows, rows4, cols, src_ptr, dst, outer, R, inner, 4);
         if (tmp_prev) dopt_hip_free(tmp_prev);
         tmp_prev = tmp;
         src_ptr = dst;
@@ -439,6 +505,11 @@ int dopt_hip_argmin(int dtype, const size_t *shape, int rank, size_t axis, const
     DOPT_ENSURE_INIT();
     hipFunction_t fn;
     std::string key = std::string("argmin") + (dtype == DOPT_HIP_F32 ? ":f32" : ":i32");
+    if (vol == 1 && A >= 64 && A < 0x7fffffffu) {
+        if (int rc = rtc_get(key + ":rows", argmin_source(dtype), "argmin_rows_k", &fn)) return rc;
+        void *rargs[] = {(void *)&in, (void *)&out, (void *)&outer, (void *)&A};
+        return rtc_launch(fn, (unsigned)ceil_div(outer, (size_t)4), 256, rargs);
+    }
     if (int rc = rtc_get(key, argmin_source(dtype), "argmin_k", &fn)) return rc;
     unsigned grid = grid_for(256, outer * vol);
     void *args[] = {(void *)&in, (void *)&out, (void *)&outer, (void *)&A, (void *)&vol};
