@@ -1139,7 +1139,8 @@ int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, 
     pc.chunks_total = (pc.Cin + 15) / 16;
     pc.out_elems = (size_t)pc.ncols * pc.Mout;
     const int tiles = pc.mtiles * pc.ntiles;
-    int splits = (blocks_wanted + tiles - 1) / tiles;
+    // never a grid slightly above what is resident at once: a second round of blocks would run nearly empty
+    int splits = tiles >= blocks_wanted ? 1 : blocks_wanted / tiles;
     if (splits > pc.chunks_total) splits = pc.chunks_total;
     if (splits > 64) splits = 64;
     if (pc.out_elems % 4 != 0 || !aligned16(out)) splits = 1;
@@ -1350,7 +1351,8 @@ int run_wgrad_patch(const dopt_hip_conv_desc *d, const float *dy, const float *x
     wp.x_bytes = (size_t)wp.N * wp.C * H * W * sizeof(float);
     const size_t out_elems = (size_t)wp.K * wp.C * 9;
     const int tiles = wp.mtiles * wp.ctiles;
-    int splits = (num_cus() + tiles - 1) / tiles;
+    // one block per CU: never a grid slightly above the CU count (a second, nearly empty round)
+    int splits = tiles >= num_cus() ? 1 : num_cus() / tiles;
     const int max_by_depth = wp.chunks_total / 2 > 0 ? wp.chunks_total / 2 : 1;  // two chunks amortise the set-up
     if (splits > max_by_depth) splits = max_by_depth;
     if (splits > 512) splits = 512;
