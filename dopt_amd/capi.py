@@ -73,6 +73,8 @@ PROTOTYPES = {
     "dopt_hip_relu_bwd": [_sz, _vp, _vp, _vp],
     "dopt_hip_bias_fwd": [_sz, _sz, _sz, _vp, _vp, _vp],
     "dopt_hip_bias_bwd": [_sz, _sz, _sz, _vp, _vp],
+    "dopt_hip_uniform": [C.c_uint64, C.c_uint64, _sz, _vp],
+    "dopt_hip_philox_raw": [C.c_uint64, C.c_uint64, _sz, _vp],
     "dopt_hip_bn_train": [_sz, _sz, _sz, _d, _vp, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_bn_train_relu": [_sz, _sz, _sz, _d, _vp, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_bn_grad": [_sz, _sz, _sz, _vp, _vp, _vp, _vp],

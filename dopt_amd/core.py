@@ -405,6 +405,14 @@ for _n in ("variable", "constant"):
                        lambda op: op.attributes["type"])
 
 
+register_operation("uniform", lambda op: len(op.deps) == 0 and "shape" in op.attributes,    # ops/random.d:19-37
+                   lambda op: (float32_t, tuple(op.attributes["shape"])))
+
+
+def uniformSample(shape):   # ops/random.d:48-51: fresh draws from (0, 1] at every evaluation
+    return Operation("uniform", [], {"shape": [int(s) for s in shape]})
+
+
 def slice(input, start, stop):   # noqa: A001, A002
     return Operation("slice", [input], {"start": list(start), "stop": list(stop)})
 

@@ -368,6 +368,54 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_k(size_t N, size_t C, size
     }
 }
 
+// ---------------------------------------------------------------------------------- uniform
+// Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", SC'11): a
+// counter-based generator, so element i of call c depends only on (seed, c, i) -- no generator
+// state in device memory, any launch shape gives the same stream.  A 128-bit counter block
+// yields four 32-bit words; word -> float in (0, 1] as curandGenerateUniform documents its range
+// (cuda/random.d:74; the CPU kernel shifts D's [0, 1) by epsilon for the same reason,
+// cpu/random.d:24).
+__device__ inline void philox_round(uint32_t (&c)[4], uint32_t k0, uint32_t k1)
+{
+    const uint32_t lo0 = 0xD2511F53u * c[0], hi0 = __umulhi(0xD2511F53u, c[0]);
+    const uint32_t lo1 = 0xCD9E8D57u * c[2], hi1 = __umulhi(0xCD9E8D57u, c[2]);
+    const uint32_t n0 = hi1 ^ c[1] ^ k0, n2 = hi0 ^ c[3] ^ k1;
+    c[0] = n0;
+    c[1] = lo1;
+    c[2] = n2;
+    c[3] = lo0;
+}
+
+__device__ inline void philox4x32_10(uint32_t (&c)[4], uint32_t k0, uint32_t k1)
+{
+#pragma unroll
+    for (int r = 0; r < 10; r++) {
+        philox_round(c, k0, k1);
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+}
+
+__device__ inline float u01(uint32_t w) { return (float)((w >> 8) + 1u) * 5.9604644775390625e-8f; }  // (0, 1], 2^-24 steps
+
+// Block b of four outputs uses counter (b, call_lo, call_hi, 0) and key (seed_lo, seed_hi).
+__global__ __launch_bounds__(kBlock) void uniform_k(size_t n, uint64_t seed, uint64_t call, float *out, uint32_t *raw)
+{
+    const size_t nb = (n + 3) / 4;
+    for (size_t b = (size_t)blockIdx.x * kBlock + threadIdx.x; b < nb; b += (size_t)gridDim.x * kBlock) {
+        uint32_t c[4] = {(uint32_t)b, (uint32_t)call, (uint32_t)(call >> 32), (uint32_t)(b >> 32)};
+        philox4x32_10(c, (uint32_t)seed, (uint32_t)(seed >> 32));
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const size_t i = b * 4 + j;
+            if (i < n) {
+                if (raw) raw[i] = c[j];
+                else out[i] = u01(c[j]);
+            }
+        }
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -501,6 +549,28 @@ int dopt_hip_softmax_bwd(size_t N, size_t C, size_t inner, const float *dy, cons
                            N, C, dy, y, dx);
     else
         hipLaunchKernelGGL(softmax_bwd_k, dim3(flat_grid(N * inner)), dim3(kBlock), 0, stream(), N, C, inner, dy, y, dx);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_uniform(uint64_t seed, uint64_t call, size_t n, float *out)
+{
+    if (n == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(out != nullptr, "dopt_hip_uniform: null argument");
+    DOPT_ENSURE_INIT();
+    hipLaunchKernelGGL(uniform_k, dim3(flat_grid((n + 3) / 4)), dim3(kBlock), 0, stream(), n, seed, call, out,
+                       (uint32_t *)nullptr);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_philox_raw(uint64_t seed, uint64_t call, size_t n, uint32_t *out)
+{
+    if (n == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(out != nullptr, "dopt_hip_philox_raw: null argument");
+    DOPT_ENSURE_INIT();
+    hipLaunchKernelGGL(uniform_k, dim3(flat_grid((n + 3) / 4)), dim3(kBlock), 0, stream(), n, seed, call,
+                       (float *)nullptr, out);
     DOPT_LAUNCH_CHECK();
     return DOPT_HIP_OK;
 }

@@ -13,6 +13,10 @@
 //   - optional rewrites (DOPT_HIP_PLAN_VIEWS) replace copies by aliases.
 #include "plan.h"
 
+#include <atomic>
+#include <cstdlib>
+#include <random>
+
 #include <algorithm>
 #include <cstring>
 #include <functional>
@@ -409,6 +413,28 @@ void registerBuiltinsOnce()
         return make([=](const std::vector<const void *> &in, void *out) {
             return dopt_hip_bn_infer(N, C, inner, (const float *)in[0], (const float *)in[1], (const float *)in[2],
                                      (const float *)in[3], (const float *)in[4], (float *)out);
+        });
+    };
+
+    // cuda/random.d:47-83: a generator per kernel object, seeded unpredictably at construction
+    // (DOPT_HIP_SEED in the environment fixes the seed, for reproducible runs); every execution
+    // continues the stream
+    R["uniform"] = [](const Graph &g, int id) -> std::unique_ptr<HIPKernel> {
+        const Operation &op = g.ops[id];
+        if (!need_deps(op, 0) || !need_f32(op)) return nullptr;
+        static std::atomic<uint64_t> objects{0};
+        uint64_t seed;
+        if (const char *fixed = std::getenv("DOPT_HIP_SEED")) {
+            seed = std::strtoull(fixed, nullptr, 0);
+        } else {
+            std::random_device rd;
+            seed = ((uint64_t)rd() << 32) ^ (uint64_t)rd();
+        }
+        seed += 0x9E3779B97F4A7C15ull * objects.fetch_add(1);  // distinct streams for the objects of one process
+        const size_t n = op.volume();
+        auto call = std::make_shared<uint64_t>(0);
+        return make([=](const std::vector<const void *> &, void *out) {
+            return dopt_hip_uniform(seed, (*call)++, n, (float *)out);
         });
     };
 }

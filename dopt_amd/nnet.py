@@ -95,6 +95,14 @@ def relu(inp):   # layers/relu.d
     return Layer([inp], core.relu(inp.output), core.relu(inp.trainOutput), [])
 
 
+def dropout(inp, drop_prob):   # layers/dropout.d:14-33
+    x, x_tr = inp.output, inp.trainOutput
+    drop_mask = float32(x_tr.shape, np.full(x_tr.volume, drop_prob, np.float32))
+    y_tr = core.gt(core.uniformSample(x_tr.shape), drop_mask) * x_tr
+    scale = float32(x.shape, np.full(x.volume, 1.0 - drop_prob, np.float32))
+    return Layer([inp], x * scale, y_tr, [])
+
+
 def maxPool(inp, dims):   # layers/maxpool.d
     return Layer([inp], maxpool(inp.output, dims), maxpool(inp.trainOutput, dims), [])
 

@@ -188,6 +188,14 @@ int dopt_hip_bias_fwd(size_t N, size_t C, size_t inner, const float *x, const fl
    this computes the plain sum (beta = 0), identical on the first execution. */
 int dopt_hip_bias_bwd(size_t N, size_t C, size_t inner, const float *dy, float *db);
 
+/* `uniform`: curandGenerateUniform at cuda/random.d:74 -- n floats drawn uniformly from (0, 1].
+   Counter-based Philox4x32-10: the values depend only on (seed, call, element index); a kernel
+   object draws `seed` once (the reference seeds with unpredictableSeed, cuda/random.d:64) and
+   passes call = 0, 1, 2, ... on successive executions.  dopt_hip_philox_raw writes the
+   generator's 32-bit words themselves (for known-answer tests of the generator). */
+int dopt_hip_uniform(uint64_t seed, uint64_t call, size_t n, float *out);
+int dopt_hip_philox_raw(uint64_t seed, uint64_t call, size_t n, uint32_t *out);
+
 /* `batchNormTrain`: cudnnBatchNormalizationForwardTraining (spatial), cudnn7.d:608-610.
    packed = [ y (N*C*inner) | newRunMean (C) | newRunVar (C) ] as core/ops/nnet.d:222-225;
    momentum is the op attribute (running = momentum*running + (1-momentum)*batch; the running

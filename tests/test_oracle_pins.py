@@ -8,6 +8,8 @@ independent evidence; nothing here retypes an oracle formula.
 import itertools
 
 import numpy as np
+
+import util
 import pytest
 
 import oracle as O
@@ -345,3 +347,14 @@ def test_fit_line_scenario(which):
             else:
                 p, st[0], st[1], st[2] = O.amsgrad_step(p, g, st[0], st[1], st[2], eta)
     assert abs(p[0] - 3) < 0.05 and abs(p[1] - 2) < 0.3, p
+
+
+# ----------------------------------------------------------------------------- Philox (checker of `uniform`)
+def test_numpy_philox_matches_published_vectors():
+    # Random123 kat_vectors, philox4x32 with 10 rounds
+    z = util.philox4x32_10(np.zeros((1, 4), np.uint32), [0, 0])[0]
+    assert [hex(v) for v in z] == ["0x6627e8d5", "0xe169c58d", "0xbc57ac4c", "0x9b00dbd8"]
+    f = util.philox4x32_10(np.full((1, 4), 0xFFFFFFFF, np.uint32), [0xFFFFFFFF, 0xFFFFFFFF])[0]
+    assert [hex(v) for v in f] == ["0x408f276d", "0x41c83b0e", "0xa20bc7c6", "0x6d5451fd"]
+    p = util.philox4x32_10(np.array([[0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344]], np.uint32), [0xA4093822, 0x299F31D0])[0]
+    assert [hex(v) for v in p] == ["0xd16cfe09", "0x94fdcceb", "0x5001e420", "0x24126ea1"]

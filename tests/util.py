@@ -29,3 +29,19 @@ def assert_close(got, want, what="", rtol=GEMM_RTOL, atol=GEMM_ATOL, scale=None)
         i = np.argmax(np.abs(got - want) - tol)
         raise AssertionError("%s: %d/%d outside tolerance; worst at %d: got %r want %r" %
                              (what, bad.sum(), bad.size, i, got.ravel()[i], want.ravel()[i]))
+
+
+M0, M1, W0, W1 = 0xD2511F53, 0xCD9E8D57, 0x9E3779B9, 0xBB67AE85
+
+
+def philox4x32_10(ctr, key):
+    """numpy restatement of the published algorithm; ctr is [n, 4] uint32, key [2]."""
+    c = [ctr[:, i].astype(np.uint64) for i in range(4)]
+    k0, k1 = np.uint64(key[0]), np.uint64(key[1])
+    mask = np.uint64(0xFFFFFFFF)
+    for _ in range(10):
+        p0, p1 = np.uint64(M0) * c[0], np.uint64(M1) * c[2]
+        hi0, lo0, hi1, lo1 = p0 >> np.uint64(32), p0 & mask, p1 >> np.uint64(32), p1 & mask
+        c = [hi1 ^ c[1] ^ k0, lo1, hi0 ^ c[3] ^ k1, lo0]
+        k0, k1 = (k0 + np.uint64(W0)) & mask, (k1 + np.uint64(W1)) & mask
+    return np.stack(c, axis=1).astype(np.uint32)
