@@ -307,36 +307,42 @@ __global__ __launch_bounds__(kBlock) void bn_grad_apply_k(IdxT total, IdxT C, Id
 // One block per channel for tensors whose channel (N * inner values) fits the block's registers:
 // x (and dy) are read ONCE, held in registers between the statistics and the output pass, and
 // the op is one launch instead of three.  Statistics are exact two-pass (mean, then centred
-// squares), reduced across the block in float64.
+// squares).
 constexpr int kResQuads = 8;  // float4 per thread
 
-__device__ inline double wave_sum_d(double v)
-{
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
-    return v;
-}
-
 // Sums kN per-thread values over the block (up to 16 wavefronts); every thread gets the totals.
+// Lanes are folded in fp32 with butterfly shuffles (a pairwise tree: error ~ log2(64) ulp), the
+// wavefront sums are added in float64 in wavefront order.  A one-wavefront block needs no LDS
+// and no barrier, which is what the many small channels of the deep layers run.
 template <int kN>
-__device__ inline void block_allsum_d(double (&v)[kN], double (*part)[16], double *total)
+__device__ inline void block_allsum(const float (&v)[kN], double (&total)[kN], float (*part)[16])
 {
-    const int wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    float w[kN];
 #pragma unroll
     for (int k = 0; k < kN; k++) {
-        v[k] = wave_sum_d(v[k]);
-        if ((threadIdx.x & 63) == 0) part[k][wave] = v[k];
+        w[k] = v[k];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) w[k] += __shfl_xor(w[k], off, 64);
     }
-    __syncthreads();
-    if (threadIdx.x < kN) {
-        double r = 0.0;
-        for (int w = 0; w < nw; w++) r += part[threadIdx.x][w];
-        total[threadIdx.x] = r;
+    const int nw = (blockDim.x + 63) >> 6;
+    if (nw == 1) {
+#pragma unroll
+        for (int k = 0; k < kN; k++) total[k] = (double)w[k];
+        return;
+    }
+    const int wave = threadIdx.x >> 6;
+    __syncthreads();  // `part` may still be read from the previous call
+    if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+        for (int k = 0; k < kN; k++) part[k][wave] = w[k];
     }
     __syncthreads();
 #pragma unroll
-    for (int k = 0; k < kN; k++) v[k] = total[k];
-    __syncthreads();
+    for (int k = 0; k < kN; k++) {
+        double r = 0.0;
+        for (int i = 0; i < nw; i++) r += (double)part[k][i];
+        total[k] = r;
+    }
 }
 
 template <bool kGrad>
@@ -346,8 +352,7 @@ __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, un
                                                        const float *ymask, int relu, float *out, float *out1, float *out2,
                                                        float *dx_sum)
 {
-    __shared__ double part[3][16];
-    __shared__ double total[3];
+    __shared__ float part[3][16];
     const unsigned c = blockIdx.x, T = blockDim.x, E4 = N * inner4;
     const float4 *x4 = (const float4 *)x, *g4 = (const float4 *)dy;
     float4 xv[kResQuads], gv[kResQuads];
@@ -368,17 +373,17 @@ __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, un
         }
     }
     const double m = 4.0 * (double)E4;
-    double red1[1] = {0.0};
+    double red1[1];
     {
         float s = 0.f;
 #pragma unroll
         for (int i = 0; i < kResQuads; i++) s += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);  // absent quads are zero
-        red1[0] = (double)s;
+        const float in1[1] = {s};
+        block_allsum<1>(in1, red1, part);
     }
-    block_allsum_d<1>(red1, part, total);
     const double mean = red1[0] / m;
     const float mean_hi = (float)mean, mean_lo = (float)(mean - (double)mean_hi);
-    double red3[3] = {0.0, 0.0, 0.0};
+    double red3[3];
     {
         float ss = 0.f, g1 = 0.f, g2 = 0.f;
 #pragma unroll
@@ -392,11 +397,9 @@ __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, un
                 g2 += (gv[i].x * d0 + gv[i].y * d1) + (gv[i].z * d2 + gv[i].w * d3);
             }
         }
-        red3[0] = (double)ss;
-        red3[1] = (double)g1;
-        red3[2] = (double)g2;
+        const float in3[3] = {ss, g1, g2};
+        block_allsum<3>(in3, red3, part);
     }
-    block_allsum_d<3>(red3, part, total);
     const double var = red3[0] / m;  // biased
     const double rstd = 1.0 / sqrt(var + eps);
     float4 *o4 = (float4 *)out;
@@ -441,8 +444,9 @@ __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, un
             out2[c] = (float)db;
         }
         if (dx_sum) {  // the per-channel sum of dx: the bias gradient of an addBias feeding this batch norm
-            double red[1] = {(double)sdx};
-            block_allsum_d<1>(red, part, total);
+            const float in1[1] = {sdx};
+            double red[1];
+            block_allsum<1>(in1, red, part);
             if (threadIdx.x == 0) dx_sum[c] = (float)red[0];
         }
     }
@@ -454,7 +458,9 @@ unsigned resident_threads(size_t N, size_t C, size_t inner, const void *a, const
     if ((inner & 3) != 0 || !aligned16(a) || (b && !aligned16(b)) || !aligned16(o)) return 0;
     const size_t E4 = N * (inner / 4);
     if (E4 == 0 || E4 > (size_t)kResQuads * 1024 || N * C * (inner / 4) >= 0xffffffffull) return 0;
-    size_t T = (ceil_div(E4, (size_t)kResQuads) + 63) / 64 * 64;
+    // two quads per thread where the channel is small enough: more wavefronts in flight per CU
+    size_t T = (ceil_div(E4, (size_t)2) + 63) / 64 * 64;
+    if (T > 1024) T = 1024;
     return (unsigned)(T < 64 ? 64 : T);
 }
 

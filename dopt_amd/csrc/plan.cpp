@@ -683,7 +683,11 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
                 size_t off;
                 const int rg = root(op.deps[0], &off);
                 const Operation &rgo = g.ops[rg];
-                if (rgo.opType == "reluGrad" && rgo.deps.size() == 3 && off == 0 && alias[rg].source < 0 &&
+                // the fused kernel tests the sign of y where reluGrad tests x: the same thing when y = relu(x)
+                const bool pair = rgo.opType == "reluGrad" && rgo.deps.size() == 3 &&
+                                  g.ops[rgo.deps[1]].opType == "relu" && g.ops[rgo.deps[1]].deps.size() == 1 &&
+                                  g.ops[rgo.deps[1]].deps[0] == rgo.deps[2];
+                if (pair && off == 0 && alias[rg].source < 0 &&
                     !isOutput(rg) && uses[rg].size() == 1 && rgo.volume() == g.ops[op.deps[1]].volume()) {
                     fusedKind[id] = 3;
                     inputsOf[id] = {rgo.deps[0], rgo.deps[1], op.deps[1], op.deps[2]};
