@@ -80,24 +80,96 @@ __global__ __launch_bounds__(kBlock) void repeat_nd(NdDesc d, size_t total, cons
     }
 }
 
-// Contiguous copy, 128-bit when both ends are 16-byte aligned.  Full tiles of 8 x 256 quads run
-// without bounds tests so that all eight loads of a lane are in flight before the first store.
+// ---- the same three maps for tensors below 2^32 elements --------------------------------------
+// Coordinates are decoded with 32-bit multiply-high divisions by precomputed reciprocals, axes the
+// map leaves alone are merged on the host, the outermost coordinate is the last quotient (no
+// division), each lane keeps four independent loads in flight, and T is a 16-byte quad when the
+// innermost axis allows it.
+struct Nd32 {
+    int rank;
+    uint32_t out_shape[kMaxRank], out_magic[kMaxRank];
+    uint32_t in_shape[kMaxRank], in_magic[kMaxRank];
+    uint32_t in_stride[kMaxRank];
+    uint32_t offset[kMaxRank];
+};
+
+// floor(2^32 / d) clamped to 32 bits: the quotient estimate is at most one too small
+inline uint32_t recip32(uint32_t d)
+{
+    uint64_t m = (1ull << 32) / d;
+    return m > 0xffffffffull ? 0xffffffffu : (uint32_t)m;
+}
+
+__device__ __forceinline__ void divmod32(uint32_t x, uint32_t d, uint32_t magic, uint32_t &q, uint32_t &r)
+{
+    q = __umulhi(x, magic);
+    r = x - q * d;
+    if (r >= d) {
+        q++;
+        r -= d;
+    }
+}
+
+enum { kSlice = 0, kPad = 1, kRepeat = 2 };
+
+template <int kMode, class T>
+__global__ __launch_bounds__(kBlock) void map_nd32(Nd32 d, uint32_t total, const T *in, T *out)
+{
+    constexpr int U = 4;
+    const uint32_t base = blockIdx.x * (uint32_t)(kBlock * U) + threadIdx.x;
+    T v[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const uint32_t idx = base + u * kBlock;
+        uint32_t rem = idx < total ? idx : 0, src = 0;   // lanes past the end decode element 0 and store nothing
+        bool inside = true;
+#pragma unroll
+        for (int i = kMaxRank - 1; i >= 0; i--) {
+            if (i >= d.rank) continue;
+            uint32_t c;
+            if (i > 0) divmod32(rem, d.out_shape[i], d.out_magic[i], rem, c);
+            else c = rem;
+            if (kMode == kSlice) c += d.offset[i];
+            if (kMode == kPad) {
+                c -= d.offset[i];            // wraps to a huge value left of the input
+                inside = inside && c < d.in_shape[i];
+            }
+            if (kMode == kRepeat) {
+                uint32_t q;
+                divmod32(c, d.in_shape[i], d.in_magic[i], q, c);
+            }
+            src += c * d.in_stride[i];
+        }
+        // an unconditional load (element 0 stands in outside the input) keeps all four in flight
+        const T got = in[inside ? src : 0];
+        v[u] = inside ? got : T{};
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const uint32_t idx = base + u * kBlock;
+        if (idx < total) out[idx] = v[u];
+    }
+}
+
+// Contiguous copy, 128-bit when both ends are 16-byte aligned.  One tile of 4 x 256 quads per block;
+// a lane's four loads are all in flight before its first store.
+constexpr int kCopyQuads = 4;
 __global__ __launch_bounds__(kBlock) void copy_vec4(size_t n4, const uint4 *in, uint4 *out)
 {
-    constexpr int U = 8;
-    const size_t tile = (size_t)kBlock * U;
-    const size_t full = n4 / tile;
-    for (size_t t = blockIdx.x; t < full; t += gridDim.x) {
-        const uint4 *src = in + t * tile + threadIdx.x;
-        uint4 *dst = out + t * tile + threadIdx.x;
-        uint4 v[U];
-#pragma unroll
-        for (int u = 0; u < U; u++) v[u] = src[u * kBlock];
-#pragma unroll
-        for (int u = 0; u < U; u++) dst[u * kBlock] = v[u];
+    // four named values, not an array: the compiler moved an array of quads into LDS
+    const size_t i0 = (size_t)blockIdx.x * (kBlock * kCopyQuads) + threadIdx.x;
+    const size_t i1 = i0 + kBlock, i2 = i0 + 2 * kBlock, i3 = i0 + 3 * kBlock;
+    if (i3 < n4) {
+        const uint4 a = in[i0], b = in[i1], c = in[i2], d = in[i3];
+        out[i0] = a;
+        out[i1] = b;
+        out[i2] = c;
+        out[i3] = d;
+        return;
     }
-    if (blockIdx.x == 0)
-        for (size_t i = full * tile + threadIdx.x; i < n4; i += kBlock) out[i] = in[i];
+    if (i0 < n4) out[i0] = in[i0];   // the ragged last tile
+    if (i1 < n4) out[i1] = in[i1];
+    if (i2 < n4) out[i2] = in[i2];
 }
 
 __global__ __launch_bounds__(kBlock) void copy_scalar(size_t n, const uint32_t *in, uint32_t *out)
@@ -132,10 +204,10 @@ int copy_contiguous(const uint32_t *in, uint32_t *out, size_t n)
     if (n == 0) return DOPT_HIP_OK;
     if (aligned16(in) && aligned16(out) && n >= 4) {
         size_t n4 = n / 4;
-        size_t blocks = ceil_div(n4, (size_t)kBlock * 8);
-        size_t cap = (size_t)num_cus() * 16;
-        hipLaunchKernelGGL(copy_vec4, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(kBlock), 0, stream(), n4,
-                           (const uint4 *)in, (uint4 *)out);
+        size_t blocks = ceil_div(n4, (size_t)kBlock * kCopyQuads);
+        DOPT_REQUIRE(blocks <= 0x7fffffffu, "copy: %zu elements are more than one launch covers", n);
+        hipLaunchKernelGGL(copy_vec4, dim3((unsigned)blocks), dim3(kBlock), 0, stream(), n4, (const uint4 *)in,
+                           (uint4 *)out);
         DOPT_LAUNCH_CHECK();
         size_t tail = n - n4 * 4;
         if (tail) {
@@ -163,6 +235,67 @@ void fill_strides(NdDesc &d)
         d.in_stride[i] = s;
         s *= d.in_shape[i];
     }
+}
+
+// Runs slice / pad / repeat through map_nd32 when every extent fits 32 bits; returns -1 when it
+// does not (the caller then uses the 64-bit kernels), else a status code.  The axis lists are the caller's, outermost
+// first; `offset` is the slice start or the pad-before count and is ignored for repeat.
+template <int kMode>
+int try_map32(int rank, const size_t *in_shape, const size_t *out_shape, const size_t *offset, const void *in,
+              void *out)
+{
+    size_t vin = 1, vout = 1;
+    for (int i = 0; i < rank; i++) {
+        vin *= in_shape[i];
+        vout *= out_shape[i];
+    }
+    if (rank < 1 || vin >= (1ull << 32) || vout >= (1ull << 32) || vin == 0) return -1;
+    // merge an axis into its outer neighbour when the map leaves it whole
+    size_t is[kMaxRank], os[kMaxRank], of[kMaxRank];
+    int r = 0;
+    for (int i = 0; i < rank; i++) {
+        const size_t o = kMode == kRepeat ? 0 : offset[i];
+        const bool whole = in_shape[i] == out_shape[i] && o == 0;
+        if (r > 0 && whole) {
+            is[r - 1] *= in_shape[i];
+            os[r - 1] *= out_shape[i];
+            of[r - 1] *= in_shape[i];
+        } else {
+            is[r] = in_shape[i];
+            os[r] = out_shape[i];
+            of[r] = o;
+            r++;
+        }
+    }
+    // quads when the innermost axis and both pointers allow it
+    const bool quads = is[r - 1] % 4 == 0 && os[r - 1] % 4 == 0 && of[r - 1] % 4 == 0 && aligned16(in) && aligned16(out);
+    if (quads) {
+        is[r - 1] /= 4;
+        os[r - 1] /= 4;
+        of[r - 1] /= 4;
+        vout /= 4;
+    }
+    Nd32 d{};
+    d.rank = r;
+    uint32_t stride = 1;
+    for (int i = r - 1; i >= 0; i--) {
+        d.in_shape[i] = (uint32_t)is[i];
+        d.out_shape[i] = (uint32_t)os[i];
+        d.offset[i] = (uint32_t)of[i];
+        d.in_magic[i] = recip32(d.in_shape[i]);
+        d.out_magic[i] = recip32(d.out_shape[i]);
+        d.in_stride[i] = stride;
+        stride *= d.in_shape[i];
+    }
+    const unsigned blocks = (unsigned)ceil_div(vout, (size_t)kBlock * 4);
+    if (quads)
+        hipLaunchKernelGGL((map_nd32<kMode, uint4>), dim3(blocks), dim3(kBlock), 0, stream(), d, (uint32_t)vout,
+                           (const uint4 *)in, (uint4 *)out);
+    else
+        hipLaunchKernelGGL((map_nd32<kMode, uint32_t>), dim3(blocks), dim3(kBlock), 0, stream(), d, (uint32_t)vout,
+                           (const uint32_t *)in, (uint32_t *)out);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
 }
 
 // ---- many small device-to-device copies in one launch -----------------------------------------
@@ -205,6 +338,7 @@ int dopt_hip_slice(int rank, const size_t *in_shape, const size_t *out_shape, co
         size_t off = rank > 0 ? start[0] * inner : 0;
         return copy_contiguous((const uint32_t *)in + off, (uint32_t *)out, total);
     }
+    if (int rc = try_map32<kSlice>(rank, in_shape, out_shape, start, in, out); rc >= 0) return rc;
     NdDesc d{};
     d.rank = rank;
     for (int i = 0; i < rank; i++) {
@@ -230,6 +364,7 @@ int dopt_hip_pad(int rank, const size_t *in_shape, const size_t *out_shape, cons
     size_t total = volume(out_shape, rank);
     if (total == 0) return DOPT_HIP_OK;
     if (rank == 0) return copy_contiguous((const uint32_t *)in, (uint32_t *)out, 1);
+    if (int rc = try_map32<kPad>(rank, in_shape, out_shape, before, in, out); rc >= 0) return rc;
     NdDesc d{};
     d.rank = rank;
     for (int i = 0; i < rank; i++) {
@@ -261,6 +396,7 @@ int dopt_hip_repeat(int rank, const size_t *in_shape, const size_t *reps, const 
     size_t total = volume(d.out_shape, rank);
     if (total == 0) return DOPT_HIP_OK;
     if (identity) return copy_contiguous((const uint32_t *)in, (uint32_t *)out, total);  // cuda/basic.d:168-172
+    if (int rc = try_map32<kRepeat>(rank, d.in_shape, d.out_shape, nullptr, in, out); rc >= 0) return rc;
     fill_strides(d);
     hipLaunchKernelGGL(repeat_nd, dim3(grid_for(total)), dim3(kBlock), 0, stream(), d, total, (const uint32_t *)in,
                        (uint32_t *)out);

@@ -342,6 +342,105 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_fwd_k(size_t N, size_t C,
     for (size_t c = lane; c < C; c += 64) py[c] = py[c] / s;
 }
 
+// Rows of at most 1024 values whose length is a multiple of four stay in registers: G lanes share a
+// row (64 / G rows per wavefront), each lane holds up to four quads, the row is read once and
+// written once.
+template <int G>
+__device__ __forceinline__ float group_max(float v)
+{
+#pragma unroll
+    for (int off = G / 2; off > 0; off >>= 1) v = dmax(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+template <int G>
+__device__ __forceinline__ float group_sum(float v)
+{
+#pragma unroll
+    for (int off = G / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+template <int G>
+__global__ __launch_bounds__(kBlock) void softmax_reg_fwd_k(size_t N, uint32_t C4, const float4 *x, float4 *y)
+{
+    const size_t row = ((size_t)blockIdx.x * kBlock + threadIdx.x) / G;
+    const uint32_t lig = threadIdx.x % G;
+    const bool live = row < N;                    // dead rows still take part in the shuffles
+    const float4 *px = x + (live ? row : 0) * C4;
+    float v[16];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const uint32_t c = lig + G * k;
+        const float4 q = px[c < C4 ? c : 0];
+        const bool in = c < C4;
+        v[4 * k + 0] = in ? q.x : -FLT_MAX;
+        v[4 * k + 1] = in ? q.y : -FLT_MAX;
+        v[4 * k + 2] = in ? q.z : -FLT_MAX;
+        v[4 * k + 3] = in ? q.w : -FLT_MAX;
+    }
+    float m = v[0];
+#pragma unroll
+    for (int i = 1; i < 16; i++) m = dmax(m, v[i]);
+    m = group_max<G>(m);
+    float s = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const bool in = lig + G * k < C4;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            v[4 * k + j] = in ? expf(v[4 * k + j] - m) : 0.0f;
+            s += v[4 * k + j];
+        }
+    }
+    s = group_sum<G>(s);
+    if (!live) return;
+    float4 *py = y + row * C4;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const uint32_t c = lig + G * k;
+        if (c < C4) py[c] = make_float4(v[4 * k] / s, v[4 * k + 1] / s, v[4 * k + 2] / s, v[4 * k + 3] / s);
+    }
+}
+
+template <int G>
+__global__ __launch_bounds__(kBlock) void softmax_reg_bwd_k(size_t N, uint32_t C4, const float4 *dy, const float4 *y,
+                                                             float4 *dx)
+{
+    const size_t row = ((size_t)blockIdx.x * kBlock + threadIdx.x) / G;
+    const uint32_t lig = threadIdx.x % G;
+    const bool live = row < N;
+    const size_t base = (live ? row : 0) * C4;
+    float g[16], p[16];
+    float dot = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const uint32_t c = lig + G * k;
+        const bool in = c < C4;
+        const float4 a = dy[base + (in ? c : 0)], b = y[base + (in ? c : 0)];
+        g[4 * k + 0] = a.x, g[4 * k + 1] = a.y, g[4 * k + 2] = a.z, g[4 * k + 3] = a.w;
+        p[4 * k + 0] = b.x, p[4 * k + 1] = b.y, p[4 * k + 2] = b.z, p[4 * k + 3] = b.w;
+        if (in) dot += a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w;
+    }
+    dot = group_sum<G>(dot);
+    if (!live) return;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const uint32_t c = lig + G * k;
+        if (c < C4)
+            dx[base + c] = make_float4(p[4 * k] * (g[4 * k] - dot), p[4 * k + 1] * (g[4 * k + 1] - dot),
+                                       p[4 * k + 2] * (g[4 * k + 2] - dot), p[4 * k + 3] * (g[4 * k + 3] - dot));
+    }
+}
+
+// the lanes a row of C4 quads is shared by, or 0 when the register kernels do not take it
+int softmax_group(size_t C, size_t inner, const void *a, const void *b, const void *c)
+{
+    if (inner != 1 || C % 4 != 0 || C < 64 || C > 1024 || !aligned16(a) || !aligned16(b) || !aligned16(c)) return 0;
+    const size_t C4 = C / 4;
+    return C4 <= 16 ? 16 : (C4 <= 32 ? 32 : 64);
+}
+
 __global__ __launch_bounds__(kBlock) void softmax_rows_bwd_k(size_t N, size_t C, const float *dy, const float *y,
                                                               float *dx)
 {
@@ -530,7 +629,13 @@ int dopt_hip_softmax_fwd(size_t N, size_t C, size_t inner, const float *x, float
     if (N * C * inner == 0) return DOPT_HIP_OK;
     DOPT_REQUIRE(x && y, "dopt_hip_softmax_fwd: null argument");
     DOPT_ENSURE_INIT();
-    if (inner == 1 && C >= 64)
+    if (const int G = softmax_group(C, inner, x, y, y)) {
+        const dim3 grid((unsigned)ceil_div(N * G, (size_t)kBlock)), block(kBlock);
+        const uint32_t C4 = (uint32_t)(C / 4);
+        if (G == 16) hipLaunchKernelGGL(softmax_reg_fwd_k<16>, grid, block, 0, stream(), N, C4, (const float4 *)x, (float4 *)y);
+        else if (G == 32) hipLaunchKernelGGL(softmax_reg_fwd_k<32>, grid, block, 0, stream(), N, C4, (const float4 *)x, (float4 *)y);
+        else hipLaunchKernelGGL(softmax_reg_fwd_k<64>, grid, block, 0, stream(), N, C4, (const float4 *)x, (float4 *)y);
+    } else if (inner == 1 && C >= 64)
         hipLaunchKernelGGL(softmax_rows_fwd_k, dim3((unsigned)ceil_div(N, (size_t)(kBlock / 64))), dim3(kBlock), 0, stream(),
                            N, C, x, y);
     else
@@ -544,7 +649,13 @@ int dopt_hip_softmax_bwd(size_t N, size_t C, size_t inner, const float *dy, cons
     if (N * C * inner == 0) return DOPT_HIP_OK;
     DOPT_REQUIRE(dy && y && dx, "dopt_hip_softmax_bwd: null argument");
     DOPT_ENSURE_INIT();
-    if (inner == 1 && C >= 64)
+    if (const int G = softmax_group(C, inner, dy, y, dx)) {
+        const dim3 grid((unsigned)ceil_div(N * G, (size_t)kBlock)), block(kBlock);
+        const uint32_t C4 = (uint32_t)(C / 4);
+        if (G == 16) hipLaunchKernelGGL(softmax_reg_bwd_k<16>, grid, block, 0, stream(), N, C4, (const float4 *)dy, (const float4 *)y, (float4 *)dx);
+        else if (G == 32) hipLaunchKernelGGL(softmax_reg_bwd_k<32>, grid, block, 0, stream(), N, C4, (const float4 *)dy, (const float4 *)y, (float4 *)dx);
+        else hipLaunchKernelGGL(softmax_reg_bwd_k<64>, grid, block, 0, stream(), N, C4, (const float4 *)dy, (const float4 *)y, (float4 *)dx);
+    } else if (inner == 1 && C >= 64)
         hipLaunchKernelGGL(softmax_rows_bwd_k, dim3((unsigned)ceil_div(N, (size_t)(kBlock / 64))), dim3(kBlock), 0, stream(),
                            N, C, dy, y, dx);
     else

@@ -1,11 +1,14 @@
 """Per-kernel throughput of the bandwidth-bound entry points against the HBM roofline.
 
-    python -m dopt_amd.kernel_bench [--iters 50] [--json]
+    python -m dopt_amd.kernel_bench [--iters 50] [--scale S] [--json]
 
 Each row times one C-ABI entry point at a shape taken from the benchmark configurations (the
 VGG-16 b128 activations, the 16M-parameter fused update) with HIP events on the library's stream
 and reports ALGORITHMIC bytes / time: every tensor counted once per kernel, whatever the kernel
-really moves (a two-pass batch norm reads its input twice but is charged 8 B/element).
+really moves (a two-pass batch norm reads its input twice but is charged 8 B/element).  At the
+configuration shapes (33.5 MB per tensor) a kernel lasts 5-15 us, of which 2-3 us are launch ramp
+and tail; --scale S multiplies the leading dimension of every shape by S to show the rate the same
+kernels reach on tensors that take longer to stream.
 """
 import argparse
 import ctypes as C
@@ -40,7 +43,7 @@ def _rand(shape, seed=0):
     return ops.tensor(np.random.default_rng(seed).standard_normal(shape, dtype=np.float32))
 
 
-def cases():
+def cases(scale=1):
     """(name, shape text, algorithmic bytes, callable) per row.  Every callable writes into an output
     tensor allocated once, before the timed loop, so a row times the kernels of one entry point only."""
     rows, keep = [], []
@@ -50,7 +53,7 @@ def cases():
         keep.append(o)
         rows.append((name, shape, nbytes, lambda: fn(o)))   # ... every later call reuses it
 
-    act = (128, 64, 32, 32)                      # the largest VGG activation: 8.39 M elements, 33.5 MB
+    act = (128 * scale, 64, 32, 32)              # the largest VGG activation: 8.39 M elements, 33.5 MB
     n = int(np.prod(act))
     x, dy = _rand(act, 1), _rand(act, 2)
     fa, fb = x.reshape((n,)), dy.reshape((n,))
@@ -64,7 +67,7 @@ def cases():
     add("addBias", str(act), 8 * n, lambda o: ops.add_bias(x, bias, out=o))
     add("addBiasGrad", str(act), 4 * n, lambda o: ops.add_bias_grad(dy, out=o))
     add("maxpool 2x2", str(act), 5 * n, lambda o: ops.maxpool(x, (2, 2), out=o))
-    pdy = _rand((128, 64, 16, 16), 4)
+    pdy = _rand((128 * scale, 64, 16, 16), 4)
     add("maxpoolGrad 2x2", str(act), 9 * n, lambda o: ops.maxpool_grad(pdy, x, (2, 2), out=o))
     g, b, rm, rv = (_rand((64,), 5 + i) for i in range(4))
     rv.set(np.abs(rv.numpy()) + 0.5)
@@ -74,14 +77,14 @@ def cases():
     add("sum (all axes)", str(act), 4 * n, lambda o: ops.sum(x, out=o))
     add("sum axes [0,2,3]", str(act), 4 * n, lambda o: ops.sum(x, [0, 2, 3], out=o))
     add("maxElement (all axes)", str(act), 4 * n, lambda o: ops.max_element(x, out=o))
-    m2 = x.reshape((4096, 2048))
-    add("transpose", "(4096, 2048)", 8 * n, lambda o: ops.transpose(m2, out=o))
-    add("argmin axis 1", "(4096, 2048)", 4 * n, lambda o: ops.argmin(m2, 1, out=o))
-    sm = _rand((65536, 128), 9)
-    add("softmax", "(65536, 128)", 8 * sm.size, lambda o: ops.softmax(sm, out=o))
+    m2 = x.reshape((4096 * scale, 2048))
+    add("transpose", str(tuple(m2.shape)), 8 * n, lambda o: ops.transpose(m2, out=o))
+    add("argmin axis 1", str(tuple(m2.shape)), 4 * n, lambda o: ops.argmin(m2, 1, out=o))
+    sm = _rand((65536 * scale, 128), 9)
+    add("softmax", str(tuple(sm.shape)), 8 * sm.size, lambda o: ops.softmax(sm, out=o))
     add("slice (contiguous)", "%d -> %d" % (n, n - 128), 8 * (n - 128), lambda o: ops.slice(fa, [0], [n - 128], out=o))
-    add("slice (4-d interior)", "%s -> (128, 64, 30, 30)" % (act,), 8 * 128 * 64 * 900,
-        lambda o: ops.slice(x, [0, 0, 1, 1], [128, 64, 31, 31], out=o))
+    add("slice (4-d interior)", "%s -> (.., 30, 30)" % (act,), 8 * act[0] * 64 * 900,
+        lambda o: ops.slice(x, [0, 0, 1, 1], [act[0], 64, 31, 31], out=o))
     add("pad (1-d tail)", "%d + 128" % n, 8 * n, lambda o: ops.pad(fa, [0], [128], out=o))
     add("repeat", "%s x [1,1,2,2]" % (act,), 20 * n, lambda o: ops.repeat(x, [1, 1, 2, 2], out=o))
 
@@ -102,10 +105,11 @@ def cases():
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--iters", type=int, default=50)
+    ap.add_argument("--scale", type=int, default=1, help="multiply the leading dimension of the activation shapes")
     ap.add_argument("--json", action="store_true")
     args = ap.parse_args()
     out = []
-    rows, keep = cases()
+    rows, keep = cases(args.scale)
     for name, shape, nbytes, fn in rows:
         sec = _time(fn, args.iters)
         out.append({"kernel": name, "shape": shape, "us": sec * 1e6, "GB/s": nbytes / sec / 1e9,

@@ -191,6 +191,36 @@ def test_slice_pad_repeat(shape):
     assert np.array_equal(ops.slice(tx, start, stop).numpy(), x[cut:])
 
 
+@pytest.mark.parametrize("shape,reps", [((4, 3, 8, 8), (1, 1, 2, 2)), ((6, 16), (3, 1)), ((5, 12), (1, 4)), ((2, 3, 4), (2, 1, 3)),
+                                        ((128, 64), (1, 1)), ((7,), (5,))])
+def test_repeat_quads_and_merged_axes(shape, reps):
+    x = rng(23).integers(-1000, 1000, shape).astype(np.int32)
+    assert np.array_equal(ops.repeat(T(x), list(reps)).numpy(), O.repeat(x, list(reps)))
+
+
+def test_layout_maps_aligned_quads():
+    """Extents, offsets and pointers that are all multiples of four take the 16-byte path."""
+    x = rng(24).integers(-1000, 1000, (6, 5, 16)).astype(np.int32)
+    tx = T(x)
+    assert np.array_equal(ops.slice(tx, [1, 0, 4], [5, 5, 12]).numpy(), x[1:5, :, 4:12])
+    assert np.array_equal(ops.pad(tx, [1, 0, 4], [0, 2, 8]).numpy(), O.pad(x, [1, 0, 4], [0, 2, 8]))
+    assert np.array_equal(ops.pad(tx, [0, 0, 0], [0, 0, 128]).numpy(), O.pad(x, [0, 0, 0], [0, 0, 128]))
+
+
+def test_slice_pad_large_index_range():
+    """Above 2^27 elements the reciprocal-multiply quotient is off by one for many indices; the
+    remainder correction has to catch every one of them."""
+    shape = (5, 6151, 6143)
+    x = np.arange(np.prod(shape), dtype=np.int64).astype(np.int32).reshape(shape)
+    tx = T(x)
+    got = ops.slice(tx, [1, 100, 141], [4, 6101, 6142]).numpy()
+    assert np.array_equal(got, x[1:4, 100:6101, 141:6142])
+    del got
+    small = T(x[:3])
+    got = ops.pad(small, [1, 0, 1], [0, 1, 0]).numpy()
+    assert np.array_equal(got, np.pad(x[:3], ((1, 0), (0, 1), (1, 0))))
+
+
 def test_slice_rejects_out_of_range():
     from dopt_amd import capi
     with pytest.raises(capi.HipError):
@@ -327,7 +357,7 @@ def test_maxpool_and_grad(shape, dims):
 
 
 @pytest.mark.parametrize("shape", [(1, 5), (128, 10), (256, 10), (4, 7, 3), (3, 5, 2, 2), (37, 64), (300, 1000),
-                                   (5, 130)])
+                                   (5, 130), (70, 128), (9, 132), (33, 260), (17, 1024), (3, 1028), (1, 68)])
 def test_softmax_and_grad(shape):
     r = rng(52)
     x = (r.standard_normal(shape) * 3).astype(np.float32)
