@@ -6,6 +6,8 @@ reference's own code): it exists so that the benchmark and the parity tests run 
 the reference would emit for these models.  Parameter initialisation draws from a seeded numpy
 generator instead of std.random (the benchmark prescribes its own seeded inputs).
 """
+import math
+
 import numpy as np
 
 from . import core
@@ -42,41 +44,61 @@ def dataSource(inputs):   # layers/datasource.d
     return Layer([], inputs, inputs, [])
 
 
-def dense(inp, num_outputs, init, use_bias=True, weight_decay=0.0):   # layers/dense.d:67-150
+def _safe_add(a, b):   # layers/dense.d:82-93
+    if a is None:
+        return b
+    return a if b is None else a + b
+
+
+def dense(inp, num_outputs, init, use_bias=True, weight_decay=0.0, weight_proj=None, bias_proj=None,
+          maxgain=math.inf, spectral_decay=0.0):   # layers/dense.d:67-150
+    from . import lipschitz
     x, x_tr = inp.output, inp.trainOutput
     x = x.reshape([x.shape[0], x.volume // x.shape[0]])
     x_tr = x_tr.reshape([x_tr.shape[0], x_tr.volume // x_tr.shape[0]])
     weights = float32([num_outputs, x.shape[1]])
     init.he_gaussian(weights)
     weight_loss = None if weight_decay == 0.0 else weight_decay * core.sum(weights * weights)
+    weight_loss = _safe_add(weight_loss,
+                            None if spectral_decay == 0.0 else spectral_decay * lipschitz.denseSpectralNorm(weights))
     y = matmul(x, transpose(weights, [1, 0]))
     y_tr = matmul(x_tr, transpose(weights, [1, 0]))
-    params = [Parameter(weights, weight_loss, None)]
+    if maxgain != math.inf:
+        weight_proj = lipschitz.maxGainProjection(x_tr, y_tr, maxgain, weight_proj)
+    params = [Parameter(weights, weight_loss, weight_proj)]
     if use_bias:
         bias = float32([num_outputs])
         y = y + core.repeat(bias, y.shape[0])
         y_tr = y_tr + core.repeat(bias, y_tr.shape[0])
-        params.append(Parameter(bias, None, None))
+        params.append(Parameter(bias, None, bias_proj))
     return Layer([inp], y, y_tr, params)
 
 
 def conv2D(inp, out_channels, filter_dims, init, padding=(0, 0), stride=(1, 1), use_bias=True,
-           weight_decay=0.0):   # layers/conv.d:66-151
+           weight_decay=0.0, filter_proj=None, bias_proj=None, maxgain=math.inf,
+           spectral_decay=0.0):   # layers/conv.d:66-165
+    from . import lipschitz
     x, x_tr = inp.output, inp.trainOutput
     filters = float32([out_channels, x.shape[1]] + list(filter_dims))
     init.he_gaussian(filters)
     filter_loss = None if weight_decay == 0.0 else weight_decay * core.sum(filters * filters)
+    filter_loss = _safe_add(filter_loss,
+                            None if spectral_decay == 0.0 else spectral_decay * lipschitz.convSpectralNorm(filters))
     y = convolution(x, filters, padding, stride)
     y_tr = convolution(x_tr, filters, padding, stride)
-    params = [Parameter(filters, filter_loss, None)]
+    if maxgain != math.inf:   # measured on the pre-bias response, as the reference does
+        filter_proj = lipschitz.maxGainProjection(x_tr, y_tr, maxgain, filter_proj)
+    params = [Parameter(filters, filter_loss, filter_proj)]
     if use_bias:
         biases = float32([out_channels])
         y, y_tr = addBias(y, biases), addBias(y_tr, biases)
-        params.append(Parameter(biases, None, None))
+        params.append(Parameter(biases, None, bias_proj))
     return Layer([inp], y, y_tr, params)
 
 
-def batchNorm(inp, momentum=0.9):   # layers/batchnorm.d:57-156
+def batchNorm(inp, momentum=0.9, gamma_decay=0.0, gamma_proj=None, beta_proj=None, maxgain=math.inf,
+              lipschitz=math.inf):   # layers/batchnorm.d:57-156
+    from . import lipschitz as lip
     x, x_tr = inp.output, inp.trainOutput
     c = x.shape[1]
     gamma = float32([1, c, 1, 1], np.ones(c, np.float32))
@@ -86,7 +108,19 @@ def batchNorm(inp, momentum=0.9):   # layers/batchnorm.d:57-156
     # the layer holds its momentum as a float and hands it to the op's double attribute
     y_tr, mean_update, var_update = batchNormTrain(x_tr, gamma, beta, mean, var, float(np.float32(momentum)))
     y = batchNormInference(x, gamma, beta, mean, var)
-    return Layer([inp], y, y_tr, [Parameter(gamma), Parameter(beta),
+    if maxgain != math.inf:
+        # the gain of the scaling alone: the layer's response with zero mean and zero shift
+        zeros = float32Constant([c], np.zeros(c, np.float32))
+        gamma_proj = lip.maxGainProjection(x_tr, batchNormInference(x_tr, gamma, zeros, zeros, var), maxgain, gamma_proj)
+    elif lipschitz != math.inf:
+        user_proj = gamma_proj
+
+        def gamma_proj(new_gamma):   # batchnorm.d:113-127: max |gamma / sqrt(var + 1e-6)| held below the bound
+            norm = core.maxElement(core.abs(new_gamma / core.sqrt(var_update.reshape(new_gamma.shape) + 1e-6)))
+            g = new_gamma * (1.0 / core.max(float32Constant([], [1.0]), norm / lipschitz))
+            return g if user_proj is None else user_proj(g)
+    gamma_loss = None if gamma_decay == 0.0 else gamma_decay * core.sum(gamma * gamma)
+    return Layer([inp], y, y_tr, [Parameter(gamma, gamma_loss, gamma_proj), Parameter(beta, None, beta_proj),
                                   Parameter(mean, None, lambda ignored: mean_update),
                                   Parameter(var, None, lambda ignored: var_update)])
 

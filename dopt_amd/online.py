@@ -10,7 +10,8 @@ un-fused ground truth.
 computes only the outputs and the gradients (plus projections that do not depend on the updated
 value, i.e. batch-norm's running statistics), and ONE multi-tensor kernel applies the rule in
 place with the same per-node fp32 rounding, so parameters and optimizer state match the un-fused
-form bit for bit.
+form bit for bit.  Projections of the updated value itself (operator-norm constraints) run as a
+second small plan after the kernel.
 """
 import numpy as np
 
@@ -107,20 +108,37 @@ class _FusedUpdater:
         projs = projs or {}
         self.rule, self.hyper, self.outputs, self.wrt = rule, hyper, list(outputs), list(wrt)
         grads = grad(outputs[0], wrt)
-        # A projection may only be applied here if it ignores the updated value (batch-norm replaces
-        # its running statistics by graph outputs, nnet/layers/batchnorm.d:140-154).
-        proj_ops, skip = [], []
+        # Three kinds of projection (online/sgd.d:75-85 applies them to the updated value inside
+        # the one plan):
+        #  - it ignores the updated value (batch-norm replaces its running statistics by graph
+        #    outputs, nnet/layers/batchnorm.d:140-154): computed by the step's plan, the kernel skips
+        #    the parameter;
+        #  - it depends on the updated value and otherwise on nothing the step reads (the
+        #    operator-norm projections of nnet/lipschitz.d: constants, their own scalar variables,
+        #    fresh random draws): a second plan, run after the fused kernel, reads the updated
+        #    parameter and writes the projected one over it;
+        #  - it also reads other variables (the max-gain projections read this batch's
+        #    activations, computed from the OLD parameters): only the op-graph optimizers can
+        #    reproduce that ordering.
+        proj_ops, skip, post = [], [], []
+        step_nodes = {id(o) for o in core.topological_sort(list(outputs))}   # what the step itself reads
         for w in wrt:
-            if w in projs:
-                probe = float32(w.shape)
-                p = projs[w](probe)
-                if any(o is probe for o in core.topological_sort([p])):
-                    raise NotImplementedError("fused updaters only take projections that do not depend on the "
-                                              "updated value; use dopt_amd.online.%s for this model" % rule)
+            skip.append(False)
+            if w not in projs:
+                continue
+            probe = float32(w.shape)
+            p = projs[w](probe)
+            nodes = core.topological_sort([p])
+            if not any(o is probe for o in nodes):
                 proj_ops.append((w, p))
-                skip.append(True)
+                skip[-1] = True
+            elif all(o is probe or o.opType != "variable" or id(o) not in step_nodes for o in nodes):
+                post.append((w, projs[w](w)))
             else:
-                skip.append(False)
+                raise NotImplementedError("fused updaters cannot order a projection that reads both the updated "
+                                          "value and other variables; use dopt_amd.online.%s for this model" % rule)
+        self._post_plan = core.compile([p for _, p in post], flags) if post else None
+        self._post_rets = [w.device_ptr()[0] for w, _ in post]
         self._proj = proj_ops
         self.plan = core.compile(list(outputs) + grads + [p for _, p in proj_ops], flags)
         self._out_bufs = [ops.Tensor(o.shape, o.dtype) for o in outputs]
@@ -150,6 +168,8 @@ class _FusedUpdater:
             self.opt.adam(h["alpha"], h["beta1"], h["beta2"], h["eps"])
         else:
             self.opt.amsgrad(h["alpha"], h["beta1"], h["beta2"], h["eps"])
+        if self._post_plan is not None:
+            self._post_plan.execute(None, self._post_rets)
 
     def __call__(self, args=None):
         self.step_async(args)
