@@ -45,6 +45,9 @@ PROTOTYPES = {
     "dopt_hip_copy_h2d": [_vp, _vp, _sz],
     "dopt_hip_copy_d2h": [_vp, _vp, _sz],
     "dopt_hip_copy_d2d": [_vp, _vp, _sz],
+    "dopt_hip_host_alloc": [C.POINTER(_vp), _sz],
+    "dopt_hip_host_free": [_vp],
+    "dopt_hip_copy_h2d_async": [_vp, _vp, _sz],
     "dopt_hip_copy_d2d_batch": [C.c_int, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_sz)],
     "dopt_hip_sync": [],
     "dopt_hip_event_create": [C.POINTER(_vp)],
@@ -75,6 +78,7 @@ PROTOTYPES = {
     "dopt_hip_bias_bwd": [_sz, _sz, _sz, _vp, _vp],
     "dopt_hip_uniform": [C.c_uint64, C.c_uint64, _sz, _vp],
     "dopt_hip_philox_raw": [C.c_uint64, C.c_uint64, _sz, _vp],
+    "dopt_hip_image_transform": [_sz, _sz, _sz, _sz, _sz, _sz, _vp, _vp, _vp],
     "dopt_hip_bn_train": [_sz, _sz, _sz, _d, _vp, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_bn_train_relu": [_sz, _sz, _sz, _d, _vp, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_bn_grad": [_sz, _sz, _sz, _vp, _vp, _vp, _vp],

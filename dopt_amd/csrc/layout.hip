@@ -298,6 +298,34 @@ int try_map32(int rank, const size_t *in_shape, const size_t *out_shape, const s
     return DOPT_HIP_OK;
 }
 
+// ---- image augmentation: mirrored pad, crop, flips -------------------------------------------
+// One lane per output pixel.  The source of output (y, x) is found backwards: undo the flips, add
+// the crop offset, subtract the pad, and mirror coordinates that fall outside the image about its
+// edge (edge pixel repeated, as the reference's reversed copies do).
+__global__ __launch_bounds__(kBlock) void image_transform_k(uint32_t total, uint32_t C, uint32_t H, uint32_t W,
+                                                            uint32_t magicW, uint32_t magicH, uint32_t magicC,
+                                                            int jx, int jy, const int32_t *geom, const float *in,
+                                                            float *out)
+{
+    const uint32_t idx = blockIdx.x * kBlock + threadIdx.x;
+    if (idx >= total) return;
+    uint32_t rest, x, y, c, n;
+    divmod32(idx, W, magicW, rest, x);
+    divmod32(rest, H, magicH, rest, y);
+    divmod32(rest, C, magicC, n, c);
+    const int xoff = geom[3 * n], yoff = geom[3 * n + 1], flags = geom[3 * n + 2];
+    int sx = (flags & 1) ? (int)(W - 1 - x) : (int)x;
+    int sy = (flags & 2) ? (int)(H - 1 - y) : (int)y;
+    sx += xoff - jx;
+    sy += yoff - jy;
+    sx = sx < 0 ? -sx - 1 : (sx >= (int)W ? 2 * (int)W - 1 - sx : sx);
+    sy = sy < 0 ? -sy - 1 : (sy >= (int)H ? 2 * (int)H - 1 - sy : sy);
+    // offsets come from device memory the host never saw: an out-of-range one must not become a stray read
+    sx = sx < 0 ? 0 : (sx >= (int)W ? (int)W - 1 : sx);
+    sy = sy < 0 ? 0 : (sy >= (int)H ? (int)H - 1 : sy);
+    out[idx] = in[((size_t)(n * C + c) * H + sy) * W + sx];
+}
+
 // ---- many small device-to-device copies in one launch -----------------------------------------
 constexpr int kBatchCopies = 48;
 struct CopyBatch {  // passed by value: no table to upload
@@ -400,6 +428,25 @@ int dopt_hip_repeat(int rank, const size_t *in_shape, const size_t *reps, const 
     fill_strides(d);
     hipLaunchKernelGGL(repeat_nd, dim3(grid_for(total)), dim3(kBlock), 0, stream(), d, total, (const uint32_t *)in,
                        (uint32_t *)out);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_image_transform(size_t N, size_t C, size_t H, size_t W, size_t jitterX, size_t jitterY,
+                             const int32_t *geom, const float *in, float *out)
+{
+    const size_t total = N * C * H * W;
+    if (total == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(geom && in && out, "dopt_hip_image_transform: null argument");
+    DOPT_REQUIRE(in != out, "dopt_hip_image_transform: the batch cannot be transformed in place");
+    DOPT_REQUIRE(total < (1ull << 32), "dopt_hip_image_transform: batch of %zu values is too large", total);
+    // one mirror image per side: the pad cannot be wider than the image it mirrors
+    DOPT_REQUIRE(jitterX <= W && jitterY <= H, "dopt_hip_image_transform: jitter (%zu, %zu) exceeds the image (%zu, %zu)",
+                 jitterX, jitterY, W, H);
+    DOPT_ENSURE_INIT();
+    hipLaunchKernelGGL(image_transform_k, dim3((unsigned)ceil_div(total, (size_t)kBlock)), dim3(kBlock), 0, stream(),
+                       (uint32_t)total, (uint32_t)C, (uint32_t)H, (uint32_t)W, recip32((uint32_t)W),
+                       recip32((uint32_t)H), recip32((uint32_t)C), (int)jitterX, (int)jitterY, geom, in, out);
     DOPT_LAUNCH_CHECK();
     return DOPT_HIP_OK;
 }

@@ -334,6 +334,38 @@ int dopt_hip_copy_h2d(void *dst, const void *host_src, size_t bytes)
     return DOPT_HIP_OK;
 }
 
+int dopt_hip_host_alloc(void **host_ptr, size_t bytes)
+{
+    DOPT_REQUIRE(host_ptr != nullptr, "dopt_hip_host_alloc: null argument");
+    DOPT_ENSURE_INIT();
+    *host_ptr = nullptr;
+    if (bytes == 0) return DOPT_HIP_OK;
+    if (hipHostMalloc(host_ptr, bytes, hipHostMallocDefault) != hipSuccess) {
+        (void)hipGetLastError();
+        *host_ptr = nullptr;
+        return fail(DOPT_HIP_ERR_OOM, "page-locked host allocation of %zu bytes failed", bytes);
+    }
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_host_free(void *host_ptr)
+{
+    if (!host_ptr) return DOPT_HIP_OK;
+    DOPT_ENSURE_INIT();
+    DOPT_HIP_CHECK(hipStreamSynchronize(stream()));   // a queued copy may still read it
+    DOPT_HIP_CHECK(hipHostFree(host_ptr));
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_copy_h2d_async(void *dst, const void *pinned_src, size_t bytes)
+{
+    if (bytes == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(dst && pinned_src, "dopt_hip_copy_h2d_async: null pointer");
+    DOPT_ENSURE_INIT();
+    DOPT_HIP_CHECK(hipMemcpyAsync(dst, pinned_src, bytes, hipMemcpyHostToDevice, stream()));
+    return DOPT_HIP_OK;
+}
+
 int dopt_hip_copy_d2h(void *host_dst, const void *src, size_t bytes)
 {
     if (bytes == 0) return DOPT_HIP_OK;

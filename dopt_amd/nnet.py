@@ -170,6 +170,20 @@ class DAGNetwork:   # nnet/networks.d:20-128
             self.paramLoss = float32([], [0.0])
 
 
+    def save(self, filename):   # nnet/networks.d:130-143: the parameters' float32 values, back to back, in order
+        with open(filename, "wb") as f:
+            for p in self.params:
+                f.write(np.ascontiguousarray(p.value, "<f4").tobytes())
+
+    def load(self, filename):   # nnet/networks.d:145-160
+        with open(filename, "rb") as f:
+            for p in self.params:
+                raw = f.read(p.volume * 4)
+                if len(raw) != p.volume * 4:
+                    raise IOError("%s ends before the parameter of shape %s" % (filename, list(p.shape)))
+                p.set_value(np.frombuffer(raw, "<f4").reshape(p.shape))
+
+
 def crossEntropy(hypothesis, ground_truth):   # nnet/losses.d:23-26
     return core.sum(ground_truth * log(hypothesis + 1e-6)) * (-1.0 / hypothesis.shape[0])
 

@@ -68,6 +68,15 @@ int dopt_hip_copy_h2d(void *dst, const void *host_src, size_t bytes);
 int dopt_hip_copy_d2h(void *host_dst, const void *src, size_t bytes);
 /* CUDABuffer.set(DeviceBuffer) -> cuMemcpyDtoD, cuda/package.d:187-190 */
 int dopt_hip_copy_d2d(void *dst, const void *src, size_t bytes);
+/* Page-locked host staging for the feed path.  The reference hands pageable `float[]` batches to
+   CUDABuffer.set each step (examples/cifar10.d:70-76 -> cuda/package.d:172-176, a blocking
+   cuMemcpyHtoD); a batch filled into memory from dopt_hip_host_alloc can instead be queued with
+   dopt_hip_copy_h2d_async, which returns at once: the copy runs in stream order before the kernels
+   queued after it, and the host may refill the same staging memory after the next dopt_hip_sync
+   (or keep two and alternate). */
+int dopt_hip_host_alloc(void **host_ptr, size_t bytes);
+int dopt_hip_host_free(void *host_ptr);
+int dopt_hip_copy_h2d_async(void *dst, const void *pinned_src, size_t bytes);
 /* n device-to-device copies, in order; copies of at most 64 KiB share kernel launches.  Stands
    for the loop of cuMemcpy calls that hands a plan's outputs to the caller's buffers
    (cuda/package.d:419-422): most of them are a few hundred bytes of batch-norm statistics. */
@@ -195,6 +204,16 @@ int dopt_hip_bias_bwd(size_t N, size_t C, size_t inner, const float *dy, float *
    generator's 32-bit words themselves (for known-answer tests of the generator). */
 int dopt_hip_uniform(uint64_t seed, uint64_t call, size_t n, float *out);
 int dopt_hip_philox_raw(uint64_t seed, uint64_t call, size_t n, uint32_t *out);
+
+/* Training-time image augmentation of nnet/data/imagetransformer.d:45-138 (ImageTransformer.getBatch),
+   which the reference runs on the host, one image at a time, before the batch is uploaded: pad by
+   (jitterY, jitterX) with the image mirrored about its edges, crop an H x W window at (yoff, xoff)
+   in the padded image, then reverse rows (flip X) and/or columns (flip Y).  Here the batch is
+   already on the device and one kernel writes every output pixel from its source pixel.
+   geom: N triples on the device {xoff in [0, 2*jitterX], yoff in [0, 2*jitterY], flags: bit 0 = flip
+   X, bit 1 = flip Y}; the caller draws them (the reference uses std.random on the host too). */
+int dopt_hip_image_transform(size_t N, size_t C, size_t H, size_t W, size_t jitterX, size_t jitterY,
+                             const int32_t *geom, const float *in, float *out);
 
 /* `batchNormTrain`: cudnnBatchNormalizationForwardTraining (spatial), cudnn7.d:608-610.
    packed = [ y (N*C*inner) | newRunMean (C) | newRunVar (C) ] as core/ops/nnet.d:222-225;

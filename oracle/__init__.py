@@ -310,3 +310,15 @@ def amsgrad_step(w, g, m, v, vhat, eta, beta1=0.9, beta2=0.999, eps=1e-8):
                                 C.c_float(eps), _p(w), _p(g), _p(m), _p(v), _p(vhat), _p(wo), _p(mo), _p(vo),
                                 _p(vho)), "amsgrad")
     return wo, mo, vo, vho
+
+
+def image_transform(batch, jitter_x, jitter_y, geom):
+    """ImageTransformer.getBatch on a [N, C, H, W] batch with the random draws given: geom is
+    [N, 3] int32 rows of (xOff, yOff, flip X | flip Y << 1)."""
+    out = _f32(batch).copy()
+    n, c, h, w = out.shape
+    g = np.ascontiguousarray(geom, np.int32).reshape(n, 3)
+    padded = np.zeros(c * (h + 2 * jitter_y) * (w + 2 * jitter_x), np.float32)
+    _chk(lib().ref_image_transform(*map(C.c_size_t, (n, c, h, w, jitter_x, jitter_y)), _p(g), _p(out), _p(padded)),
+         "image_transform")
+    return out

@@ -25,6 +25,8 @@
  *                      the nnet/layers/batchnorm.d:158-177 scenario (running mean -> [3,4])
  *   ref_sgd/adam/amsgrad  numpy float32 one-ufunc-per-node evaluation of the same trees +
  *                      the fit-a-line scenario of online/{sgd,adam,amsgrad}.d unittests
+ *   ref_image_transform  np.pad(mode="symmetric") + slicing + reversed views, every offset of a
+ *                      small image enumerated (the reference holds no test for this class)
  */
 #include "dopt_oracle.h"
 
@@ -822,4 +824,59 @@ int ref_amsgrad_step(size_t n, float eta, float beta1, float beta2, float eps, c
     /* vhat' = max(vhat, OLD v) is computed before v may be overwritten in place. */
     for (size_t i = 0; i < n; i++) vhatOut[i] = maxf_d(vhat[i], v[i]); /* amsgrad.d:63-66 */
     return ref_adam_step(n, eta, beta1, beta2, eps, w, g, m, v, wOut, mOut, vOut);
+}
+
+/* ---- nnet/data/imagetransformer.d:45-138 (ImageTransformer.getBatch), one image at a time ----
+ * The loops, the padded scratch image and the in-place reversals are the reference's; the random
+ * draws (xOff, yOff, the two coin flips) are arguments here.  `img` is transformed in place, as in
+ * the reference; `padded` holds C * (H + 2 jy) * (W + 2 jx) floats. */
+static void reverse_run(float *a, size_t n, size_t stride)
+{
+    for (size_t i = 0; i < n / 2; i++) {
+        float t = a[i * stride];
+        a[i * stride] = a[(n - 1 - i) * stride];
+        a[(n - 1 - i) * stride] = t;
+    }
+}
+
+int ref_image_transform(size_t N, size_t C, size_t H, size_t W, size_t jx, size_t jy,
+                        const int32_t *geom, float *batch, float *padded)
+{
+    const size_t pw = W + 2 * jx, ph = H + 2 * jy;
+    for (size_t n = 0; n < N; n++) {
+        float *img = batch + n * C * H * W;
+        const size_t xOff = (size_t)geom[3 * n], yOff = (size_t)geom[3 * n + 1];
+        const int flipX = geom[3 * n + 2] & 1, flipY = geom[3 * n + 2] & 2;
+        if (jx != 0 || jy != 0) {                                    /* :58 */
+            for (size_t c = 0; c < C; c++) {
+                for (size_t y = 0; y < H; y++) {
+                    for (size_t x = 0; x < W; x++)                   /* :65-69 */
+                        padded[c * ph * pw + (y + jy) * pw + x + jx] = img[c * H * W + y * W + x];
+                    if (jx != 0) {                                   /* :71-80 */
+                        size_t o = c * ph * pw + (y + jy) * pw;
+                        memcpy(padded + o, padded + o + jx, jx * sizeof(float));
+                        reverse_run(padded + o, jx, 1);
+                        o += W;
+                        memcpy(padded + o + jx, padded + o, jx * sizeof(float));
+                        reverse_run(padded + o + jx, jx, 1);
+                    }
+                }
+                for (size_t y = 0; y < jy; y++) {                    /* :83-94 */
+                    const size_t o = c * pw * ph;
+                    memcpy(padded + o + y * pw, padded + o + (2 * jy - y - 1) * pw, pw * sizeof(float));
+                    memcpy(padded + o + (ph - y - 1) * pw, padded + o + (ph - 2 * jy + y) * pw, pw * sizeof(float));
+                }
+            }
+            for (size_t c = 0; c < C; c++)                           /* :100-110 */
+                for (size_t y = 0; y < H; y++)
+                    for (size_t x = 0; x < W; x++)
+                        img[c * H * W + y * W + x] = padded[c * ph * pw + (y + yOff) * pw + x + xOff];
+        }
+        if (flipX)                                                   /* :113-119: every row of every channel */
+            for (size_t r = 0; r < C * H; r++) reverse_run(img + r * W, W, 1);
+        if (flipY)                                                   /* :121-132: every column of every channel */
+            for (size_t c = 0; c < C; c++)
+                for (size_t x = 0; x < W; x++) reverse_run(img + c * H * W + x, H, W);
+    }
+    return 0;
 }

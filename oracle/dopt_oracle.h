@@ -112,6 +112,10 @@ int ref_amsgrad_step(size_t n, float eta, float beta1, float beta2, float eps, c
                      const float *g, const float *m, const float *v, const float *vhat,
                      float *wOut, float *mOut, float *vOut, float *vhatOut);
 
+/* nnet/data/imagetransformer.d:45-138; geom = N x {xOff, yOff, bit 0 flip X | bit 1 flip Y}. */
+int ref_image_transform(size_t N, size_t C, size_t H, size_t W, size_t jx, size_t jy,
+                        const int32_t *geom, float *batch, float *padded);
+
 #ifdef __cplusplus
 }
 #endif
