@@ -752,6 +752,99 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
             });
             prebuiltLabel[id] = outT ? "matmul+transpose" : "matmul";
         }
+
+        // Pointwise chains: a pointwise operation whose value is read only by pointwise operations
+        // of one chain (and by no plan output) is computed inside that chain's kernel and never
+        // stored; an operand of the form repeat(one-element tensor) is read from the element itself.
+        // Walking consumers before producers, an operation joins the chain all its readers belong to
+        // or starts a chain of its own.
+        auto is_pw = [&](int id) {
+            const Operation &o = g.ops[id];
+            const int arity = dopt_hip_pointwise_arity(o.opType.c_str());
+            return live[id] && alias[id].source < 0 && !fusedKind[id] && o.dtype == DOPT_HIP_F32 && arity > 0 &&
+                   arity == (int)o.deps.size() && o.volume() > 0;
+        };
+        std::vector<int> chainOf((size_t)nops, -1);              // the operation that ends the chain
+        std::vector<std::vector<int>> chainOps((size_t)nops);    // per chain end: its members
+        for (auto it = p->mOps.rbegin(); it != p->mOps.rend(); ++it) {
+            const int id = *it;
+            if (!is_pw(id)) continue;
+            int target = -1;
+            bool joins = !isOutput(id) && !uses[id].empty();
+            for (const Use &u : uses[id]) {
+                if (!joins) break;
+                if (chainOf[u.op] < 0 || u.off != 0 || g.ops[u.op].volume() != g.ops[id].volume()) joins = false;
+                else if (target < 0) target = chainOf[u.op];
+                else if (target != chainOf[u.op]) joins = false;
+            }
+            if (joins && chainOps[target].size() >= 48) joins = false;
+            chainOf[id] = joins ? target : id;
+            chainOps[chainOf[id]].push_back(id);
+        }
+        for (int end : p->mOps) {
+            if (chainOf[end] != end || chainOps[end].size() < 2) continue;
+            std::vector<int> members;                             // in execution order
+            for (int id : p->mOps)
+                if (chainOf[id] == end) members.push_back(id);
+            std::vector<int> inputs;                              // operations whose buffers the kernel reads
+            std::vector<unsigned char> scalar;
+            std::vector<int> nodeOf((size_t)nops, -1);
+            struct Node { std::string op; int lhs, rhs; };
+            std::vector<Node> nodes;
+            std::vector<std::pair<int, int>> operands;            // per node slot: (is node, index) before renumbering
+            bool ok = true;
+            auto input_index = [&](int op, bool is_scalar) {
+                for (size_t k = 0; k < inputs.size(); k++)
+                    if (inputs[k] == op && scalar[k] == (unsigned char)is_scalar) return (int)k;
+                inputs.push_back(op);
+                scalar.push_back(is_scalar);
+                return (int)inputs.size() - 1;
+            };
+            for (int id : members) {
+                const Operation &o = g.ops[id];
+                int ref[2] = {-1, -1};
+                for (size_t j = 0; j < o.deps.size(); j++) {
+                    size_t off;
+                    const int r = root(o.deps[j], &off);
+                    if (chainOf[r] == end && nodeOf[r] >= 0 && off == 0) {
+                        ref[j] = -2 - nodeOf[r];                  // a node, renumbered once the inputs are known
+                        continue;
+                    }
+                    const Operation &ro = g.ops[r];
+                    size_t soff = 0;
+                    if (ro.opType == "repeat" && ro.deps.size() == 1 && off == 0 && alias[r].source < 0 &&
+                        g.ops[ro.deps[0]].volume() == 1 && g.ops[root(ro.deps[0], &soff)].dtype == DOPT_HIP_F32)
+                        ref[j] = input_index(ro.deps[0], true);
+                    else
+                        ref[j] = input_index(o.deps[j], false);
+                }
+                nodeOf[id] = (int)nodes.size();
+                nodes.push_back({o.opType, ref[0], ref[1]});
+            }
+            if (inputs.empty() || inputs.size() > 12) ok = false;
+            if (!ok) continue;                                    // too wide: its members keep their own kernels
+            const int nin = (int)inputs.size();
+            for (Node &n : nodes) {
+                if (n.lhs <= -2) n.lhs = nin + (-2 - n.lhs);
+                if (n.rhs <= -2) n.rhs = nin + (-2 - n.rhs);
+                if (n.rhs < 0) n.rhs = n.lhs;
+            }
+            for (int id : members) fusedKind[id] = 7;
+            inputsOf[end] = inputs;
+            const size_t count = g.ops[end].volume();
+            prebuilt[end] = make([=](const std::vector<const void *> &in, void *out) {
+                const char *names[64];
+                int lhs[64], rhs[64];
+                for (size_t j = 0; j < nodes.size(); j++) {
+                    names[j] = nodes[j].op.c_str();
+                    lhs[j] = nodes[j].lhs;
+                    rhs[j] = nodes[j].rhs;
+                }
+                return dopt_hip_pointwise_chain(DOPT_HIP_F32, count, nin, in.data(), scalar.data(), (int)nodes.size(), names,
+                                                lhs, rhs, out);
+            });
+            prebuiltLabel[end] = "pointwise*" + std::to_string(nodes.size());   // no spaces: profile lines are split on them
+        }
     }
 
     // addBiasGrad(dx of a batchNormGrad): the batch-norm kernel writes the bias gradient too.  The

@@ -159,6 +159,98 @@ std::string pointwise_source(const OpInfo &op, int dtype)
     return s;
 }
 
+// ------------------------------------------------------------------------------ pointwise chains
+// A DAG of pointwise nodes over equally long operands as ONE kernel: every node keeps its own
+// function (the same expression the stand-alone kernel of that op evaluates, compiled without
+// contraction), intermediate values stay in fp32 registers, so the result equals running the
+// nodes one kernel at a time bit for bit.  Operand k < nin is input k (a vector, or a one-element
+// tensor broadcast to every position); operand nin + j is node j.  Outputs: the last node.
+std::string chain_source(int dtype, int nin, const unsigned char *scalar, int nnodes, const OpInfo *const *ops,
+                         const int *lhs, const int *rhs)
+{
+    std::string s = dtype == DOPT_HIP_F32 ? "typedef float T;\n" : "typedef int T;\n";
+    s += "typedef T T4 __attribute__((ext_vector_type(4)));\n#define BLOCK 256\n";
+    s += R"SRC(
+__device__ inline int dopt_ipow(int x, int n)
+{
+    if (n < 0) {
+        if (x == 1) return 1;
+        if (x == -1) return (n & 1) ? -1 : 1;
+        return 0;
+    }
+    unsigned p = 1u, v = (unsigned)x, m = (unsigned)n;
+    while (m) {
+        if (m & 1u) p *= v;
+        m >>= 1;
+        v *= v;
+    }
+    return (int)p;
+}
+)SRC";
+    for (int j = 0; j < nnodes; j++)
+        s += "__device__ inline T f" + std::to_string(j) + "(T a, T b) { return (T)(" +
+             (dtype == DOPT_HIP_F32 ? ops[j]->expr_f32 : ops[j]->expr_i32) + "); }\n";
+    auto operand = [&](int k, const char *lane) -> std::string {
+        if (k >= nin) return "t" + std::to_string(k - nin);
+        if (scalar[k]) return "s" + std::to_string(k);
+        return "x" + std::to_string(k) + lane;
+    };
+    auto body = [&](const char *lane, const std::string &dst) {
+        std::string b = "        {\n";
+        for (int j = 0; j < nnodes; j++) {
+            const std::string a = operand(lhs[j], lane), c = ops[j]->arity == 2 ? operand(rhs[j], lane) : a;
+            b += "            const T t" + std::to_string(j) + " = f" + std::to_string(j) + "(" + a + ", " + c + ");\n";
+        }
+        b += "            " + dst + " = t" + std::to_string(nnodes - 1) + ";\n        }\n";
+        return b;
+    };
+    std::string params = "size_t n";
+    for (int k = 0; k < nin; k++) params += ", const T *i" + std::to_string(k);
+    params += ", T *o";
+    std::string scalars;
+    for (int k = 0; k < nin; k++)
+        if (scalar[k]) scalars += "    const T s" + std::to_string(k) + " = i" + std::to_string(k) + "[0];\n";
+
+    // quads: two independent 128-bit loads per operand and lane in flight
+    s += "extern \"C\" __global__ __launch_bounds__(BLOCK) void chain_vec(" + params + ")\n{\n" + scalars;
+    s += "    const size_t n4 = n >> 2;\n";
+    s += "    for (size_t base = (size_t)blockIdx.x * (BLOCK * 2) + threadIdx.x; base < n4; base += (size_t)gridDim.x * (BLOCK * 2)) {\n";
+    s += "        const size_t second = base + BLOCK < n4 ? base + BLOCK : base;\n";
+    for (int k = 0; k < nin; k++)
+        if (!scalar[k]) {
+            const std::string i = std::to_string(k);
+            s += "        const T4 x" + i + " = ((const T4 *)i" + i + ")[base], y" + i + " = ((const T4 *)i" + i + ")[second];\n";
+        }
+    s += "        T4 r, q;\n";
+    for (const char *lane : {".x", ".y", ".z", ".w"}) s += body(lane, std::string("r") + lane);
+    // the second quad: the same code over y instead of x
+    {
+        std::string second;
+        for (const char *lane : {".x", ".y", ".z", ".w"}) second += body(lane, std::string("q") + lane);
+        for (int k = 0; k < nin; k++) {
+            if (scalar[k]) continue;
+            const std::string from = "x" + std::to_string(k) + ".", to = "y" + std::to_string(k) + ".";
+            for (size_t at = second.find(from); at != std::string::npos; at = second.find(from, at + to.size()))
+                second.replace(at, from.size(), to);
+        }
+        s += second;
+    }
+    s += "        ((T4 *)o)[base] = r;\n        if (second != base) ((T4 *)o)[second] = q;\n    }\n";
+    s += "    if (blockIdx.x == 0) {\n        const size_t i = (n4 << 2) + threadIdx.x;\n        if (i < n) {\n";
+    for (int k = 0; k < nin; k++)
+        if (!scalar[k]) s += "            const T x" + std::to_string(k) + " = i" + std::to_string(k) + "[i];\n";
+    s += body("", "o[i]");
+    s += "        }\n    }\n}\n";
+
+    s += "extern \"C\" __global__ __launch_bounds__(BLOCK) void chain_scalar(" + params + ")\n{\n" + scalars;
+    s += "    for (size_t i = (size_t)blockIdx.x * BLOCK + threadIdx.x; i < n; i += (size_t)gridDim.x * BLOCK) {\n";
+    for (int k = 0; k < nin; k++)
+        if (!scalar[k]) s += "        const T x" + std::to_string(k) + " = i" + std::to_string(k) + "[i];\n";
+    s += body("", "o[i]");
+    s += "    }\n}\n";
+    return s;
+}
+
 // ------------------------------------------------------------------------------ reductions
 
 const char *kReduceBody = R"SRC(
@@ -426,6 +518,75 @@ int dopt_hip_pointwise(const char *op, int dtype, size_t n, const void *a, const
     unsigned grid = vec ? grid_for(256 * 4, ceil_div(n, 4)) : grid_for(256, n);
     void *args[] = {(void *)&n, (void *)&a, (void *)&bb, (void *)&out};
     return rtc_launch(fn, grid, 256, args);
+}
+
+// Checks a chain description and produces its cache key and source.
+static int chain_prepare(int dtype, int nin, const unsigned char *in_is_scalar, int nnodes, const char *const *node_op,
+                         const int *node_lhs, const int *node_rhs, std::string *key, std::string *source)
+{
+    DOPT_REQUIRE(nin >= 1 && nin <= 16 && nnodes >= 1 && nnodes <= 64, "dopt_hip_pointwise_chain: %d inputs, %d nodes", nin,
+                 nnodes);
+    DOPT_REQUIRE(in_is_scalar && node_op && node_lhs && node_rhs, "dopt_hip_pointwise_chain: null argument");
+    if (int rc = check_dtype(dtype)) return rc;
+    const OpInfo *ops[64];
+    *key = dtype == DOPT_HIP_F32 ? "chain:f32" : "chain:i32";
+    for (int k = 0; k < nin; k++) *key += in_is_scalar[k] ? ":s" : ":v";
+    for (int j = 0; j < nnodes; j++) {
+        DOPT_REQUIRE(node_op[j] != nullptr, "dopt_hip_pointwise_chain: node %d has no operation", j);
+        ops[j] = find_op(node_op[j]);
+        if (!ops[j]) return fail(DOPT_HIP_ERR_UNSUPPORTED, "dopt_hip_pointwise_chain: unknown operation '%s'", node_op[j]);
+        const int limit = nin + j;   // a node may only read inputs and earlier nodes
+        DOPT_REQUIRE(node_lhs[j] >= 0 && node_lhs[j] < limit && (ops[j]->arity == 1 || (node_rhs[j] >= 0 && node_rhs[j] < limit)),
+                     "dopt_hip_pointwise_chain: node %d reads an operand that is not computed before it", j);
+        *key += std::string("|") + node_op[j] + "," + std::to_string(node_lhs[j]) + "," +
+                std::to_string(ops[j]->arity == 2 ? node_rhs[j] : -1);
+    }
+    *source = chain_source(dtype, nin, in_is_scalar, nnodes, ops, node_lhs, node_rhs);
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_pointwise_chain(int dtype, size_t n, int nin, const void *const *in, const unsigned char *in_is_scalar,
+                             int nnodes, const char *const *node_op, const int *node_lhs, const int *node_rhs, void *out)
+{
+    std::string key, source;
+    if (int rc = chain_prepare(dtype, nin, in_is_scalar, nnodes, node_op, node_lhs, node_rhs, &key, &source)) return rc;
+    if (n == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(in && out, "dopt_hip_pointwise_chain: null argument");
+    bool vec = aligned16(out);
+    for (int k = 0; k < nin; k++) {
+        DOPT_REQUIRE(in[k] != nullptr, "dopt_hip_pointwise_chain: input %d is null", k);
+        vec = vec && (in_is_scalar[k] || aligned16(in[k]));
+    }
+    DOPT_ENSURE_INIT();
+    const char *kname = vec ? "chain_vec" : "chain_scalar";
+    hipFunction_t fn;
+    if (int rc = rtc_get(key + ":" + kname, source, kname, &fn)) return rc;
+    const void *ptrs[16];
+    void *args[18];
+    args[0] = (void *)&n;
+    for (int k = 0; k < nin; k++) {
+        ptrs[k] = in[k];
+        args[1 + k] = (void *)&ptrs[k];
+    }
+    args[1 + nin] = (void *)&out;
+    unsigned grid = vec ? grid_for(256 * 2, ceil_div(n, 4)) : grid_for(256, n);
+    return rtc_launch(fn, grid, 256, args);
+}
+
+int dopt_hip_pointwise_chain_compile_only(int dtype, int nin, const unsigned char *in_is_scalar, int nnodes,
+                                          const char *const *node_op, const int *node_lhs, const int *node_rhs,
+                                          const char *arch)
+{
+    DOPT_REQUIRE(arch != nullptr, "dopt_hip_pointwise_chain_compile_only: null argument");
+    std::string key, source;
+    if (int rc = chain_prepare(dtype, nin, in_is_scalar, nnodes, node_op, node_lhs, node_rhs, &key, &source)) return rc;
+    return rtc_compile_only(source, arch, nullptr);
+}
+
+int dopt_hip_pointwise_arity(const char *op)
+{
+    const OpInfo *info = op ? find_op(op) : nullptr;
+    return info ? info->arity : 0;
 }
 
 int dopt_hip_reduce(const char *op, int dtype, const size_t *shape, int rank, const size_t *axes, int naxes,

@@ -104,6 +104,22 @@ int dopt_hip_event_destroy(void *event);
            (b == NULL).  The reference's CUDA backend sends everything after sqrt to a host
            round trip (cuda/package.d:81-119); here they run on the device. */
 int dopt_hip_pointwise(const char *op, int dtype, size_t n, const void *a, const void *b_or_null, void *out);
+/* A DAG of pointwise nodes over n-element operands as one kernel.  The reference has no counterpart:
+   it launches one generated kernel per node (cuda/math.d:129-205) and its operator sugar broadcasts
+   a scalar by materialising `repeat(scalar, n)` first (core/ops/package.d:94-168).  Operand index
+   k < nin is input k - an n-element tensor, or, where in_is_scalar[k] is set, a one-element tensor
+   read at every position; index nin + j is the value of node j.  A node reads only inputs and
+   earlier nodes; unary nodes ignore node_rhs.  The last node's value is written to `out`.  Every
+   node is rounded to its own fp32 result exactly as the stand-alone kernel of that op rounds it. */
+int dopt_hip_pointwise_chain(int dtype, size_t n, int nin, const void *const *in,
+                             const unsigned char *in_is_scalar, int nnodes, const char *const *node_op,
+                             const int *node_lhs, const int *node_rhs, void *out);
+/* Generates and compiles the kernel of such a chain for `arch` without loading it (no GPU needed). */
+int dopt_hip_pointwise_chain_compile_only(int dtype, int nin, const unsigned char *in_is_scalar,
+                                          int nnodes, const char *const *node_op, const int *node_lhs,
+                                          const int *node_rhs, const char *arch);
+/* 1 or 2 for the names dopt_hip_pointwise accepts, 0 otherwise. */
+int dopt_hip_pointwise_arity(const char *op);
 
 /* `sum` / `maxElement` (op = "sum" | "maxElement"): cpu/math.d:90-247, reached in the reference through
    the host fallback cuda/package.d:81-119.  Reduces `axes` (distinct, each < rank) of a dense

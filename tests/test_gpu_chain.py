@@ -1,0 +1,109 @@
+"""Pointwise chains: one generated kernel against the same nodes run one kernel at a time (which the
+pointwise tests pin against the oracle), bit for bit; and plans that fuse such chains against plans
+that do not."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from dopt_amd import capi, core, nnet, online, ops
+
+pytestmark = pytest.mark.gpu
+T = ops.tensor
+
+
+def _one_by_one(inputs, nodes):
+    vals = list(inputs)
+    n = max(t.size for t in inputs)
+    full = next(t for t in inputs if t.size == n)
+    for i, t in enumerate(vals):
+        if t.size != n:
+            vals[i] = T(np.full(full.shape, t.numpy().ravel()[0], t.dtype))
+    for op, lhs, rhs in nodes:
+        vals.append(ops.pointwise(op, vals[lhs], None if rhs is None else vals[rhs]))
+    return vals[-1].numpy()
+
+
+CHAINS = [
+    # w - lr * g with lr a one-element tensor (the SGD update of online/sgd.d:58-63)
+    ([(1000,), (1,), (1000,)], [("mul", 1, 2), ("sub", 0, 3)]),
+    # beta2 * v + (1 - beta2) * g * g                       (online/adam.d:56)
+    ([(4099,), (4099,), (1,), (1,)], [("mul", 2, 0), ("mul", 3, 1), ("mul", 5, 1), ("add", 4, 6)]),
+    # w - eta * (m / (sqrt(v) + eps))                        (online/adam.d:58-60)
+    ([(513,), (513,), (513,), (1,), (1,)], [("sqrt", 2, None), ("add", 5, 4), ("div", 1, 6), ("mul", 3, 7), ("sub", 0, 8)]),
+    # a diamond: the same node read twice, comparisons and max in the mix
+    ([(33, 65), (33, 65)], [("add", 0, 1), ("mul", 2, 2), ("exp", 0, None), ("max", 3, 4), ("gt", 5, 1), ("mul", 6, 5),
+                            ("tanh", 7, None)]),
+    ([(7,)], [("neg", 0, None), ("abs", 1, None)]),
+    ([(1 << 20,), (1 << 20,), (1,)], [("div", 0, 2), ("log", 3, None), ("atan2", 4, 1), ("min", 5, 0)]),
+]
+
+
+@pytest.mark.parametrize("shapes,nodes", CHAINS)
+def test_chain_equals_the_nodes_run_one_by_one(shapes, nodes):
+    r = np.random.default_rng(len(nodes))
+    inputs = [T((np.abs(r.standard_normal(s)) + 0.5).astype(np.float32)) for s in shapes]
+    got = ops.pointwise_chain(inputs, nodes).numpy()
+    want = _one_by_one(inputs, nodes)
+    assert np.array_equal(got, want, equal_nan=True)
+
+
+def test_chain_unaligned_operands_and_int32():
+    r = np.random.default_rng(0)
+    base = T(r.standard_normal(1003).astype(np.float32))
+    a, b = base.view(1, [1001]), base.view(2, [1001])          # 4- and 8-byte offsets: the scalar kernel
+    nodes = [("mul", 0, 1), ("add", 2, 0)]
+    assert np.array_equal(ops.pointwise_chain([a, b], nodes).numpy(), _one_by_one([a, b], nodes))
+    ia, ib = T(r.integers(-50, 50, 300).astype(np.int32)), T(r.integers(0, 5, 300).astype(np.int32))
+    nodes = [("pow", 0, 1), ("mul", 2, 0), ("sub", 3, 1)]
+    assert np.array_equal(ops.pointwise_chain([ia, ib], nodes).numpy(), _one_by_one([ia, ib], nodes))
+
+
+def test_chain_rejects_forward_references_and_unknown_ops():
+    a = T(np.ones(8, np.float32))
+    with pytest.raises(capi.HipError):
+        ops.pointwise_chain([a], [("add", 0, 2), ("neg", 0, None)])
+    with pytest.raises(capi.HipError):
+        ops.pointwise_chain([a], [("frobnicate", 0, 0)])
+    assert capi.load().dopt_hip_pointwise_arity(b"atan2") == 2
+    assert capi.load().dopt_hip_pointwise_arity(b"sqrt") == 1
+    assert capi.load().dopt_hip_pointwise_arity(b"matmul") == 0
+
+
+def _mlp(seed):
+    init = nnet.Init(seed)
+    x, y = core.float32([32, 20]), core.float32([32, 5])
+    top = nnet.softmax(nnet.dense(nnet.relu(nnet.dense(nnet.dataSource(x), 16, init, weight_decay=1e-3)), 5, init))
+    net = nnet.DAGNetwork([x], [top])
+    return x, y, net, nnet.crossEntropy(top.trainOutput, y) + net.paramLoss
+
+
+@pytest.mark.parametrize("maker", [online.sgd, online.adam, online.amsgrad])
+def test_op_graph_optimizers_fuse_their_update_rules_without_changing_a_bit(maker):
+    r = np.random.default_rng(1)
+    xs = r.standard_normal((32, 20)).astype(np.float32)
+    ys = np.eye(5, dtype=np.float32)[r.integers(0, 5, 32)]
+    runs, kernels = [], []
+    for flags in (0, core.PLAN_VIEWS | core.PLAN_FUSE):
+        x, y, net, loss = _mlp(3)
+        up = maker([loss], net.params, net.paramProj, flags=flags)
+        losses = [up({x: xs, y: ys})[0] for _ in range(4)]
+        runs.append((losses, [p.value for p in net.params]))
+        kernels.append(up.plan.stats()["kernels"])
+    assert kernels[1] < kernels[0] * 0.7
+    for a, b in zip(runs[0][0], runs[1][0]):
+        assert a == b
+    for a, b in zip(runs[0][1], runs[1][1]):
+        assert np.array_equal(a, b)
+
+
+def test_chain_keeps_values_that_something_else_reads():
+    a = core.float32([64], np.arange(64, dtype=np.float32))
+    b = core.float32([64], np.ones(64, np.float32))
+    s = a + b                      # read by the chain AND returned
+    t = core.exp(s * 0.5) - b
+    u = core.sum(s)                # a reduction reads s too
+    want = core.compile([t, s, u]).execute()
+    got = core.compile([t, s, u], core.PLAN_VIEWS | core.PLAN_FUSE).execute()
+    for g, w in zip(got, want):
+        assert np.array_equal(g, w)

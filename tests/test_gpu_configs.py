@@ -256,3 +256,36 @@ def test_config5_wrn_block_step_matches_the_oracle():
         assert np.array_equal(a, b), k
     rm1 = O.bn_train(X, P["g1"], P["b1"], P["rm1"], P["rv1"], 0.9)[X.size:X.size + cin]
     assert_close(after[0][names.index("rm1")], rm1, "running mean after the step")
+
+
+# ------------------------------------------------------------------------------ evaluation path
+@pytest.mark.parametrize("flags", [0, core.PLAN_VIEWS | core.PLAN_FUSE])
+def test_eval_plan_uses_running_statistics(flags):
+    """examples/cifar10.d:84-87 compiles a second plan on the layers' `output` (batchNormInference,
+    dropout scaled instead of sampled).  After a few training steps the running statistics differ from
+    their initial values; the test plan must normalise with them, not with batch statistics."""
+    init = nnet.Init(5)
+    x, y = float32([16, 3, 8, 8]), float32([16, 10])
+    l1 = nnet.relu(nnet.batchNorm(nnet.conv2D(nnet.dataSource(x), 8, (3, 3), init, padding=(1, 1))))
+    l2 = nnet.dropout(nnet.maxPool(l1, (2, 2)), 0.25)
+    top = nnet.softmax(nnet.dense(l2, 10, init))
+    net = nnet.DAGNetwork([x], [top])
+    loss = nnet.crossEntropy(top.trainOutput, y) + net.paramLoss
+    r = np.random.default_rng(0)
+    xs = r.standard_normal((16, 3, 8, 8)).astype(np.float32)
+    ys = np.eye(10, dtype=np.float32)[r.integers(0, 10, 16)]
+    up = online.fused_sgd([loss], net.params, net.paramProj, 0.05, flags=flags)
+    for _ in range(4):
+        up({x: xs, y: ys})
+    w, b, gamma, beta, mean, var, wd, bd = [p.value for p in net.params]
+    assert np.abs(mean).max() > 1e-3 and np.abs(var - 1).max() > 1e-3
+
+    test_plan = core.compile([top.output], flags)
+    xt = r.standard_normal((16, 3, 8, 8)).astype(np.float32)
+    got, = test_plan.execute({x: xt})
+    h = O.add_bias(O.convolution(xt, w, (1, 1), (1, 1)), b)
+    h = O.relu(O.bn_infer(h, gamma.ravel(), beta, mean, var))
+    h = O.maxpool(h, (2, 2)) * np.float32(0.75)
+    z = (h.reshape(16, -1).astype(np.float64) @ wd.astype(np.float64).T + bd).astype(np.float32)
+    assert_close(got, O.softmax(z, f64=True), "eval plan")
+    assert np.array_equal(got, test_plan.execute({x: xt})[0])   # no sampling on the eval path
