@@ -153,7 +153,8 @@ def main():
         fwd = sum(conv_flops(BATCH, c, k, h) for c, k, h in VGG_CONVS)
         bwd_data = fwd - conv_flops(BATCH, *VGG_CONVS[0])   # the first layer's input needs no gradient
         conv_keys = [k for k in ("convolution", "convolution+addBias", "convolutionFeaturesGrad") if k in per_step]
-        gather_us = sum(per_step[k][0] for k in conv_keys)
+        # the one launch that packs every filter of the step belongs to these convolutions' cost
+        gather_us = sum(per_step[k][0] for k in conv_keys) + per_step.get("filterPack", (0.0, 0))[0]
         gather_launches = sum(per_step[k][1] for k in conv_keys)
         gather_tflops = (fwd + bwd_data) / (gather_us * 1e-6) / 1e12
         wgrad_tflops = fwd / (per_step["convolutionFiltersGrad"][0] * 1e-6) / 1e12

@@ -72,6 +72,9 @@ PROTOTYPES = {
     "dopt_hip_conv_fwd": [C.POINTER(ConvDesc), _vp, _vp, _vp],
     "dopt_hip_conv_fwd_bias": [C.POINTER(ConvDesc), _vp, _vp, _vp, _vp],
     "dopt_hip_conv_bwd_data": [C.POINTER(ConvDesc), _vp, _vp, _vp],
+    "dopt_hip_conv_pack_batch": [_i, C.POINTER(ConvDesc), C.POINTER(_i), C.POINTER(_vp), C.POINTER(_vp)],
+    "dopt_hip_conv_fwd_bias_packed": [C.POINTER(ConvDesc), _vp, _vp, _vp, _vp],
+    "dopt_hip_conv_bwd_data_packed": [C.POINTER(ConvDesc), _vp, _vp, _vp],
     "dopt_hip_conv_bwd_filter": [C.POINTER(ConvDesc), _vp, _vp, _vp],
     "dopt_hip_maxpool_fwd": [_sz, _sz, _sz, _sz, _sz, _sz, _vp, _vp],
     "dopt_hip_maxpool_bwd": [_sz, _sz, _sz, _sz, _sz, _sz, _vp, _vp, _vp],
@@ -99,6 +102,7 @@ PROTOTYPES = {
 _SPECIAL = {
     "dopt_hip_last_error": ([], C.c_char_p),
     "dopt_hip_stream": ([], _vp),
+    "dopt_hip_conv_packed_bytes": ([C.POINTER(ConvDesc), _i], _sz),
 }
 
 _lib = None

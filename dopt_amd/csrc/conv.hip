@@ -410,12 +410,10 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_patch_k(Pat
 // once; the scattered side of the transposition is the LDS read, whose strides spread the lanes
 // over the banks.
 template <bool kBwd>
-__global__ __launch_bounds__(256) void pack_patch_k(int M, int Cred, int Mp, size_t sm, size_t sc, const float *w,
-                                                     float *wp)
+__device__ __forceinline__ void pack_tile(int M, int Cred, int Mp, size_t sm, size_t sc, const float *w, float *wp,
+                                          int chunk, int m0, float *stage)
 {
     constexpr int PITCH = kBwd ? 148 : 145;  // floats between runs in LDS
-    __shared__ float stage[16 * PITCH];
-    const int chunk = blockIdx.y, m0 = blockIdx.x * 16;
     float v[9];
 #pragma unroll
     for (int i = 0; i < 9; i++) {
@@ -451,6 +449,41 @@ __global__ __launch_bounds__(256) void pack_patch_k(int M, int Cred, int Mp, siz
         }
         *(float4 *)&wp[(((size_t)chunk * 9 + tap) * Mp + m0 + ml) * 16 + j4 * 4] = q;
     }
+}
+
+template <bool kBwd>
+__global__ __launch_bounds__(256) void pack_patch_k(int M, int Cred, int Mp, size_t sm, size_t sc, const float *w,
+                                                     float *wp)
+{
+    __shared__ float stage[16 * 148];
+    pack_tile<kBwd>(M, Cred, Mp, sm, sc, w, wp, blockIdx.y, blockIdx.x * 16, stage);
+}
+
+// The filters of many layers in one launch (a training step packs each filter twice, once per
+// direction, and most of those launches are far too small to fill the chip on their own).
+constexpr int kPackJobs = 32;
+struct PackJob {
+    const float *w;
+    float *wp;
+    int M, Cred, Mp, bwd;
+    unsigned sm, sc;
+    unsigned first_block, mblocks;   // blocks [first_block, next job's first_block): (chunk, row block) pairs
+};
+struct PackBatch {
+    PackJob job[kPackJobs];
+    int njobs;
+};
+
+__global__ __launch_bounds__(256) void pack_batch_k(PackBatch b)
+{
+    __shared__ float stage[16 * 148];
+    int j = 0;
+    while (j + 1 < b.njobs && blockIdx.x >= b.job[j + 1].first_block) j++;
+    const PackJob &q = b.job[j];
+    const unsigned local = blockIdx.x - q.first_block;
+    const int chunk = (int)(local / q.mblocks), m0 = (int)(local % q.mblocks) * 16;
+    if (q.bwd) pack_tile<true>(q.M, q.Cred, q.Mp, q.sm, q.sc, q.w, q.wp, chunk, m0, stage);
+    else pack_tile<false>(q.M, q.Cred, q.Mp, q.sm, q.sc, q.w, q.wp, chunk, m0, stage);
 }
 
 // ------------------------------------------------------------------------------------ backward-filter
@@ -1087,13 +1120,22 @@ int launch_patch(const PatchConv &pc, bool c_full, dim3 grid, size_t lds_bytes)
 
 // 3x3 unit-stride layers whose pixel tiles are whole rows of one image or whole images.
 // Returns DOPT_HIP_OK with *done = false when the layer does not fit this path.
+// What the patch kernel needs to know about one convolution, without any pointer: which tile
+// shape runs it and how its filter is packed.  `ok` is false when the generic kernel takes the shape.
+struct PatchSetup {
+    bool ok;
+    PatchConv pc;
+    int shape;            // 0 wide, 1 square, 2 deep
+    int BM, BN, blocks_wanted, tiles;
+    size_t lds_bytes, wp_elems;
+};
+
 template <bool kBwd>
-int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, const float *w, const float *bias,
-              float *out, bool *done)
+PatchSetup patch_setup(const dopt_hip_conv_desc *d, size_t P, size_t Q)
 {
-    *done = false;
-    if (d->R != 3 || d->S != 3 || d->strideH != 1 || d->strideW != 1 || d->padH > 2 || d->padW > 2) return DOPT_HIP_OK;
-    PatchConv pc{};
+    PatchSetup u{};
+    if (d->R != 3 || d->S != 3 || d->strideH != 1 || d->strideW != 1 || d->padH > 2 || d->padW > 2) return u;
+    PatchConv &pc = u.pc;
     pc.N = (int)d->N;
     if (!kBwd) {
         pc.Cin = (int)d->C; pc.IH = (int)d->H; pc.IW = (int)d->W;
@@ -1105,31 +1147,31 @@ int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, 
         pc.PT = 2 - (int)d->padH; pc.PL = 2 - (int)d->padW; pc.flip = 0;
     }
     pc.ncols = pc.N * pc.OH * pc.OW;
-    enum { kWide, kSquare, kDeep } shape;
-    int BM, BN, blocks_wanted, npmax, threads;
+    int npmax, threads;
     if (pc.Mout <= 64) {
-        shape = kWide; BM = 64; BN = 256; blocks_wanted = 2 * num_cus(); npmax = 24; threads = 256;
+        u.shape = 0; u.BM = 64; u.BN = 256; u.blocks_wanted = 2 * num_cus(); npmax = 24; threads = 256;
     } else {
-        BM = 128; BN = 128;
+        u.BM = 128; u.BN = 128;
         const int t = ((pc.Mout + 127) / 128) * ((pc.ncols + 127) / 128);
-        if (t >= 2 * num_cus()) { shape = kSquare; blocks_wanted = 2 * num_cus(); npmax = 16; threads = 256; }
-        else { shape = kDeep; blocks_wanted = num_cus(); npmax = 16; threads = 512; }
+        if (t >= 2 * num_cus()) { u.shape = 1; u.blocks_wanted = 2 * num_cus(); npmax = 16; threads = 256; }
+        else { u.shape = 2; u.blocks_wanted = num_cus(); npmax = 16; threads = 512; }
     }
+    const int BM = u.BM, BN = u.BN;
     // pixel tile = `rows` full rows of one image, or `nimg` whole images
-    if (BN % pc.OW != 0) return DOPT_HIP_OK;
+    if (BN % pc.OW != 0) return u;
     const int tile_rows = BN / pc.OW;
     if (tile_rows <= pc.OH) {
-        if (pc.OH % tile_rows != 0) return DOPT_HIP_OK;
+        if (pc.OH % tile_rows != 0) return u;
         pc.nimg = 1; pc.rows = tile_rows;
     } else {
-        if (tile_rows % pc.OH != 0) return DOPT_HIP_OK;
+        if (tile_rows % pc.OH != 0) return u;
         pc.nimg = tile_rows / pc.OH; pc.rows = pc.OH;
     }
     pc.PR = pc.rows + 2; pc.PC = pc.OW + 2;
     pc.psz = pc.nimg * pc.PR * pc.PC;
-    if ((size_t)pc.psz * 16 > (size_t)npmax * threads) return DOPT_HIP_OK;
-    const size_t lds_bytes = ((size_t)2 * BM * 20 + (size_t)2 * (pc.psz + 1) * 20) * sizeof(float);
-    if (lds_bytes > 160 * 1024) return DOPT_HIP_OK;
+    if ((size_t)pc.psz * 16 > (size_t)npmax * threads) return u;
+    u.lds_bytes = ((size_t)2 * BM * 20 + (size_t)2 * (pc.psz + 1) * 20) * sizeof(float);
+    if (u.lds_bytes > 160 * 1024) return u;
     pc.magic_psz = div_magic((unsigned)pc.psz);
     pc.magic_img = div_magic((unsigned)(pc.PR * pc.PC));
     pc.magic_pc = div_magic((unsigned)pc.PC);
@@ -1138,9 +1180,38 @@ int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, 
     pc.Mp = pc.mtiles * BM;
     pc.chunks_total = (pc.Cin + 15) / 16;
     pc.out_elems = (size_t)pc.ncols * pc.Mout;
-    const int tiles = pc.mtiles * pc.ntiles;
+    u.tiles = pc.mtiles * pc.ntiles;
+    u.wp_elems = (size_t)pc.chunks_total * 9 * pc.Mp * 16;
+    u.ok = true;
+    return u;
+}
+
+template <bool kBwd>
+PackJob pack_job(const dopt_hip_conv_desc *d, const PatchSetup &u, const float *w, float *wp)
+{
+    const unsigned C9 = (unsigned)(d->C * 9);
+    PackJob j{};
+    j.w = w; j.wp = wp;
+    j.M = u.pc.Mout; j.Cred = u.pc.Cin; j.Mp = u.pc.Mp; j.bwd = kBwd;
+    j.sm = kBwd ? 9u : C9;
+    j.sc = kBwd ? C9 : 9u;
+    j.mblocks = (unsigned)(u.pc.Mp / 16);
+    return j;
+}
+
+// `prepacked`: the filter already in the kernel's layout (dopt_hip_conv_pack_batch), or null to
+// pack it here first.
+template <bool kBwd>
+int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, const float *w, const float *bias,
+              float *out, bool *done, const float *prepacked = nullptr)
+{
+    *done = false;
+    PatchSetup u = patch_setup<kBwd>(d, P, Q);
+    if (!u.ok) return DOPT_HIP_OK;
+    PatchConv &pc = u.pc;
+    const int tiles = u.tiles;
     // never a grid slightly above what is resident at once: a second round of blocks would run nearly empty
-    int splits = tiles >= blocks_wanted ? 1 : blocks_wanted / tiles;
+    int splits = tiles >= u.blocks_wanted ? 1 : u.blocks_wanted / tiles;
     if (splits > pc.chunks_total) splits = pc.chunks_total;
     if (splits > 64) splits = 64;
     if (pc.out_elems % 4 != 0 || !aligned16(out)) splits = 1;
@@ -1148,34 +1219,33 @@ int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, 
     splits = (pc.chunks_total + pc.chunks_per_split - 1) / pc.chunks_per_split;
     pc.splits = splits;
 
-    const size_t wp_elems = (size_t)pc.chunks_total * 9 * pc.Mp * 16;
-    const size_t wp_bytes = (wp_elems * sizeof(float) + 255) / 256 * 256;
+    const size_t wp_bytes = prepacked ? 0 : (u.wp_elems * sizeof(float) + 255) / 256 * 256;
     const size_t part_bytes = splits > 1 ? (size_t)splits * pc.out_elems * sizeof(float) : 0;
-    char *ws = (char *)workspace(wp_bytes + part_bytes);
-    if (!ws) return DOPT_HIP_ERR_OOM;
-    float *wp = (float *)ws;
+    char *ws = wp_bytes + part_bytes > 0 ? (char *)workspace(wp_bytes + part_bytes) : nullptr;
+    if (wp_bytes + part_bytes > 0 && !ws) return DOPT_HIP_ERR_OOM;
     float *partial = (float *)(ws + wp_bytes);
-    {
-        const size_t C9 = (size_t)d->C * 9;
-        const dim3 pgrid((unsigned)(pc.Mp / 16), (unsigned)pc.chunks_total);
-        if (!kBwd) hipLaunchKernelGGL(pack_patch_k<false>, pgrid, dim3(256), 0, stream(), pc.Mout, pc.Cin, pc.Mp, C9,
-                                      (size_t)9, w, wp);
-        else hipLaunchKernelGGL(pack_patch_k<true>, pgrid, dim3(256), 0, stream(), pc.Mout, pc.Cin, pc.Mp, (size_t)9, C9,
-                                w, wp);
+    if (!prepacked) {
+        const PackJob j = pack_job<kBwd>(d, u, w, (float *)ws);
+        const dim3 pgrid(j.mblocks, (unsigned)pc.chunks_total);
+        if (!kBwd) hipLaunchKernelGGL(pack_patch_k<false>, pgrid, dim3(256), 0, stream(), j.M, j.Cred, j.Mp, (size_t)j.sm,
+                                      (size_t)j.sc, w, j.wp);
+        else hipLaunchKernelGGL(pack_patch_k<true>, pgrid, dim3(256), 0, stream(), j.M, j.Cred, j.Mp, (size_t)j.sm,
+                                (size_t)j.sc, w, j.wp);
         DOPT_LAUNCH_CHECK();
+        prepacked = j.wp;
     }
     pc.in = in;
-    pc.wp = wp;
+    pc.wp = prepacked;
     pc.bias = bias;
     pc.in_bytes = (size_t)pc.N * pc.Cin * pc.IH * pc.IW * sizeof(float);
-    pc.wp_bytes = wp_elems * sizeof(float);
+    pc.wp_bytes = u.wp_elems * sizeof(float);
     pc.out = splits > 1 ? partial : out;
     const dim3 grid(xcd_grid((unsigned)(tiles * splits)));
     const bool c_full = pc.Cin % 16 == 0;
     int rc;
-    if (shape == kWide) rc = launch_patch<GatherWide, 24>(pc, c_full, grid, lds_bytes);
-    else if (shape == kSquare) rc = launch_patch<GatherSquare, 16>(pc, c_full, grid, lds_bytes);
-    else rc = launch_patch<GatherDeep, 16>(pc, c_full, grid, lds_bytes);
+    if (u.shape == 0) rc = launch_patch<GatherWide, 24>(pc, c_full, grid, u.lds_bytes);
+    else if (u.shape == 1) rc = launch_patch<GatherSquare, 16>(pc, c_full, grid, u.lds_bytes);
+    else rc = launch_patch<GatherDeep, 16>(pc, c_full, grid, u.lds_bytes);
     if (rc) return rc;
     *done = true;
     if (splits > 1)
@@ -1427,6 +1497,73 @@ int dopt_hip_conv_bwd_data(const dopt_hip_conv_desc *d, const float *dy, const f
     DOPT_REQUIRE(dy && w && dx, "dopt_hip_conv_bwd_data: null argument");
     DOPT_ENSURE_INIT();
     return run_gather<true>(d, P, Q, dy, w, dx);
+}
+
+size_t dopt_hip_conv_packed_bytes(const dopt_hip_conv_desc *d, int bwd_data)
+{
+    size_t P, Q;
+    if (check_desc(d, &P, &Q, "dopt_hip_conv_packed_bytes") || !ensure_init()) return 0;
+    const PatchSetup u = bwd_data ? patch_setup<true>(d, P, Q) : patch_setup<false>(d, P, Q);
+    // PackJob keeps strides in 32 bits
+    return u.ok && d->C * 9 < (1ull << 32) ? u.wp_elems * sizeof(float) : 0;
+}
+
+int dopt_hip_conv_pack_batch(int n, const dopt_hip_conv_desc *descs, const int *bwd_data, const float *const *w,
+                             float *const *packed)
+{
+    if (n == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(n > 0 && descs && bwd_data && w && packed, "dopt_hip_conv_pack_batch: null argument");
+    DOPT_ENSURE_INIT();
+    PackBatch b{};
+    unsigned blocks = 0;
+    auto flush = [&]() -> int {
+        if (b.njobs == 0) return DOPT_HIP_OK;
+        hipLaunchKernelGGL(pack_batch_k, dim3(blocks), dim3(256), 0, stream(), b);
+        DOPT_LAUNCH_CHECK();
+        b.njobs = 0;
+        blocks = 0;
+        return DOPT_HIP_OK;
+    };
+    for (int i = 0; i < n; i++) {
+        size_t P, Q;
+        if (int rc = check_desc(&descs[i], &P, &Q, "dopt_hip_conv_pack_batch")) return rc;
+        DOPT_REQUIRE(w[i] && packed[i] && aligned16(packed[i]), "dopt_hip_conv_pack_batch: filter %d: null or unaligned pointer", i);
+        const PatchSetup u = bwd_data[i] ? patch_setup<true>(&descs[i], P, Q) : patch_setup<false>(&descs[i], P, Q);
+        DOPT_REQUIRE(u.ok && dopt_hip_conv_packed_bytes(&descs[i], bwd_data[i]) > 0,
+                     "dopt_hip_conv_pack_batch: convolution %d does not take a packed filter", i);
+        PackJob j = bwd_data[i] ? pack_job<true>(&descs[i], u, w[i], packed[i]) : pack_job<false>(&descs[i], u, w[i], packed[i]);
+        j.first_block = blocks;
+        blocks += j.mblocks * (unsigned)u.pc.chunks_total;
+        b.job[b.njobs++] = j;
+        if (b.njobs == kPackJobs)
+            if (int rc = flush()) return rc;
+    }
+    return flush();
+}
+
+int dopt_hip_conv_fwd_bias_packed(const dopt_hip_conv_desc *d, const float *x, const float *packed, const float *bias,
+                                  float *y)
+{
+    size_t P, Q;
+    if (int rc = check_desc(d, &P, &Q, "dopt_hip_conv_fwd_bias_packed")) return rc;
+    DOPT_REQUIRE(x && packed && y, "dopt_hip_conv_fwd_bias_packed: null argument");
+    DOPT_ENSURE_INIT();
+    bool done = false;
+    if (int rc = run_patch<false>(d, P, Q, x, nullptr, bias, y, &done, packed)) return rc;
+    DOPT_REQUIRE(done, "dopt_hip_conv_fwd_bias_packed: this convolution does not take a packed filter");
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_conv_bwd_data_packed(const dopt_hip_conv_desc *d, const float *dy, const float *packed, float *dx)
+{
+    size_t P, Q;
+    if (int rc = check_desc(d, &P, &Q, "dopt_hip_conv_bwd_data_packed")) return rc;
+    DOPT_REQUIRE(dy && packed && dx, "dopt_hip_conv_bwd_data_packed: null argument");
+    DOPT_ENSURE_INIT();
+    bool done = false;
+    if (int rc = run_patch<true>(d, P, Q, dy, nullptr, nullptr, dx, &done, packed)) return rc;
+    DOPT_REQUIRE(done, "dopt_hip_conv_bwd_data_packed: this convolution does not take a packed filter");
+    return DOPT_HIP_OK;
 }
 
 int dopt_hip_conv_bwd_filter(const dopt_hip_conv_desc *d, const float *dy, const float *x, float *dw)

@@ -884,6 +884,71 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         }
     }
 
+    // Filters packed ahead (DOPT_HIP_PLAN_FUSE): the forward and backward-data kernels of 3x3
+    // convolutions read the filter in their own layout.  When the filter is a variable or a constant
+    // - fixed while the plan runs - every such layout of the plan is produced by ONE launch at the
+    // start of each execution instead of one small launch in front of every convolution.
+    struct Prepack { int op, filter; int bwd; dopt_hip_conv_desc d; void *buf; };
+    std::vector<Prepack> packs;
+    std::vector<int> packOf((size_t)nops, -1);
+    if (flags & DOPT_HIP_PLAN_FUSE) {
+        for (int id : p->mOps) {
+            if (!needed[id] || alias[id].source >= 0 || absorbed[id] || prebuilt[id]) continue;
+            const Operation &op = g.ops[id];
+            Prepack k{};
+            k.op = id;
+            const Operation *cv = nullptr;
+            if (fusedKind[id] == 1) cv = &g.ops[op.deps[0]];
+            else if (!fusedKind[id] && op.opType == "convolution" && op.deps.size() == 2) cv = &op;
+            if (cv) {
+                const auto *pad = sizes_attr(*cv, "padding"), *stride = sizes_attr(*cv, "stride");
+                const auto &x = g.ops[cv->deps[0]].shape, &w = g.ops[cv->deps[1]].shape;
+                if (!pad || !stride || x.size() != 4 || w.size() != 4 || cv->dtype != DOPT_HIP_F32) continue;
+                k.filter = cv->deps[1];
+                k.d = conv_desc(x, w, *pad, *stride);
+            } else if (!fusedKind[id] && op.opType == "convolutionFeaturesGrad" && op.deps.size() == 2) {
+                const auto *pad = sizes_attr(op, "padding"), *stride = sizes_attr(op, "stride");
+                const auto &w = g.ops[op.deps[1]].shape;
+                if (!pad || !stride || op.shape.size() != 4 || w.size() != 4 || op.dtype != DOPT_HIP_F32) continue;
+                k.filter = op.deps[1];
+                k.bwd = 1;
+                k.d = conv_desc(op.shape, w, *pad, *stride);
+            } else {
+                continue;
+            }
+            if (!is_leaf(g.ops[k.filter])) continue;
+            const size_t bytes = dopt_hip_conv_packed_bytes(&k.d, k.bwd);
+            if (bytes == 0) continue;
+            if (int rc = dopt_hip_malloc(&k.buf, bytes)) return rc;
+            p->mOwned.push_back(k.buf);
+            p->mBufferBytes += bytes;
+            packOf[id] = (int)packs.size();
+            packs.push_back(k);
+        }
+    }
+    if (!packs.empty()) {
+        std::vector<dopt_hip_conv_desc> descs;
+        std::vector<int> bwd;
+        std::vector<float *> bufs;
+        Step s;
+        s.op = -1;
+        s.label = "filterPack";
+        for (const Prepack &k : packs) {
+            descs.push_back(k.d);
+            bwd.push_back(k.bwd);
+            bufs.push_back((float *)k.buf);
+            s.inputOps.push_back(k.filter);
+        }
+        s.kernel = make([=](const std::vector<const void *> &in, void *) {
+            return dopt_hip_conv_pack_batch((int)descs.size(), descs.data(), bwd.data(), (const float *const *)in.data(),
+                                            bufs.data());
+        });
+        s.inputs.resize(s.inputOps.size());
+        s.inputBytes.resize(s.inputOps.size());
+        for (size_t i = 0; i < s.inputOps.size(); i++) s.inputBytes[i] = g.ops[s.inputOps[i]].bytes();
+        p->mSteps.push_back(std::move(s));
+    }
+
     // buffers first: a fused kernel may write into the buffer of a later operation
     for (int id : p->mOps) {
         if (!needed[id] || is_leaf(g.ops[id]) || alias[id].source >= 0) continue;
@@ -909,7 +974,29 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         std::unique_ptr<HIPKernel> k;
         std::string label = op.opType;
         void *extra = biasGradOf[id] >= 0 && needed[biasGradOf[id]] ? p->mResults[biasGradOf[id]] : nullptr;
-        if (prebuilt[id]) {
+        std::vector<int> stepInputs = inputsOf[id];
+        if (packOf[id] >= 0) {  // the filter operand is read from its packed copy
+            const Prepack pk = packs[(size_t)packOf[id]];
+            const float *packed = (const float *)pk.buf;
+            const dopt_hip_conv_desc d = pk.d;
+            if (pk.bwd) {
+                stepInputs = {op.deps[0]};
+                k = make([=](const std::vector<const void *> &in, void *out) {
+                    return dopt_hip_conv_bwd_data_packed(&d, (const float *)in[0], packed, (float *)out);
+                });
+            } else if (fusedKind[id] == 1) {
+                stepInputs = {inputsOf[id][0], inputsOf[id][2]};
+                k = make([=](const std::vector<const void *> &in, void *out) {
+                    return dopt_hip_conv_fwd_bias_packed(&d, (const float *)in[0], packed, (const float *)in[1], (float *)out);
+                });
+                label = "convolution+addBias";
+            } else {
+                stepInputs = {op.deps[0]};
+                k = make([=](const std::vector<const void *> &in, void *out) {
+                    return dopt_hip_conv_fwd_bias_packed(&d, (const float *)in[0], packed, nullptr, (float *)out);
+                });
+            }
+        } else if (prebuilt[id]) {
             k = std::move(prebuilt[id]);
             label = prebuiltLabel[id];
         } else if (fusedKind[id] || extra) {
@@ -930,7 +1017,7 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         Step s;
         s.op = id;
         s.label = label;
-        s.inputOps = inputsOf[id];
+        s.inputOps = stepInputs;
         s.kernel = std::move(k);
         s.inputs.resize(s.inputOps.size());
         s.inputBytes.resize(s.inputOps.size());
@@ -1019,7 +1106,9 @@ int HIPPlan::execute(int nargs, const int *argOps, const void *const *argPtrs, c
     for (size_t i = 0; i < mSteps.size(); i++) {
         Step &s = mSteps[i];
         if (timing) DOPT_HIP_CHECK(hipEventRecord(mEvents[i].first, stream()));
-        if (int rc = s.kernel->execute(s.inputs, s.inputBytes, mResults[s.op], mGraph->ops[s.op].bytes())) return rc;
+        void *result = s.op >= 0 ? mResults[s.op] : nullptr;   // a step that serves other steps has no operation of its own
+        const size_t resultBytes = s.op >= 0 ? mGraph->ops[s.op].bytes() : 0;
+        if (int rc = s.kernel->execute(s.inputs, s.inputBytes, result, resultBytes)) return rc;
         if (timing) DOPT_HIP_CHECK(hipEventRecord(mEvents[i].second, stream()));
     }
     if (timing) {

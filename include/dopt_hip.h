@@ -182,6 +182,22 @@ int dopt_hip_conv_fwd_bias(const dopt_hip_conv_desc *d, const float *x, const fl
                            const float *bias, float *y);
 /* `convolutionFeaturesGrad` (also convolutionTranspose): cudnnConvolutionBackwardData, cudnn7.d:199. */
 int dopt_hip_conv_bwd_data(const dopt_hip_conv_desc *d, const float *dy, const float *w, float *dx);
+/* Filters packed ahead of the convolutions that read them.  The forward and backward-data kernels
+   of 3x3 unit-stride convolutions read the filter in a layout of their own, which the entry points
+   above produce on every call; a caller that runs many convolutions per step (a plan) can pack all
+   their filters in ONE launch and hand the packed copies over instead.  The reference has no
+   counterpart: cuDNN reads [K, C, R, S] directly (cuda/nnet/cudnn7.d:161-175, :229-241).
+   dopt_hip_conv_packed_bytes: size of the packed copy for the forward (bwd_data = 0) or the
+   backward-data (1) direction, or 0 when that convolution does not take one (the caller then uses
+   the unpacked entry points).  A packed copy depends on the descriptor, the direction and the
+   device, and is valid until the filter changes. */
+size_t dopt_hip_conv_packed_bytes(const dopt_hip_conv_desc *d, int bwd_data);
+int dopt_hip_conv_pack_batch(int n, const dopt_hip_conv_desc *descs, const int *bwd_data,
+                             const float *const *w, float *const *packed /* 16-byte aligned */);
+/* bias may be null */
+int dopt_hip_conv_fwd_bias_packed(const dopt_hip_conv_desc *d, const float *x, const float *packed,
+                                  const float *bias, float *y);
+int dopt_hip_conv_bwd_data_packed(const dopt_hip_conv_desc *d, const float *dy, const float *packed, float *dx);
 /* `convolutionFiltersGrad`: cudnnConvolutionBackwardFilter, cudnn7.d:244. */
 int dopt_hip_conv_bwd_filter(const dopt_hip_conv_desc *d, const float *dy, const float *x, float *dw);
 

@@ -321,3 +321,56 @@ def test_plan_fusion_does_not_change_results():
     # three conv blocks each lose addBias, relu, reluGrad and addBiasGrad as separate kernels, and the
     # two dense layers lose their transposes
     assert kernels[2] <= kernels[1] - 12 - 8, kernels
+
+
+def test_packed_filter_entry_points_match_the_unpacked_ones():
+    """dopt_hip_conv_pack_batch + the *_packed entry points against dopt_hip_conv_fwd_bias /
+    dopt_hip_conv_bwd_data (themselves checked against the oracle in test_gpu_ops.py): same kernels,
+    same packed layout, so the results are identical."""
+    import ctypes as C
+    from dopt_amd import capi
+    lib = capi.load()
+    r = np.random.default_rng(0)
+    cases = [((4, 16, 8, 8), 32), ((2, 64, 32, 32), 64), ((8, 128, 4, 4), 256), ((16, 48, 2, 2), 40), ((3, 3, 16, 16), 8)]
+    descs, flags, ws, packed, shapes = [], [], [], [], []
+    for xs, k in cases:
+        for bwd in (0, 1):
+            d = ops.conv_desc(xs, (k, xs[1], 3, 3), (1, 1), (1, 1))
+            nbytes = lib.dopt_hip_conv_packed_bytes(C.byref(d), bwd)
+            if nbytes == 0:            # this shape and direction runs on the generic kernel
+                continue
+            assert nbytes % 4 == 0
+            shapes.append((xs, k))
+            w = ops.tensor(r.standard_normal((k, xs[1], 3, 3)).astype(np.float32))
+            buf = ops.Tensor([nbytes // 4])
+            descs.append(d); flags.append(bwd); ws.append(w); packed.append(buf)
+    n = len(descs)
+    assert n >= 6
+    capi.check(lib.dopt_hip_conv_pack_batch(n, (type(descs[0]) * n)(*descs), (C.c_int * n)(*flags),
+                                            (C.c_void_p * n)(*[w.ptr for w in ws]), (C.c_void_p * n)(*[b.ptr for b in packed])))
+    for i, (xs, k) in enumerate(shapes):
+        d, bwd, w, buf = descs[i], flags[i], ws[i], packed[i]
+        ys = (xs[0], k, xs[2], xs[3])
+        if not bwd:
+            x = ops.tensor(r.standard_normal(xs).astype(np.float32))
+            b = ops.tensor(r.standard_normal(k).astype(np.float32))
+            want = ops.convolution_bias(x, w, b, (1, 1), (1, 1)).numpy()
+            got = ops.Tensor(ys)
+            capi.check(lib.dopt_hip_conv_fwd_bias_packed(C.byref(d), x.ptr, buf.ptr, b.ptr, got.ptr))
+            assert np.array_equal(got.numpy(), want)
+            capi.check(lib.dopt_hip_conv_fwd_bias_packed(C.byref(d), x.ptr, buf.ptr, None, got.ptr))
+            assert np.array_equal(got.numpy(), ops.convolution(x, w, (1, 1), (1, 1)).numpy())
+        else:
+            dy = ops.tensor(r.standard_normal(ys).astype(np.float32))
+            want = ops.conv_bwd_data(dy, w, xs, (1, 1), (1, 1)).numpy()
+            got = ops.Tensor(xs)
+            capi.check(lib.dopt_hip_conv_bwd_data_packed(C.byref(d), dy.ptr, buf.ptr, got.ptr))
+            assert np.array_equal(got.numpy(), want)
+    # shapes the patch kernels do not take report 0 and are refused by the packed entry points
+    d5 = ops.conv_desc((2, 8, 8, 8), (8, 8, 5, 5), (2, 2), (1, 1))
+    assert lib.dopt_hip_conv_packed_bytes(C.byref(d5), 0) == 0
+    ds = ops.conv_desc((2, 16, 8, 8), (8, 16, 3, 3), (1, 1), (2, 2))
+    assert lib.dopt_hip_conv_packed_bytes(C.byref(ds), 1) == 0
+    x, y, scratch = ops.Tensor((2, 8, 8, 8)), ops.Tensor((2, 8, 8, 8)), ops.Tensor([1024])
+    with pytest.raises(capi.HipError):
+        capi.check(lib.dopt_hip_conv_fwd_bias_packed(C.byref(d5), x.ptr, scratch.ptr, None, y.ptr))
