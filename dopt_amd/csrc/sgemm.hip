@@ -163,6 +163,84 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_k(Gemm p)
     }
 }
 
+// Small outputs (a dense layer at batch 128: 128 x 512 values from a 512-deep reduction).  The tile
+// engine above would run four blocks plus a reduction launch; here one block owns a 32 x 32 tile of
+// C, its eight wavefronts each take an eighth of K straight from memory into MFMA operands (no LDS
+// staging: nothing is reused inside a 32-wide tile), and the eight partial tiles are summed through
+// LDS in wavefront order.  Per step of 8 reductions a lane holds four k values for its row of A and
+// four for its column of B; v_mfma_f32_32x32x2 number e pairs element e of lanes 0-31 (k = 8q + e)
+// with element e of lanes 32-63 (k = 8q + 4 + e) - any pairing works as long as A and B agree.
+//
+// X is "k-contiguous" when element (r, k) sits at X[r * ld + k] (A as given, B transposed), else
+// "r-contiguous" at X[k * ld + r].
+template <bool kKContig, bool kVec>
+__device__ __forceinline__ void small_load(const float *X, int ld, int r, bool r_ok, int kk, int k_end, float (&v)[4])
+{
+    if (kKContig) {
+        const float *src = X + (size_t)r * ld + kk;
+        if (kVec && r_ok && kk + 3 < k_end) {
+            const float4 q = *(const float4 *)src;
+            v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = (r_ok && kk + e < k_end) ? src[e] : 0.0f;
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = (r_ok && kk + e < k_end) ? X[(size_t)(kk + e) * ld + r] : 0.0f;
+    }
+}
+
+constexpr int kSmallWaves = 8;
+
+template <bool kTA, bool kTB, bool kVec>
+__global__ __launch_bounds__(64 * kSmallWaves) void sgemm_small_k(int M, int N, int K, int lda, int ldb, int kslice,
+                                                                   const float *A, const float *B, float *C)
+{
+    __shared__ float red[kSmallWaves][32 * 33];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, r = lane & 31;
+    const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+    const int row = m0 + r, col = n0 + r;
+    const bool row_ok = row < M, col_ok = col < N;
+    const int k_begin = wave * kslice, k_end = min(K, k_begin + kslice);
+
+    v16f acc;
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = 0.0f;
+    float a[4], b[4], an[4], bn[4];
+    if (k_begin < k_end) {
+        small_load<!kTA, kVec>(A, lda, row, row_ok, k_begin + 4 * half, k_end, a);
+        small_load<kTB, kVec>(B, ldb, col, col_ok, k_begin + 4 * half, k_end, b);
+    }
+    for (int k = k_begin; k < k_end; k += 8) {
+        const bool more = k + 8 < k_end;
+        if (more) {   // the next step's operands are in flight while this step multiplies
+            small_load<!kTA, kVec>(A, lda, row, row_ok, k + 8 + 4 * half, k_end, an);
+            small_load<kTB, kVec>(B, ldb, col, col_ok, k + 8 + 4 * half, k_end, bn);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], acc, 0, 0, 0);
+        if (more) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                a[e] = an[e];
+                b[e] = bn[e];
+            }
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < 16; v++) red[wave][acc_row(v, lane) * 33 + r] = acc[v];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int idx = tid + i * 64 * kSmallWaves, rr = idx >> 5, cc = idx & 31;
+        float sum = red[0][rr * 33 + cc];
+#pragma unroll
+        for (int w = 1; w < kSmallWaves; w++) sum += red[w][rr * 33 + cc];
+        if (m0 + rr < M && n0 + cc < N) C[(size_t)(m0 + rr) * N + n0 + cc] = sum;
+    }
+}
+
 __global__ __launch_bounds__(256) void splitk_reduce_k(size_t n, int splits, const float *partial, float *out)
 {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
@@ -273,6 +351,33 @@ int dopt_hip_sgemm_t(int transA, int transB, size_t M, size_t N, size_t K, const
             DOPT_LAUNCH_CHECK();
         }
         return DOPT_HIP_OK;
+    }
+
+    // small outputs: one block per 32 x 32 tile, the reduction split over its wavefronts.  Each tile
+    // reads its own 32 rows of A and 32 columns of B, so the operand traffic grows with the number
+    // of tiles; past a few hundred tiles the LDS-tiled engine below is the better fit.
+    {
+        const size_t tiles = ceil_div(M, (size_t)32) * ceil_div(N, (size_t)32);
+        if (tiles <= 512 && tiles * 64 * K * sizeof(float) <= ((size_t)256 << 20)) {
+            const int lda = (int)(transA ? M : K), ldb = (int)(transB ? K : N);
+            int kslice = (int)ceil_div(ceil_div(K, (size_t)kSmallWaves), (size_t)8) * 8;
+            const bool vec = aligned16(A) && aligned16(B) && lda % 4 == 0 && ldb % 4 == 0;
+            const dim3 grid((unsigned)ceil_div(N, (size_t)32), (unsigned)ceil_div(M, (size_t)32)), block(64 * kSmallWaves);
+#define DOPT_SMALL(TA, TB)                                                                                             \
+    do {                                                                                                               \
+        if (vec) hipLaunchKernelGGL((sgemm_small_k<TA, TB, true>), grid, block, 0, stream(), (int)M, (int)N, (int)K, lda, \
+                                    ldb, kslice, A, B, C);                                                             \
+        else hipLaunchKernelGGL((sgemm_small_k<TA, TB, false>), grid, block, 0, stream(), (int)M, (int)N, (int)K, lda,  \
+                                ldb, kslice, A, B, C);                                                                 \
+    } while (0)
+            if (transA && transB) DOPT_SMALL(true, true);
+            else if (transA) DOPT_SMALL(true, false);
+            else if (transB) DOPT_SMALL(false, true);
+            else DOPT_SMALL(false, false);
+#undef DOPT_SMALL
+            DOPT_LAUNCH_CHECK();
+            return DOPT_HIP_OK;
+        }
     }
 
     Gemm g{};
