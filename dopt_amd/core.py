@@ -693,6 +693,7 @@ def grad(objective, wrt):
 PLAN_VIEWS = 1
 PLAN_TIMING = 2
 PLAN_FUSE = 4
+PLAN_OVERLAP = 8
 
 
 class Plan:

@@ -25,6 +25,11 @@ bool ensure_init();
 // cuda/nnet/cudnn7.d:111).  Valid until the next call that asks for more; all users enqueue on
 // the one library stream, so consecutive users never overlap.
 void *workspace(size_t bytes);
+// The library owns two in-order queues.  Everything enqueues on the main one unless a plan has
+// switched to the side queue for a step it overlaps with its main chain (set_lane(1) ... set_lane(0));
+// each queue has its own workspace.
+void set_lane(int lane);
+hipStream_t lane_stream(int lane);
 
 // Number of compute units of the active device (256 on MI355X); used to size grids.
 int num_cus();

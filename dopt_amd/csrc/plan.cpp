@@ -1035,6 +1035,36 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
             p->mAliasOffset[id] = alias[id].offset;
         }
     p->mNeeded = needed;
+    if (flags & DOPT_HIP_PLAN_OVERLAP) {
+        // A filter gradient feeds nothing of the backward chain: it, and every step that reads a
+        // side-queue result, goes to the side queue.  Steps keep their order within each queue.
+        std::vector<char> onSide((size_t)nops, 0);
+        auto producer = [&](int id) {   // the operation whose kernel wrote the buffer `id` names
+            while (alias[id].source >= 0) id = alias[id].source;
+            return id;
+        };
+        int fences = 1;   // the final join
+        for (Step &st : p->mSteps) {
+            if (st.op < 0) continue;
+            bool reads_side = false;
+            for (int in : st.inputOps) reads_side = reads_side || onSide[producer(in)];
+            const bool wgrad = g.ops[st.op].opType == "convolutionFiltersGrad";
+            // a step with a second output (the absorbed bias gradient) stays on the main queue
+            if ((wgrad || reads_side) && biasGradOf[st.op] < 0) {
+                st.lane = 1;
+                onSide[st.op] = 1;
+                p->mUsesSide = true;
+                fences++;
+            } else if (reads_side) {
+                st.joinSide = true;
+                fences++;
+            }
+        }
+        if (p->mUsesSide) {
+            p->mFences.resize((size_t)fences);
+            for (hipEvent_t &ev : p->mFences) DOPT_HIP_CHECK(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+        }
+    }
     if (flags & DOPT_HIP_PLAN_TIMING) {
         p->mEvents.resize(p->mSteps.size());
         for (auto &ev : p->mEvents) {
@@ -1063,6 +1093,8 @@ void HIPPlan::cleanup()
         (void)hipEventDestroy(ev.second);
     }
     mEvents.clear();
+    for (hipEvent_t ev : mFences) (void)hipEventDestroy(ev);
+    mFences.clear();
     mClean = true;
 }
 
@@ -1103,14 +1135,31 @@ int HIPPlan::execute(int nargs, const int *argOps, const void *const *argPtrs, c
     if (nrets > (int)mOutputs.size()) return fail(DOPT_HIP_ERR_INVALID, "more return buffers than plan outputs");
     if (int rc = resolve(nargs, argOps, argPtrs, argOnHost)) return rc;
     const bool timing = !mEvents.empty();
+    size_t fence = 0;
+    auto order = [&](int first, int then) -> int {   // work queued on `then` from here on follows all of `first` so far
+        DOPT_HIP_CHECK(hipEventRecord(mFences[fence], lane_stream(first)));
+        DOPT_HIP_CHECK(hipStreamWaitEvent(lane_stream(then), mFences[fence], 0));
+        fence++;
+        return DOPT_HIP_OK;
+    };
     for (size_t i = 0; i < mSteps.size(); i++) {
         Step &s = mSteps[i];
+        if (s.lane == 1) {
+            if (int rc = order(0, 1)) return rc;   // its inputs come from main-queue steps before it
+        } else if (s.joinSide) {
+            if (int rc = order(1, 0)) return rc;
+        }
+        set_lane(s.lane);
         if (timing) DOPT_HIP_CHECK(hipEventRecord(mEvents[i].first, stream()));
         void *result = s.op >= 0 ? mResults[s.op] : nullptr;   // a step that serves other steps has no operation of its own
         const size_t resultBytes = s.op >= 0 ? mGraph->ops[s.op].bytes() : 0;
-        if (int rc = s.kernel->execute(s.inputs, s.inputBytes, result, resultBytes)) return rc;
-        if (timing) DOPT_HIP_CHECK(hipEventRecord(mEvents[i].second, stream()));
+        const int rc = s.kernel->execute(s.inputs, s.inputBytes, result, resultBytes);
+        if (!rc && timing) DOPT_HIP_CHECK(hipEventRecord(mEvents[i].second, stream()));
+        set_lane(0);
+        if (rc) return rc;
     }
+    if (mUsesSide)
+        if (int rc = order(1, 0)) return rc;       // the outputs, and whatever the caller queues next, see both queues' work
     if (timing) {
         DOPT_HIP_CHECK(hipStreamSynchronize(stream()));
         for (size_t i = 0; i < mSteps.size(); i++) {

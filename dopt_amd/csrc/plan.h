@@ -95,6 +95,8 @@ private:
         std::unique_ptr<HIPKernel> kernel;
         std::vector<const void *> inputs;
         std::vector<size_t> inputBytes;
+        int lane = 0;                            // 1: runs on the side queue, beside the main chain
+        bool joinSide = false;                   // main-queue step that reads a side-queue result
     };
     Graph *mGraph = nullptr;
     unsigned mFlags = 0;
@@ -108,6 +110,8 @@ private:
     std::vector<size_t> mAliasOffset;            // per op: byte offset into the aliased buffer
     std::vector<char> mNeeded;                   // per op: its result is consumed
     std::vector<std::pair<hipEvent_t, hipEvent_t>> mEvents;
+    std::vector<hipEvent_t> mFences;             // ordering between the two queues, one per crossing
+    bool mUsesSide = false;
     size_t mBufferBytes = 0;
     bool mClean = false;
     std::vector<void *> mRetDst;                 // scratch of execute(): the return copies

@@ -24,15 +24,17 @@ struct Runtime {
     int cus = 256;
     std::string arch = "gfx950";
     hipStream_t stream = nullptr;
+    hipStream_t side = nullptr;     // second in-order queue for work a plan overlaps with its main chain
+    int lane = 0;                   // which of the two the entry points currently enqueue on
 
     // pool
     std::unordered_map<void *, size_t> live;           // ptr -> class size
     std::map<size_t, std::vector<void *>> cached;      // class size -> free blocks
     size_t live_bytes = 0, cached_bytes = 0, device_allocs = 0;
 
-    // workspace
-    void *ws = nullptr;
-    size_t ws_bytes = 0;
+    // workspace, one per queue: kernels of the two queues run at the same time
+    void *ws[2] = {nullptr, nullptr};
+    size_t ws_bytes[2] = {0, 0};
 
     // rtc
     std::unordered_map<std::string, hipFunction_t> kernels;
@@ -81,6 +83,7 @@ int init_locked(int device)
         return fail(DOPT_HIP_ERR_UNSUPPORTED, "dopt_hip_init: this library is built for gfx950 only, device is %s",
                     r.arch.c_str());
     DOPT_HIP_CHECK(hipStreamCreateWithFlags(&r.stream, hipStreamNonBlocking));
+    DOPT_HIP_CHECK(hipStreamCreateWithFlags(&r.side, hipStreamNonBlocking));   // same (default) priority
     r.device = device;
     r.ready = true;
     return DOPT_HIP_OK;
@@ -109,24 +112,27 @@ bool ensure_init()
     return init_locked(0) == DOPT_HIP_OK;
 }
 
-hipStream_t stream() { return rt().stream; }
+hipStream_t stream() { return rt().lane ? rt().side : rt().stream; }
+hipStream_t lane_stream(int lane) { return lane ? rt().side : rt().stream; }
+void set_lane(int lane) { rt().lane = lane ? 1 : 0; }
 int num_cus() { return rt().cus; }
 
 void *workspace(size_t bytes)
 {
     Runtime &r = rt();
-    if (bytes <= r.ws_bytes) return r.ws;
-    // Growing: earlier users were enqueued on the same stream, and hipFree waits for the device.
-    if (r.ws) (void)hipFree(r.ws);
-    r.ws = nullptr;
-    r.ws_bytes = 0;
+    const int l = r.lane;
+    if (bytes <= r.ws_bytes[l]) return r.ws[l];
+    // Growing: earlier users were enqueued on the same queue, and hipFree waits for the device.
+    if (r.ws[l]) (void)hipFree(r.ws[l]);
+    r.ws[l] = nullptr;
+    r.ws_bytes[l] = 0;
     size_t want = size_class(bytes);
-    if (hipMalloc(&r.ws, want) != hipSuccess) {
+    if (hipMalloc(&r.ws[l], want) != hipSuccess) {
         fail(DOPT_HIP_ERR_OOM, "workspace: unable to allocate %zu bytes", want);
         return nullptr;
     }
-    r.ws_bytes = want;
-    return r.ws;
+    r.ws_bytes[l] = want;
+    return r.ws[l];
 }
 
 // ------------------------------------------------------------------------------- hipRTC
@@ -211,6 +217,7 @@ int dopt_hip_shutdown(void)
     std::lock_guard<std::mutex> lk(r.mu);
     if (!r.ready) return DOPT_HIP_OK;
     (void)hipStreamSynchronize(r.stream);
+    (void)hipStreamSynchronize(r.side);
     for (auto &kv : r.cached)
         for (void *p : kv.second) (void)hipFree(p);
     r.cached.clear();
@@ -218,14 +225,18 @@ int dopt_hip_shutdown(void)
     for (auto &kv : r.live) (void)hipFree(kv.first);
     r.live.clear();
     r.live_bytes = 0;
-    if (r.ws) (void)hipFree(r.ws);
-    r.ws = nullptr;
-    r.ws_bytes = 0;
+    for (int l = 0; l < 2; l++) {
+        if (r.ws[l]) (void)hipFree(r.ws[l]);
+        r.ws[l] = nullptr;
+        r.ws_bytes[l] = 0;
+    }
+    r.lane = 0;
     for (hipModule_t m : r.modules) (void)hipModuleUnload(m);
     r.modules.clear();
     r.kernels.clear();
     (void)hipStreamDestroy(r.stream);
-    r.stream = nullptr;
+    (void)hipStreamDestroy(r.side);
+    r.stream = r.side = nullptr;
     r.ready = false;
     return DOPT_HIP_OK;
 }
@@ -388,7 +399,8 @@ int dopt_hip_copy_d2d(void *dst, const void *src, size_t bytes)
 int dopt_hip_sync(void)
 {
     DOPT_ENSURE_INIT();
-    DOPT_HIP_CHECK(hipStreamSynchronize(stream()));
+    DOPT_HIP_CHECK(hipStreamSynchronize(lane_stream(0)));
+    DOPT_HIP_CHECK(hipStreamSynchronize(lane_stream(1)));   // idle unless a plan is overlapping work
     return DOPT_HIP_OK;
 }
 

@@ -72,9 +72,13 @@ enum {
     DOPT_HIP_PLAN_VIEWS = 1,  /* contiguous slices alias their input; slice(pad(x)) that undoes the
                                  pad aliases x; operations left without a consumer are dropped */
     DOPT_HIP_PLAN_TIMING = 2, /* bracket every kernel with HIP events (CUDAPlan.profiler) */
-    DOPT_HIP_PLAN_FUSE = 4    /* with VIEWS: run adjacent operations as one kernel where the middle value
+    DOPT_HIP_PLAN_FUSE = 4,   /* with VIEWS: run adjacent operations as one kernel where the middle value
                                  has no other reader -- addBias(convolution), relu(batchNormTrain.y) and
                                  batchNormGrad(reluGrad) -- with the values of the separate kernels */
+    DOPT_HIP_PLAN_OVERLAP = 8 /* filter gradients, and whatever only they feed, run on a second in-order
+                                 queue beside the chain that produces the feature gradients; the queues
+                                 are ordered by events where a value crosses, and joined before the
+                                 outputs are returned.  Same kernels, same values. */
 };
 
 /* new CUDAPlan(outputs) (cuda/package.d:267-312): topological sort, one kernel object per

@@ -374,3 +374,34 @@ def test_packed_filter_entry_points_match_the_unpacked_ones():
     x, y, scratch = ops.Tensor((2, 8, 8, 8)), ops.Tensor((2, 8, 8, 8)), ops.Tensor([1024])
     with pytest.raises(capi.HipError):
         capi.check(lib.dopt_hip_conv_fwd_bias_packed(C.byref(d5), x.ptr, scratch.ptr, None, y.ptr))
+
+
+def _small_convnet(seed):
+    init = nnet.Init(seed)
+    x, y = core.float32([16, 3, 16, 16]), core.float32([16, 10])
+    h = nnet.relu(nnet.batchNorm(nnet.conv2D(nnet.dataSource(x), 16, (3, 3), init, padding=(1, 1), weight_decay=1e-3)))
+    h = nnet.maxPool(nnet.relu(nnet.batchNorm(nnet.conv2D(h, 32, (3, 3), init, padding=(1, 1)))), (2, 2))
+    h = nnet.relu(nnet.batchNorm(nnet.conv2D(h, 32, (3, 3), init, padding=(1, 1), weight_decay=1e-3)))
+    top = nnet.softmax(nnet.dense(h, 10, init))
+    net = nnet.DAGNetwork([x], [top])
+    return x, y, net, nnet.crossEntropy(top.trainOutput, y) + net.paramLoss
+
+
+@pytest.mark.parametrize("maker", [online.fused_sgd, online.sgd, online.adam])
+def test_overlapped_filter_gradients_change_nothing(maker):
+    """DOPT_HIP_PLAN_OVERLAP moves the filter gradients (and what only they feed) to a second queue:
+    the same kernels on the same data, so losses and parameters stay identical bit for bit, step
+    after step (every step re-enters buffers the other queue read in the previous one)."""
+    r = np.random.default_rng(0)
+    xs = r.standard_normal((16, 3, 16, 16)).astype(np.float32)
+    ys = np.eye(10, dtype=np.float32)[r.integers(0, 10, 16)]
+    base = core.PLAN_VIEWS | core.PLAN_FUSE
+    runs = []
+    for flags in (base, base | core.PLAN_OVERLAP):
+        x, y, net, loss = _small_convnet(4)
+        up = maker([loss], net.params, net.paramProj, flags=flags)
+        losses = [up({x: xs, y: ys})[0] for _ in range(6)]
+        runs.append((losses, [p.value for p in net.params]))
+    assert runs[0][0] == runs[1][0]
+    for a, b in zip(runs[0][1], runs[1][1]):
+        assert np.array_equal(a, b)
