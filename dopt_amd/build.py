@@ -13,7 +13,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(HERE, "libdopthip.so")
 
-SOURCES = ["runtime.cpp", "rtc_ops.cpp", "layout.hip", "nn.hip", "bn.hip", "optim.hip", "sgemm.hip", "conv.hip",
+SOURCES = ["runtime.cpp", "rtc_ops.cpp", "layout.hip", "nn.hip", "bn.hip", "optim.hip", "sgemm.hip", "conv.hip", "conv_smallc.hip",
            "plan.cpp"]
 HEADERS = ["common.h", "mfma_core.h", "plan.h", os.path.join("..", "..", "include", "dopt_hip.h"),
            os.path.join("..", "..", "include", "dopt_hip_plan.h")]

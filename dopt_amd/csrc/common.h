@@ -29,6 +29,11 @@ void *workspace(size_t bytes);
 // switched to the side queue for a step it overlaps with its main chain (set_lane(1) ... set_lane(0));
 // each queue has its own workspace.
 void set_lane(int lane);
+// conv_smallc.hip: 3x3 pad-1 unit-stride convolutions over at most three input channels.  `done`
+// stays false when the shape is not theirs (the caller then uses the general kernels).
+bool conv_smallc_takes(const dopt_hip_conv_desc *d);
+int conv_smallc_fwd(const dopt_hip_conv_desc *d, const float *x, const float *w, const float *bias, float *y, bool *done);
+int conv_smallc_wgrad(const dopt_hip_conv_desc *d, const float *dy, const float *x, float *dw, bool *done);
 hipStream_t lane_stream(int lane);
 
 // Number of compute units of the active device (256 on MI355X); used to size grids.

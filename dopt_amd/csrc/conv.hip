@@ -1258,6 +1258,11 @@ template <bool kBwd>
 int run_gather(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, const float *w, float *out,
                const float *bias = nullptr)
 {
+    if (!kBwd) {
+        bool done = false;
+        if (int rc = conv_smallc_fwd(d, in, w, bias, out, &done)) return rc;
+        if (done) return DOPT_HIP_OK;
+    }
     {
         bool done = false;
         if (int rc = run_patch<kBwd>(d, P, Q, in, w, bias, out, &done)) return rc;
@@ -1503,6 +1508,7 @@ size_t dopt_hip_conv_packed_bytes(const dopt_hip_conv_desc *d, int bwd_data)
 {
     size_t P, Q;
     if (check_desc(d, &P, &Q, "dopt_hip_conv_packed_bytes") || !ensure_init()) return 0;
+    if (!bwd_data && conv_smallc_takes(d)) return 0;   // that forward kernel reads the filter as it is
     const PatchSetup u = bwd_data ? patch_setup<true>(d, P, Q) : patch_setup<false>(d, P, Q);
     // PackJob keeps strides in 32 bits
     return u.ok && d->C * 9 < (1ull << 32) ? u.wp_elems * sizeof(float) : 0;
@@ -1574,6 +1580,8 @@ int dopt_hip_conv_bwd_filter(const dopt_hip_conv_desc *d, const float *dy, const
     DOPT_ENSURE_INIT();
     {
         bool done = false;
+        if (int rc = conv_smallc_wgrad(d, dy, x, dw, &done)) return rc;
+        if (done) return DOPT_HIP_OK;
         if (int rc = run_wgrad_patch(d, dy, x, dw, &done)) return rc;
         if (done) return DOPT_HIP_OK;
     }

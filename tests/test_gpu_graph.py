@@ -331,7 +331,8 @@ def test_packed_filter_entry_points_match_the_unpacked_ones():
     from dopt_amd import capi
     lib = capi.load()
     r = np.random.default_rng(0)
-    cases = [((4, 16, 8, 8), 32), ((2, 64, 32, 32), 64), ((8, 128, 4, 4), 256), ((16, 48, 2, 2), 40), ((3, 3, 16, 16), 8)]
+    cases = [((4, 16, 8, 8), 32), ((2, 64, 32, 32), 64), ((8, 128, 4, 4), 256), ((16, 48, 2, 2), 40), ((3, 3, 16, 16), 8),
+             ((2, 32, 16, 16), 96)]
     descs, flags, ws, packed, shapes = [], [], [], [], []
     for xs, k in cases:
         for bwd in (0, 1):

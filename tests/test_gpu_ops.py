@@ -313,6 +313,16 @@ CONV_CASES = [  # N, C, H, W, K, R, S, pad, stride
     (32, 48, 2, 2, 130, 3, 3, (1, 1), (1, 1)),    # 2x2 images, sixteen per chunk
     (16, 70, 2, 2, 32, 3, 3, (1, 1), (1, 1)),
     (6, 32, 4, 4, 128, 3, 3, (1, 1), (1, 1)),     # batch not a multiple of the chunk: generic kernel
+    # at most three input channels, pad 1: the first-layer kernels (rows of 8 .. 128 pixels, one to
+    # sixteen rows per sub-tile, output channels off the 32-row fragment, a single-channel image)
+    (3, 3, 32, 32, 40, 3, 3, (1, 1), (1, 1)),
+    (2, 1, 16, 16, 8, 3, 3, (1, 1), (1, 1)),
+    (5, 2, 16, 8, 33, 3, 3, (1, 1), (1, 1)),
+    (2, 3, 4, 64, 64, 3, 3, (1, 1), (1, 1)),
+    (1, 3, 3, 128, 20, 3, 3, (1, 1), (1, 1)),
+    (7, 3, 24, 16, 64, 3, 3, (1, 1), (1, 1)),
+    (2, 3, 28, 28, 16, 3, 3, (1, 1), (1, 1)),     # 28 is no power of two: general kernels
+    (2, 3, 32, 32, 96, 3, 3, (1, 1), (1, 1)),     # more than 64 output channels: general kernels
 ]
 
 
