@@ -72,6 +72,7 @@ PROTOTYPES = {
     "dopt_hip_conv_fwd": [C.POINTER(ConvDesc), _vp, _vp, _vp],
     "dopt_hip_conv_fwd_bias": [C.POINTER(ConvDesc), _vp, _vp, _vp, _vp],
     "dopt_hip_conv_bwd_data": [C.POINTER(ConvDesc), _vp, _vp, _vp],
+    "dopt_hip_conv_packed_layout": [C.POINTER(ConvDesc), _i],
     "dopt_hip_conv_pack_batch": [_i, C.POINTER(ConvDesc), C.POINTER(_i), C.POINTER(_vp), C.POINTER(_vp)],
     "dopt_hip_conv_fwd_bias_packed": [C.POINTER(ConvDesc), _vp, _vp, _vp, _vp],
     "dopt_hip_conv_bwd_data_packed": [C.POINTER(ConvDesc), _vp, _vp, _vp],

@@ -29,6 +29,10 @@ void *workspace(size_t bytes);
 // switched to the side queue for a step it overlaps with its main chain (set_lane(1) ... set_lane(0));
 // each queue has its own workspace.
 void set_lane(int lane);
+// sgemm.hip: C = op(A) * op(B) (+ colbias[col >> bias_shift] per element when colbias is given and the
+// shape takes a kernel with that epilogue; *biased says whether it did).
+int sgemm_bias(int transA, int transB, size_t M, size_t N, size_t K, const float *A, const float *B, float *C,
+               const float *colbias, int bias_shift, bool *biased);
 // conv_smallc.hip: 3x3 pad-1 unit-stride convolutions over at most three input channels.  `done`
 // stays false when the shape is not theirs (the caller then uses the general kernels).
 bool conv_smallc_takes(const dopt_hip_conv_desc *d);

@@ -1253,6 +1253,70 @@ int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, 
     return DOPT_HIP_OK;
 }
 
+// ---- 2 x 2 images -------------------------------------------------------------------------------
+// On a 2 x 2 image with pad 1 every output pixel sees every input pixel, each through exactly one
+// tap, and the five taps that fall on padding contribute nothing.  The convolution is then a plain
+// product of the batch, flattened [N, C*4], with a [C*4, K*4] matrix built from the filter:
+//     Wd[(c, iy, ix)][(k, oy, ox)] = w[k][c][2 - (iy - oy + 1)][2 - (ix - ox + 1)]
+// (the flipped filter, core/source/dopt/core/ops/nnet.d:270-293) - 4/9 of the multiplications of
+// the nine-tap form.  NCHW needs no rearranging on either side, forward is x * Wd and backward-data
+// is dy * Wd^T, so one copy of Wd serves both directions.
+__global__ __launch_bounds__(256) void pack_2x2_k(unsigned C, unsigned K, const float *w, float *wd)
+{
+    const size_t total = (size_t)16 * C * K;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        const unsigned col = (unsigned)(i % (4 * K)), row = (unsigned)(i / (4 * K));
+        const unsigned k = col >> 2, oy = (col >> 1) & 1, ox = col & 1;
+        const unsigned c = row >> 2, iy = (row >> 1) & 1, ix = row & 1;
+        const unsigned r = iy - oy + 1, s = ix - ox + 1;
+        wd[i] = w[((size_t)k * C + c) * 9 + (2 - r) * 3 + (2 - s)];
+    }
+}
+
+bool dense2x2_takes(const dopt_hip_conv_desc *d)
+{
+    return d->R == 3 && d->S == 3 && d->strideH == 1 && d->strideW == 1 && d->padH == 1 && d->padW == 1 && d->H == 2 &&
+           d->W == 2 && d->C * 4 < ((size_t)1 << 30) && d->K * 4 < ((size_t)1 << 30);
+}
+
+size_t dense2x2_elems(const dopt_hip_conv_desc *d) { return (size_t)16 * d->C * d->K; }
+
+int dense2x2_pack(const dopt_hip_conv_desc *d, const float *w, float *wd)
+{
+    const size_t blocks = ceil_div(dense2x2_elems(d), (size_t)256);
+    const size_t cap = (size_t)num_cus() * 16;
+    hipLaunchKernelGGL(pack_2x2_k, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0, stream(), (unsigned)d->C,
+                       (unsigned)d->K, w, wd);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+// `wd`: the matrix already built, or null to build it from `w` in the workspace first
+template <bool kBwd>
+int run_dense2x2(const dopt_hip_conv_desc *d, const float *in, const float *w, const float *wd, const float *bias,
+                 float *out)
+{
+    void *mine = nullptr;   // from the pool, not the workspace: the product below may use the workspace itself
+    if (!wd) {
+        if (int rc = dopt_hip_malloc(&mine, dense2x2_elems(d) * sizeof(float))) return rc;
+        if (int rc = dense2x2_pack(d, w, (float *)mine)) {
+            dopt_hip_free(mine);
+            return rc;
+        }
+        wd = (const float *)mine;
+    }
+    bool biased = false;
+    int rc;
+    if (!kBwd) {
+        rc = sgemm_bias(0, 0, d->N, 4 * d->K, 4 * d->C, in, wd, out, bias, 2, &biased);
+        if (!rc && bias && !biased) rc = dopt_hip_bias_fwd(d->N, d->K, 4, out, bias, out);
+    } else {
+        rc = sgemm_bias(0, 1, d->N, 4 * d->C, 4 * d->K, in, wd, out, nullptr, 0, &biased);
+    }
+    if (mine) dopt_hip_free(mine);   // back to the pool; whoever gets it next queues behind the product
+    return rc;
+}
+
 // Shared host driver of forward (kBwd = false) and backward-data (kBwd = true).
 template <bool kBwd>
 int run_gather(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, const float *w, float *out,
@@ -1263,6 +1327,7 @@ int run_gather(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in,
         if (int rc = conv_smallc_fwd(d, in, w, bias, out, &done)) return rc;
         if (done) return DOPT_HIP_OK;
     }
+    if (dense2x2_takes(d)) return run_dense2x2<kBwd>(d, in, w, nullptr, bias, out);
     {
         bool done = false;
         if (int rc = run_patch<kBwd>(d, P, Q, in, w, bias, out, &done)) return rc;
@@ -1509,9 +1574,17 @@ size_t dopt_hip_conv_packed_bytes(const dopt_hip_conv_desc *d, int bwd_data)
     size_t P, Q;
     if (check_desc(d, &P, &Q, "dopt_hip_conv_packed_bytes") || !ensure_init()) return 0;
     if (!bwd_data && conv_smallc_takes(d)) return 0;   // that forward kernel reads the filter as it is
+    if (dense2x2_takes(d)) return dense2x2_elems(d) * sizeof(float);
     const PatchSetup u = bwd_data ? patch_setup<true>(d, P, Q) : patch_setup<false>(d, P, Q);
     // PackJob keeps strides in 32 bits
     return u.ok && d->C * 9 < (1ull << 32) ? u.wp_elems * sizeof(float) : 0;
+}
+
+int dopt_hip_conv_packed_layout(const dopt_hip_conv_desc *d, int bwd_data)
+{
+    if (dopt_hip_conv_packed_bytes(d, bwd_data) == 0) return -1;
+    if (dense2x2_takes(d)) return 2;   // the same matrix, read transposed by backward-data
+    return bwd_data ? 1 : 0;
 }
 
 int dopt_hip_conv_pack_batch(int n, const dopt_hip_conv_desc *descs, const int *bwd_data, const float *const *w,
@@ -1534,6 +1607,10 @@ int dopt_hip_conv_pack_batch(int n, const dopt_hip_conv_desc *descs, const int *
         size_t P, Q;
         if (int rc = check_desc(&descs[i], &P, &Q, "dopt_hip_conv_pack_batch")) return rc;
         DOPT_REQUIRE(w[i] && packed[i] && aligned16(packed[i]), "dopt_hip_conv_pack_batch: filter %d: null or unaligned pointer", i);
+        if (dense2x2_takes(&descs[i]) && !(!bwd_data[i] && conv_smallc_takes(&descs[i]))) {
+            if (int rc = dense2x2_pack(&descs[i], w[i], packed[i])) return rc;   // a launch of its own: the matrix is large
+            continue;
+        }
         const PatchSetup u = bwd_data[i] ? patch_setup<true>(&descs[i], P, Q) : patch_setup<false>(&descs[i], P, Q);
         DOPT_REQUIRE(u.ok && dopt_hip_conv_packed_bytes(&descs[i], bwd_data[i]) > 0,
                      "dopt_hip_conv_pack_batch: convolution %d does not take a packed filter", i);
@@ -1554,6 +1631,7 @@ int dopt_hip_conv_fwd_bias_packed(const dopt_hip_conv_desc *d, const float *x, c
     if (int rc = check_desc(d, &P, &Q, "dopt_hip_conv_fwd_bias_packed")) return rc;
     DOPT_REQUIRE(x && packed && y, "dopt_hip_conv_fwd_bias_packed: null argument");
     DOPT_ENSURE_INIT();
+    if (dopt_hip_conv_packed_layout(d, 0) == 2) return run_dense2x2<false>(d, x, nullptr, packed, bias, y);
     bool done = false;
     if (int rc = run_patch<false>(d, P, Q, x, nullptr, bias, y, &done, packed)) return rc;
     DOPT_REQUIRE(done, "dopt_hip_conv_fwd_bias_packed: this convolution does not take a packed filter");
@@ -1566,6 +1644,7 @@ int dopt_hip_conv_bwd_data_packed(const dopt_hip_conv_desc *d, const float *dy, 
     if (int rc = check_desc(d, &P, &Q, "dopt_hip_conv_bwd_data_packed")) return rc;
     DOPT_REQUIRE(dy && packed && dx, "dopt_hip_conv_bwd_data_packed: null argument");
     DOPT_ENSURE_INIT();
+    if (dopt_hip_conv_packed_layout(d, 1) == 2) return run_dense2x2<true>(d, dy, nullptr, packed, nullptr, dx);
     bool done = false;
     if (int rc = run_patch<true>(d, P, Q, dy, nullptr, nullptr, dx, &done, packed)) return rc;
     DOPT_REQUIRE(done, "dopt_hip_conv_bwd_data_packed: this convolution does not take a packed filter");

@@ -888,7 +888,7 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
     // convolutions read the filter in their own layout.  When the filter is a variable or a constant
     // - fixed while the plan runs - every such layout of the plan is produced by ONE launch at the
     // start of each execution instead of one small launch in front of every convolution.
-    struct Prepack { int op, filter; int bwd; dopt_hip_conv_desc d; void *buf; };
+    struct Prepack { int op, filter; int bwd; dopt_hip_conv_desc d; void *buf; bool owner; };
     std::vector<Prepack> packs;
     std::vector<int> packOf((size_t)nops, -1);
     if (flags & DOPT_HIP_PLAN_FUSE) {
@@ -919,9 +919,18 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
             if (!is_leaf(g.ops[k.filter])) continue;
             const size_t bytes = dopt_hip_conv_packed_bytes(&k.d, k.bwd);
             if (bytes == 0) continue;
-            if (int rc = dopt_hip_malloc(&k.buf, bytes)) return rc;
-            p->mOwned.push_back(k.buf);
-            p->mBufferBytes += bytes;
+            // the forward and the backward-data convolution of a layer may read the very same copy
+            const int layout = dopt_hip_conv_packed_layout(&k.d, k.bwd);
+            for (const Prepack &other : packs)
+                if (other.owner && other.filter == k.filter && memcmp(&other.d, &k.d, sizeof(k.d)) == 0 &&
+                    dopt_hip_conv_packed_layout(&other.d, other.bwd) == layout)
+                    k.buf = other.buf;
+            k.owner = k.buf == nullptr;
+            if (k.owner) {
+                if (int rc = dopt_hip_malloc(&k.buf, bytes)) return rc;
+                p->mOwned.push_back(k.buf);
+                p->mBufferBytes += bytes;
+            }
             packOf[id] = (int)packs.size();
             packs.push_back(k);
         }
@@ -934,6 +943,7 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         s.op = -1;
         s.label = "filterPack";
         for (const Prepack &k : packs) {
+            if (!k.owner) continue;
             descs.push_back(k.d);
             bwd.push_back(k.bwd);
             bufs.push_back((float *)k.buf);

@@ -195,7 +195,8 @@ constexpr int kSmallWaves = 8;
 
 template <bool kTA, bool kTB, bool kVec>
 __global__ __launch_bounds__(64 * kSmallWaves) void sgemm_small_k(int M, int N, int K, int lda, int ldb, int kslice,
-                                                                   const float *A, const float *B, float *C)
+                                                                   const float *A, const float *B, float *C,
+                                                                   const float *colbias, int bias_shift)
 {
     __shared__ float red[kSmallWaves][32 * 33];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, r = lane & 31;
@@ -237,7 +238,10 @@ __global__ __launch_bounds__(64 * kSmallWaves) void sgemm_small_k(int M, int N, 
         float sum = red[0][rr * 33 + cc];
 #pragma unroll
         for (int w = 1; w < kSmallWaves; w++) sum += red[w][rr * 33 + cc];
-        if (m0 + rr < M && n0 + cc < N) C[(size_t)(m0 + rr) * N + n0 + cc] = sum;
+        if (m0 + rr < M && n0 + cc < N) {
+            if (colbias) sum += colbias[(n0 + cc) >> bias_shift];   // one value per group of 2^bias_shift columns
+            C[(size_t)(m0 + rr) * N + n0 + cc] = sum;
+        }
     }
 }
 
@@ -298,12 +302,17 @@ unsigned flat_grid(size_t n)
 
 }  // namespace
 
-extern "C" {
+namespace dopt {
 
 // C[M,N] = op(A) * op(B) with op(X) = X or its transpose: transA means A is stored [K][M], transB
 // means B is stored [N][K].
-int dopt_hip_sgemm_t(int transA, int transB, size_t M, size_t N, size_t K, const float *A, const float *B, float *C)
+
+// C = op(A) * op(B), plus colbias[col >> bias_shift] on every element when colbias is given.  Returns
+// *biased = false when the shape took a kernel without that epilogue (the caller adds the bias itself).
+int sgemm_bias(int transA, int transB, size_t M, size_t N, size_t K, const float *A, const float *B, float *C,
+               const float *colbias, int bias_shift, bool *biased)
 {
+    *biased = false;
     if (M * N == 0) return DOPT_HIP_OK;
     DOPT_REQUIRE(C != nullptr, "dopt_hip_sgemm: C is null");
     DOPT_ENSURE_INIT();
@@ -366,9 +375,9 @@ int dopt_hip_sgemm_t(int transA, int transB, size_t M, size_t N, size_t K, const
 #define DOPT_SMALL(TA, TB)                                                                                             \
     do {                                                                                                               \
         if (vec) hipLaunchKernelGGL((sgemm_small_k<TA, TB, true>), grid, block, 0, stream(), (int)M, (int)N, (int)K, lda, \
-                                    ldb, kslice, A, B, C);                                                             \
+                                    ldb, kslice, A, B, C, colbias, bias_shift);                                        \
         else hipLaunchKernelGGL((sgemm_small_k<TA, TB, false>), grid, block, 0, stream(), (int)M, (int)N, (int)K, lda,  \
-                                ldb, kslice, A, B, C);                                                                 \
+                                ldb, kslice, A, B, C, colbias, bias_shift);                                            \
     } while (0)
             if (transA && transB) DOPT_SMALL(true, true);
             else if (transA) DOPT_SMALL(true, false);
@@ -376,6 +385,7 @@ int dopt_hip_sgemm_t(int transA, int transB, size_t M, size_t N, size_t K, const
             else DOPT_SMALL(false, false);
 #undef DOPT_SMALL
             DOPT_LAUNCH_CHECK();
+            *biased = colbias != nullptr;
             return DOPT_HIP_OK;
         }
     }
@@ -435,6 +445,16 @@ int dopt_hip_sgemm_t(int transA, int transB, size_t M, size_t N, size_t K, const
         DOPT_LAUNCH_CHECK();
     }
     return DOPT_HIP_OK;
+}
+
+}  // namespace dopt
+
+extern "C" {
+
+int dopt_hip_sgemm_t(int transA, int transB, size_t M, size_t N, size_t K, const float *A, const float *B, float *C)
+{
+    bool biased;
+    return dopt::sgemm_bias(transA, transB, M, N, K, A, B, C, nullptr, 0, &biased);
 }
 
 int dopt_hip_sgemm(size_t M, size_t N, size_t K, const float *A, const float *B, float *C)

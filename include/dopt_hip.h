@@ -192,6 +192,9 @@ int dopt_hip_conv_bwd_data(const dopt_hip_conv_desc *d, const float *dy, const f
    the unpacked entry points).  A packed copy depends on the descriptor, the direction and the
    device, and is valid until the filter changes. */
 size_t dopt_hip_conv_packed_bytes(const dopt_hip_conv_desc *d, int bwd_data);
+/* Which layout that packed copy has, or -1 when there is none: two packed copies of the same filter
+   under the same descriptor and with equal layout ids are identical, so a caller needs only one. */
+int dopt_hip_conv_packed_layout(const dopt_hip_conv_desc *d, int bwd_data);
 int dopt_hip_conv_pack_batch(int n, const dopt_hip_conv_desc *descs, const int *bwd_data,
                              const float *const *w, float *const *packed /* 16-byte aligned */);
 /* bias may be null */
