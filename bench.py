@@ -173,9 +173,12 @@ def main():
             one = 4 * (BATCH * c * h * h + BATCH * k * h * h + k * c * 9)
             conv_bytes += one * (1 if i == 0 else 2)
         result["roofline"] = {
-            "kernel": "conv_patch_k (3x3 implicit-GEMM convolution forward + backward-data, incl. filter pack and split reduction)",
+            "kernel": "conv_patch_k (3x3 implicit-GEMM convolution forward + backward-data of all 13 layers as the plan runs "
+                      "them, incl. filter pack and split reductions; layer 1 and the 2x2-image layers take their own kernels)",
             "bound": "mfma", "achieved": round(gather_tflops, 2), "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": round(gather_tflops / MFMA_FP32_PEAK_TFLOPS, 4), "traffic": traffic,
+            "traffic_of": "conv_patch_k launches only (layers 2-10, 18 of the 25; 25.1 MB algorithmic per launch); the "
+                          "first layer and the 2x2-image layers run other kernels, listed in the same profile",
             "algorithmic_bytes_per_launch": int(conv_bytes / gather_launches),
             "launches_per_step": int(gather_launches),
             "flops_per_launch": round((fwd + bwd_data) / gather_launches, 1),

@@ -1261,15 +1261,26 @@ int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, 
 // (the flipped filter, core/source/dopt/core/ops/nnet.d:270-293) - 4/9 of the multiplications of
 // the nine-tap form.  NCHW needs no rearranging on either side, forward is x * Wd and backward-data
 // is dy * Wd^T, so one copy of Wd serves both directions.
-__global__ __launch_bounds__(256) void pack_2x2_k(unsigned C, unsigned K, const float *w, float *wd)
+__global__ __launch_bounds__(256) void pack_2x2_k(unsigned C, unsigned K, const float *w, float4 *wd)
 {
-    const size_t total = (size_t)16 * C * K;
+    // a lane per (input channel c, output channel k), k fastest: it reads the nine taps of that filter
+    // plane once and writes the four quads (one per input pixel) of column group k; lanes of a
+    // wavefront write neighbouring quads
+    const size_t total = (size_t)C * K;
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
-        const unsigned col = (unsigned)(i % (4 * K)), row = (unsigned)(i / (4 * K));
-        const unsigned k = col >> 2, oy = (col >> 1) & 1, ox = col & 1;
-        const unsigned c = row >> 2, iy = (row >> 1) & 1, ix = row & 1;
-        const unsigned r = iy - oy + 1, s = ix - ox + 1;
-        wd[i] = w[((size_t)k * C + c) * 9 + (2 - r) * 3 + (2 - s)];
+        const unsigned k = (unsigned)(i % K), c = (unsigned)(i / K);
+        const float *src = w + ((size_t)k * C + c) * 9;
+        float f[9];
+#pragma unroll
+        for (int t = 0; t < 9; t++) f[t] = src[t];
+        // input pixel (iy, ix), output pixel (oy, ox): tap (1 - iy + oy, 1 - ix + ox)
+#pragma unroll
+        for (int iy = 0; iy < 2; iy++)
+#pragma unroll
+            for (int ix = 0; ix < 2; ix++) {
+                const int t0 = (1 - iy) * 3 + (1 - ix);
+                wd[((size_t)c * 4 + iy * 2 + ix) * K + k] = make_float4(f[t0], f[t0 + 1], f[t0 + 3], f[t0 + 4]);
+            }
     }
 }
 
@@ -1283,10 +1294,10 @@ size_t dense2x2_elems(const dopt_hip_conv_desc *d) { return (size_t)16 * d->C * 
 
 int dense2x2_pack(const dopt_hip_conv_desc *d, const float *w, float *wd)
 {
-    const size_t blocks = ceil_div(dense2x2_elems(d), (size_t)256);
+    const size_t blocks = ceil_div(dense2x2_elems(d) / 16, (size_t)256);
     const size_t cap = (size_t)num_cus() * 16;
     hipLaunchKernelGGL(pack_2x2_k, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0, stream(), (unsigned)d->C,
-                       (unsigned)d->K, w, wd);
+                       (unsigned)d->K, w, (float4 *)wd);   // pool and plan buffers are 256-byte aligned
     DOPT_LAUNCH_CHECK();
     return DOPT_HIP_OK;
 }
