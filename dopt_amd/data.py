@@ -101,7 +101,10 @@ class PinnedArray:
     def __del__(self):
         if getattr(self, "ptr", None):
             self.array = None
-            capi.load().dopt_hip_host_free(self.ptr)
+            try:
+                capi.load().dopt_hip_host_free(self.ptr)
+            except Exception:   # interpreter shutdown: the library may already be gone
+                pass
             self.ptr = None
 
 
