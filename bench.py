@@ -35,7 +35,7 @@ def conv_flops(n, c, k, h):
     return 2.0 * n * k * c * 9 * h * h
 
 
-def build_step(batch, fused, views, timing, seed=0, fuse=True, overlap=False):
+def build_step(batch, fused, views, timing, seed=0, fuse=True, overlap=False, graph=False):
     from dopt_amd import core, nnet, online, ops
     rng = np.random.default_rng(seed)
     features = core.float32([batch, 3, 32, 32])
@@ -47,6 +47,7 @@ def build_step(batch, fused, views, timing, seed=0, fuse=True, overlap=False):
     flags = (core.PLAN_VIEWS if views else 0) | (core.PLAN_TIMING if timing else 0)
     flags |= core.PLAN_FUSE if (fuse and views) else 0
     flags |= core.PLAN_OVERLAP if overlap else 0
+    flags |= core.PLAN_GRAPH if (graph and not timing) else 0
     if fused:
         updater = online.fused_sgd([loss, preds.trainOutput], net.params, net.paramProj, 0.01, 0.0, flags=flags)
     else:
@@ -95,6 +96,7 @@ def main():
     ap.add_argument("--no-views", action="store_true", help="disable the copy-eliding plan rewrites")
     ap.add_argument("--no-fuse", action="store_true", help="run every operation as its own kernel")
     ap.add_argument("--overlap", action="store_true", help="run the filter gradients on a second queue")
+    ap.add_argument("--graph", action="store_true", help="replay the step's kernels as a recorded HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-kernel-timing", action="store_true", help="skip the per-kernel event pass")
     a = ap.parse_args()
@@ -105,7 +107,7 @@ def main():
     capi.check(capi.load().dopt_hip_init(0))
     fused, views, fuse = not a.unfused, not a.no_views, not a.no_fuse
 
-    updater, args, net = build_step(BATCH, fused, views, timing=False, fuse=fuse, overlap=a.overlap)
+    updater, args, net = build_step(BATCH, fused, views, timing=False, fuse=fuse, overlap=a.overlap, graph=a.graph)
     for _ in range(a.warmup):
         updater.step_async(args)
     ops.sync()

@@ -76,6 +76,7 @@ def _lib():
             "dopt_hip_plan_execute": [vp, i, C.POINTER(i), C.POINTER(vp), C.POINTER(i), i, C.POINTER(vp)],
             "dopt_hip_plan_result": [vp, i, C.POINTER(vp), C.POINTER(sz)],
             "dopt_hip_plan_stats": [vp, C.POINTER(sz), C.POINTER(sz)],
+            "dopt_hip_plan_recordings": [vp, C.POINTER(sz), C.POINTER(sz)],
             "dopt_hip_plan_profile": [vp, C.c_char_p, sz, C.POINTER(sz)],
             "dopt_hip_plan_destroy": [vp],
         }
@@ -91,7 +92,7 @@ PLAN_SYMBOLS = ["dopt_hip_graph_create", "dopt_hip_graph_destroy", "dopt_hip_gra
                 "dopt_hip_graph_set_attr_sizes", "dopt_hip_graph_set_attr_double", "dopt_hip_graph_value",
                 "dopt_hip_graph_op_type", "dopt_hip_graph_op_dep", "dopt_hip_register_kernel",
                 "dopt_hip_deregister_kernel", "dopt_hip_list_operations", "dopt_hip_plan_create",
-                "dopt_hip_plan_execute", "dopt_hip_plan_result", "dopt_hip_plan_stats", "dopt_hip_plan_profile",
+                "dopt_hip_plan_execute", "dopt_hip_plan_result", "dopt_hip_plan_stats", "dopt_hip_plan_recordings", "dopt_hip_plan_profile",
                 "dopt_hip_plan_destroy"]
 
 
@@ -694,6 +695,7 @@ PLAN_VIEWS = 1
 PLAN_TIMING = 2
 PLAN_FUSE = 4
 PLAN_OVERLAP = 8
+PLAN_GRAPH = 16
 
 
 class Plan:
@@ -755,6 +757,11 @@ class Plan:
         k, b = C.c_size_t(), C.c_size_t()
         capi.check(_lib().dopt_hip_plan_stats(self._h, C.byref(k), C.byref(b)))
         return {"kernels": k.value, "buffer_bytes": b.value}
+
+    def recordings(self):
+        a, b = C.c_size_t(), C.c_size_t()
+        capi.check(_lib().dopt_hip_plan_recordings(self._h, C.byref(a), C.byref(b)))
+        return {"recorded": a.value, "replays": b.value}
 
     def profile(self):
         need = C.c_size_t()

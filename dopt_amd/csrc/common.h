@@ -29,6 +29,11 @@ void *workspace(size_t bytes);
 // switched to the side queue for a step it overlaps with its main chain (set_lane(1) ... set_lane(0));
 // each queue has its own workspace.
 void set_lane(int lane);
+// While a plan records its kernels into a HIP graph, entry points that would allocate or fill
+// device memory fail instead (neither can be replayed), and the plan runs its kernels directly.
+void set_capturing(bool on);
+bool capturing();
+int scratch_alloc(void **ptr, size_t bytes);   // pooled block, NOT zero-filled; release with dopt_hip_free
 // sgemm.hip: C = op(A) * op(B) (+ colbias[col >> bias_shift] per element when colbias is given and the
 // shape takes a kernel with that epilogue; *biased says whether it did).
 int sgemm_bias(int transA, int transB, size_t M, size_t N, size_t K, const float *A, const float *B, float *C,

@@ -1309,7 +1309,7 @@ int run_dense2x2(const dopt_hip_conv_desc *d, const float *in, const float *w, c
 {
     void *mine = nullptr;   // from the pool, not the workspace: the product below may use the workspace itself
     if (!wd) {
-        if (int rc = dopt_hip_malloc(&mine, dense2x2_elems(d) * sizeof(float))) return rc;
+        if (int rc = scratch_alloc(&mine, dense2x2_elems(d) * sizeof(float))) return rc;
         if (int rc = dense2x2_pack(d, w, (float *)mine)) {
             dopt_hip_free(mine);
             return rc;
@@ -1400,7 +1400,10 @@ int run_gather(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in,
     float *partial = (float *)(ws + wp_bytes);
 
     // pack the filter
-    if (g.CinPad != g.Cin || g.Mp != g.Mout) DOPT_HIP_CHECK(hipMemsetAsync(wp, 0, wp_elems * sizeof(float), stream()));
+    if (g.CinPad != g.Cin || g.Mp != g.Mout) {
+        if (capturing()) return fail(DOPT_HIP_ERR_UNSUPPORTED, "convolution: a fill cannot be recorded into a graph");
+        DOPT_HIP_CHECK(hipMemsetAsync(wp, 0, wp_elems * sizeof(float), stream()));
+    }
     const int K = (int)d->K, C = (int)d->C;
     if (!kBwd) {
         dim3 grid((unsigned)((K + 63) / 64), (unsigned)((C * taps + 63) / 64));

@@ -1075,6 +1075,11 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
             for (hipEvent_t &ev : p->mFences) DOPT_HIP_CHECK(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
         }
     }
+    // what a recorded graph cannot reproduce: per-kernel timing events, the second queue, and `uniform`,
+    // whose kernel takes a call counter that changes with every execution
+    p->mGraphOk = !(flags & DOPT_HIP_PLAN_TIMING) && !p->mUsesSide;
+    for (const Step &st : p->mSteps)
+        if (st.op >= 0 && g.ops[st.op].opType == "uniform") p->mGraphOk = false;
     if (flags & DOPT_HIP_PLAN_TIMING) {
         p->mEvents.resize(p->mSteps.size());
         for (auto &ev : p->mEvents) {
@@ -1105,6 +1110,11 @@ void HIPPlan::cleanup()
     mEvents.clear();
     for (hipEvent_t ev : mFences) (void)hipEventDestroy(ev);
     mFences.clear();
+    for (CapturedRun &c : mRuns) {
+        if (c.exec) (void)hipGraphExecDestroy(c.exec);
+        if (c.graph) (void)hipGraphDestroy(c.graph);
+    }
+    mRuns.clear();
     mClean = true;
 }
 
@@ -1138,12 +1148,10 @@ int HIPPlan::resolve(int nargs, const int *argOps, const void *const *argPtrs, c
     return DOPT_HIP_OK;
 }
 
-int HIPPlan::execute(int nargs, const int *argOps, const void *const *argPtrs, const int *argOnHost, int nrets,
-                     void *const *rets)
+// The kernels of one execution, in order, on whatever the library's queues are; shared by the direct
+// path and by graph capture.
+int HIPPlan::enqueue(int nrets, void *const *rets)
 {
-    if (mClean) return fail(DOPT_HIP_ERR_INVALID, "plan was cleaned up");
-    if (nrets > (int)mOutputs.size()) return fail(DOPT_HIP_ERR_INVALID, "more return buffers than plan outputs");
-    if (int rc = resolve(nargs, argOps, argPtrs, argOnHost)) return rc;
     const bool timing = !mEvents.empty();
     size_t fence = 0;
     auto order = [&](int first, int then) -> int {   // work queued on `then` from here on follows all of `first` so far
@@ -1192,6 +1200,67 @@ int HIPPlan::execute(int nargs, const int *argOps, const void *const *argPtrs, c
         mRetBytes.push_back(mGraph->ops[o].bytes());
     }
     return dopt_hip_copy_d2d_batch((int)mRetDst.size(), mRetDst.data(), mRetSrc.data(), mRetBytes.data());
+}
+
+int HIPPlan::execute(int nargs, const int *argOps, const void *const *argPtrs, const int *argOnHost, int nrets,
+                     void *const *rets)
+{
+    if (mClean) return fail(DOPT_HIP_ERR_INVALID, "plan was cleaned up");
+    if (nrets > (int)mOutputs.size()) return fail(DOPT_HIP_ERR_INVALID, "more return buffers than plan outputs");
+
+    // DOPT_HIP_PLAN_GRAPH: an execution is identified by the device pointers it binds (arguments and
+    // return buffers).  The first execution with a given binding runs directly (run-time compilation,
+    // workspace growth and pool allocations all happen there), the second is recorded into a HIP
+    // graph while it runs, later ones replay that graph with one launch.
+    bool graphable = mGraphOk && (mFlags & DOPT_HIP_PLAN_GRAPH);
+    for (int a = 0; a < nargs && graphable; a++) graphable = !argOnHost[a];   // a host argument is uploaded anew every time
+    if (graphable) {
+        std::vector<const void *> key;
+        for (int a = 0; a < nargs; a++) {
+            key.push_back((const void *)(intptr_t)argOps[a]);
+            key.push_back(argPtrs[a]);
+        }
+        key.push_back(nullptr);
+        for (int i = 0; i < nrets; i++) key.push_back(rets[i]);
+        CapturedRun *run = nullptr;
+        for (CapturedRun &c : mRuns)
+            if (c.key == key) run = &c;
+        if (run && run->exec) {
+            mReplays++;
+            DOPT_HIP_CHECK(hipGraphLaunch(run->exec, stream()));
+            return DOPT_HIP_OK;
+        }
+        if (!run) {
+            if (mRuns.size() >= 8) {   // bindings keep changing: drop the oldest recording
+                if (mRuns.front().exec) (void)hipGraphExecDestroy(mRuns.front().exec);
+                if (mRuns.front().graph) (void)hipGraphDestroy(mRuns.front().graph);
+                mRuns.erase(mRuns.begin());
+            }
+            mRuns.push_back(CapturedRun{key, nullptr, nullptr});
+        } else {
+            if (int rc = resolve(nargs, argOps, argPtrs, argOnHost)) return rc;
+            DOPT_HIP_CHECK(hipStreamBeginCapture(stream(), hipStreamCaptureModeRelaxed));
+            set_capturing(true);
+            const int rc = enqueue(nrets, rets);
+            set_capturing(false);
+            hipGraph_t graph = nullptr;
+            const hipError_t ended = hipStreamEndCapture(stream(), &graph);
+            if (rc == DOPT_HIP_OK && ended == hipSuccess && graph &&
+                hipGraphInstantiate(&run->exec, graph, nullptr, nullptr, 0) == hipSuccess) {
+                run->graph = graph;
+                DOPT_HIP_CHECK(hipGraphLaunch(run->exec, stream()));
+                return DOPT_HIP_OK;
+            }
+            // something in this plan cannot be recorded (an allocation, a fill): nothing ran, run it directly from now on
+            (void)hipGetLastError();
+            if (graph) (void)hipGraphDestroy(graph);
+            run->exec = nullptr;
+            mGraphOk = false;
+            clear_error();
+        }
+    }
+    if (int rc = resolve(nargs, argOps, argPtrs, argOnHost)) return rc;
+    return enqueue(nrets, rets);
 }
 
 int HIPPlan::result(int op, void **ptr, size_t *bytes) const
@@ -1402,6 +1471,13 @@ int dopt_hip_plan_stats(void *plan, size_t *kernels, size_t *buffer_bytes)
     DOPT_REQUIRE(plan != nullptr, "dopt_hip_plan_stats: plan is null");
     if (kernels) *kernels = ((HIPPlan *)plan)->kernelCount();
     if (buffer_bytes) *buffer_bytes = ((HIPPlan *)plan)->bufferBytes();
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_plan_recordings(void *plan, size_t *recorded, size_t *replays)
+{
+    DOPT_REQUIRE(plan != nullptr, "dopt_hip_plan_recordings: plan is null");
+    ((HIPPlan *)plan)->recordings(recorded, replays);
     return DOPT_HIP_OK;
 }
 

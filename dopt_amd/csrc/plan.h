@@ -82,6 +82,13 @@ public:
                 void *const *rets);
     int result(int op, void **ptr, size_t *bytes) const;
     size_t kernelCount() const { return mSteps.size(); }
+    void recordings(size_t *recorded, size_t *replays) const
+    {
+        size_t n = 0;
+        for (const CapturedRun &c : mRuns) n += c.exec != nullptr;
+        if (recorded) *recorded = n;
+        if (replays) *replays = mReplays;
+    }
     size_t bufferBytes() const { return mBufferBytes; }
     std::string profile();
     std::map<std::string, std::pair<double, size_t>> profiler;  // opType -> (microseconds, executions)
@@ -112,6 +119,15 @@ private:
     std::vector<std::pair<hipEvent_t, hipEvent_t>> mEvents;
     std::vector<hipEvent_t> mFences;             // ordering between the two queues, one per crossing
     bool mUsesSide = false;
+    struct CapturedRun {
+        std::vector<const void *> key;           // argument ops and pointers, return pointers
+        hipGraph_t graph;
+        hipGraphExec_t exec;                     // null until the second execution with this key
+    };
+    std::vector<CapturedRun> mRuns;
+    bool mGraphOk = false;
+    size_t mReplays = 0;
+    int enqueue(int nrets, void *const *rets);
     size_t mBufferBytes = 0;
     bool mClean = false;
     std::vector<void *> mRetDst;                 // scratch of execute(): the return copies

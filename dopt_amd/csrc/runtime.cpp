@@ -26,6 +26,7 @@ struct Runtime {
     hipStream_t stream = nullptr;
     hipStream_t side = nullptr;     // second in-order queue for work a plan overlaps with its main chain
     int lane = 0;                   // which of the two the entry points currently enqueue on
+    bool capturing = false;         // a plan is recording its kernels into a HIP graph
 
     // pool
     std::unordered_map<void *, size_t> live;           // ptr -> class size
@@ -115,6 +116,8 @@ bool ensure_init()
 hipStream_t stream() { return rt().lane ? rt().side : rt().stream; }
 hipStream_t lane_stream(int lane) { return lane ? rt().side : rt().stream; }
 void set_lane(int lane) { rt().lane = lane ? 1 : 0; }
+void set_capturing(bool on) { rt().capturing = on; }
+bool capturing() { return rt().capturing; }
 int num_cus() { return rt().cus; }
 
 void *workspace(size_t bytes)
@@ -122,6 +125,10 @@ void *workspace(size_t bytes)
     Runtime &r = rt();
     const int l = r.lane;
     if (bytes <= r.ws_bytes[l]) return r.ws[l];
+    if (r.capturing) {   // allocation cannot be recorded; the plan falls back to running its kernels directly
+        fail(DOPT_HIP_ERR_UNSUPPORTED, "workspace: cannot grow to %zu bytes while a graph is being captured", bytes);
+        return nullptr;
+    }
     // Growing: earlier users were enqueued on the same queue, and hipFree waits for the device.
     if (r.ws[l]) (void)hipFree(r.ws[l]);
     r.ws[l] = nullptr;
@@ -243,13 +250,16 @@ int dopt_hip_shutdown(void)
 
 const char *dopt_hip_last_error(void) { return g_last_error.c_str(); }
 
-int dopt_hip_malloc(void **ptr, size_t bytes)
+// zero = false: a pooled block without the fill, for scratch that its user overwrites entirely
+static int pool_take(void **ptr, size_t bytes, bool zero)
 {
     DOPT_REQUIRE(ptr != nullptr, "dopt_hip_malloc: ptr is null");
     *ptr = nullptr;
     if (bytes == 0) return DOPT_HIP_OK;
     DOPT_ENSURE_INIT();
     Runtime &r = rt();
+    if (r.capturing && zero)
+        return fail(DOPT_HIP_ERR_UNSUPPORTED, "dopt_hip_malloc: a zero-filled allocation cannot be recorded into a graph");
     std::lock_guard<std::mutex> lk(r.mu);
     size_t cls = size_class(bytes);
     void *p = nullptr;
@@ -259,6 +269,8 @@ int dopt_hip_malloc(void **ptr, size_t bytes)
         it->second.pop_back();
         r.cached_bytes -= cls;
     } else {
+        if (r.capturing)
+            return fail(DOPT_HIP_ERR_UNSUPPORTED, "dopt_hip_malloc: a device allocation cannot be recorded into a graph");
         hipError_t e = hipMalloc(&p, cls);
         if (e != hipSuccess) {
             // give cached blocks back to the driver and retry once
@@ -275,7 +287,7 @@ int dopt_hip_malloc(void **ptr, size_t bytes)
         }
         r.device_allocs++;
     }
-    hipError_t e = hipMemsetAsync(p, 0, bytes, r.stream);
+    hipError_t e = zero ? hipMemsetAsync(p, 0, bytes, r.stream) : hipSuccess;
     if (e != hipSuccess) {
         r.cached[cls].push_back(p);
         r.cached_bytes += cls;
@@ -286,6 +298,8 @@ int dopt_hip_malloc(void **ptr, size_t bytes)
     *ptr = p;
     return DOPT_HIP_OK;
 }
+
+int dopt_hip_malloc(void **ptr, size_t bytes) { return pool_take(ptr, bytes, true); }
 
 int dopt_hip_free(void *ptr)
 {
@@ -330,6 +344,7 @@ int dopt_hip_memset(void *dst, int byte_value, size_t bytes)
     if (bytes == 0) return DOPT_HIP_OK;
     DOPT_REQUIRE(dst != nullptr, "dopt_hip_memset: dst is null");
     DOPT_ENSURE_INIT();
+    if (rt().capturing) return fail(DOPT_HIP_ERR_UNSUPPORTED, "dopt_hip_memset: a fill cannot be recorded into a graph");
     DOPT_HIP_CHECK(hipMemsetAsync(dst, byte_value, bytes, stream()));
     return DOPT_HIP_OK;
 }
@@ -439,3 +454,9 @@ int dopt_hip_event_destroy(void *event)
 }
 
 }  // extern "C"
+
+namespace dopt {
+
+int scratch_alloc(void **ptr, size_t bytes) { return pool_take(ptr, bytes, false); }
+
+}  // namespace dopt

@@ -75,6 +75,10 @@ enum {
     DOPT_HIP_PLAN_FUSE = 4,   /* with VIEWS: run adjacent operations as one kernel where the middle value
                                  has no other reader -- addBias(convolution), relu(batchNormTrain.y) and
                                  batchNormGrad(reluGrad) -- with the values of the separate kernels */
+    DOPT_HIP_PLAN_GRAPH = 16, /* executions whose arguments and return buffers are all device pointers are
+                                 recorded into a HIP graph the second time a given set of pointers is bound
+                                 and replayed with one launch from then on (plans with per-kernel timing, the
+                                 second queue, a `uniform` operation, or a kernel that allocates stay direct) */
     DOPT_HIP_PLAN_OVERLAP = 8 /* filter gradients, and whatever only they feed, run on a second in-order
                                  queue beside the chain that produces the feature gradients; the queues
                                  are ordered by events where a value crosses, and joined before the
@@ -95,6 +99,9 @@ int dopt_hip_plan_execute(void *plan, int nargs, const int *arg_ops, const void 
 int dopt_hip_plan_result(void *plan, int op, void **device_ptr, size_t *bytes);
 /* Number of kernel executions one plan execution issues, and the plan's device footprint. */
 int dopt_hip_plan_stats(void *plan, size_t *kernels, size_t *buffer_bytes);
+/* With DOPT_HIP_PLAN_GRAPH: how many argument bindings are currently recorded as HIP graphs, and how
+   many executions so far were replays of one. */
+int dopt_hip_plan_recordings(void *plan, size_t *recorded, size_t *replays);
 /* CUDAPlan.profiler (cuda/package.d:265): accumulated device microseconds per op type as
    "opType usec count\n" lines; needs DOPT_HIP_PLAN_TIMING. */
 int dopt_hip_plan_profile(void *plan, char *buf, size_t buf_bytes, size_t *needed);

@@ -406,3 +406,44 @@ def test_overlapped_filter_gradients_change_nothing(maker):
     assert runs[0][0] == runs[1][0]
     for a, b in zip(runs[0][1], runs[1][1]):
         assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("maker", [online.fused_sgd, online.adam])
+def test_recorded_graph_replays_match_direct_execution(maker):
+    """DOPT_HIP_PLAN_GRAPH: the first execution with a set of device pointers runs directly, the second
+    is recorded, later ones are replays.  Two identically seeded networks take the same steps, one
+    through replays and one directly, with the direct one's kernels and host reads interleaved between
+    the replays; every loss and, at the end, every parameter must be identical."""
+    r = np.random.default_rng(0)
+    batches = [(ops.tensor(r.standard_normal((16, 3, 16, 16)).astype(np.float32)),
+                ops.tensor(np.eye(10, dtype=np.float32)[r.integers(0, 10, 16)])) for _ in range(2)]
+    base = core.PLAN_VIEWS | core.PLAN_FUSE
+    xa, ya, neta, lossa = _small_convnet(9)
+    xb, yb, netb, lossb = _small_convnet(9)
+    direct = maker([lossa], neta.params, neta.paramProj, flags=base)
+    replay = maker([lossb], netb.params, netb.paramProj, flags=base | core.PLAN_GRAPH)
+    for step in range(8):
+        fx, fy = batches[step % 2]        # two bindings: two recordings, each replayed three times
+        la = direct({xa: fx, ya: fy})[0]
+        lb = replay({xb: fx, yb: fy})[0]
+        assert la == lb, step
+    for a, b in zip(neta.params, netb.params):
+        assert np.array_equal(a.value, b.value)
+    assert replay.plan.recordings() == {"recorded": 2, "replays": 4}      # per binding: direct, recorded, 2 replays
+    assert direct.plan.recordings() == {"recorded": 0, "replays": 0}
+    # host arrays as arguments: every execution uploads anew, so nothing is recorded and nothing breaks
+    lb = replay({xb: batches[0][0].numpy(), yb: batches[0][1].numpy()})[0]
+    la = direct({xa: batches[0][0].numpy(), ya: batches[0][1].numpy()})[0]
+    assert la == lb
+
+
+def test_graph_flag_leaves_plans_with_random_draws_direct():
+    x = core.float32([64], np.ones(64, np.float32))
+    y = core.uniformSample([64]) * x
+    plan = core.compile([y], core.PLAN_VIEWS | core.PLAN_FUSE | core.PLAN_GRAPH)
+    out = ops.Tensor([64])
+    draws = []
+    for _ in range(4):
+        plan.execute(None, [out])
+        draws.append(out.numpy().copy())
+    assert all(not np.array_equal(draws[0], d) for d in draws[1:])     # a replayed kernel would repeat its draws
