@@ -107,3 +107,51 @@ def test_chain_keeps_values_that_something_else_reads():
     got = core.compile([t, s, u], core.PLAN_VIEWS | core.PLAN_FUSE).execute()
     for g, w in zip(got, want):
         assert np.array_equal(g, w)
+
+
+def _random_graph(r, n_leaves=4, n_ops=18, size=96):
+    """A random DAG over [size]-vectors and [8, size/8] matrices: pointwise nodes, scalar broadcasts,
+    reshapes, contiguous slices padded back, reductions as side consumers, a few outputs in the middle."""
+    shape2 = [8, size // 8]
+    pool = [core.float32([size], (np.abs(r.standard_normal(size)) + 0.5).astype(np.float32)) for _ in range(n_leaves)]
+    scalars = [core.float32([], [float(r.uniform(0.5, 1.5))]) for _ in range(2)]
+    outputs = []
+    for _ in range(n_ops):
+        kind = r.integers(0, 10)
+        a = pool[r.integers(0, len(pool))]
+        b = pool[r.integers(0, len(pool))]
+        if kind <= 3:
+            node = [core.add, core.sub, core.mul, core.max][kind](a, b)
+        elif kind == 4:
+            node = core.abs(a) if r.integers(0, 2) else core.sqrt(core.abs(a))
+        elif kind == 5:
+            node = a * scalars[r.integers(0, 2)]                    # repeat(scalar) + reshape + mul
+        elif kind == 6:
+            node = core.reshape(core.reshape(a, shape2) * core.reshape(b, shape2), [size])
+        elif kind == 7:
+            half = size // 2
+            lo = core.slice(a, [0], [half])                         # a view under PLAN_VIEWS
+            node = core.pad(lo * lo, [0], [size - half])
+        elif kind == 8:
+            node = a + core.sum(b) * 0.01                           # a reduction reads b, its result is broadcast
+        else:
+            node = core.min(core.exp(a * 0.1), b)
+        pool.append(node)
+        if r.integers(0, 4) == 0:
+            outputs.append(node)                                    # exposed in the middle of a would-be chain
+    outputs.append(pool[-1])
+    outputs.append(core.sum(pool[-2]))
+    return outputs
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_graphs_give_the_same_values_with_every_rewrite(seed):
+    outs = _random_graph(np.random.default_rng(100 + seed))
+    want = core.compile(outs).execute()
+    for flags in (core.PLAN_VIEWS, core.PLAN_VIEWS | core.PLAN_FUSE, core.PLAN_VIEWS | core.PLAN_FUSE | core.PLAN_GRAPH):
+        plan = core.compile(outs, flags)
+        bufs = [ops.Tensor(o.shape) for o in outs]
+        for _ in range(3):                                           # direct, recorded, replayed
+            plan.execute(None, bufs)
+            for got, w in zip(bufs, want):
+                assert np.array_equal(got.numpy(), w, equal_nan=True), flags
