@@ -1148,7 +1148,8 @@ PatchSetup patch_setup(const dopt_hip_conv_desc *d, size_t P, size_t Q)
     }
     pc.ncols = pc.N * pc.OH * pc.OW;
     int npmax, threads;
-    if (pc.Mout <= 64) {
+    // 64-row tiles for up to 64 output channels, and wherever 128-row tiles would pad more (160 -> 192, not 256)
+    if (pc.Mout <= 64 || (pc.Mout + 63) / 64 * 64 < (pc.Mout + 127) / 128 * 128) {
         u.shape = 0; u.BM = 64; u.BN = 256; u.blocks_wanted = 2 * num_cus(); npmax = 24; threads = 256;
     } else {
         u.BM = 128; u.BN = 128;
@@ -1493,7 +1494,8 @@ int run_wgrad_patch(const dopt_hip_conv_desc *d, const float *dy, const float *x
         return DOPT_HIP_OK;
     }
     while (wp.cstride % 8 != 4) wp.cstride += 4;  // 128-bit reads by 32 channels at this stride touch every LDS bank once
-    const bool tall = d->K >= 128;  // 128 rows x 32 channels, else 64 x 64
+    // 128 rows x 32 channels, or 64 x 64 when that pads the output channels less (160 -> 192, not 256)
+    const bool tall = d->K >= 128 && (d->K + 127) / 128 * 128 <= (d->K + 63) / 64 * 64;
     if (!tall && W == 64) return DOPT_HIP_OK;
     const int BM = tall ? 128 : 64, BC = tall ? 32 : 64;
     wp.dy = dy; wp.x = x;
