@@ -44,6 +44,10 @@ struct GatherConv {
     int CinPad, Mp, ncols;
     int mtiles, ntiles, slabs_total, slabs_per_split, splits;
     size_t out_elems, in_bytes, wp_bytes;
+    // where output pixel (oh, ow) of this problem lands: row oh * out_sy + out_oy, column ow * out_sx +
+    // out_ox of a plane of out_plane elements and out_OW columns (the whole tensor, or every
+    // stride-th pixel of it when a strided backward-data pass is run class by class)
+    int out_plane, out_OW, out_sy, out_sx, out_oy, out_ox;
 };
 
 // kMode: 0 = forward, 1 = backward-data with unit stride (no divisions), 2 = backward-data, any stride
@@ -173,13 +177,15 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_gather_k(Ga
         const int col = n0 + wn * (BN / T::WN) + j * 32 + (lane & 31);
         if (col >= p.ncols) continue;
         const int n2 = col / OHW, pq2 = col - n2 * OHW;
-        float *base = outp + (size_t)n2 * p.Mout * OHW + pq2;
+        const int oh2 = pq2 / p.OW, ow2 = pq2 - oh2 * p.OW;
+        float *base = outp + (size_t)n2 * p.Mout * p.out_plane + (size_t)(oh2 * p.out_sy + p.out_oy) * p.out_OW +
+                      ow2 * p.out_sx + p.out_ox;
 #pragma unroll
         for (int i = 0; i < T::MI; i++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int m = m0 + wm * (BM / T::WM) + i * 32 + acc_row(v, lane);
-                if (m < p.Mout) base[(size_t)m * OHW] = acc[i][j][v];
+                if (m < p.Mout) base[(size_t)m * p.out_plane] = acc[i][j][v];
             }
     }
 }
@@ -1329,6 +1335,157 @@ int run_dense2x2(const dopt_hip_conv_desc *d, const float *in, const float *w, c
     return rc;
 }
 
+// Packs the filter w[K][C][g.R * g.S] and runs conv_gather_k on a problem whose geometry the caller
+// has filled in (dimensions, padding, stride, output placement).  mode as conv_gather_k's kMode.
+int gather_launch(GatherConv g, int mode, int K, int C, const float *in, const float *w, float *out)
+{
+    const bool bwd = mode != 0;
+    const int taps = g.R * g.S;
+    g.CinPad = round_up(g.Cin, BK);
+    g.Mp = round_up(g.Mout, 4);
+    g.ncols = g.N * g.OH * g.OW;
+    g.slabs_total = taps * g.CinPad / BK;
+    g.out_elems = (size_t)g.ncols * g.Mout;
+    const bool dense = g.out_sy == 1 && g.out_sx == 1 && g.out_plane == g.OH * g.OW;
+
+    // tile shape: 64-row tiles for <= 64 output channels and wherever 128-row tiles would pad more;
+    // otherwise 128x128, with 8 wavefronts per workgroup when there are too few tiles to give every
+    // CU two 4-wavefront workgroups
+    enum { kWide, kSquare, kDeep } shape;
+    int BM, BN, blocks_wanted;
+    if (g.Mout <= 64 || (g.Mout + 63) / 64 * 64 < (g.Mout + 127) / 128 * 128) {
+        shape = kWide; BM = 64; BN = 256; blocks_wanted = 2 * num_cus();
+    } else {
+        BM = 128; BN = 128;
+        const int t = ((g.Mout + 127) / 128) * ((g.ncols + 127) / 128);
+        if (t >= 2 * num_cus()) { shape = kSquare; blocks_wanted = 2 * num_cus(); }
+        else { shape = kDeep; blocks_wanted = num_cus(); }
+    }
+    g.mtiles = (g.Mout + BM - 1) / BM;
+    g.ntiles = (g.ncols + BN - 1) / BN;
+    const int tiles = g.mtiles * g.ntiles;
+    int splits = pick_splits(tiles, g.slabs_total, blocks_wanted, 64);
+    // the split reduction works on float4 over a dense output
+    if (g.out_elems % 4 != 0 || !aligned16(out) || !dense) splits = 1;
+    g.slabs_per_split = (g.slabs_total + splits - 1) / splits;
+    splits = (g.slabs_total + g.slabs_per_split - 1) / g.slabs_per_split;  // no empty split
+    g.splits = splits;
+
+    const size_t wp_elems = (size_t)taps * g.CinPad * g.Mp;
+    const size_t wp_bytes = (wp_elems * sizeof(float) + 255) / 256 * 256;
+    const size_t part_bytes = splits > 1 ? (size_t)splits * g.out_elems * sizeof(float) : 0;
+    char *ws = (char *)workspace(wp_bytes + part_bytes);
+    if (!ws) return DOPT_HIP_ERR_OOM;
+    float *wp = (float *)ws;
+    float *partial = (float *)(ws + wp_bytes);
+
+    // pack the filter
+    if (g.CinPad != g.Cin || g.Mp != g.Mout) {
+        if (capturing()) return fail(DOPT_HIP_ERR_UNSUPPORTED, "convolution: a fill cannot be recorded into a graph");
+        DOPT_HIP_CHECK(hipMemsetAsync(wp, 0, wp_elems * sizeof(float), stream()));
+    }
+    if (!bwd) {
+        dim3 grid((unsigned)((K + 63) / 64), (unsigned)((C * taps + 63) / 64));
+        hipLaunchKernelGGL(pack_fwd_k, grid, dim3(256), 0, stream(), K, C, taps, g.CinPad, g.Mp, w, wp);
+    } else {
+        dim3 grid((unsigned)K, (unsigned)((C + 63) / 64));
+        hipLaunchKernelGGL(pack_bwd_k, grid, dim3(256), (size_t)64 * taps * sizeof(float), stream(), K, C, taps,
+                           g.CinPad, g.Mp, w, wp);
+    }
+    DOPT_LAUNCH_CHECK();
+
+    g.in = in;
+    g.wp = wp;
+    g.in_bytes = (size_t)g.N * g.Cin * g.IH * g.IW * sizeof(float);
+    g.wp_bytes = wp_elems * sizeof(float);
+    g.out = splits > 1 ? partial : out;
+    dim3 grid(xcd_grid((unsigned)(tiles * splits)));
+#define DOPT_GATHER(TILE)                                                                                      \
+    do {                                                                                                       \
+        if (mode == 0) hipLaunchKernelGGL((conv_gather_k<TILE, 0>), grid, dim3(TILE::THREADS), 0, stream(), g); \
+        else if (mode == 1) hipLaunchKernelGGL((conv_gather_k<TILE, 1>), grid, dim3(TILE::THREADS), 0, stream(), g); \
+        else hipLaunchKernelGGL((conv_gather_k<TILE, 2>), grid, dim3(TILE::THREADS), 0, stream(), g);          \
+    } while (0)
+    if (shape == kWide) DOPT_GATHER(GatherWide);
+    else if (shape == kSquare) DOPT_GATHER(GatherSquare);
+    else DOPT_GATHER(GatherDeep);
+#undef DOPT_GATHER
+    DOPT_LAUNCH_CHECK();
+    if (splits > 1) return launch_splitk_reduce(g.out_elems, splits, partial, out);
+    return DOPT_HIP_OK;
+}
+
+// ---- backward-data with a stride, one residue class of output pixels at a time -------------------
+// dx[n, c, h, w] = sum over k, r, s with (h + padH - r) and (w + padW - s) multiples of the stride of
+// dy[n, k, (h + padH - r) / sH, (w + padW - s) / sW] * w[k, c, R - 1 - r, S - 1 - s] (the flipped filter).  Which taps qualify depends only
+// on (h mod sH, w mod sW).  Taking all pixels together (conv_gather_k mode 2) multiplies every pixel
+// by every tap and masks three quarters of the products of a stride-2 3x3 layer; taking the pixels
+// of one class (a, b) = (h mod sH, w mod sW) at a time, only its taps r = r0, r0 + sH, ... and s = s0,
+// s0 + sW, ... are multiplied, and the class is a UNIT-stride problem on the grid (i, j) = (h / sH, w / sW):
+//     dy row = i + (a + padH - r0) / sH - t   for its t-th tap row,
+// i.e. backward-data of a filter with ceil((R - r0) / sH) rows, padding (a + padH - r0) / sH and rows
+// stored in reverse order of r.  The sub-filter is copied out of w, the kernel's output placement
+// scatters the class back into dx.
+__global__ __launch_bounds__(256) void subfilter_k(int KC, int R, int S, int R2, int S2, int r0, int s0, int sH, int sW,
+                                                    const float *w, float *sub)
+{
+    const int total = KC * R2 * S2;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256) {
+        const int kc = i / (R2 * S2), t = i - kc * (R2 * S2), tr = t / S2, ts = t - tr * S2;
+        // stored row tr of the sub-filter stands for tap offset r = r0 + (R2 - 1 - tr) * sH, and the filter
+        // element that multiplies offset r is the flipped one, w[.., R - 1 - r, S - 1 - s]
+        const int r = r0 + (R2 - 1 - tr) * sH, sc = s0 + (S2 - 1 - ts) * sW;
+        sub[i] = w[(size_t)kc * (R * S) + (R - 1 - r) * S + (S - 1 - sc)];
+    }
+}
+
+int run_bwd_strided(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *dy, const float *w, float *dx)
+{
+    const int sH = (int)d->strideH, sW = (int)d->strideW, R = (int)d->R, S = (int)d->S;
+    const int H = (int)d->H, W = (int)d->W, padH = (int)d->padH, padW = (int)d->padW;
+    struct Cls { int n, first, taps, pad; };   // pixels of the class along one axis, its first tap, tap count, padding
+    auto cls = [](int a, int extent, int stride, int pad, int filt) {
+        Cls c{};
+        c.n = a < extent ? (extent - a + stride - 1) / stride : 0;
+        c.first = (a + pad) % stride;
+        c.taps = c.first < filt ? (filt - c.first + stride - 1) / stride : 0;
+        c.pad = (a + pad - c.first) / stride;
+        return c;
+    };
+    bool gaps = false;   // classes no tap reaches: those pixels of dx are zero
+    for (int a = 0; a < sH; a++) gaps = gaps || (cls(a, H, sH, padH, R).n > 0 && cls(a, H, sH, padH, R).taps == 0);
+    for (int b = 0; b < sW; b++) gaps = gaps || (cls(b, W, sW, padW, S).n > 0 && cls(b, W, sW, padW, S).taps == 0);
+    if (gaps)
+        if (int rc = dopt_hip_memset(dx, 0, d->N * d->C * d->H * d->W * sizeof(float))) return rc;
+    void *sub = nullptr;
+    if (int rc = scratch_alloc(&sub, d->K * d->C * d->R * d->S * sizeof(float))) return rc;
+    int rc = DOPT_HIP_OK;
+    for (int a = 0; a < sH && !rc; a++)
+        for (int b = 0; b < sW && !rc; b++) {
+            const Cls ch = cls(a, H, sH, padH, R), cw = cls(b, W, sW, padW, S);
+            if (ch.n == 0 || cw.n == 0 || ch.taps == 0 || cw.taps == 0) continue;
+            const int KC = (int)(d->K * d->C);
+            hipLaunchKernelGGL(subfilter_k, dim3((unsigned)ceil_div((size_t)KC * ch.taps * cw.taps, (size_t)256)), dim3(256), 0,
+                               stream(), KC, R, S, ch.taps, cw.taps, ch.first, cw.first, sH, sW, w, (float *)sub);
+            if (hipGetLastError() != hipSuccess) {
+                rc = fail(DOPT_HIP_ERR_RUNTIME, "convolution: sub-filter launch failed");
+                break;
+            }
+            GatherConv g{};
+            g.N = (int)d->N;
+            g.R = ch.taps; g.S = cw.taps;
+            g.padH = ch.pad; g.padW = cw.pad;
+            g.strideH = g.strideW = 1;
+            g.Cin = (int)d->K; g.IH = (int)P; g.IW = (int)Q;
+            g.Mout = (int)d->C; g.OH = ch.n; g.OW = cw.n;
+            g.out_plane = H * W; g.out_OW = W;
+            g.out_sy = sH; g.out_sx = sW; g.out_oy = a; g.out_ox = b;
+            rc = gather_launch(g, 1, (int)d->K, (int)d->C, dy, (const float *)sub, dx);
+        }
+    dopt_hip_free(sub);
+    return rc;
+}
+
 // Shared host driver of forward (kBwd = false) and backward-data (kBwd = true).
 template <bool kBwd>
 int run_gather(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, const float *w, float *out,
@@ -1349,8 +1506,8 @@ int run_gather(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in,
         if (int rc = run_gather<kBwd>(d, P, Q, in, w, out, nullptr)) return rc;
         return dopt_hip_bias_fwd(d->N, kBwd ? d->C : d->K, kBwd ? d->H * d->W : P * Q, out, bias, out);
     }
+    if (kBwd && (d->strideH > 1 || d->strideW > 1)) return run_bwd_strided(d, P, Q, in, w, out);
     GatherConv g{};
-    const int taps = (int)(d->R * d->S);
     g.N = (int)d->N;
     g.R = (int)d->R;
     g.S = (int)d->S;
@@ -1365,77 +1522,10 @@ int run_gather(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in,
         g.Cin = (int)d->K; g.IH = (int)P; g.IW = (int)Q;
         g.Mout = (int)d->C; g.OH = (int)d->H; g.OW = (int)d->W;
     }
-    g.CinPad = round_up(g.Cin, BK);
-    g.Mp = round_up(g.Mout, 4);
-    g.ncols = g.N * g.OH * g.OW;
-    g.slabs_total = taps * g.CinPad / BK;
-    g.out_elems = (size_t)g.ncols * g.Mout;
-
-    // tile shape: wide tiles for <= 64 output channels; otherwise 128x128, with 8 wavefronts per
-    // workgroup when there are too few tiles to give every CU two 4-wavefront workgroups
-    enum { kWide, kSquare, kDeep } shape;
-    int BM, BN, blocks_wanted;
-    if (g.Mout <= 64) {
-        shape = kWide; BM = 64; BN = 256; blocks_wanted = 2 * num_cus();
-    } else {
-        BM = 128; BN = 128;
-        const int t = ((g.Mout + 127) / 128) * ((g.ncols + 127) / 128);
-        if (t >= 2 * num_cus()) { shape = kSquare; blocks_wanted = 2 * num_cus(); }
-        else { shape = kDeep; blocks_wanted = num_cus(); }
-    }
-    g.mtiles = (g.Mout + BM - 1) / BM;
-    g.ntiles = (g.ncols + BN - 1) / BN;
-    const int tiles = g.mtiles * g.ntiles;
-    int splits = pick_splits(tiles, g.slabs_total, blocks_wanted, 64);
-    if (g.out_elems % 4 != 0 || !aligned16(out)) splits = 1;  // the split reduction works on float4
-    g.slabs_per_split = (g.slabs_total + splits - 1) / splits;
-    splits = (g.slabs_total + g.slabs_per_split - 1) / g.slabs_per_split;  // no empty split
-    g.splits = splits;
-
-    const size_t wp_elems = (size_t)taps * g.CinPad * g.Mp;
-    const size_t wp_bytes = (wp_elems * sizeof(float) + 255) / 256 * 256;
-    const size_t part_bytes = splits > 1 ? (size_t)splits * g.out_elems * sizeof(float) : 0;
-    char *ws = (char *)workspace(wp_bytes + part_bytes);
-    if (!ws) return DOPT_HIP_ERR_OOM;
-    float *wp = (float *)ws;
-    float *partial = (float *)(ws + wp_bytes);
-
-    // pack the filter
-    if (g.CinPad != g.Cin || g.Mp != g.Mout) {
-        if (capturing()) return fail(DOPT_HIP_ERR_UNSUPPORTED, "convolution: a fill cannot be recorded into a graph");
-        DOPT_HIP_CHECK(hipMemsetAsync(wp, 0, wp_elems * sizeof(float), stream()));
-    }
-    const int K = (int)d->K, C = (int)d->C;
-    if (!kBwd) {
-        dim3 grid((unsigned)((K + 63) / 64), (unsigned)((C * taps + 63) / 64));
-        hipLaunchKernelGGL(pack_fwd_k, grid, dim3(256), 0, stream(), K, C, taps, g.CinPad, g.Mp, w, wp);
-    } else {
-        dim3 grid((unsigned)K, (unsigned)((C + 63) / 64));
-        hipLaunchKernelGGL(pack_bwd_k, grid, dim3(256), (size_t)64 * taps * sizeof(float), stream(), K, C, taps,
-                           g.CinPad, g.Mp, w, wp);
-    }
-    DOPT_LAUNCH_CHECK();
-
-    g.in = in;
-    g.wp = wp;
-    g.in_bytes = (size_t)g.N * g.Cin * g.IH * g.IW * sizeof(float);
-    g.wp_bytes = wp_elems * sizeof(float);
-    g.out = splits > 1 ? partial : out;
-    dim3 grid(xcd_grid((unsigned)(tiles * splits)));
-    const int mode = !kBwd ? 0 : (g.strideH == 1 && g.strideW == 1 ? 1 : 2);
-#define DOPT_GATHER(TILE)                                                                                      \
-    do {                                                                                                       \
-        if (mode == 0) hipLaunchKernelGGL((conv_gather_k<TILE, 0>), grid, dim3(TILE::THREADS), 0, stream(), g); \
-        else if (mode == 1) hipLaunchKernelGGL((conv_gather_k<TILE, 1>), grid, dim3(TILE::THREADS), 0, stream(), g); \
-        else hipLaunchKernelGGL((conv_gather_k<TILE, 2>), grid, dim3(TILE::THREADS), 0, stream(), g);          \
-    } while (0)
-    if (shape == kWide) DOPT_GATHER(GatherWide);
-    else if (shape == kSquare) DOPT_GATHER(GatherSquare);
-    else DOPT_GATHER(GatherDeep);
-#undef DOPT_GATHER
-    DOPT_LAUNCH_CHECK();
-    if (splits > 1) return launch_splitk_reduce(g.out_elems, splits, partial, out);
-    return DOPT_HIP_OK;
+    g.out_plane = g.OH * g.OW;
+    g.out_OW = g.OW;
+    g.out_sy = g.out_sx = 1;
+    return gather_launch(g, kBwd ? 1 : 0, (int)d->K, (int)d->C, in, w, out);
 }
 
 template <int WM, int WC, int kGeo>

@@ -323,6 +323,14 @@ CONV_CASES = [  # N, C, H, W, K, R, S, pad, stride
     (7, 3, 24, 16, 64, 3, 3, (1, 1), (1, 1)),
     (2, 3, 28, 28, 16, 3, 3, (1, 1), (1, 1)),     # 28 is no power of two: general kernels
     (2, 3, 32, 32, 96, 3, 3, (1, 1), (1, 1)),     # more than 64 output channels: general kernels
+    # strides: backward-data runs one residue class of pixels at a time (classes without a tap, uneven
+    # class sizes, different strides per axis, a stride above the filter size, 5x5 filters)
+    (2, 5, 9, 11, 7, 3, 3, (1, 1), (3, 3)),
+    (3, 4, 10, 7, 6, 3, 3, (0, 1), (2, 1)),
+    (2, 6, 8, 8, 5, 2, 2, (0, 0), (3, 3)),
+    (1, 3, 13, 12, 4, 5, 5, (2, 2), (2, 2)),
+    (2, 8, 7, 9, 3, 3, 2, (2, 0), (1, 2)),
+    (4, 20, 16, 16, 36, 3, 3, (1, 1), (2, 2)),
 ]
 
 
