@@ -1206,6 +1206,34 @@ PackJob pack_job(const dopt_hip_conv_desc *d, const PatchSetup &u, const float *
     return j;
 }
 
+// How many ways to split the channel chunks of a patch convolution over blocks.  `slots` blocks run
+// at once (one or two per CU); the blocks of a launch run in ceil(blocks / slots) rounds and a round
+// lasts as long as one block, so 320 tiles on 256 slots cost two full rounds - unless the reduction
+// is split four ways, which makes 1280 quarter-length blocks in exactly five rounds.  The estimate,
+// in microseconds: rounds x (chunks per block x time per chunk + a fixed prologue/epilogue) plus,
+// when split, writing and re-reading the partial tiles.  The split with the lowest estimate wins;
+// ties go to the smaller one.
+int patch_splits(int tiles, int chunks, int slots, int BM, int BN, size_t out_elems)
+{
+    const double cu_tflops = 0.47;                                   // what one CU sustains in these main loops
+    const double per_cu = (double)slots / num_cus();                 // blocks sharing a CU
+    const double t_chunk = 2.0 * BM * BN * 144 / (cu_tflops * 1e6 / per_cu);   // 16 channels x 9 taps
+    int best = 1;
+    double best_cost = 0.0;
+    for (int sp = 1; sp <= chunks && sp <= 64; sp++) {
+        const int per_block = (chunks + sp - 1) / sp;
+        if (sp > 1 && (chunks + per_block - 1) / per_block != sp) continue;   // would leave an empty split
+        const double rounds = (double)(((long long)tiles * sp + slots - 1) / slots);
+        double cost = rounds * (per_block * t_chunk + 6.0);
+        if (sp > 1) cost += 3.0 + (sp + 1.0) * out_elems * 4.0 / 4.5e6;       // partial tiles at ~4.5 TB/s
+        if (sp == 1 || cost < best_cost * 0.97) {                    // a larger split must pay for itself clearly
+            best = sp;
+            best_cost = cost;
+        }
+    }
+    return best;
+}
+
 // `prepacked`: the filter already in the kernel's layout (dopt_hip_conv_pack_batch), or null to
 // pack it here first.
 template <bool kBwd>
@@ -1217,10 +1245,7 @@ int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, 
     if (!u.ok) return DOPT_HIP_OK;
     PatchConv &pc = u.pc;
     const int tiles = u.tiles;
-    // never a grid slightly above what is resident at once: a second round of blocks would run nearly empty
-    int splits = tiles >= u.blocks_wanted ? 1 : u.blocks_wanted / tiles;
-    if (splits > pc.chunks_total) splits = pc.chunks_total;
-    if (splits > 64) splits = 64;
+    int splits = patch_splits(tiles, pc.chunks_total, u.blocks_wanted, u.BM, u.BN, pc.out_elems);
     if (pc.out_elems % 4 != 0 || !aligned16(out)) splits = 1;
     pc.chunks_per_split = (pc.chunks_total + splits - 1) / splits;
     splits = (pc.chunks_total + pc.chunks_per_split - 1) / pc.chunks_per_split;
