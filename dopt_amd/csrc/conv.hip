@@ -1623,10 +1623,28 @@ int run_wgrad_patch(const dopt_hip_conv_desc *d, const float *dy, const float *x
     const size_t out_elems = (size_t)wp.K * wp.C * 9;
     const int tiles = wp.mtiles * wp.ctiles;
     // one block per CU: never a grid slightly above the CU count (a second, nearly empty round)
-    int splits = tiles >= num_cus() ? 1 : num_cus() / tiles;
-    const int max_by_depth = wp.chunks_total / 2 > 0 ? wp.chunks_total / 2 : 1;  // two chunks amortise the set-up
-    if (splits > max_by_depth) splits = max_by_depth;
-    if (splits > 512) splits = 512;
+    // Splits of the pixel chunks: one block per CU runs at a time, the launch takes ceil(blocks / CUs)
+    // rounds of one block's duration.  Estimate (microseconds) per candidate: rounds x (chunks per
+    // block x time per chunk + a fixed set-up and epilogue) + writing and re-reading the partial
+    // filters; 100 tiles are better served by 5 splits (500 blocks, two nearly full rounds) than by
+    // 2 (200 blocks on 256 CUs).
+    int splits = 1;
+    {
+        const int max_by_depth = wp.chunks_total / 2 > 0 ? wp.chunks_total / 2 : 1;  // two chunks amortise the set-up
+        const double t_chunk = 2.0 * BM * BC * 9 * 64 / 0.45e6;
+        double best = 0.0;
+        for (int sp = 1; sp <= max_by_depth && sp <= 512; sp++) {
+            const int per_block = (wp.chunks_total + sp - 1) / sp;
+            if (sp > 1 && (wp.chunks_total + per_block - 1) / per_block != sp) continue;
+            const double rounds = (double)(((long long)tiles * sp + num_cus() - 1) / num_cus());
+            double cost = rounds * (per_block * t_chunk + 8.0);
+            if (sp > 1) cost += 3.0 + 2.0 * sp * out_elems * 4.0 / 4.5e6;
+            if (sp == 1 || cost < best * 0.97) {
+                splits = sp;
+                best = cost;
+            }
+        }
+    }
     if (out_elems % 4 != 0 || !aligned16(dw)) splits = 1;  // the split sum works on float4
     wp.chunks_per_split = (wp.chunks_total + splits - 1) / splits;
     splits = (wp.chunks_total + wp.chunks_per_split - 1) / wp.chunks_per_split;
