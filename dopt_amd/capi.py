@@ -55,7 +55,7 @@ PROTOTYPES = {
     "dopt_hip_event_elapsed_ms": [_vp, _vp, C.POINTER(_f)],
     "dopt_hip_event_destroy": [_vp],
     "dopt_hip_pointwise": [C.c_char_p, _i, _sz, _vp, _vp, _vp],
-    "dopt_hip_pointwise_chain": [_i, _sz, _i, C.POINTER(_vp), C.POINTER(C.c_ubyte), _i, C.POINTER(C.c_char_p),
+    "dopt_hip_pointwise_chain": [_i, _sz, _sz, _i, C.POINTER(_vp), C.POINTER(C.c_ubyte), _i, C.POINTER(C.c_char_p),
                                  C.POINTER(_i), C.POINTER(_i), _vp],
     "dopt_hip_pointwise_chain_compile_only": [_i, _i, C.POINTER(C.c_ubyte), _i, C.POINTER(C.c_char_p), C.POINTER(_i),
                                               C.POINTER(_i), C.c_char_p],

@@ -758,14 +758,32 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         // stored; an operand of the form repeat(one-element tensor) is read from the element itself.
         // Walking consumers before producers, an operation joins the chain all its readers belong to
         // or starts a chain of its own.
+        // What may be a node: the pointwise operations; relu and reluGrad(dy, y, x) (a node of dy and x),
+        // unless a batch-norm fusion above already reads around them; and a product [m,1] x [1,n] - the
+        // reference's way to broadcast a column or a row (core/ops/basic.d:370-381) - as the node
+        // mul(per-row element, per-column element) of the chain's [m, n] view.
+        auto outer_cols = [&](int id) -> size_t {   // n of such a product, else 0
+            const Operation &o = g.ops[id];
+            if (o.opType != "matmul" || o.deps.size() != 2 || o.rank() != 2 || o.dtype != DOPT_HIP_F32) return 0;
+            const Operation &l = g.ops[o.deps[0]], &r = g.ops[o.deps[1]];
+            if (l.rank() != 2 || r.rank() != 2 || l.shape[1] != 1 || r.shape[0] != 1) return 0;
+            return o.shape[1];
+        };
         auto is_pw = [&](int id) {
             const Operation &o = g.ops[id];
+            if (!live[id] || alias[id].source >= 0 || fusedKind[id] || o.dtype != DOPT_HIP_F32 || o.volume() == 0) return false;
+            if (o.opType == "reluGrad" && o.deps.size() == 3) {
+                for (const Use &u : uses[id])
+                    if (fusedKind[u.op] == 3) return false;   // that batchNormGrad reads dy and y itself
+                return true;
+            }
+            if (outer_cols(id)) return true;
             const int arity = dopt_hip_pointwise_arity(o.opType.c_str());
-            return live[id] && alias[id].source < 0 && !fusedKind[id] && o.dtype == DOPT_HIP_F32 && arity > 0 &&
-                   arity == (int)o.deps.size() && o.volume() > 0;
+            return arity > 0 && arity == (int)o.deps.size();
         };
         std::vector<int> chainOf((size_t)nops, -1);              // the operation that ends the chain
         std::vector<std::vector<int>> chainOps((size_t)nops);    // per chain end: its members
+        std::vector<size_t> chainInner((size_t)nops, 0);         // per chain end: columns of its [rows, inner] view, once a member needs one
         for (auto it = p->mOps.rbegin(); it != p->mOps.rend(); ++it) {
             const int id = *it;
             if (!is_pw(id)) continue;
@@ -774,12 +792,16 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
             for (const Use &u : uses[id]) {
                 if (!joins) break;
                 if (chainOf[u.op] < 0 || u.off != 0 || g.ops[u.op].volume() != g.ops[id].volume()) joins = false;
+                else if (g.ops[u.op].opType == "reluGrad" && u.slot == 1) joins = false;   // the y operand is not part of the node
                 else if (target < 0) target = chainOf[u.op];
                 else if (target != chainOf[u.op]) joins = false;
             }
             if (joins && chainOps[target].size() >= 48) joins = false;
+            const size_t cols = outer_cols(id);
+            if (joins && cols && chainInner[target] && chainInner[target] != cols) joins = false;
             chainOf[id] = joins ? target : id;
             chainOps[chainOf[id]].push_back(id);
+            if (cols) chainInner[chainOf[id]] = cols;
         }
         for (int end : p->mOps) {
             if (chainOf[end] != end || chainOps[end].size() < 2) continue;
@@ -787,42 +809,46 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
             for (int id : p->mOps)
                 if (chainOf[id] == end) members.push_back(id);
             std::vector<int> inputs;                              // operations whose buffers the kernel reads
-            std::vector<unsigned char> scalar;
+            std::vector<unsigned char> kinds;                     // 0 tensor, 1 one element, 2 per row, 3 per column
             std::vector<int> nodeOf((size_t)nops, -1);
             struct Node { std::string op; int lhs, rhs; };
             std::vector<Node> nodes;
-            std::vector<std::pair<int, int>> operands;            // per node slot: (is node, index) before renumbering
-            bool ok = true;
-            auto input_index = [&](int op, bool is_scalar) {
+            auto input_index = [&](int op, int kind) {
                 for (size_t k = 0; k < inputs.size(); k++)
-                    if (inputs[k] == op && scalar[k] == (unsigned char)is_scalar) return (int)k;
+                    if (inputs[k] == op && kinds[k] == (unsigned char)kind) return (int)k;
                 inputs.push_back(op);
-                scalar.push_back(is_scalar);
+                kinds.push_back((unsigned char)kind);
                 return (int)inputs.size() - 1;
+            };
+            auto operand = [&](int dep) {                         // index of a member's operand: a node (<= -2) or an input
+                size_t off;
+                const int r = root(dep, &off);
+                if (chainOf[r] == end && nodeOf[r] >= 0 && off == 0) return -2 - nodeOf[r];
+                const Operation &ro = g.ops[r];
+                size_t soff = 0;
+                if (ro.opType == "repeat" && ro.deps.size() == 1 && off == 0 && alias[r].source < 0 &&
+                    g.ops[ro.deps[0]].volume() == 1 && g.ops[root(ro.deps[0], &soff)].dtype == DOPT_HIP_F32)
+                    return input_index(ro.deps[0], 1);
+                return input_index(dep, 0);
             };
             for (int id : members) {
                 const Operation &o = g.ops[id];
-                int ref[2] = {-1, -1};
-                for (size_t j = 0; j < o.deps.size(); j++) {
-                    size_t off;
-                    const int r = root(o.deps[j], &off);
-                    if (chainOf[r] == end && nodeOf[r] >= 0 && off == 0) {
-                        ref[j] = -2 - nodeOf[r];                  // a node, renumbered once the inputs are known
-                        continue;
-                    }
-                    const Operation &ro = g.ops[r];
-                    size_t soff = 0;
-                    if (ro.opType == "repeat" && ro.deps.size() == 1 && off == 0 && alias[r].source < 0 &&
-                        g.ops[ro.deps[0]].volume() == 1 && g.ops[root(ro.deps[0], &soff)].dtype == DOPT_HIP_F32)
-                        ref[j] = input_index(ro.deps[0], true);
-                    else
-                        ref[j] = input_index(o.deps[j], false);
+                Node node{o.opType, -1, -1};
+                if (outer_cols(id)) {
+                    node.op = "mul";
+                    node.lhs = input_index(o.deps[0], 2);
+                    node.rhs = input_index(o.deps[1], 3);
+                } else if (o.opType == "reluGrad") {
+                    node.lhs = operand(o.deps[0]);
+                    node.rhs = operand(o.deps[2]);
+                } else {
+                    node.lhs = operand(o.deps[0]);
+                    if (o.deps.size() > 1) node.rhs = operand(o.deps[1]);
                 }
                 nodeOf[id] = (int)nodes.size();
-                nodes.push_back({o.opType, ref[0], ref[1]});
+                nodes.push_back(node);
             }
-            if (inputs.empty() || inputs.size() > 12) ok = false;
-            if (!ok) continue;                                    // too wide: its members keep their own kernels
+            if (inputs.empty() || inputs.size() > 12) continue;   // too wide: its members keep their own kernels
             const int nin = (int)inputs.size();
             for (Node &n : nodes) {
                 if (n.lhs <= -2) n.lhs = nin + (-2 - n.lhs);
@@ -831,7 +857,7 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
             }
             for (int id : members) fusedKind[id] = 7;
             inputsOf[end] = inputs;
-            const size_t count = g.ops[end].volume();
+            const size_t count = g.ops[end].volume(), inner = chainInner[end];
             prebuilt[end] = make([=](const std::vector<const void *> &in, void *out) {
                 const char *names[64];
                 int lhs[64], rhs[64];
@@ -840,8 +866,8 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
                     lhs[j] = nodes[j].lhs;
                     rhs[j] = nodes[j].rhs;
                 }
-                return dopt_hip_pointwise_chain(DOPT_HIP_F32, count, nin, in.data(), scalar.data(), (int)nodes.size(), names,
-                                                lhs, rhs, out);
+                return dopt_hip_pointwise_chain(DOPT_HIP_F32, count, inner, nin, in.data(), kinds.data(), (int)nodes.size(),
+                                                names, lhs, rhs, out);
             });
             prebuiltLabel[end] = "pointwise*" + std::to_string(nodes.size());   // no spaces: profile lines are split on them
         }

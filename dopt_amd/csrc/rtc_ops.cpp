@@ -56,6 +56,10 @@ const OpInfo kOps[] = {
     {"asinh", 1, "asinhf(a)", "(int)asinhf((float)a)"},
     {"acosh", 1, "acoshf(a)", "(int)acoshf((float)a)"},
     {"atanh", 1, "atanhf(a)", "(int)atanhf((float)a)"},
+    // the two activations of cuda/nnet/cudnn7.d:406-461 in the form nn.hip computes them (NaN passes through
+    // relu); reluGrad takes (dy, x).  They exist so that a plan can run them inside a pointwise chain.
+    {"relu", 1, "(a < 0 ? 0 : a)", "(a < 0 ? 0 : a)"},
+    {"reluGrad", 2, "(b > 0 ? a : 0)", "(b > 0 ? a : 0)"},
 };
 
 const OpInfo *find_op(const char *name)
@@ -165,9 +169,13 @@ std::string pointwise_source(const OpInfo &op, int dtype)
 // contraction), intermediate values stay in fp32 registers, so the result equals running the
 // nodes one kernel at a time bit for bit.  Operand k < nin is input k (a vector, or a one-element
 // tensor broadcast to every position); operand nin + j is node j.  Outputs: the last node.
-std::string chain_source(int dtype, int nin, const unsigned char *scalar, int nnodes, const OpInfo *const *ops,
+std::string chain_source(int dtype, int nin, const unsigned char *kind, int nnodes, const OpInfo *const *ops,
                          const int *lhs, const int *rhs)
 {
+    // kind: 0 an n-element tensor; 1 one element, read at every position; 2 one element per row of the
+    // [n / inner, inner] view (index e / inner); 3 one element per column (index e % inner)
+    bool grid = false;
+    for (int k = 0; k < nin; k++) grid = grid || kind[k] >= 2;
     std::string s = dtype == DOPT_HIP_F32 ? "typedef float T;\n" : "typedef int T;\n";
     s += "typedef T T4 __attribute__((ext_vector_type(4)));\n#define BLOCK 256\n";
     s += R"SRC(
@@ -190,9 +198,11 @@ __device__ inline int dopt_ipow(int x, int n)
     for (int j = 0; j < nnodes; j++)
         s += "__device__ inline T f" + std::to_string(j) + "(T a, T b) { return (T)(" +
              (dtype == DOPT_HIP_F32 ? ops[j]->expr_f32 : ops[j]->expr_i32) + "); }\n";
+    // `lane` is a component suffix of the quads (".x") or "" in the one-element-at-a-time code
     auto operand = [&](int k, const char *lane) -> std::string {
         if (k >= nin) return "t" + std::to_string(k - nin);
-        if (scalar[k]) return "s" + std::to_string(k);
+        if (kind[k] == 1) return "s" + std::to_string(k);
+        if (kind[k] == 2) return "r" + std::to_string(k);
         return "x" + std::to_string(k) + lane;
     };
     auto body = [&](const char *lane, const std::string &dst) {
@@ -204,49 +214,50 @@ __device__ inline int dopt_ipow(int x, int n)
         b += "            " + dst + " = t" + std::to_string(nnodes - 1) + ";\n        }\n";
         return b;
     };
-    std::string params = "size_t n";
+    std::string params = "size_t n, size_t inner";
     for (int k = 0; k < nin; k++) params += ", const T *i" + std::to_string(k);
     params += ", T *o";
     std::string scalars;
     for (int k = 0; k < nin; k++)
-        if (scalar[k]) scalars += "    const T s" + std::to_string(k) + " = i" + std::to_string(k) + "[0];\n";
+        if (kind[k] == 1) scalars += "    const T s" + std::to_string(k) + " = i" + std::to_string(k) + "[0];\n";
 
-    // quads: two independent 128-bit loads per operand and lane in flight
+    // quads (inner is a multiple of four whenever rows or columns are indexed, so a quad never
+    // straddles a row): one quad per lane and pass, all loads before the first use
     s += "extern \"C\" __global__ __launch_bounds__(BLOCK) void chain_vec(" + params + ")\n{\n" + scalars;
-    s += "    const size_t n4 = n >> 2;\n";
-    s += "    for (size_t base = (size_t)blockIdx.x * (BLOCK * 2) + threadIdx.x; base < n4; base += (size_t)gridDim.x * (BLOCK * 2)) {\n";
-    s += "        const size_t second = base + BLOCK < n4 ? base + BLOCK : base;\n";
-    for (int k = 0; k < nin; k++)
-        if (!scalar[k]) {
-            const std::string i = std::to_string(k);
-            s += "        const T4 x" + i + " = ((const T4 *)i" + i + ")[base], y" + i + " = ((const T4 *)i" + i + ")[second];\n";
-        }
-    s += "        T4 r, q;\n";
-    for (const char *lane : {".x", ".y", ".z", ".w"}) s += body(lane, std::string("r") + lane);
-    // the second quad: the same code over y instead of x
-    {
-        std::string second;
-        for (const char *lane : {".x", ".y", ".z", ".w"}) second += body(lane, std::string("q") + lane);
-        for (int k = 0; k < nin; k++) {
-            if (scalar[k]) continue;
-            const std::string from = "x" + std::to_string(k) + ".", to = "y" + std::to_string(k) + ".";
-            for (size_t at = second.find(from); at != std::string::npos; at = second.find(from, at + to.size()))
-                second.replace(at, from.size(), to);
-        }
-        s += second;
+    s += "    const size_t n4 = n >> 2, inner4 = inner >> 2;\n";
+    s += "    for (size_t q = (size_t)blockIdx.x * BLOCK + threadIdx.x; q < n4; q += (size_t)gridDim.x * BLOCK) {\n";
+    if (grid) s += "        const size_t row = q / inner4, colq = q - row * inner4;\n";
+    for (int k = 0; k < nin; k++) {
+        const std::string i = std::to_string(k);
+        if (kind[k] == 0) s += "        const T4 x" + i + " = ((const T4 *)i" + i + ")[q];\n";
+        if (kind[k] == 2) s += "        const T r" + i + " = i" + i + "[row];\n";
+        if (kind[k] == 3) s += "        const T4 x" + i + " = ((const T4 *)i" + i + ")[colq];\n";
     }
-    s += "        ((T4 *)o)[base] = r;\n        if (second != base) ((T4 *)o)[second] = q;\n    }\n";
-    s += "    if (blockIdx.x == 0) {\n        const size_t i = (n4 << 2) + threadIdx.x;\n        if (i < n) {\n";
-    for (int k = 0; k < nin; k++)
-        if (!scalar[k]) s += "            const T x" + std::to_string(k) + " = i" + std::to_string(k) + "[i];\n";
-    s += body("", "o[i]");
+    s += "        T4 r;\n";
+    for (const char *lane : {".x", ".y", ".z", ".w"}) s += body(lane, std::string("r") + lane);
+    s += "        ((T4 *)o)[q] = r;\n    }\n";
+    // the last n % 4 elements (none when rows or columns are indexed)
+    s += "    if (blockIdx.x == 0) {\n        const size_t e = (n4 << 2) + threadIdx.x;\n        if (e < n) {\n";
+    if (grid) s += "            const size_t row = e / inner, col = e - row * inner;\n";
+    for (int k = 0; k < nin; k++) {
+        const std::string i = std::to_string(k);
+        if (kind[k] == 0) s += "            const T x" + i + " = i" + i + "[e];\n";
+        if (kind[k] == 2) s += "            const T r" + i + " = i" + i + "[row];\n";
+        if (kind[k] == 3) s += "            const T x" + i + " = i" + i + "[col];\n";
+    }
+    s += body("", "o[e]");
     s += "        }\n    }\n}\n";
 
     s += "extern \"C\" __global__ __launch_bounds__(BLOCK) void chain_scalar(" + params + ")\n{\n" + scalars;
-    s += "    for (size_t i = (size_t)blockIdx.x * BLOCK + threadIdx.x; i < n; i += (size_t)gridDim.x * BLOCK) {\n";
-    for (int k = 0; k < nin; k++)
-        if (!scalar[k]) s += "        const T x" + std::to_string(k) + " = i" + std::to_string(k) + "[i];\n";
-    s += body("", "o[i]");
+    s += "    for (size_t e = (size_t)blockIdx.x * BLOCK + threadIdx.x; e < n; e += (size_t)gridDim.x * BLOCK) {\n";
+    if (grid) s += "        const size_t row = e / inner, col = e - row * inner;\n";
+    for (int k = 0; k < nin; k++) {
+        const std::string i = std::to_string(k);
+        if (kind[k] == 0) s += "        const T x" + i + " = i" + i + "[e];\n";
+        if (kind[k] == 2) s += "        const T r" + i + " = i" + i + "[row];\n";
+        if (kind[k] == 3) s += "        const T x" + i + " = i" + i + "[col];\n";
+    }
+    s += body("", "o[e]");
     s += "    }\n}\n";
     return s;
 }
@@ -530,7 +541,10 @@ static int chain_prepare(int dtype, int nin, const unsigned char *in_is_scalar, 
     if (int rc = check_dtype(dtype)) return rc;
     const OpInfo *ops[64];
     *key = dtype == DOPT_HIP_F32 ? "chain:f32" : "chain:i32";
-    for (int k = 0; k < nin; k++) *key += in_is_scalar[k] ? ":s" : ":v";
+    for (int k = 0; k < nin; k++) {
+        DOPT_REQUIRE(in_is_scalar[k] <= 3, "dopt_hip_pointwise_chain: input %d has unknown kind %d", k, (int)in_is_scalar[k]);
+        *key += in_is_scalar[k] == 0 ? ":v" : in_is_scalar[k] == 1 ? ":s" : in_is_scalar[k] == 2 ? ":r" : ":c";
+    }
     for (int j = 0; j < nnodes; j++) {
         DOPT_REQUIRE(node_op[j] != nullptr, "dopt_hip_pointwise_chain: node %d has no operation", j);
         ops[j] = find_op(node_op[j]);
@@ -545,31 +559,40 @@ static int chain_prepare(int dtype, int nin, const unsigned char *in_is_scalar, 
     return DOPT_HIP_OK;
 }
 
-int dopt_hip_pointwise_chain(int dtype, size_t n, int nin, const void *const *in, const unsigned char *in_is_scalar,
-                             int nnodes, const char *const *node_op, const int *node_lhs, const int *node_rhs, void *out)
+int dopt_hip_pointwise_chain(int dtype, size_t n, size_t inner, int nin, const void *const *in,
+                             const unsigned char *in_is_scalar, int nnodes, const char *const *node_op, const int *node_lhs,
+                             const int *node_rhs, void *out)
 {
     std::string key, source;
     if (int rc = chain_prepare(dtype, nin, in_is_scalar, nnodes, node_op, node_lhs, node_rhs, &key, &source)) return rc;
     if (n == 0) return DOPT_HIP_OK;
     DOPT_REQUIRE(in && out, "dopt_hip_pointwise_chain: null argument");
-    bool vec = aligned16(out);
+    bool vec = aligned16(out), grid_kinds = false;
     for (int k = 0; k < nin; k++) {
         DOPT_REQUIRE(in[k] != nullptr, "dopt_hip_pointwise_chain: input %d is null", k);
-        vec = vec && (in_is_scalar[k] || aligned16(in[k]));
+        grid_kinds = grid_kinds || in_is_scalar[k] >= 2;
+        vec = vec && (in_is_scalar[k] == 1 || in_is_scalar[k] == 2 || aligned16(in[k]));
+    }
+    if (grid_kinds) {
+        DOPT_REQUIRE(inner > 0 && n % inner == 0, "dopt_hip_pointwise_chain: %zu elements are not rows of %zu", n, inner);
+        vec = vec && inner % 4 == 0;
+    } else {
+        inner = n;
     }
     DOPT_ENSURE_INIT();
     const char *kname = vec ? "chain_vec" : "chain_scalar";
     hipFunction_t fn;
     if (int rc = rtc_get(key + ":" + kname, source, kname, &fn)) return rc;
     const void *ptrs[16];
-    void *args[18];
+    void *args[19];
     args[0] = (void *)&n;
+    args[1] = (void *)&inner;
     for (int k = 0; k < nin; k++) {
         ptrs[k] = in[k];
-        args[1 + k] = (void *)&ptrs[k];
+        args[2 + k] = (void *)&ptrs[k];
     }
-    args[1 + nin] = (void *)&out;
-    unsigned grid = vec ? grid_for(256 * 2, ceil_div(n, 4)) : grid_for(256, n);
+    args[2 + nin] = (void *)&out;
+    unsigned grid = vec ? grid_for(256, ceil_div(n, 4)) : grid_for(256, n);
     return rtc_launch(fn, grid, 256, args);
 }
 

@@ -113,20 +113,22 @@ def pointwise(op, a, b=None, out=None):
     return out
 
 
-def pointwise_chain(inputs, nodes, out=None):
+def pointwise_chain(inputs, nodes, out=None, kinds=None, inner=0):
     """One kernel for a DAG of pointwise nodes.  inputs: tensors; a one-element tensor among longer
-    ones is broadcast.  nodes: (op, lhs, rhs-or-None) with operand indices counting the inputs first
-    and then the nodes; the last node is the result."""
+    ones is broadcast.  kinds (optional, per input): 0 full tensor, 1 one element, 2 one element per
+    row, 3 one element per column of the [n / inner, inner] view.  nodes: (op, lhs, rhs-or-None) with
+    operand indices counting the inputs first and then the nodes; the last node is the result."""
     n = max(t.size for t in inputs)
     full = next(t for t in inputs if t.size == n)
-    scalar = [1 if (t.size == 1 and n != 1) else 0 for t in inputs]
-    if any(t.size != n and not sc for t, sc in zip(inputs, scalar)) or any(t.dtype != full.dtype for t in inputs):
+    if kinds is None:
+        kinds = [1 if (t.size == 1 and n != 1) else 0 for t in inputs]
+    if any(t.size != n and k == 0 for t, k in zip(inputs, kinds)) or any(t.dtype != full.dtype for t in inputs):
         raise capi.HipError(1, "pointwise operands must have the same type")
     out = _out(out, full.shape, full.dtype)
     k = len(nodes)
     capi.check(capi.load().dopt_hip_pointwise_chain(
-        full.code, n, len(inputs), (C.c_void_p * len(inputs))(*[t.ptr for t in inputs]),
-        (C.c_ubyte * len(inputs))(*scalar), k, (C.c_char_p * k)(*[nd[0].encode() for nd in nodes]),
+        full.code, n, inner, len(inputs), (C.c_void_p * len(inputs))(*[t.ptr for t in inputs]),
+        (C.c_ubyte * len(inputs))(*kinds), k, (C.c_char_p * k)(*[nd[0].encode() for nd in nodes]),
         (C.c_int * k)(*[nd[1] for nd in nodes]), (C.c_int * k)(*[-1 if nd[2] is None else nd[2] for nd in nodes]), out.ptr))
     return out
 

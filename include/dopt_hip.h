@@ -105,17 +105,21 @@ int dopt_hip_event_destroy(void *event);
            round trip (cuda/package.d:81-119); here they run on the device. */
 int dopt_hip_pointwise(const char *op, int dtype, size_t n, const void *a, const void *b_or_null, void *out);
 /* A DAG of pointwise nodes over n-element operands as one kernel.  The reference has no counterpart:
-   it launches one generated kernel per node (cuda/math.d:129-205) and its operator sugar broadcasts
-   a scalar by materialising `repeat(scalar, n)` first (core/ops/package.d:94-168).  Operand index
-   k < nin is input k - an n-element tensor, or, where in_is_scalar[k] is set, a one-element tensor
-   read at every position; index nin + j is the value of node j.  A node reads only inputs and
-   earlier nodes; unary nodes ignore node_rhs.  The last node's value is written to `out`.  Every
-   node is rounded to its own fp32 result exactly as the stand-alone kernel of that op rounds it. */
-int dopt_hip_pointwise_chain(int dtype, size_t n, int nin, const void *const *in,
-                             const unsigned char *in_is_scalar, int nnodes, const char *const *node_op,
+   it launches one generated kernel per node (cuda/math.d:129-205), its operator sugar broadcasts a
+   scalar by materialising `repeat(scalar, n)` first (core/ops/package.d:94-168), and row / column
+   broadcasts are products with a ones vector (core/ops/basic.d:370-381).  Operand index k < nin is
+   input k, of the kind in_kind[k] says: 0 an n-element tensor; 1 a one-element tensor read at every
+   position; 2 one element per row and 3 one element per column of the [n / inner, inner] view of the
+   operands (`inner` is ignored when no input is of kind 2 or 3).  Index nin + j is the value of node
+   j.  A node reads only inputs and earlier nodes; unary nodes ignore node_rhs.  Besides the names
+   dopt_hip_pointwise accepts, nodes may be "relu" and "reluGrad" (operands dy, x).  The last node's
+   value is written to `out`.  Every node is rounded to its own fp32 result exactly as the
+   stand-alone kernel of that op rounds it. */
+int dopt_hip_pointwise_chain(int dtype, size_t n, size_t inner, int nin, const void *const *in,
+                             const unsigned char *in_kind, int nnodes, const char *const *node_op,
                              const int *node_lhs, const int *node_rhs, void *out);
 /* Generates and compiles the kernel of such a chain for `arch` without loading it (no GPU needed). */
-int dopt_hip_pointwise_chain_compile_only(int dtype, int nin, const unsigned char *in_is_scalar,
+int dopt_hip_pointwise_chain_compile_only(int dtype, int nin, const unsigned char *in_kind,
                                           int nnodes, const char *const *node_op, const int *node_lhs,
                                           const int *node_rhs, const char *arch);
 /* 1 or 2 for the names dopt_hip_pointwise accepts, 0 otherwise. */

@@ -59,6 +59,27 @@ def test_chain_unaligned_operands_and_int32():
     assert np.array_equal(ops.pointwise_chain([ia, ib], nodes).numpy(), _one_by_one([ia, ib], nodes))
 
 
+@pytest.mark.parametrize("m,n", [(7, 12), (5, 10), (128, 512), (1, 8), (9, 1), (33, 20)])
+def test_chain_row_and_column_operands_and_relu_nodes(m, n):
+    """relu(x + ones[m,1] . b[1,n]) and reluGrad(dy * a[m,1] . ones[1,n], x): the outer products are read as
+    a per-row and a per-column element; n % 4 != 0 takes the one-element-at-a-time kernel."""
+    r = np.random.default_rng(m * 100 + n)
+    x = r.standard_normal((m, n)).astype(np.float32)
+    dy = r.standard_normal((m, n)).astype(np.float32)
+    col = r.standard_normal((m, 1)).astype(np.float32)
+    row = r.standard_normal((1, n)).astype(np.float32)
+    # inputs: x (tensor), col (per row), row (per column); t0 = col*row, t1 = x + t0, t2 = relu(t1)
+    got = ops.pointwise_chain([T(x), T(col), T(row)], [("mul", 1, 2), ("add", 0, 3), ("relu", 4, None)],
+                              kinds=[0, 2, 3], inner=n).numpy()
+    outer = ops.matmul(T(col), T(row))
+    want = ops.relu(ops.pointwise("add", T(x), outer)).numpy()
+    assert np.array_equal(got, want)
+    got = ops.pointwise_chain([T(dy), T(x), T(col), T(row)], [("mul", 2, 3), ("mul", 0, 4), ("reluGrad", 5, 1)],
+                              kinds=[0, 0, 2, 3], inner=n).numpy()
+    want = ops.relu_grad(ops.pointwise("mul", T(dy), outer), T(x)).numpy()
+    assert np.array_equal(got, want)
+
+
 def test_chain_rejects_forward_references_and_unknown_ops():
     a = T(np.ones(8, np.float32))
     with pytest.raises(capi.HipError):
@@ -134,6 +155,12 @@ def _random_graph(r, n_leaves=4, n_ops=18, size=96):
             node = core.pad(lo * lo, [0], [size - half])
         elif kind == 8:
             node = a + core.sum(b) * 0.01                           # a reduction reads b, its result is broadcast
+        elif kind == 9 and r.integers(0, 2):
+            # a dense layer's bias add and activation on the [8, size/8] view, and the activation's gradient
+            bias = core.float32([shape2[1]], r.standard_normal(shape2[1]).astype(np.float32))
+            pre = core.reshape(a, shape2) + core.repeat(bias, shape2[0])
+            act = core.relu(pre)
+            node = core.reshape(core.reluGrad(core.reshape(b, shape2), act) + act, [size])
         else:
             node = core.min(core.exp(a * 0.1), b)
         pool.append(node)
@@ -144,7 +171,7 @@ def _random_graph(r, n_leaves=4, n_ops=18, size=96):
     return outputs
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(20))
 def test_random_graphs_give_the_same_values_with_every_rewrite(seed):
     outs = _random_graph(np.random.default_rng(100 + seed))
     want = core.compile(outs).execute()
