@@ -557,24 +557,73 @@ std::unique_ptr<HIPKernel> make_fused(const Graph &g, int id, int kind, void *ex
 
 }  // namespace
 
-int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flags, std::unique_ptr<HIPPlan> *out)
+// HIPPlan::create in passes.  The builder holds what the passes share: per operation, which buffer it
+// aliases, which operations' buffers feed its kernel, which fused kernel (if any) computes it, who
+// reads it.  `p` is the plan under construction.
+struct HIPPlan::Builder {
+    const Graph &g;
+    HIPPlan *p;
+    const std::vector<int> &outputs;
+    const unsigned flags;
+    const int nops;
+
+    std::vector<Alias> alias;
+    // inputsOf[id]: the operations whose buffers feed id's kernel (its deps, unless fused);
+    // fusedKind[id]: 1 conv+bias, 2 bn+relu, 3 relugrad+bngrad, 6 matmul with transposes, 7 pointwise chain
+    std::vector<std::vector<int>> inputsOf;
+    std::vector<int> fusedKind;
+    std::vector<std::unique_ptr<HIPKernel>> prebuilt;
+    std::vector<std::string> prebuiltLabel;
+    // readers, counted among the operations that are live after the alias rewrites
+    struct Use { int op; int slot; size_t off; };
+    std::vector<char> live;
+    std::vector<std::vector<Use>> uses;
+    std::vector<std::vector<size_t>> exposed;   // byte offsets at which plan outputs (or aliases of them) expose a buffer
+    std::vector<int> biasGradOf;                // batchNormGrad op -> the addBiasGrad op it serves
+    std::vector<char> absorbed;
+    std::vector<char> needed;
+    struct Prepack { int op, filter; int bwd; dopt_hip_conv_desc d; void *buf; bool owner; };
+    std::vector<Prepack> packs;
+    std::vector<int> packOf;
+
+    Builder(const Graph &graph, HIPPlan *plan, const std::vector<int> &outs, unsigned f)
+        : g(graph), p(plan), outputs(outs), flags(f), nops((int)graph.ops.size()), alias((size_t)nops),
+          inputsOf((size_t)nops), fusedKind((size_t)nops, 0), prebuilt((size_t)nops), prebuiltLabel((size_t)nops),
+          live((size_t)nops, 0), uses((size_t)nops), exposed((size_t)nops), biasGradOf((size_t)nops, -1),
+          absorbed((size_t)nops, 0), needed((size_t)nops, 0), packOf((size_t)nops, -1)
+    {
+    }
+
+    int root(int id, size_t *off) const   // the operation whose buffer `id` names, and the byte offset into it
+    {
+        size_t o = 0;
+        while (alias[id].source >= 0) {
+            o += alias[id].offset;
+            id = alias[id].source;
+        }
+        *off = o;
+        return id;
+    }
+    bool isOutput(int id) const { return !exposed[id].empty(); }
+
+    int findAliases();
+    void countReaders();
+    void fusePairs();
+    void foldTransposes();
+    void formChains();
+    void absorbBiasGrads();
+    void markNeeded();
+    int prepackFilters();
+    int allocateBuffers();
+    int buildSteps();
+    void rememberAliases();
+    int assignQueues();
+    int createEvents();
+};
+
+int HIPPlan::Builder::findAliases()
 {
-    registerBuiltinKernels();
-    if (!ensure_init()) return DOPT_HIP_ERR_RUNTIME;
-    const Graph &g = *graph;
-    const int nops = (int)g.ops.size();
-    for (int o : outputs)
-        if (o < 0 || o >= nops) return fail(DOPT_HIP_ERR_INVALID, "plan output %d is not an operation of the graph", o);
-
-    std::unique_ptr<HIPPlan> p(new HIPPlan());
-    p->mGraph = graph;
-    p->mFlags = flags;
-    p->mOutputs = outputs;
-    std::vector<char> seen((size_t)nops, 0);
-    for (int o : outputs) toposort(g, o, seen, p->mOps);
-
     // aliases: reshape always (package.d:295-299); contiguous slices and slice-of-pad under VIEWS
-    std::vector<Alias> alias((size_t)nops);
     for (int id : p->mOps) {
         const Operation &op = g.ops[id];
         if (op.opType == "reshape") {
@@ -603,280 +652,272 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
             }
         }
     }
+    return DOPT_HIP_OK;
+}
 
-    // Fusion (DOPT_HIP_PLAN_FUSE): a pair of operations runs as one kernel when the value between
-    // them has no other reader.  inputsOf[id] lists the operations whose buffers feed id's kernel
-    // (its deps, unless fused); fusedKind[id] names the fused kernel.
-    std::vector<std::vector<int>> inputsOf((size_t)nops);
-    std::vector<int> fusedKind((size_t)nops, 0);  // 1 conv+bias, 2 bn+relu, 3 relugrad+bngrad, 6 matmul with transposes
-    std::vector<std::unique_ptr<HIPKernel>> prebuilt((size_t)nops);
-    std::vector<std::string> prebuiltLabel((size_t)nops);
-    for (int id : p->mOps) inputsOf[id] = g.ops[id].deps;
-    if (flags & DOPT_HIP_PLAN_FUSE) {
-        auto root = [&](int id, size_t *off) {
-            size_t o = 0;
-            while (alias[id].source >= 0) {
-                o += alias[id].offset;
-                id = alias[id].source;
-            }
-            *off = o;
-            return id;
-        };
-        // readers are counted among the operations that are live after the alias rewrites
-        std::vector<char> live((size_t)nops, 0);
-        {
-            std::vector<int> work(outputs.begin(), outputs.end());
-            while (!work.empty()) {
-                int id = work.back();
-                work.pop_back();
-                if (live[id]) continue;
-                live[id] = 1;
-                if (alias[id].source >= 0) work.push_back(alias[id].source);
-                else for (int d : g.ops[id].deps) work.push_back(d);
-            }
-        }
-        struct Use { int op; int slot; size_t off; };
-        std::vector<std::vector<Use>> uses((size_t)nops);
-        for (int id : p->mOps) {
-            if (!live[id] || alias[id].source >= 0) continue;
-            const Operation &op = g.ops[id];
-            for (size_t j = 0; j < op.deps.size(); j++) {
-                size_t off;
-                const int r = root(op.deps[j], &off);
-                uses[r].push_back({id, (int)j, off});
-            }
-        }
-        // byte offsets at which plan outputs (or aliases of them) expose a buffer
-        std::vector<std::vector<size_t>> exposed((size_t)nops);
-        for (int o : outputs) {
-            size_t off;
-            const int r = root(o, &off);
-            exposed[r].push_back(off);
-        }
-        auto isOutput = [&](int id) { return !exposed[id].empty(); };
-        for (int id : p->mOps) {
-            const Operation &op = g.ops[id];
-            if (alias[id].source >= 0) continue;
-            if (op.opType == "addBias" && op.deps.size() == 2) {
-                const int c = op.deps[0];
-                if (g.ops[c].opType == "convolution" && g.ops[c].deps.size() == 2 && alias[c].source < 0 && !isOutput(c) &&
-                    uses[c].size() == 1 && g.ops[c].dtype == DOPT_HIP_F32) {
-                    fusedKind[id] = 1;
-                    inputsOf[id] = {g.ops[c].deps[0], g.ops[c].deps[1], op.deps[1]};
-                }
-            } else if (op.opType == "relu" && op.deps.size() == 1) {
-                size_t off;
-                const int b = root(op.deps[0], &off);
-                const Operation &bn = g.ops[b];
-                if (bn.opType != "batchNormTrain" || bn.deps.size() != 5 || off != 0 || fusedKind[b] ||
-                    op.volume() != g.ops[bn.deps[0]].volume())
-                    continue;
-                bool ok = true;  // the y part may only feed this relu and the x operand of reluGrad (a sign test)
-                for (size_t e : exposed[b]) ok = ok && e >= op.bytes();  // outputs may expose the statistics only
-                for (const Use &u : uses[b])
-                    if (u.off == 0 && !(u.op == id || (g.ops[u.op].opType == "reluGrad" && u.slot == 2))) ok = false;
-                if (!ok) continue;
-                fusedKind[b] = 2;
-                alias[id].source = b;  // the relu output IS the y part now
-                alias[id].offset = 0;
-            } else if (op.opType == "batchNormGrad" && op.deps.size() == 3) {
-                size_t off;
-                const int rg = root(op.deps[0], &off);
-                const Operation &rgo = g.ops[rg];
-                // the fused kernel tests the sign of y where reluGrad tests x: the same thing when y = relu(x)
-                const bool pair = rgo.opType == "reluGrad" && rgo.deps.size() == 3 &&
-                                  g.ops[rgo.deps[1]].opType == "relu" && g.ops[rgo.deps[1]].deps.size() == 1 &&
-                                  g.ops[rgo.deps[1]].deps[0] == rgo.deps[2];
-                if (pair && off == 0 && alias[rg].source < 0 &&
-                    !isOutput(rg) && uses[rg].size() == 1 && rgo.volume() == g.ops[op.deps[1]].volume()) {
-                    fusedKind[id] = 3;
-                    inputsOf[id] = {rgo.deps[0], rgo.deps[1], op.deps[1], op.deps[2]};
-                }
-            }
-        }
-
-        // matmul reads a transposed operand in place instead of a copy made by `transpose`, and
-        // transpose(matmul(A, B)) is computed as matmul(B^T, A^T); the transposes left without a
-        // reader drop out.
-        auto is_swap = [&](int t) {
-            const Operation &o = g.ops[t];
-            if (o.opType != "transpose" || o.deps.size() != 1 || o.rank() != 2 || alias[t].source >= 0) return false;
-            auto it = o.sizeAttrs.find("order");
-            return it != o.sizeAttrs.end() && it->second.size() == 2 && it->second[0] == 1 && it->second[1] == 0 &&
-                   o.dtype == DOPT_HIP_F32;
-        };
-        auto through = [&](int id, bool *flip) {  // the matrix behind a chain of 2-d transposes
-            *flip = false;
-            while (is_swap(id)) {
-                id = g.ops[id].deps[0];
-                *flip = !*flip;
-            }
-            return id;
-        };
-        auto plain_matmul = [&](int m) {
-            const Operation &o = g.ops[m];
-            return o.opType == "matmul" && o.deps.size() == 2 && o.rank() == 2 && o.dtype == DOPT_HIP_F32 &&
-                   alias[m].source < 0;
-        };
-        for (int id : p->mOps) {
-            if (!live[id]) continue;
-            int mm = id;
-            bool outT = false;  // compute the transpose of the product
-            if (is_swap(id) && plain_matmul(g.ops[id].deps[0]) && uses[g.ops[id].deps[0]].size() == 1 &&
-                !isOutput(g.ops[id].deps[0])) {
-                mm = g.ops[id].deps[0];
-                outT = true;
-            } else if (!plain_matmul(id)) {
-                continue;
-            }
-            if (!outT && fusedKind[id]) continue;
-            bool tA, tB;
-            int a = through(g.ops[mm].deps[0], &tA), b = through(g.ops[mm].deps[1], &tB);
-            if (!outT && a == g.ops[mm].deps[0] && b == g.ops[mm].deps[1]) continue;  // nothing to fold
-            if (!outT && uses[mm].size() == 1 && is_swap(uses[mm][0].op) && !isOutput(mm)) continue;  // folded into its transpose
-            size_t M = g.ops[mm].shape[0], N = g.ops[mm].shape[1];
-            const Operation &ao = g.ops[g.ops[mm].deps[0]];
-            size_t K = ao.shape[1];
-            if (outT) {  // (A B)^T = B^T A^T
-                std::swap(a, b);
-                const bool na = !tB, nb = !tA;
-                tA = na;
-                tB = nb;
-                std::swap(M, N);
-            }
-            fusedKind[id] = 6;
-            inputsOf[id] = {a, b};
-            const int ta = tA, tb = tB;
-            prebuilt[id] = make([=](const std::vector<const void *> &in, void *out) {
-                return dopt_hip_sgemm_t(ta, tb, M, N, K, (const float *)in[0], (const float *)in[1], (float *)out);
-            });
-            prebuiltLabel[id] = outT ? "matmul+transpose" : "matmul";
-        }
-
-        // Pointwise chains: a pointwise operation whose value is read only by pointwise operations
-        // of one chain (and by no plan output) is computed inside that chain's kernel and never
-        // stored; an operand of the form repeat(one-element tensor) is read from the element itself.
-        // Walking consumers before producers, an operation joins the chain all its readers belong to
-        // or starts a chain of its own.
-        // What may be a node: the pointwise operations; relu and reluGrad(dy, y, x) (a node of dy and x),
-        // unless a batch-norm fusion above already reads around them; and a product [m,1] x [1,n] - the
-        // reference's way to broadcast a column or a row (core/ops/basic.d:370-381) - as the node
-        // mul(per-row element, per-column element) of the chain's [m, n] view.
-        auto outer_cols = [&](int id) -> size_t {   // n of such a product, else 0
-            const Operation &o = g.ops[id];
-            if (o.opType != "matmul" || o.deps.size() != 2 || o.rank() != 2 || o.dtype != DOPT_HIP_F32) return 0;
-            const Operation &l = g.ops[o.deps[0]], &r = g.ops[o.deps[1]];
-            if (l.rank() != 2 || r.rank() != 2 || l.shape[1] != 1 || r.shape[0] != 1) return 0;
-            return o.shape[1];
-        };
-        auto is_pw = [&](int id) {
-            const Operation &o = g.ops[id];
-            if (!live[id] || alias[id].source >= 0 || fusedKind[id] || o.dtype != DOPT_HIP_F32 || o.volume() == 0) return false;
-            if (o.opType == "reluGrad" && o.deps.size() == 3) {
-                for (const Use &u : uses[id])
-                    if (fusedKind[u.op] == 3) return false;   // that batchNormGrad reads dy and y itself
-                return true;
-            }
-            if (outer_cols(id)) return true;
-            const int arity = dopt_hip_pointwise_arity(o.opType.c_str());
-            return arity > 0 && arity == (int)o.deps.size();
-        };
-        std::vector<int> chainOf((size_t)nops, -1);              // the operation that ends the chain
-        std::vector<std::vector<int>> chainOps((size_t)nops);    // per chain end: its members
-        std::vector<size_t> chainInner((size_t)nops, 0);         // per chain end: columns of its [rows, inner] view, once a member needs one
-        for (auto it = p->mOps.rbegin(); it != p->mOps.rend(); ++it) {
-            const int id = *it;
-            if (!is_pw(id)) continue;
-            int target = -1;
-            bool joins = !isOutput(id) && !uses[id].empty();
-            for (const Use &u : uses[id]) {
-                if (!joins) break;
-                if (chainOf[u.op] < 0 || u.off != 0 || g.ops[u.op].volume() != g.ops[id].volume()) joins = false;
-                else if (g.ops[u.op].opType == "reluGrad" && u.slot == 1) joins = false;   // the y operand is not part of the node
-                else if (target < 0) target = chainOf[u.op];
-                else if (target != chainOf[u.op]) joins = false;
-            }
-            if (joins && chainOps[target].size() >= 48) joins = false;
-            const size_t cols = outer_cols(id);
-            if (joins && cols && chainInner[target] && chainInner[target] != cols) joins = false;
-            chainOf[id] = joins ? target : id;
-            chainOps[chainOf[id]].push_back(id);
-            if (cols) chainInner[chainOf[id]] = cols;
-        }
-        for (int end : p->mOps) {
-            if (chainOf[end] != end || chainOps[end].size() < 2) continue;
-            std::vector<int> members;                             // in execution order
-            for (int id : p->mOps)
-                if (chainOf[id] == end) members.push_back(id);
-            std::vector<int> inputs;                              // operations whose buffers the kernel reads
-            std::vector<unsigned char> kinds;                     // 0 tensor, 1 one element, 2 per row, 3 per column
-            std::vector<int> nodeOf((size_t)nops, -1);
-            struct Node { std::string op; int lhs, rhs; };
-            std::vector<Node> nodes;
-            auto input_index = [&](int op, int kind) {
-                for (size_t k = 0; k < inputs.size(); k++)
-                    if (inputs[k] == op && kinds[k] == (unsigned char)kind) return (int)k;
-                inputs.push_back(op);
-                kinds.push_back((unsigned char)kind);
-                return (int)inputs.size() - 1;
-            };
-            auto operand = [&](int dep) {                         // index of a member's operand: a node (<= -2) or an input
-                size_t off;
-                const int r = root(dep, &off);
-                if (chainOf[r] == end && nodeOf[r] >= 0 && off == 0) return -2 - nodeOf[r];
-                const Operation &ro = g.ops[r];
-                size_t soff = 0;
-                if (ro.opType == "repeat" && ro.deps.size() == 1 && off == 0 && alias[r].source < 0 &&
-                    g.ops[ro.deps[0]].volume() == 1 && g.ops[root(ro.deps[0], &soff)].dtype == DOPT_HIP_F32)
-                    return input_index(ro.deps[0], 1);
-                return input_index(dep, 0);
-            };
-            for (int id : members) {
-                const Operation &o = g.ops[id];
-                Node node{o.opType, -1, -1};
-                if (outer_cols(id)) {
-                    node.op = "mul";
-                    node.lhs = input_index(o.deps[0], 2);
-                    node.rhs = input_index(o.deps[1], 3);
-                } else if (o.opType == "reluGrad") {
-                    node.lhs = operand(o.deps[0]);
-                    node.rhs = operand(o.deps[2]);
-                } else {
-                    node.lhs = operand(o.deps[0]);
-                    if (o.deps.size() > 1) node.rhs = operand(o.deps[1]);
-                }
-                nodeOf[id] = (int)nodes.size();
-                nodes.push_back(node);
-            }
-            if (inputs.empty() || inputs.size() > 12) continue;   // too wide: its members keep their own kernels
-            const int nin = (int)inputs.size();
-            for (Node &n : nodes) {
-                if (n.lhs <= -2) n.lhs = nin + (-2 - n.lhs);
-                if (n.rhs <= -2) n.rhs = nin + (-2 - n.rhs);
-                if (n.rhs < 0) n.rhs = n.lhs;
-            }
-            for (int id : members) fusedKind[id] = 7;
-            inputsOf[end] = inputs;
-            const size_t count = g.ops[end].volume(), inner = chainInner[end];
-            prebuilt[end] = make([=](const std::vector<const void *> &in, void *out) {
-                const char *names[64];
-                int lhs[64], rhs[64];
-                for (size_t j = 0; j < nodes.size(); j++) {
-                    names[j] = nodes[j].op.c_str();
-                    lhs[j] = nodes[j].lhs;
-                    rhs[j] = nodes[j].rhs;
-                }
-                return dopt_hip_pointwise_chain(DOPT_HIP_F32, count, inner, nin, in.data(), kinds.data(), (int)nodes.size(),
-                                                names, lhs, rhs, out);
-            });
-            prebuiltLabel[end] = "pointwise*" + std::to_string(nodes.size());   // no spaces: profile lines are split on them
+void HIPPlan::Builder::countReaders()
+{
+    // readers are counted among the operations that are live after the alias rewrites
+    {
+        std::vector<int> work(outputs.begin(), outputs.end());
+        while (!work.empty()) {
+            int id = work.back();
+            work.pop_back();
+            if (live[id]) continue;
+            live[id] = 1;
+            if (alias[id].source >= 0) work.push_back(alias[id].source);
+            else for (int d : g.ops[id].deps) work.push_back(d);
         }
     }
+    for (int id : p->mOps) {
+        if (!live[id] || alias[id].source >= 0) continue;
+        const Operation &op = g.ops[id];
+        for (size_t j = 0; j < op.deps.size(); j++) {
+            size_t off;
+            const int r = root(op.deps[j], &off);
+            uses[r].push_back({id, (int)j, off});
+        }
+    }
+    // byte offsets at which plan outputs (or aliases of them) expose a buffer
+    for (int o : outputs) {
+        size_t off;
+        const int r = root(o, &off);
+        exposed[r].push_back(off);
+    }
+}
 
+// A pair of operations runs as one kernel when the value between them has no other reader.
+void HIPPlan::Builder::fusePairs()
+{
+    for (int id : p->mOps) {
+        const Operation &op = g.ops[id];
+        if (alias[id].source >= 0) continue;
+        if (op.opType == "addBias" && op.deps.size() == 2) {
+            const int c = op.deps[0];
+            if (g.ops[c].opType == "convolution" && g.ops[c].deps.size() == 2 && alias[c].source < 0 && !isOutput(c) &&
+                uses[c].size() == 1 && g.ops[c].dtype == DOPT_HIP_F32) {
+                fusedKind[id] = 1;
+                inputsOf[id] = {g.ops[c].deps[0], g.ops[c].deps[1], op.deps[1]};
+            }
+        } else if (op.opType == "relu" && op.deps.size() == 1) {
+            size_t off;
+            const int b = root(op.deps[0], &off);
+            const Operation &bn = g.ops[b];
+            if (bn.opType != "batchNormTrain" || bn.deps.size() != 5 || off != 0 || fusedKind[b] ||
+                op.volume() != g.ops[bn.deps[0]].volume())
+                continue;
+            bool ok = true;  // the y part may only feed this relu and the x operand of reluGrad (a sign test)
+            for (size_t e : exposed[b]) ok = ok && e >= op.bytes();  // outputs may expose the statistics only
+            for (const Use &u : uses[b])
+                if (u.off == 0 && !(u.op == id || (g.ops[u.op].opType == "reluGrad" && u.slot == 2))) ok = false;
+            if (!ok) continue;
+            fusedKind[b] = 2;
+            alias[id].source = b;  // the relu output IS the y part now
+            alias[id].offset = 0;
+        } else if (op.opType == "batchNormGrad" && op.deps.size() == 3) {
+            size_t off;
+            const int rg = root(op.deps[0], &off);
+            const Operation &rgo = g.ops[rg];
+            // the fused kernel tests the sign of y where reluGrad tests x: the same thing when y = relu(x)
+            const bool pair = rgo.opType == "reluGrad" && rgo.deps.size() == 3 &&
+                              g.ops[rgo.deps[1]].opType == "relu" && g.ops[rgo.deps[1]].deps.size() == 1 &&
+                              g.ops[rgo.deps[1]].deps[0] == rgo.deps[2];
+            if (pair && off == 0 && alias[rg].source < 0 &&
+                !isOutput(rg) && uses[rg].size() == 1 && rgo.volume() == g.ops[op.deps[1]].volume()) {
+                fusedKind[id] = 3;
+                inputsOf[id] = {rgo.deps[0], rgo.deps[1], op.deps[1], op.deps[2]};
+            }
+        }
+    }
+}
+
+void HIPPlan::Builder::foldTransposes()
+{
+    // matmul reads a transposed operand in place instead of a copy made by `transpose`, and
+    // transpose(matmul(A, B)) is computed as matmul(B^T, A^T); the transposes left without a
+    // reader drop out.
+    auto is_swap = [&](int t) {
+        const Operation &o = g.ops[t];
+        if (o.opType != "transpose" || o.deps.size() != 1 || o.rank() != 2 || alias[t].source >= 0) return false;
+        auto it = o.sizeAttrs.find("order");
+        return it != o.sizeAttrs.end() && it->second.size() == 2 && it->second[0] == 1 && it->second[1] == 0 &&
+               o.dtype == DOPT_HIP_F32;
+    };
+    auto through = [&](int id, bool *flip) {  // the matrix behind a chain of 2-d transposes
+        *flip = false;
+        while (is_swap(id)) {
+            id = g.ops[id].deps[0];
+            *flip = !*flip;
+        }
+        return id;
+    };
+    auto plain_matmul = [&](int m) {
+        const Operation &o = g.ops[m];
+        return o.opType == "matmul" && o.deps.size() == 2 && o.rank() == 2 && o.dtype == DOPT_HIP_F32 &&
+               alias[m].source < 0;
+    };
+    for (int id : p->mOps) {
+        if (!live[id]) continue;
+        int mm = id;
+        bool outT = false;  // compute the transpose of the product
+        if (is_swap(id) && plain_matmul(g.ops[id].deps[0]) && uses[g.ops[id].deps[0]].size() == 1 &&
+            !isOutput(g.ops[id].deps[0])) {
+            mm = g.ops[id].deps[0];
+            outT = true;
+        } else if (!plain_matmul(id)) {
+            continue;
+        }
+        if (!outT && fusedKind[id]) continue;
+        bool tA, tB;
+        int a = through(g.ops[mm].deps[0], &tA), b = through(g.ops[mm].deps[1], &tB);
+        if (!outT && a == g.ops[mm].deps[0] && b == g.ops[mm].deps[1]) continue;  // nothing to fold
+        if (!outT && uses[mm].size() == 1 && is_swap(uses[mm][0].op) && !isOutput(mm)) continue;  // folded into its transpose
+        size_t M = g.ops[mm].shape[0], N = g.ops[mm].shape[1];
+        const Operation &ao = g.ops[g.ops[mm].deps[0]];
+        size_t K = ao.shape[1];
+        if (outT) {  // (A B)^T = B^T A^T
+            std::swap(a, b);
+            const bool na = !tB, nb = !tA;
+            tA = na;
+            tB = nb;
+            std::swap(M, N);
+        }
+        fusedKind[id] = 6;
+        inputsOf[id] = {a, b};
+        const int ta = tA, tb = tB;
+        prebuilt[id] = make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_sgemm_t(ta, tb, M, N, K, (const float *)in[0], (const float *)in[1], (float *)out);
+        });
+        prebuiltLabel[id] = outT ? "matmul+transpose" : "matmul";
+    }
+}
+
+void HIPPlan::Builder::formChains()
+{
+    // Pointwise chains: a pointwise operation whose value is read only by pointwise operations
+    // of one chain (and by no plan output) is computed inside that chain's kernel and never
+    // stored; an operand of the form repeat(one-element tensor) is read from the element itself.
+    // Walking consumers before producers, an operation joins the chain all its readers belong to
+    // or starts a chain of its own.
+    // What may be a node: the pointwise operations; relu and reluGrad(dy, y, x) (a node of dy and x),
+    // unless a batch-norm fusion above already reads around them; and a product [m,1] x [1,n] - the
+    // reference's way to broadcast a column or a row (core/ops/basic.d:370-381) - as the node
+    // mul(per-row element, per-column element) of the chain's [m, n] view.
+    auto outer_cols = [&](int id) -> size_t {   // n of such a product, else 0
+        const Operation &o = g.ops[id];
+        if (o.opType != "matmul" || o.deps.size() != 2 || o.rank() != 2 || o.dtype != DOPT_HIP_F32) return 0;
+        const Operation &l = g.ops[o.deps[0]], &r = g.ops[o.deps[1]];
+        if (l.rank() != 2 || r.rank() != 2 || l.shape[1] != 1 || r.shape[0] != 1) return 0;
+        return o.shape[1];
+    };
+    auto is_pw = [&](int id) {
+        const Operation &o = g.ops[id];
+        if (!live[id] || alias[id].source >= 0 || fusedKind[id] || o.dtype != DOPT_HIP_F32 || o.volume() == 0) return false;
+        if (o.opType == "reluGrad" && o.deps.size() == 3) {
+            for (const Use &u : uses[id])
+                if (fusedKind[u.op] == 3) return false;   // that batchNormGrad reads dy and y itself
+            return true;
+        }
+        if (outer_cols(id)) return true;
+        const int arity = dopt_hip_pointwise_arity(o.opType.c_str());
+        return arity > 0 && arity == (int)o.deps.size();
+    };
+    std::vector<int> chainOf((size_t)nops, -1);              // the operation that ends the chain
+    std::vector<std::vector<int>> chainOps((size_t)nops);    // per chain end: its members
+    std::vector<size_t> chainInner((size_t)nops, 0);         // per chain end: columns of its [rows, inner] view, once a member needs one
+    for (auto it = p->mOps.rbegin(); it != p->mOps.rend(); ++it) {
+        const int id = *it;
+        if (!is_pw(id)) continue;
+        int target = -1;
+        bool joins = !isOutput(id) && !uses[id].empty();
+        for (const Use &u : uses[id]) {
+            if (!joins) break;
+            if (chainOf[u.op] < 0 || u.off != 0 || g.ops[u.op].volume() != g.ops[id].volume()) joins = false;
+            else if (g.ops[u.op].opType == "reluGrad" && u.slot == 1) joins = false;   // the y operand is not part of the node
+            else if (target < 0) target = chainOf[u.op];
+            else if (target != chainOf[u.op]) joins = false;
+        }
+        if (joins && chainOps[target].size() >= 48) joins = false;
+        const size_t cols = outer_cols(id);
+        if (joins && cols && chainInner[target] && chainInner[target] != cols) joins = false;
+        chainOf[id] = joins ? target : id;
+        chainOps[chainOf[id]].push_back(id);
+        if (cols) chainInner[chainOf[id]] = cols;
+    }
+    for (int end : p->mOps) {
+        if (chainOf[end] != end || chainOps[end].size() < 2) continue;
+        std::vector<int> members;                             // in execution order
+        for (int id : p->mOps)
+            if (chainOf[id] == end) members.push_back(id);
+        std::vector<int> inputs;                              // operations whose buffers the kernel reads
+        std::vector<unsigned char> kinds;                     // 0 tensor, 1 one element, 2 per row, 3 per column
+        std::vector<int> nodeOf((size_t)nops, -1);
+        struct Node { std::string op; int lhs, rhs; };
+        std::vector<Node> nodes;
+        auto input_index = [&](int op, int kind) {
+            for (size_t k = 0; k < inputs.size(); k++)
+                if (inputs[k] == op && kinds[k] == (unsigned char)kind) return (int)k;
+            inputs.push_back(op);
+            kinds.push_back((unsigned char)kind);
+            return (int)inputs.size() - 1;
+        };
+        auto operand = [&](int dep) {                         // index of a member's operand: a node (<= -2) or an input
+            size_t off;
+            const int r = root(dep, &off);
+            if (chainOf[r] == end && nodeOf[r] >= 0 && off == 0) return -2 - nodeOf[r];
+            const Operation &ro = g.ops[r];
+            size_t soff = 0;
+            if (ro.opType == "repeat" && ro.deps.size() == 1 && off == 0 && alias[r].source < 0 &&
+                g.ops[ro.deps[0]].volume() == 1 && g.ops[root(ro.deps[0], &soff)].dtype == DOPT_HIP_F32)
+                return input_index(ro.deps[0], 1);
+            return input_index(dep, 0);
+        };
+        for (int id : members) {
+            const Operation &o = g.ops[id];
+            Node node{o.opType, -1, -1};
+            if (outer_cols(id)) {
+                node.op = "mul";
+                node.lhs = input_index(o.deps[0], 2);
+                node.rhs = input_index(o.deps[1], 3);
+            } else if (o.opType == "reluGrad") {
+                node.lhs = operand(o.deps[0]);
+                node.rhs = operand(o.deps[2]);
+            } else {
+                node.lhs = operand(o.deps[0]);
+                if (o.deps.size() > 1) node.rhs = operand(o.deps[1]);
+            }
+            nodeOf[id] = (int)nodes.size();
+            nodes.push_back(node);
+        }
+        if (inputs.empty() || inputs.size() > 12) continue;   // too wide: its members keep their own kernels
+        const int nin = (int)inputs.size();
+        for (Node &n : nodes) {
+            if (n.lhs <= -2) n.lhs = nin + (-2 - n.lhs);
+            if (n.rhs <= -2) n.rhs = nin + (-2 - n.rhs);
+            if (n.rhs < 0) n.rhs = n.lhs;
+        }
+        for (int id : members) fusedKind[id] = 7;
+        inputsOf[end] = inputs;
+        const size_t count = g.ops[end].volume(), inner = chainInner[end];
+        prebuilt[end] = make([=](const std::vector<const void *> &in, void *out) {
+            const char *names[64];
+            int lhs[64], rhs[64];
+            for (size_t j = 0; j < nodes.size(); j++) {
+                names[j] = nodes[j].op.c_str();
+                lhs[j] = nodes[j].lhs;
+                rhs[j] = nodes[j].rhs;
+            }
+            return dopt_hip_pointwise_chain(DOPT_HIP_F32, count, inner, nin, in.data(), kinds.data(), (int)nodes.size(),
+                                            names, lhs, rhs, out);
+        });
+        prebuiltLabel[end] = "pointwise*" + std::to_string(nodes.size());   // no spaces: profile lines are split on them
+    }
+}
+
+void HIPPlan::Builder::absorbBiasGrads()
+{
     // addBiasGrad(dx of a batchNormGrad): the batch-norm kernel writes the bias gradient too.  The
     // addBiasGrad operation keeps its buffer but gets no kernel of its own.
-    std::vector<int> biasGradOf((size_t)nops, -1);  // batchNormGrad op -> the addBiasGrad op it serves
-    std::vector<char> absorbed((size_t)nops, 0);
     if (flags & DOPT_HIP_PLAN_FUSE) {
         for (int id : p->mOps) {
             const Operation &op = g.ops[id];
@@ -895,9 +936,11 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
             absorbed[id] = 1;
         }
     }
+}
 
+void HIPPlan::Builder::markNeeded()
+{
     // operations whose results are actually consumed (everything, unless rewrites created dead ones)
-    std::vector<char> needed((size_t)nops, 0);
     {
         std::vector<int> work(outputs.begin(), outputs.end());
         while (!work.empty()) {
@@ -909,14 +952,14 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
             else for (int d : inputsOf[id]) work.push_back(d);
         }
     }
+}
 
+int HIPPlan::Builder::prepackFilters()
+{
     // Filters packed ahead (DOPT_HIP_PLAN_FUSE): the forward and backward-data kernels of 3x3
     // convolutions read the filter in their own layout.  When the filter is a variable or a constant
     // - fixed while the plan runs - every such layout of the plan is produced by ONE launch at the
     // start of each execution instead of one small launch in front of every convolution.
-    struct Prepack { int op, filter; int bwd; dopt_hip_conv_desc d; void *buf; bool owner; };
-    std::vector<Prepack> packs;
-    std::vector<int> packOf((size_t)nops, -1);
     if (flags & DOPT_HIP_PLAN_FUSE) {
         for (int id : p->mOps) {
             if (!needed[id] || alias[id].source >= 0 || absorbed[id] || prebuilt[id]) continue;
@@ -984,7 +1027,11 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         for (size_t i = 0; i < s.inputOps.size(); i++) s.inputBytes[i] = g.ops[s.inputOps[i]].bytes();
         p->mSteps.push_back(std::move(s));
     }
+    return DOPT_HIP_OK;
+}
 
+int HIPPlan::Builder::allocateBuffers()
+{
     // buffers first: a fused kernel may write into the buffer of a later operation
     for (int id : p->mOps) {
         if (!needed[id] || is_leaf(g.ops[id]) || alias[id].source >= 0) continue;
@@ -994,7 +1041,11 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         p->mBufferBytes += g.ops[id].bytes();
         p->mResults[id] = buf;
     }
+    return DOPT_HIP_OK;
+}
 
+int HIPPlan::Builder::buildSteps()
+{
     // kernels and buffers
     for (int id : p->mOps) {
         if (!needed[id]) continue;
@@ -1060,6 +1111,11 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         for (size_t i = 0; i < s.inputOps.size(); i++) s.inputBytes[i] = g.ops[s.inputOps[i]].bytes();
         p->mSteps.push_back(std::move(s));
     }
+    return DOPT_HIP_OK;
+}
+
+void HIPPlan::Builder::rememberAliases()
+{
     // remember aliases for the per-execution resolve pass
     for (int id : p->mOps)
         if (needed[id] && alias[id].source >= 0) p->mResults[id] = nullptr;
@@ -1071,6 +1127,10 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
             p->mAliasOffset[id] = alias[id].offset;
         }
     p->mNeeded = needed;
+}
+
+int HIPPlan::Builder::assignQueues()
+{
     if (flags & DOPT_HIP_PLAN_OVERLAP) {
         // A filter gradient feeds nothing of the backward chain: it, and every step that reads a
         // side-queue result, goes to the side queue.  Steps keep their order within each queue.
@@ -1101,6 +1161,11 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
             for (hipEvent_t &ev : p->mFences) DOPT_HIP_CHECK(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
         }
     }
+    return DOPT_HIP_OK;
+}
+
+int HIPPlan::Builder::createEvents()
+{
     // what a recorded graph cannot reproduce: per-kernel timing events, the second queue, and `uniform`,
     // whose kernel takes a call counter that changes with every execution
     p->mGraphOk = !(flags & DOPT_HIP_PLAN_TIMING) && !p->mUsesSide;
@@ -1113,6 +1178,44 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
             DOPT_HIP_CHECK(hipEventCreate(&ev.second));
         }
     }
+    return DOPT_HIP_OK;
+}
+
+int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flags, std::unique_ptr<HIPPlan> *out)
+{
+    registerBuiltinKernels();
+    if (!ensure_init()) return DOPT_HIP_ERR_RUNTIME;
+    const Graph &g = *graph;
+    const int nops = (int)g.ops.size();
+    for (int o : outputs)
+        if (o < 0 || o >= nops) return fail(DOPT_HIP_ERR_INVALID, "plan output %d is not an operation of the graph", o);
+
+    std::unique_ptr<HIPPlan> p(new HIPPlan());
+    p->mGraph = graph;
+    p->mFlags = flags;
+    p->mOutputs = outputs;
+    std::vector<char> seen((size_t)nops, 0);
+    for (int o : outputs) toposort(g, o, seen, p->mOps);
+
+    Builder b(g, p.get(), outputs, flags);
+    if (int rc = b.findAliases()) return rc;
+    for (int id : p->mOps) b.inputsOf[id] = g.ops[id].deps;
+    if (flags & DOPT_HIP_PLAN_FUSE) {
+        b.countReaders();
+        b.fusePairs();
+        b.foldTransposes();
+        b.formChains();
+        b.absorbBiasGrads();
+    }
+    b.markNeeded();
+    if (flags & DOPT_HIP_PLAN_FUSE)
+        if (int rc = b.prepackFilters()) return rc;
+    if (int rc = b.allocateBuffers()) return rc;
+    if (int rc = b.buildSteps()) return rc;
+    b.rememberAliases();
+    if (flags & DOPT_HIP_PLAN_OVERLAP)
+        if (int rc = b.assignQueues()) return rc;
+    if (int rc = b.createEvents()) return rc;
     // Resolve aliases once against the variables' own values so that result() is meaningful before
     // the first execution (an alias of a variable that is later passed as an argument moves with it).
     if (int rc = p->resolve(0, nullptr, nullptr, nullptr)) return rc;

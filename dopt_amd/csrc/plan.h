@@ -95,6 +95,7 @@ public:
 
 private:
     HIPPlan() = default;
+    struct Builder;                              // create() in passes (plan.cpp)
     struct Step {
         int op;
         std::string label;                       // profiler key: the opType, or "a+b" for a fused pair
