@@ -810,6 +810,11 @@ void HIPPlan::Builder::formChains()
         if (l.rank() != 2 || r.rank() != 2 || l.shape[1] != 1 || r.shape[0] != 1) return 0;
         return o.shape[1];
     };
+    // with one row or one column the product is a tensor times a single element: no [rows, inner] view needed
+    auto outer_grid = [&](int id) -> size_t {
+        const size_t n = outer_cols(id);
+        return n > 1 && g.ops[id].shape[0] > 1 ? n : 0;
+    };
     auto is_pw = [&](int id) {
         const Operation &o = g.ops[id];
         if (!live[id] || alias[id].source >= 0 || fusedKind[id] || o.dtype != DOPT_HIP_F32 || o.volume() == 0) return false;
@@ -838,7 +843,7 @@ void HIPPlan::Builder::formChains()
             else if (target != chainOf[u.op]) joins = false;
         }
         if (joins && chainOps[target].size() >= 48) joins = false;
-        const size_t cols = outer_cols(id);
+        const size_t cols = outer_grid(id);
         if (joins && cols && chainInner[target] && chainInner[target] != cols) joins = false;
         chainOf[id] = joins ? target : id;
         chainOps[chainOf[id]].push_back(id);
@@ -877,8 +882,9 @@ void HIPPlan::Builder::formChains()
             Node node{o.opType, -1, -1};
             if (outer_cols(id)) {
                 node.op = "mul";
-                node.lhs = input_index(o.deps[0], 2);
-                node.rhs = input_index(o.deps[1], 3);
+                const bool one_col = o.shape[1] == 1, one_row = o.shape[0] == 1;
+                node.lhs = input_index(o.deps[0], one_row ? 1 : (one_col ? 0 : 2));
+                node.rhs = input_index(o.deps[1], one_col ? 1 : (one_row ? 0 : 3));
             } else if (o.opType == "reluGrad") {
                 node.lhs = operand(o.deps[0]);
                 node.rhs = operand(o.deps[2]);
