@@ -1360,6 +1360,55 @@ int run_dense2x2(const dopt_hip_conv_desc *d, const float *in, const float *w, c
     return rc;
 }
 
+// Filter gradient of the same layers: dWd = x^T * dy, [4C, N] x [N, 4K], is the gradient of the matrix
+// above; every filter tap collects the (input pixel, output pixel) pairs that read it - one pair for
+// a corner tap, two for an edge tap, four for the centre - in a fixed order.
+__global__ __launch_bounds__(256) void fold_2x2_k(unsigned C, unsigned K, const float4 *dwd, float *dw)
+{
+    const size_t total = (size_t)C * K;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        const unsigned k = (unsigned)(i % K), c = (unsigned)(i / K);
+        float q[4][4];   // [input pixel iy*2+ix][output pixel oy*2+ox]
+#pragma unroll
+        for (int pin = 0; pin < 4; pin++) {
+            const float4 v = dwd[((size_t)c * 4 + pin) * K + k];
+            q[pin][0] = v.x; q[pin][1] = v.y; q[pin][2] = v.z; q[pin][3] = v.w;
+        }
+        float *out = dw + ((size_t)k * C + c) * 9;
+#pragma unroll
+        for (int a = 0; a < 3; a++)
+#pragma unroll
+            for (int b = 0; b < 3; b++) {
+                float sum = 0.0f;   // pairs with 1 - iy + oy == a and 1 - ix + ox == b
+#pragma unroll
+                for (int iy = 0; iy < 2; iy++)
+#pragma unroll
+                    for (int ix = 0; ix < 2; ix++) {
+                        const int oy = a - 1 + iy, ox = b - 1 + ix;
+                        if (oy >= 0 && oy < 2 && ox >= 0 && ox < 2) sum += q[iy * 2 + ix][oy * 2 + ox];
+                    }
+                out[a * 3 + b] = sum;
+            }
+    }
+}
+
+int run_dense2x2_wgrad(const dopt_hip_conv_desc *d, const float *dy, const float *x, float *dw)
+{
+    void *dwd = nullptr;
+    if (int rc = scratch_alloc(&dwd, dense2x2_elems(d) * sizeof(float))) return rc;
+    bool biased = false;
+    int rc = sgemm_bias(1, 0, 4 * d->C, 4 * d->K, d->N, x, dy, (float *)dwd, nullptr, 0, &biased);
+    if (!rc) {
+        const size_t blocks = ceil_div(d->C * d->K, (size_t)256);
+        const size_t cap = (size_t)num_cus() * 16;
+        hipLaunchKernelGGL(fold_2x2_k, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0, stream(), (unsigned)d->C,
+                           (unsigned)d->K, (const float4 *)dwd, dw);
+        if (hipGetLastError() != hipSuccess) rc = fail(DOPT_HIP_ERR_RUNTIME, "convolution: fold launch failed");
+    }
+    dopt_hip_free(dwd);
+    return rc;
+}
+
 // Packs the filter w[K][C][g.R * g.S] and runs conv_gather_k on a problem whose geometry the caller
 // has filled in (dimensions, padding, stride, output placement).  mode as conv_gather_k's kMode.
 int gather_launch(GatherConv g, int mode, int K, int C, const float *in, const float *w, float *out)
@@ -1810,6 +1859,7 @@ int dopt_hip_conv_bwd_filter(const dopt_hip_conv_desc *d, const float *dy, const
         bool done = false;
         if (int rc = conv_smallc_wgrad(d, dy, x, dw, &done)) return rc;
         if (done) return DOPT_HIP_OK;
+        if (dense2x2_takes(d)) return run_dense2x2_wgrad(d, dy, x, dw);
         if (int rc = run_wgrad_patch(d, dy, x, dw, &done)) return rc;
         if (done) return DOPT_HIP_OK;
     }

@@ -362,12 +362,14 @@ int sgemm_bias(int transA, int transB, size_t M, size_t N, size_t K, const float
         return DOPT_HIP_OK;
     }
 
-    // small outputs: one block per 32 x 32 tile, the reduction split over its wavefronts.  Each tile
-    // reads its own 32 rows of A and 32 columns of B, so the operand traffic grows with the number
-    // of tiles; past a few hundred tiles the LDS-tiled engine below is the better fit.
+    // small and medium outputs: one block per 32 x 32 tile, the reduction split over its wavefronts.
+    // Each tile reads its own 32 rows of A and 32 columns of B, so the operand traffic grows with the
+    // number of tiles: up to 256 MB of it (served by the L2) this beats the LDS-tiled engine below,
+    // whose 128-wide tiles leave most CUs with one four-wavefront block (1024 x 1024 x 256: 11 against
+    // 22 us; 2048 x 2048 x 128: 21 against 31 us); beyond that the tile engine's operand reuse wins.
     {
         const size_t tiles = ceil_div(M, (size_t)32) * ceil_div(N, (size_t)32);
-        if (tiles <= 512 && tiles * 64 * K * sizeof(float) <= ((size_t)256 << 20)) {
+        if (tiles <= 4096 && tiles * 64 * K * sizeof(float) <= ((size_t)256 << 20)) {
             const int lda = (int)(transA ? M : K), ldb = (int)(transB ? K : N);
             int kslice = (int)ceil_div(ceil_div(K, (size_t)kSmallWaves), (size_t)8) * 8;
             const bool vec = aligned16(A) && aligned16(B) && lda % 4 == 0 && ldb % 4 == 0;
