@@ -1295,24 +1295,30 @@ int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, 
 // is dy * Wd^T, so one copy of Wd serves both directions.
 __global__ __launch_bounds__(256) void pack_2x2_k(unsigned C, unsigned K, const float *w, float4 *wd)
 {
-    // a lane per (input channel c, output channel k), k fastest: it reads the nine taps of that filter
-    // plane once and writes the four quads (one per input pixel) of column group k; lanes of a
-    // wavefront write neighbouring quads
-    const size_t total = (size_t)C * K;
-    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
-        const unsigned k = (unsigned)(i % K), c = (unsigned)(i / K);
-        const float *src = w + ((size_t)k * C + c) * 9;
-        float f[9];
+    // A block takes 8 output channels x 64 input channels.  It reads their filter planes as eight
+    // contiguous runs of 64 x 9 floats, and after a pass through LDS writes, for each of the 256
+    // (input channel, input pixel) rows, the eight quads of its output channels: one full 128-byte line.
+    __shared__ float stage[8][64 * 9 + 1];
+    const unsigned k0 = blockIdx.x * 8, c0 = blockIdx.y * 64;
+    const unsigned nk = min(8u, K - k0), nc = min(64u, C - c0);
+    float v[18];   // 8 * 64 * 9 / 256 loads per thread, all issued before the first is used (clamped, not branched)
 #pragma unroll
-        for (int t = 0; t < 9; t++) f[t] = src[t];
+    for (int u = 0; u < 18; u++) {
+        const unsigned i = threadIdx.x + 256 * u, kk = i / (64 * 9), r = i - kk * (64 * 9);
+        v[u] = w[((size_t)(k0 + min(kk, nk - 1)) * C + c0) * 9 + min(r, nc * 9 - 1)];
+    }
+#pragma unroll
+    for (int u = 0; u < 18; u++) {
+        const unsigned i = threadIdx.x + 256 * u, kk = i / (64 * 9), r = i - kk * (64 * 9);
+        stage[kk][r] = v[u];   // rows and channels past the end are never read back
+    }
+    __syncthreads();
+    for (unsigned i = threadIdx.x; i < 64 * 4 * 8; i += 256) {
+        const unsigned kk = i & 7, row = i >> 3, cc = row >> 2, iy = (row >> 1) & 1, ix = row & 1;
+        if (kk >= nk || cc >= nc) continue;
         // input pixel (iy, ix), output pixel (oy, ox): tap (1 - iy + oy, 1 - ix + ox)
-#pragma unroll
-        for (int iy = 0; iy < 2; iy++)
-#pragma unroll
-            for (int ix = 0; ix < 2; ix++) {
-                const int t0 = (1 - iy) * 3 + (1 - ix);
-                wd[((size_t)c * 4 + iy * 2 + ix) * K + k] = make_float4(f[t0], f[t0 + 1], f[t0 + 3], f[t0 + 4]);
-            }
+        const float *f = &stage[kk][cc * 9 + (1 - iy) * 3 + (1 - ix)];
+        wd[((size_t)(c0 + cc) * 4 + iy * 2 + ix) * K + k0 + kk] = make_float4(f[0], f[1], f[3], f[4]);
     }
 }
 
@@ -1326,10 +1332,8 @@ size_t dense2x2_elems(const dopt_hip_conv_desc *d) { return (size_t)16 * d->C * 
 
 int dense2x2_pack(const dopt_hip_conv_desc *d, const float *w, float *wd)
 {
-    const size_t blocks = ceil_div(dense2x2_elems(d) / 16, (size_t)256);
-    const size_t cap = (size_t)num_cus() * 16;
-    hipLaunchKernelGGL(pack_2x2_k, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0, stream(), (unsigned)d->C,
-                       (unsigned)d->K, w, (float4 *)wd);   // pool and plan buffers are 256-byte aligned
+    hipLaunchKernelGGL(pack_2x2_k, dim3((unsigned)ceil_div(d->K, (size_t)8), (unsigned)ceil_div(d->C, (size_t)64)), dim3(256), 0,
+                       stream(), (unsigned)d->C, (unsigned)d->K, w, (float4 *)wd);   // pool and plan buffers are 256-byte aligned
     DOPT_LAUNCH_CHECK();
     return DOPT_HIP_OK;
 }
