@@ -998,17 +998,40 @@ __global__ __launch_bounds__(768, 1) void conv_wgrad_patch_k(WgradPatch p)
 
 // out[i] = sum_s partial[s][i], s ascending; plus bias[channel of i] when a bias is given
 // (channel = (i / inner) % C for an [N, C, inner] output).
+// kS > 0: exactly kS splits, all loads issued before the first add.
+template <int kS>
 __global__ __launch_bounds__(256) void splitk_reduce_k(size_t n4, int splits, const float4 *partial, float4 *out,
                                                         const float *bias, unsigned C, unsigned inner)
 {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (size_t)gridDim.x * 256) {
-        float4 acc = partial[i];
-        for (int s = 1; s < splits; s++) {
-            const float4 v = partial[(size_t)s * n4 + i];
-            acc.x += v.x;
-            acc.y += v.y;
-            acc.z += v.z;
-            acc.w += v.w;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        if constexpr (kS > 0) {
+            float4 v[kS];
+#pragma unroll
+            for (int s = 0; s < kS; s++) v[s] = partial[(size_t)s * n4 + i];
+            acc = v[0];
+#pragma unroll
+            for (int s = 1; s < kS; s++) {
+                acc.x += v[s].x;
+                acc.y += v[s].y;
+                acc.z += v[s].z;
+                acc.w += v[s].w;
+            }
+        } else {
+            // Rounds of four loads in flight (indices clamped to the last split, surplus values
+            // replaced by zero); the adds stay in ascending split order.
+            const int last = splits - 1;
+            for (int s = 0; s < splits; s += 4) {
+                const float4 v0 = partial[(size_t)s * n4 + i];
+                const float4 v1 = partial[(size_t)min(s + 1, last) * n4 + i];
+                const float4 v2 = partial[(size_t)min(s + 2, last) * n4 + i];
+                const float4 v3 = partial[(size_t)min(s + 3, last) * n4 + i];
+                const bool h1 = s + 1 <= last, h2 = s + 2 <= last, h3 = s + 3 <= last;
+                acc.x = (((acc.x + v0.x) + (h1 ? v1.x : 0.f)) + (h2 ? v2.x : 0.f)) + (h3 ? v3.x : 0.f);
+                acc.y = (((acc.y + v0.y) + (h1 ? v1.y : 0.f)) + (h2 ? v2.y : 0.f)) + (h3 ? v3.y : 0.f);
+                acc.z = (((acc.z + v0.z) + (h1 ? v1.z : 0.f)) + (h2 ? v2.z : 0.f)) + (h3 ? v3.z : 0.f);
+                acc.w = (((acc.w + v0.w) + (h1 ? v1.w : 0.f)) + (h2 ? v2.w : 0.f)) + (h3 ? v3.w : 0.f);
+            }
         }
         if (bias) {
             const size_t e = i * 4;
@@ -1096,8 +1119,15 @@ int launch_splitk_reduce(size_t elems, int splits, const float *partial, float *
     const size_t n4 = elems / 4;
     size_t blocks = ceil_div(n4, (size_t)256);
     size_t cap = (size_t)num_cus() * 8;
-    hipLaunchKernelGGL(splitk_reduce_k, dim3((unsigned)(blocks > cap ? cap : (blocks < 1 ? 1 : blocks))), dim3(256), 0,
-                       stream(), n4, splits, (const float4 *)partial, (float4 *)out, bias, C, inner);
+    const dim3 grid((unsigned)(blocks > cap ? cap : (blocks < 1 ? 1 : blocks)));
+    const float4 *p4 = (const float4 *)partial;
+    float4 *o4 = (float4 *)out;
+    switch (splits) {
+    case 2: hipLaunchKernelGGL(splitk_reduce_k<2>, grid, dim3(256), 0, stream(), n4, splits, p4, o4, bias, C, inner); break;
+    case 3: hipLaunchKernelGGL(splitk_reduce_k<3>, grid, dim3(256), 0, stream(), n4, splits, p4, o4, bias, C, inner); break;
+    case 4: hipLaunchKernelGGL(splitk_reduce_k<4>, grid, dim3(256), 0, stream(), n4, splits, p4, o4, bias, C, inner); break;
+    default: hipLaunchKernelGGL(splitk_reduce_k<0>, grid, dim3(256), 0, stream(), n4, splits, p4, o4, bias, C, inner); break;
+    }
     DOPT_LAUNCH_CHECK();
     return DOPT_HIP_OK;
 }
@@ -1398,10 +1428,12 @@ __global__ __launch_bounds__(256) void fold_2x2_k(unsigned C, unsigned K, const 
 
 int run_dense2x2_wgrad(const dopt_hip_conv_desc *d, const float *dy, const float *x, float *dw)
 {
+    int rc = DOPT_HIP_OK;
+    if (sgemm_fold2x2(d->C, d->K, d->N, x, dy, dw, &rc)) return rc;   // product and fold in one kernel
     void *dwd = nullptr;
-    if (int rc = scratch_alloc(&dwd, dense2x2_elems(d) * sizeof(float))) return rc;
+    if ((rc = scratch_alloc(&dwd, dense2x2_elems(d) * sizeof(float)))) return rc;
     bool biased = false;
-    int rc = sgemm_bias(1, 0, 4 * d->C, 4 * d->K, d->N, x, dy, (float *)dwd, nullptr, 0, &biased);
+    rc = sgemm_bias(1, 0, 4 * d->C, 4 * d->K, d->N, x, dy, (float *)dwd, nullptr, 0, &biased);
     if (!rc) {
         const size_t blocks = ceil_div(d->C * d->K, (size_t)256);
         const size_t cap = (size_t)num_cus() * 16;

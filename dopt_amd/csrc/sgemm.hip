@@ -245,11 +245,127 @@ __global__ __launch_bounds__(64 * kSmallWaves) void sgemm_small_k(int M, int N, 
     }
 }
 
+// Short reductions over large outputs with both operands stored k-major (A as [K][M], B as [K][N]:
+// the product x^T * dy of a filter gradient).  With K <= 128 a 128 x 128 output tile needs 128 KB of
+// operands, which fit in LDS whole: every load of the block is issued before the first multiply, so
+// the memory latency is paid once per tile instead of once per slab, and each operand byte enters
+// the CU once per 128 x 128 outputs (a quarter of what 32 x 32 tiles fetch).  The reduction runs in
+// four chunks of 32; a chunk is multiplied as soon as it is in LDS while the later ones are still
+// in flight.  Eight wavefronts as 2 x 4, 64 x 32 outputs each.
+constexpr int kPanelK = 128, kPanelTile = 128, kPanelThreads = 512, kPanelLd = kPanelTile + 4;
+constexpr size_t kPanelLds = (size_t)2 * kPanelK * kPanelLd * sizeof(float);
+
+// Element (k, r .. r + 3) of an operand stored [K][R] (R % 4 == 0, 16-byte aligned), zero outside.
+__device__ __forceinline__ float4 panel_load(const float *X, int ld, int k, int K, int r, int R)
+{
+    return (k < K && r < R) ? *(const float4 *)(X + (size_t)k * ld + r) : make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
+// kFold: the product is the filter gradient of a 3x3, pad-1 convolution over 2x2 images written as a
+// dense product -- row 4c + (input pixel), column 4k + (output pixel) -- and the kernel stores the
+// nine tap sums of every (k, c) pair to C[k][c][3][3] instead of the 4 x 4 block itself: tap (a, b)
+// collects the pixel pairs with 1 - iy + oy == a and 1 - ix + ox == b.
+template <bool kFold>
+__global__ __launch_bounds__(kPanelThreads) void sgemm_panel_k(int M, int N, int K, int mtiles, int ntiles, const float *A,
+                                                                const float *B, float *C)
+{
+    extern __shared__ __attribute__((aligned(16))) float panel_lds[];
+    float *As = panel_lds, *Bs = panel_lds + kPanelK * kPanelLd;
+    unsigned L;
+    if (!xcd_remap(blockIdx.x, (unsigned)(mtiles * ntiles), &L)) return;
+    const int m0 = (int)(L % (unsigned)mtiles) * kPanelTile, n0 = (int)(L / (unsigned)mtiles) * kPanelTile;
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, wm = w >> 2, wn = w & 3;
+
+    // chunk c = reduction steps [32c, 32c + 32): 1024 float4 per operand, two per thread
+    float4 ra[4][2], rb[4][2];
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const int f = tid + kPanelThreads * i, k = 32 * c + (f >> 5), r = (f & 31) * 4;
+            ra[c][i] = panel_load(A, M, k, K, m0 + r, M);
+            rb[c][i] = panel_load(B, N, k, K, n0 + r, N);
+        }
+    v16f acc[2][1];
+    zero_acc(acc);
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        if (32 * c < K) {   // uniform
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                const int f = tid + kPanelThreads * i, o = (32 * c + (f >> 5)) * kPanelLd + (f & 31) * 4;
+                *(float4 *)&As[o] = ra[c][i];
+                *(float4 *)&Bs[o] = rb[c][i];
+            }
+            __syncthreads();
+            mma_slab<32, kPanelLd, kPanelLd>(As + 32 * c * kPanelLd, Bs + 32 * c * kPanelLd, wm * 64, wn * 32, acc, lane);
+        }
+    }
+    if constexpr (!kFold) {
+        const int col = n0 + wn * 32 + (lane & 31);
+        if (col < N) {
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int m = m0 + wm * 64 + i * 32 + acc_row(v, lane);
+                    if (m < M) C[(size_t)m * N + col] = acc[i][0][v];
+                }
+        }
+    } else {
+        // the tile goes back through LDS (the operands are spent) so that one thread sees the 4 x 4
+        // block of a (c, k) pair; threads run along c, which is contiguous in the filter gradient
+        __syncthreads();
+        float *tile = panel_lds;   // [128][kPanelLd]
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++)
+                tile[(wm * 64 + i * 32 + acc_row(v, lane)) * kPanelLd + wn * 32 + (lane & 31)] = acc[i][0][v];
+        __syncthreads();
+        const int Cin = M / 4, Kout = N / 4;
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int pair = tid + kPanelThreads * j, cl = pair & 31, kl = pair >> 5;
+            const int c = m0 / 4 + cl, k = n0 / 4 + kl;
+            if (c < Cin && k < Kout) {
+                float q[4][4];   // [input pixel iy*2+ix][output pixel oy*2+ox]
+#pragma unroll
+                for (int pin = 0; pin < 4; pin++) {
+                    const float4 v = *(const float4 *)&tile[(cl * 4 + pin) * kPanelLd + kl * 4];
+                    q[pin][0] = v.x; q[pin][1] = v.y; q[pin][2] = v.z; q[pin][3] = v.w;
+                }
+                float *out = C + ((size_t)k * Cin + c) * 9;
+#pragma unroll
+                for (int a = 0; a < 3; a++)
+#pragma unroll
+                    for (int b = 0; b < 3; b++) {
+                        float sum = 0.0f;
+#pragma unroll
+                        for (int iy = 0; iy < 2; iy++)
+#pragma unroll
+                            for (int ix = 0; ix < 2; ix++) {
+                                const int oy = a - 1 + iy, ox = b - 1 + ix;
+                                if (oy >= 0 && oy < 2 && ox >= 0 && ox < 2) sum += q[iy * 2 + ix][oy * 2 + ox];
+                            }
+                        out[a * 3 + b] = sum;
+                    }
+            }
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void splitk_reduce_k(size_t n, int splits, const float *partial, float *out)
 {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
-        float acc = partial[i];
-        for (int s = 1; s < splits; s++) acc += partial[(size_t)s * n + i];
+        // four loads in flight per round (indices clamped, surplus values dropped); adds in split order
+        float acc = 0.f;
+        const int last = splits - 1;
+        for (int s = 0; s < splits; s += 4) {
+            const float v0 = partial[(size_t)s * n + i], v1 = partial[(size_t)min(s + 1, last) * n + i];
+            const float v2 = partial[(size_t)min(s + 2, last) * n + i], v3 = partial[(size_t)min(s + 3, last) * n + i];
+            acc = (((acc + v0) + (s + 1 <= last ? v1 : 0.f)) + (s + 2 <= last ? v2 : 0.f)) + (s + 3 <= last ? v3 : 0.f);
+        }
         out[i] = acc;
     }
 }
@@ -298,6 +414,34 @@ unsigned flat_grid(size_t n)
     size_t blocks = ceil_div(n, (size_t)256);
     size_t cap = (size_t)num_cus() * 16;
     return (unsigned)(blocks < 1 ? 1 : (blocks > cap ? cap : blocks));
+}
+
+// The LDS-resident kernel wins where its 128 x 128 tiles give every CU one or two blocks and the
+// operands take 128-bit loads (2048 x 2048 x 128: 17 us against 22 us for the 32 x 32 tiles); with
+// fewer tiles CUs idle, with more the tile engine's two resident blocks per CU overlap better.
+bool panel_takes(size_t M, size_t N, size_t K, const float *A, const float *B)
+{
+    const size_t tiles = ceil_div(M, (size_t)kPanelTile) * ceil_div(N, (size_t)kPanelTile);
+    return K >= 1 && K <= (size_t)kPanelK && tiles >= (size_t)num_cus() && tiles <= (size_t)2 * num_cus() &&
+           aligned16(A) && aligned16(B) && M % 4 == 0 && N % 4 == 0;
+}
+
+int panel_launch(bool fold, size_t M, size_t N, size_t K, const float *A, const float *B, float *C)
+{
+    static bool raised = false;
+    if (!raised) {   // above 64 KB of dynamic LDS a kernel has to be told once
+        DOPT_HIP_CHECK(hipFuncSetAttribute((const void *)sgemm_panel_k<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)kPanelLds));
+        DOPT_HIP_CHECK(hipFuncSetAttribute((const void *)sgemm_panel_k<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)kPanelLds));
+        raised = true;
+    }
+    const int mt = (int)ceil_div(M, (size_t)kPanelTile), nt = (int)ceil_div(N, (size_t)kPanelTile);
+    const dim3 grid(xcd_grid((unsigned)(mt * nt))), block(kPanelThreads);
+    if (fold) hipLaunchKernelGGL(sgemm_panel_k<true>, grid, block, kPanelLds, stream(), (int)M, (int)N, (int)K, mt, nt, A, B, C);
+    else hipLaunchKernelGGL(sgemm_panel_k<false>, grid, block, kPanelLds, stream(), (int)M, (int)N, (int)K, mt, nt, A, B, C);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
 }
 
 }  // namespace
@@ -361,6 +505,9 @@ int sgemm_bias(int transA, int transB, size_t M, size_t N, size_t K, const float
         }
         return DOPT_HIP_OK;
     }
+
+    // short reduction, both operands k-major, enough 128 x 128 tiles to fill the machine
+    if (transA && !transB && !colbias && panel_takes(M, N, K, A, B)) return panel_launch(false, M, N, K, A, B, C);
 
     // small and medium outputs: one block per 32 x 32 tile, the reduction split over its wavefronts.
     // Each tile reads its own 32 rows of A and 32 columns of B, so the operand traffic grows with the
@@ -447,6 +594,16 @@ int sgemm_bias(int transA, int transB, size_t M, size_t N, size_t K, const float
         DOPT_LAUNCH_CHECK();
     }
     return DOPT_HIP_OK;
+}
+
+// Filter gradient of a 3x3, pad-1, unit-stride convolution over 2x2 images in one launch:
+// dw[K][C][3][3] from x[N][4C] and dy[N][4K].  Returns false (nothing launched) when the shape does
+// not suit the LDS-resident kernel; the caller then takes the product and folds it itself.
+bool sgemm_fold2x2(size_t C, size_t K, size_t N, const float *x, const float *dy, float *dw, int *rc)
+{
+    if (!panel_takes(4 * C, 4 * K, N, x, dy)) return false;
+    *rc = panel_launch(true, 4 * C, 4 * K, N, x, dy, dw);
+    return true;
 }
 
 }  // namespace dopt

@@ -313,6 +313,10 @@ CONV_CASES = [  # N, C, H, W, K, R, S, pad, stride
     (32, 48, 2, 2, 130, 3, 3, (1, 1), (1, 1)),    # 2x2 images, sixteen per chunk
     (16, 70, 2, 2, 32, 3, 3, (1, 1), (1, 1)),
     (6, 32, 4, 4, 128, 3, 3, (1, 1), (1, 1)),     # batch not a multiple of the chunk: generic kernel
+    # 2x2 images at sizes whose filter gradient is one launch (dense product with the fold in its
+    # epilogue): the VGG shape, and one with a shorter batch and ragged edge tiles
+    (128, 512, 2, 2, 512, 3, 3, (1, 1), (1, 1)),
+    (100, 500, 2, 2, 520, 3, 3, (1, 1), (1, 1)),
     # at most three input channels, pad 1: the first-layer kernels (rows of 8 .. 128 pixels, one to
     # sixteen rows per sub-tile, output channels off the 32-row fragment, a single-channel image)
     (3, 3, 32, 32, 40, 3, 3, (1, 1), (1, 1)),
@@ -529,6 +533,19 @@ def test_batched_device_copies():
     b = (C.c_size_t * 2)(32, 32)
     capi.check(lib.dopt_hip_copy_d2d_batch(2, d, s, b))
     assert np.array_equal(c.numpy(), np.arange(8, dtype=np.float32))
+
+
+@pytest.mark.parametrize("shape", [(2048, 2048, 128), (2048, 2048, 100), (2048, 2052, 17), (2044, 2080, 64)])
+def test_sgemm_short_reduction_large_output(shape):
+    # A stored [K][M], B stored [K][N], K <= 128 and about one 128 x 128 tile per CU: the kernel that
+    # keeps both operand panels in LDS (full and ragged edge tiles, reductions that end inside a chunk)
+    M, N, K = shape
+    r = rng(M + 3 * N + 7 * K)
+    a = r.standard_normal((M, K)).astype(np.float32)
+    b = r.standard_normal((K, N)).astype(np.float32)
+    got = ops.matmul_t(T(np.ascontiguousarray(a.T)), T(b), True, False)
+    assert got.shape == (M, N)
+    assert_close(got.numpy(), O.matmul(a, b, f64=True), "sgemm_t panel", scale=np.sqrt(K))
 
 
 @pytest.mark.parametrize("shape", [(128, 512, 512), (70, 33, 129), (130, 10, 512), (1, 300, 77), (200, 1, 64), (5, 7, 1),
