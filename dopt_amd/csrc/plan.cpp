@@ -582,7 +582,9 @@ struct HIPPlan::Builder {
     std::vector<int> biasGradOf;                // batchNormGrad op -> the addBiasGrad op it serves
     std::vector<char> absorbed;
     std::vector<char> needed;
-    struct Prepack { int op, filter; int bwd; dopt_hip_conv_desc d; void *buf; bool owner; };
+    // late: the copy is made right in front of its first reader instead of at the start of the run
+    struct Prepack { int op, filter; int bwd; dopt_hip_conv_desc d; void *buf; bool owner, late; };
+    void pushPackStep(const std::vector<Prepack> &which);
     std::vector<Prepack> packs;
     std::vector<int> packOf;
 
@@ -1001,6 +1003,7 @@ int HIPPlan::Builder::prepackFilters()
                     dopt_hip_conv_packed_layout(&other.d, other.bwd) == layout)
                     k.buf = other.buf;
             k.owner = k.buf == nullptr;
+            k.late = layout == 2;
             if (k.owner) {
                 if (int rc = dopt_hip_malloc(&k.buf, bytes)) return rc;
                 p->mOwned.push_back(k.buf);
@@ -1010,30 +1013,38 @@ int HIPPlan::Builder::prepackFilters()
             packs.push_back(k);
         }
     }
-    if (!packs.empty()) {
-        std::vector<dopt_hip_conv_desc> descs;
-        std::vector<int> bwd;
-        std::vector<float *> bufs;
-        Step s;
-        s.op = -1;
-        s.label = "filterPack";
-        for (const Prepack &k : packs) {
-            if (!k.owner) continue;
-            descs.push_back(k.d);
-            bwd.push_back(k.bwd);
-            bufs.push_back((float *)k.buf);
-            s.inputOps.push_back(k.filter);
-        }
-        s.kernel = make([=](const std::vector<const void *> &in, void *) {
-            return dopt_hip_conv_pack_batch((int)descs.size(), descs.data(), bwd.data(), (const float *const *)in.data(),
-                                            bufs.data());
-        });
-        s.inputs.resize(s.inputOps.size());
-        s.inputBytes.resize(s.inputOps.size());
-        for (size_t i = 0; i < s.inputOps.size(); i++) s.inputBytes[i] = g.ops[s.inputOps[i]].bytes();
-        p->mSteps.push_back(std::move(s));
-    }
+    // The 3x3 layouts are small and many: one launch at the start of the run makes them all.  The
+    // dense matrices of 2x2-image layers are 16 MB each and made by a launch of their own, so each is
+    // made just before the convolution that reads it first and is still in the caches when it does.
+    std::vector<Prepack> early;
+    for (const Prepack &k : packs)
+        if (k.owner && !k.late) early.push_back(k);
+    if (!early.empty()) pushPackStep(early);
     return DOPT_HIP_OK;
+}
+
+void HIPPlan::Builder::pushPackStep(const std::vector<Prepack> &which)
+{
+    std::vector<dopt_hip_conv_desc> descs;
+    std::vector<int> bwd;
+    std::vector<float *> bufs;
+    Step s;
+    s.op = -1;
+    s.label = "filterPack";
+    for (const Prepack &k : which) {
+        descs.push_back(k.d);
+        bwd.push_back(k.bwd);
+        bufs.push_back((float *)k.buf);
+        s.inputOps.push_back(k.filter);
+    }
+    s.kernel = make([=](const std::vector<const void *> &in, void *) {
+        return dopt_hip_conv_pack_batch((int)descs.size(), descs.data(), bwd.data(), (const float *const *)in.data(),
+                                        bufs.data());
+    });
+    s.inputs.resize(s.inputOps.size());
+    s.inputBytes.resize(s.inputOps.size());
+    for (size_t i = 0; i < s.inputOps.size(); i++) s.inputBytes[i] = g.ops[s.inputOps[i]].bytes();
+    p->mSteps.push_back(std::move(s));
 }
 
 int HIPPlan::Builder::allocateBuffers()
@@ -1070,6 +1081,7 @@ int HIPPlan::Builder::buildSteps()
         std::vector<int> stepInputs = inputsOf[id];
         if (packOf[id] >= 0) {  // the filter operand is read from its packed copy
             const Prepack pk = packs[(size_t)packOf[id]];
+            if (pk.owner && pk.late) pushPackStep({pk});
             const float *packed = (const float *)pk.buf;
             const dopt_hip_conv_desc d = pk.d;
             if (pk.bwd) {
