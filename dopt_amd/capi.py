@@ -25,6 +25,12 @@ class ConvDesc(C.Structure):
                 ("N", "C", "H", "W", "K", "R", "S", "padH", "padW", "strideH", "strideW")]
 
 
+class SplitSum(C.Structure):
+    """dopt_hip_split_sum: a convolution result left as partial copies for its reader to add."""
+    _fields_ = [("partial", C.c_void_p), ("splits", C.c_int), ("elems", C.c_size_t), ("C", C.c_size_t),
+                ("inner", C.c_size_t), ("bias", C.c_void_p), ("value", C.c_void_p)]
+
+
 class TensorRef(C.Structure):
     _fields_ = [("w", C.c_void_p), ("g", C.c_void_p), ("m", C.c_void_p), ("v", C.c_void_p),
                 ("vhat", C.c_void_p), ("n", C.c_size_t), ("skip_w", C.c_int)]
@@ -76,6 +82,9 @@ PROTOTYPES = {
     "dopt_hip_conv_pack_batch": [_i, C.POINTER(ConvDesc), C.POINTER(_i), C.POINTER(_vp), C.POINTER(_vp)],
     "dopt_hip_conv_fwd_bias_packed": [C.POINTER(ConvDesc), _vp, _vp, _vp, _vp],
     "dopt_hip_conv_bwd_data_packed": [C.POINTER(ConvDesc), _vp, _vp, _vp],
+    "dopt_hip_conv_fwd_bias_packed_open": [C.POINTER(ConvDesc), _vp, _vp, _vp, _vp, C.POINTER(SplitSum)],
+    "dopt_hip_conv_bwd_data_packed_open": [C.POINTER(ConvDesc), _vp, _vp, _vp, C.POINTER(SplitSum)],
+    "dopt_hip_split_sum_close": [C.POINTER(SplitSum)],
     "dopt_hip_conv_bwd_filter": [C.POINTER(ConvDesc), _vp, _vp, _vp],
     "dopt_hip_maxpool_fwd": [_sz, _sz, _sz, _sz, _sz, _sz, _vp, _vp],
     "dopt_hip_maxpool_bwd": [_sz, _sz, _sz, _sz, _sz, _sz, _vp, _vp, _vp],
@@ -93,6 +102,8 @@ PROTOTYPES = {
     "dopt_hip_bn_grad": [_sz, _sz, _sz, _vp, _vp, _vp, _vp],
     "dopt_hip_bn_grad_relu": [_sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_bn_grad_fused": [_sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp],
+    "dopt_hip_bn_train_open": [_sz, _sz, _sz, _d, C.POINTER(SplitSum), _vp, _vp, _vp, _vp, _vp, _i],
+    "dopt_hip_bn_grad_open": [_sz, _sz, _sz, C.POINTER(SplitSum), _i, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_bn_infer": [_sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_optim_create": [_i, C.POINTER(TensorRef), C.POINTER(_vp)],
     "dopt_hip_optim_destroy": [_vp],

@@ -309,6 +309,7 @@ __global__ __launch_bounds__(kBlock) void bn_grad_apply_k(IdxT total, IdxT C, Id
 // the op is one launch instead of three.  Statistics are exact two-pass (mean, then centred
 // squares).
 constexpr int kResQuads = 8;  // float4 per thread
+constexpr int kOpenQuads = 2; // the same where an operand arrives as partial copies
 
 // Sums kN per-thread values over the block (up to 16 wavefronts); every thread gets the totals.
 // Lanes are folded in fp32 with butterfly shuffles (a pairwise tree: error ~ log2(64) ulp), the
@@ -345,31 +346,100 @@ __device__ inline void block_allsum(const float (&v)[kN], double (&total)[kN], f
     }
 }
 
-template <bool kGrad>
+// An operand that a convolution left as `splits` partial copies (x of the forward kernel, dy of the
+// gradient kernel): the kernel adds the copies in order, plus the convolution's bias, exactly as the
+// convolution's own finishing pass would, and writes the finished value to `value` when that is
+// not null (the forward input is read again by the backward pass).
+struct OpenSum {
+    const float4 *partial;
+    int splits;
+    unsigned stride4;   // float4 per copy
+    const float *bias;  // per channel, or null
+    float4 *value;      // or null
+};
+
+// sum[i] = copy 0 + copy 1 + ... at float4 index at[i], in that order.  kS > 0: exactly kS copies,
+// unrolled; kS == 0: any number, copy by copy with the quads of one copy in flight together.
+template <int kS, int kQ>
+__device__ __forceinline__ void open_add(const OpenSum &open, const unsigned (&at)[kQ], float4 (&sum)[kQ])
+{
+    if constexpr (kS > 0) {
+        float4 v[kS][kQ];
+#pragma unroll
+        for (int sp = 0; sp < kS; sp++)
+#pragma unroll
+            for (int i = 0; i < kQ; i++) v[sp][i] = open.partial[(size_t)sp * open.stride4 + at[i]];
+#pragma unroll
+        for (int i = 0; i < kQ; i++) {
+            sum[i] = v[0][i];
+#pragma unroll
+            for (int sp = 1; sp < kS; sp++)
+                sum[i] = make_float4(sum[i].x + v[sp][i].x, sum[i].y + v[sp][i].y, sum[i].z + v[sp][i].z, sum[i].w + v[sp][i].w);
+        }
+    } else {
+        for (int sp = 0; sp < open.splits; sp++) {
+            const float4 *src = open.partial + (size_t)sp * open.stride4;
+            float4 v[kQ];
+#pragma unroll
+            for (int i = 0; i < kQ; i++) v[i] = src[at[i]];
+#pragma unroll
+            for (int i = 0; i < kQ; i++) {
+                if (sp == 0) sum[i] = v[i];
+                else sum[i] = make_float4(sum[i].x + v[i].x, sum[i].y + v[i].y, sum[i].z + v[i].z, sum[i].w + v[i].w);
+            }
+        }
+    }
+}
+
+// kQ: float4 per thread (a thread of the open variant holds kQ quads of every copy at once, so it is
+// built for small channels only).
+template <bool kGrad, bool kOpen, int kQ>
 __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, unsigned inner4, double factor, double eps,
                                                        const float *x, const float *dy, const float *scale,
                                                        const float *bias, const float *run_mean, const float *run_var,
                                                        const float *ymask, int relu, float *out, float *out1, float *out2,
-                                                       float *dx_sum)
+                                                       float *dx_sum, OpenSum open)
 {
     __shared__ float part[3][16];
     const unsigned c = blockIdx.x, T = blockDim.x, E4 = N * inner4;
     const float4 *x4 = (const float4 *)x, *g4 = (const float4 *)dy;
-    float4 xv[kResQuads], gv[kResQuads];
-    unsigned idx[kResQuads];
+    float4 xv[kQ], gv[kQ];
+    unsigned idx[kQ];
 #pragma unroll
-    for (int i = 0; i < kResQuads; i++) {
+    for (int i = 0; i < kQ; i++) {
         const unsigned q = i * T + threadIdx.x;
         const unsigned n = q / inner4, r = q - n * inner4;
         idx[i] = q < E4 ? (n * C + c) * inner4 + r : 0xffffffffu;
         xv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         gv[i] = xv[i];
         if (q < E4) {
-            xv[i] = x4[idx[i]];
-            if (kGrad) {
+            if (!(kOpen && !kGrad)) xv[i] = x4[idx[i]];
+            if (kGrad && !kOpen) {
                 gv[i] = g4[idx[i]];
                 if (ymask) gv[i] = masked4(gv[i], ((const float4 *)ymask)[idx[i]]);
             }
+        }
+    }
+    if (kOpen) {
+        float4 sum[kQ];
+        unsigned at[kQ];
+#pragma unroll
+        for (int i = 0; i < kQ; i++) at[i] = idx[i] == 0xffffffffu ? 0u : idx[i];   // clamped, not branched
+        // two to four copies: every load of the thread is issued before the first add
+        if (open.splits == 2) open_add<2, kQ>(open, at, sum);
+        else if (open.splits == 3) open_add<3, kQ>(open, at, sum);
+        else if (open.splits == 4) open_add<4, kQ>(open, at, sum);
+        else open_add<0, kQ>(open, at, sum);
+        const bool biased = open.bias != nullptr;
+        const float bc = biased ? open.bias[c] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < kQ; i++) {
+            if (idx[i] == 0xffffffffu) continue;
+            float4 r = sum[i];
+            if (biased) r = make_float4(r.x + bc, r.y + bc, r.z + bc, r.w + bc);
+            if (open.value) open.value[idx[i]] = r;
+            if (kGrad) gv[i] = ymask ? masked4(r, ((const float4 *)ymask)[idx[i]]) : r;
+            else xv[i] = r;
         }
     }
     const double m = 4.0 * (double)E4;
@@ -377,7 +447,7 @@ __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, un
     {
         float s = 0.f;
 #pragma unroll
-        for (int i = 0; i < kResQuads; i++) s += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);  // absent quads are zero
+        for (int i = 0; i < kQ; i++) s += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);  // absent quads are zero
         const float in1[1] = {s};
         block_allsum<1>(in1, red1, part);
     }
@@ -387,7 +457,7 @@ __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, un
     {
         float ss = 0.f, g1 = 0.f, g2 = 0.f;
 #pragma unroll
-        for (int i = 0; i < kResQuads; i++) {
+        for (int i = 0; i < kQ; i++) {
             if (idx[i] == 0xffffffffu) continue;
             const float d0 = (xv[i].x - mean_hi) - mean_lo, d1 = (xv[i].y - mean_hi) - mean_lo;
             const float d2 = (xv[i].z - mean_hi) - mean_lo, d3 = (xv[i].w - mean_hi) - mean_lo;
@@ -406,7 +476,7 @@ __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, un
     if (!kGrad) {
         const float a = (float)((double)scale[c] * rstd), b = bias[c];
 #pragma unroll
-        for (int i = 0; i < kResQuads; i++) {
+        for (int i = 0; i < kQ; i++) {
             if (idx[i] == 0xffffffffu) continue;
             float4 r;
             r.x = a * ((xv[i].x - mean_hi) - mean_lo) + b;
@@ -432,7 +502,7 @@ __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, un
         k.d = (float)(ds / m);
         float sdx = 0.f;
 #pragma unroll
-        for (int i = 0; i < kResQuads; i++) {
+        for (int i = 0; i < kQ; i++) {
             if (idx[i] == 0xffffffffu) continue;
             const float4 r = make_float4(bn_dx(k, gv[i].x, xv[i].x), bn_dx(k, gv[i].y, xv[i].y),
                                          bn_dx(k, gv[i].z, xv[i].z), bn_dx(k, gv[i].w, xv[i].w));
@@ -521,9 +591,24 @@ int launch_apply(size_t total, size_t C, size_t inner, const float *x, const Coe
     return DOPT_HIP_OK;
 }
 
+// The kernel-side description of an open operand, or false when `o` does not describe `elems` values
+// in [N, C, inner] that the resident kernel can read (the caller then closes it first).
+bool open_sum(const dopt_hip_split_sum *o, size_t elems, size_t C, size_t inner, bool keep, OpenSum *k)
+{
+    if (!o || o->splits < 2 || o->elems != elems || o->C != C || o->inner != inner || !o->partial || !o->value ||
+        !aligned16(o->partial) || !aligned16(o->value) || elems % 4 != 0)
+        return false;
+    k->partial = (const float4 *)o->partial;
+    k->splits = o->splits;
+    k->stride4 = (unsigned)(elems / 4);
+    k->bias = o->bias;
+    k->value = keep ? (float4 *)o->value : nullptr;
+    return true;
+}
+
 int bn_train_impl(size_t N, size_t C, size_t inner, double momentum, const float *x, const float *scale,
                   const float *bias, const float *run_mean, const float *run_var, float *packed, int relu,
-                  const char *who)
+                  const char *who, const dopt_hip_split_sum *x_open = nullptr)
 {
     size_t total = N * C * inner;
     DOPT_REQUIRE(total > 0, "%s: empty input", who);
@@ -532,10 +617,30 @@ int bn_train_impl(size_t N, size_t C, size_t inner, double momentum, const float
     DOPT_ENSURE_INIT();
     double factor = 1.0 - momentum;    // cudnn7.d:592
     double eps = (double)1e-5f;        // cudnn7.d:610
-    if (unsigned T = resident_threads(N, C, inner, x, nullptr, packed)) {
-        hipLaunchKernelGGL(bn_resident_k<false>, dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N, (unsigned)C,
-                           (unsigned)(inner / 4), factor, eps, x, (const float *)nullptr, scale, bias, run_mean, run_var,
-                           (const float *)nullptr, relu, packed, packed + total, packed + total + C, (float *)nullptr);
+    const unsigned T = resident_threads(N, C, inner, x, nullptr, packed);
+    if (x_open && x_open->splits) {   // x is still in pieces
+        OpenSum os;
+        if (T && N * (inner / 4) <= (size_t)kOpenQuads * T && open_sum(x_open, total, C, inner, true, &os)) {
+            hipLaunchKernelGGL((bn_resident_k<false, true, kOpenQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N, (unsigned)C,
+                               (unsigned)(inner / 4), factor, eps, x, (const float *)nullptr, scale, bias, run_mean, run_var,
+                               (const float *)nullptr, relu, packed, packed + total, packed + total + C, (float *)nullptr, os);
+            DOPT_LAUNCH_CHECK();
+            return DOPT_HIP_OK;
+        }
+        if (int rc = dopt_hip_split_sum_close(x_open)) return rc;
+    }
+    if (T) {
+        // small channels (two quads per thread) take the variant built for two: a third of the registers
+        if (N * (inner / 4) <= (size_t)kOpenQuads * T)
+            hipLaunchKernelGGL((bn_resident_k<false, false, kOpenQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N,
+                               (unsigned)C, (unsigned)(inner / 4), factor, eps, x, (const float *)nullptr, scale, bias, run_mean,
+                               run_var, (const float *)nullptr, relu, packed, packed + total, packed + total + C,
+                               (float *)nullptr, OpenSum{});
+        else
+            hipLaunchKernelGGL((bn_resident_k<false, false, kResQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N,
+                               (unsigned)C, (unsigned)(inner / 4), factor, eps, x, (const float *)nullptr, scale, bias, run_mean,
+                               run_var, (const float *)nullptr, relu, packed, packed + total, packed + total + C,
+                               (float *)nullptr, OpenSum{});
         DOPT_LAUNCH_CHECK();
         return DOPT_HIP_OK;
     }
@@ -555,7 +660,8 @@ int bn_train_impl(size_t N, size_t C, size_t inner, double momentum, const float
 }
 
 int bn_grad_impl(size_t N, size_t C, size_t inner, const float *dy, const float *ymask, const float *x,
-                 const float *scale, float *packed, float *dx_sum, const char *who)
+                 const float *scale, float *packed, float *dx_sum, const char *who,
+                 const dopt_hip_split_sum *dy_open = nullptr, bool keep_dy = true)
 {
     size_t total = N * C * inner;
     DOPT_REQUIRE(total > 0, "%s: empty input", who);
@@ -563,15 +669,32 @@ int bn_grad_impl(size_t N, size_t C, size_t inner, const float *dy, const float 
     DOPT_REQUIRE(C <= 0x7fffffffu / kMaxSlices, "%s: too many channels", who);
     DOPT_ENSURE_INIT();
     double eps = (double)1e-5f;  // cudnn7.d:634
-    if (unsigned T = resident_threads(N, C, inner, x, dy, packed)) {
-        if (!ymask || aligned16(ymask)) {
-            hipLaunchKernelGGL(bn_resident_k<true>, dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N, (unsigned)C,
+    const unsigned T = (!ymask || aligned16(ymask)) ? resident_threads(N, C, inner, x, dy, packed) : 0;
+    if (dy_open && dy_open->splits) {   // dy is still in pieces
+        OpenSum os;
+        if (T && N * (inner / 4) <= (size_t)kOpenQuads * T && open_sum(dy_open, total, C, inner, keep_dy, &os)) {
+            hipLaunchKernelGGL((bn_resident_k<true, true, kOpenQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N, (unsigned)C,
                                (unsigned)(inner / 4), 0.0, eps, x, dy, scale, (const float *)nullptr,
                                (const float *)nullptr, (const float *)nullptr, ymask, 0, packed, packed + total,
-                               packed + total + C, dx_sum);
+                               packed + total + C, dx_sum, os);
             DOPT_LAUNCH_CHECK();
             return DOPT_HIP_OK;
         }
+        if (int rc = dopt_hip_split_sum_close(dy_open)) return rc;
+    }
+    if (T) {
+        if (N * (inner / 4) <= (size_t)kOpenQuads * T)
+            hipLaunchKernelGGL((bn_resident_k<true, false, kOpenQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N,
+                               (unsigned)C, (unsigned)(inner / 4), 0.0, eps, x, dy, scale, (const float *)nullptr,
+                               (const float *)nullptr, (const float *)nullptr, ymask, 0, packed, packed + total,
+                               packed + total + C, dx_sum, OpenSum{});
+        else
+            hipLaunchKernelGGL((bn_resident_k<true, false, kResQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N,
+                               (unsigned)C, (unsigned)(inner / 4), 0.0, eps, x, dy, scale, (const float *)nullptr,
+                               (const float *)nullptr, (const float *)nullptr, ymask, 0, packed, packed + total,
+                               packed + total + C, dx_sum, OpenSum{});
+        DOPT_LAUNCH_CHECK();
+        return DOPT_HIP_OK;
     }
     size_t part_bytes = C * kMaxSlices * 4 * sizeof(float);
     char *ws = (char *)workspace(part_bytes + C * sizeof(CoefG));
@@ -633,6 +756,23 @@ int dopt_hip_bn_grad_relu(size_t N, size_t C, size_t inner, const float *dy, con
 {
     DOPT_REQUIRE(y != nullptr, "dopt_hip_bn_grad_relu: null argument");
     return bn_grad_impl(N, C, inner, dy, y, x, scale, packed, nullptr, "dopt_hip_bn_grad_relu");
+}
+
+int dopt_hip_bn_train_open(size_t N, size_t C, size_t inner, double momentum, const dopt_hip_split_sum *x_open,
+                           const float *scale, const float *bias, const float *run_mean, const float *run_var,
+                           float *packed, int relu)
+{
+    DOPT_REQUIRE(x_open && x_open->value, "dopt_hip_bn_train_open: null argument");
+    return bn_train_impl(N, C, inner, momentum, x_open->value, scale, bias, run_mean, run_var, packed, relu != 0,
+                         "dopt_hip_bn_train_open", x_open);
+}
+
+int dopt_hip_bn_grad_open(size_t N, size_t C, size_t inner, const dopt_hip_split_sum *dy_open, int keep_dy,
+                          const float *y, const float *x, const float *scale, float *packed, float *dx_sum)
+{
+    DOPT_REQUIRE(dy_open && dy_open->value, "dopt_hip_bn_grad_open: null argument");
+    return bn_grad_impl(N, C, inner, dy_open->value, y, x, scale, packed, dx_sum, "dopt_hip_bn_grad_open", dy_open,
+                        keep_dy != 0);
 }
 
 int dopt_hip_bn_grad_fused(size_t N, size_t C, size_t inner, const float *dy, const float *y, const float *x,

@@ -1019,7 +1019,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_k(size_t n4, int splits, co
             }
         } else {
             // Rounds of four loads in flight (indices clamped to the last split, surplus values
-            // replaced by zero); the adds stay in ascending split order.
+            // dropped); the adds stay in ascending split order.
             const int last = splits - 1;
             for (int s = 0; s < splits; s += 4) {
                 const float4 v0 = partial[(size_t)s * n4 + i];
@@ -1027,10 +1027,11 @@ __global__ __launch_bounds__(256) void splitk_reduce_k(size_t n4, int splits, co
                 const float4 v2 = partial[(size_t)min(s + 2, last) * n4 + i];
                 const float4 v3 = partial[(size_t)min(s + 3, last) * n4 + i];
                 const bool h1 = s + 1 <= last, h2 = s + 2 <= last, h3 = s + 3 <= last;
-                acc.x = (((acc.x + v0.x) + (h1 ? v1.x : 0.f)) + (h2 ? v2.x : 0.f)) + (h3 ? v3.x : 0.f);
-                acc.y = (((acc.y + v0.y) + (h1 ? v1.y : 0.f)) + (h2 ? v2.y : 0.f)) + (h3 ? v3.y : 0.f);
-                acc.z = (((acc.z + v0.z) + (h1 ? v1.z : 0.f)) + (h2 ? v2.z : 0.f)) + (h3 ? v3.z : 0.f);
-                acc.w = (((acc.w + v0.w) + (h1 ? v1.w : 0.f)) + (h2 ? v2.w : 0.f)) + (h3 ? v3.w : 0.f);
+                if (s == 0) acc = v0;   // not 0 + v0: the sum of negative zeros stays a negative zero
+                else acc = make_float4(acc.x + v0.x, acc.y + v0.y, acc.z + v0.z, acc.w + v0.w);
+                if (h1) acc = make_float4(acc.x + v1.x, acc.y + v1.y, acc.z + v1.z, acc.w + v1.w);
+                if (h2) acc = make_float4(acc.x + v2.x, acc.y + v2.y, acc.z + v2.z, acc.w + v2.w);
+                if (h3) acc = make_float4(acc.x + v3.x, acc.y + v3.y, acc.z + v3.z, acc.w + v3.w);
             }
         }
         if (bias) {
@@ -1268,7 +1269,7 @@ int patch_splits(int tiles, int chunks, int slots, int BM, int BN, size_t out_el
 // pack it here first.
 template <bool kBwd>
 int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, const float *w, const float *bias,
-              float *out, bool *done, const float *prepacked = nullptr)
+              float *out, bool *done, const float *prepacked = nullptr, dopt_hip_split_sum *open = nullptr)
 {
     *done = false;
     PatchSetup u = patch_setup<kBwd>(d, P, Q);
@@ -1310,6 +1311,16 @@ int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, 
     else rc = launch_patch<GatherDeep, 16>(pc, c_full, grid, u.lds_bytes);
     if (rc) return rc;
     *done = true;
+    if (splits > 1 && open) {   // the caller's next call adds the copies
+        open->partial = partial;
+        open->splits = splits;
+        open->elems = pc.out_elems;
+        open->C = (size_t)pc.Mout;
+        open->inner = (size_t)pc.OH * pc.OW;
+        open->bias = bias;
+        open->value = out;
+        return DOPT_HIP_OK;
+    }
     if (splits > 1)
         return launch_splitk_reduce(pc.out_elems, splits, partial, out, bias, (unsigned)pc.Mout, (unsigned)(pc.OH * pc.OW));
     return DOPT_HIP_OK;
@@ -1858,31 +1869,62 @@ int dopt_hip_conv_pack_batch(int n, const dopt_hip_conv_desc *descs, const int *
     return flush();
 }
 
-int dopt_hip_conv_fwd_bias_packed(const dopt_hip_conv_desc *d, const float *x, const float *packed, const float *bias,
-                                  float *y)
+int dopt_hip_conv_fwd_bias_packed_open(const dopt_hip_conv_desc *d, const float *x, const float *packed,
+                                       const float *bias, float *y, dopt_hip_split_sum *open)
 {
     size_t P, Q;
+    if (open) {   // complete unless the patch kernel splits below
+        *open = dopt_hip_split_sum{};
+        open->value = y;
+    }
     if (int rc = check_desc(d, &P, &Q, "dopt_hip_conv_fwd_bias_packed")) return rc;
     DOPT_REQUIRE(x && packed && y, "dopt_hip_conv_fwd_bias_packed: null argument");
     DOPT_ENSURE_INIT();
     if (dopt_hip_conv_packed_layout(d, 0) == 2) return run_dense2x2<false>(d, x, nullptr, packed, bias, y);
     bool done = false;
-    if (int rc = run_patch<false>(d, P, Q, x, nullptr, bias, y, &done, packed)) return rc;
+    if (int rc = run_patch<false>(d, P, Q, x, nullptr, bias, y, &done, packed, open)) return rc;
     DOPT_REQUIRE(done, "dopt_hip_conv_fwd_bias_packed: this convolution does not take a packed filter");
     return DOPT_HIP_OK;
 }
 
-int dopt_hip_conv_bwd_data_packed(const dopt_hip_conv_desc *d, const float *dy, const float *packed, float *dx)
+int dopt_hip_conv_fwd_bias_packed(const dopt_hip_conv_desc *d, const float *x, const float *packed, const float *bias,
+                                  float *y)
+{
+    return dopt_hip_conv_fwd_bias_packed_open(d, x, packed, bias, y, nullptr);
+}
+
+int dopt_hip_conv_bwd_data_packed_open(const dopt_hip_conv_desc *d, const float *dy, const float *packed, float *dx,
+                                       dopt_hip_split_sum *open)
 {
     size_t P, Q;
+    if (open) {
+        *open = dopt_hip_split_sum{};
+        open->value = dx;
+    }
     if (int rc = check_desc(d, &P, &Q, "dopt_hip_conv_bwd_data_packed")) return rc;
     DOPT_REQUIRE(dy && packed && dx, "dopt_hip_conv_bwd_data_packed: null argument");
     DOPT_ENSURE_INIT();
     if (dopt_hip_conv_packed_layout(d, 1) == 2) return run_dense2x2<true>(d, dy, nullptr, packed, nullptr, dx);
     bool done = false;
-    if (int rc = run_patch<true>(d, P, Q, dy, nullptr, nullptr, dx, &done, packed)) return rc;
+    if (int rc = run_patch<true>(d, P, Q, dy, nullptr, nullptr, dx, &done, packed, open)) return rc;
     DOPT_REQUIRE(done, "dopt_hip_conv_bwd_data_packed: this convolution does not take a packed filter");
     return DOPT_HIP_OK;
+}
+
+int dopt_hip_conv_bwd_data_packed(const dopt_hip_conv_desc *d, const float *dy, const float *packed, float *dx)
+{
+    return dopt_hip_conv_bwd_data_packed_open(d, dy, packed, dx, nullptr);
+}
+
+int dopt_hip_split_sum_close(const dopt_hip_split_sum *open)
+{
+    DOPT_REQUIRE(open != nullptr, "dopt_hip_split_sum_close: null argument");
+    if (open->splits == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(open->splits > 1 && open->partial && open->value && open->elems % 4 == 0 && open->C > 0 && open->inner > 0,
+                 "dopt_hip_split_sum_close: malformed description");
+    DOPT_ENSURE_INIT();
+    return launch_splitk_reduce(open->elems, open->splits, open->partial, open->value, open->bias, (unsigned)open->C,
+                                (unsigned)open->inner);
 }
 
 int dopt_hip_conv_bwd_filter(const dopt_hip_conv_desc *d, const float *dy, const float *x, float *dw)

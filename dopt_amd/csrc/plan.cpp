@@ -587,6 +587,9 @@ struct HIPPlan::Builder {
     void pushPackStep(const std::vector<Prepack> &which);
     std::vector<Prepack> packs;
     std::vector<int> packOf;
+    // steps that run a convolution on a packed filter (candidates for leaving their result open)
+    struct ConvStep { size_t step; int op; int bwd; bool bias; dopt_hip_conv_desc d; const float *packed; };
+    std::vector<ConvStep> convSteps;
 
     Builder(const Graph &graph, HIPPlan *plan, const std::vector<int> &outs, unsigned f)
         : g(graph), p(plan), outputs(outs), flags(f), nops((int)graph.ops.size()), alias((size_t)nops),
@@ -618,6 +621,7 @@ struct HIPPlan::Builder {
     int prepackFilters();
     int allocateBuffers();
     int buildSteps();
+    void openSplitSums();
     void rememberAliases();
     int assignQueues();
     int createEvents();
@@ -1079,11 +1083,14 @@ int HIPPlan::Builder::buildSteps()
         std::string label = op.opType;
         void *extra = biasGradOf[id] >= 0 && needed[biasGradOf[id]] ? p->mResults[biasGradOf[id]] : nullptr;
         std::vector<int> stepInputs = inputsOf[id];
+        bool onPacked = false;
         if (packOf[id] >= 0) {  // the filter operand is read from its packed copy
             const Prepack pk = packs[(size_t)packOf[id]];
             if (pk.owner && pk.late) pushPackStep({pk});
             const float *packed = (const float *)pk.buf;
             const dopt_hip_conv_desc d = pk.d;
+            onPacked = true;
+            convSteps.push_back({0, id, pk.bwd, !pk.bwd && fusedKind[id] == 1, d, packed});
             if (pk.bwd) {
                 stepInputs = {op.deps[0]};
                 k = make([=](const std::vector<const void *> &in, void *out) {
@@ -1128,8 +1135,66 @@ int HIPPlan::Builder::buildSteps()
         s.inputBytes.resize(s.inputOps.size());
         for (size_t i = 0; i < s.inputOps.size(); i++) s.inputBytes[i] = g.ops[s.inputOps[i]].bytes();
         p->mSteps.push_back(std::move(s));
+        if (onPacked) convSteps.back().step = p->mSteps.size() - 1;
     }
     return DOPT_HIP_OK;
+}
+
+// A convolution that splits its reduction normally ends with a pass that adds the partial copies.
+// When the step right behind it is the batch norm (forward) or batch-norm gradient (backward) that
+// reads the whole result anyway, the convolution leaves the result open and that step adds the
+// copies while it loads them: one launch and one pass over the data less per such pair
+// (DOPT_HIP_PLAN_FUSE).  The two steps share a description of the open result; whether a result is
+// open at all is decided by the library at each run (it is not when the reduction was not split).
+void HIPPlan::Builder::openSplitSums()
+{
+    if (!(flags & DOPT_HIP_PLAN_FUSE)) return;
+    for (const ConvStep &cs : convSteps) {
+        if (cs.step + 1 >= p->mSteps.size()) continue;
+        Step &conv = p->mSteps[cs.step], &next = p->mSteps[cs.step + 1];
+        const int b = next.op;
+        if (b < 0 || prebuilt[b] || next.inputOps.empty()) continue;
+        const Operation &bo = g.ops[b];
+        size_t off;
+        if (root(next.inputOps[0], &off) != cs.op || off != 0) continue;   // first operand: x (forward) or dy (gradient)
+        auto open = std::make_shared<dopt_hip_split_sum>();
+        const dopt_hip_conv_desc d = cs.d;
+        const float *packed = cs.packed;
+        size_t N, C, inner;
+        if (!cs.bwd && bo.opType == "batchNormTrain" && bo.deps.size() == 5 && next.inputOps.size() == 5 &&
+            (fusedKind[b] == 0 || fusedKind[b] == 2)) {
+            auto it = bo.doubleAttrs.find("momentum");
+            if (it == bo.doubleAttrs.end()) continue;
+            const double momentum = it->second;
+            const int relu = fusedKind[b] == 2;
+            nci(g.ops[bo.deps[0]].shape, &N, &C, &inner);
+            const bool bias = cs.bias;
+            conv.kernel = make([=](const std::vector<const void *> &in, void *out) {
+                return dopt_hip_conv_fwd_bias_packed_open(&d, (const float *)in[0], packed, bias ? (const float *)in[1] : nullptr,
+                                                          (float *)out, open.get());
+            });
+            next.kernel = make([=](const std::vector<const void *> &in, void *out) {
+                if (open->value != in[0]) return fail(DOPT_HIP_ERR_RUNTIME, "plan: open convolution result is not the batch norm's input");
+                return dopt_hip_bn_train_open(N, C, inner, momentum, open.get(), (const float *)in[1], (const float *)in[2],
+                                              (const float *)in[3], (const float *)in[4], (float *)out, relu);
+            });
+        } else if (cs.bwd && bo.opType == "batchNormGrad" && bo.deps.size() == 3 &&
+                   ((fusedKind[b] == 3 && next.inputOps.size() == 4) || (fusedKind[b] == 0 && next.inputOps.size() == 3))) {
+            const bool relu = fusedKind[b] == 3;
+            void *extra = biasGradOf[b] >= 0 && needed[biasGradOf[b]] ? p->mResults[biasGradOf[b]] : nullptr;
+            nci(g.ops[bo.deps[1]].shape, &N, &C, &inner);
+            const int keep = uses[cs.op].size() == 1 && !isOutput(cs.op) ? 0 : 1;   // does anything else read dy?
+            conv.kernel = make([=](const std::vector<const void *> &in, void *out) {
+                return dopt_hip_conv_bwd_data_packed_open(&d, (const float *)in[0], packed, (float *)out, open.get());
+            });
+            next.kernel = make([=](const std::vector<const void *> &in, void *out) {
+                if (open->value != in[0]) return fail(DOPT_HIP_ERR_RUNTIME, "plan: open convolution result is not the gradient's input");
+                const float *y = relu ? (const float *)in[1] : nullptr;
+                const float *x = (const float *)in[relu ? 2 : 1], *scale = (const float *)in[relu ? 3 : 2];
+                return dopt_hip_bn_grad_open(N, C, inner, open.get(), keep, y, x, scale, (float *)out, (float *)extra);
+            });
+        }
+    }
 }
 
 void HIPPlan::Builder::rememberAliases()
@@ -1230,6 +1295,7 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         if (int rc = b.prepackFilters()) return rc;
     if (int rc = b.allocateBuffers()) return rc;
     if (int rc = b.buildSteps()) return rc;
+    b.openSplitSums();
     b.rememberAliases();
     if (flags & DOPT_HIP_PLAN_OVERLAP)
         if (int rc = b.assignQueues()) return rc;

@@ -205,6 +205,29 @@ int dopt_hip_conv_pack_batch(int n, const dopt_hip_conv_desc *descs, const int *
 int dopt_hip_conv_fwd_bias_packed(const dopt_hip_conv_desc *d, const float *x, const float *packed,
                                   const float *bias, float *y);
 int dopt_hip_conv_bwd_data_packed(const dopt_hip_conv_desc *d, const float *dy, const float *packed, float *dx);
+/* A convolution result left open: convolutions with few output tiles split their reduction over
+   several workgroups and finish with a pass that adds the partial copies (and the bias).  When the
+   next reader is a batch norm that reads the whole value anyway, that reader can add the copies
+   itself and the finishing pass is dropped.  The *_open entry points below are the packed entry
+   points above, except that when the reduction was split they skip the finishing pass and describe
+   the partial copies here; the value then MUST be closed by the very next call into this library
+   (dopt_hip_split_sum_close, dopt_hip_bn_train_open or dopt_hip_bn_grad_open): the copies live in
+   the library's workspace.  splits == 0 means the value is complete and there is nothing to close.
+   No counterpart in the reference, where cuDNN owns its workspace (cuda/nnet/cudnn7.d:111). */
+typedef struct dopt_hip_split_sum {
+    const float *partial; /* [splits][elems], copy s before copy s + 1 */
+    int splits;           /* 0: value is complete */
+    size_t elems;         /* N * C * inner */
+    size_t C, inner;      /* the value is [N, C, inner] */
+    const float *bias;    /* per-channel addend of the finished sum, or null */
+    float *value;         /* where the finished sum belongs */
+} dopt_hip_split_sum;
+int dopt_hip_conv_fwd_bias_packed_open(const dopt_hip_conv_desc *d, const float *x, const float *packed,
+                                       const float *bias, float *y, dopt_hip_split_sum *open);
+int dopt_hip_conv_bwd_data_packed_open(const dopt_hip_conv_desc *d, const float *dy, const float *packed,
+                                       float *dx, dopt_hip_split_sum *open);
+/* value = sum of the copies in order (+ bias): what the closed entry points do themselves. */
+int dopt_hip_split_sum_close(const dopt_hip_split_sum *open);
 /* `convolutionFiltersGrad`: cudnnConvolutionBackwardFilter, cudnn7.d:244. */
 int dopt_hip_conv_bwd_filter(const dopt_hip_conv_desc *d, const float *dy, const float *x, float *dw);
 
@@ -285,6 +308,16 @@ int dopt_hip_bn_grad_relu(size_t N, size_t C, size_t inner, const float *dy, con
    sums it (same value up to fp32 rounding). */
 int dopt_hip_bn_grad_fused(size_t N, size_t C, size_t inner, const float *dy, const float *y,
                            const float *x, const float *scale, float *packed, float *dx_sum);
+/* The same two kernels reading an open convolution result (see dopt_hip_split_sum): x_open->value is
+   the batch norm's input x; it is closed on the way (written in full, bit for bit what
+   dopt_hip_split_sum_close writes) because the backward pass reads it.  relu != 0: as
+   dopt_hip_bn_train_relu.  For the gradient, dy_open->value is dy; keep_dy == 0 says that nothing
+   else reads dy, which is then not written at all. */
+int dopt_hip_bn_train_open(size_t N, size_t C, size_t inner, double momentum, const dopt_hip_split_sum *x_open,
+                           const float *scale, const float *bias, const float *run_mean, const float *run_var,
+                           float *packed, int relu);
+int dopt_hip_bn_grad_open(size_t N, size_t C, size_t inner, const dopt_hip_split_sum *dy_open, int keep_dy,
+                          const float *y, const float *x, const float *scale, float *packed, float *dx_sum);
 /* `batchNormInference`: cudnnBatchNormalizationForwardInference, cudnn7.d:650-652; eps = 1e-5. */
 int dopt_hip_bn_infer(size_t N, size_t C, size_t inner, const float *x, const float *scale,
                       const float *bias, const float *mean, const float *var, float *y);

@@ -377,6 +377,82 @@ def test_packed_filter_entry_points_match_the_unpacked_ones():
         capi.check(lib.dopt_hip_conv_fwd_bias_packed(C.byref(d5), x.ptr, scratch.ptr, None, y.ptr))
 
 
+@pytest.mark.parametrize("xs,k", [((8, 256, 4, 4), 512),     # split reduction: the result is left open
+                                  ((16, 128, 8, 8), 256),
+                                  ((2, 64, 32, 32), 64),
+                                  ((16, 48, 2, 2), 40)])     # dense 2x2 route: never open
+def test_open_convolution_results_closed_by_batch_norm(xs, k):
+    """The *_open convolutions followed by dopt_hip_bn_train_open / dopt_hip_bn_grad_open /
+    dopt_hip_split_sum_close against the closed entry points (checked against the oracle elsewhere):
+    the copies are added in the same order, so everything is identical to the last bit."""
+    import ctypes as C
+    from dopt_amd import capi
+    lib = capi.load()
+    r = np.random.default_rng(xs[1] + k)
+    N, Cin, H, W = xs
+    ys = (N, k, H, W)
+    d = ops.conv_desc(xs, (k, Cin, 3, 3), (1, 1), (1, 1))
+    w = ops.tensor((r.standard_normal((k, Cin, 3, 3)) * 0.05).astype(np.float32))
+    packs = []
+    for bwd in (0, 1):
+        nbytes = lib.dopt_hip_conv_packed_bytes(C.byref(d), bwd)
+        assert nbytes > 0
+        packs.append(ops.Tensor([nbytes // 4]))
+    capi.check(lib.dopt_hip_conv_pack_batch(2, (type(d) * 2)(d, d), (C.c_int * 2)(0, 1), (C.c_void_p * 2)(w.ptr, w.ptr),
+                                            (C.c_void_p * 2)(packs[0].ptr, packs[1].ptr)))
+    inner = H * W
+
+    # forward: conv + bias -> batch norm + relu
+    x = ops.tensor(r.standard_normal(xs).astype(np.float32))
+    b = ops.tensor(r.standard_normal(k).astype(np.float32))
+    scale, bias = ops.tensor(r.uniform(0.5, 1.5, k).astype(np.float32)), ops.tensor(r.standard_normal(k).astype(np.float32))
+    mean, var = ops.tensor(np.zeros(k, np.float32)), ops.tensor(np.ones(k, np.float32))
+    conv_want = ops.Tensor(ys)
+    capi.check(lib.dopt_hip_conv_fwd_bias_packed(C.byref(d), x.ptr, packs[0].ptr, b.ptr, conv_want.ptr))
+    bn_want = ops.bn_train_relu(conv_want, scale, bias, mean, var, 0.9).numpy()
+    conv_want = conv_want.numpy()
+    for closer in ("bn", "close"):
+        conv_got, bn_got = ops.Tensor(ys), ops.Tensor([int(np.prod(ys)) + 2 * k])
+        conv_got.set(np.full(ys, np.nan, np.float32))
+        o = capi.SplitSum()
+        capi.check(lib.dopt_hip_conv_fwd_bias_packed_open(C.byref(d), x.ptr, packs[0].ptr, b.ptr, conv_got.ptr, C.byref(o)))
+        assert o.value == conv_got.ptr
+        if xs == (8, 256, 4, 4):
+            assert o.splits > 1 and o.elems == np.prod(ys) and o.C == k and o.inner == inner
+        if xs == (16, 48, 2, 2):
+            assert o.splits == 0
+        if closer == "close":
+            capi.check(lib.dopt_hip_split_sum_close(C.byref(o)))
+            o.splits = 0
+        capi.check(lib.dopt_hip_bn_train_open(N, k, inner, 0.9, C.byref(o), scale.ptr, bias.ptr, mean.ptr, var.ptr, bn_got.ptr, 1))
+        assert np.array_equal(conv_got.numpy(), conv_want)
+        assert np.array_equal(bn_got.numpy(), bn_want)
+
+    # backward: conv backward-data -> relu gradient + batch-norm gradient (+ bias gradient)
+    dy = ops.tensor(r.standard_normal(ys).astype(np.float32))
+    xin = ops.tensor(r.standard_normal(xs).astype(np.float32))         # the batch norm's input one layer down
+    yrelu = ops.tensor(np.maximum(r.standard_normal(xs), 0).astype(np.float32))
+    sc = ops.tensor(r.uniform(0.5, 1.5, Cin).astype(np.float32))
+    dx_want = ops.Tensor(xs)
+    capi.check(lib.dopt_hip_conv_bwd_data_packed(C.byref(d), dy.ptr, packs[1].ptr, dx_want.ptr))
+    g_want, db_want = ops.Tensor([int(np.prod(xs)) + 2 * Cin]), ops.Tensor([Cin])
+    capi.check(lib.dopt_hip_bn_grad_fused(N, Cin, inner, dx_want.ptr, yrelu.ptr, xin.ptr, sc.ptr, g_want.ptr, db_want.ptr))
+    dx_want, g_want, db_want = dx_want.numpy(), g_want.numpy(), db_want.numpy()
+    for keep in (1, 0):
+        dx_got, g_got, db_got = ops.Tensor(xs), ops.Tensor([int(np.prod(xs)) + 2 * Cin]), ops.Tensor([Cin])
+        dx_got.set(np.full(xs, 7.0, np.float32))
+        o = capi.SplitSum()
+        capi.check(lib.dopt_hip_conv_bwd_data_packed_open(C.byref(d), dy.ptr, packs[1].ptr, dx_got.ptr, C.byref(o)))
+        was_open = o.splits > 1
+        capi.check(lib.dopt_hip_bn_grad_open(N, Cin, inner, C.byref(o), keep, yrelu.ptr, xin.ptr, sc.ptr, g_got.ptr, db_got.ptr))
+        assert np.array_equal(g_got.numpy(), g_want)
+        assert np.array_equal(db_got.numpy(), db_want)
+        if keep or not was_open:
+            assert np.array_equal(dx_got.numpy(), dx_want)
+        else:
+            assert np.all(dx_got.numpy() == 7.0)   # nobody reads dy: it is not written
+
+
 def _small_convnet(seed):
     init = nnet.Init(seed)
     x, y = core.float32([16, 3, 16, 16]), core.float32([16, 10])
