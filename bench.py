@@ -176,7 +176,8 @@ def main():
             conv_bytes += one * (1 if i == 0 else 2)
         result["roofline"] = {
             "kernel": "conv_patch_k (3x3 implicit-GEMM convolution forward + backward-data of all 13 layers as the plan runs "
-                      "them, incl. filter pack and split reductions; layer 1 and the 2x2-image layers take their own kernels)",
+                      "them, incl. filter pack and the split reductions not taken over by the batch norm that follows; layer 1 and the "
+                      "2x2-image layers take their own kernels)",
             "bound": "mfma", "achieved": round(gather_tflops, 2), "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": round(gather_tflops / MFMA_FP32_PEAK_TFLOPS, 4), "traffic": traffic,
             "traffic_of": "conv_patch_k launches only (layers 2-10, 18 of the 25; 25.1 MB algorithmic per launch); the "
