@@ -196,12 +196,13 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_gather_k(Ga
 // re-fetched per filter tap: for a chunk of 16 input channels the block loads the input patch
 // under its pixel tile ONCE -- the tile's rows plus a one-pixel halo, zero-filled outside the
 // image by the buffer range check -- and the nine taps read it at nine offsets.  LDS holds the
-// patch position-major, Bp[pos][16 channels (+4 pad)], and the filter slab of one tap row-major,
-// As[m][16 channels (+4 pad)], so that a lane's operands for a whole 16-channel slab are two
-// 128-bit LDS reads per 32-wide fragment: lane half kh (= lane / 32) multiplies channels
-// kh*8 .. kh*8+7 of the chunk over the slab's eight matrix steps (the same channel permutation on
-// both operands, so every channel is counted once).  Per 32 matrix instructions a wavefront
-// issues 8 fragment reads, 1-2 filter loads and stores and ~5 patch loads and stores.
+// patch position-major, Bp[pos][16 channels (+4 pad)], so that a lane's pixel operands for a whole
+// 16-channel slab are two 128-bit LDS reads per 32-wide fragment; the packed filter,
+// wp[slab][m][16 channels], has the same shape per row, and a lane's filter operands are two 128-bit
+// loads straight from it.  Lane half kh (= lane / 32) multiplies channels kh*8 .. kh*8+7 of the
+// chunk over the slab's eight matrix steps (the same channel permutation on both operands, so
+// every channel is counted once).  Per 32 matrix instructions a wavefront issues 4 patch fragment
+// reads, 4 filter loads and ~5 patch loads and stores.
 
 struct PatchConv {
     const float *in;   // gathered operand [N, Cin, IH, IW]
@@ -221,17 +222,20 @@ struct PatchConv {
 
 __device__ inline unsigned fast_div(unsigned x, unsigned magic) { return __umulhi(x, magic); }
 
+// The filter fragments go from memory straight into the registers the matrix cores read: the
+// packed layout is the fragment layout (a wavefront fetches 32 rows x 64 bytes, 2 KB contiguous, per
+// 32 output channels and tap; the four wavefronts of a tile row fetch the same lines, three of them
+// from the L1), one tap ahead.  Only the patch goes through LDS, double buffered, so the workgroup
+// meets once per 16-channel chunk, when the patch buffers swap.  (Staging the filter slab in LDS as
+// well costs a barrier per tap: 1.1 % slower on the VGG step.)
 template <class T, int NPMAX, bool kCFull>
 __global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_patch_k(PatchConv p)
 {
     constexpr int BM = T::BM, BN = T::BN, THREADS = T::THREADS, MI = T::MI, NI = T::NI;
     constexpr int TAPS = 9, CH = 16, LDP = 20;
-    constexpr int NA = BM * CH / 4 / THREADS;  // float4 of the filter slab per thread
-    static_assert(NA >= 1, "tile too small for the thread count");
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int pstride = (p.psz + 1) * LDP;  // one spare position absorbs the stores of unused slots
-    float *const As0 = lds;                  // [2][BM * LDP]
-    float *const Bp0 = lds + 2 * BM * LDP;   // [2][pstride]
+    float *const Bp0 = lds;                  // [2][pstride]
 
     unsigned L;
     const unsigned tiles = (unsigned)(p.mtiles * p.ntiles);
@@ -280,28 +284,17 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_patch_k(Pat
     };
     auto patch_store = [&](int i, float *buf) { *(float *)((char *)buf + p_lds[i]) = preg[i]; };
 
-    // ---- filter slab slots: float4 f = ii*THREADS + tid -> (row f / 4, channel quad f % 4)
-    unsigned a_voff[NA];
-    int a_lds[NA];
-#pragma unroll
-    for (int ii = 0; ii < NA; ii++) {
-        const int f = ii * THREADS + tid;
-        a_voff[ii] = (unsigned)((m0 + f / 4) * CH + (f % 4) * 4) * 4u;  // m0 + row < Mp always
-        a_lds[ii] = (f / 4) * LDP + (f % 4) * 4;
-    }
-    float4 areg[NA];
+    // ---- filter fragments: this lane's 8 channels (kh * 8 ..) of row l32 of each 32-row group
     const unsigned slab_bytes = (unsigned)p.Mp * CH * 4u;
-    auto a_load = [&](int sidx) {
+    const unsigned fa_voff = (unsigned)((m0 + wm * (BM / T::WM) + l32) * CH + kh * 8) * 4u;   // m0 + row < Mp always
+    float4 fa_next[MI][2];
+    auto fa_load = [&](int slab) {   // past the last slab the range check returns zeros
 #pragma unroll
-        for (int ii = 0; ii < NA; ii++) areg[ii] = buffer_load_f32x4(rwp, a_voff[ii], (unsigned)sidx * slab_bytes);
+        for (int i = 0; i < MI; i++) {
+            fa_next[i][0] = buffer_load_f32x4(rwp, fa_voff + (unsigned)(i * 32 * CH) * 4u, (unsigned)slab * slab_bytes);
+            fa_next[i][1] = buffer_load_f32x4(rwp, fa_voff + (unsigned)(i * 32 * CH) * 4u + 16u, (unsigned)slab * slab_bytes);
+        }
     };
-    auto a_store = [&](float *buf) {
-#pragma unroll
-        for (int ii = 0; ii < NA; ii++) *(float4 *)&buf[a_lds[ii]] = areg[ii];
-    };
-
-    // ---- fragment addresses
-    const float *a_frag = As0 + (wm * (BM / T::WM) + l32) * LDP + kh * 8;
     int b_frag[NI];  // float offset inside a patch buffer of this lane's pixel, tap offset (0,0)
 #pragma unroll
     for (int j = 0; j < NI; j++) {
@@ -316,13 +309,12 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_patch_k(Pat
     // prologue: the first patch and the first filter slab
 #pragma unroll
     for (int i = 0; i < NPMAX; i++) patch_load(i, cb);
-    a_load(cb * TAPS);
+    fa_load(cb * TAPS);
 #pragma unroll
     for (int i = 0; i < NPMAX; i++) patch_store(i, Bp0);
-    a_store(As0);
     __syncthreads();
 
-    int acur = 0, pcur = 0;
+    int pcur = 0;
     int sidx = cb * TAPS;  // filter slab being multiplied
     // loads of the next patch are issued during taps 0..3 of a chunk, its LDS stores during taps 5..8
     constexpr int PER = (NPMAX + 3) / 4;
@@ -333,13 +325,11 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_patch_k(Pat
             constexpr int t = decltype(ttag)::value;
             constexpr int tr = t / 3, ts = t % 3;
             const int tapoff = (p.flip ? (2 - tr) * p.PC + (2 - ts) : tr * p.PC + ts) * LDP;
-            const float *ap = a_frag + acur * (BM * LDP);
-            float *const as_nxt = As0 + (acur ^ 1) * (BM * LDP);
             float4 fa[MI][2], fb[NI][2];
 #pragma unroll
             for (int i = 0; i < MI; i++) {
-                fa[i][0] = *(const float4 *)(ap + i * 32 * LDP);
-                fa[i][1] = *(const float4 *)(ap + i * 32 * LDP + 4);
+                fa[i][0] = fa_next[i][0];
+                fa[i][1] = fa_next[i][1];
             }
 #pragma unroll
             for (int j = 0; j < NI; j++) {
@@ -349,8 +339,7 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_patch_k(Pat
             static_for<0, 8>([&](auto stag) {
                 constexpr int ks = decltype(stag)::value;
                 // side work of this step
-                if constexpr (ks == 0) a_load(sidx + 1);
-                if constexpr (ks == 7) a_store(as_nxt);
+                if constexpr (ks == 0) fa_load(sidx + 1);
                 if constexpr (t < 4 && ks >= 1 && ks <= 6) {
                     // PER loads of tap t, dealt over steps 1..6
                     constexpr int first = t * PER + (ks - 1) * ((PER + 5) / 6);
@@ -382,8 +371,7 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_patch_k(Pat
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
-            __syncthreads();
-            acur ^= 1;
+            if constexpr (t == TAPS - 1) __syncthreads();
             ++sidx;
         });
         pcur ^= 1;
@@ -1208,7 +1196,7 @@ PatchSetup patch_setup(const dopt_hip_conv_desc *d, size_t P, size_t Q)
     pc.PR = pc.rows + 2; pc.PC = pc.OW + 2;
     pc.psz = pc.nimg * pc.PR * pc.PC;
     if ((size_t)pc.psz * 16 > (size_t)npmax * threads) return u;
-    u.lds_bytes = ((size_t)2 * BM * 20 + (size_t)2 * (pc.psz + 1) * 20) * sizeof(float);
+    u.lds_bytes = (size_t)2 * (pc.psz + 1) * 20 * sizeof(float);
     if (u.lds_bytes > 160 * 1024) return u;
     pc.magic_psz = div_magic((unsigned)pc.psz);
     pc.magic_img = div_magic((unsigned)(pc.PR * pc.PC));
