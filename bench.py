@@ -46,7 +46,8 @@ def build_step(batch, fused, views, timing, seed=0, fuse=True, overlap=False, gr
     loss = nnet.crossEntropy(preds.trainOutput, labels) + net.paramLoss
     flags = (core.PLAN_VIEWS if views else 0) | (core.PLAN_TIMING if timing else 0)
     flags |= core.PLAN_FUSE if (fuse and views) else 0
-    flags |= core.PLAN_OVERLAP if overlap else 0
+    flags |= core.PLAN_OVERLAP if overlap is True else 0
+    flags |= core.PLAN_OVERLAP_LIGHT if overlap == "light" else 0
     flags |= core.PLAN_GRAPH if (graph and not timing) else 0
     if fused:
         updater = online.fused_sgd([loss, preds.trainOutput], net.params, net.paramProj, 0.01, 0.0, flags=flags)
@@ -96,6 +97,8 @@ def main():
     ap.add_argument("--no-views", action="store_true", help="disable the copy-eliding plan rewrites")
     ap.add_argument("--no-fuse", action="store_true", help="run every operation as its own kernel")
     ap.add_argument("--overlap", action="store_true", help="run the filter gradients on a second queue")
+    ap.add_argument("--overlap-light", action="store_true",
+                    help="run only the small steps off the main chain (dense-layer gradients) on a second queue")
     ap.add_argument("--graph", action="store_true", help="replay the step's kernels as a recorded HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-kernel-timing", action="store_true", help="skip the per-kernel event pass")
@@ -107,7 +110,7 @@ def main():
     capi.check(capi.load().dopt_hip_init(0))
     fused, views, fuse = not a.unfused, not a.no_views, not a.no_fuse
 
-    updater, args, net = build_step(BATCH, fused, views, timing=False, fuse=fuse, overlap=a.overlap, graph=a.graph)
+    updater, args, net = build_step(BATCH, fused, views, timing=False, fuse=fuse, overlap=("light" if a.overlap_light else a.overlap), graph=a.graph)
     for _ in range(a.warmup):
         updater.step_async(args)
     ops.sync()
@@ -142,7 +145,7 @@ def main():
     if not a.no_kernel_timing:
         # Same step, every kernel object bracketed by hipEvents on the library stream.
         del updater
-        tup, targs, _ = build_step(BATCH, fused, views, timing=True, fuse=fuse, overlap=a.overlap)
+        tup, targs, _ = build_step(BATCH, fused, views, timing=True, fuse=fuse, overlap=("light" if a.overlap_light else a.overlap))
         for _ in range(2):
             tup.step_async(targs)
         ops.sync()

@@ -696,6 +696,7 @@ PLAN_TIMING = 2
 PLAN_FUSE = 4
 PLAN_OVERLAP = 8
 PLAN_GRAPH = 16
+PLAN_OVERLAP_LIGHT = 32
 
 
 class Plan:

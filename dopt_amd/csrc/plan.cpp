@@ -1231,6 +1231,7 @@ int HIPPlan::Builder::assignQueues()
             // a step with a second output (the absorbed bias gradient) stays on the main queue
             if ((wgrad || reads_side) && biasGradOf[st.op] < 0) {
                 st.lane = 1;
+                st.fenceBefore = true;
                 onSide[st.op] = 1;
                 p->mUsesSide = true;
                 fences++;
@@ -1240,6 +1241,88 @@ int HIPPlan::Builder::assignQueues()
             }
         }
         if (p->mUsesSide) {
+            p->mFences.resize((size_t)fences);
+            for (hipEvent_t &ev : p->mFences) DOPT_HIP_CHECK(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+        }
+    }
+    else if (flags & DOPT_HIP_PLAN_OVERLAP_LIGHT) {
+        // Small steps off the main chain: a step whose value reaches only plan outputs (directly or
+        // through other such steps) and that moves at most a few megabytes.  Each is moved up to
+        // right behind the last step that produces one of its inputs and runs on the side queue.
+        const size_t n = p->mSteps.size();
+        auto producer = [&](int id) {
+            while (alias[id].source >= 0) id = alias[id].source;
+            return id;
+        };
+        std::vector<int> stepOf((size_t)nops, -1);   // which step writes an operation's buffer
+        for (size_t i = 0; i < n; i++) {
+            const int op = p->mSteps[i].op;
+            if (op < 0) continue;
+            stepOf[op] = (int)i;
+            if (biasGradOf[op] >= 0) stepOf[biasGradOf[op]] = (int)i;
+        }
+        std::vector<std::vector<int>> readers(n), producers(n);
+        for (size_t i = 0; i < n; i++)
+            for (int in : p->mSteps[i].inputOps) {
+                const int s = stepOf[producer(in)];
+                if (s >= 0 && s != (int)i) {
+                    readers[(size_t)s].push_back((int)i);
+                    producers[i].push_back(s);
+                }
+            }
+        const size_t kLightBytes = (size_t)4 << 20;
+        std::vector<char> side(n, 0);
+        for (size_t i = n; i-- > 0;) {   // readers come later in the order, so they are decided first
+            const Step &st = p->mSteps[i];
+            if (st.op < 0 || biasGradOf[st.op] >= 0 || producers[i].empty()) continue;
+            const std::string &t = g.ops[st.op].opType;
+            if (t.compare(0, 11, "convolution") == 0 || t.compare(0, 9, "batchNorm") == 0 || t == "uniform") continue;
+            size_t bytes = g.ops[st.op].bytes();
+            for (size_t b : st.inputBytes) bytes += b;
+            bool off = bytes <= kLightBytes;
+            for (int r : readers[i]) off = off && side[(size_t)r];
+            side[i] = off;
+        }
+        // new order: a side step goes right behind the last of its producers in the new order (behind
+        // that producer's batch norm if the two share an open convolution result, and behind side steps
+        // already placed there); a producer that is a side step itself counts where it was placed
+        std::vector<char> glued(n, 0);   // step i must stay right in front of step i + 1
+        for (const ConvStep &cs : convSteps)
+            if (cs.step + 1 < n) glued[cs.step] = 1;
+        std::vector<std::vector<int>> behind(n);
+        std::vector<int> anchorOf(n, -1);
+        for (size_t i = 0; i < n; i++) {
+            if (!side[i]) continue;
+            int a = -1;
+            for (int pr : producers[i]) {
+                int at = side[(size_t)pr] ? anchorOf[(size_t)pr] : pr;
+                if (!side[(size_t)pr] && glued[(size_t)pr]) at += 1;
+                a = std::max(a, at);
+            }
+            anchorOf[i] = a;
+            behind[(size_t)a].push_back((int)i);
+        }
+        std::vector<Step> ordered;
+        ordered.reserve(n);
+        int fences = 1;
+        bool any = false;
+        for (size_t i = 0; i < n; i++) {
+            if (side[i]) continue;
+            ordered.push_back(std::move(p->mSteps[i]));
+            bool first = true;
+            for (int j : behind[i]) {
+                Step &st = p->mSteps[(size_t)j];
+                st.lane = 1;
+                st.fenceBefore = first;   // one wait covers the steps placed together
+                if (first) fences++;
+                first = false;
+                any = true;
+                ordered.push_back(std::move(st));
+            }
+        }
+        p->mSteps = std::move(ordered);
+        if (any) {
+            p->mUsesSide = true;
             p->mFences.resize((size_t)fences);
             for (hipEvent_t &ev : p->mFences) DOPT_HIP_CHECK(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
         }
@@ -1297,7 +1380,7 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
     if (int rc = b.buildSteps()) return rc;
     b.openSplitSums();
     b.rememberAliases();
-    if (flags & DOPT_HIP_PLAN_OVERLAP)
+    if (flags & (DOPT_HIP_PLAN_OVERLAP | DOPT_HIP_PLAN_OVERLAP_LIGHT))
         if (int rc = b.assignQueues()) return rc;
     if (int rc = b.createEvents()) return rc;
     // Resolve aliases once against the variables' own values so that result() is meaningful before
@@ -1375,7 +1458,7 @@ int HIPPlan::enqueue(int nrets, void *const *rets)
     };
     for (size_t i = 0; i < mSteps.size(); i++) {
         Step &s = mSteps[i];
-        if (s.lane == 1) {
+        if (s.lane == 1 && s.fenceBefore) {
             if (int rc = order(0, 1)) return rc;   // its inputs come from main-queue steps before it
         } else if (s.joinSide) {
             if (int rc = order(1, 0)) return rc;

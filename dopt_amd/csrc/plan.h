@@ -104,6 +104,7 @@ private:
         std::vector<const void *> inputs;
         std::vector<size_t> inputBytes;
         int lane = 0;                            // 1: runs on the side queue, beside the main chain
+        bool fenceBefore = false;                // side-queue step: first wait for what the main queue holds so far
         bool joinSide = false;                   // main-queue step that reads a side-queue result
     };
     Graph *mGraph = nullptr;

@@ -30,7 +30,9 @@ struct Runtime {
 
     // pool
     std::unordered_map<void *, size_t> live;           // ptr -> class size
-    std::map<size_t, std::vector<void *>> cached;      // class size -> free blocks
+    // class size -> free blocks, per queue: a block is reused in the order of the queue whose work
+    // last touched it, so only allocations made while that queue is current may take it
+    std::map<size_t, std::vector<void *>> cached[2];
     size_t live_bytes = 0, cached_bytes = 0, device_allocs = 0;
 
     // workspace, one per queue: kernels of the two queues run at the same time
@@ -225,9 +227,11 @@ int dopt_hip_shutdown(void)
     if (!r.ready) return DOPT_HIP_OK;
     (void)hipStreamSynchronize(r.stream);
     (void)hipStreamSynchronize(r.side);
-    for (auto &kv : r.cached)
-        for (void *p : kv.second) (void)hipFree(p);
-    r.cached.clear();
+    for (auto &lane_cache : r.cached) {
+        for (auto &kv : lane_cache)
+            for (void *p : kv.second) (void)hipFree(p);
+        lane_cache.clear();
+    }
     r.cached_bytes = 0;
     for (auto &kv : r.live) (void)hipFree(kv.first);
     r.live.clear();
@@ -263,8 +267,9 @@ static int pool_take(void **ptr, size_t bytes, bool zero)
     std::lock_guard<std::mutex> lk(r.mu);
     size_t cls = size_class(bytes);
     void *p = nullptr;
-    auto it = r.cached.find(cls);
-    if (it != r.cached.end() && !it->second.empty()) {
+    auto &mine = r.cached[r.lane];
+    auto it = mine.find(cls);
+    if (it != mine.end() && !it->second.empty()) {
         p = it->second.back();
         it->second.pop_back();
         r.cached_bytes -= cls;
@@ -275,9 +280,14 @@ static int pool_take(void **ptr, size_t bytes, bool zero)
         if (e != hipSuccess) {
             // give cached blocks back to the driver and retry once
             (void)hipGetLastError();
-            for (auto &kv : r.cached)
-                for (void *q : kv.second) (void)hipFree(q);
-            r.cached.clear();
+            // (blocks of the other queue may still be in use by its kernels: wait for both)
+            (void)hipStreamSynchronize(r.stream);
+            (void)hipStreamSynchronize(r.side);
+            for (auto &lane_cache : r.cached) {
+                for (auto &kv : lane_cache)
+                    for (void *q : kv.second) (void)hipFree(q);
+                lane_cache.clear();
+            }
             r.cached_bytes = 0;
             e = hipMalloc(&p, cls);
         }
@@ -287,9 +297,9 @@ static int pool_take(void **ptr, size_t bytes, bool zero)
         }
         r.device_allocs++;
     }
-    hipError_t e = zero ? hipMemsetAsync(p, 0, bytes, r.stream) : hipSuccess;
+    hipError_t e = zero ? hipMemsetAsync(p, 0, bytes, r.lane ? r.side : r.stream) : hipSuccess;
     if (e != hipSuccess) {
-        r.cached[cls].push_back(p);
+        mine[cls].push_back(p);
         r.cached_bytes += cls;
         return fail(DOPT_HIP_ERR_RUNTIME, "HIP default buffer initialisation failed: %s", hipGetErrorString(e));
     }
@@ -311,7 +321,7 @@ int dopt_hip_free(void *ptr)
     size_t cls = it->second;
     r.live.erase(it);
     r.live_bytes -= cls;
-    r.cached[cls].push_back(ptr);
+    r.cached[r.lane][cls].push_back(ptr);
     r.cached_bytes += cls;
     return DOPT_HIP_OK;
 }
@@ -322,9 +332,12 @@ int dopt_hip_pool_trim(void)
     std::lock_guard<std::mutex> lk(r.mu);
     if (!r.ready) return DOPT_HIP_OK;
     DOPT_HIP_CHECK(hipStreamSynchronize(r.stream));
-    for (auto &kv : r.cached)
-        for (void *p : kv.second) (void)hipFree(p);
-    r.cached.clear();
+    DOPT_HIP_CHECK(hipStreamSynchronize(r.side));
+    for (auto &lane_cache : r.cached) {
+        for (auto &kv : lane_cache)
+            for (void *p : kv.second) (void)hipFree(p);
+        lane_cache.clear();
+    }
     r.cached_bytes = 0;
     return DOPT_HIP_OK;
 }

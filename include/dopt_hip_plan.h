@@ -79,10 +79,16 @@ enum {
                                  recorded into a HIP graph the second time a given set of pointers is bound
                                  and replayed with one launch from then on (plans with per-kernel timing, the
                                  second queue, a `uniform` operation, or a kernel that allocates stay direct) */
-    DOPT_HIP_PLAN_OVERLAP = 8 /* filter gradients, and whatever only they feed, run on a second in-order
+    DOPT_HIP_PLAN_OVERLAP = 8, /* filter gradients, and whatever only they feed, run on a second in-order
                                  queue beside the chain that produces the feature gradients; the queues
                                  are ordered by events where a value crosses, and joined before the
                                  outputs are returned.  Same kernels, same values. */
+    DOPT_HIP_PLAN_OVERLAP_LIGHT = 32 /* the same second queue for small work only: a step that moves a few
+                                 megabytes and whose value reaches nothing but the plan's outputs (the
+                                 weight and bias gradients of dense layers) is enqueued right behind its
+                                 producers, on the second queue, instead of where the topological order
+                                 put it; it then runs beside the large kernels of the main chain, which
+                                 it would otherwise follow one launch latency at a time. */
 };
 
 /* new CUDAPlan(outputs) (cuda/package.d:267-312): topological sort, one kernel object per
