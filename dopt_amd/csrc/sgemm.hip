@@ -409,6 +409,32 @@ __global__ __launch_bounds__(256) void gemv_cols_k(size_t K, size_t N, size_t ks
     partial[(size_t)blockIdx.y * N + n] = acc;
 }
 
+// The same for a short reduction (K <= 256) in one launch: a block takes 64 columns, its four
+// groups of 64 threads take every fourth k, sixteen loads in flight per thread (clamped, not
+// branched), and the four sums are added in group order through LDS.
+__global__ __launch_bounds__(256) void gemv_cols_short_k(int K, int N, const float *a, const float *B, float *c)
+{
+    __shared__ float part[4][64];
+    const int col = threadIdx.x & 63, kl = threadIdx.x >> 6;
+    const int n = min((int)blockIdx.x * 64 + col, N - 1);
+    float acc = 0.0f;
+    for (int k0 = kl; k0 < K; k0 += 64) {
+        float av[16], bv[16];
+#pragma unroll
+        for (int u = 0; u < 16; u++) {
+            const int k = min(k0 + 4 * u, K - 1);
+            av[u] = a[k];
+            bv[u] = B[(size_t)k * N + n];
+        }
+#pragma unroll
+        for (int u = 0; u < 16; u++)
+            if (k0 + 4 * u < K) acc += av[u] * bv[u];
+    }
+    part[kl][col] = acc;
+    __syncthreads();
+    if (kl == 0 && (int)blockIdx.x * 64 + col < N) c[n] = ((part[0][col] + part[1][col]) + part[2][col]) + part[3][col];
+}
+
 unsigned flat_grid(size_t n)
 {
     size_t blocks = ceil_div(n, (size_t)256);
@@ -484,6 +510,12 @@ int sgemm_bias(int transA, int transB, size_t M, size_t N, size_t K, const float
     if (mv_cols) {
         const size_t R = M == 1 ? N : M;
         const float *mat = M == 1 ? B : A, *vec = M == 1 ? A : B;
+        if (K <= 256 && R < ((size_t)1 << 30)) {   // one launch, no partial sums
+            hipLaunchKernelGGL(gemv_cols_short_k, dim3((unsigned)ceil_div(R, (size_t)64)), dim3(256), 0, stream(), (int)K, (int)R,
+                               vec, mat, C);
+            DOPT_LAUNCH_CHECK();
+            return DOPT_HIP_OK;
+        }
         size_t nblocks = ceil_div(R, (size_t)256);
         size_t slices = ceil_div((size_t)num_cus() * 2, nblocks);
         if (slices > ceil_div(K, (size_t)32)) slices = ceil_div(K, (size_t)32);
