@@ -587,6 +587,9 @@ struct HIPPlan::Builder {
     void pushPackStep(const std::vector<Prepack> &which);
     std::vector<Prepack> packs;
     std::vector<int> packOf;
+    // what foldTransposes made of a matmul (or of the transpose behind one): C[M,N] = op(a) * op(b)
+    struct MatmulInfo { bool valid = false; int a = -1, b = -1, tA = 0, tB = 0; size_t M = 0, N = 0, K = 0; };
+    std::vector<MatmulInfo> mmInfo;
     // steps that run a convolution on a packed filter (candidates for leaving their result open)
     struct ConvStep { size_t step; int op; int bwd; bool bias; dopt_hip_conv_desc d; const float *packed; };
     std::vector<ConvStep> convSteps;
@@ -595,7 +598,7 @@ struct HIPPlan::Builder {
         : g(graph), p(plan), outputs(outs), flags(f), nops((int)graph.ops.size()), alias((size_t)nops),
           inputsOf((size_t)nops), fusedKind((size_t)nops, 0), prebuilt((size_t)nops), prebuiltLabel((size_t)nops),
           live((size_t)nops, 0), uses((size_t)nops), exposed((size_t)nops), biasGradOf((size_t)nops, -1),
-          absorbed((size_t)nops, 0), needed((size_t)nops, 0), packOf((size_t)nops, -1)
+          absorbed((size_t)nops, 0), needed((size_t)nops, 0), packOf((size_t)nops, -1), mmInfo((size_t)nops)
     {
     }
 
@@ -615,6 +618,7 @@ struct HIPPlan::Builder {
     void countReaders();
     void fusePairs();
     void foldTransposes();
+    void fuseDenseLayers();
     void formChains();
     void absorbBiasGrads();
     void markNeeded();
@@ -791,10 +795,83 @@ void HIPPlan::Builder::foldTransposes()
         fusedKind[id] = 6;
         inputsOf[id] = {a, b};
         const int ta = tA, tb = tB;
+        mmInfo[id].valid = true;
+        mmInfo[id].a = a; mmInfo[id].b = b; mmInfo[id].tA = ta; mmInfo[id].tB = tb;
+        mmInfo[id].M = M; mmInfo[id].N = N; mmInfo[id].K = K;
         prebuilt[id] = make([=](const std::vector<const void *> &in, void *out) {
             return dopt_hip_sgemm_t(ta, tb, M, N, K, (const float *)in[0], (const float *)in[1], (float *)out);
         });
         prebuiltLabel[id] = outT ? "matmul+transpose" : "matmul";
+    }
+}
+
+// A dense layer as the reference builds it: add(matmul(x, W^T), matmul(ones[m,1], bias[1,n])), usually
+// followed by relu.  When the product and the broadcast have no other reader they run as one kernel
+// (dopt_hip_sgemm_rank1); when, besides that, the sum is only read by a relu and by the x operand of
+// reluGrad (a sign test, and sign(relu(x)) = sign(x) where it matters), the kernel clamps as well
+// and the relu becomes an alias of its output - the same arrangement as batch norm + relu above.
+void HIPPlan::Builder::fuseDenseLayers()
+{
+    auto plain_product = [&](int id, MatmulInfo *mi) {   // a matmul this pass may absorb: no other reader, not an output
+        if (alias[id].source >= 0 || isOutput(id) || uses[id].size() != 1 || g.ops[id].dtype != DOPT_HIP_F32 ||
+            g.ops[id].rank() != 2)
+            return false;
+        if (fusedKind[id] == 6 && mmInfo[id].valid) {
+            *mi = mmInfo[id];
+            return true;
+        }
+        const Operation &o = g.ops[id];
+        if (fusedKind[id] || o.opType != "matmul" || o.deps.size() != 2) return false;
+        const Operation &l = g.ops[o.deps[0]], &r = g.ops[o.deps[1]];
+        if (l.rank() != 2 || r.rank() != 2 || l.dtype != DOPT_HIP_F32 || r.dtype != DOPT_HIP_F32) return false;
+        mi->valid = true;
+        mi->a = o.deps[0]; mi->b = o.deps[1]; mi->tA = mi->tB = 0;
+        mi->M = o.shape[0]; mi->N = o.shape[1]; mi->K = l.shape[1];
+        return true;
+    };
+    for (int id : p->mOps) {
+        const Operation &op = g.ops[id];
+        if (!live[id] || alias[id].source >= 0 || fusedKind[id] || op.opType != "add" || op.deps.size() != 2 ||
+            op.rank() != 2 || op.dtype != DOPT_HIP_F32 || op.volume() == 0)
+            continue;
+        for (int order = 0; order < 2; order++) {
+            // either operand may arrive through a reshape (repeat(bias, m) ends in one): look at the buffer's owner
+            size_t poff, qoff;
+            const int pid = root(op.deps[(size_t)order], &poff), qid = root(op.deps[(size_t)(1 - order)], &qoff);
+            MatmulInfo prod, outer;
+            if (pid == qid || poff != 0 || qoff != 0 || !plain_product(pid, &prod) || !plain_product(qid, &outer)) continue;
+            if (outer.K != 1 || outer.tA || outer.tB || prod.K == 0 || fusedKind[qid]) continue;   // u[M,1] * v[1,N] as written
+            if (prod.M != op.shape[0] || prod.N != op.shape[1] || outer.M != prod.M || outer.N != prod.N) continue;
+            // relu behind it?
+            int relu_op = -1;
+            bool clamp = !isOutput(id);
+            for (const Use &u : uses[id]) {
+                const Operation &r = g.ops[u.op];
+                if (u.off != 0) clamp = false;
+                else if (r.opType == "relu" && r.deps.size() == 1 && r.volume() == op.volume() && alias[u.op].source < 0 &&
+                         !fusedKind[u.op] && relu_op < 0)
+                    relu_op = u.op;
+                else if (!(r.opType == "reluGrad" && u.slot == 2)) clamp = false;
+            }
+            clamp = clamp && relu_op >= 0;
+            fusedKind[id] = 8;
+            inputsOf[id] = {prod.a, prod.b, outer.a, outer.b};
+            const MatmulInfo mi = prod;
+            const int relu = clamp ? 1 : 0;
+            prebuilt[id] = make([=](const std::vector<const void *> &in, void *out) {
+                return dopt_hip_sgemm_rank1(mi.tA, mi.tB, mi.M, mi.N, mi.K, (const float *)in[0], (const float *)in[1],
+                                            (const float *)in[2], (const float *)in[3], relu, (float *)out);
+            });
+            prebuiltLabel[id] = clamp ? "matmul+broadcast+relu" : "matmul+broadcast";
+            prebuilt[pid].reset();   // the product no longer runs on its own
+            prebuiltLabel[pid].clear();
+            fusedKind[pid] = 0;
+            if (clamp) {
+                alias[relu_op].source = id;   // the relu output IS this buffer now
+                alias[relu_op].offset = 0;
+            }
+            break;
+        }
     }
 }
 
@@ -1370,6 +1447,7 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         b.countReaders();
         b.fusePairs();
         b.foldTransposes();
+        b.fuseDenseLayers();
         b.formChains();
         b.absorbBiasGrads();
     }

@@ -196,7 +196,8 @@ constexpr int kSmallWaves = 8;
 template <bool kTA, bool kTB, bool kVec>
 __global__ __launch_bounds__(64 * kSmallWaves) void sgemm_small_k(int M, int N, int K, int lda, int ldb, int kslice,
                                                                    const float *A, const float *B, float *C,
-                                                                   const float *colbias, int bias_shift)
+                                                                   const float *colbias, int bias_shift,
+                                                                   const float *rowvec, int relu)
 {
     __shared__ float red[kSmallWaves][32 * 33];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, r = lane & 31;
@@ -239,7 +240,12 @@ __global__ __launch_bounds__(64 * kSmallWaves) void sgemm_small_k(int M, int N, 
 #pragma unroll
         for (int w = 1; w < kSmallWaves; w++) sum += red[w][rr * 33 + cc];
         if (m0 + rr < M && n0 + cc < N) {
-            if (colbias) sum += colbias[(n0 + cc) >> bias_shift];   // one value per group of 2^bias_shift columns
+            if (colbias) {   // one value per group of 2^bias_shift columns, times the row's factor when there is one
+                float add = colbias[(n0 + cc) >> bias_shift];
+                if (rowvec) add = __fmul_rn(rowvec[m0 + rr], add);   // rounded on its own, as the separate product is
+                sum += add;
+            }
+            if (relu) sum = sum < 0.0f ? 0.0f : sum;
             C[(size_t)(m0 + rr) * N + n0 + cc] = sum;
         }
     }
@@ -435,6 +441,20 @@ __global__ __launch_bounds__(256) void gemv_cols_short_k(int K, int N, const flo
     if (kl == 0 && (int)blockIdx.x * 64 + col < N) c[n] = ((part[0][col] + part[1][col]) + part[2][col]) + part[3][col];
 }
 
+// c[m][n] = relu?(c[m][n] + u[m] * v[n]): the epilogue of dopt_hip_sgemm_rank1 as a pass of its own, for the
+// shapes whose product kernel has none.  Each step rounds on its own, like the separate operations.
+__global__ __launch_bounds__(256) void rank1_epilogue_k(size_t M, size_t N, const float *u, const float *v, int relu, float *c)
+{
+    const size_t total = M * N;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        const size_t m = i / N, n = i - m * N;
+        float x = c[i];
+        if (v) x += __fmul_rn(u[m], v[n]);
+        if (relu) x = x < 0.0f ? 0.0f : x;
+        c[i] = x;
+    }
+}
+
 unsigned flat_grid(size_t n)
 {
     size_t blocks = ceil_div(n, (size_t)256);
@@ -479,8 +499,19 @@ namespace dopt {
 
 // C = op(A) * op(B), plus colbias[col >> bias_shift] on every element when colbias is given.  Returns
 // *biased = false when the shape took a kernel without that epilogue (the caller adds the bias itself).
+int sgemm_epilogue(int transA, int transB, size_t M, size_t N, size_t K, const float *A, const float *B, float *C,
+                   const float *colbias, int bias_shift, const float *rowvec, int relu, bool *biased);
+
 int sgemm_bias(int transA, int transB, size_t M, size_t N, size_t K, const float *A, const float *B, float *C,
                const float *colbias, int bias_shift, bool *biased)
+{
+    return sgemm_epilogue(transA, transB, M, N, K, A, B, C, colbias, bias_shift, nullptr, 0, biased);
+}
+
+// The products with an epilogue: + rowvec[row] * colbias[col >> bias_shift] (rowvec optional), then relu.
+// *biased says whether the kernel that ran applied it; if not, C holds the plain product.
+int sgemm_epilogue(int transA, int transB, size_t M, size_t N, size_t K, const float *A, const float *B, float *C,
+                   const float *colbias, int bias_shift, const float *rowvec, int relu, bool *biased)
 {
     *biased = false;
     if (M * N == 0) return DOPT_HIP_OK;
@@ -539,7 +570,7 @@ int sgemm_bias(int transA, int transB, size_t M, size_t N, size_t K, const float
     }
 
     // short reduction, both operands k-major, enough 128 x 128 tiles to fill the machine
-    if (transA && !transB && !colbias && panel_takes(M, N, K, A, B)) return panel_launch(false, M, N, K, A, B, C);
+    if (transA && !transB && !colbias && !relu && panel_takes(M, N, K, A, B)) return panel_launch(false, M, N, K, A, B, C);
 
     // small and medium outputs: one block per 32 x 32 tile, the reduction split over its wavefronts.
     // Each tile reads its own 32 rows of A and 32 columns of B, so the operand traffic grows with the
@@ -556,9 +587,9 @@ int sgemm_bias(int transA, int transB, size_t M, size_t N, size_t K, const float
 #define DOPT_SMALL(TA, TB)                                                                                             \
     do {                                                                                                               \
         if (vec) hipLaunchKernelGGL((sgemm_small_k<TA, TB, true>), grid, block, 0, stream(), (int)M, (int)N, (int)K, lda, \
-                                    ldb, kslice, A, B, C, colbias, bias_shift);                                        \
+                                    ldb, kslice, A, B, C, colbias, bias_shift, rowvec, relu);                           \
         else hipLaunchKernelGGL((sgemm_small_k<TA, TB, false>), grid, block, 0, stream(), (int)M, (int)N, (int)K, lda,  \
-                                ldb, kslice, A, B, C, colbias, bias_shift);                                            \
+                                ldb, kslice, A, B, C, colbias, bias_shift, rowvec, relu);                               \
     } while (0)
             if (transA && transB) DOPT_SMALL(true, true);
             else if (transA) DOPT_SMALL(true, false);
@@ -566,7 +597,7 @@ int sgemm_bias(int transA, int transB, size_t M, size_t N, size_t K, const float
             else DOPT_SMALL(false, false);
 #undef DOPT_SMALL
             DOPT_LAUNCH_CHECK();
-            *biased = colbias != nullptr;
+            *biased = true;   // whatever epilogue was asked for, this kernel applied it
             return DOPT_HIP_OK;
         }
     }
@@ -641,6 +672,18 @@ bool sgemm_fold2x2(size_t C, size_t K, size_t N, const float *x, const float *dy
 }  // namespace dopt
 
 extern "C" {
+
+int dopt_hip_sgemm_rank1(int transA, int transB, size_t M, size_t N, size_t K, const float *A, const float *B,
+                         const float *u, const float *v, int relu, float *C)
+{
+    DOPT_REQUIRE((u == nullptr) == (v == nullptr), "dopt_hip_sgemm_rank1: u and v go together");
+    bool applied = false;
+    if (int rc = dopt::sgemm_epilogue(transA, transB, M, N, K, A, B, C, v, 0, u, relu, &applied)) return rc;
+    if (applied || M * N == 0 || (!v && !relu)) return DOPT_HIP_OK;
+    hipLaunchKernelGGL(rank1_epilogue_k, dim3(flat_grid(M * N)), dim3(256), 0, dopt::stream(), M, N, u, v, relu, C);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
 
 int dopt_hip_sgemm_t(int transA, int transB, size_t M, size_t N, size_t K, const float *A, const float *B, float *C)
 {

@@ -215,6 +215,19 @@ def matmul_t(a, b, trans_a=False, trans_b=False, out=None):
     return out
 
 
+def matmul_rank1(a, b, u, v, relu=False, trans_a=False, trans_b=False, out=None):
+    """op(a) . op(b) + u[M,1] . v[1,N], then relu: a dense layer in one kernel (u, v may both be None)."""
+    K, M = (a.shape if trans_a else a.shape[::-1])
+    N, K2 = (b.shape if trans_b else b.shape[::-1])
+    if K != K2:
+        raise capi.HipError(1, "matmul: inner dimensions differ")
+    out = _out(out, (M, N))
+    capi.check(capi.load().dopt_hip_sgemm_rank1(int(trans_a), int(trans_b), M, N, K, a.ptr, b.ptr,
+                                                u.ptr if u is not None else None, v.ptr if v is not None else None,
+                                                int(bool(relu)), out.ptr))
+    return out
+
+
 def conv_desc(xshape, wshape, padding=(0, 0), stride=(1, 1)):
     N, Cc, H, W = xshape
     K, C2, R, S = wshape

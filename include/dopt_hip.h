@@ -169,6 +169,15 @@ int dopt_hip_sgemm(size_t M, size_t N, size_t K, const float *A, const float *B,
    the `transpose` kernels that only feed a matmul. */
 int dopt_hip_sgemm_t(int transA, int transB, size_t M, size_t N, size_t K, const float *A,
                      const float *B, float *C);
+/* C = op(A) * op(B) + u[M,1] * v[1,N], then relu when relu != 0: a dense layer as the reference
+   spells it -- matmul(x, W^T) (nnet/layers/dense.d:107) plus the bias broadcast over the rows, which
+   is itself a matmul with a ones column (dense.d:143, core/ops/basic.d:370-381), then the relu
+   layer -- in one kernel.  u and v may both be null (no rank-one term).  The product, the rank-one
+   term, the sum and the relu are each rounded as the four separate kernels round them, so the
+   result is identical to running them one after the other.  Used by plans compiled with
+   DOPT_HIP_PLAN_FUSE. */
+int dopt_hip_sgemm_rank1(int transA, int transB, size_t M, size_t N, size_t K, const float *A,
+                         const float *B, const float *u, const float *v, int relu, float *C);
 
 typedef struct {
     size_t N, C, H, W;       /* features [N,C,H,W] */

@@ -535,6 +535,29 @@ def test_batched_device_copies():
     assert np.array_equal(c.numpy(), np.arange(8, dtype=np.float32))
 
 
+@pytest.mark.parametrize("shape", [(128, 512, 512), (70, 33, 129), (1024, 1024, 1024), (1, 300, 77), (200, 1, 64), (5, 7, 1)])
+@pytest.mark.parametrize("tb", [False, True])
+def test_sgemm_with_rank_one_term_and_relu(shape, tb):
+    """dopt_hip_sgemm_rank1 (a dense layer in one kernel) against the four kernels it stands for, bit for
+    bit: small-output kernel (epilogue in the kernel), tile engine and the matrix-vector / outer-product
+    paths (epilogue as a pass of its own)."""
+    M, N, K = shape
+    r = rng(M + 5 * N + 11 * K + tb)
+    a = T(r.standard_normal((M, K)).astype(np.float32))
+    bh = r.standard_normal((K, N)).astype(np.float32)
+    b = T(np.ascontiguousarray(bh.T) if tb else bh)
+    u, v = T(r.standard_normal((M, 1)).astype(np.float32)), T(r.standard_normal((1, N)).astype(np.float32))
+    prod = ops.matmul_t(a, b, False, tb)
+    want = ops.pointwise("add", prod, ops.matmul(u, v))
+    assert np.array_equal(ops.matmul_rank1(a, b, u, v, trans_b=tb).numpy(), want.numpy())
+    assert np.array_equal(ops.matmul_rank1(a, b, u, v, relu=True, trans_b=tb).numpy(), ops.relu(want).numpy())
+    assert np.array_equal(ops.matmul_rank1(a, b, None, None, relu=True, trans_b=tb).numpy(), ops.relu(prod).numpy())
+    assert np.array_equal(ops.matmul_rank1(a, b, None, None, trans_b=tb).numpy(), prod.numpy())
+    # and against the oracle
+    ref = O.matmul(a.numpy(), bh, f64=True) + u.numpy().astype(np.float64) @ v.numpy().astype(np.float64)
+    assert_close(ops.matmul_rank1(a, b, u, v, relu=True, trans_b=tb).numpy(), np.maximum(ref, 0), "sgemm_rank1", scale=np.sqrt(K))
+
+
 @pytest.mark.parametrize("shape", [(2048, 2048, 128), (2048, 2048, 100), (2048, 2052, 17), (2044, 2080, 64)])
 def test_sgemm_short_reduction_large_output(shape):
     # A stored [K][M], B stored [K][N], K <= 128 and about one 128 x 128 tile per CU: the kernel that
