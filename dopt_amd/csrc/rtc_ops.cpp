@@ -663,7 +663,7 @@ int dopt_hip_reduce(const char *op, int dtype, const size_t *shape, int rank, co
         void *dst = out;
         void *tmp = nullptr;
         if (ri > 0) {
-            rc = dopt_hip_malloc(&tmp, outer * inner * 4);
+            rc = scratch_alloc(&tmp, outer * inner * 4);   // every element is written by the pass below: no fill
             if (rc) break;
             dst = tmp;
         }
