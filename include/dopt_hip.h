@@ -321,7 +321,7 @@ int dopt_hip_bn_grad_fused(size_t N, size_t C, size_t inner, const float *dy, co
    the batch norm's input x; it is closed on the way (written in full, bit for bit what
    dopt_hip_split_sum_close writes) because the backward pass reads it.  relu != 0: as
    dopt_hip_bn_train_relu.  For the gradient, dy_open->value is dy; keep_dy == 0 says that nothing
-   else reads dy, which is then not written at all. */
+   else reads dy, which then need not be written (and is not, where the kernel adds the copies itself). */
 int dopt_hip_bn_train_open(size_t N, size_t C, size_t inner, double momentum, const dopt_hip_split_sum *x_open,
                            const float *scale, const float *bias, const float *run_mean, const float *run_var,
                            float *packed, int relu);
