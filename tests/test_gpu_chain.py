@@ -175,7 +175,9 @@ def _random_graph(r, n_leaves=4, n_ops=18, size=96):
 def test_random_graphs_give_the_same_values_with_every_rewrite(seed):
     outs = _random_graph(np.random.default_rng(100 + seed))
     want = core.compile(outs).execute()
-    for flags in (core.PLAN_VIEWS, core.PLAN_VIEWS | core.PLAN_FUSE, core.PLAN_VIEWS | core.PLAN_FUSE | core.PLAN_GRAPH):
+    for flags in (core.PLAN_VIEWS, core.PLAN_VIEWS | core.PLAN_FUSE, core.PLAN_VIEWS | core.PLAN_FUSE | core.PLAN_GRAPH,
+                  core.PLAN_OVERLAP_LIGHT, core.PLAN_VIEWS | core.PLAN_FUSE | core.PLAN_OVERLAP_LIGHT,
+                  core.PLAN_VIEWS | core.PLAN_FUSE | core.PLAN_OVERLAP):
         plan = core.compile(outs, flags)
         bufs = [ops.Tensor(o.shape) for o in outs]
         for _ in range(3):                                           # direct, recorded, replayed
