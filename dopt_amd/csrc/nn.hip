@@ -361,16 +361,16 @@ __device__ __forceinline__ float group_sum(float v)
     return v;
 }
 
-template <int G>
+template <int G, int Q>   // G lanes share a row, Q quads per lane (G * Q >= C / 4)
 __global__ __launch_bounds__(kBlock) void softmax_reg_fwd_k(size_t N, uint32_t C4, const float4 *x, float4 *y)
 {
     const size_t row = ((size_t)blockIdx.x * kBlock + threadIdx.x) / G;
     const uint32_t lig = threadIdx.x % G;
     const bool live = row < N;                    // dead rows still take part in the shuffles
     const float4 *px = x + (live ? row : 0) * C4;
-    float v[16];
+    float v[4 * Q];
 #pragma unroll
-    for (int k = 0; k < 4; k++) {
+    for (int k = 0; k < Q; k++) {
         const uint32_t c = lig + G * k;
         const float4 q = px[c < C4 ? c : 0];
         const bool in = c < C4;
@@ -381,11 +381,11 @@ __global__ __launch_bounds__(kBlock) void softmax_reg_fwd_k(size_t N, uint32_t C
     }
     float m = v[0];
 #pragma unroll
-    for (int i = 1; i < 16; i++) m = dmax(m, v[i]);
+    for (int i = 1; i < 4 * Q; i++) m = dmax(m, v[i]);
     m = group_max<G>(m);
     float s = 0.0f;
 #pragma unroll
-    for (int k = 0; k < 4; k++) {
+    for (int k = 0; k < Q; k++) {
         const bool in = lig + G * k < C4;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -397,13 +397,13 @@ __global__ __launch_bounds__(kBlock) void softmax_reg_fwd_k(size_t N, uint32_t C
     if (!live) return;
     float4 *py = y + row * C4;
 #pragma unroll
-    for (int k = 0; k < 4; k++) {
+    for (int k = 0; k < Q; k++) {
         const uint32_t c = lig + G * k;
         if (c < C4) py[c] = make_float4(v[4 * k] / s, v[4 * k + 1] / s, v[4 * k + 2] / s, v[4 * k + 3] / s);
     }
 }
 
-template <int G>
+template <int G, int Q>
 __global__ __launch_bounds__(kBlock) void softmax_reg_bwd_k(size_t N, uint32_t C4, const float4 *dy, const float4 *y,
                                                              float4 *dx)
 {
@@ -411,10 +411,10 @@ __global__ __launch_bounds__(kBlock) void softmax_reg_bwd_k(size_t N, uint32_t C
     const uint32_t lig = threadIdx.x % G;
     const bool live = row < N;
     const size_t base = (live ? row : 0) * C4;
-    float g[16], p[16];
+    float g[4 * Q], p[4 * Q];
     float dot = 0.0f;
 #pragma unroll
-    for (int k = 0; k < 4; k++) {
+    for (int k = 0; k < Q; k++) {
         const uint32_t c = lig + G * k;
         const bool in = c < C4;
         const float4 a = dy[base + (in ? c : 0)], b = y[base + (in ? c : 0)];
@@ -425,7 +425,7 @@ __global__ __launch_bounds__(kBlock) void softmax_reg_bwd_k(size_t N, uint32_t C
     dot = group_sum<G>(dot);
     if (!live) return;
 #pragma unroll
-    for (int k = 0; k < 4; k++) {
+    for (int k = 0; k < Q; k++) {
         const uint32_t c = lig + G * k;
         if (c < C4)
             dx[base + c] = make_float4(p[4 * k] * (g[4 * k] - dot), p[4 * k + 1] * (g[4 * k + 1] - dot),
@@ -632,9 +632,15 @@ int dopt_hip_softmax_fwd(size_t N, size_t C, size_t inner, const float *x, float
     if (const int G = softmax_group(C, inner, x, y, y)) {
         const dim3 grid((unsigned)ceil_div(N * G, (size_t)kBlock)), block(kBlock);
         const uint32_t C4 = (uint32_t)(C / 4);
-        if (G == 16) hipLaunchKernelGGL(softmax_reg_fwd_k<16>, grid, block, 0, stream(), N, C4, (const float4 *)x, (float4 *)y);
-        else if (G == 32) hipLaunchKernelGGL(softmax_reg_fwd_k<32>, grid, block, 0, stream(), N, C4, (const float4 *)x, (float4 *)y);
-        else hipLaunchKernelGGL(softmax_reg_fwd_k<64>, grid, block, 0, stream(), N, C4, (const float4 *)x, (float4 *)y);
+        // quads per lane: one up to 256 classes, two or four above (no work on lanes' absent quads)
+#define DOPT_SOFTMAX_FWD(GV, QV) \
+    hipLaunchKernelGGL((softmax_reg_fwd_k<GV, QV>), grid, block, 0, stream(), N, C4, (const float4 *)x, (float4 *)y)
+        if (G == 16) DOPT_SOFTMAX_FWD(16, 1);
+        else if (G == 32) DOPT_SOFTMAX_FWD(32, 1);
+        else if (C4 <= 64) DOPT_SOFTMAX_FWD(64, 1);
+        else if (C4 <= 128) DOPT_SOFTMAX_FWD(64, 2);
+        else DOPT_SOFTMAX_FWD(64, 4);
+#undef DOPT_SOFTMAX_FWD
     } else if (inner == 1 && C >= 64)
         hipLaunchKernelGGL(softmax_rows_fwd_k, dim3((unsigned)ceil_div(N, (size_t)(kBlock / 64))), dim3(kBlock), 0, stream(),
                            N, C, x, y);
@@ -652,9 +658,15 @@ int dopt_hip_softmax_bwd(size_t N, size_t C, size_t inner, const float *dy, cons
     if (const int G = softmax_group(C, inner, dy, y, dx)) {
         const dim3 grid((unsigned)ceil_div(N * G, (size_t)kBlock)), block(kBlock);
         const uint32_t C4 = (uint32_t)(C / 4);
-        if (G == 16) hipLaunchKernelGGL(softmax_reg_bwd_k<16>, grid, block, 0, stream(), N, C4, (const float4 *)dy, (const float4 *)y, (float4 *)dx);
-        else if (G == 32) hipLaunchKernelGGL(softmax_reg_bwd_k<32>, grid, block, 0, stream(), N, C4, (const float4 *)dy, (const float4 *)y, (float4 *)dx);
-        else hipLaunchKernelGGL(softmax_reg_bwd_k<64>, grid, block, 0, stream(), N, C4, (const float4 *)dy, (const float4 *)y, (float4 *)dx);
+#define DOPT_SOFTMAX_BWD(GV, QV)                                                                                  \
+    hipLaunchKernelGGL((softmax_reg_bwd_k<GV, QV>), grid, block, 0, stream(), N, C4, (const float4 *)dy, (const float4 *)y, \
+                       (float4 *)dx)
+        if (G == 16) DOPT_SOFTMAX_BWD(16, 1);
+        else if (G == 32) DOPT_SOFTMAX_BWD(32, 1);
+        else if (C4 <= 64) DOPT_SOFTMAX_BWD(64, 1);
+        else if (C4 <= 128) DOPT_SOFTMAX_BWD(64, 2);
+        else DOPT_SOFTMAX_BWD(64, 4);
+#undef DOPT_SOFTMAX_BWD
     } else if (inner == 1 && C >= 64)
         hipLaunchKernelGGL(softmax_rows_bwd_k, dim3((unsigned)ceil_div(N, (size_t)(kBlock / 64))), dim3(kBlock), 0, stream(),
                            N, C, dy, y, dx);

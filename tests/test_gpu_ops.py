@@ -379,7 +379,7 @@ def test_maxpool_and_grad(shape, dims):
 
 
 @pytest.mark.parametrize("shape", [(1, 5), (128, 10), (256, 10), (4, 7, 3), (3, 5, 2, 2), (37, 64), (300, 1000),
-                                   (5, 130), (70, 128), (9, 132), (33, 260), (17, 1024), (3, 1028), (1, 68)])
+                                   (5, 130), (70, 128), (9, 132), (33, 260), (17, 1024), (3, 1028), (1, 68), (6, 256), (6, 512), (6, 516)])
 def test_softmax_and_grad(shape):
     r = rng(52)
     x = (r.standard_normal(shape) * 3).astype(np.float32)
