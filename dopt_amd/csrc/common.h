@@ -20,17 +20,22 @@ void clear_error();
 // The library stream (created by dopt_hip_init; lazily initialises device 0 otherwise).
 hipStream_t stream();
 bool ensure_init();
+bool is_initialised();   // dopt_hip_init (or a lazily initialising entry point) has run
 
 // Process-wide scratch memory, grown on demand (the analogue of the single conv workspace at
 // cuda/nnet/cudnn7.d:111).  Valid until the next call that asks for more; all users enqueue on
 // the one library stream, so consecutive users never overlap.
 void *workspace(size_t bytes);
+// Changes whenever a workspace is reallocated (its address may have changed): whoever keeps the
+// address beyond one call -- a recorded HIP graph -- compares generations before using it again.
+unsigned long workspace_generation();
 // The library owns two in-order queues.  Everything enqueues on the main one unless a plan has
 // switched to the side queue for a step it overlaps with its main chain (set_lane(1) ... set_lane(0));
 // each queue has its own workspace.
 void set_lane(int lane);
-// While a plan records its kernels into a HIP graph, entry points that would allocate or fill
-// device memory fail instead (neither can be replayed), and the plan runs its kernels directly.
+// While a plan records its kernels into a HIP graph, entry points that would allocate (from the
+// driver or from the pool), fill device memory or grow the workspace fail instead (none of these can
+// be replayed), and the plan runs its kernels directly.
 void set_capturing(bool on);
 bool capturing();
 int scratch_alloc(void **ptr, size_t bytes);   // pooled block, NOT zero-filled; release with dopt_hip_free

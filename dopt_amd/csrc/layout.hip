@@ -484,15 +484,19 @@ int dopt_hip_copy_d2d_batch(int n, void *const *dst, const void *const *src, con
         const bool small = bytes[i] <= 65536 && bytes[i] % 4 == 0 &&
                            (reinterpret_cast<uintptr_t>(dst[i]) & 3u) == 0 && (reinterpret_cast<uintptr_t>(src[i]) & 3u) == 0;
         if (!small) {
+            // the copies are sequential: what is still waiting in the batch goes first
+            if (int rc = flush()) return rc;
             if (int rc = dopt_hip_copy_d2d(dst[i], src[i], bytes[i])) return rc;
             continue;
         }
         // copies of one launch run side by side: a copy that reads or rewrites what an earlier one
-        // of the batch writes starts a new launch
+        // of the batch writes, or that writes what an earlier one reads, starts a new launch
         for (int j = 0; j < filled; j++) {
-            const char *d0 = (const char *)b.dst[j], *d1 = d0 + (size_t)b.words[j] * 4;
+            const size_t len = (size_t)b.words[j] * 4;
+            const char *d0 = (const char *)b.dst[j], *d1 = d0 + len;
+            const char *r0 = (const char *)b.src[j], *r1 = r0 + len;
             const char *s0 = (const char *)src[i], *t0 = (const char *)dst[i];
-            if ((s0 < d1 && s0 + bytes[i] > d0) || (t0 < d1 && t0 + bytes[i] > d0)) {
+            if ((s0 < d1 && s0 + bytes[i] > d0) || (t0 < d1 && t0 + bytes[i] > d0) || (t0 < r1 && t0 + bytes[i] > r0)) {
                 if (int rc = flush()) return rc;
                 break;
             }

@@ -1412,8 +1412,10 @@ int HIPPlan::Builder::createEvents()
     // what a recorded graph cannot reproduce: per-kernel timing events, the second queue, and `uniform`,
     // whose kernel takes a call counter that changes with every execution
     p->mGraphOk = !(flags & DOPT_HIP_PLAN_TIMING) && !p->mUsesSide;
-    for (const Step &st : p->mSteps)
+    for (const Step &st : p->mSteps) {
         if (st.op >= 0 && g.ops[st.op].opType == "uniform") p->mGraphOk = false;
+        if (!st.kernel->replayable()) p->mGraphOk = false;
+    }
     if (flags & DOPT_HIP_PLAN_TIMING) {
         p->mEvents.resize(p->mSteps.size());
         for (auto &ev : p->mEvents) {
@@ -1599,6 +1601,14 @@ int HIPPlan::execute(int nargs, const int *argOps, const void *const *argPtrs, c
         CapturedRun *run = nullptr;
         for (CapturedRun &c : mRuns)
             if (c.key == key) run = &c;
+        if (run && run->exec && run->wsGeneration != workspace_generation()) {
+            // the workspace moved since this run was recorded (some other plan or call needed a larger
+            // one): the recording holds the old address and must not be launched again; record anew
+            (void)hipGraphExecDestroy(run->exec);
+            if (run->graph) (void)hipGraphDestroy(run->graph);
+            run->exec = nullptr;
+            run->graph = nullptr;
+        }
         if (run && run->exec) {
             mReplays++;
             DOPT_HIP_CHECK(hipGraphLaunch(run->exec, stream()));
@@ -1610,13 +1620,14 @@ int HIPPlan::execute(int nargs, const int *argOps, const void *const *argPtrs, c
                 if (mRuns.front().graph) (void)hipGraphDestroy(mRuns.front().graph);
                 mRuns.erase(mRuns.begin());
             }
-            mRuns.push_back(CapturedRun{key, nullptr, nullptr});
+            mRuns.push_back(CapturedRun{key, nullptr, nullptr, 0});
         } else {
             if (int rc = resolve(nargs, argOps, argPtrs, argOnHost)) return rc;
             DOPT_HIP_CHECK(hipStreamBeginCapture(stream(), hipStreamCaptureModeRelaxed));
             set_capturing(true);
             const int rc = enqueue(nrets, rets);
             set_capturing(false);
+            run->wsGeneration = workspace_generation();   // cannot change while recording: growth is refused
             hipGraph_t graph = nullptr;
             const hipError_t ended = hipStreamEndCapture(stream(), &graph);
             if (rc == DOPT_HIP_OK && ended == hipSuccess && graph &&
@@ -1688,6 +1699,7 @@ public:
     {
         return mK.execute(mK.self, (int)inputs.size(), inputs.data(), inputBytes.data(), output, outputBytes);
     }
+    bool replayable() const override { return false; }   // the callback's host code would not run on a replay
 
 private:
     dopt_hip_kernel mK;

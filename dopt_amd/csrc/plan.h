@@ -61,6 +61,9 @@ public:
     // inputs[i] is the buffer of op.deps[i]; output is preallocated by the plan.
     virtual int execute(const std::vector<const void *> &inputs, const std::vector<size_t> &inputBytes, void *output,
                         size_t outputBytes) = 0;
+    // false: execute() does host work that a replayed HIP graph would skip (a caller-registered kernel
+    // may do anything); a plan with such a kernel is never recorded.
+    virtual bool replayable() const { return true; }
 };
 
 // alias CUDAKernelCtr = CUDAKernel delegate(Operation op) (cuda/package.d:25).  A constructor
@@ -125,6 +128,7 @@ private:
         std::vector<const void *> key;           // argument ops and pointers, return pointers
         hipGraph_t graph;
         hipGraphExec_t exec;                     // null until the second execution with this key
+        unsigned long wsGeneration;              // workspace_generation() when it was recorded
     };
     std::vector<CapturedRun> mRuns;
     bool mGraphOk = false;

@@ -38,6 +38,7 @@ struct Runtime {
     // workspace, one per queue: kernels of the two queues run at the same time
     void *ws[2] = {nullptr, nullptr};
     size_t ws_bytes[2] = {0, 0};
+    unsigned long ws_generation = 0;   // bumped whenever a workspace moves: recorded graphs hold its address
 
     // rtc
     std::unordered_map<std::string, hipFunction_t> kernels;
@@ -115,12 +116,15 @@ bool ensure_init()
     return init_locked(0) == DOPT_HIP_OK;
 }
 
+bool is_initialised() { return rt().ready; }
+
 hipStream_t stream() { return rt().lane ? rt().side : rt().stream; }
 hipStream_t lane_stream(int lane) { return lane ? rt().side : rt().stream; }
 void set_lane(int lane) { rt().lane = lane ? 1 : 0; }
 void set_capturing(bool on) { rt().capturing = on; }
 bool capturing() { return rt().capturing; }
 int num_cus() { return rt().cus; }
+unsigned long workspace_generation() { return rt().ws_generation; }
 
 void *workspace(size_t bytes)
 {
@@ -135,6 +139,7 @@ void *workspace(size_t bytes)
     if (r.ws[l]) (void)hipFree(r.ws[l]);
     r.ws[l] = nullptr;
     r.ws_bytes[l] = 0;
+    r.ws_generation++;
     size_t want = size_class(bytes);
     if (hipMalloc(&r.ws[l], want) != hipSuccess) {
         fail(DOPT_HIP_ERR_OOM, "workspace: unable to allocate %zu bytes", want);
@@ -241,6 +246,7 @@ int dopt_hip_shutdown(void)
         r.ws[l] = nullptr;
         r.ws_bytes[l] = 0;
     }
+    r.ws_generation++;
     r.lane = 0;
     for (hipModule_t m : r.modules) (void)hipModuleUnload(m);
     r.modules.clear();
@@ -262,8 +268,10 @@ static int pool_take(void **ptr, size_t bytes, bool zero)
     if (bytes == 0) return DOPT_HIP_OK;
     DOPT_ENSURE_INIT();
     Runtime &r = rt();
-    if (r.capturing && zero)
-        return fail(DOPT_HIP_ERR_UNSUPPORTED, "dopt_hip_malloc: a zero-filled allocation cannot be recorded into a graph");
+    // A block taken while a graph is being recorded would be written by every replay, long after it was
+    // handed back and given to someone else: the plan runs its kernels directly instead.
+    if (r.capturing)
+        return fail(DOPT_HIP_ERR_UNSUPPORTED, "dopt_hip_malloc: a device allocation cannot be recorded into a graph");
     std::lock_guard<std::mutex> lk(r.mu);
     size_t cls = size_class(bytes);
     void *p = nullptr;
@@ -274,8 +282,6 @@ static int pool_take(void **ptr, size_t bytes, bool zero)
         it->second.pop_back();
         r.cached_bytes -= cls;
     } else {
-        if (r.capturing)
-            return fail(DOPT_HIP_ERR_UNSUPPORTED, "dopt_hip_malloc: a device allocation cannot be recorded into a graph");
         hipError_t e = hipMalloc(&p, cls);
         if (e != hipSuccess) {
             // give cached blocks back to the driver and retry once

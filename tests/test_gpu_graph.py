@@ -522,6 +522,75 @@ def test_recorded_graph_replays_match_direct_execution(maker):
     assert la == lb
 
 
+def test_recorded_graph_survives_a_workspace_move_and_pool_reuse():
+    """A recording holds device addresses.  The library's workspace moves when a later caller needs a larger
+    one, and pooled blocks released after a run are handed to new tensors: replays after both events must
+    still equal direct execution (the plan records anew instead of launching a stale graph), and tensors
+    allocated in between must keep their contents."""
+    r = np.random.default_rng(3)
+    fx = ops.tensor(r.standard_normal((16, 3, 16, 16)).astype(np.float32))
+    fy = ops.tensor(np.eye(10, dtype=np.float32)[r.integers(0, 10, 16)])
+    base = core.PLAN_VIEWS | core.PLAN_FUSE
+    xa, ya, neta, lossa = _small_convnet(11)
+    xb, yb, netb, lossb = _small_convnet(11)
+    direct = online.fused_sgd([lossa], neta.params, neta.paramProj, flags=base)
+    replay = online.fused_sgd([lossb], netb.params, netb.paramProj, flags=base | core.PLAN_GRAPH)
+    for step in range(3):
+        assert direct({xa: fx, ya: fy})[0] == replay({xb: fx, yb: fy})[0]
+    assert replay.plan.recordings()["recorded"] == 1
+    # a filter gradient with a long reduction needs far more workspace than the small network did
+    big_x = ops.tensor(r.standard_normal((64, 64, 32, 32)).astype(np.float32))
+    big_dy = ops.tensor(r.standard_normal((64, 64, 32, 32)).astype(np.float32))
+    ops.conv_bwd_filter(big_dy, big_x, (64, 64, 3, 3), (1, 1), (1, 1))
+    ops.sum(ops.tensor(r.standard_normal((4096, 2048)).astype(np.float32)), [0])
+    # blocks of every small size class, handed out after the recording and filled with a pattern
+    guards = [ops.tensor(np.full(n, 3.25, np.float32)) for n in (64, 256, 1024, 4096, 16384, 65536, 262144, 1 << 20) for _ in range(4)]
+    for step in range(3):
+        assert direct({xa: fx, ya: fy})[0] == replay({xb: fx, yb: fy})[0]
+    for a, b in zip(neta.params, netb.params):
+        assert np.array_equal(a.value, b.value)
+    for gd in guards:
+        assert np.all(gd.numpy() == 3.25)
+
+
+def test_graph_flag_leaves_plans_with_caller_registered_kernels_direct():
+    """A kernel registered through the C ABI runs host code in execute(); a replay would skip it."""
+    lib = core._lib()
+
+    class Kernel(C.Structure):
+        _fields_ = [("self", C.c_void_p), ("execute", C.c_void_p), ("destroy", C.c_void_p)]
+
+    EXEC = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int, C.POINTER(C.c_void_p), C.POINTER(C.c_size_t), C.c_void_p,
+                       C.c_size_t)
+    CTOR = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.POINTER(Kernel))
+    calls = []
+
+    def execute(self, nin, inputs, nbytes, out, out_bytes):
+        calls.append(1)
+        return capi.load().dopt_hip_copy_d2d(out, inputs[0], out_bytes)
+    exec_c = EXEC(execute)
+
+    def ctor(graph, op, user, out):
+        out[0].self = None
+        out[0].execute = C.cast(exec_c, C.c_void_p)
+        out[0].destroy = None
+        return 0
+    ctor_c = CTOR(ctor)
+    lib.dopt_hip_deregister_kernel(b"atanh")
+    assert lib.dopt_hip_register_kernel(b"atanh", C.cast(ctor_c, C.c_void_p), None) == 0
+    try:
+        x = core.float32([64])
+        plan = core.compile([core.atanh(x) + x], core.PLAN_GRAPH)
+        xin, out = ops.tensor(np.arange(64, dtype=np.float32)), ops.Tensor([64])
+        for _ in range(4):
+            plan.execute({x: xin}, [out])
+            assert np.array_equal(out.numpy(), 2 * np.arange(64, dtype=np.float32))
+        assert len(calls) == 4
+        assert plan.recordings() == {"recorded": 0, "replays": 0}
+    finally:
+        lib.dopt_hip_deregister_kernel(b"atanh")
+
+
 def test_graph_flag_leaves_plans_with_random_draws_direct():
     x = core.float32([64], np.ones(64, np.float32))
     y = core.uniformSample([64]) * x

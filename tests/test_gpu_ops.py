@@ -533,6 +533,25 @@ def test_batched_device_copies():
     b = (C.c_size_t * 2)(32, 32)
     capi.check(lib.dopt_hip_copy_d2d_batch(2, d, s, b))
     assert np.array_equal(c.numpy(), np.arange(8, dtype=np.float32))
+    # write-after-read inside one call: copy 1 reads `a`, copy 2 overwrites `a`; copy 1 must see the old `a`
+    a, z, out = T(np.arange(8, dtype=np.float32)), T(np.full(8, 7, np.float32)), ops.Tensor((8,))
+    d = (C.c_void_p * 2)(out.ptr, a.ptr)
+    s = (C.c_void_p * 2)(a.ptr, z.ptr)
+    capi.check(lib.dopt_hip_copy_d2d_batch(2, d, s, b))
+    assert np.array_equal(out.numpy(), np.arange(8, dtype=np.float32))
+    assert np.array_equal(a.numpy(), np.full(8, 7, np.float32))
+    # a large copy (its own transfer) behind a small one whose destination it reads
+    big = 20000
+    a, m, out = T(np.arange(big, dtype=np.float32)), ops.Tensor((big,)), ops.Tensor((big,))
+    head = T(np.full(8, -1, np.float32))
+    capi.check(lib.dopt_hip_copy_d2d(m.ptr, a.ptr, 4 * big))
+    d = (C.c_void_p * 2)(m.ptr, out.ptr)
+    s = (C.c_void_p * 2)(head.ptr, m.ptr)
+    b = (C.c_size_t * 2)(32, 4 * big)
+    capi.check(lib.dopt_hip_copy_d2d_batch(2, d, s, b))
+    want = np.arange(big, dtype=np.float32)
+    want[:8] = -1
+    assert np.array_equal(out.numpy(), want)
 
 
 @pytest.mark.parametrize("shape", [(128, 512, 512), (70, 33, 129), (1024, 1024, 1024), (1, 300, 77), (200, 1, 64), (5, 7, 1)])
