@@ -95,6 +95,7 @@ PROTOTYPES = {
     "dopt_hip_relu_bwd": [_sz, _vp, _vp, _vp],
     "dopt_hip_bias_fwd": [_sz, _sz, _sz, _vp, _vp, _vp],
     "dopt_hip_bias_bwd": [_sz, _sz, _sz, _vp, _vp],
+    "dopt_hip_bias_bwd_noalloc": [_sz, _sz, _sz, _vp, _vp],
     "dopt_hip_uniform": [C.c_uint64, C.c_uint64, _sz, _vp],
     "dopt_hip_philox_raw": [C.c_uint64, C.c_uint64, _sz, _vp],
     "dopt_hip_image_transform": [_sz, _sz, _sz, _sz, _sz, _sz, _vp, _vp, _vp],

@@ -149,6 +149,12 @@ __device__ inline float block_sum(float v, float *part)
     return r;  // valid in thread 0
 }
 
+__global__ __launch_bounds__(kBlock) void fill_zero_k(size_t n, float *out)
+{
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) out[i] = 0.0f;
+}
+
 // Stage 1 of db[c] = sum_{n,i} dy[n,c,i]: block (c, s) sums images n = s, s+S, ... of channel c.
 __global__ __launch_bounds__(kBlock) void bias_bwd_partial_k(size_t N, size_t C, size_t inner, size_t S,
                                                               const float *dy, float *partial)
@@ -561,6 +567,29 @@ int dopt_hip_bias_fwd(size_t N, size_t C, size_t inner, const float *x, const fl
     return DOPT_HIP_OK;
 }
 
+// How many image slices per channel the two-stage sum uses: enough (channel, slice) blocks to fill the machine.
+static size_t bias_bwd_slices(size_t N, size_t C)
+{
+    size_t S = ceil_div((size_t)num_cus() * 8, C);
+    if (S > N) S = N;
+    if (S > 64) S = 64;
+    if (S < 1) S = 1;
+    return S;
+}
+
+// The two launches of the sliced sum; `partial` holds C * S floats, every one of which stage 1 writes
+// before stage 2 reads it (nothing has to be cleared).
+static int bias_bwd_two_stage(size_t N, size_t C, size_t inner, size_t S, const float *dy, float *partial, float *db)
+{
+    hipLaunchKernelGGL(bias_bwd_partial_k, dim3((unsigned)(C * S)), dim3(kBlock), 0, stream(), N, C, inner, S, dy,
+                       partial);
+    DOPT_LAUNCH_CHECK();
+    hipLaunchKernelGGL(bias_bwd_final_k, dim3((unsigned)ceil_div(C, (size_t)kBlock)), dim3(kBlock), 0, stream(), C, S,
+                       partial, db);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
 int dopt_hip_bias_bwd(size_t N, size_t C, size_t inner, const float *dy, float *db)
 {
     if (C == 0) return DOPT_HIP_OK;
@@ -573,20 +602,51 @@ int dopt_hip_bias_bwd(size_t N, size_t C, size_t inner, const float *dy, float *
         DOPT_LAUNCH_CHECK();
         return DOPT_HIP_OK;
     }
-    // Enough (channel, image-slice) blocks to fill the machine; partials are then summed in a fixed order.
-    size_t S = ceil_div((size_t)num_cus() * 8, C);
-    if (S > N) S = N;
-    if (S > 64) S = 64;
-    if (S < 1) S = 1;
+    const size_t S = bias_bwd_slices(N, C);
     float *partial = (float *)workspace(C * S * sizeof(float));
     if (!partial) return DOPT_HIP_ERR_OOM;
-    hipLaunchKernelGGL(bias_bwd_partial_k, dim3((unsigned)(C * S)), dim3(kBlock), 0, stream(), N, C, inner, S, dy,
-                       partial);
-    DOPT_LAUNCH_CHECK();
-    hipLaunchKernelGGL(bias_bwd_final_k, dim3((unsigned)ceil_div(C, (size_t)kBlock)), dim3(kBlock), 0, stream(), C, S,
-                       partial, db);
-    DOPT_LAUNCH_CHECK();
-    return DOPT_HIP_OK;
+    return bias_bwd_two_stage(N, C, inner, S, dy, partial, db);
+}
+
+// ---- the same sum for callers that must not allocate
+// The per-(channel, slice) partial sums live in this array instead of the library's grown-on-demand
+// workspace.  Every device the library runs on holds its own copy at its own address until the process
+// ends; host code only ever uses the address hipGetSymbolAddress reports for the current device.
+static constexpr size_t kBiasScratchFloats = 65536;   // 256 KiB
+static __device__ __align__(256) float scratch[kBiasScratchFloats];
+static constexpr int kMaxDevices = 64;
+static float *g_scratch_ptr[kMaxDevices];             // per device; null until that device's first call
+
+int dopt_hip_bias_bwd_noalloc(size_t N, size_t C, size_t inner, const float *dy, float *db)
+{
+    if (C == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(db && (N * inner == 0 || dy), "dopt_hip_bias_bwd_noalloc: null argument");
+    DOPT_REQUIRE(is_initialised(), "dopt_hip_bias_bwd_noalloc: call dopt_hip_init first (this entry point sets nothing up)");
+    DOPT_REQUIRE(C <= 0x7fffffffu / 64, "dopt_hip_bias_bwd_noalloc: too many channels");
+    if (N * inner == 0) {   // a fill kernel, not a memset node: callers may be recording a graph
+        hipLaunchKernelGGL(fill_zero_k, dim3((unsigned)ceil_div(C, (size_t)kBlock)), dim3(kBlock), 0, stream(), C, db);
+        DOPT_LAUNCH_CHECK();
+        return DOPT_HIP_OK;
+    }
+    if (inner < 256) {      // one launch, no partial sums: same kernel as dopt_hip_bias_bwd
+        hipLaunchKernelGGL(bias_bwd_flat_k, dim3((unsigned)C), dim3(kBlock), 0, stream(), N, C, inner, dy, db);
+        DOPT_LAUNCH_CHECK();
+        return DOPT_HIP_OK;
+    }
+    const size_t S = bias_bwd_slices(N, C);
+    DOPT_REQUIRE(C * S <= kBiasScratchFloats,
+                 "dopt_hip_bias_bwd_noalloc: %zu channels x %zu slices exceed the built-in scratch of %zu partial sums; "
+                 "use dopt_hip_bias_bwd", C, S, kBiasScratchFloats);
+    int dev = -1;
+    DOPT_HIP_CHECK(hipGetDevice(&dev));
+    DOPT_REQUIRE(dev >= 0 && dev < kMaxDevices, "dopt_hip_bias_bwd_noalloc: device index %d out of range", dev);
+    if (!g_scratch_ptr[dev]) {   // once per device, with that device current
+        float *p = nullptr;
+        DOPT_HIP_CHECK(hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch)));
+        DOPT_REQUIRE(p != nullptr, "dopt_hip_bias_bwd_noalloc: the scratch array has no device address");
+        g_scratch_ptr[dev] = p;
+    }
+    return bias_bwd_two_stage(N, C, inner, S, dy, g_scratch_ptr[dev], db);
 }
 
 int dopt_hip_maxpool_fwd(size_t N, size_t C, size_t H, size_t W, size_t ph, size_t pw, const float *x, float *y)
