@@ -24,3 +24,19 @@ def pytest_configure(config):
 def kats():
     with open(os.path.join(ROOT, "tests", "golden", "reference_kats.json")) as f:
         return json.load(f)
+
+
+def pytest_sessionfinish(session, exitstatus):
+    """The configuration tests record the largest error they saw per quantity; keep the table where a
+    GPU run's outputs are collected."""
+    try:
+        import util
+    except ImportError:
+        return
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    if not util.ERROR_ROWS or not os.path.isdir(out_dir):
+        return
+    with open(os.path.join(out_dir, "parity_errors.txt"), "w") as f:
+        f.write("%-34s %-40s %12s %14s %12s\n" % ("case", "quantity", "max|err|", "err/(a+r|w|)", "max|want|"))
+        for case, what, err, ratio, mag in util.ERROR_ROWS:
+            f.write("%-34s %-40s %12.3e %14.3f %12.3e\n" % (case, what, err, ratio, mag))

@@ -2,8 +2,10 @@
 
 Tolerances are the ones the project states: bit-exact for integer, index and layout work and
 for single-rounding fp32 arithmetic; <= 2 ulp for fp32 transcendentals; rtol 1e-4 / atol 1e-5
-for GEMM, convolution and reductions (atol scaled by sqrt(reduction length) where the summed
-terms are O(1) random numbers, since the sum itself then has that magnitude).
+for GEMM, convolution and reductions.  Where a test sums n products of N(0,1) numbers the sum itself
+has magnitude sqrt(n) and atol is scaled by that; the same kernel is then run again on operands scaled
+as the configurations scale them (He-scaled weights, gradients that carry the 1/batch of a mean loss),
+where results are O(1) or smaller, and must meet the stated tolerance with no rescaling.
 """
 import numpy as np
 import pytest
@@ -131,6 +133,8 @@ def test_sum_and_max(shape, axes):
     want64 = x.astype(np.float64).sum(axis=tuple(axes) if axes else None)
     assert got.shape == np.asarray(want64).shape
     assert_close(got, want64, "sum", scale=np.sqrt(red))
+    xm = (x * np.float32(1.0 / np.sqrt(red))).astype(np.float32)      # sums of O(1): stated tolerance as it stands
+    assert_close(ops.sum(T(xm), axes).numpy(), xm.astype(np.float64).sum(axis=tuple(axes) if axes else None), "sum, O(1)")
     if red <= 4096:  # the reference's own fp32 left-fold is itself within tolerance of the device result
         assert_close(got, O.sum(x, axes), "sum vs reference order", scale=np.sqrt(red))
     assert np.array_equal(ops.max_element(T(x), axes).numpy(), O.max_element(x, axes))
@@ -255,6 +259,10 @@ def test_matmul(M, N, K):
         return
     want = O.matmul(a, b, f64=True) if M * N * K < 5e8 else (a.astype(np.float64) @ b.astype(np.float64))
     assert_close(got, want, "matmul %dx%dx%d" % (M, N, K), scale=np.sqrt(K))
+    # a dense layer's operands: He-scaled weights keep the products O(1); stated tolerance as it stands
+    bw = (b * np.sqrt(2.0 / K)).astype(np.float32)
+    want = O.matmul(a, bw, f64=True) if M * N * K < 5e8 else (a.astype(np.float64) @ bw.astype(np.float64))
+    assert_close(ops.matmul(T(a), T(bw)).numpy(), want, "matmul, He-scaled %dx%dx%d" % (M, N, K))
 
 
 def test_matmul_broadcast_by_ones_is_exact():
@@ -285,7 +293,11 @@ CONV_CASES = [  # N, C, H, W, K, R, S, pad, stride
     (4, 3, 32, 32, 64, 3, 3, (1, 1), (1, 1)),     # VGG conv1 shape at batch 4
     (2, 64, 32, 32, 64, 3, 3, (1, 1), (1, 1)),    # VGG conv2
     (2, 64, 16, 16, 128, 3, 3, (1, 1), (1, 1)),   # VGG conv3
+    (2, 128, 16, 16, 128, 3, 3, (1, 1), (1, 1)),  # VGG conv4
+    (2, 128, 8, 8, 256, 3, 3, (1, 1), (1, 1)),    # VGG conv5
+    (2, 256, 8, 8, 256, 3, 3, (1, 1), (1, 1)),    # VGG conv6-7
     (8, 256, 4, 4, 512, 3, 3, (1, 1), (1, 1)),    # VGG conv8: split reduction
+    (8, 512, 4, 4, 512, 3, 3, (1, 1), (1, 1)),    # VGG conv9-10
     (16, 512, 2, 2, 512, 3, 3, (1, 1), (1, 1)),   # VGG conv11-13
     (2, 16, 32, 32, 160, 1, 1, (0, 0), (1, 1)),   # WRN 1x1 shortcut
     (2, 160, 32, 32, 320, 3, 3, (1, 1), (2, 2)),  # WRN stage entry, stride 2
@@ -354,6 +366,10 @@ def test_convolution_all_three(case):
     dw = ops.conv_bwd_filter(T(dy), T(x), w.shape, pad, st).numpy()
     npix = N * y_ref.shape[2] * y_ref.shape[3]
     assert_close(dw, O.conv_bwd_filter(dy, x, w.shape, pad, st), "conv bwd-filter", scale=np.sqrt(npix))
+    # an upstream gradient with the 1/(pixels summed) scale of a mean loss: stated tolerance as it stands
+    dys = (dy * np.float32(1.0 / npix)).astype(np.float32)
+    dw = ops.conv_bwd_filter(T(dys), T(x), w.shape, pad, st).numpy()
+    assert_close(dw, O.conv_bwd_filter(dys, x, w.shape, pad, st), "conv bwd-filter, mean-loss gradient")
 
 
 def test_convolution_matches_reference_cpu_kernel_on_same_shapes():
@@ -414,6 +430,8 @@ def test_bias(shape):
     assert np.array_equal(ops.add_bias(T(x), T(b)).numpy(), O.add_bias(x, b))
     red = x.size // shape[1]
     assert_close(ops.add_bias_grad(T(x)).numpy(), O.add_bias_grad(x), "bias grad", scale=np.sqrt(red))
+    xs = (x * np.float32(1.0 / red)).astype(np.float32)
+    assert_close(ops.add_bias_grad(T(xs)).numpy(), O.add_bias_grad(xs), "bias grad, mean-loss gradient")
 
 
 # ----------------------------------------------------------------------------- batch norm
@@ -443,6 +461,11 @@ def test_batchnorm_train_grad_infer(shape):
     gw = O.bn_grad(dy, x, gamma)
     assert_close(g[:vol], gw[:vol], "bn dx")
     assert_close(g[vol:], gw[vol:], "bn dscale/dbias", scale=np.sqrt(m))
+    dys = (dy * np.float32(1.0 / m)).astype(np.float32)     # mean-loss scale: stated tolerance as it stands
+    g = ops.bn_grad(T(dys), T(x), T(gamma)).numpy()
+    gw = O.bn_grad(dys, x, gamma)
+    assert_close(g[:vol], gw[:vol], "bn dx, mean-loss gradient")
+    assert_close(g[vol:], gw[vol:], "bn dscale/dbias, mean-loss gradient")
     assert_close(ops.bn_infer(T(x), T(gamma), T(beta), T(rm), T(rv)).numpy(), O.bn_infer(x, gamma, beta, rm, rv),
                  "bn infer")
 

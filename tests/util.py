@@ -31,6 +31,27 @@ def assert_close(got, want, what="", rtol=GEMM_RTOL, atol=GEMM_ATOL, scale=None)
                              (what, bad.sum(), bad.size, i, got.ravel()[i], want.ravel()[i]))
 
 
+# Rows of (case, quantity, max |err|, max |err| / (atol + rtol |want|), max |want|) collected by the
+# configuration tests; conftest.py writes them to gpurun_out/parity_errors.txt at the end of a session.
+ERROR_ROWS = []
+
+
+def err_ratio(got, want, what=None, case=None, rtol=GEMM_RTOL, atol=GEMM_ATOL):
+    """max |got - want| / (atol + rtol |want|): at most 1 exactly when assert_close(got, want) with the same
+    unscaled tolerance passes.  Recorded under (case, what) when both are given."""
+    got = np.asarray(got, np.float64).ravel()
+    want = np.asarray(want, np.float64).ravel()
+    assert got.shape == want.shape, (what, got.shape, want.shape)
+    err = np.abs(got - want)
+    ratio = float((err / (atol + rtol * np.abs(want))).max()) if err.size else 0.0
+    if not np.isfinite(got).all():
+        ratio = float("inf")
+    if what is not None:
+        ERROR_ROWS.append((case or "", what, float(err.max()) if err.size else 0.0, ratio,
+                           float(np.abs(want).max()) if want.size else 0.0))
+    return ratio
+
+
 M0, M1, W0, W1 = 0xD2511F53, 0xCD9E8D57, 0x9E3779B9, 0xBB67AE85
 
 
