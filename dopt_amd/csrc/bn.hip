@@ -522,6 +522,297 @@ __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, un
     }
 }
 
+// ---- cluster-resident path -------------------------------------------------------------------
+// Channels too large for one block's registers but small enough for a few blocks' (up to kMaxCluster x
+// 32768 values: the first VGG layers at batch 128 hold 131072 values per channel): S consecutive
+// blocks share a channel, each keeps its piece in registers, and the pieces' statistics meet once in
+// device memory.  x (and dy) are still read once and the op is still one launch.
+//
+// Every block publishes (the mean it centred on, centred squares about that mean, sum dy,
+// sum dy*(x - that mean)) and waits for its S - 1 partners; all of them then fold the S records in
+// block order in float64 (M2 = sum of M2_j + n_j (mean_j - mean)^2, the pairwise update of Chan et
+// al.), so every block of a channel derives bit-identical statistics and the result does not depend
+// on arrival order.
+//
+// What travels between blocks are single 64-bit words written and read with device-scope atomics: a
+// double as its (high float, low float) pair, 48 significant bits, with all-ones standing for "not
+// there yet".  Value and presence arrive together, so no fence is needed (a release fence would first
+// push everything the compute unit's cache holds out to memory).  The last block to leave a channel
+// puts its words back to all-ones, so a launch -- or a replay of a recorded launch -- always starts
+// from "nothing there".
+//
+// The wait is safe because partners have consecutive block ids (workgroups are dispatched in id order,
+// so a waiting block only ever waits for blocks that are already resident or next in line, and a
+// cluster needs at most kMaxCluster of the machine's CUs), and it is bounded: a block that gives up
+// raises `error`, finishes with whatever it found and exits; the host reports the error at the next
+// synchronisation point and re-initialises the words.
+constexpr unsigned kMaxCluster = 16;
+constexpr unsigned kClusterRecs = 16384;      // records (channel x piece) one launch may use
+constexpr unsigned kClusterChannels = 16384;
+constexpr unsigned long long kAbsent = ~0ull;
+
+struct ClusterMem {
+    unsigned long long *rec;   // [C * S][4]: centre, m2, g1, g2 of a piece
+    unsigned long long *sdx;   // [C * S]: per-piece sums of dx, each one word {1, float bits}; 0 = not there yet
+    unsigned *depart;          // [C]
+    int *error;
+};
+static __device__ __align__(256) unsigned long long g_cl_rec[kClusterRecs * 4];
+static __device__ __align__(256) unsigned long long g_cl_sdx[kClusterRecs];
+static __device__ __align__(256) unsigned g_cl_depart[kClusterChannels];
+static __device__ int g_cl_error;
+
+__device__ inline unsigned long long pack_double(double d)
+{
+    float hi = (float)d;
+    float lo = (float)(d - (double)hi);
+    unsigned h = __float_as_uint(hi), l = __float_as_uint(lo);
+    if (hi != hi) { h = 0x7fc00000u; l = 0u; }     // any NaN travels as the canonical one: never as "absent"
+    return ((unsigned long long)h << 32) | l;
+}
+__device__ inline double unpack_double(unsigned long long w)
+{
+    return (double)__uint_as_float((unsigned)(w >> 32)) + (double)__uint_as_float((unsigned)w);
+}
+
+template <bool kGrad>
+__global__ __launch_bounds__(1024) void bn_cluster_k(unsigned N, unsigned C, unsigned inner4, unsigned S, unsigned per,
+                                                      double factor, double eps, const float *x, const float *dy,
+                                                      const float *scale, const float *bias, const float *run_mean,
+                                                      const float *run_var, const float *ymask, int relu, float *out,
+                                                      float *out1, float *out2, float *dx_sum, ClusterMem cm,
+                                                      unsigned spin_limit)
+{
+    constexpr int kQ = kResQuads;
+    __shared__ float part[3][16];
+    __shared__ double comb[4];
+    const unsigned c = blockIdx.x / S, piece = blockIdx.x - c * S, T = blockDim.x, E4 = N * inner4;
+    const unsigned q0 = piece * per;                                  // this block's quads: [q0, q0 + mine)
+    const unsigned mine = E4 - q0 < per ? E4 - q0 : per;
+    const float4 *x4 = (const float4 *)x, *g4 = (const float4 *)dy;
+    float4 xv[kQ], gv[kQ];
+    unsigned idx[kQ];
+#pragma unroll
+    for (int i = 0; i < kQ; i++) {
+        const unsigned l = i * T + threadIdx.x;
+        const unsigned q = q0 + l;
+        const unsigned n = q / inner4, r = q - n * inner4;
+        idx[i] = l < mine ? (n * C + c) * inner4 + r : 0xffffffffu;
+        xv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        gv[i] = xv[i];
+        if (l < mine) {
+            xv[i] = x4[idx[i]];
+            if (kGrad) {
+                gv[i] = g4[idx[i]];
+                if (ymask) gv[i] = masked4(gv[i], ((const float4 *)ymask)[idx[i]]);
+            }
+        }
+    }
+    // the piece's own statistics: exact two-pass, as in the one-block kernel
+    const double nb = 4.0 * (double)mine;
+    double red1[1];
+    {
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < kQ; i++) sum += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);
+        const float in1[1] = {sum};
+        block_allsum<1>(in1, red1, part);
+    }
+    const double mu = red1[0] / nb;
+    const float mu_hi = (float)mu, mu_lo = (float)(mu - (double)mu_hi);
+    double red3[3];
+    {
+        float ss = 0.f, g1 = 0.f, g2 = 0.f;
+#pragma unroll
+        for (int i = 0; i < kQ; i++) {
+            if (idx[i] == 0xffffffffu) continue;
+            const float d0 = (xv[i].x - mu_hi) - mu_lo, d1 = (xv[i].y - mu_hi) - mu_lo;
+            const float d2 = (xv[i].z - mu_hi) - mu_lo, d3 = (xv[i].w - mu_hi) - mu_lo;
+            ss += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+            if (kGrad) {
+                g1 += (gv[i].x + gv[i].y) + (gv[i].z + gv[i].w);
+                g2 += (gv[i].x * d0 + gv[i].y * d1) + (gv[i].z * d2 + gv[i].w * d3);
+            }
+        }
+        const float in3[3] = {ss, g1, g2};
+        block_allsum<3>(in3, red3, part);
+    }
+    // publish, meet the partners, fold their records in block order.  The first word of a record is the
+    // mean the piece centred on (exactly the float pair it used), then its moments about that mean.
+    if (threadIdx.x < 4) {
+        const double centre = (double)mu_hi + (double)mu_lo;
+        const double mineVal = threadIdx.x == 0 ? centre : red3[threadIdx.x - 1];
+        __hip_atomic_store(cm.rec + (size_t)(c * S + piece) * 4 + threadIdx.x, pack_double(mineVal), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (threadIdx.x < 64) {
+        // lane l fetches word l of the channel's 4 * S (at most 64): all of them are polled side by side
+        const unsigned nwords = 4 * S;
+        unsigned long long w = 0;
+        if (threadIdx.x < nwords) {
+            w = kAbsent;
+            for (unsigned spin = 0; spin <= spin_limit; spin++) {
+                w = __hip_atomic_load(cm.rec + (size_t)c * S * 4 + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (w != kAbsent) break;
+                __builtin_amdgcn_s_sleep(2);
+            }
+            if (w == kAbsent) __hip_atomic_store(cm.error, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        const double val = unpack_double(w);
+        // every lane folds the same records in the same order
+        const double m = 4.0 * (double)E4;
+        double total = 0.0;
+        for (unsigned j = 0; j < S; j++) {
+            const unsigned qj = j * per;
+            const double nj = 4.0 * (double)(E4 - qj < per ? E4 - qj : per);
+            total += nj * __shfl(val, (int)(4 * j), 64);
+        }
+        const double mean = total / m;
+        double m2 = 0.0, g1 = 0.0, g2 = 0.0;
+        for (unsigned j = 0; j < S; j++) {
+            const unsigned qj = j * per;
+            const double nj = 4.0 * (double)(E4 - qj < per ? E4 - qj : per);
+            const double dm = __shfl(val, (int)(4 * j), 64) - mean;
+            const double rg1 = __shfl(val, (int)(4 * j + 2), 64);
+            m2 += __shfl(val, (int)(4 * j + 1), 64) + nj * dm * dm;
+            g1 += rg1;
+            g2 += __shfl(val, (int)(4 * j + 3), 64) + dm * rg1;
+        }
+        if (threadIdx.x == 0) {
+            comb[0] = mean;
+            comb[1] = m2;
+            comb[2] = g1;
+            comb[3] = g2;
+            // the last block to leave puts the channel's words back to "not there" for the next launch
+            const unsigned left = __hip_atomic_fetch_add(cm.depart + c, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (left == S - 1) {
+                for (unsigned k = 0; k < nwords; k++)
+                    __hip_atomic_store(cm.rec + (size_t)c * S * 4 + k, kAbsent, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(cm.depart + c, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    }
+    __syncthreads();
+    const double m = 4.0 * (double)E4;
+    const double mean = comb[0];
+    const float mean_hi = (float)mean, mean_lo = (float)(mean - (double)mean_hi);
+    const double var = comb[1] / m;  // biased
+    const double rstd = 1.0 / sqrt(var + eps);
+    float4 *o4 = (float4 *)out;
+    if (!kGrad) {
+        const float a = (float)((double)scale[c] * rstd), b = bias[c];
+#pragma unroll
+        for (int i = 0; i < kQ; i++) {
+            if (idx[i] == 0xffffffffu) continue;
+            float4 r;
+            r.x = a * ((xv[i].x - mean_hi) - mean_lo) + b;
+            r.y = a * ((xv[i].y - mean_hi) - mean_lo) + b;
+            r.z = a * ((xv[i].z - mean_hi) - mean_lo) + b;
+            r.w = a * ((xv[i].w - mean_hi) - mean_lo) + b;
+            if (relu) r = make_float4(relu1(r.x), relu1(r.y), relu1(r.z), relu1(r.w));
+            o4[idx[i]] = r;
+        }
+        if (threadIdx.x == 0 && piece == 0) {
+            const double unbiased = m > 1.0 ? var * m / (m - 1.0) : var;
+            out1[c] = (float)((1.0 - factor) * (double)run_mean[c] + factor * mean);
+            out2[c] = (float)((1.0 - factor) * (double)run_var[c] + factor * unbiased);
+        }
+    } else {
+        const double db = comb[2], ds = rstd * comb[3];  // sum dy, sum dy * xhat
+        CoefG k;
+        k.mean = mean_hi;
+        k.mean_lo = mean_lo;
+        k.rstd = (float)rstd;
+        k.a = (float)((double)scale[c] * rstd);
+        k.b = (float)(db / m);
+        k.d = (float)(ds / m);
+        float sdx = 0.f;
+#pragma unroll
+        for (int i = 0; i < kQ; i++) {
+            if (idx[i] == 0xffffffffu) continue;
+            const float4 r = make_float4(bn_dx(k, gv[i].x, xv[i].x), bn_dx(k, gv[i].y, xv[i].y),
+                                         bn_dx(k, gv[i].z, xv[i].z), bn_dx(k, gv[i].w, xv[i].w));
+            o4[idx[i]] = r;
+            sdx += (r.x + r.y) + (r.z + r.w);
+        }
+        if (threadIdx.x == 0 && piece == 0) {
+            out1[c] = (float)ds;
+            out2[c] = (float)db;
+        }
+        if (dx_sum) {
+            // Per-channel sum of dx: piece 0 adds the pieces' sums in piece order.  A piece's sum travels as ONE
+            // 64-bit word {1, float bits} written and read with device-scope atomics: value and "it is there"
+            // arrive together, so no fence has to push the 128 KB of dx this block has just stored out of the
+            // cache first.  Piece 0 puts the words back to 0 for the next launch.
+            const float in1[1] = {sdx};
+            double red[1];
+            block_allsum<1>(in1, red, part);
+            if (threadIdx.x == 0) {
+                const unsigned long long word = (1ull << 32) | (unsigned long long)__float_as_uint((float)red[0]);
+                __hip_atomic_store(cm.sdx + c * S + piece, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (piece == 0) {
+                    double t = 0.0;
+                    for (unsigned j = 0; j < S; j++) {
+                        unsigned long long w = 0;
+                        for (unsigned spin = 0; spin <= spin_limit; spin++) {
+                            w = __hip_atomic_load(cm.sdx + c * S + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            if (w >> 32) break;
+                            __builtin_amdgcn_s_sleep(4);
+                        }
+                        if (!(w >> 32)) __hip_atomic_store(cm.error, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        t += (double)__uint_as_float((unsigned)w);
+                        __hip_atomic_store(cm.sdx + c * S + j, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                    dx_sum[c] = (float)t;
+                }
+            }
+        }
+    }
+}
+
+// Host side of the cluster path: the device addresses of its records and counters (taken once per
+// device), whether a launch is outstanding whose error flag has not been read, and the spin limit.
+ClusterMem g_cluster_mem[64];
+bool g_cluster_ready[64];
+bool g_cluster_unchecked = false;
+unsigned g_cluster_spin_limit = 1u << 21;   // polls of ~1 us each before a block gives up
+
+int cluster_mem(ClusterMem *out)
+{
+    int dev = -1;
+    DOPT_HIP_CHECK(hipGetDevice(&dev));
+    DOPT_REQUIRE(dev >= 0 && dev < 64, "batch norm: device index %d out of range", dev);
+    if (!g_cluster_ready[dev]) {
+        ClusterMem m;
+        DOPT_HIP_CHECK(hipGetSymbolAddress((void **)&m.rec, HIP_SYMBOL(g_cl_rec)));
+        DOPT_HIP_CHECK(hipGetSymbolAddress((void **)&m.sdx, HIP_SYMBOL(g_cl_sdx)));
+        DOPT_HIP_CHECK(hipGetSymbolAddress((void **)&m.depart, HIP_SYMBOL(g_cl_depart)));
+        DOPT_HIP_CHECK(hipGetSymbolAddress((void **)&m.error, HIP_SYMBOL(g_cl_error)));
+        // "nothing there" is all-ones (the loader zero-fills); once per device, before the first launch
+        DOPT_HIP_CHECK(hipMemset(m.rec, 0xff, sizeof(unsigned long long) * kClusterRecs * 4));
+        DOPT_HIP_CHECK(hipDeviceSynchronize());
+        g_cluster_mem[dev] = m;
+        g_cluster_ready[dev] = true;
+    }
+    *out = g_cluster_mem[dev];
+    return DOPT_HIP_OK;
+}
+
+// Pieces per channel for the cluster path and quads per piece, or 0 when the tensor does not take it.
+// (Channels that fit one block stay there even when they are too few to give every compute unit a
+// block: 128 channels of 32768 values as 256 half-channel blocks measured 16.5 against 11.6 us.)
+unsigned cluster_pieces(size_t N, size_t C, size_t inner, const void *a, const void *b, const void *m, const void *o,
+                        unsigned *per)
+{
+    if ((inner & 3) != 0 || !aligned16(a) || (b && !aligned16(b)) || (m && !aligned16(m)) || !aligned16(o)) return 0;
+    const size_t E4 = N * (inner / 4), cap = (size_t)kResQuads * 1024;
+    if (E4 <= cap || E4 > cap * kMaxCluster || N * C * (inner / 4) >= 0xffffffffull) return 0;
+    const size_t S = ceil_div(E4, cap);
+    if (C > kClusterChannels || C * S > kClusterRecs) return 0;
+    *per = (unsigned)ceil_div(E4, S);          // balanced pieces
+    return (unsigned)S;
+}
+
 // Threads for the resident path, or 0 when the channel does not fit (or is not 128-bit addressable).
 unsigned resident_threads(size_t N, size_t C, size_t inner, const void *a, const void *b, const void *o)
 {
@@ -629,6 +920,18 @@ int bn_train_impl(size_t N, size_t C, size_t inner, double momentum, const float
         }
         if (int rc = dopt_hip_split_sum_close(x_open)) return rc;
     }
+    unsigned per = 0;
+    if (const unsigned S = cluster_pieces(N, C, inner, x, nullptr, nullptr, packed, &per)) {
+        ClusterMem cm;
+        if (int rc = cluster_mem(&cm)) return rc;
+        hipLaunchKernelGGL((bn_cluster_k<false>), dim3((unsigned)(C * S)), dim3(1024), 0, stream(), (unsigned)N, (unsigned)C,
+                           (unsigned)(inner / 4), S, per, factor, eps, x, (const float *)nullptr, scale, bias, run_mean,
+                           run_var, (const float *)nullptr, relu, packed, packed + total, packed + total + C,
+                           (float *)nullptr, cm, g_cluster_spin_limit);
+        DOPT_LAUNCH_CHECK();
+        g_cluster_unchecked = true;
+        return DOPT_HIP_OK;
+    }
     if (T) {
         // small channels (two quads per thread) take the variant built for two: a third of the registers
         if (N * (inner / 4) <= (size_t)kOpenQuads * T)
@@ -682,6 +985,18 @@ int bn_grad_impl(size_t N, size_t C, size_t inner, const float *dy, const float 
         }
         if (int rc = dopt_hip_split_sum_close(dy_open)) return rc;
     }
+    unsigned per = 0;
+    if (const unsigned S = cluster_pieces(N, C, inner, x, dy, ymask, packed, &per)) {
+        ClusterMem cm;
+        if (int rc = cluster_mem(&cm)) return rc;
+        hipLaunchKernelGGL((bn_cluster_k<true>), dim3((unsigned)(C * S)), dim3(1024), 0, stream(), (unsigned)N, (unsigned)C,
+                           (unsigned)(inner / 4), S, per, 0.0, eps, x, dy, scale, (const float *)nullptr,
+                           (const float *)nullptr, (const float *)nullptr, ymask, 0, packed, packed + total,
+                           packed + total + C, dx_sum, cm, g_cluster_spin_limit);
+        DOPT_LAUNCH_CHECK();
+        g_cluster_unchecked = true;
+        return DOPT_HIP_OK;
+    }
     if (T) {
         if (N * (inner / 4) <= (size_t)kOpenQuads * T)
             hipLaunchKernelGGL((bn_resident_k<true, false, kOpenQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N,
@@ -730,6 +1045,31 @@ int bn_grad_impl(size_t N, size_t C, size_t inner, const float *dy, const float 
 }
 
 }  // namespace
+
+namespace dopt {
+
+// Called by the library's synchronisation points once the queues are idle: reports a cluster kernel
+// whose blocks gave up waiting for each other, and puts the counters back to zero.
+int bn_cluster_poll()
+{
+    if (!g_cluster_unchecked) return DOPT_HIP_OK;
+    g_cluster_unchecked = false;
+    ClusterMem cm;
+    if (int rc = cluster_mem(&cm)) return rc;
+    int err = 0;
+    DOPT_HIP_CHECK(hipMemcpy(&err, cm.error, sizeof(int), hipMemcpyDeviceToHost));
+    if (!err) return DOPT_HIP_OK;
+    DOPT_HIP_CHECK(hipMemset(cm.error, 0, sizeof(int)));
+    DOPT_HIP_CHECK(hipMemset(cm.rec, 0xff, sizeof(unsigned long long) * kClusterRecs * 4));
+    DOPT_HIP_CHECK(hipMemset(cm.depart, 0, kClusterChannels * sizeof(unsigned)));
+    DOPT_HIP_CHECK(hipMemset(cm.sdx, 0, kClusterRecs * sizeof(unsigned long long)));
+    return fail(DOPT_HIP_ERR_RUNTIME, "batch norm: blocks sharing a channel did not meet within the wait limit; the "
+                                      "results of batch-norm calls since the last synchronisation are invalid");
+}
+
+void bn_cluster_set_spin_limit(unsigned polls) { g_cluster_spin_limit = polls; }
+
+}  // namespace dopt
 
 extern "C" {
 

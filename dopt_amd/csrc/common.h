@@ -52,6 +52,8 @@ bool conv_smallc_takes(const dopt_hip_conv_desc *d);
 int conv_smallc_fwd(const dopt_hip_conv_desc *d, const float *x, const float *w, const float *bias, float *y, bool *done);
 int conv_smallc_wgrad(const dopt_hip_conv_desc *d, const float *dy, const float *x, float *dw, bool *done);
 hipStream_t lane_stream(int lane);
+// bn.hip: error report of the multi-block batch-norm kernels; call with the queues idle.
+int bn_cluster_poll();
 
 // Number of compute units of the active device (256 on MI355X); used to size grids.
 int num_cus();

@@ -418,7 +418,7 @@ int dopt_hip_copy_d2h(void *host_dst, const void *src, size_t bytes)
     DOPT_ENSURE_INIT();
     DOPT_HIP_CHECK(hipMemcpyAsync(host_dst, src, bytes, hipMemcpyDeviceToHost, stream()));
     DOPT_HIP_CHECK(hipStreamSynchronize(stream()));
-    return DOPT_HIP_OK;
+    return bn_cluster_poll();
 }
 
 int dopt_hip_copy_d2d(void *dst, const void *src, size_t bytes)
@@ -435,7 +435,7 @@ int dopt_hip_sync(void)
     DOPT_ENSURE_INIT();
     DOPT_HIP_CHECK(hipStreamSynchronize(lane_stream(0)));
     DOPT_HIP_CHECK(hipStreamSynchronize(lane_stream(1)));   // idle unless a plan is overlapping work
-    return DOPT_HIP_OK;
+    return bn_cluster_poll();
 }
 
 void *dopt_hip_stream(void) { return ensure_init() ? (void *)stream() : nullptr; }

@@ -470,6 +470,53 @@ def test_batchnorm_train_grad_infer(shape):
                  "bn infer")
 
 
+@pytest.mark.parametrize("shape", [(128, 64, 32, 32),    # the benchmark's largest channel: four blocks share one
+                                   (130, 3, 32, 32),     # ragged pieces
+                                   (33, 5, 16, 64),      # two pieces, the second much shorter than a full block
+                                   (512, 2, 32, 32),     # the most blocks one channel may span
+                                   (520, 1, 32, 32)])    # beyond that: the three-launch path
+def test_batchnorm_channels_spanning_several_blocks(shape):
+    """Channels of more than 32768 values: their statistics are combined across blocks.  Same checks as
+    above plus the fused forms (ReLU on the way out, ReLU mask on the way in, per-channel sum of dx)."""
+    import ctypes as C_
+    from dopt_amd import capi
+    lib = capi.load()
+    r = rng(63)
+    N, C = shape[:2]
+    inner = shape[2] * shape[3]
+    x = (r.standard_normal(shape) * 1.5 + 2).astype(np.float32)
+    gamma, beta, rm = (r.standard_normal(C).astype(np.float32) for _ in range(3))
+    rv = (r.random(C) + 0.5).astype(np.float32)
+    vol, m = x.size, x.size // C
+    dy = (r.standard_normal(shape) / m).astype(np.float32)
+    mom = float(np.float32(0.9))
+    tx, tg, tb, trm, trv, tdy = T(x), T(gamma), T(beta), T(rm), T(rv), T(dy)
+    got = ops.bn_train(tx, tg, tb, trm, trv, mom).numpy()
+    want = O.bn_train(x, gamma, beta, rm, rv, mom)
+    assert_close(got[:vol], want[:vol], "bn y")
+    assert_close(got[vol:], want[vol:], "bn running stats")
+    fused = ops.bn_train_relu(tx, tg, tb, trm, trv, mom)
+    assert np.array_equal(fused.numpy()[:vol], np.maximum(got[:vol], 0))
+    assert np.array_equal(fused.numpy()[vol:], got[vol:])
+    g = ops.bn_grad(tdy, tx, tg).numpy()
+    gw = O.bn_grad(dy, x, gamma)
+    assert_close(g[:vol], gw[:vol], "bn dx")
+    assert_close(g[vol:], gw[vol:], "bn dscale/dbias")
+    # relu mask on the way in, sum of dx on the way out
+    y = fused.view(0, shape)
+    packed, dxs = ops.Tensor((vol + 2 * C,)), ops.Tensor((C,))
+    capi.check(lib.dopt_hip_bn_grad_fused(N, C, inner, tdy.ptr, y.ptr, tx.ptr, tg.ptr, packed.ptr, dxs.ptr))
+    masked = O.relu_grad(dy, y.numpy())
+    gw = O.bn_grad(masked, x, gamma)
+    assert_close(packed.numpy()[:vol], gw[:vol], "bn dx behind a relu")
+    assert_close(packed.numpy()[vol:], gw[vol:], "bn dscale/dbias behind a relu")
+    assert_close(dxs.numpy(), O.add_bias_grad(packed.numpy()[:vol].reshape(shape)), "sum of dx")
+    # twice the same call: the counters the blocks meet at are back at zero after every launch
+    again = ops.bn_train(tx, tg, tb, trm, trv, mom).numpy()
+    assert np.array_equal(again, got)
+    ops.sync()
+
+
 def test_batchnorm_large_mean_small_variance():
     # E[x^2] - E[x]^2 would lose everything here; the shifted moments must not
     r = rng(62)
