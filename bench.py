@@ -3,17 +3,24 @@
 CIFAR-shape network with batch norm at batch 128 in fp32, on one MI355X, through HIPPlan and the
 kernel library.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--unfused] [--no-views] [--no-fuse] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config N] [--unfused] [--no-views] [--no-fuse]
+                    [--graph] [--no-cpu] [--no-kernel-timing]
 
-A step is one execution of the update plan on device-resident synthetic inputs (inputs are in
-HBM before the timed region starts).  After the timed region the same step is run again with
-per-kernel HIP events (on the library's stream) to measure the convolution kernels against the
-fp32 MFMA roofline, and the reference's CPU convolution (this repository's C restatement of it)
-is timed on the host cores as the reported CPU baseline.
+A step is one execution of the update plan on device-resident synthetic inputs (inputs are in HBM
+before the timed region starts).  W warm-up steps, then EXACTLY K timed steps between two device
+synchronisations give `value`; four more windows of K steps give the median and the spread reported
+beside it.  After the timed region the same step is run again with per-kernel HIP events (on the
+library's stream, where the kernels are launched) to measure the dominant convolution kernel against
+the fp32 MFMA roofline, and the reference's CPU path (this repository's C restatement of it) is timed
+on the host cores as the reported CPU baseline.
+
+--config 1|2|3|5 times one of the other configurations instead (a secondary line: they are parity
+cases, not the headline); --config 4 is the default.
 """
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -26,52 +33,53 @@ BATCH = 128
 MFMA_FP32_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBS = 8000.0
 
-# (C, K, H) of the 13 VGG-16 3x3 pad-1 convolutions on a 32x32 input
-VGG_CONVS = [(3, 64, 32), (64, 64, 32), (64, 128, 16), (128, 128, 16), (128, 256, 8), (256, 256, 8), (256, 256, 8),
-             (256, 512, 4), (512, 512, 4), (512, 512, 4), (512, 512, 2), (512, 512, 2), (512, 512, 2)]
+
+def timed_windows(step, steps, warmup, windows=5):
+    """W warm-up steps, then `windows` windows of exactly `steps` steps, each between two device
+    synchronisations.  Returns seconds per window; the first is the official one."""
+    from dopt_amd import ops
+    step.run(warmup)
+    ops.sync()
+    out = []
+    for _ in range(windows):
+        t0 = time.perf_counter()
+        step.run(steps)
+        ops.sync()
+        out.append(time.perf_counter() - t0)
+    return out
 
 
-def conv_flops(n, c, k, h):
-    return 2.0 * n * k * c * 9 * h * h
+def window_stats(win, steps):
+    ms = [w / steps * 1e3 for w in win]
+    return {"windows_ms_per_step": [round(m, 4) for m in ms], "median_ms_per_step": round(statistics.median(ms), 4),
+            "spread_ms_per_step": round(max(ms) - min(ms), 4)}
 
 
-def build_step(batch, fused, views, timing, seed=0, fuse=True, overlap=False, graph=False):
-    from dopt_amd import core, nnet, online, ops
-    rng = np.random.default_rng(seed)
-    features = core.float32([batch, 3, 32, 32])
-    labels = core.float32([batch, 10])
-    init = nnet.Init(seed + 1)
-    preds = nnet.softmax(nnet.dense(nnet.vgg16(features, [512, 512], init), 10, init))
-    net = nnet.DAGNetwork([features], [preds])
-    loss = nnet.crossEntropy(preds.trainOutput, labels) + net.paramLoss
-    flags = (core.PLAN_VIEWS if views else 0) | (core.PLAN_TIMING if timing else 0)
-    flags |= core.PLAN_FUSE if (fuse and views) else 0
-    flags |= core.PLAN_OVERLAP if overlap is True else 0
-    flags |= core.PLAN_OVERLAP_LIGHT if overlap == "light" else 0
-    flags |= core.PLAN_GRAPH if (graph and not timing) else 0
-    if fused:
-        updater = online.fused_sgd([loss, preds.trainOutput], net.params, net.paramProj, 0.01, 0.0, flags=flags)
-    else:
-        updater = online.sgd([loss, preds.trainOutput], net.params, net.paramProj, flags=flags)
-    x = rng.standard_normal((batch, 3, 32, 32)).astype(np.float32)
-    y = np.zeros((batch, 10), np.float32)
-    y[np.arange(batch), rng.integers(0, 10, batch)] = 1.0
-    args = {features: ops.tensor(x), labels: ops.tensor(y)}   # resident in HBM before timing starts
-    return updater, args, net
+def host_cores():
+    try:
+        return len(os.sched_getaffinity(0))
+    except AttributeError:
+        return os.cpu_count() or 1
 
 
 def cpu_baseline(seconds_budget=20.0):
-    """The reference's CPU convolution kernel (cpu/source/dopt/cpu/nnet.d:20-87, single-threaded
-    direct loops; the reference CPU backend has no backward or batch-norm kernels at all) over the
-    13 VGG layers at a small batch, expressed as images/s of conv-forward alone."""
+    """The reference's CPU path on the host cores (C restatement, `kind: port`):
+      * the headline figure: its convolution kernel (cpu/source/dopt/cpu/nnet.d:20-87, single-threaded
+        direct loops) over the 13 VGG layers at a small batch, as images/s of conv-forward alone -- the
+        reference CPU backend has no backward, bias, ReLU or batch-norm kernels, so a CPU training step of
+        the benchmark network does not exist;
+      * configuration 1 (the one network the reference CPU backend can train end to end): whole training
+        steps through the CPU evaluator, operation by operation in the reference's order."""
     import oracle as O
+    from oracle import evaluator
+    from dopt_amd import configs
     rng = np.random.default_rng(0)
     b = 1
     t_total = 0.0
     # calibrate on batch 1, then spend the remaining budget on one larger batch
     for attempt in range(2):
         t0 = time.perf_counter()
-        for (c, k, h) in VGG_CONVS:
+        for (c, k, h) in configs.VGG_CONVS:
             x = rng.standard_normal((b, c, h, h)).astype(np.float32)
             w = rng.standard_normal((k, c, 3, 3)).astype(np.float32)
             O.convolution(x, w, (1, 1), (1, 1), f64=False)
@@ -81,11 +89,59 @@ def cpu_baseline(seconds_budget=20.0):
             if nb == b:
                 break
             b = nb
-    return {"value": round(b / t_total, 3), "unit": "images/s", "cores": 1, "kind": "port",
+    # configuration 1 on the CPU evaluator: graph outputs = loss, predictions, new W, new b, new momenta
+    s1 = configs.softmax_regression(flags=0, host_args=True)
+    outs = s1.updater.plan.outputs
+    evaluator.evaluate(outs, s1.args)
+    n1, t0 = 0, time.perf_counter()
+    while n1 < 3 or (time.perf_counter() - t0 < 2.0 and n1 < 200):
+        evaluator.evaluate(outs, s1.args)
+        n1 += 1
+    cfg1_ms = (time.perf_counter() - t0) / n1 * 1e3
+    return {"value": round(b / t_total, 3), "unit": "images/s", "cores": 1, "host_cores": host_cores(), "kind": "port",
             "sample": "conv-forward only: the 13 VGG-16 3x3 convolutions at batch %d through the C restatement of "
                       "the reference's single-threaded CPU kernel (%.1f s); the reference CPU backend implements no "
                       "backward, bias, ReLU or batch-norm kernels, so a full CPU training step does not exist" % (
-                          b, t_total)}
+                          b, t_total),
+            "config1_step_ms": round(cfg1_ms, 3),
+            "config1_sample": "%d whole softmax-regression steps ([100,784] -> 10, forward + backward + SGD) through the "
+                              "CPU evaluator, one restated reference kernel per operation, 1 thread" % n1}
+
+
+def secondary(cfg, a):
+    """One of the other configurations: a secondary JSON line."""
+    from dopt_amd import configs, core
+    flags = configs.REWRITES | (core.PLAN_GRAPH if a.graph else 0)
+    if cfg == 1:
+        step = configs.softmax_regression(flags=flags)
+    elif cfg == 2:
+        step = configs.mlp(fused=not a.unfused, flags=flags)
+    elif cfg == 3:
+        step = configs.fused_update("amsgrad" if a.unfused else "adam")
+    else:
+        step = configs.wide_resnet(BATCH, fused=not a.unfused, flags=flags)
+    steps = a.steps if cfg != 5 else max(3, min(a.steps, 10))
+    win = timed_windows(step, steps, a.warmup)
+    sec = win[0] / steps
+    res = {"metric": "secondary: training steps/sec of %s" % step.name, "value": round(1.0 / sec, 2), "unit": "steps/s",
+           "n_gpus": 1, "steps": steps, "warmup": a.warmup, "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": step.name, "plan_rewrites": "views+fuse" + ("+graph" if a.graph else "")}}
+    res.update(window_stats(win, steps))
+    if cfg == 3:
+        res["roofline"] = {"kernel": "optim_k (fused multi-tensor update)", "bound": "hbm",
+                           "achieved": round(step.extra["bytes_per_step"] / sec / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": round(step.extra["bytes_per_step"] / sec / 1e9 / HBM_PEAK_GBS, 4), "traffic": None}
+    else:
+        res["config"]["kernels_per_step"] = step.kernels()
+        res["config"]["loss_after"] = round(step.loss_value(), 5)
+    if cfg in (1, 2, 5):
+        res["images_per_s"] = round(step.batch / sec, 1)
+    if cfg == 5:
+        fl = 3.0 * configs.wrn_conv_flops(BATCH)
+        res["conv_TFLOPs"] = round(fl / sec / 1e12, 2)
+        res["conv_flops_per_step"] = fl
+    print(json.dumps(res))
 
 
 def main():
@@ -93,7 +149,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--unfused", action="store_true", help="run the reference's op-graph SGD instead of the fused kernel")
+    ap.add_argument("--config", type=int, default=4, choices=[1, 2, 3, 4, 5])
+    ap.add_argument("--unfused", action="store_true", help="run the reference's op-graph optimizer instead of the fused kernel")
     ap.add_argument("--no-views", action="store_true", help="disable the copy-eliding plan rewrites")
     ap.add_argument("--no-fuse", action="store_true", help="run every operation as its own kernel")
     ap.add_argument("--overlap", action="store_true", help="run the filter gradients on a second queue")
@@ -106,22 +163,26 @@ def main():
     if a.gpus != 1:
         sys.exit("bench.py: this build drives one GPU per process and implements no collectives; run with --gpus 1")
 
-    from dopt_amd import capi, ops
+    from dopt_amd import capi, configs, core, ops
     capi.check(capi.load().dopt_hip_init(0))
+    if a.config != 4:
+        return secondary(a.config, a)
     fused, views, fuse = not a.unfused, not a.no_views, not a.no_fuse
 
-    updater, args, net = build_step(BATCH, fused, views, timing=False, fuse=fuse, overlap=("light" if a.overlap_light else a.overlap), graph=a.graph)
-    for _ in range(a.warmup):
-        updater.step_async(args)
-    ops.sync()
-    t0 = time.perf_counter()
-    for _ in range(a.steps):
-        updater.step_async(args)
-    ops.sync()
-    elapsed = time.perf_counter() - t0
-    loss = float(updater._out_bufs[0].numpy())
+    def flags_for(timing):
+        f = (core.PLAN_VIEWS if views else 0) | (core.PLAN_FUSE if (fuse and views) else 0)
+        f |= (core.PLAN_TIMING | core.PLAN_TIMING_SHAPES) if timing else 0
+        f |= core.PLAN_OVERLAP if a.overlap else 0
+        f |= core.PLAN_OVERLAP_LIGHT if a.overlap_light else 0
+        f |= core.PLAN_GRAPH if (a.graph and not timing) else 0
+        return f
+
+    step = configs.vgg16(BATCH, fused, flags_for(False))
+    win = timed_windows(step, a.steps, a.warmup)
+    elapsed = win[0]
+    loss = step.loss_value()
     ms_per_step = elapsed / a.steps * 1e3
-    stats = updater.plan.stats()
+    stats = step.updater.plan.stats()
 
     result = {
         "metric": "train images/sec, VGG-16 CIFAR-shape fp32 b128",
@@ -131,75 +192,101 @@ def main():
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "config 4: VGG-16 + batch norm, input [128,3,32,32], FC 512-512-10, softmax "
-                               "cross-entropy, one forward + backward + SGD(lr 0.01) step",
+        "config": {"workload": step.name,
                    "global_batch": BATCH, "optimizer": "fused multi-tensor SGD" if fused else "op-graph SGD",
                    "plan_rewrites": ("views+fuse" if fuse else "views") if views else "none",
                    "kernels_per_step": stats["kernels"] + (1 if fused else 0),
                    "plan_buffer_MB": round(stats["buffer_bytes"] / 2**20, 1),
-                   "parameters": int(sum(p.volume for p in net.params)), "loss_after": round(loss, 5)},
+                   "parameters": int(sum(p.volume for p in step.params)), "loss_after": round(loss, 5)},
     }
+    result.update(window_stats(win, a.steps))
     if not np.isfinite(loss):
         sys.exit("bench.py: the loss is not finite (%r)" % loss)
 
     if not a.no_kernel_timing:
-        # Same step, every kernel object bracketed by hipEvents on the library stream.
-        del updater
-        tup, targs, _ = build_step(BATCH, fused, views, timing=True, fuse=fuse, overlap=("light" if a.overlap_light else a.overlap))
-        for _ in range(2):
-            tup.step_async(targs)
+        # Same step, every kernel object bracketed by hipEvents on the library stream, keyed by operation
+        # type and output shape.
+        del step
+        tstep = configs.vgg16(BATCH, fused, flags_for(True))
+        tstep.run(2)
         ops.sync()
-        before = tup.plan.profile()
+        before = tstep.updater.plan.profile()
         nsteps = max(3, min(a.steps, 10))
-        for _ in range(nsteps):
-            tup.step_async(targs)
+        tstep.run(nsteps)
         ops.sync()
-        after = tup.plan.profile()
-        per_step = {k: ((after[k][0] - before.get(k, (0, 0))[0]) / nsteps, (after[k][1] - before.get(k, (0, 0))[1]) // nsteps)
-                    for k in after}
-        fwd = sum(conv_flops(BATCH, c, k, h) for c, k, h in VGG_CONVS)
-        bwd_data = fwd - conv_flops(BATCH, *VGG_CONVS[0])   # the first layer's input needs no gradient
-        conv_keys = [k for k in ("convolution", "convolution+addBias", "convolutionFeaturesGrad") if k in per_step]
-        # the one launch that packs every filter of the step belongs to these convolutions' cost
-        gather_us = sum(per_step[k][0] for k in conv_keys) + per_step.get("filterPack", (0.0, 0))[0]
-        gather_launches = sum(per_step[k][1] for k in conv_keys)
-        gather_tflops = (fwd + bwd_data) / (gather_us * 1e-6) / 1e12
-        wgrad_tflops = fwd / (per_step["convolutionFiltersGrad"][0] * 1e-6) / 1e12
-        # HBM bytes per launch of the same kernel, as measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-        # (calibrated against a plain copy); the summary of those runs is kept under profiles/
+        after = tstep.updater.plan.profile()
+        per_shape = {k: ((after[k][0] - before.get(k, (0, 0))[0]) / nsteps, (after[k][1] - before.get(k, (0, 0))[1]) // nsteps)
+                     for k in after}
+        per_op = {}
+        for k, (us, n) in per_shape.items():
+            name = k.split("@")[0]
+            per_op[name] = (per_op.get(name, (0.0, 0))[0] + us, per_op.get(name, (0.0, 0))[1] + n)
+
+        # The dominant kernel: conv_patch_k with 128 x 128 tiles = every 3x3 convolution whose GEMM has at
+        # least 128 rows (output channels forward, input channels backward-data) on images of 4x4 pixels and
+        # more: forward layers 3-10 and backward-data layers 4-10, 15 launches per step.  Its steps hold
+        # nothing else (filters are packed by a step of their own; where a reduction is split the partial sums
+        # are added by the batch norm behind it), and the kernel multiplies every tap of every pixel, padding
+        # included, so the conventional FLOP count below is also the executed one.
+        flops = us = launches = bytes_alg = 0
+        for i, (c, k, h) in enumerate(configs.VGG_CONVS):
+            if h < 4:
+                continue
+            fl = configs.conv_flops(BATCH, c, k, h)
+            by = 4 * (BATCH * c * h * h + BATCH * k * h * h + k * c * 9)     # input, output and filter once
+            fwd_keys = [n for n in ("convolution+addBias", "convolution") if "%s@%dx%dx%dx%d" % (n, BATCH, k, h, h) in per_shape]
+            if k >= 128 and fwd_keys:
+                # forward layers sharing an output shape share a key: charge each layer its share
+                same = sum(1 for (c2, k2, h2) in configs.VGG_CONVS if (k2, h2) == (k, h))
+                t, n = per_shape["%s@%dx%dx%dx%d" % (fwd_keys[0], BATCH, k, h, h)]
+                flops, us, launches, bytes_alg = flops + fl, us + t / same, launches + 1, bytes_alg + by
+            bkey = "convolutionFeaturesGrad@%dx%dx%dx%d" % (BATCH, c, h, h)
+            if i > 0 and c >= 128 and bkey in per_shape:
+                same = sum(1 for j, (c2, k2, h2) in enumerate(configs.VGG_CONVS) if j > 0 and (c2, h2) == (c, h))
+                t, n = per_shape[bkey]
+                flops, us, launches, bytes_alg = flops + fl, us + t / same, launches + 1, bytes_alg + by
+        tflops = flops / (us * 1e-6) / 1e12 if us else 0.0
+        # HBM bytes per launch of the same kernel over the same launches, from the committed rocprofv3 --pmc
+        # summary (FETCH_SIZE / WRITE_SIZE calibrated against a plain copy): NOT measured in this run
         traffic = None
-        tpath = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "conv_kernels_vgg16_b128_hbm_traffic.txt")
+        tpath = os.path.join(ROOT, "profiles", "conv_kernels_vgg16_b128_hbm_traffic.txt")
         if os.path.exists(tpath):
             for line in open(tpath):
-                if line.startswith("traffic_bytes_per_launch conv_patch_k"):
+                if line.startswith("traffic_bytes_per_launch conv_patch_k_128x128"):
                     traffic = int(line.split()[-1])
-        conv_bytes = 0   # algorithmic: input and output once, filter once
-        for i, (c, k, h) in enumerate(VGG_CONVS):
-            one = 4 * (BATCH * c * h * h + BATCH * k * h * h + k * c * 9)
-            conv_bytes += one * (1 if i == 0 else 2)
         result["roofline"] = {
-            "kernel": "conv_patch_k (3x3 implicit-GEMM convolution forward + backward-data of all 13 layers as the plan runs "
-                      "them, incl. filter pack and the split reductions not taken over by the batch norm that follows; layer 1 and the "
-                      "2x2-image layers take their own kernels)",
-            "bound": "mfma", "achieved": round(gather_tflops, 2), "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(gather_tflops / MFMA_FP32_PEAK_TFLOPS, 4), "traffic": traffic,
-            "traffic_of": "conv_patch_k launches only (layers 2-10, 18 of the 25; 25.1 MB algorithmic per launch); the "
-                          "first layer and the 2x2-image layers run other kernels, listed in the same profile",
-            "algorithmic_bytes_per_launch": int(conv_bytes / gather_launches),
-            "launches_per_step": int(gather_launches),
-            "flops_per_launch": round((fwd + bwd_data) / gather_launches, 1),
-            "flops_convention": "2*N*K*C*R*S*P*Q per convolution, taps that fall on zero padding included; the six "
-                                "launches on 2x2 images (9 % of these FLOPs) execute 4/9 of that count as a dense product",
-            "avg_launch_us": round(gather_us / gather_launches, 2),
+            "kernel": "conv_patch_k<Tile<128,128,2,4>,16,true>: 3x3 implicit-GEMM convolution, forward of layers 3-10 and "
+                      "backward-data of layers 4-10 of the 13 (the other layers run the 64x256-tile variant, the first-layer "
+                      "kernels and the dense 2x2-image route, listed under `kernels`)",
+            "bound": "mfma", "achieved": round(tflops, 2), "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(tflops / MFMA_FP32_PEAK_TFLOPS, 4), "traffic": traffic,
+            "traffic_source": "profiles/conv_kernels_vgg16_b128_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of "
+                              "the same %d launches per step; taken from that file, not measured in this run)" % launches,
+            "algorithmic_bytes_per_launch": int(bytes_alg / launches) if launches else None,
+            "launches_per_step": int(launches),
+            "flops_per_launch": round(flops / launches, 1) if launches else None,
+            "flops_convention": "2*N*K*C*R*S*P*Q per launch = what the kernel executes (it multiplies the taps that fall on "
+                                "zero padding too)",
+            "avg_launch_us": round(us / launches, 2) if launches else None,
         }
+        fwd = sum(configs.conv_flops(BATCH, c, k, h) for c, k, h in configs.VGG_CONVS)
+        wgrad_us = per_op["convolutionFiltersGrad"][0]
+        allconv_us = sum(per_op[k][0] for k in ("convolution", "convolution+addBias", "convolutionFeaturesGrad") if k in per_op)
+        allconv_us += per_op.get("filterPack", (0.0, 0))[0]
+        bwd_data = fwd - configs.conv_flops(BATCH, *configs.VGG_CONVS[0])
         result["kernels"] = {
-            "conv_wgrad_k": {"achieved_TFLOPs": round(wgrad_tflops, 2),
-                             "frac_of_mfma_peak": round(wgrad_tflops / MFMA_FP32_PEAK_TFLOPS, 4),
-                             "us_per_step": round(per_step["convolutionFiltersGrad"][0], 1)},
-            "device_us_per_step_by_op": {k: round(v[0], 1) for k, v in sorted(per_step.items(), key=lambda kv: -kv[1][0])},
-            "device_us_per_step_total": round(sum(v[0] for v in per_step.values()), 1),
+            "conv_wgrad_patch_k (all 13 filter gradients incl. their split sums)": {
+                "achieved_TFLOPs": round(fwd / (wgrad_us * 1e-6) / 1e12, 2),
+                "frac_of_mfma_peak": round(fwd / (wgrad_us * 1e-6) / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
+                "us_per_step": round(wgrad_us, 1)},
+            "all forward + backward-data convolutions incl. filter packing (2x2-image layers counted at the conventional "
+            "9-tap FLOPs although their dense route executes 4/9 of them)": {
+                "achieved_TFLOPs": round((fwd + bwd_data) / (allconv_us * 1e-6) / 1e12, 2),
+                "us_per_step": round(allconv_us, 1)},
+            "device_us_per_step_by_op": {k: round(v[0], 1) for k, v in sorted(per_op.items(), key=lambda kv: -kv[1][0])},
+            "device_us_per_step_total": round(sum(v[0] for v in per_op.values()), 1),
         }
-        del tup
+        del tstep
 
     if not a.no_cpu:
         result["cpu_baseline"] = cpu_baseline()

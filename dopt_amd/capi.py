@@ -106,6 +106,7 @@ PROTOTYPES = {
     "dopt_hip_bn_grad_fused": [_sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_bn_train_open": [_sz, _sz, _sz, _d, C.POINTER(SplitSum), _vp, _vp, _vp, _vp, _vp, _i],
     "dopt_hip_bn_grad_open": [_sz, _sz, _sz, C.POINTER(SplitSum), _i, _vp, _vp, _vp, _vp, _vp],
+    "dopt_hip_bn_wait_limit": [C.c_uint],
     "dopt_hip_bn_infer": [_sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_optim_create": [_i, C.POINTER(TensorRef), C.POINTER(_vp)],
     "dopt_hip_optim_destroy": [_vp],

@@ -697,6 +697,7 @@ PLAN_FUSE = 4
 PLAN_OVERLAP = 8
 PLAN_GRAPH = 16
 PLAN_OVERLAP_LIGHT = 32
+PLAN_TIMING_SHAPES = 64
 
 
 class Plan:

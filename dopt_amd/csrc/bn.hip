@@ -1067,11 +1067,15 @@ int bn_cluster_poll()
                                       "results of batch-norm calls since the last synchronisation are invalid");
 }
 
-void bn_cluster_set_spin_limit(unsigned polls) { g_cluster_spin_limit = polls; }
-
 }  // namespace dopt
 
 extern "C" {
+
+int dopt_hip_bn_wait_limit(unsigned polls)
+{
+    g_cluster_spin_limit = polls;
+    return DOPT_HIP_OK;
+}
 
 int dopt_hip_bn_train(size_t N, size_t C, size_t inner, double momentum, const float *x, const float *scale,
                       const float *bias, const float *run_mean, const float *run_var, float *packed)

@@ -1203,6 +1203,10 @@ int HIPPlan::Builder::buildSteps()
             return fail(DOPT_HIP_ERR_INVALID, "Could not construct a HIP kernel for operation of type '%s': %s",
                         op.opType.c_str(), why.empty() ? "constructor returned null" : why.c_str());
         }
+        if (flags & DOPT_HIP_PLAN_TIMING_SHAPES) {
+            label += "@";
+            for (size_t i = 0; i < op.shape.size(); i++) label += (i ? "x" : "") + std::to_string(op.shape[i]);
+        }
         Step s;
         s.op = id;
         s.label = label;

@@ -338,6 +338,13 @@ int dopt_hip_bn_train_open(size_t N, size_t C, size_t inner, double momentum, co
                            float *packed, int relu);
 int dopt_hip_bn_grad_open(size_t N, size_t C, size_t inner, const dopt_hip_split_sum *dy_open, int keep_dy,
                           const float *y, const float *x, const float *scale, float *packed, float *dx_sum);
+/* Channels of more than 32768 values are normalised by a few workgroups each, which meet once inside the
+   kernel; a workgroup polls for its partners at most `polls` times (about a microsecond each; default
+   2^21) and then gives up: the kernel still ends, and the next dopt_hip_sync or dopt_hip_copy_d2h
+   returns DOPT_HIP_ERR_RUNTIME (the batch-norm results since the previous synchronisation are invalid).
+   No counterpart in the reference.  A limit of 0 makes every such call give up unless its partners have
+   already arrived (used to test the error path). */
+int dopt_hip_bn_wait_limit(unsigned polls);
 /* `batchNormInference`: cudnnBatchNormalizationForwardInference, cudnn7.d:650-652; eps = 1e-5. */
 int dopt_hip_bn_infer(size_t N, size_t C, size_t inner, const float *x, const float *scale,
                       const float *bias, const float *mean, const float *var, float *y);

@@ -72,6 +72,8 @@ enum {
     DOPT_HIP_PLAN_VIEWS = 1,  /* contiguous slices alias their input; slice(pad(x)) that undoes the
                                  pad aliases x; operations left without a consumer are dropped */
     DOPT_HIP_PLAN_TIMING = 2, /* bracket every kernel with HIP events (CUDAPlan.profiler) */
+    DOPT_HIP_PLAN_TIMING_SHAPES = 64, /* with TIMING: profiler keys are "opType@d0xd1x..." (the operation's output
+                                 shape), so that layers of one type are told apart */
     DOPT_HIP_PLAN_FUSE = 4,   /* with VIEWS: run adjacent operations as one kernel where the middle value
                                  has no other reader -- addBias(convolution), relu(batchNormTrain.y) and
                                  batchNormGrad(reluGrad) -- with the values of the separate kernels */

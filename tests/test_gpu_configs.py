@@ -1,6 +1,7 @@
 """The benchmark configurations as parity cases: whole training steps (or the whole fused update)
 run through compiled plans on the GPU and compared with the CPU oracle on the same seeded inputs.
 
+  config 1  softmax regression as examples/mnistlogit.d writes it: whole steps against the CPU evaluator
   config 2  MLP 784-512-512-10, batch 256, one ADAM step (op-graph form and fused form)
   config 3  fused ADAM / AMSGrad over 16 777 216 parameters in 40 tensors (full size, bit-exact)
   config 4  VGG-16 + batch norm, the benchmark itself: tests/test_gpu_config4.py
@@ -11,7 +12,8 @@ import numpy as np
 import pytest
 
 import oracle as O
-from dopt_amd import core, nnet, online, ops, workloads
+from dopt_amd import configs, core, nnet, online, ops, workloads
+from oracle import evaluator
 from dopt_amd.core import float32, grad
 from util import assert_close
 
@@ -21,6 +23,29 @@ T = ops.tensor
 
 def _f(shape, vals):
     return float32(list(shape), np.asarray(vals, np.float32).reshape(-1))
+
+
+# ------------------------------------------------------------------------------ config 1
+@pytest.mark.parametrize("flags", [0, configs.REWRITES, configs.REWRITES | core.PLAN_GRAPH], ids=["plain", "rewrites", "graph"])
+def test_config1_whole_steps_match_the_cpu_evaluator(flags):
+    """The one configuration the reference's CPU backend can train: every output of the update plan (loss,
+    predictions, new weights, new bias, new momenta) against the same graph evaluated on the CPU, one
+    restated reference kernel per operation (cpu/package.d:182-280), over three consecutive steps."""
+    step = configs.softmax_regression(flags=flags, host_args=(flags & core.PLAN_GRAPH) == 0)
+    outs = step.updater.plan.outputs
+    host_args = {k: (v if isinstance(v, np.ndarray) else v.numpy()) for k, v in step.args.items()}
+    W, b = step.params
+    losses = []
+    for it in range(3):
+        want = evaluator.evaluate(outs, host_args)          # reads the variables' current values
+        got_loss, got_preds = step.updater(step.args)        # runs the step and writes the variables back
+        assert_close(got_loss, want[0], "loss, step %d" % it)
+        assert_close(got_preds, want[1], "predictions, step %d" % it)
+        assert_close(W.value, want[2], "weights after step %d" % it)
+        assert_close(b.value, want[3], "bias after step %d" % it)
+        losses.append(float(got_loss))
+    assert losses[0] == pytest.approx(np.log(10), rel=1e-4)   # zero weights: uniform predictions
+    assert losses[2] < losses[1] < losses[0]
 
 
 # ------------------------------------------------------------------------------ config 2

@@ -517,6 +517,30 @@ def test_batchnorm_channels_spanning_several_blocks(shape):
     ops.sync()
 
 
+def test_batchnorm_blocks_that_do_not_meet_are_reported_and_recovered_from():
+    """The blocks sharing a channel wait for each other a bounded number of polls.  With the bound at zero
+    every block gives up at once (each still finishes and exits): the next synchronisation reports it, and
+    with the bound restored the same call is correct again."""
+    from dopt_amd import capi
+    lib = capi.load()
+    r = rng(64)
+    shape = (128, 64, 32, 32)
+    x = r.standard_normal(shape).astype(np.float32)
+    ones, zeros = np.ones(64, np.float32), np.zeros(64, np.float32)
+    tx, t1, t0 = T(x), T(ones), T(zeros)
+    ops.sync()
+    capi.check(lib.dopt_hip_bn_wait_limit(0))
+    try:
+        out = ops.bn_train(tx, t1, t0, t0, t1, 0.9)
+        with pytest.raises(capi.HipError, match="did not meet"):
+            ops.sync()
+    finally:
+        capi.check(lib.dopt_hip_bn_wait_limit(1 << 21))
+    ops.sync()                                     # the error was reported once
+    got = ops.bn_train(tx, t1, t0, t0, t1, 0.9, out=out).numpy()
+    assert_close(got[:x.size], O.bn_train(x, ones, zeros, zeros, ones, 0.9)[:x.size], "bn y after recovery")
+
+
 def test_batchnorm_large_mean_small_variance():
     # E[x^2] - E[x]^2 would lose everything here; the shifted moments must not
     r = rng(62)

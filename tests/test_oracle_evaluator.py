@@ -1,0 +1,67 @@
+"""The CPU graph evaluator (oracle/evaluator.py) against closed forms: a softmax regression written out by
+hand as examples/mnistlogit.d:39-47 writes it, its loss and the gradients that reverse-mode differentiation
+of the graph produces, against the textbook expressions in float64.  No GPU: the graph is never registered
+with the device library."""
+import numpy as np
+
+from dopt_amd import core, nnet
+from dopt_amd.core import float32, grad
+from oracle import evaluator
+
+
+def test_softmax_regression_graph_on_the_cpu_evaluator():
+    n, d, k = 6, 7, 3
+    r = np.random.default_rng(0)
+    x = r.random((n, d)).astype(np.float32)
+    y = np.eye(k, dtype=np.float32)[r.integers(0, k, n)]
+    f, l = float32([n, d]), float32([n, k])
+    W = float32([d, k], r.standard_normal((d, k)).astype(np.float32))
+    b = float32([k], r.standard_normal(k).astype(np.float32))
+    lin = core.matmul(f, W) + core.repeat(b, n)
+    num = core.exp(lin - core.maxElement(lin))
+    den = core.repeat(core.sum(num, [1]).reshape([n, 1]), [1, k])
+    p = num / den
+    loss = nnet.crossEntropy(p, l)
+    gW, gb = grad(loss, [W, b])
+    got = evaluator.evaluate([loss, p, gW, gb], {f: x, l: y})
+
+    z = x.astype(np.float64) @ W.value.astype(np.float64) + b.value
+    e = np.exp(z - z.max())
+    pp = e / e.sum(axis=1, keepdims=True)
+    dp = -(y / (pp + 1e-6)) / n
+    dz = pp * (dp - (dp * pp).sum(axis=1, keepdims=True))
+    assert np.isclose(got[0], -(y * np.log(pp + 1e-6)).sum() / n, rtol=1e-6)
+    assert np.allclose(got[1], pp, rtol=1e-5, atol=1e-7)
+    assert np.allclose(got[2], x.astype(np.float64).T @ dz, rtol=1e-4, atol=1e-6)
+    assert np.allclose(got[3], dz.sum(axis=0), rtol=1e-4, atol=1e-6)
+
+
+def test_convolution_block_graph_on_the_cpu_evaluator():
+    """conv -> addBias -> batchNormTrain -> relu -> maxpool and its gradients: the evaluator's dispatch
+    against the oracle's operations called by hand."""
+    import oracle as O
+    r = np.random.default_rng(1)
+    x = r.standard_normal((2, 3, 4, 4)).astype(np.float32)
+    feats = float32([2, 3, 4, 4])
+    init = nnet.Init(3)
+    layer = nnet.maxPool(nnet.relu(nnet.batchNorm(nnet.conv2D(nnet.dataSource(feats), 4, [3, 3], init, padding=(1, 1)))), [2, 2])
+    out = layer.trainOutput
+    net = nnet.DAGNetwork([feats], [layer])
+    loss = core.sum(out * out)
+    g = grad(loss, net.params[:4])
+    got = evaluator.evaluate([out] + g, {feats: x})
+    w, bias, gamma, beta = (p.value for p in net.params[:4])
+    c = O.add_bias(O.convolution(x, w, (1, 1), (1, 1), f64=False), bias)
+    packed = O.bn_train(c, gamma.reshape(-1), beta, np.zeros(4, np.float32), np.ones(4, np.float32), float(np.float32(0.9)))
+    yb = packed[:c.size].reshape(c.shape)
+    rl = O.relu(yb)
+    pooled = O.maxpool(rl, (2, 2))
+    assert np.array_equal(got[0], pooled)
+    dpool = (2 * pooled).astype(np.float32)
+    dy = O.relu_grad(O.maxpool_grad(dpool, rl, (2, 2)), yb)
+    gp = O.bn_grad(dy, c, gamma.reshape(-1))
+    dc = gp[:c.size].reshape(c.shape)
+    assert np.allclose(got[1], O.conv_bwd_filter(dc, x, w.shape, (1, 1), (1, 1)), rtol=1e-5, atol=1e-6)
+    assert np.allclose(got[2], O.add_bias_grad(dc), rtol=1e-5, atol=1e-6)
+    assert np.allclose(got[3].reshape(-1), gp[c.size:c.size + 4], rtol=1e-5, atol=1e-6)
+    assert np.allclose(got[4], gp[c.size + 4:], rtol=1e-5, atol=1e-6)
