@@ -173,6 +173,42 @@ __global__ __launch_bounds__(kBlock) void bn_infer_prepare_k(size_t C, double ep
     coef[c] = k;
 }
 
+// Inference in one launch: block (c, slice) derives its channel's coefficients itself (one float64
+// reciprocal square root per thread) and streams that channel's rows of images slice, slice + S, ...
+// with four 128-bit loads in flight per thread.  Same arithmetic as the coefficient table + bn_apply_k.
+__global__ __launch_bounds__(kBlock) void bn_infer_chan_k(unsigned N, unsigned C, unsigned inner4, unsigned S, double eps,
+                                                           const float *x, const float *scale, const float *bias,
+                                                           const float *mean, const float *var, float *y)
+{
+    const unsigned c = blockIdx.x % C, s = blockIdx.x / C;
+    const double rstd = 1.0 / sqrt((double)var[c] + eps);
+    const float m = mean[c], a = (float)((double)scale[c] * rstd), b = bias[c];
+    const unsigned nimg = (N - s + S - 1) / S, tot = nimg * inner4;
+    const float4 *x4 = (const float4 *)x;
+    float4 *y4 = (float4 *)y;
+    for (unsigned base = threadIdx.x; base < tot; base += kUnroll * kBlock) {
+        float4 v[kUnroll];
+        size_t at[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            const unsigned t = base + u * kBlock;
+            const unsigned j = t / inner4, i = t - j * inner4;
+            at[u] = ((size_t)(s + j * S) * C + c) * inner4 + i;
+            if (t < tot) v[u] = x4[at[u]];
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            if (base + u * kBlock >= tot) continue;
+            float4 r;
+            r.x = a * ((v[u].x - m) - 0.0f) + b;
+            r.y = a * ((v[u].y - m) - 0.0f) + b;
+            r.z = a * ((v[u].z - m) - 0.0f) + b;
+            r.w = a * ((v[u].w - m) - 0.0f) + b;
+            y4[at[u]] = r;
+        }
+    }
+}
+
 __global__ __launch_bounds__(kBlock) void bn_grad_finalize_k(size_t N, size_t C, size_t inner, size_t S, double eps,
                                                               const float *x, const float *partial,
                                                               const float *scale, CoefG *coef, float *dscale,
@@ -1132,6 +1168,14 @@ int dopt_hip_bn_infer(size_t N, size_t C, size_t inner, const float *x, const fl
     if (total == 0) return DOPT_HIP_OK;
     DOPT_REQUIRE(x && scale && bias && mean && var && y, "dopt_hip_bn_infer: null argument");
     DOPT_ENSURE_INIT();
+    if ((inner & 3) == 0 && inner >= 256 && aligned16(x) && aligned16(y) && total / 4 < 0xffffffffull && N < (1u << 24) &&
+        C <= 0x7fffffffu / kMaxSlices) {
+        const size_t S = pick_slices(N, C);
+        hipLaunchKernelGGL(bn_infer_chan_k, dim3((unsigned)(C * S)), dim3(kBlock), 0, stream(), (unsigned)N, (unsigned)C,
+                           (unsigned)(inner / 4), (unsigned)S, 1e-5 /* cudnn7.d:652 */, x, scale, bias, mean, var, y);
+        DOPT_LAUNCH_CHECK();
+        return DOPT_HIP_OK;
+    }
     Coef *coef = (Coef *)workspace(C * sizeof(Coef));
     if (!coef) return DOPT_HIP_ERR_OOM;
     hipLaunchKernelGGL(bn_infer_prepare_k, dim3((unsigned)ceil_div(C, (size_t)kBlock)), dim3(kBlock), 0, stream(), C,

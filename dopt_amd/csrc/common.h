@@ -51,6 +51,8 @@ bool sgemm_fold2x2(size_t C, size_t K, size_t N, const float *x, const float *dy
 bool conv_smallc_takes(const dopt_hip_conv_desc *d);
 int conv_smallc_fwd(const dopt_hip_conv_desc *d, const float *x, const float *w, const float *bias, float *y, bool *done);
 int conv_smallc_wgrad(const dopt_hip_conv_desc *d, const float *dy, const float *x, float *dw, bool *done);
+// nn.hip: out[c] = sum_{n,i} in[n][c][i] in one launch; false, with nothing launched, for shapes it does not take.
+bool channel_sum(size_t N, size_t C, size_t inner, const float *in, float *out, int *rc);
 hipStream_t lane_stream(int lane);
 // bn.hip: error report of the multi-block batch-norm kernels; call with the queues idle.
 int bn_cluster_poll();

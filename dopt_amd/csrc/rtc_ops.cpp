@@ -404,13 +404,59 @@ extern "C" __global__ __launch_bounds__(BLOCK) void argmin_rows_k(const T *in, i
     const T *p = in + row * A;
     T best = (T)(TMAX);
     int bi = 0x7fffffff;  // "never fired"
-    for (size_t i = lane; i < A; i += 64) {
+    size_t i = lane;
+    for (; i + 192 < A; i += 256) {   // four loads in flight; tested in index order
+        T v0 = p[i], v1 = p[i + 64], v2 = p[i + 128], v3 = p[i + 192];
+        if (v0 < best) { best = v0; bi = (int)i; }
+        if (v1 < best) { best = v1; bi = (int)(i + 64); }
+        if (v2 < best) { best = v2; bi = (int)(i + 128); }
+        if (v3 < best) { best = v3; bi = (int)(i + 192); }
+    }
+    for (; i < A; i += 64) {
         T v = p[i];
         if (v < best) {
             best = v;
             bi = (int)i;
         }
     }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        T ov = __shfl_down(best, off, 64);
+        int oi = __shfl_down(bi, off, 64);
+        if (ov < best || (ov == best && oi < bi)) {
+            best = ov;
+            bi = oi;
+        }
+    }
+    if (lane == 0) out[row] = bi == 0x7fffffff ? 0 : bi;
+}
+
+// The same with 128-bit loads (A a multiple of four, 16-byte aligned rows): a lane's elements still
+// come in ascending index order, so its first minimum is found the same way.
+extern "C" __global__ __launch_bounds__(BLOCK) void argmin_rows4_k(const T *in, int *out, size_t rows, size_t A)
+{
+    const size_t row = (size_t)blockIdx.x * (BLOCK / 64) + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int lane = threadIdx.x & 63;
+    const T4 *p = (const T4 *)(in + row * A);
+    const size_t A4 = A / 4;
+    T best = (T)(TMAX);
+    int bi = 0x7fffffff;
+#define TEST4(v, q)                                              \
+    if (v.x < best) { best = v.x; bi = (int)(4 * (q)); }         \
+    if (v.y < best) { best = v.y; bi = (int)(4 * (q) + 1); }     \
+    if (v.z < best) { best = v.z; bi = (int)(4 * (q) + 2); }     \
+    if (v.w < best) { best = v.w; bi = (int)(4 * (q) + 3); }
+    size_t i = lane;
+    for (; i + 192 < A4; i += 256) {
+        T4 v0 = p[i], v1 = p[i + 64], v2 = p[i + 128], v3 = p[i + 192];
+        TEST4(v0, i) TEST4(v1, i + 64) TEST4(v2, i + 128) TEST4(v3, i + 192)
+    }
+    for (; i < A4; i += 64) {
+        T4 v = p[i];
+        TEST4(v, i)
+    }
+#undef TEST4
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
         T ov = __shfl_down(best, off, 64);
@@ -444,8 +490,8 @@ std::string reduce_source(bool is_sum, int dtype)
 std::string argmin_source(int dtype)
 {
     std::string s;
-    s += dtype == DOPT_HIP_F32 ? "typedef float T;\n#define TMAX 3.402823466e+38f\n"
-                               : "typedef int T;\n#define TMAX 2147483647\n";
+    s += dtype == DOPT_HIP_F32 ? "typedef float T;\ntypedef float4 T4;\n#define TMAX 3.402823466e+38f\n"
+                               : "typedef int T;\ntypedef int4 T4;\n#define TMAX 2147483647\n";
     s += kArgminBody;
     return s;
 }
@@ -651,6 +697,16 @@ int dopt_hip_reduce(const char *op, int dtype, const size_t *shape, int rank, co
         runs.push_back({i, j});
         i = j + 1;
     }
+    // fp32 sum over everything but one run of axes in the middle ([N, C, inner] -> [C], the shape of a
+    // per-channel statistic): one launch instead of one pass per run of reduced axes
+    if (is_sum && dtype == DOPT_HIP_F32 && runs.size() == 2 && runs[0].first == 0 && runs[1].second == rank - 1) {
+        size_t N = 1, C = 1, inner = 1;
+        for (int i = 0; i <= runs[0].second; i++) N *= cur[i];
+        for (int i = runs[0].second + 1; i < runs[1].first; i++) C *= cur[i];
+        for (int i = runs[1].first; i < rank; i++) inner *= cur[i];
+        int crc = DOPT_HIP_OK;
+        if (channel_sum(N, C, inner, (const float *)in, (float *)out, &crc)) return crc;
+    }
     const void *src_ptr = in;
     void *tmp_prev = nullptr;
     int rc = DOPT_HIP_OK;
@@ -690,7 +746,9 @@ int dopt_hip_argmin(int dtype, const size_t *shape, int rank, size_t axis, const
     hipFunction_t fn;
     std::string key = std::string("argmin") + (dtype == DOPT_HIP_F32 ? ":f32" : ":i32");
     if (vol == 1 && A >= 64 && A < 0x7fffffffu) {
-        if (int rc = rtc_get(key + ":rows", argmin_source(dtype), "argmin_rows_k", &fn)) return rc;
+        const bool vec = A % 4 == 0 && A >= 256 && aligned16(in);
+        if (int rc = rtc_get(key + (vec ? ":rows4" : ":rows"), argmin_source(dtype), vec ? "argmin_rows4_k" : "argmin_rows_k", &fn))
+            return rc;
         void *rargs[] = {(void *)&in, (void *)&out, (void *)&outer, (void *)&A};
         return rtc_launch(fn, (unsigned)ceil_div(outer, (size_t)4), 256, rargs);
     }

@@ -269,14 +269,15 @@ int dopt_hip_bias_fwd(size_t N, size_t C, size_t inner, const float *x, const fl
 int dopt_hip_bias_bwd(size_t N, size_t C, size_t inner, const float *dy, float *db);
 /* dopt_hip_bias_bwd for callers that cannot allocate device memory (code recording a HIP graph, tight
    serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same kernels and
-   the same result bit for bit, but the per-(channel, image-slice) partial sums of the two-stage path
-   go to a 256 KiB array built into the library (one copy per device, held until the process ends)
-   instead of the grown-on-demand workspace, and nothing in the call allocates, frees or fills through
-   the runtime.  Needs dopt_hip_init to have run.  Limit: C * S <= 65536 partial sums, where
-   S = min(64, N, ceil(8 * CUs / C)) -- with 256 compute units that is every C <= 65536; beyond it the
-   call fails with DOPT_HIP_ERR_INVALID and launches nothing.  All calls on a device share that array
-   (each overwrites what it reads before reading it, so nothing has to be cleared): calls that overlap
-   on one device -- two host threads, two streams -- race. */
+   the same result bit for bit, but the per-(channel, image-slice) partial sums of the sliced path
+   (rows of at least 256 values) go to a 256 KiB array built into the library for this entry point alone
+   (one copy per device, held until the process ends), and the call sets nothing up: no lazy
+   initialisation, no allocation, no free, no fill through the runtime.  Needs dopt_hip_init to have run.
+   Limit: C * S <= 65536 partial sums, where S = min(64, N, ceil(8 * CUs / C)) -- with 256 compute
+   units that is every C <= 65536; beyond it the call fails with DOPT_HIP_ERR_INVALID and launches
+   nothing.  All calls on a device share that array (each call overwrites what it reads before reading
+   it, so nothing has to be cleared): calls that overlap on one device -- two host threads, two streams
+   -- race. */
 int dopt_hip_bias_bwd_noalloc(size_t N, size_t C, size_t inner, const float *dy, float *db);
 
 /* `uniform`: curandGenerateUniform at cuda/random.d:74 -- n floats drawn uniformly from (0, 1].

@@ -124,6 +124,10 @@ def test_pointwise_rejects_bad_arity_and_names():
     ((128, 10), None), ((100, 10), None), ((7,), None), ((3, 4, 5), (1,)), ((3, 4, 5), (0, 2)),
     ((2, 3, 4, 5), (1, 2)), ((2, 3, 4, 5), (3,)), ((2, 3, 4, 5), (0,)), ((640, 640, 3, 3), None),
     ((5, 70000), (1,)), ((2048, 33), (1,)), ((4, 6), (0,)),
+    # everything but a run of axes in the middle (a per-channel statistic): the one-launch sliced kernel
+    ((128, 64, 32, 32), (0, 2, 3)), ((16, 8, 16, 32), (0, 2, 3)), ((3, 5, 7, 300), (0, 3)), ((70, 3, 2, 258), (0, 3)),
+    ((2, 3, 100000), None),                       # one row split over many blocks, finished by the last of them
+    ((3, 2 * 4096 * 5 + 8), (1,)),                # the same for several rows
 ])
 def test_sum_and_max(shape, axes):
     r = rng(11)
@@ -149,7 +153,8 @@ def test_max_identity_is_minus_type_max():
 
 
 @pytest.mark.parametrize("shape,axis", [((5,), 0), ((2, 3), 1), ((2, 3), 0), ((4, 5, 6), 1), ((3, 1000), 1),
-                                        ((1000, 3), 0), ((37, 64), 1), ((300, 4097), 1), ((2, 3, 130), 2)])
+                                        ((1000, 3), 0), ((37, 64), 1), ((300, 4097), 1), ((2, 3, 130), 2),
+                                        ((64, 2048), 1), ((5, 256), 1), ((3, 1028), 1)])
 def test_argmin(shape, axis):
     r = rng(12)
     x = r.integers(-5, 5, shape).astype(np.float32)   # many ties: first minimum must win
@@ -232,10 +237,15 @@ def test_slice_rejects_out_of_range():
 
 
 @pytest.mark.parametrize("rows,cols", [(2, 2), (1, 9), (9, 1), (5, 9), (64, 64), (65, 130), (512, 512), (10, 784),
-                                       (1000, 3)])
+                                       (1000, 3),
+                                       (68, 132), (4, 4), (4096, 2048), (100, 260), (8, 1028)])   # 128-bit tiles, ragged edges
 def test_transpose(rows, cols):
     x = rng(22).standard_normal((rows, cols)).astype(np.float32)
     assert np.array_equal(ops.transpose(T(x)).numpy(), O.transpose(x))
+    if rows % 4 == 0 and cols % 4 == 0 and rows * cols > 16:
+        # an operand off the 16-byte grid takes the 32-bit tile kernel
+        buf = T(np.concatenate([np.zeros(1, np.float32), x.ravel()]))
+        assert np.array_equal(ops.transpose(buf.view(1, (rows, cols))).numpy(), O.transpose(x))
 
 
 # ----------------------------------------------------------------------------- matmul
