@@ -948,6 +948,7 @@ int bn_train_impl(size_t N, size_t C, size_t inner, double momentum, const float
     if (x_open && x_open->splits) {   // x is still in pieces
         OpenSum os;
         if (T && N * (inner / 4) <= (size_t)kOpenQuads * T && open_sum(x_open, total, C, inner, true, &os)) {
+            open_split_clear(x_open->partial);
             hipLaunchKernelGGL((bn_resident_k<false, true, kOpenQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N, (unsigned)C,
                                (unsigned)(inner / 4), factor, eps, x, (const float *)nullptr, scale, bias, run_mean, run_var,
                                (const float *)nullptr, relu, packed, packed + total, packed + total + C, (float *)nullptr, os);
@@ -1012,6 +1013,7 @@ int bn_grad_impl(size_t N, size_t C, size_t inner, const float *dy, const float 
     if (dy_open && dy_open->splits) {   // dy is still in pieces
         OpenSum os;
         if (T && N * (inner / 4) <= (size_t)kOpenQuads * T && open_sum(dy_open, total, C, inner, keep_dy, &os)) {
+            open_split_clear(dy_open->partial);
             hipLaunchKernelGGL((bn_resident_k<true, true, kOpenQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N, (unsigned)C,
                                (unsigned)(inner / 4), 0.0, eps, x, dy, scale, (const float *)nullptr,
                                (const float *)nullptr, (const float *)nullptr, ymask, 0, packed, packed + total,

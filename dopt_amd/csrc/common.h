@@ -29,6 +29,10 @@ void *workspace(size_t bytes);
 // Changes whenever a workspace is reallocated (its address may have changed): whoever keeps the
 // address beyond one call -- a recorded HIP graph -- compares generations before using it again.
 unsigned long workspace_generation();
+// A convolution that leaves its result open parks partial sums in the workspace until the next call adds
+// them up; until open_split_clear, any other request for the workspace fails instead of overwriting them.
+void open_split_set(const void *partial);
+void open_split_clear(const void *partial);
 // The library owns two in-order queues.  Everything enqueues on the main one unless a plan has
 // switched to the side queue for a step it overlaps with its main chain (set_lane(1) ... set_lane(0));
 // each queue has its own workspace.

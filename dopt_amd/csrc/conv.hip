@@ -1307,6 +1307,7 @@ int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, 
         open->inner = (size_t)pc.OH * pc.OW;
         open->bias = bias;
         open->value = out;
+        open_split_set(partial);
         return DOPT_HIP_OK;
     }
     if (splits > 1)
@@ -1911,6 +1912,7 @@ int dopt_hip_split_sum_close(const dopt_hip_split_sum *open)
     DOPT_REQUIRE(open->splits > 1 && open->partial && open->value && open->elems % 4 == 0 && open->C > 0 && open->inner > 0,
                  "dopt_hip_split_sum_close: malformed description");
     DOPT_ENSURE_INIT();
+    open_split_clear(open->partial);
     return launch_splitk_reduce(open->elems, open->splits, open->partial, open->value, open->bias, (unsigned)open->C,
                                 (unsigned)open->inner);
 }

@@ -255,15 +255,18 @@ __global__ __launch_bounds__(kBlock) void maxpool_fwd_k(size_t maps, size_t H, s
     }
 }
 
-// Gradient goes to the first maximum of the window in row-major order (strict '>' keeps the earlier one).
+// Gradient goes to the element the forward pass selected: the same chain of `acc < v` tests starting from
+// -FLT_MAX, in row-major order, so the first maximum wins and an element that never compares greater (a NaN)
+// is never selected; a window in which nothing fires sends its gradient to its first element.
 __device__ inline void route2x2(float a, float b, float c, float d, float g, float &oa, float &ob, float &oc,
                                 float &od)
 {
     int best = 0;
-    float bv = a;
-    if (b > bv) { bv = b; best = 1; }
-    if (c > bv) { bv = c; best = 2; }
-    if (d > bv) { bv = d; best = 3; }
+    float bv = -FLT_MAX;
+    if (bv < a) { bv = a; best = 0; }
+    if (bv < b) { bv = b; best = 1; }
+    if (bv < c) { bv = c; best = 2; }
+    if (bv < d) { bv = d; best = 3; }
     oa = best == 0 ? g : 0.0f;
     ob = best == 1 ? g : 0.0f;
     oc = best == 2 ? g : 0.0f;
@@ -304,12 +307,12 @@ __global__ __launch_bounds__(kBlock) void maxpool_bwd_k(size_t maps, size_t H, s
         if (p < P && q < Q) {
             const float *img = x + m * H * W;
             size_t best = (p * ph) * W + q * pw;
-            float bv = img[best];
+            float bv = -FLT_MAX;   // the forward pass's own chain of tests
             for (size_t j = 0; j < ph; j++)
                 for (size_t i = 0; i < pw; i++) {
                     size_t e = (p * ph + j) * W + q * pw + i;
                     float v = img[e];
-                    if (v > bv) { bv = v; best = e; }
+                    if (bv < v) { bv = v; best = e; }
                 }
             if (best == h * W + w) out = dy[(m * P + p) * Q + q];
         }

@@ -13,7 +13,12 @@
  *     dopt_hip_copy_d2h and dopt_hip_sync are the synchronisation points (the reference
  *     synchronises after nearly every launch, but callers only rely on ordering and on a
  *     device-to-host read seeing finished data);
- *   - single host thread per process, like the reference's registries.
+ *   - NOT thread-safe: one host thread at a time may be inside the library (the reference's registries and
+ *     plans are thread-local D globals; this library keeps one process-wide device, stream pair, workspace
+ *     and kernel cache instead).  The lock inside the buffer pool only protects dopt_hip_malloc /
+ *     dopt_hip_free / dopt_hip_pool_* against a garbage collector's finaliser thread releasing buffers while
+ *     the owning thread allocates; everything else, including the queue an entry point enqueues on and the
+ *     graph-recording state, is unguarded.
  */
 #ifndef DOPT_HIP_H
 #define DOPT_HIP_H

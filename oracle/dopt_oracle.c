@@ -568,12 +568,15 @@ int f64_maxpool_grad(size_t N, size_t C, size_t H, size_t W, size_t ph, size_t p
         float *gimg = dx + m * H * W;
         for (size_t yy = 0; yy < P; yy++)
             for (size_t xx = 0; xx < Q; xx++) {
+                /* the element the forward loop (cpu/nnet.d:103-113: acc = max(acc, v) = acc < v ? v : acc from
+                   -float.max) ends up holding: first maximum in row-major order, a NaN never; the window's first
+                   element when no test fires */
                 size_t best = (yy * ph) * W + xx * pw;
-                float bestv = inimg[best];
+                float bestv = -FLT_MAX;
                 for (size_t j = 0; j < ph; j++)
                     for (size_t i = 0; i < pw; i++) {
                         size_t idx = (yy * ph + j) * W + xx * pw + i;
-                        if (inimg[idx] > bestv) { bestv = inimg[idx]; best = idx; }
+                        if (bestv < inimg[idx]) { bestv = inimg[idx]; best = idx; }
                     }
                 gimg[best] = dy[m * P * Q + yy * Q + xx];
             }

@@ -58,3 +58,25 @@ def test_errors_are_reported_not_swallowed():
     p = C.c_void_p(1)
     assert lib.dopt_hip_malloc(C.byref(p), 0) == 0 and not p.value
     assert lib.dopt_hip_free(None) == 0
+
+
+def test_convolutions_refuse_tensors_their_32_bit_offsets_cannot_reach():
+    """The convolution kernels address their operands with 32-bit byte offsets (buffer resources whose range
+    check supplies the zero padding): a descriptor with a tensor of 2 GiB or more is refused on the host,
+    before the device is touched, instead of reading zeros past the range."""
+    import ctypes as C
+    from dopt_amd import capi
+    lib = capi.load()
+    d = capi.ConvDesc(N=1 << 20, C=64, H=32, W=32, K=64, R=3, S=3, padH=1, padW=1, strideH=1, strideW=1)
+    dummy = C.c_void_p(256)     # never dereferenced: the descriptor is checked first
+    for call in (lambda: lib.dopt_hip_conv_fwd(C.byref(d), dummy, dummy, dummy),
+                 lambda: lib.dopt_hip_conv_fwd_bias(C.byref(d), dummy, dummy, dummy, dummy),
+                 lambda: lib.dopt_hip_conv_bwd_data(C.byref(d), dummy, dummy, dummy),
+                 lambda: lib.dopt_hip_conv_bwd_filter(C.byref(d), dummy, dummy, dummy),
+                 lambda: lib.dopt_hip_conv_fwd_bias_packed(C.byref(d), dummy, dummy, dummy, dummy),
+                 lambda: lib.dopt_hip_conv_bwd_data_packed(C.byref(d), dummy, dummy, dummy)):
+        assert call() == 1
+        assert b"2^29 elements or more" in lib.dopt_hip_last_error()
+    # a filter that large is refused as well
+    d = capi.ConvDesc(N=1, C=1 << 14, H=4, W=4, K=1 << 14, R=3, S=3, padH=1, padW=1, strideH=1, strideW=1)
+    assert lib.dopt_hip_conv_fwd(C.byref(d), dummy, dummy, dummy) == 1

@@ -457,6 +457,31 @@ def test_open_convolution_results_closed_by_batch_norm(xs, k):
                 assert np.all(got == 7.0)
 
 
+def test_an_open_convolution_result_must_be_closed_by_the_next_call():
+    """The partial sums of an open result live in the library's workspace; a call that would reuse the workspace
+    before they are added up is refused (once), and the library carries on."""
+    lib = capi.load()
+    r = np.random.default_rng(5)
+    xs, ws = (8, 256, 4, 4), (512, 256, 3, 3)
+    x = ops.tensor(r.standard_normal(xs).astype(np.float32))
+    w = ops.tensor(r.standard_normal(ws).astype(np.float32))
+    d = ops.conv_desc(xs, ws, (1, 1), (1, 1))
+    nbytes = lib.dopt_hip_conv_packed_bytes(C.byref(d), 0)
+    packed = ops.Tensor([nbytes // 4])
+    descs = (capi.ConvDesc * 1)(d)
+    capi.check(lib.dopt_hip_conv_pack_batch(1, descs, (C.c_int * 1)(0), (C.c_void_p * 1)(w.ptr), (C.c_void_p * 1)(packed.ptr)))
+    y = ops.Tensor((8, 512, 4, 4))
+    o = capi.SplitSum()
+    capi.check(lib.dopt_hip_conv_fwd_bias_packed_open(C.byref(d), x.ptr, packed.ptr, None, y.ptr, C.byref(o)))
+    assert o.splits > 1
+    with pytest.raises(capi.HipError, match="was not closed"):
+        ops.sum(ops.tensor(r.standard_normal((4, 100000)).astype(np.float32)), [1])     # wants the workspace
+    # the refusal is reported once; the same convolution, closed properly, gives the plain entry point's result
+    capi.check(lib.dopt_hip_conv_fwd_bias_packed_open(C.byref(d), x.ptr, packed.ptr, None, y.ptr, C.byref(o)))
+    capi.check(lib.dopt_hip_split_sum_close(C.byref(o)))
+    assert np.array_equal(y.numpy(), ops.convolution(x, w, (1, 1), (1, 1)).numpy())
+
+
 def _small_convnet(seed):
     init = nnet.Init(seed)
     x, y = core.float32([16, 3, 16, 16]), core.float32([16, 10])

@@ -402,6 +402,19 @@ def test_maxpool_and_grad(shape, dims):
     assert np.array_equal(ops.maxpool(T(x), dims).numpy(), y_ref)
     dy = r.standard_normal(y_ref.shape).astype(np.float32)
     assert np.array_equal(ops.maxpool_grad(T(dy), T(x), dims).numpy(), O.maxpool_grad(dy, x, dims))
+    # NaNs: forward never selects one (acc < NaN is false), so backward must not route a gradient to one either
+    xn = x.copy()
+    xn.ravel()[::3] = np.nan
+    yn = ops.maxpool(T(xn), dims).numpy()
+    assert np.array_equal(yn, O.maxpool(xn, dims))
+    gn = ops.maxpool_grad(T(dy), T(xn), dims).numpy()
+    assert np.array_equal(gn, O.maxpool_grad(dy, xn, dims))
+    ph, pw = dims
+    P, Q = shape[2] // ph, shape[3] // pw
+    win = xn[:, :, :P * ph, :Q * pw].reshape(shape[0], shape[1], P, ph, Q, pw)
+    gw = gn[:, :, :P * ph, :Q * pw].reshape(shape[0], shape[1], P, ph, Q, pw)
+    some_number = ~np.isnan(win).all(axis=(3, 5), keepdims=True)
+    assert not (gw != 0)[np.isnan(win) & some_number].any()     # (an all-NaN window sends it to its first element)
 
 
 @pytest.mark.parametrize("shape", [(1, 5), (128, 10), (256, 10), (4, 7, 3), (3, 5, 2, 2), (37, 64), (300, 1000),

@@ -223,6 +223,23 @@ def test_maxpool_grad_tie_goes_to_first_in_row_major_scan():
     assert dx.ravel().tolist() == [2, 0, 0, 3, 0, 0, 0, 0]
 
 
+def test_maxpool_grad_follows_the_forward_selection_through_nans():
+    """The forward loop keeps acc = (acc < v ? v : acc) from -float.max (cpu/nnet.d:103-113): a NaN never
+    replaces acc.  The gradient goes to the element that loop ends up holding; the expected arrays are
+    worked out by hand."""
+    nan = np.nan
+    x = np.array([[[[nan, 1.0, 4.0, nan],
+                    [2.0, nan, nan, 4.0]]]], np.float32)
+    y = O.maxpool(x, (2, 2))
+    assert y.ravel().tolist() == [2.0, 4.0]
+    dx = O.maxpool_grad(np.array([[[[7.0, 9.0]]]], np.float32), x, (2, 2))
+    # window 0 holds {nan, 1, 2, nan}: 2 at (1, 0); window 1 holds {4, nan, nan, 4}: the first 4 at (0, 2)
+    assert dx.ravel().tolist() == [0, 0, 9, 0, 7, 0, 0, 0]
+    allnan = np.full((1, 1, 2, 2), nan, np.float32)
+    assert O.maxpool(allnan, (2, 2)).ravel().tolist() == [-np.finfo(np.float32).max]
+    assert O.maxpool_grad(np.array([[[[5.0]]]], np.float32), allnan, (2, 2)).ravel().tolist() == [5, 0, 0, 0]
+
+
 def test_softmax_and_grad():
     from scipy.special import softmax as sp_softmax
     x = (rng.standard_normal((4, 7, 3)) * 3).astype(np.float32)
