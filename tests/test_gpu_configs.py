@@ -289,6 +289,57 @@ def test_config5_wrn_block_step_matches_the_oracle():
     assert_close(after[0][names.index("rm1")], rm1, "running mean after the step")
 
 
+def test_config5_small_wide_resnet_step_matches_the_cpu_evaluator():
+    """The whole Wide-ResNet graph (nnet/models/wrn.d:56-219: strided stage entries, 1x1 projections from the
+    block input, weight decay, mean pool as a GEMV) at depth 10, width 2, batch 4: loss, predictions and
+    every parameter gradient from HIPPlan, with and without the rewrites, against the same graph on the CPU
+    evaluator."""
+    n = 4
+    r = np.random.default_rng(70)
+    X = r.standard_normal((n, 3, 32, 32)).astype(np.float32)
+    Y = workloads.one_hot(r.integers(0, 10, n))
+    feats, labels = float32([n, 3, 32, 32]), float32([n, 10])
+    init = nnet.Init(71)
+    preds = nnet.softmax(nnet.dense(nnet.wideResNet(feats, 10, 2, init), 10, init))
+    net = nnet.DAGNetwork([feats], [preds])
+    loss = nnet.crossEntropy(preds.trainOutput, labels) + net.paramLoss
+    grads = grad(loss, net.params)
+    outs = [loss, preds.trainOutput] + grads
+    want = evaluator.evaluate(outs, {feats: X, labels: Y})
+    for flags in (0, configs.REWRITES):
+        got = core.compile(outs, flags).execute({feats: X, labels: Y})
+        for i, (g, w) in enumerate(zip(got, want)):
+            assert_close(g, w, "output %d (%s), flags %d" % (i, outs[i].opType, flags))
+
+
+def test_config5_wide_resnet_28_10_step_at_batch_128_rewrites_and_fused_update_change_nothing():
+    """The full-size step through size-independent properties: every output of the plan with the rewrites on
+    equals the plan without them bit for bit, and one fused ADAM step leaves the parameters the op-graph ADAM
+    step leaves, bit for bit."""
+    results = []
+    for flags in (0, configs.REWRITES):
+        step = configs.wide_resnet(128, fused=True, flags=flags)
+        net, loss, preds = step.extra["net"], step.loss, step.extra["preds"]
+        grads = grad(loss, net.params)
+        plan = core.compile([loss, preds.trainOutput] + grads, flags)
+        results.append(plan.execute(step.args))
+        plan.cleanup()
+        del step, plan
+    for i, (a, b) in enumerate(zip(*results)):
+        assert np.array_equal(a, b), i
+    assert np.isfinite(results[0][0]) and all(np.isfinite(g).all() for g in results[0][2:])
+    del results
+    after = []
+    for fused in (False, True):
+        step = configs.wide_resnet(128, fused=fused, flags=configs.REWRITES)
+        step.run(1)
+        after.append((step.loss_value(), [p.value.copy() for p in step.params]))
+        del step
+    assert after[0][0] == after[1][0]
+    for i, (a, b) in enumerate(zip(after[0][1], after[1][1])):
+        assert np.array_equal(a, b), i
+
+
 # ------------------------------------------------------------------------------ evaluation path
 @pytest.mark.parametrize("flags", [0, core.PLAN_VIEWS | core.PLAN_FUSE])
 def test_eval_plan_uses_running_statistics(flags):

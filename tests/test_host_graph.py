@@ -122,6 +122,39 @@ def test_vgg16_step_census_matches_the_reference_graph():
     assert len(net.paramProj) == 26                    # running mean / variance of 13 BN layers
 
 
+def test_wide_resnet_28_10_step_census_matches_the_reference_graph():
+    """nnet/models/wrn.d:56-219 with the default options: a 3 -> 16 stem, three stages of four pre-activation
+    blocks (widths 160 / 320 / 640, strides 1 / 2 / 2), a 1x1 projection from the block input wherever the
+    width changes, batch norm + relu + mean pool, dense(10); no convolution has a bias, every one has weight decay."""
+    init = nnet.Init(0)
+    features, labels = float32([128, 3, 32, 32]), float32([128, 10])
+    preds = nnet.softmax(nnet.dense(nnet.wideResNet(features, 28, 10, init), 10, init))
+    net = nnet.DAGNetwork([features], [preds])
+    loss = nnet.crossEntropy(preds.trainOutput, labels) + net.paramLoss
+    grads = grad(loss, net.params)
+    c = census([loss] + grads)
+    convs = 1 + 3 * 4 * 2 + 3                                       # stem, two per block, three projections
+    bns = 3 * 4 * 2 + 1                                             # two per block, one before the pool
+    assert c["convolution"] == convs and c["convolutionFiltersGrad"] == convs
+    assert c["convolutionFeaturesGrad"] == convs - 1                # the stem's input needs no gradient
+    assert c["batchNormTrain"] == bns and c["batchNormGrad"] == bns
+    assert c["relu"] == bns and c["reluGrad"] == bns
+    assert c["addBias"] == 0 and c["maxpool"] == 0
+    assert len(net.params) == convs + 4 * bns + 2
+    assert len(net.paramProj) == 2 * bns
+    stats = sum(p.volume for p in net.paramProj)                   # running means and variances
+    assert stats == 17952 and sum(p.volume for p in net.params) - stats == 36479194
+    shapes = sorted({tuple(p.shape) for p in net.params if p.rank == 4 and p.shape[2] == 3})
+    assert shapes == [(16, 3, 3, 3), (160, 16, 3, 3), (160, 160, 3, 3), (320, 160, 3, 3), (320, 320, 3, 3),
+                      (640, 320, 3, 3), (640, 640, 3, 3)]
+    strides = collections.Counter(tuple(o.attributes["stride"]) for o in core.topological_sort([loss])
+                                  if o.opType == "convolution")
+    assert strides == {(1, 1): convs - 4, (2, 2): 4}                # two stage entries, 3x3 and 1x1 each
+    # weight decay: one sum(w * w) per convolution, plus the cross entropy's sum; the mean pool's row sums are
+    # rank-2 single-axis sums, which the op constructor turns into products with a ones vector
+    assert c["sum"] == convs + 1
+
+
 def test_op_graph_optimizers_have_the_reference_shape():
     w = float32([5, 4])
     loss = core.sum(w * w)
