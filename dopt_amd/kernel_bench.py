@@ -19,6 +19,24 @@ import numpy as np
 from . import capi, ops, workloads
 
 HBM_PEAK = 8.0e12
+MFMA_FP32_PEAK = 157.3e12
+
+# [M, K] x [K, N] products: cubes, the dense layers of the MLP configuration (forward and the two gradient
+# products of the widest layer), and the dense form of a 3x3 convolution over 2x2 images at batch 128
+GEMM_SHAPES = [(1024, 1024, 1024), (2048, 2048, 2048), (4096, 4096, 4096), (8192, 8192, 8192),
+               (256, 512, 784), (256, 512, 512), (256, 10, 512), (784, 512, 256), (256, 784, 512),
+               (128, 2048, 2048), (2048, 2048, 128)]
+
+
+def gemm_rows():
+    """(M, N, K, seconds-callable) per product, C = A . B through dopt_hip_sgemm."""
+    rows, keep = [], []
+    for (M, N, K) in GEMM_SHAPES:
+        a, b = _rand((M, K), 11), _rand((K, N), 12)
+        o = ops.matmul(a, b)
+        keep += [a, b, o]
+        rows.append((M, N, K, (lambda a=a, b=b, o=o: ops.matmul(a, b, out=o))))
+    return rows, keep
 
 
 def _time(fn, iters, warm=5):
@@ -107,7 +125,24 @@ def main():
     ap.add_argument("--iters", type=int, default=50)
     ap.add_argument("--scale", type=int, default=1, help="multiply the leading dimension of the activation shapes")
     ap.add_argument("--json", action="store_true")
+    ap.add_argument("--gemm", action="store_true", help="the fp32 matrix products against the MFMA roofline instead")
     args = ap.parse_args()
+    if args.gemm:
+        rows, keep = gemm_rows()
+        res = []
+        for M, N, K, fn in rows:
+            sec = _time(fn, args.iters)
+            res.append({"M": M, "N": N, "K": K, "us": sec * 1e6, "TFLOP/s": 2.0 * M * N * K / sec / 1e12,
+                        "frac_of_157.3": 2.0 * M * N * K / sec / MFMA_FP32_PEAK})
+        ops.sync()
+        if args.json:
+            print(json.dumps(res))
+            return
+        print("%-28s %10s %10s %8s" % ("matmul [M,K] x [K,N]", "us", "TFLOP/s", "of peak"))
+        for r in res:
+            print("%-28s %10.1f %10.1f %7.1f%%" % ("[%d,%d] x [%d,%d]" % (r["M"], r["K"], r["K"], r["N"]), r["us"], r["TFLOP/s"],
+                                                    100 * r["frac_of_157.3"]))
+        return
     out = []
     rows, keep = cases(args.scale)
     for name, shape, nbytes, fn in rows:
