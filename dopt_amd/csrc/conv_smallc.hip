@@ -34,29 +34,38 @@ struct SmallC {
     int G, groups_per_image;       // forward: sub-tiles per block (one per wavefront)
 };
 
-// zero-bordered input rows p0-1 .. p0+rows of image n.  U loads per thread are issued before the
-// first is used (clamped addresses instead of branches): a plain loop would wait out the memory
-// latency once per element.
+// Zero-bordered input rows p0-1 .. p0+rows of image n into xs[c][rows + 2][W + 2].  Image rows are whole
+// 16-byte quads (W is a power of two >= 8, x is 16-byte aligned), so a thread's unit is a quad and its
+// coordinates are shifts and compares; U quads per thread are in flight before the first is used.
+// Rows outside the image arrive as zeros (clamped address, value masked), the border columns are
+// written separately.
 template <int U>
 __device__ __forceinline__ void load_patch(const SmallC &p, int n, int p0, int rows, int nthreads, float *xs)
 {
-    const int PW = p.W + 2, PR = rows + 2, per_c = PR * PW, total = p.C * per_c;
+    const int PW = p.W + 2, PR = rows + 2, qshift = p.wshift - 2, qmask = (1 << qshift) - 1;
+    const int nrows = p.C * PR, total = nrows << qshift;
     for (int base = threadIdx.x; base < total; base += U * nthreads) {
-        float v[U];
-        bool in[U];
+        float4 v[U];
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int i = min(base + u * nthreads, total - 1);
-            const int c = i / per_c, rem = i - c * per_c, rr = rem / PW, cc = rem - rr * PW;
-            const int row = p0 - 1 + rr, col = cc - 1;
-            in[u] = row >= 0 && row < p.H && col >= 0 && col < p.W;
-            v[u] = p.x[((size_t)(n * p.C + c) * p.H + min(max(row, 0), p.H - 1)) * p.W + min(max(col, 0), p.W - 1)];
+            const int r = i >> qshift, q = i & qmask;
+            const int c = (r >= PR) + (r >= 2 * PR), row = p0 - 1 + (r - c * PR);
+            v[u] = *(const float4 *)(p.x + ((size_t)(n * p.C + c) * p.H + min(max(row, 0), p.H - 1)) * p.W + 4 * q);
+            if (row < 0 || row >= p.H) v[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int i = base + u * nthreads;
-            if (i < total) xs[i] = in[u] ? v[u] : 0.0f;
+            if (i < total) {
+                float *d = xs + (i >> qshift) * PW + 1 + 4 * (i & qmask);
+                d[0] = v[u].x; d[1] = v[u].y; d[2] = v[u].z; d[3] = v[u].w;
+            }
         }
+    }
+    for (int r = threadIdx.x; r < nrows; r += nthreads) {
+        xs[r * PW] = 0.0f;
+        xs[r * PW + PW - 1] = 0.0f;
     }
 }
 
@@ -91,15 +100,12 @@ __global__ __launch_bounds__(512) void smallc_fwd_k(SmallC p)
         for (int u = 0; u < 14; u++)
             if ((int)threadIdx.x + u * nthreads < count) ws[threadIdx.x + u * nthreads] = v[u];
     }
-    load_patch<8>(p, n, p0, p.G * p.RT, nthreads, xs);
-    // accumulators start at the bias of their row
-    v16f acc[4];
+    load_patch<2>(p, n, p0, p.G * p.RT, nthreads, xs);
+    float bv[16];   // accumulators start at the bias of their row
 #pragma unroll
     for (int v = 0; v < 16; v++) {
         const int k = k0 + acc_row(v, lane);
-        const float bv = p.bias ? p.bias[min(k, p.K - 1)] : 0.0f;
-#pragma unroll
-        for (int j = 0; j < 4; j++) acc[j][v] = bv;
+        bv[v] = p.bias ? p.bias[min(k, p.K - 1)] : 0.0f;
     }
     __syncthreads();
 
@@ -115,26 +121,25 @@ __global__ __launch_bounds__(512) void smallc_fwd_k(SmallC p)
         const float wv = ws[(min(r32, krows - 1) * p.C + (live ? c : 0)) * 9 + (2 - r) * 3 + (2 - s)];
         aw[t] = (live && r32 < krows) ? wv : 0.0f;
     }
-    // four 32-pixel columns of this wavefront's sub-tile
-    int poff[4];
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int px = wave * kPix + j * 32 + r32;
-        poff[j] = (px >> p.wshift) * (p.W + 2) + (px & (p.W - 1));
-    }
-#pragma unroll
-    for (int t = 0; t < kSteps; t++)
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-            acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(aw[t], xs[poff[j] + koff[t]], acc[j], 0, 0, 0);
+    // Four 32-pixel columns of this wavefront's sub-tile, one after the other: the stores of a finished
+    // column drain while the next one multiplies (with all four columns multiplied first and stored last,
+    // every wavefront of the chip computed at the same time and then wrote at the same time).
     const size_t plane = (size_t)p.H * p.W;
     float *out = p.y + ((size_t)n * p.K + k0) * plane + (size_t)p0 * p.W + wave * kPix + r32;
 #pragma unroll
-    for (int v = 0; v < 16; v++) {
-        const int kr = acc_row(v, lane);
-        if (kr < krows) {
+    for (int j = 0; j < 4; j++) {
+        const int px = wave * kPix + j * 32 + r32;
+        const int poff = (px >> p.wshift) * (p.W + 2) + (px & (p.W - 1));
+        v16f acc;
 #pragma unroll
-            for (int j = 0; j < 4; j++) out[(size_t)kr * plane + j * 32] = acc[j][v];
+        for (int v = 0; v < 16; v++) acc[v] = bv[v];
+#pragma unroll
+        for (int t = 0; t < kSteps; t++)
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(aw[t], xs[poff + koff[t]], acc, 0, 0, 0);
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int kr = acc_row(v, lane);
+            if (kr < krows) out[(size_t)kr * plane + j * 32] = acc[v];
         }
     }
 }
@@ -160,9 +165,14 @@ __global__ __launch_bounds__(kThreads) void smallc_wgrad_k(SmallC p)
     const bool active = xcd_remap(blockIdx.x, (unsigned)p.blocks, &L);
     const int first = active ? (int)L * p.tiles_per_block : 0;
     const int last = active ? min(first + p.tiles_per_block, p.tiles) : 0;
-    // dy of a sub-tile: 64 rows of 128 consecutive floats, eight 16-byte loads per thread, fetched one
-    // sub-tile ahead so that the loads are in flight while the current one multiplies
+    // dy of a sub-tile (64 rows of 128 consecutive floats, eight 16-byte loads per thread) and the input
+    // patch under it (at most 288 quads, two per thread) are fetched one sub-tile ahead, so
+    // that the loads are in flight while the current one multiplies
+    constexpr int XQ = 2;   // at most 3 channels x 3 rows x 32 quads (W = 128) for 256 threads
+    const int PW = p.W + 2, PR = p.RT + 2, qshift = p.wshift - 2, qmask = (1 << qshift) - 1;
+    const int prows = p.C * PR, pquads = prows << qshift;
     float4 pre[8];
+    float4 xq[XQ];
     auto fetch = [&](int tile) {
         const int n = tile / p.tiles_per_image, p0 = (tile % p.tiles_per_image) * p.RT;
 #pragma unroll
@@ -170,10 +180,22 @@ __global__ __launch_bounds__(kThreads) void smallc_wgrad_k(SmallC p)
             const int f = i * kThreads + threadIdx.x, k = f >> 5, q4 = f & 31;
             pre[i] = *(const float4 *)(p.dy + ((size_t)n * p.K + min(k, p.K - 1)) * plane + (size_t)p0 * p.W + q4 * 4);
         }
+#pragma unroll
+        for (int u = 0; u < XQ; u++) {   // the same quads, rows and masks as load_patch
+            const int i = min((int)threadIdx.x + u * kThreads, pquads - 1);
+            const int r = i >> qshift, q = i & qmask;
+            const int c = (r >= PR) + (r >= 2 * PR), row = p0 - 1 + (r - c * PR);
+            xq[u] = *(const float4 *)(p.x + ((size_t)(n * p.C + c) * p.H + min(max(row, 0), p.H - 1)) * p.W + 4 * q);
+            if (row < 0 || row >= p.H) xq[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
     };
+    // the border columns of xs stay zero for the whole kernel
+    for (int r = threadIdx.x; r < prows; r += kThreads) {
+        xs[r * PW] = 0.0f;
+        xs[r * PW + PW - 1] = 0.0f;
+    }
     if (first < last) fetch(first);
     for (int tile = first; tile < last; tile++) {
-        const int n = tile / p.tiles_per_image, p0 = (tile % p.tiles_per_image) * p.RT;
         __syncthreads();   // the previous sub-tile's readers are done
 #pragma unroll
         for (int i = 0; i < 8; i++) {
@@ -185,7 +207,14 @@ __global__ __launch_bounds__(kThreads) void smallc_wgrad_k(SmallC p)
             d[2] = row ? pre[i].z : 0.0f;
             d[3] = row ? pre[i].w : 0.0f;
         }
-        load_patch<3>(p, n, p0, p.RT, kThreads, xs);
+#pragma unroll
+        for (int u = 0; u < XQ; u++) {
+            const int i = threadIdx.x + u * kThreads;
+            if (i < pquads) {
+                float *d = xs + (i >> qshift) * PW + 1 + 4 * (i & qmask);
+                d[0] = xq[u].x; d[1] = xq[u].y; d[2] = xq[u].z; d[3] = xq[u].w;
+            }
+        }
         __syncthreads();
         if (tile + 1 < last) fetch(tile + 1);
 #pragma unroll
@@ -257,7 +286,7 @@ int conv_smallc_fwd(const dopt_hip_conv_desc *d, const float *x, const float *w,
 {
     SmallC p{};
     *done = false;
-    if (!smallc_setup(d, &p)) return DOPT_HIP_OK;
+    if (!smallc_setup(d, &p) || !aligned16(x)) return DOPT_HIP_OK;
     p.x = x; p.w = w; p.bias = bias; p.y = y;
     p.G = 1;
     for (int g = 2; g <= 8; g++)
@@ -274,7 +303,7 @@ int conv_smallc_wgrad(const dopt_hip_conv_desc *d, const float *dy, const float 
 {
     SmallC p{};
     *done = false;
-    if (!smallc_setup(d, &p) || !aligned16(dy)) return DOPT_HIP_OK;
+    if (!smallc_setup(d, &p) || !aligned16(dy) || !aligned16(x)) return DOPT_HIP_OK;
     const int want = num_cus();
     p.tiles_per_block = (p.tiles + want - 1) / want;
     const int blocks = (p.tiles + p.tiles_per_block - 1) / p.tiles_per_block;
