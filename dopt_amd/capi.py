@@ -104,6 +104,8 @@ PROTOTYPES = {
     "dopt_hip_bn_grad": [_sz, _sz, _sz, _vp, _vp, _vp, _vp],
     "dopt_hip_bn_grad_relu": [_sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_bn_grad_fused": [_sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp],
+    "dopt_hip_bn_train_pool": [_sz, _sz, _sz, _sz, _d, _vp, C.POINTER(SplitSum), _vp, _vp, _vp, _vp, _vp, _i, _vp],
+    "dopt_hip_bn_grad_pool": [_sz, _sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_bn_train_open": [_sz, _sz, _sz, _d, C.POINTER(SplitSum), _vp, _vp, _vp, _vp, _vp, _i],
     "dopt_hip_bn_grad_open": [_sz, _sz, _sz, C.POINTER(SplitSum), _i, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_bn_wait_limit": [C.c_uint],

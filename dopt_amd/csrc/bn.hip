@@ -11,6 +11,7 @@
 //      small per-channel outputs, and writes a per-channel coefficient table;
 //   3. apply: a flat 128-bit streaming pass over the tensor using the table.
 #include "common.h"
+#include "pool2x2.h"
 
 namespace {
 
@@ -45,6 +46,65 @@ __device__ inline float masked(float g, float y) { return y > 0.0f ? g : 0.0f; }
 __device__ inline float4 masked4(float4 g, float4 y)
 {
     return make_float4(masked(g.x, y.x), masked(g.y, y.y), masked(g.z, y.z), masked(g.w, y.w));
+}
+
+// A 2 x 2 max-pool riding on the quads of a register-resident batch norm: forward, the pooled value of the
+// kernel's own output y is written as well; backward, dy is not read but made from the gradient of the
+// pooled tensor, routed to the element of y the pool selected.  A lane holds four consecutive values of
+// one image row; the other row of its two windows sits `wq` lanes away in the same wavefront (wq = W / 4
+// quads per row, a power of two below 64; the kernels' quad index has the lane in its low six bits and
+// planes are whole pairs of rows), so one exchange per quad serves both rows.  mode 2: the images are
+// 2 x 2, a quad is a whole image and its own window.
+struct Pool {
+    int mode;             // 0: no pooling; 1: rows of quads; 2: 2 x 2 images
+    unsigned wq, wshift;  // quads per image row and its log2 (mode 1)
+    float *pooled;        // forward: [N, C, H/2, W/2]
+    const float *dpool;   // backward: gradient of that tensor
+};
+
+__device__ inline float4 quad_xor(float4 v, unsigned lanes)
+{
+    return make_float4(__shfl_xor(v.x, (int)lanes, 64), __shfl_xor(v.y, (int)lanes, 64), __shfl_xor(v.z, (int)lanes, 64),
+                       __shfl_xor(v.w, (int)lanes, 64));
+}
+
+// Forward: y is this lane's finished quad at float4 index idx of [N, C, H, W] (absent: idx == ~0u, y
+// arbitrary).  Every lane of the wavefront must call it.  With idx = map * H * wq + h * wq + cq, idx >> wshift
+// is the row index map * H + h over the whole tensor, and H is even: its parity is the row's, its half the
+// pooled row.
+__device__ inline void pool_store(const Pool &pl, float4 y, unsigned idx)
+{
+    const bool present = idx != 0xffffffffu;
+    if (pl.mode == 2) {
+        if (present) pl.pooled[idx] = pool2x2(y.x, y.y, y.z, y.w);
+        return;
+    }
+    const float4 o = quad_xor(y, pl.wq);
+    const unsigned row = idx >> pl.wshift, cq = idx & (pl.wq - 1);
+    if (present && !(row & 1))
+        ((float2 *)pl.pooled)[(size_t)(row >> 1) * pl.wq + cq] = make_float2(pool2x2(y.x, y.y, o.x, o.y), pool2x2(y.z, y.w, o.z, o.w));
+}
+
+// Backward: the quad of dy = maxpoolGrad(dpool, y) at float4 index idx, from this lane's quad of y (zeros
+// when absent).  Every lane of the wavefront must call it.
+__device__ inline float4 pool_grad(const Pool &pl, float4 y, unsigned idx)
+{
+    const bool present = idx != 0xffffffffu;
+    float4 r;
+    if (pl.mode == 2) {
+        const float g = present ? pl.dpool[idx] : 0.0f;
+        route2x2(y.x, y.y, y.z, y.w, g, r.x, r.y, r.z, r.w);
+        return r;
+    }
+    const float4 o = quad_xor(y, pl.wq);
+    const unsigned row = present ? idx >> pl.wshift : 0u, cq = idx & (pl.wq - 1);
+    const bool odd = row & 1;
+    const float2 g = present ? ((const float2 *)pl.dpool)[(size_t)(row >> 1) * pl.wq + cq] : make_float2(0.0f, 0.0f);
+    const float4 top = odd ? o : y, bot = odd ? y : o;
+    float4 t, b;
+    route2x2(top.x, top.y, bot.x, bot.y, g.x, t.x, t.y, b.x, b.y);
+    route2x2(top.z, top.w, bot.z, bot.w, g.y, t.z, t.w, b.z, b.w);
+    return odd ? b : t;
 }
 
 // Sums four per-thread values over the block; results valid in thread 0.
@@ -434,7 +494,7 @@ __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, un
                                                        const float *x, const float *dy, const float *scale,
                                                        const float *bias, const float *run_mean, const float *run_var,
                                                        const float *ymask, int relu, float *out, float *out1, float *out2,
-                                                       float *dx_sum, OpenSum open)
+                                                       float *dx_sum, OpenSum open, Pool pool)
 {
     __shared__ float part[3][16];
     const unsigned c = blockIdx.x, T = blockDim.x, E4 = N * inner4;
@@ -451,10 +511,17 @@ __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, un
         if (q < E4) {
             if (!(kOpen && !kGrad)) xv[i] = x4[idx[i]];
             if (kGrad && !kOpen) {
-                gv[i] = g4[idx[i]];
-                if (ymask) gv[i] = masked4(gv[i], ((const float4 *)ymask)[idx[i]]);
+                if (pool.mode) gv[i] = ((const float4 *)ymask)[idx[i]];   // y for now; dy below
+                else {
+                    gv[i] = g4[idx[i]];
+                    if (ymask) gv[i] = masked4(gv[i], ((const float4 *)ymask)[idx[i]]);
+                }
             }
         }
+    }
+    if (kGrad && !kOpen && pool.mode) {   // dy = reluGrad(maxpoolGrad(dpool, y), y)
+#pragma unroll
+        for (int i = 0; i < kQ; i++) gv[i] = masked4(pool_grad(pool, gv[i], idx[i]), gv[i]);
     }
     if (kOpen) {
         float4 sum[kQ];
@@ -521,6 +588,11 @@ __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, un
             r.w = a * ((xv[i].w - mean_hi) - mean_lo) + b;
             if (relu) r = make_float4(relu1(r.x), relu1(r.y), relu1(r.z), relu1(r.w));
             o4[idx[i]] = r;
+            xv[i] = r;
+        }
+        if (pool.mode) {
+#pragma unroll
+            for (int i = 0; i < kQ; i++) pool_store(pool, xv[i], idx[i]);
         }
         if (threadIdx.x == 0) {
             const double unbiased = m > 1.0 ? var * m / (m - 1.0) : var;
@@ -617,7 +689,7 @@ __global__ __launch_bounds__(1024) void bn_cluster_k(unsigned N, unsigned C, uns
                                                       const float *scale, const float *bias, const float *run_mean,
                                                       const float *run_var, const float *ymask, int relu, float *out,
                                                       float *out1, float *out2, float *dx_sum, ClusterMem cm,
-                                                      unsigned spin_limit)
+                                                      unsigned spin_limit, Pool pool)
 {
     constexpr int kQ = kResQuads;
     __shared__ float part[3][16];
@@ -639,10 +711,17 @@ __global__ __launch_bounds__(1024) void bn_cluster_k(unsigned N, unsigned C, uns
         if (l < mine) {
             xv[i] = x4[idx[i]];
             if (kGrad) {
-                gv[i] = g4[idx[i]];
-                if (ymask) gv[i] = masked4(gv[i], ((const float4 *)ymask)[idx[i]]);
+                if (pool.mode) gv[i] = ((const float4 *)ymask)[idx[i]];   // y for now; dy below
+                else {
+                    gv[i] = g4[idx[i]];
+                    if (ymask) gv[i] = masked4(gv[i], ((const float4 *)ymask)[idx[i]]);
+                }
             }
         }
+    }
+    if (kGrad && pool.mode) {   // dy = reluGrad(maxpoolGrad(dpool, y), y)
+#pragma unroll
+        for (int i = 0; i < kQ; i++) gv[i] = masked4(pool_grad(pool, gv[i], idx[i]), gv[i]);
     }
     // the piece's own statistics: exact two-pass, as in the one-block kernel
     const double nb = 4.0 * (double)mine;
@@ -747,6 +826,11 @@ __global__ __launch_bounds__(1024) void bn_cluster_k(unsigned N, unsigned C, uns
             r.w = a * ((xv[i].w - mean_hi) - mean_lo) + b;
             if (relu) r = make_float4(relu1(r.x), relu1(r.y), relu1(r.z), relu1(r.w));
             o4[idx[i]] = r;
+            xv[i] = r;
+        }
+        if (pool.mode) {
+#pragma unroll
+            for (int i = 0; i < kQ; i++) pool_store(pool, xv[i], idx[i]);
         }
         if (threadIdx.x == 0 && piece == 0) {
             const double unbiased = m > 1.0 ? var * m / (m - 1.0) : var;
@@ -933,11 +1017,43 @@ bool open_sum(const dopt_hip_split_sum *o, size_t elems, size_t C, size_t inner,
     return true;
 }
 
+// What the caller wants pooled (null: nothing) and whether the register-resident kernels can do it on the way:
+// images of W = 4 .. 128 (a power of two) by an even H, or 2 x 2 images.
+struct PoolArg {
+    size_t H, W;
+    float *pooled;        // forward
+    const float *dpool;   // backward
+};
+
+bool pool_inline(const PoolArg *a, Pool *k)
+{
+    *k = Pool{};
+    if (!a) return false;
+    const void *ptr = a->pooled ? (const void *)a->pooled : (const void *)a->dpool;
+    if (a->H == 2 && a->W == 2) {
+        k->mode = 2;
+    } else if (a->W >= 4 && a->W <= 128 && (a->W & (a->W - 1)) == 0 && (a->H & 1) == 0 && ((uintptr_t)ptr & 7) == 0) {
+        k->mode = 1;
+        k->wq = (unsigned)(a->W / 4);
+        k->wshift = (unsigned)__builtin_ctz(k->wq);
+    } else {
+        return false;
+    }
+    k->pooled = a->pooled;
+    k->dpool = a->dpool;
+    return true;
+}
+
 int bn_train_impl(size_t N, size_t C, size_t inner, double momentum, const float *x, const float *scale,
                   const float *bias, const float *run_mean, const float *run_var, float *packed, int relu,
-                  const char *who, const dopt_hip_split_sum *x_open = nullptr)
+                  const char *who, const dopt_hip_split_sum *x_open = nullptr, const PoolArg *pool = nullptr)
 {
     size_t total = N * C * inner;
+    Pool pl;
+    const bool pool_in = pool_inline(pool, &pl);   // a resident kernel pools on the way; else a pass of its own follows
+    auto pooled_after = [&]() -> int {
+        return pool ? dopt_hip_maxpool_fwd(N, C, pool->H, pool->W, 2, 2, packed, pool->pooled) : DOPT_HIP_OK;
+    };
     DOPT_REQUIRE(total > 0, "%s: empty input", who);
     DOPT_REQUIRE(x && scale && bias && run_mean && run_var && packed, "%s: null argument", who);
     DOPT_REQUIRE(C <= 0x7fffffffu / kMaxSlices, "%s: too many channels", who);
@@ -951,9 +1067,10 @@ int bn_train_impl(size_t N, size_t C, size_t inner, double momentum, const float
             open_split_clear(x_open->partial);
             hipLaunchKernelGGL((bn_resident_k<false, true, kOpenQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N, (unsigned)C,
                                (unsigned)(inner / 4), factor, eps, x, (const float *)nullptr, scale, bias, run_mean, run_var,
-                               (const float *)nullptr, relu, packed, packed + total, packed + total + C, (float *)nullptr, os);
+                               (const float *)nullptr, relu, packed, packed + total, packed + total + C, (float *)nullptr, os,
+                               pool_in ? pl : Pool{});
             DOPT_LAUNCH_CHECK();
-            return DOPT_HIP_OK;
+            return pool_in ? DOPT_HIP_OK : pooled_after();
         }
         if (int rc = dopt_hip_split_sum_close(x_open)) return rc;
     }
@@ -961,13 +1078,14 @@ int bn_train_impl(size_t N, size_t C, size_t inner, double momentum, const float
     if (const unsigned S = cluster_pieces(N, C, inner, x, nullptr, nullptr, packed, &per)) {
         ClusterMem cm;
         if (int rc = cluster_mem(&cm)) return rc;
+        const bool in = pool_in && (pl.mode == 2 || per % (2 * pl.wq) == 0);   // pieces hold whole pairs of rows
         hipLaunchKernelGGL((bn_cluster_k<false>), dim3((unsigned)(C * S)), dim3(1024), 0, stream(), (unsigned)N, (unsigned)C,
                            (unsigned)(inner / 4), S, per, factor, eps, x, (const float *)nullptr, scale, bias, run_mean,
                            run_var, (const float *)nullptr, relu, packed, packed + total, packed + total + C,
-                           (float *)nullptr, cm, g_cluster_spin_limit);
+                           (float *)nullptr, cm, g_cluster_spin_limit, in ? pl : Pool{});
         DOPT_LAUNCH_CHECK();
         g_cluster_unchecked = true;
-        return DOPT_HIP_OK;
+        return in ? DOPT_HIP_OK : pooled_after();
     }
     if (T) {
         // small channels (two quads per thread) take the variant built for two: a third of the registers
@@ -975,14 +1093,14 @@ int bn_train_impl(size_t N, size_t C, size_t inner, double momentum, const float
             hipLaunchKernelGGL((bn_resident_k<false, false, kOpenQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N,
                                (unsigned)C, (unsigned)(inner / 4), factor, eps, x, (const float *)nullptr, scale, bias, run_mean,
                                run_var, (const float *)nullptr, relu, packed, packed + total, packed + total + C,
-                               (float *)nullptr, OpenSum{});
+                               (float *)nullptr, OpenSum{}, pool_in ? pl : Pool{});
         else
             hipLaunchKernelGGL((bn_resident_k<false, false, kResQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N,
                                (unsigned)C, (unsigned)(inner / 4), factor, eps, x, (const float *)nullptr, scale, bias, run_mean,
                                run_var, (const float *)nullptr, relu, packed, packed + total, packed + total + C,
-                               (float *)nullptr, OpenSum{});
+                               (float *)nullptr, OpenSum{}, pool_in ? pl : Pool{});
         DOPT_LAUNCH_CHECK();
-        return DOPT_HIP_OK;
+        return pool_in ? DOPT_HIP_OK : pooled_after();
     }
     // workspace: [partials C*S*4 floats | coefficient table C * 16 bytes]
     size_t part_bytes = C * kMaxSlices * 4 * sizeof(float);
@@ -996,20 +1114,35 @@ int bn_train_impl(size_t N, size_t C, size_t inner, double momentum, const float
                        C, inner, S, factor, eps, x, partial, scale, bias, run_mean, run_var, coef, packed + total,
                        packed + total + C);
     DOPT_LAUNCH_CHECK();
-    return launch_apply(total, C, inner, x, coef, packed, relu);
+    if (int rc = launch_apply(total, C, inner, x, coef, packed, relu)) return rc;
+    return pooled_after();
 }
 
 int bn_grad_impl(size_t N, size_t C, size_t inner, const float *dy, const float *ymask, const float *x,
                  const float *scale, float *packed, float *dx_sum, const char *who,
-                 const dopt_hip_split_sum *dy_open = nullptr, bool keep_dy = true)
+                 const dopt_hip_split_sum *dy_open = nullptr, bool keep_dy = true, const PoolArg *pool = nullptr)
 {
     size_t total = N * C * inner;
     DOPT_REQUIRE(total > 0, "%s: empty input", who);
-    DOPT_REQUIRE(dy && x && scale && packed, "%s: null argument", who);
+    DOPT_REQUIRE((dy || pool) && x && scale && packed, "%s: null argument", who);
     DOPT_REQUIRE(C <= 0x7fffffffu / kMaxSlices, "%s: too many channels", who);
     DOPT_ENSURE_INIT();
     double eps = (double)1e-5f;  // cudnn7.d:634
-    const unsigned T = (!ymask || aligned16(ymask)) ? resident_threads(N, C, inner, x, dy, packed) : 0;
+    unsigned T = (!ymask || aligned16(ymask)) ? resident_threads(N, C, inner, x, dy, packed) : 0;
+    Pool pl{};
+    if (pool) {
+        // dy = maxpoolGrad(dpool, y): made inside a register-resident kernel where one will run, else by a pass
+        // of its own into the output buffer, which every path below may read as dy while it writes dx (each
+        // thread reads its elements before it writes them)
+        unsigned per = 0;
+        const unsigned S = cluster_pieces(N, C, inner, x, nullptr, ymask, packed, &per);
+        const bool in = pool_inline(pool, &pl) && (S ? (pl.mode == 2 || per % (2 * pl.wq) == 0) : T != 0);
+        if (!in) {
+            pl = Pool{};
+            if (int rc = dopt_hip_maxpool_bwd(N, C, pool->H, pool->W, 2, 2, pool->dpool, ymask, packed)) return rc;
+            dy = packed;
+        }
+    }
     if (dy_open && dy_open->splits) {   // dy is still in pieces
         OpenSum os;
         if (T && N * (inner / 4) <= (size_t)kOpenQuads * T && open_sum(dy_open, total, C, inner, keep_dy, &os)) {
@@ -1017,7 +1150,7 @@ int bn_grad_impl(size_t N, size_t C, size_t inner, const float *dy, const float 
             hipLaunchKernelGGL((bn_resident_k<true, true, kOpenQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N, (unsigned)C,
                                (unsigned)(inner / 4), 0.0, eps, x, dy, scale, (const float *)nullptr,
                                (const float *)nullptr, (const float *)nullptr, ymask, 0, packed, packed + total,
-                               packed + total + C, dx_sum, os);
+                               packed + total + C, dx_sum, os, Pool{});
             DOPT_LAUNCH_CHECK();
             return DOPT_HIP_OK;
         }
@@ -1030,7 +1163,7 @@ int bn_grad_impl(size_t N, size_t C, size_t inner, const float *dy, const float 
         hipLaunchKernelGGL((bn_cluster_k<true>), dim3((unsigned)(C * S)), dim3(1024), 0, stream(), (unsigned)N, (unsigned)C,
                            (unsigned)(inner / 4), S, per, 0.0, eps, x, dy, scale, (const float *)nullptr,
                            (const float *)nullptr, (const float *)nullptr, ymask, 0, packed, packed + total,
-                           packed + total + C, dx_sum, cm, g_cluster_spin_limit);
+                           packed + total + C, dx_sum, cm, g_cluster_spin_limit, pl);
         DOPT_LAUNCH_CHECK();
         g_cluster_unchecked = true;
         return DOPT_HIP_OK;
@@ -1040,12 +1173,12 @@ int bn_grad_impl(size_t N, size_t C, size_t inner, const float *dy, const float 
             hipLaunchKernelGGL((bn_resident_k<true, false, kOpenQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N,
                                (unsigned)C, (unsigned)(inner / 4), 0.0, eps, x, dy, scale, (const float *)nullptr,
                                (const float *)nullptr, (const float *)nullptr, ymask, 0, packed, packed + total,
-                               packed + total + C, dx_sum, OpenSum{});
+                               packed + total + C, dx_sum, OpenSum{}, pl);
         else
             hipLaunchKernelGGL((bn_resident_k<true, false, kResQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N,
                                (unsigned)C, (unsigned)(inner / 4), 0.0, eps, x, dy, scale, (const float *)nullptr,
                                (const float *)nullptr, (const float *)nullptr, ymask, 0, packed, packed + total,
-                               packed + total + C, dx_sum, OpenSum{});
+                               packed + total + C, dx_sum, OpenSum{}, pl);
         DOPT_LAUNCH_CHECK();
         return DOPT_HIP_OK;
     }
@@ -1155,6 +1288,26 @@ int dopt_hip_bn_grad_open(size_t N, size_t C, size_t inner, const dopt_hip_split
     DOPT_REQUIRE(dy_open && dy_open->value, "dopt_hip_bn_grad_open: null argument");
     return bn_grad_impl(N, C, inner, dy_open->value, y, x, scale, packed, dx_sum, "dopt_hip_bn_grad_open", dy_open,
                         keep_dy != 0);
+}
+
+int dopt_hip_bn_train_pool(size_t N, size_t C, size_t H, size_t W, double momentum, const float *x,
+                           const dopt_hip_split_sum *x_open, const float *scale, const float *bias,
+                           const float *run_mean, const float *run_var, float *packed, int relu, float *pooled)
+{
+    DOPT_REQUIRE(pooled != nullptr && (x_open ? x_open->value != nullptr : x != nullptr), "dopt_hip_bn_train_pool: null argument");
+    DOPT_REQUIRE((H & 1) == 0 && (W & 1) == 0, "dopt_hip_bn_train_pool: images of %zu x %zu do not split into 2 x 2 windows", H, W);
+    const PoolArg pa{H, W, pooled, nullptr};
+    return bn_train_impl(N, C, H * W, momentum, x_open ? x_open->value : x, scale, bias, run_mean, run_var, packed, relu != 0,
+                         "dopt_hip_bn_train_pool", x_open, &pa);
+}
+
+int dopt_hip_bn_grad_pool(size_t N, size_t C, size_t H, size_t W, const float *dpooled, const float *y, const float *x,
+                          const float *scale, float *packed, float *dx_sum)
+{
+    DOPT_REQUIRE(dpooled != nullptr && y != nullptr, "dopt_hip_bn_grad_pool: null argument");
+    DOPT_REQUIRE((H & 1) == 0 && (W & 1) == 0, "dopt_hip_bn_grad_pool: images of %zu x %zu do not split into 2 x 2 windows", H, W);
+    const PoolArg pa{H, W, nullptr, dpooled};
+    return bn_grad_impl(N, C, H * W, nullptr, y, x, scale, packed, dx_sum, "dopt_hip_bn_grad_pool", nullptr, true, &pa);
 }
 
 int dopt_hip_bn_grad_fused(size_t N, size_t C, size_t inner, const float *dy, const float *y, const float *x,

@@ -5,6 +5,7 @@
 #include <cfloat>
 
 #include "common.h"
+#include "pool2x2.h"
 
 namespace {
 
@@ -219,8 +220,7 @@ __global__ __launch_bounds__(kBlock) void bias_bwd_flat_k(size_t N, size_t C, si
 }
 
 // ---------------------------------------------------------------------------------- maxpool
-// std.algorithm.max(acc, v) = acc < v ? v : acc, starting from -float.max (cpu/nnet.d:103-113).
-__device__ inline float dmax(float acc, float v) { return acc < v ? v : acc; }
+// The comparison chains (dmax, pool2x2, route2x2) live in pool2x2.h: the batch-norm kernels share them.
 
 // 2x2 windows, W % 4 == 0, 16-byte aligned: one thread makes two adjacent outputs from two float4 rows.
 __global__ __launch_bounds__(kBlock) void maxpool2x2_fwd_k(size_t maps, size_t H, size_t W, const float *x, float *y)
@@ -233,8 +233,8 @@ __global__ __launch_bounds__(kBlock) void maxpool2x2_fwd_k(size_t maps, size_t H
         const float4 *r0 = (const float4 *)(x + (m * H + 2 * p) * W) + q2;
         const float4 *r1 = (const float4 *)(x + (m * H + 2 * p + 1) * W) + q2;
         float4 a = *r0, b = *r1;
-        float o0 = dmax(dmax(dmax(dmax(-FLT_MAX, a.x), a.y), b.x), b.y);
-        float o1 = dmax(dmax(dmax(dmax(-FLT_MAX, a.z), a.w), b.z), b.w);
+        float o0 = pool2x2(a.x, a.y, b.x, b.y);
+        float o1 = pool2x2(a.z, a.w, b.z, b.w);
         ((float2 *)(y + (m * P + p) * (W >> 1)))[q2] = make_float2(o0, o1);
     }
 }
@@ -253,24 +253,6 @@ __global__ __launch_bounds__(kBlock) void maxpool_fwd_k(size_t maps, size_t H, s
             for (size_t i = 0; i < pw; i++) acc = dmax(acc, img[(p * ph + j) * W + q * pw + i]);
         y[idx] = acc;
     }
-}
-
-// Gradient goes to the element the forward pass selected: the same chain of `acc < v` tests starting from
-// -FLT_MAX, in row-major order, so the first maximum wins and an element that never compares greater (a NaN)
-// is never selected; a window in which nothing fires sends its gradient to its first element.
-__device__ inline void route2x2(float a, float b, float c, float d, float g, float &oa, float &ob, float &oc,
-                                float &od)
-{
-    int best = 0;
-    float bv = -FLT_MAX;
-    if (bv < a) { bv = a; best = 0; }
-    if (bv < b) { bv = b; best = 1; }
-    if (bv < c) { bv = c; best = 2; }
-    if (bv < d) { bv = d; best = 3; }
-    oa = best == 0 ? g : 0.0f;
-    ob = best == 1 ? g : 0.0f;
-    oc = best == 2 ? g : 0.0f;
-    od = best == 3 ? g : 0.0f;
 }
 
 // 2x2, H even, W % 4 == 0, aligned: a thread owns two adjacent windows = a float4 of each of two rows.

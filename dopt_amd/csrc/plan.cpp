@@ -542,6 +542,15 @@ std::unique_ptr<HIPKernel> make_fused(const Graph &g, int id, int kind, void *ex
                                           (const float *)in[2], (const float *)in[3], (const float *)in[4], (float *)out);
         });
     }
+    if (kind == 8) {  // batchNormGrad(reluGrad(maxpoolGrad(dp, ., y), y, .), x, scale): inputs [dp, y, x, scale]
+        const auto &xs = g.ops[op.deps[1]].shape;
+        const size_t N = xs[0], C = xs[1], H = xs[2], W = xs[3];
+        *label = std::string("maxpoolGrad+reluGrad+batchNormGrad") + (extra ? "+addBiasGrad" : "");
+        return make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_bn_grad_pool(N, C, H, W, (const float *)in[0], (const float *)in[1], (const float *)in[2],
+                                         (const float *)in[3], (float *)out, (float *)extra);
+        });
+    }
     // batchNormGrad, with reluGrad folded in (kind 3: inputs [dy, y, x, scale]; else [dy, x, scale])
     // and/or the bias gradient of the preceding addBias written to `extra`
     size_t N, C, inner;
@@ -569,7 +578,8 @@ struct HIPPlan::Builder {
 
     std::vector<Alias> alias;
     // inputsOf[id]: the operations whose buffers feed id's kernel (its deps, unless fused);
-    // fusedKind[id]: 1 conv+bias, 2 bn+relu, 3 relugrad+bngrad, 6 matmul with transposes, 7 pointwise chain
+    // fusedKind[id]: 1 conv+bias, 2 bn+relu, 3 relugrad+bngrad, 6 matmul with transposes, 7 pointwise chain,
+    // 8 maxpoolgrad+relugrad+bngrad
     std::vector<std::vector<int>> inputsOf;
     std::vector<int> fusedKind;
     std::vector<std::unique_ptr<HIPKernel>> prebuilt;
@@ -580,6 +590,7 @@ struct HIPPlan::Builder {
     std::vector<std::vector<Use>> uses;
     std::vector<std::vector<size_t>> exposed;   // byte offsets at which plan outputs (or aliases of them) expose a buffer
     std::vector<int> biasGradOf;                // batchNormGrad op -> the addBiasGrad op it serves
+    std::vector<int> poolOf;                    // batchNormTrain op -> the 2 x 2 maxpool op whose buffer its kernel fills too
     std::vector<char> absorbed;
     std::vector<char> needed;
     // late: the copy is made right in front of its first reader instead of at the start of the run
@@ -597,7 +608,7 @@ struct HIPPlan::Builder {
     Builder(const Graph &graph, HIPPlan *plan, const std::vector<int> &outs, unsigned f)
         : g(graph), p(plan), outputs(outs), flags(f), nops((int)graph.ops.size()), alias((size_t)nops),
           inputsOf((size_t)nops), fusedKind((size_t)nops, 0), prebuilt((size_t)nops), prebuiltLabel((size_t)nops),
-          live((size_t)nops, 0), uses((size_t)nops), exposed((size_t)nops), biasGradOf((size_t)nops, -1),
+          live((size_t)nops, 0), uses((size_t)nops), exposed((size_t)nops), biasGradOf((size_t)nops, -1), poolOf((size_t)nops, -1),
           absorbed((size_t)nops, 0), needed((size_t)nops, 0), packOf((size_t)nops, -1), mmInfo((size_t)nops)
     {
     }
@@ -621,6 +632,8 @@ struct HIPPlan::Builder {
     void fuseDenseLayers();
     void formChains();
     void absorbBiasGrads();
+    void absorbPools();
+    std::unique_ptr<HIPKernel> makePooledTrain(int id, std::shared_ptr<dopt_hip_split_sum> open, std::string *label);
     void markNeeded();
     int prepackFilters();
     int allocateBuffers();
@@ -736,6 +749,20 @@ void HIPPlan::Builder::fusePairs()
                 !isOutput(rg) && uses[rg].size() == 1 && rgo.volume() == g.ops[op.deps[1]].volume()) {
                 fusedKind[id] = 3;
                 inputsOf[id] = {rgo.deps[0], rgo.deps[1], op.deps[1], op.deps[2]};
+                // ... and the gradient of a 2 x 2 max-pool of that relu output in front of the reluGrad: the kernel
+                // routes the pooled tensor's gradient itself and the full-size gradient of the pool is never stored
+                size_t moff, yoff1, yoff2;
+                const int mg = root(rgo.deps[0], &moff);
+                const Operation &mgo = g.ops[mg];
+                const auto *dims = sizes_attr(mgo, "dims");
+                const auto &xs = g.ops[op.deps[1]].shape;
+                if (mgo.opType == "maxpoolGrad" && mgo.deps.size() == 3 && moff == 0 && alias[mg].source < 0 && !isOutput(mg) &&
+                    uses[mg].size() == 1 && mgo.dtype == DOPT_HIP_F32 && dims && dims->size() == 2 && (*dims)[0] == 2 &&
+                    (*dims)[1] == 2 && xs.size() == 4 && xs[2] % 2 == 0 && xs[3] % 2 == 0 && g.ops[mgo.deps[2]].shape == xs &&
+                    root(mgo.deps[2], &yoff1) == root(rgo.deps[1], &yoff2) && yoff1 == yoff2) {
+                    fusedKind[id] = 8;
+                    inputsOf[id] = {mgo.deps[0], rgo.deps[1], op.deps[1], op.deps[2]};
+                }
             }
         }
     }
@@ -903,7 +930,7 @@ void HIPPlan::Builder::formChains()
         if (!live[id] || alias[id].source >= 0 || fusedKind[id] || o.dtype != DOPT_HIP_F32 || o.volume() == 0) return false;
         if (o.opType == "reluGrad" && o.deps.size() == 3) {
             for (const Use &u : uses[id])
-                if (fusedKind[u.op] == 3) return false;   // that batchNormGrad reads dy and y itself
+                if (fusedKind[u.op] == 3 || fusedKind[u.op] == 8) return false;   // that batchNormGrad reads dy and y itself
             return true;
         }
         if (outer_cols(id)) return true;
@@ -1027,6 +1054,29 @@ void HIPPlan::Builder::absorbBiasGrads()
     }
 }
 
+void HIPPlan::Builder::absorbPools()
+{
+    // maxpool [2, 2] of a batch norm's y part (through the relu that became an alias of it, or directly): the
+    // batch-norm kernel has the values in registers and writes the pooled tensor too.  The maxpool operation
+    // keeps its buffer but gets no kernel of its own.
+    if (!(flags & DOPT_HIP_PLAN_FUSE)) return;
+    for (int id : p->mOps) {
+        const Operation &op = g.ops[id];
+        if (op.opType != "maxpool" || op.deps.size() != 1 || alias[id].source >= 0 || op.dtype != DOPT_HIP_F32) continue;
+        const auto *dims = sizes_attr(op, "dims");
+        const auto &xs = g.ops[op.deps[0]].shape;
+        if (!dims || dims->size() != 2 || (*dims)[0] != 2 || (*dims)[1] != 2 || xs.size() != 4 || xs[2] % 2 || xs[3] % 2) continue;
+        size_t off;
+        const int b = root(op.deps[0], &off);
+        const Operation &bn = g.ops[b];
+        if (bn.opType != "batchNormTrain" || bn.deps.size() != 5 || off != 0 || poolOf[b] >= 0 || prebuilt[b] ||
+            (fusedKind[b] != 0 && fusedKind[b] != 2) || g.ops[bn.deps[0]].shape != xs || op.volume() == 0)
+            continue;
+        poolOf[b] = id;
+        absorbed[id] = 1;
+    }
+}
+
 void HIPPlan::Builder::markNeeded()
 {
     // operations whose results are actually consumed (everything, unless rewrites created dead ones)
@@ -1142,6 +1192,29 @@ int HIPPlan::Builder::allocateBuffers()
     return DOPT_HIP_OK;
 }
 
+// batchNormTrain (+ relu) whose kernel also fills the buffer of the maxpool behind it; `open`: its input is a
+// convolution result that may arrive as partial copies (see openSplitSums).
+std::unique_ptr<HIPKernel> HIPPlan::Builder::makePooledTrain(int id, std::shared_ptr<dopt_hip_split_sum> open, std::string *label)
+{
+    const Operation &op = g.ops[id];
+    auto it = op.doubleAttrs.find("momentum");
+    if (it == op.doubleAttrs.end()) {
+        fail(DOPT_HIP_ERR_INVALID, "batchNormTrain has no 'momentum' attribute");
+        return nullptr;
+    }
+    const double momentum = it->second;
+    const auto &xs = g.ops[op.deps[0]].shape;
+    const size_t N = xs[0], C = xs[1], H = xs[2], W = xs[3];
+    const int relu = fusedKind[id] == 2;
+    float *pooled = (float *)p->mResults[poolOf[id]];
+    *label = std::string("batchNormTrain") + (relu ? "+relu" : "") + "+maxpool";
+    return make([=](const std::vector<const void *> &in, void *out) {
+        if (open && open->value != in[0]) return fail(DOPT_HIP_ERR_RUNTIME, "plan: open convolution result is not the batch norm's input");
+        return dopt_hip_bn_train_pool(N, C, H, W, momentum, (const float *)in[0], open.get(), (const float *)in[1],
+                                      (const float *)in[2], (const float *)in[3], (const float *)in[4], (float *)out, relu, pooled);
+    });
+}
+
 int HIPPlan::Builder::buildSteps()
 {
     // kernels and buffers
@@ -1155,7 +1228,7 @@ int HIPPlan::Builder::buildSteps()
             continue;
         }
         if (alias[id].source >= 0) continue;  // resolved per execution
-        if (absorbed[id]) continue;           // written by the batchNormGrad kernel it follows
+        if (absorbed[id]) continue;           // written by the batch-norm kernel it follows
         std::unique_ptr<HIPKernel> k;
         std::string label = op.opType;
         void *extra = biasGradOf[id] >= 0 && needed[biasGradOf[id]] ? p->mResults[biasGradOf[id]] : nullptr;
@@ -1188,6 +1261,8 @@ int HIPPlan::Builder::buildSteps()
         } else if (prebuilt[id]) {
             k = std::move(prebuilt[id]);
             label = prebuiltLabel[id];
+        } else if (poolOf[id] >= 0 && needed[poolOf[id]]) {
+            k = makePooledTrain(id, nullptr, &label);
         } else if (fusedKind[id] || extra) {
             k = make_fused(g, id, fusedKind[id], extra, &label);
         } else {
@@ -1254,11 +1329,16 @@ void HIPPlan::Builder::openSplitSums()
                 return dopt_hip_conv_fwd_bias_packed_open(&d, (const float *)in[0], packed, bias ? (const float *)in[1] : nullptr,
                                                           (float *)out, open.get());
             });
-            next.kernel = make([=](const std::vector<const void *> &in, void *out) {
-                if (open->value != in[0]) return fail(DOPT_HIP_ERR_RUNTIME, "plan: open convolution result is not the batch norm's input");
-                return dopt_hip_bn_train_open(N, C, inner, momentum, open.get(), (const float *)in[1], (const float *)in[2],
-                                              (const float *)in[3], (const float *)in[4], (float *)out, relu);
-            });
+            if (poolOf[b] >= 0 && needed[poolOf[b]]) {
+                std::string unused;
+                next.kernel = makePooledTrain(b, open, &unused);
+            } else {
+                next.kernel = make([=](const std::vector<const void *> &in, void *out) {
+                    if (open->value != in[0]) return fail(DOPT_HIP_ERR_RUNTIME, "plan: open convolution result is not the batch norm's input");
+                    return dopt_hip_bn_train_open(N, C, inner, momentum, open.get(), (const float *)in[1], (const float *)in[2],
+                                                  (const float *)in[3], (const float *)in[4], (float *)out, relu);
+                });
+            }
         } else if (cs.bwd && bo.opType == "batchNormGrad" && bo.deps.size() == 3 &&
                    ((fusedKind[b] == 3 && next.inputOps.size() == 4) || (fusedKind[b] == 0 && next.inputOps.size() == 3))) {
             const bool relu = fusedKind[b] == 3;
@@ -1310,7 +1390,7 @@ int HIPPlan::Builder::assignQueues()
             for (int in : st.inputOps) reads_side = reads_side || onSide[producer(in)];
             const bool wgrad = g.ops[st.op].opType == "convolutionFiltersGrad";
             // a step with a second output (the absorbed bias gradient) stays on the main queue
-            if ((wgrad || reads_side) && biasGradOf[st.op] < 0) {
+            if ((wgrad || reads_side) && biasGradOf[st.op] < 0 && poolOf[st.op] < 0) {
                 st.lane = 1;
                 st.fenceBefore = true;
                 onSide[st.op] = 1;
@@ -1341,6 +1421,7 @@ int HIPPlan::Builder::assignQueues()
             if (op < 0) continue;
             stepOf[op] = (int)i;
             if (biasGradOf[op] >= 0) stepOf[biasGradOf[op]] = (int)i;
+            if (poolOf[op] >= 0) stepOf[poolOf[op]] = (int)i;
         }
         std::vector<std::vector<int>> readers(n), producers(n);
         for (size_t i = 0; i < n; i++)
@@ -1456,6 +1537,7 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         b.fuseDenseLayers();
         b.formChains();
         b.absorbBiasGrads();
+        b.absorbPools();
     }
     b.markNeeded();
     if (flags & DOPT_HIP_PLAN_FUSE)

@@ -355,6 +355,25 @@ def bn_grad_relu(dy, y, x, scale, out=None):
     return packed
 
 
+def bn_train_pool(x, scale, bias, run_mean, run_var, momentum, relu=True, out=None, pooled=None):
+    """batchNormTrain (+ relu) and maxpool(y, [2, 2]) in one call: (packed, pooled)."""
+    N, Cc, H, W = x.shape
+    packed = _out(out, (x.size + 2 * Cc,))
+    pooled = _out(pooled, (N, Cc, H // 2, W // 2))
+    capi.check(capi.load().dopt_hip_bn_train_pool(N, Cc, H, W, float(momentum), x.ptr, None, scale.ptr, bias.ptr,
+                                                  run_mean.ptr, run_var.ptr, packed.ptr, 1 if relu else 0, pooled.ptr))
+    return packed, pooled
+
+
+def bn_grad_pool(dpooled, y, x, scale, out=None, dx_sum=None):
+    """batchNormGrad(reluGrad(maxpoolGrad(dpooled, ., y), y, .), x, scale)."""
+    N, Cc, H, W = x.shape
+    packed = _out(out, (x.size + 2 * Cc,))
+    capi.check(capi.load().dopt_hip_bn_grad_pool(N, Cc, H, W, dpooled.ptr, y.ptr, x.ptr, scale.ptr, packed.ptr,
+                                                 dx_sum.ptr if dx_sum is not None else None))
+    return packed
+
+
 def bn_grad(dy, x, scale, out=None):
     N, Cc, inner = _nci(x.shape)
     packed = _out(out, (x.size + 2 * Cc,))

@@ -344,6 +344,23 @@ int dopt_hip_bn_train_open(size_t N, size_t C, size_t inner, double momentum, co
                            float *packed, int relu);
 int dopt_hip_bn_grad_open(size_t N, size_t C, size_t inner, const dopt_hip_split_sum *dy_open, int keep_dy,
                           const float *y, const float *x, const float *scale, float *packed, float *dx_sum);
+/* Batch norm with the 2 x 2 max-pool behind it (`maxpool` with dims [2, 2], cudnn7.d:300-357) in the same
+   launch, for [N, C, H, W] with H and W even.  No counterpart in the reference, which runs
+   cudnnBatchNormalization* and cudnnPooling* one after the other; results are bit for bit those of the
+   separate calls.
+   bn_train_pool: packed is what dopt_hip_bn_train (relu == 0) or dopt_hip_bn_train_relu writes, and
+   pooled[N, C, H/2, W/2] = maxpool(y).  x_open (optional) is an open convolution result as in
+   dopt_hip_bn_train_open; x is ignored then.
+   bn_grad_pool: batchNormGrad(reluGrad(maxpoolGrad(dpooled, ., y), y, .), x, scale) where y is the ReLU
+   output that was pooled; dx_sum as in dopt_hip_bn_grad_fused.  The [N, C, H, W] gradient of the pool is never
+   stored.
+   Images of 2 x 2, or of W = 4 .. 128 a power of two, are pooled inside the register-resident kernels;
+   other shapes run the pooling kernel as a pass of its own (for the gradient: into `packed`, in place). */
+int dopt_hip_bn_train_pool(size_t N, size_t C, size_t H, size_t W, double momentum, const float *x,
+                           const dopt_hip_split_sum *x_open, const float *scale, const float *bias,
+                           const float *run_mean, const float *run_var, float *packed, int relu, float *pooled);
+int dopt_hip_bn_grad_pool(size_t N, size_t C, size_t H, size_t W, const float *dpooled, const float *y,
+                          const float *x, const float *scale, float *packed, float *dx_sum);
 /* Channels of more than 32768 values are normalised by a few workgroups each, which meet once inside the
    kernel; a workgroup polls for its partners at most `polls` times (about a microsecond each; default
    2^21) and then gives up: the kernel still ends, and the next dopt_hip_sync or dopt_hip_copy_d2h

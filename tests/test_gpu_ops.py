@@ -540,6 +540,65 @@ def test_batchnorm_channels_spanning_several_blocks(shape):
     ops.sync()
 
 
+@pytest.mark.parametrize("shape", [(128, 8, 32, 32),    # four blocks per channel (the first pooled layer of the benchmark, fewer channels)
+                                   (40, 4, 32, 32),     # two blocks per channel
+                                   (35, 3, 30, 32),     # two blocks whose pieces split a pair of rows: pooled by a pass of its own
+                                   (64, 6, 16, 16),     # one block, eight quads per lane
+                                   (16, 5, 8, 8), (7, 3, 4, 4), (9, 4, 6, 4), (3, 2, 2, 128),   # one block, two quads per lane
+                                   (16, 12, 2, 2),      # a quad is an image
+                                   (5, 3, 4, 6), (4, 3, 4, 2), (6, 2, 6, 2), (2, 2, 2, 256)])   # shapes the resident kernels do not pool
+def test_batchnorm_with_the_pool_behind_it(shape):
+    """batchNormTrain + relu + maxpool [2,2] as one call and its gradient as one call: bit for bit the
+    separate calls, which are the ones checked against the oracle; ties, zeros and NaNs in the windows."""
+    r = rng(64)
+    N, C, H, W = shape
+    x = (r.standard_normal(shape) * 1.5 + 0.5).astype(np.float32)
+    x[:, :, : H // 2 * 2 : 2, :] = np.round(x[:, :, : H // 2 * 2 : 2, :])     # plenty of equal values inside windows
+    x[0, 0, 0, 0] = np.nan if N * H * W > 64 else x[0, 0, 0, 0]                # poisons channel 0 only
+    gamma, beta, rm = (r.standard_normal(C).astype(np.float32) for _ in range(3))
+    rv = (r.random(C) + 0.5).astype(np.float32)
+    mom = float(np.float32(0.9))
+    tx, tg, tb, trm, trv = T(x), T(gamma), T(beta), T(rm), T(rv)
+    vol = x.size
+    for relu in (True, False):
+        sep = ops.bn_train_relu(tx, tg, tb, trm, trv, mom) if relu else ops.bn_train(tx, tg, tb, trm, trv, mom)
+        sep_pool = ops.maxpool(sep.view(0, shape), (2, 2))
+        packed, pooled = ops.bn_train_pool(tx, tg, tb, trm, trv, mom, relu=relu)
+        assert np.array_equal(packed.numpy(), sep.numpy(), equal_nan=True), relu
+        assert np.array_equal(pooled.numpy(), sep_pool.numpy(), equal_nan=True), relu
+    # the oracle's view of the fused forward (channels without the NaN)
+    want = O.bn_train(x[:, 1:], gamma[1:], beta[1:], rm[1:], rv[1:], mom)
+    yo = O.relu(want[: x[:, 1:].size].reshape(x[:, 1:].shape))
+    packed, pooled = ops.bn_train_pool(tx, tg, tb, trm, trv, mom)
+    y = packed.view(0, shape)
+    assert_close(y.numpy()[:, 1:], yo, "bn + relu y")
+    assert np.array_equal(pooled.numpy()[:, 1:], O.maxpool(np.ascontiguousarray(y.numpy()[:, 1:]), (2, 2)))
+    # gradient: dy of the pooled tensor at the scale a mean loss hands down
+    dp = (r.standard_normal((N, C, H // 2, W // 2)) / (N * H * W)).astype(np.float32)
+    tdp = T(dp)
+    full = ops.maxpool_grad(tdp, y, (2, 2))
+    sep, sep_sum = ops.Tensor((vol + 2 * C,)), ops.Tensor((C,))
+    import ctypes as C_
+    from dopt_amd import capi
+    lib = capi.load()
+    capi.check(lib.dopt_hip_bn_grad_fused(N, C, H * W, full.ptr, y.ptr, tx.ptr, tg.ptr, sep.ptr, sep_sum.ptr))
+    dxs = ops.Tensor((C,))
+    got = ops.bn_grad_pool(tdp, y, tx, tg, dx_sum=dxs)
+    assert np.array_equal(got.numpy(), sep.numpy(), equal_nan=True)
+    assert np.array_equal(dxs.numpy(), sep_sum.numpy(), equal_nan=True)
+    got2 = ops.bn_grad_pool(tdp, y, tx, tg)      # without the sum of dx
+    assert np.array_equal(got2.numpy(), sep.numpy(), equal_nan=True)
+    # and against the oracle, composed operation by operation
+    yh = np.ascontiguousarray(y.numpy()[:, 1:])
+    gw = O.bn_grad(O.relu_grad(O.maxpool_grad(np.ascontiguousarray(dp[:, 1:]), yh, (2, 2)), yh),
+                   np.ascontiguousarray(x[:, 1:]), gamma[1:])
+    sub = x[:, 1:].size
+    assert_close(got.numpy()[:vol].reshape(shape)[:, 1:].ravel(), gw[:sub], "bn dx behind relu and pool")
+    assert_close(got.numpy()[vol + 1:vol + C], gw[sub:sub + C - 1], "bn dscale behind relu and pool")
+    assert_close(got.numpy()[vol + C + 1:], gw[sub + C - 1:], "bn dbias behind relu and pool")
+    ops.sync()
+
+
 def test_batchnorm_blocks_that_do_not_meet_are_reported_and_recovered_from():
     """The blocks sharing a channel wait for each other a bounded number of polls.  With the bound at zero
     every block gives up at once (each still finishes and exits): the next synchronisation reports it, and
