@@ -323,6 +323,32 @@ def test_plan_fusion_does_not_change_results():
     assert kernels[2] <= kernels[1] - 12 - 8, kernels
 
 
+def test_pools_ride_in_the_batch_norm_kernels():
+    """With the rewrites on, the 2 x 2 max-pools of a VGG block and their gradients have no kernels of their
+    own: the batch norm in front pools, the batch-norm gradient routes.  (That the values do not change is the
+    test above and the configuration tests; this one checks that the rewrite really fires.)"""
+    r = np.random.default_rng(83)
+    X = r.standard_normal((8, 3, 8, 8)).astype(np.float32)
+    Y = np.zeros((8, 10), np.float32)
+    Y[np.arange(8), r.integers(0, 10, 8)] = 1
+    feats, labels = float32([8, 3, 8, 8]), float32([8, 10])
+    init = nnet.Init(84)
+    body = nnet.vgg(feats, [16, -1, 32, 32, -1], [24], init)
+    preds = nnet.softmax(nnet.dense(body, 10, init))
+    net = nnet.DAGNetwork([feats], [preds])
+    loss = nnet.crossEntropy(preds.trainOutput, labels) + net.paramLoss
+    outs = [loss] + core.grad(loss, net.params)
+    plan = core.compile(outs, core.PLAN_VIEWS | core.PLAN_FUSE | core.PLAN_TIMING)
+    fused = plan.execute({feats: X, labels: Y})
+    prof = plan.profile()
+    assert prof["batchNormTrain+relu+maxpool"][1] == 2, prof
+    assert prof["maxpoolGrad+reluGrad+batchNormGrad+addBiasGrad"][1] == 2, prof
+    assert "maxpool" not in prof and "maxpoolGrad" not in prof, prof
+    plain = core.compile(outs, core.PLAN_VIEWS).execute({feats: X, labels: Y})
+    for a, b in zip(plain, fused):
+        assert np.array_equal(a, b) or (a.ndim == 1 and np.allclose(a, b, rtol=0, atol=2e-5))
+
+
 def test_packed_filter_entry_points_match_the_unpacked_ones():
     """dopt_hip_conv_pack_batch + the *_packed entry points against dopt_hip_conv_fwd_bias /
     dopt_hip_conv_bwd_data (themselves checked against the oracle in test_gpu_ops.py): same kernels,
