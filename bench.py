@@ -212,8 +212,14 @@ def main():
         ops.sync()
         before = tstep.updater.plan.profile()
         nsteps = max(3, min(a.steps, 10))
+        lib = capi.load()
+        capi.check(lib.dopt_hip_conv_pair_probe(1))      # events around every conv_bwd_pair_k launch, on its own stream
         tstep.run(nsteps)
         ops.sync()
+        import ctypes as C
+        pl, pus, pfl, pby = C.c_int(), C.c_double(), C.c_double(), C.c_double()
+        capi.check(lib.dopt_hip_conv_pair_probe_read(C.byref(pl), C.byref(pus), C.byref(pfl), C.byref(pby)))
+        capi.check(lib.dopt_hip_conv_pair_probe(0))
         after = tstep.updater.plan.profile()
         per_shape = {k: ((after[k][0] - before.get(k, (0, 0))[0]) / nsteps, (after[k][1] - before.get(k, (0, 0))[1]) // nsteps)
                      for k in after}
@@ -222,66 +228,70 @@ def main():
             name = k.split("@")[0]
             per_op[name] = (per_op.get(name, (0.0, 0))[0] + us, per_op.get(name, (0.0, 0))[1] + n)
 
-        # The dominant kernel: conv_patch_k with 128 x 128 tiles = every 3x3 convolution whose GEMM has at
-        # least 128 rows (output channels forward, input channels backward-data) on images of 4x4 pixels and
-        # more: forward layers 3-10 and backward-data layers 4-10, 15 launches per step.  Its steps hold
-        # nothing else (filters are packed by a step of their own; where a reduction is split the partial sums
-        # are added by the batch norm behind it), and the kernel multiplies every tap of every pixel, padding
-        # included, so the conventional FLOP count below is also the executed one.
-        flops = us = launches = bytes_alg = 0
+        def profile_line(tag):
+            """A figure of the committed rocprofv3 --pmc summary (FETCH_SIZE / WRITE_SIZE calibrated against a plain
+            copy): NOT measured in this run."""
+            tpath = os.path.join(ROOT, "profiles", "conv_kernels_vgg16_b128_hbm_traffic.txt")
+            if os.path.exists(tpath):
+                for line in open(tpath):
+                    if line.startswith(tag + " "):
+                        return int(line.split()[-1])
+            return None
+
+        # The dominant kernel, by its share of the step: conv_bwd_pair_k, the backward-data convolution and the filter
+        # gradient of one layer in one launch (128 x 128 backward-data tiles first, 128 x 32 x 9 filter-gradient tiles
+        # behind them on the same compute units): layers 4-10 of the 13, 7 launches per step.  Timed by events recorded
+        # around each launch inside the library, on the stream the kernel runs on (the step around it also runs the split
+        # sum of the filter gradient, which is not part of this figure).  FLOPs are the executed ones: both products
+        # multiply every tap of every pixel, zero padding included.
+        launches = pl.value / nsteps if nsteps else 0
+        tflops = pfl.value / (pus.value * 1e-6) / 1e12 if pus.value else 0.0
+        result["roofline"] = {
+            "kernel": "conv_bwd_pair_k<Tile<128,128,2,4>,16,4,1,*>: backward-data convolution (3x3 implicit GEMM on the packed "
+                      "filter) and filter gradient of one layer in one launch, layers 4-10 of the 13 (both template "
+                      "instances: rows of 8-16 pixels and 4x4 images); the other convolution kernels are listed under `kernels`",
+            "bound": "mfma", "achieved": round(tflops, 2), "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(tflops / MFMA_FP32_PEAK_TFLOPS, 4), "traffic": profile_line("traffic_bytes_per_launch conv_bwd_pair_k"),
+            "traffic_source": "profiles/conv_kernels_vgg16_b128_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of "
+                              "the same %d launches per step; taken from that file, not measured in this run)" % round(launches),
+            "algorithmic_bytes_per_launch": int(pby.value / pl.value) if pl.value else None,
+            "algorithmic_bytes_convention": "dy, x, dx, the filter and its gradient once each",
+            "launches_per_step": int(round(launches)),
+            "flops_per_launch": round(pfl.value / pl.value, 1) if pl.value else None,
+            "flops_convention": "2 x 2*N*K*C*R*S*P*Q per launch (backward-data + filter gradient) = what the kernel executes "
+                                "(it multiplies the taps that fall on zero padding too)",
+            "avg_launch_us": round(pus.value / pl.value, 2) if pl.value else None,
+            "timing": "HIP events around each launch on the library's stream, %d steps" % nsteps,
+        }
+
+        # conv_patch_k with 128 x 128 tiles on its own: the forward convolutions of layers 3-10 (8 launches per step).
+        # Their steps hold nothing else (filters are packed by a step of their own; where a reduction is split the
+        # partial sums are added by the batch norm behind it).
+        flops = us = n128 = bytes_alg = 0
         for i, (c, k, h) in enumerate(configs.VGG_CONVS):
-            if h < 4:
-                continue
-            fl = configs.conv_flops(BATCH, c, k, h)
-            by = 4 * (BATCH * c * h * h + BATCH * k * h * h + k * c * 9)     # input, output and filter once
             fwd_keys = [n for n in ("convolution+addBias", "convolution") if "%s@%dx%dx%dx%d" % (n, BATCH, k, h, h) in per_shape]
-            if k >= 128 and fwd_keys:
+            if h >= 4 and k >= 128 and fwd_keys:
                 # forward layers sharing an output shape share a key: charge each layer its share
                 same = sum(1 for (c2, k2, h2) in configs.VGG_CONVS if (k2, h2) == (k, h))
                 t, n = per_shape["%s@%dx%dx%dx%d" % (fwd_keys[0], BATCH, k, h, h)]
-                flops, us, launches, bytes_alg = flops + fl, us + t / same, launches + 1, bytes_alg + by
-            bkey = "convolutionFeaturesGrad@%dx%dx%dx%d" % (BATCH, c, h, h)
-            if i > 0 and c >= 128 and bkey in per_shape:
-                same = sum(1 for j, (c2, k2, h2) in enumerate(configs.VGG_CONVS) if j > 0 and (c2, h2) == (c, h))
-                t, n = per_shape[bkey]
-                flops, us, launches, bytes_alg = flops + fl, us + t / same, launches + 1, bytes_alg + by
-        tflops = flops / (us * 1e-6) / 1e12 if us else 0.0
-        # HBM bytes per launch of the same kernel over the same launches, from the committed rocprofv3 --pmc
-        # summary (FETCH_SIZE / WRITE_SIZE calibrated against a plain copy): NOT measured in this run
-        traffic = None
-        tpath = os.path.join(ROOT, "profiles", "conv_kernels_vgg16_b128_hbm_traffic.txt")
-        if os.path.exists(tpath):
-            for line in open(tpath):
-                if line.startswith("traffic_bytes_per_launch conv_patch_k_128x128"):
-                    traffic = int(line.split()[-1])
-        result["roofline"] = {
-            "kernel": "conv_patch_k<Tile<128,128,2,4>,16,true>: 3x3 implicit-GEMM convolution, forward of layers 3-10 and "
-                      "backward-data of layers 4-10 of the 13 (the other layers run the 64x256-tile variant, the first-layer "
-                      "kernels and the dense 2x2-image route, listed under `kernels`)",
-            "bound": "mfma", "achieved": round(tflops, 2), "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(tflops / MFMA_FP32_PEAK_TFLOPS, 4), "traffic": traffic,
-            "traffic_source": "profiles/conv_kernels_vgg16_b128_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of "
-                              "the same %d launches per step; taken from that file, not measured in this run)" % launches,
-            "algorithmic_bytes_per_launch": int(bytes_alg / launches) if launches else None,
-            "launches_per_step": int(launches),
-            "flops_per_launch": round(flops / launches, 1) if launches else None,
-            "flops_convention": "2*N*K*C*R*S*P*Q per launch = what the kernel executes (it multiplies the taps that fall on "
-                                "zero padding too)",
-            "avg_launch_us": round(us / launches, 2) if launches else None,
-        }
+                flops, us, n128 = flops + configs.conv_flops(BATCH, c, k, h), us + t / same, n128 + 1
+                bytes_alg += 4 * (BATCH * c * h * h + BATCH * k * h * h + k * c * 9)     # input, output and filter once
         fwd = sum(configs.conv_flops(BATCH, c, k, h) for c, k, h in configs.VGG_CONVS)
-        wgrad_us = per_op["convolutionFiltersGrad"][0]
-        allconv_us = sum(per_op[k][0] for k in ("convolution", "convolution+addBias", "convolutionFeaturesGrad") if k in per_op)
-        allconv_us += per_op.get("filterPack", (0.0, 0))[0]
         bwd_data = fwd - configs.conv_flops(BATCH, *configs.VGG_CONVS[0])
+        conv_ops = ("convolution", "convolution+addBias", "convolutionFeaturesGrad", "convolutionFiltersGrad",
+                    "convolutionFeaturesGrad+convolutionFiltersGrad", "filterPack")
+        allconv_us = sum(per_op[k][0] for k in conv_ops if k in per_op)
         result["kernels"] = {
-            "conv_wgrad_patch_k (all 13 filter gradients incl. their split sums)": {
-                "achieved_TFLOPs": round(fwd / (wgrad_us * 1e-6) / 1e12, 2),
-                "frac_of_mfma_peak": round(fwd / (wgrad_us * 1e-6) / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
-                "us_per_step": round(wgrad_us, 1)},
-            "all forward + backward-data convolutions incl. filter packing (2x2-image layers counted at the conventional "
-            "9-tap FLOPs although their dense route executes 4/9 of them)": {
-                "achieved_TFLOPs": round((fwd + bwd_data) / (allconv_us * 1e-6) / 1e12, 2),
+            "conv_patch_k<Tile<128,128,2,4>,16,true> (forward convolutions of layers 3-10)": {
+                "achieved_TFLOPs": round(flops / (us * 1e-6) / 1e12, 2) if us else None,
+                "frac_of_mfma_peak": round(flops / (us * 1e-6) / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4) if us else None,
+                "launches_per_step": n128, "avg_launch_us": round(us / n128, 2) if n128 else None,
+                "algorithmic_bytes_per_launch": int(bytes_alg / n128) if n128 else None,
+                "traffic": profile_line("traffic_bytes_per_launch conv_patch_k_128x128")},
+            "all 38 convolution operations of the step incl. filter packing and split sums (2x2-image layers counted at the "
+            "conventional 9-tap FLOPs although their dense route executes 4/9 of them)": {
+                "achieved_TFLOPs": round((2 * fwd + bwd_data) / (allconv_us * 1e-6) / 1e12, 2),
+                "frac_of_mfma_peak": round((2 * fwd + bwd_data) / (allconv_us * 1e-6) / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
                 "us_per_step": round(allconv_us, 1)},
             "device_us_per_step_by_op": {k: round(v[0], 1) for k, v in sorted(per_op.items(), key=lambda kv: -kv[1][0])},
             "device_us_per_step_total": round(sum(v[0] for v in per_op.values()), 1),

@@ -85,6 +85,9 @@ PROTOTYPES = {
     "dopt_hip_conv_bwd_data_packed": [C.POINTER(ConvDesc), _vp, _vp, _vp],
     "dopt_hip_conv_fwd_bias_packed_open": [C.POINTER(ConvDesc), _vp, _vp, _vp, _vp, C.POINTER(SplitSum)],
     "dopt_hip_conv_bwd_data_packed_open": [C.POINTER(ConvDesc), _vp, _vp, _vp, C.POINTER(SplitSum)],
+    "dopt_hip_conv_pair_probe": [_i],
+    "dopt_hip_conv_pair_probe_read": [C.POINTER(_i), C.POINTER(_d), C.POINTER(_d), C.POINTER(_d)],
+    "dopt_hip_conv_bwd_pair_packed_open": [C.POINTER(ConvDesc), _vp, _vp, _vp, _vp, _vp, C.POINTER(SplitSum)],
     "dopt_hip_split_sum_close": [C.POINTER(SplitSum)],
     "dopt_hip_conv_bwd_filter": [C.POINTER(ConvDesc), _vp, _vp, _vp],
     "dopt_hip_maxpool_fwd": [_sz, _sz, _sz, _sz, _sz, _sz, _vp, _vp],

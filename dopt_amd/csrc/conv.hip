@@ -24,6 +24,9 @@
 // the inner loops are branch-free.  Layers with few output tiles split the reduction; partial
 // tiles go to the workspace and are summed in a fixed order -- no float atomics, so results are
 // reproducible.
+#include <utility>
+#include <vector>
+
 #include "common.h"
 #include "mfma_core.h"
 
@@ -229,7 +232,7 @@ __device__ inline unsigned fast_div(unsigned x, unsigned magic) { return __umulh
 // meets once per 16-channel chunk, when the patch buffers swap.  (Staging the filter slab in LDS as
 // well costs a barrier per tap: 1.1 % slower on the VGG step.)
 template <class T, int NPMAX, bool kCFull>
-__global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_patch_k(PatchConv p)
+__device__ __forceinline__ void conv_patch_body(const PatchConv &p, const unsigned block_id)
 {
     constexpr int BM = T::BM, BN = T::BN, THREADS = T::THREADS, MI = T::MI, NI = T::NI;
     constexpr int TAPS = 9, CH = 16, LDP = 20;
@@ -239,7 +242,7 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_patch_k(Pat
 
     unsigned L;
     const unsigned tiles = (unsigned)(p.mtiles * p.ntiles);
-    if (!xcd_remap(blockIdx.x, tiles * (unsigned)p.splits, &L)) return;
+    if (!xcd_remap(block_id, tiles * (unsigned)p.splits, &L)) return;
     const int split = (int)(L / tiles);
     const unsigned tile = L - (unsigned)split * tiles;
     const int mt = (int)(tile % (unsigned)p.mtiles), nt = (int)(tile / (unsigned)p.mtiles);
@@ -393,6 +396,12 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_patch_k(Pat
                 if (m < p.Mout) base[(size_t)m * OHW] = add_bias ? acc[i][j][v] + p.bias[m] : acc[i][j][v];
             }
     }
+}
+
+template <class T, int NPMAX, bool kCFull>
+__global__ __launch_bounds__(T::THREADS, T::THREADS / 256) void conv_patch_k(PatchConv p)
+{
+    conv_patch_body<T, NPMAX, kCFull>(p, blockIdx.x);
 }
 
 // Packed filter of the patch kernel: wp[((chunk*9 + tap)*Mp + m)*16 + j] = w[m*sm + (chunk*16+j)*sc + tap]
@@ -742,7 +751,7 @@ struct WgradPatch {
 };
 
 template <int WM, int WC, int kGeo>
-__global__ __launch_bounds__(768, 1) void conv_wgrad_patch_k(WgradPatch p)
+__device__ __forceinline__ void conv_wgrad_patch_body(const WgradPatch &p, const unsigned block_id)
 {
     constexpr int BM = 32 * WM, BC = 32 * WC, THREADS = 768, NPIX = 64, APITCH = NPIX + 4;
     constexpr int NAQ = (BM * NPIX / 4 + THREADS - 1) / THREADS;  // float4 slots of dy per thread
@@ -758,7 +767,7 @@ __global__ __launch_bounds__(768, 1) void conv_wgrad_patch_k(WgradPatch p)
 
     unsigned L;
     const unsigned tiles = (unsigned)(p.mtiles * p.ctiles);
-    if (!xcd_remap(blockIdx.x, tiles * (unsigned)p.splits, &L)) return;
+    if (!xcd_remap(block_id, tiles * (unsigned)p.splits, &L)) return;
     const int split = (int)(L / tiles);
     const unsigned tile = L - (unsigned)split * tiles;
     const int mt = (int)(tile % (unsigned)p.mtiles), ct = (int)(tile / (unsigned)p.mtiles);
@@ -979,6 +988,29 @@ __global__ __launch_bounds__(768, 1) void conv_wgrad_patch_k(WgradPatch p)
             for (int j = lane; j < ncv; j += 64) dst[j] = lds[r * RP + j];
         }
         __syncthreads();
+    }
+}
+
+template <int WM, int WC, int kGeo>
+__global__ __launch_bounds__(768, 1) void conv_wgrad_patch_k(WgradPatch p)
+{
+    conv_wgrad_patch_body<WM, WC, kGeo>(p, blockIdx.x);
+}
+
+// Backward-data and filter gradient of one layer in ONE launch: both read dy and nothing of each other.
+// The first `grid_a` workgroups run the backward-data tiles, the rest the filter-gradient tiles; workgroups are
+// dispatched in id order, so a compute unit that has finished its backward-data tile starts a filter-gradient
+// tile at once instead of idling until the slowest tile of the launch is done and the next launch has ramped up.
+// Launched with the filter gradient's 768 threads: the wavefronts a backward-data workgroup does not need end
+// at once (a barrier waits for the surviving wavefronts only).
+template <class T, int NPMAX, int WM, int WC, int kGeo>
+__global__ __launch_bounds__(768, 1) void conv_bwd_pair_k(PatchConv a, WgradPatch b, unsigned grid_a)
+{
+    if (blockIdx.x < grid_a) {
+        if (threadIdx.x >= (unsigned)T::THREADS) return;
+        conv_patch_body<T, NPMAX, true>(a, blockIdx.x);
+    } else {
+        conv_wgrad_patch_body<WM, WC, kGeo>(b, blockIdx.x - grid_a);
     }
 }
 
@@ -1253,6 +1285,18 @@ int patch_splits(int tiles, int chunks, int slots, int BM, int BN, size_t out_el
     return best;
 }
 
+// Fills in how a patch convolution splits its channel chunks over blocks; returns the number of splits.
+int patch_decide_splits(PatchSetup *u, const float *out)
+{
+    PatchConv &pc = u->pc;
+    int splits = patch_splits(u->tiles, pc.chunks_total, u->blocks_wanted, u->BM, u->BN, pc.out_elems);
+    if (pc.out_elems % 4 != 0 || !aligned16(out)) splits = 1;
+    pc.chunks_per_split = (pc.chunks_total + splits - 1) / splits;
+    splits = (pc.chunks_total + pc.chunks_per_split - 1) / pc.chunks_per_split;
+    pc.splits = splits;
+    return splits;
+}
+
 // `prepacked`: the filter already in the kernel's layout (dopt_hip_conv_pack_batch), or null to
 // pack it here first.
 template <bool kBwd>
@@ -1264,11 +1308,7 @@ int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, 
     if (!u.ok) return DOPT_HIP_OK;
     PatchConv &pc = u.pc;
     const int tiles = u.tiles;
-    int splits = patch_splits(tiles, pc.chunks_total, u.blocks_wanted, u.BM, u.BN, pc.out_elems);
-    if (pc.out_elems % 4 != 0 || !aligned16(out)) splits = 1;
-    pc.chunks_per_split = (pc.chunks_total + splits - 1) / splits;
-    splits = (pc.chunks_total + pc.chunks_per_split - 1) / pc.chunks_per_split;
-    pc.splits = splits;
+    const int splits = patch_decide_splits(&u, out);
 
     const size_t wp_bytes = prepacked ? 0 : (u.wp_elems * sizeof(float) + 255) / 256 * 256;
     const size_t part_bytes = splits > 1 ? (size_t)splits * pc.out_elems * sizeof(float) : 0;
@@ -1663,19 +1703,28 @@ int launch_wgrad_reduce(int K, int C, int Cp, int taps, int splits, size_t out_e
     return DOPT_HIP_OK;
 }
 
-// 3x3, unit stride, pad 1; rows of 8 / 16 / 32 / 64 pixels, or 4x4 or 2x2 images.  *done = false: not this path.
-int run_wgrad_patch(const dopt_hip_conv_desc *d, const float *dy, const float *x, float *dw, bool *done)
+// What run_wgrad_patch decides before it touches memory: ok = false when the shape is not this path's
+// (3x3, unit stride, pad 1; rows of 8 / 16 / 32 / 64 pixels, or 4x4 or 2x2 images).
+struct WgradSetup {
+    bool ok;
+    WgradPatch wp;
+    bool tall;            // 128 rows x 32 channels per block, else 64 x 64
+    int geo, tiles, splits;
+    size_t out_elems, lds_bytes;
+};
+
+WgradSetup wgrad_patch_setup(const dopt_hip_conv_desc *d, const float *dw)
 {
-    *done = false;
-    if (d->R != 3 || d->S != 3 || d->strideH != 1 || d->strideW != 1 || d->padH != 1 || d->padW != 1) return DOPT_HIP_OK;
-    if (d->C < 16) return DOPT_HIP_OK;  // a 32-channel fragment would be mostly padding
+    WgradSetup u{};
+    if (d->R != 3 || d->S != 3 || d->strideH != 1 || d->strideW != 1 || d->padH != 1 || d->padW != 1) return u;
+    if (d->C < 16) return u;  // a 32-channel fragment would be mostly padding
     const int W = (int)d->W, H = (int)d->H;
-    WgradPatch wp{};
+    WgradPatch &wp = u.wp;
     int geo;
     if (W == 8 || W == 16 || W == 32 || W == 64) {
         geo = 0;
         wp.G = 64 / W;
-        if (H % wp.G != 0) return DOPT_HIP_OK;
+        if (H % wp.G != 0) return u;
         wp.bands = H / wp.G;
         wp.imgs = 1;
         wp.ppitch = W + 8;
@@ -1686,19 +1735,18 @@ int run_wgrad_patch(const dopt_hip_conv_desc *d, const float *dy, const float *x
         wp.G = H;
         wp.bands = 1;
         wp.imgs = 64 / (H * W);
-        if (d->N % wp.imgs != 0) return DOPT_HIP_OK;
+        if (d->N % wp.imgs != 0) return u;
         wp.ppitch = geo == 1 ? 12 : 4;
         wp.cstride = geo == 1 ? 4 * 72 : 16 * 16;
         wp.chunks_total = (int)d->N / wp.imgs;
     } else {
-        return DOPT_HIP_OK;
+        return u;
     }
     while (wp.cstride % 8 != 4) wp.cstride += 4;  // 128-bit reads by 32 channels at this stride touch every LDS bank once
     // 128 rows x 32 channels, or 64 x 64 when that pads the output channels less (160 -> 192, not 256)
     const bool tall = d->K >= 128 && (d->K + 127) / 128 * 128 <= (d->K + 63) / 64 * 64;
-    if (!tall && W == 64) return DOPT_HIP_OK;
+    if (!tall && W == 64) return u;
     const int BM = tall ? 128 : 64, BC = tall ? 32 : 64;
-    wp.dy = dy; wp.x = x;
     wp.N = (int)d->N; wp.C = (int)d->C; wp.K = (int)d->K; wp.H = H; wp.W = W;
     wp.quads_row = W / 4;
     wp.mtiles = (wp.K + BM - 1) / BM;
@@ -1736,36 +1784,153 @@ int run_wgrad_patch(const dopt_hip_conv_desc *d, const float *dy, const float *x
     wp.splits = splits;
     const size_t lds_main = ((size_t)2 * BM * 68 + (size_t)2 * BC * wp.cstride + 4) * sizeof(float);
     const size_t lds_epi = (size_t)32 * (BC * 9 + 1) * sizeof(float);
-    const size_t lds_bytes = lds_main > lds_epi ? lds_main : lds_epi;
-    if (lds_bytes > 160 * 1024) return DOPT_HIP_OK;
+    u.lds_bytes = lds_main > lds_epi ? lds_main : lds_epi;
+    if (u.lds_bytes > 160 * 1024) return u;
+    wp.split_stride = out_elems;
+    u.tall = tall; u.geo = geo; u.tiles = tiles; u.splits = splits; u.out_elems = out_elems;
+    u.ok = true;
+    return u;
+}
+
+// dw = the partial filters added in split order
+int wgrad_split_sum(const WgradSetup &u, const float *partial, float *dw)
+{
+    // enough blocks for small filters with hundreds of splits: more split lanes per block
+    const size_t n4 = u.out_elems / 4;
+    if (n4 >= (size_t)64 * 512)
+        hipLaunchKernelGGL(split_sum_k<4>, dim3((unsigned)ceil_div(n4, (size_t)64)), dim3(256), 0, stream(), n4, u.splits,
+                           n4, (const float4 *)partial, (float4 *)dw);
+    else
+        hipLaunchKernelGGL(split_sum_k<16>, dim3((unsigned)ceil_div(n4, (size_t)16)), dim3(256), 0, stream(), n4, u.splits,
+                           n4, (const float4 *)partial, (float4 *)dw);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+int run_wgrad_patch(const dopt_hip_conv_desc *d, const float *dy, const float *x, float *dw, bool *done)
+{
+    *done = false;
+    WgradSetup u = wgrad_patch_setup(d, dw);
+    if (!u.ok) return DOPT_HIP_OK;
+    WgradPatch &wp = u.wp;
     float *partial = nullptr;
-    if (splits > 1) {
-        partial = (float *)workspace((size_t)splits * out_elems * sizeof(float));
+    if (u.splits > 1) {
+        partial = (float *)workspace((size_t)u.splits * u.out_elems * sizeof(float));
         if (!partial) return DOPT_HIP_ERR_OOM;
     }
-    wp.out = splits > 1 ? partial : dw;
-    wp.split_stride = out_elems;
-    const dim3 grid(xcd_grid((unsigned)(tiles * splits)));
+    wp.dy = dy; wp.x = x;
+    wp.out = u.splits > 1 ? partial : dw;
+    const dim3 grid(xcd_grid((unsigned)(u.tiles * u.splits)));
+    const int geo = u.geo;
     int rc;
-    if (tall) rc = geo == 0 ? launch_wgrad_patch<4, 1, 0>(wp, grid, lds_bytes)
-                 : geo == 1 ? launch_wgrad_patch<4, 1, 1>(wp, grid, lds_bytes)
-                            : launch_wgrad_patch<4, 1, 2>(wp, grid, lds_bytes);
-    else rc = geo == 0 ? launch_wgrad_patch<2, 2, 0>(wp, grid, lds_bytes)
-            : geo == 1 ? launch_wgrad_patch<2, 2, 1>(wp, grid, lds_bytes)
-                       : launch_wgrad_patch<2, 2, 2>(wp, grid, lds_bytes);
+    if (u.tall) rc = geo == 0 ? launch_wgrad_patch<4, 1, 0>(wp, grid, u.lds_bytes)
+                   : geo == 1 ? launch_wgrad_patch<4, 1, 1>(wp, grid, u.lds_bytes)
+                              : launch_wgrad_patch<4, 1, 2>(wp, grid, u.lds_bytes);
+    else rc = geo == 0 ? launch_wgrad_patch<2, 2, 0>(wp, grid, u.lds_bytes)
+            : geo == 1 ? launch_wgrad_patch<2, 2, 1>(wp, grid, u.lds_bytes)
+                       : launch_wgrad_patch<2, 2, 2>(wp, grid, u.lds_bytes);
     if (rc) return rc;
     *done = true;
-    if (splits > 1) {
-        // enough blocks for small filters with hundreds of splits: more split lanes per block
-        const size_t n4 = out_elems / 4;
-        if (n4 >= (size_t)64 * 512)
-            hipLaunchKernelGGL(split_sum_k<4>, dim3((unsigned)ceil_div(n4, (size_t)64)), dim3(256), 0, stream(), n4, splits,
-                               n4, (const float4 *)partial, (float4 *)dw);
-        else
-            hipLaunchKernelGGL(split_sum_k<16>, dim3((unsigned)ceil_div(n4, (size_t)16)), dim3(256), 0, stream(), n4, splits,
-                               n4, (const float4 *)partial, (float4 *)dw);
-        DOPT_LAUNCH_CHECK();
+    if (u.splits > 1) return wgrad_split_sum(u, partial, dw);
+    return DOPT_HIP_OK;
+}
+
+// Backward-data (on a packed filter) and filter gradient of one 3x3 layer as one launch (conv_bwd_pair_k).
+// *done = false: one of the two is not a patch-kernel shape, or a combination that is not built; the
+// caller runs them one after the other.  `open` as in run_patch.
+template <class T, int NPMAX, int WM, int WC, int kGeo>
+int launch_bwd_pair(const PatchConv &pc, const WgradPatch &wp, unsigned grid_a, unsigned grid_b, size_t lds_bytes)
+{
+    static bool raised = false;
+    if (!raised) {
+        DOPT_HIP_CHECK(hipFuncSetAttribute((const void *)conv_bwd_pair_k<T, NPMAX, WM, WC, kGeo>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        raised = true;
     }
+    hipLaunchKernelGGL((conv_bwd_pair_k<T, NPMAX, WM, WC, kGeo>), dim3(grid_a + grid_b), dim3(768), lds_bytes, stream(), pc,
+                       wp, grid_a);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+// Device time of the one-launch pairs alone (their entry point also runs the split sums): while the probe is on,
+// every conv_bwd_pair_k launch is bracketed by two events on the stream it is launched on.
+struct PairProbe {
+    bool on = false;
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> events;   // kept for the process's lifetime, reused
+    size_t used = 0;
+    double flops = 0.0, bytes = 0.0;
+};
+PairProbe g_pair_probe;
+
+int run_bwd_pair(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *dy, const float *prepacked, const float *x,
+                 float *dx, float *dw, dopt_hip_split_sum *open, bool *done)
+{
+    *done = false;
+    PatchSetup a = patch_setup<true>(d, P, Q);
+    WgradSetup b = wgrad_patch_setup(d, dw);
+    if (!a.ok || !b.ok || !prepacked || a.pc.Cin % 16 != 0) return DOPT_HIP_OK;
+    // The combinations that are built: 128 x 128 backward-data tiles on eight wavefronts, one workgroup per CU
+    // (the 64 x 256 tiles of layers with up to 64 input channels run two 256-thread workgroups per CU, which a
+    // launch shaped for the filter gradient's 768 threads cannot hold), with 128 x 32 filter-gradient tiles on
+    // rows of 8 .. 64 pixels or on 4 x 4 images.
+    const int combo = a.shape == 2 && b.tall && b.geo == 0 ? 0 : a.shape == 2 && b.tall && b.geo == 1 ? 1 : -1;
+    if (combo < 0) return DOPT_HIP_OK;
+    PatchConv &pc = a.pc;
+    WgradPatch &wp = b.wp;
+    const int splits_a = patch_decide_splits(&a, dx);
+    const size_t part_a = splits_a > 1 ? ((size_t)splits_a * pc.out_elems * sizeof(float) + 255) / 256 * 256 : 0;
+    const size_t part_b = b.splits > 1 ? (size_t)b.splits * b.out_elems * sizeof(float) : 0;
+    char *ws = part_a + part_b > 0 ? (char *)workspace(part_a + part_b) : nullptr;
+    if (part_a + part_b > 0 && !ws) return DOPT_HIP_ERR_OOM;
+    float *partial_a = (float *)ws, *partial_b = (float *)(ws + part_a);
+    pc.in = dy;
+    pc.wp = prepacked;
+    pc.bias = nullptr;
+    pc.in_bytes = (size_t)pc.N * pc.Cin * pc.IH * pc.IW * sizeof(float);
+    pc.wp_bytes = a.wp_elems * sizeof(float);
+    pc.out = splits_a > 1 ? partial_a : dx;
+    wp.dy = dy; wp.x = x;
+    wp.out = b.splits > 1 ? partial_b : dw;
+    const unsigned grid_a = xcd_grid((unsigned)(a.tiles * splits_a)), grid_b = xcd_grid((unsigned)(b.tiles * b.splits));
+    const size_t lds_bytes = a.lds_bytes > b.lds_bytes ? a.lds_bytes : b.lds_bytes;
+    PairProbe &probe = g_pair_probe;
+    const bool probing = probe.on && !capturing();
+    if (probing) {
+        if (probe.used == probe.events.size()) {
+            hipEvent_t e0, e1;
+            DOPT_HIP_CHECK(hipEventCreate(&e0));
+            DOPT_HIP_CHECK(hipEventCreate(&e1));
+            probe.events.push_back({e0, e1});
+        }
+        DOPT_HIP_CHECK(hipEventRecord(probe.events[probe.used].first, stream()));
+    }
+    int rc;
+    if (combo == 0) rc = launch_bwd_pair<GatherDeep, 16, 4, 1, 0>(pc, wp, grid_a, grid_b, lds_bytes);
+    else rc = launch_bwd_pair<GatherDeep, 16, 4, 1, 1>(pc, wp, grid_a, grid_b, lds_bytes);
+    if (rc) return rc;
+    if (probing) {
+        DOPT_HIP_CHECK(hipEventRecord(probe.events[probe.used++].second, stream()));
+        const double px = (double)d->N * d->H * d->W;
+        probe.flops += 2.0 * 2.0 * px * d->K * d->C * 9.0;                              // both products, every tap
+        probe.bytes += 4.0 * (2.0 * px * d->C + px * d->K + 2.0 * (double)d->K * d->C * 9.0);   // dy, x, dx, filter, dw once each
+    }
+    *done = true;
+    if (b.splits > 1)
+        if (int rc2 = wgrad_split_sum(b, partial_b, dw)) return rc2;
+    if (splits_a > 1 && open) {   // the caller's next call adds the copies
+        open->partial = partial_a;
+        open->splits = splits_a;
+        open->elems = pc.out_elems;
+        open->C = (size_t)pc.Mout;
+        open->inner = (size_t)pc.OH * pc.OW;
+        open->bias = nullptr;
+        open->value = dx;
+        open_split_set(partial_a);
+        return DOPT_HIP_OK;
+    }
+    if (splits_a > 1)
+        return launch_splitk_reduce(pc.out_elems, splits_a, partial_a, dx, nullptr, (unsigned)pc.Mout, (unsigned)(pc.OH * pc.OW));
     return DOPT_HIP_OK;
 }
 
@@ -1903,6 +2068,57 @@ int dopt_hip_conv_bwd_data_packed_open(const dopt_hip_conv_desc *d, const float 
 int dopt_hip_conv_bwd_data_packed(const dopt_hip_conv_desc *d, const float *dy, const float *packed, float *dx)
 {
     return dopt_hip_conv_bwd_data_packed_open(d, dy, packed, dx, nullptr);
+}
+
+int dopt_hip_conv_bwd_pair_packed_open(const dopt_hip_conv_desc *d, const float *dy, const float *packed, const float *x,
+                                       float *dx, float *dw, dopt_hip_split_sum *open)
+{
+    size_t P, Q;
+    if (int rc = check_desc(d, &P, &Q, "dopt_hip_conv_bwd_pair_packed_open")) return rc;
+    DOPT_REQUIRE(dy && packed && x && dx && dw, "dopt_hip_conv_bwd_pair_packed_open: null argument");
+    DOPT_ENSURE_INIT();
+    if (open) {
+        *open = dopt_hip_split_sum{};
+        open->value = dx;
+    }
+    bool done = false;
+    if (int rc = run_bwd_pair(d, P, Q, dy, packed, x, dx, dw, open, &done)) return rc;
+    if (done) return DOPT_HIP_OK;
+    // not a pair the one-launch kernel takes: filter gradient first (it may use the workspace), then backward-data,
+    // which may leave its result open in it
+    if (int rc = dopt_hip_conv_bwd_filter(d, dy, x, dw)) return rc;
+    if (open) return dopt_hip_conv_bwd_data_packed_open(d, dy, packed, dx, open);
+    return dopt_hip_conv_bwd_data_packed(d, dy, packed, dx);
+}
+
+int dopt_hip_conv_pair_probe(int enable)
+{
+    DOPT_ENSURE_INIT();
+    g_pair_probe.on = enable != 0;
+    if (enable) {
+        g_pair_probe.used = 0;
+        g_pair_probe.flops = g_pair_probe.bytes = 0.0;
+    }
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_conv_pair_probe_read(int *launches, double *total_us, double *flops, double *bytes)
+{
+    DOPT_REQUIRE(launches && total_us && flops && bytes, "dopt_hip_conv_pair_probe_read: null argument");
+    DOPT_ENSURE_INIT();
+    PairProbe &probe = g_pair_probe;
+    double us = 0.0;
+    for (size_t i = 0; i < probe.used; i++) {
+        DOPT_HIP_CHECK(hipEventSynchronize(probe.events[i].second));
+        float ms = 0.0f;
+        DOPT_HIP_CHECK(hipEventElapsedTime(&ms, probe.events[i].first, probe.events[i].second));
+        us += (double)ms * 1000.0;
+    }
+    *launches = (int)probe.used;
+    *total_us = us;
+    *flops = probe.flops;
+    *bytes = probe.bytes;
+    return DOPT_HIP_OK;
 }
 
 int dopt_hip_split_sum_close(const dopt_hip_split_sum *open)

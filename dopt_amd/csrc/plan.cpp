@@ -591,6 +591,9 @@ struct HIPPlan::Builder {
     std::vector<std::vector<size_t>> exposed;   // byte offsets at which plan outputs (or aliases of them) expose a buffer
     std::vector<int> biasGradOf;                // batchNormGrad op -> the addBiasGrad op it serves
     std::vector<int> poolOf;                    // batchNormTrain op -> the 2 x 2 maxpool op whose buffer its kernel fills too
+    std::vector<int> pairOf;                    // packed convolutionFeaturesGrad op -> the convolutionFiltersGrad op of the same layer
+    std::vector<int> pairLead;                  // the operation of such a pair that comes first in the order -> the backward-data op
+    std::vector<char> pairLater;                // the operation of such a pair that comes second: no step of its own
     std::vector<char> absorbed;
     std::vector<char> needed;
     // late: the copy is made right in front of its first reader instead of at the start of the run
@@ -608,7 +611,8 @@ struct HIPPlan::Builder {
     Builder(const Graph &graph, HIPPlan *plan, const std::vector<int> &outs, unsigned f)
         : g(graph), p(plan), outputs(outs), flags(f), nops((int)graph.ops.size()), alias((size_t)nops),
           inputsOf((size_t)nops), fusedKind((size_t)nops, 0), prebuilt((size_t)nops), prebuiltLabel((size_t)nops),
-          live((size_t)nops, 0), uses((size_t)nops), exposed((size_t)nops), biasGradOf((size_t)nops, -1), poolOf((size_t)nops, -1),
+          live((size_t)nops, 0), uses((size_t)nops), exposed((size_t)nops), biasGradOf((size_t)nops, -1), poolOf((size_t)nops, -1), pairOf((size_t)nops, -1), pairLead((size_t)nops, -1),
+          pairLater((size_t)nops, 0),
           absorbed((size_t)nops, 0), needed((size_t)nops, 0), packOf((size_t)nops, -1), mmInfo((size_t)nops)
     {
     }
@@ -633,6 +637,7 @@ struct HIPPlan::Builder {
     void formChains();
     void absorbBiasGrads();
     void absorbPools();
+    void pairBackward();
     std::unique_ptr<HIPKernel> makePooledTrain(int id, std::shared_ptr<dopt_hip_split_sum> open, std::string *label);
     void markNeeded();
     int prepackFilters();
@@ -1154,6 +1159,44 @@ int HIPPlan::Builder::prepackFilters()
     return DOPT_HIP_OK;
 }
 
+// convolutionFeaturesGrad and convolutionFiltersGrad of one layer read the same dy and nothing of each other: where
+// the former runs on a packed filter they become one step (dopt_hip_conv_bwd_pair_packed_open), placed where the
+// earlier of the two stands in the order - every input of either is ready there, and every reader of either comes
+// after its own, later or equal, position.
+void HIPPlan::Builder::pairBackward()
+{
+    if (!(flags & DOPT_HIP_PLAN_FUSE)) return;
+    std::vector<int> pos((size_t)nops, -1);
+    for (size_t i = 0; i < p->mOps.size(); i++) pos[p->mOps[i]] = (int)i;
+    std::vector<char> taken((size_t)nops, 0);
+    for (int bd : p->mOps) {
+        if (packOf[bd] < 0 || !needed[bd]) continue;
+        const Prepack &pk = packs[(size_t)packOf[bd]];
+        if (!pk.bwd || dopt_hip_conv_packed_layout(&pk.d, 1) != 1) continue;   // 3x3 patch layout only
+        const Operation &bo = g.ops[bd];
+        size_t dyoff;
+        const int dyroot = root(bo.deps[0], &dyoff);
+        const auto *pad = sizes_attr(bo, "padding"), *stride = sizes_attr(bo, "stride");
+        for (int fg : p->mOps) {
+            const Operation &fo = g.ops[fg];
+            if (fo.opType != "convolutionFiltersGrad" || fo.deps.size() != 2 || !needed[fg] || taken[fg] || absorbed[fg] ||
+                alias[fg].source >= 0 || prebuilt[fg] || fusedKind[fg] || fo.dtype != DOPT_HIP_F32)
+                continue;
+            size_t off2;
+            if (root(fo.deps[0], &off2) != dyroot || off2 != dyoff) continue;
+            const auto *pad2 = sizes_attr(fo, "padding"), *stride2 = sizes_attr(fo, "stride");
+            if (!pad || !stride || !pad2 || !stride2 || *pad != *pad2 || *stride != *stride2) continue;
+            if (fo.shape != g.ops[pk.filter].shape || g.ops[fo.deps[1]].shape != bo.shape) continue;
+            pairOf[bd] = fg;
+            taken[fg] = 1;
+            const int first = pos[bd] < pos[fg] ? bd : fg, second = first == bd ? fg : bd;
+            pairLead[first] = bd;
+            pairLater[second] = 1;
+            break;
+        }
+    }
+}
+
 void HIPPlan::Builder::pushPackStep(const std::vector<Prepack> &which)
 {
     std::vector<dopt_hip_conv_desc> descs;
@@ -1218,8 +1261,9 @@ std::unique_ptr<HIPKernel> HIPPlan::Builder::makePooledTrain(int id, std::shared
 int HIPPlan::Builder::buildSteps()
 {
     // kernels and buffers
-    for (int id : p->mOps) {
-        if (!needed[id]) continue;
+    for (int at : p->mOps) {
+        if (!needed[at] || pairLater[at]) continue;
+        const int id = pairLead[at] >= 0 ? pairLead[at] : at;   // a backward pair is built where its first operation stands
         const Operation &op = g.ops[id];
         if (is_leaf(op)) {
             if (!op.value && op.bytes() > 0)
@@ -1241,7 +1285,15 @@ int HIPPlan::Builder::buildSteps()
             const dopt_hip_conv_desc d = pk.d;
             onPacked = true;
             convSteps.push_back({0, id, pk.bwd, !pk.bwd && fusedKind[id] == 1, d, packed});
-            if (pk.bwd) {
+            if (pk.bwd && pairOf[id] >= 0) {
+                stepInputs = {op.deps[0], g.ops[pairOf[id]].deps[1]};
+                float *dw = (float *)p->mResults[pairOf[id]];
+                k = make([=](const std::vector<const void *> &in, void *out) {
+                    return dopt_hip_conv_bwd_pair_packed_open(&d, (const float *)in[0], packed, (const float *)in[1], (float *)out,
+                                                              dw, nullptr);
+                });
+                label = "convolutionFeaturesGrad+convolutionFiltersGrad";
+            } else if (pk.bwd) {
                 stepInputs = {op.deps[0]};
                 k = make([=](const std::vector<const void *> &in, void *out) {
                     return dopt_hip_conv_bwd_data_packed(&d, (const float *)in[0], packed, (float *)out);
@@ -1345,9 +1397,17 @@ void HIPPlan::Builder::openSplitSums()
             void *extra = biasGradOf[b] >= 0 && needed[biasGradOf[b]] ? p->mResults[biasGradOf[b]] : nullptr;
             nci(g.ops[bo.deps[1]].shape, &N, &C, &inner);
             const int keep = uses[cs.op].size() == 1 && !isOutput(cs.op) ? 0 : 1;   // does anything else read dy?
-            conv.kernel = make([=](const std::vector<const void *> &in, void *out) {
-                return dopt_hip_conv_bwd_data_packed_open(&d, (const float *)in[0], packed, (float *)out, open.get());
-            });
+            if (pairOf[cs.op] >= 0) {
+                float *dw = (float *)p->mResults[pairOf[cs.op]];
+                conv.kernel = make([=](const std::vector<const void *> &in, void *out) {
+                    return dopt_hip_conv_bwd_pair_packed_open(&d, (const float *)in[0], packed, (const float *)in[1], (float *)out,
+                                                              dw, open.get());
+                });
+            } else {
+                conv.kernel = make([=](const std::vector<const void *> &in, void *out) {
+                    return dopt_hip_conv_bwd_data_packed_open(&d, (const float *)in[0], packed, (float *)out, open.get());
+                });
+            }
             next.kernel = make([=](const std::vector<const void *> &in, void *out) {
                 if (open->value != in[0]) return fail(DOPT_HIP_ERR_RUNTIME, "plan: open convolution result is not the gradient's input");
                 const float *y = relu ? (const float *)in[1] : nullptr;
@@ -1390,7 +1450,7 @@ int HIPPlan::Builder::assignQueues()
             for (int in : st.inputOps) reads_side = reads_side || onSide[producer(in)];
             const bool wgrad = g.ops[st.op].opType == "convolutionFiltersGrad";
             // a step with a second output (the absorbed bias gradient) stays on the main queue
-            if ((wgrad || reads_side) && biasGradOf[st.op] < 0 && poolOf[st.op] < 0) {
+            if ((wgrad || reads_side) && biasGradOf[st.op] < 0 && poolOf[st.op] < 0 && pairOf[st.op] < 0) {
                 st.lane = 1;
                 st.fenceBefore = true;
                 onSide[st.op] = 1;
@@ -1422,6 +1482,7 @@ int HIPPlan::Builder::assignQueues()
             stepOf[op] = (int)i;
             if (biasGradOf[op] >= 0) stepOf[biasGradOf[op]] = (int)i;
             if (poolOf[op] >= 0) stepOf[poolOf[op]] = (int)i;
+            if (pairOf[op] >= 0) stepOf[pairOf[op]] = (int)i;
         }
         std::vector<std::vector<int>> readers(n), producers(n);
         for (size_t i = 0; i < n; i++)
@@ -1540,8 +1601,10 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         b.absorbPools();
     }
     b.markNeeded();
-    if (flags & DOPT_HIP_PLAN_FUSE)
+    if (flags & DOPT_HIP_PLAN_FUSE) {
         if (int rc = b.prepackFilters()) return rc;
+        b.pairBackward();
+    }
     if (int rc = b.allocateBuffers()) return rc;
     if (int rc = b.buildSteps()) return rc;
     b.openSplitSums();

@@ -92,6 +92,13 @@ def cases(scale=1):
     add("batchNormTrain", str(act), 8 * n, lambda o: ops.bn_train(x, g, b, rm, rv, 0.9, out=o))
     add("batchNormGrad", str(act), 12 * n, lambda o: ops.bn_grad(dy, x, g, out=o))
     add("batchNormInference", str(act), 8 * n, lambda o: ops.bn_infer(x, g, b, rm, rv, out=o))
+    # the same pair with the 2x2 max-pool of a VGG block riding along: y and its pooled quarter written by one
+    # launch; backward, dy made from the pooled tensor's gradient on the way in (dp, y, x read; dx written)
+    ybuf = ops.bn_train_relu(x, g, b, rm, rv, 0.9)
+    yv = ybuf.view(0, act)
+    pooled = ops.Tensor((act[0], 64, 16, 16))
+    add("batchNormTrain+relu+maxpool", str(act), 9 * n, lambda o: ops.bn_train_pool(x, g, b, rm, rv, 0.9, out=o, pooled=pooled)[0])
+    add("maxpoolGrad+reluGrad+batchNormGrad", str(act), 13 * n, lambda o: ops.bn_grad_pool(pdy, yv, x, g, out=o))
     add("sum (all axes)", str(act), 4 * n, lambda o: ops.sum(x, out=o))
     add("sum axes [0,2,3]", str(act), 4 * n, lambda o: ops.sum(x, [0, 2, 3], out=o))
     add("maxElement (all axes)", str(act), 4 * n, lambda o: ops.max_element(x, out=o))
@@ -116,7 +123,7 @@ def cases(scale=1):
     rows.append(("fused SGD (40 tensors)", "%d" % total, 20 * total, lambda: sgd.sgd(0.01, 0.9, False)))
     rows.append(("fused ADAM (40 tensors)", "%d" % total, 28 * total, lambda: adam.adam(1e-3, 0.9, 0.999, 1e-8)))
     rows.append(("fused AMSGrad (40 tensors)", "%d" % total, 36 * total, lambda: ams.amsgrad(1e-3, 0.9, 0.999, 1e-8)))
-    keep.extend([x, dy, bias, pdy, g, b, rm, rv, sm, tw, tg, tm, tv, tvh, sgd, adam, ams])
+    keep.extend([x, dy, bias, pdy, g, b, rm, rv, sm, tw, tg, tm, tv, tvh, sgd, adam, ams, ybuf, yv, pooled])
     return rows, keep
 
 

@@ -240,6 +240,22 @@ int dopt_hip_conv_fwd_bias_packed_open(const dopt_hip_conv_desc *d, const float 
                                        const float *bias, float *y, dopt_hip_split_sum *open);
 int dopt_hip_conv_bwd_data_packed_open(const dopt_hip_conv_desc *d, const float *dy, const float *packed,
                                        float *dx, dopt_hip_split_sum *open);
+/* Backward-data (on a packed filter, as dopt_hip_conv_bwd_data_packed_open; open may be null) and filter gradient
+   (as dopt_hip_conv_bwd_filter) of one convolution in one call: cudnnConvolutionBackwardData (cudnn7.d:195) and
+   cudnnConvolutionBackwardFilter (cudnn7.d:244) read the same dy and nothing of each other.  For 3x3 unit-stride
+   layers of at least 128 input and output channels on rows of 8 .. 64 pixels or 4 x 4 images both run as ONE
+   launch, the filter-gradient tiles starting on each compute unit as its backward-data tile ends; every other
+   shape runs the two entry points one after the other.  dx and dw are bit for bit what those write. */
+int dopt_hip_conv_bwd_pair_packed_open(const dopt_hip_conv_desc *d, const float *dy, const float *packed,
+                                       const float *x, float *dx, float *dw, dopt_hip_split_sum *open);
+/* Measurement aid (no counterpart in the reference; CUDAPlan.profiler, cuda/package.d:424-431, times whole kernel
+   objects): while enabled, every one-launch pair above is bracketed by two events on the library's queue, so its
+   device time is known apart from the split sums the same entry point runs.  probe(1) starts a fresh collection,
+   probe(0) stops it; read waits for the launches collected so far and returns their number, their summed
+   duration, the FLOPs they executed (both products, every tap) and their algorithmic bytes (dy, x, dx, filter,
+   dw once each).  Launches recorded into a HIP graph are not collected. */
+int dopt_hip_conv_pair_probe(int enable);
+int dopt_hip_conv_pair_probe_read(int *launches, double *total_us, double *flops, double *bytes);
 /* value = sum of the copies in order (+ bias): what the closed entry points do themselves. */
 int dopt_hip_split_sum_close(const dopt_hip_split_sum *open);
 /* `convolutionFiltersGrad`: cudnnConvolutionBackwardFilter, cudnn7.d:244. */

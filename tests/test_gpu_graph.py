@@ -326,12 +326,14 @@ def test_plan_fusion_does_not_change_results():
 def test_pools_ride_in_the_batch_norm_kernels():
     """With the rewrites on, the 2 x 2 max-pools of a VGG block and their gradients have no kernels of their
     own: the batch norm in front pools, the batch-norm gradient routes.  (That the values do not change is the
-    test above and the configuration tests; this one checks that the rewrite really fires.)"""
+    test above and the configuration tests; this one checks that the rewrite really fires.)  The two
+    convolutions behind the first pool run on 16 x 16 images, where backward-data takes a packed filter: each shares
+    one step with its filter gradient."""
     r = np.random.default_rng(83)
-    X = r.standard_normal((8, 3, 8, 8)).astype(np.float32)
+    X = r.standard_normal((8, 3, 32, 32)).astype(np.float32)
     Y = np.zeros((8, 10), np.float32)
     Y[np.arange(8), r.integers(0, 10, 8)] = 1
-    feats, labels = float32([8, 3, 8, 8]), float32([8, 10])
+    feats, labels = float32([8, 3, 32, 32]), float32([8, 10])
     init = nnet.Init(84)
     body = nnet.vgg(feats, [16, -1, 32, 32, -1], [24], init)
     preds = nnet.softmax(nnet.dense(body, 10, init))
@@ -344,6 +346,7 @@ def test_pools_ride_in_the_batch_norm_kernels():
     assert prof["batchNormTrain+relu+maxpool"][1] == 2, prof
     assert prof["maxpoolGrad+reluGrad+batchNormGrad+addBiasGrad"][1] == 2, prof
     assert "maxpool" not in prof and "maxpoolGrad" not in prof, prof
+    assert prof["convolutionFeaturesGrad+convolutionFiltersGrad"][1] == 2 and "convolutionFeaturesGrad" not in prof, prof
     plain = core.compile(outs, core.PLAN_VIEWS).execute({feats: X, labels: Y})
     for a, b in zip(plain, fused):
         assert np.array_equal(a, b) or (a.ndim == 1 and np.allclose(a, b, rtol=0, atol=2e-5))
@@ -401,6 +404,79 @@ def test_packed_filter_entry_points_match_the_unpacked_ones():
     x, y, scratch = ops.Tensor((2, 8, 8, 8)), ops.Tensor((2, 8, 8, 8)), ops.Tensor([1024])
     with pytest.raises(capi.HipError):
         capi.check(lib.dopt_hip_conv_fwd_bias_packed(C.byref(d5), x.ptr, scratch.ptr, None, y.ptr))
+
+
+@pytest.mark.parametrize("xs,k", [((8, 256, 4, 4), 512),     # one launch: 4 x 4 images, both reductions split
+                                  ((16, 128, 8, 8), 256),    # one launch: rows of 8 pixels
+                                  ((128, 128, 16, 16), 128), # one launch at a benchmark shape
+                                  ((4, 200, 16, 16), 240),   # one launch, ragged: partial tiles in both products
+                                  ((4, 160, 16, 16), 128),   # 160 input channels run as 64-row tiles: two launches
+                                  ((2, 64, 32, 32), 64),     # 64-row tiles: the two kernels one after the other
+                                  ((4, 64, 16, 16), 128),
+                                  ((16, 48, 2, 2), 40)])     # dense 2x2 route
+def test_backward_data_and_filter_gradient_as_one_call(xs, k):
+    """dopt_hip_conv_bwd_pair_packed_open against dopt_hip_conv_bwd_data_packed + dopt_hip_conv_bwd_filter (checked
+    against the oracle in test_gpu_ops.py): the same tiles in the same order, whether they run as one launch or two,
+    so dx and dw are identical to the last bit; an open dx is closed by the batch-norm gradient or by
+    dopt_hip_split_sum_close."""
+    import ctypes as C
+    from dopt_amd import capi
+    lib = capi.load()
+    r = np.random.default_rng(xs[1] * 7 + k)
+    N, Cin, H, W = xs
+    ys = (N, k, H, W)
+    d = ops.conv_desc(xs, (k, Cin, 3, 3), (1, 1), (1, 1))
+    w = ops.tensor((r.standard_normal((k, Cin, 3, 3)) * 0.05).astype(np.float32))
+    nbytes = lib.dopt_hip_conv_packed_bytes(C.byref(d), 1)
+    assert nbytes > 0
+    packed = ops.Tensor([nbytes // 4])
+    capi.check(lib.dopt_hip_conv_pack_batch(1, (type(d) * 1)(d), (C.c_int * 1)(1), (C.c_void_p * 1)(w.ptr), (C.c_void_p * 1)(packed.ptr)))
+    dy = ops.tensor(r.standard_normal(ys).astype(np.float32))
+    x = ops.tensor(r.standard_normal(xs).astype(np.float32))
+    dx_want, dw_want = ops.Tensor(xs), ops.Tensor((k, Cin, 3, 3))
+    capi.check(lib.dopt_hip_conv_bwd_data_packed(C.byref(d), dy.ptr, packed.ptr, dx_want.ptr))
+    capi.check(lib.dopt_hip_conv_bwd_filter(C.byref(d), dy.ptr, x.ptr, dw_want.ptr))
+    dx_want, dw_want = dx_want.numpy(), dw_want.numpy()
+    # closed
+    dx, dw = ops.Tensor(xs), ops.Tensor((k, Cin, 3, 3))
+    dx.set(np.full(xs, np.nan, np.float32)); dw.set(np.full((k, Cin, 3, 3), np.nan, np.float32))
+    capi.check(lib.dopt_hip_conv_pair_probe(1))
+    capi.check(lib.dopt_hip_conv_bwd_pair_packed_open(C.byref(d), dy.ptr, packed.ptr, x.ptr, dx.ptr, dw.ptr, None))
+    n, us, fl, by = C.c_int(), C.c_double(), C.c_double(), C.c_double()
+    capi.check(lib.dopt_hip_conv_pair_probe_read(C.byref(n), C.byref(us), C.byref(fl), C.byref(by)))
+    capi.check(lib.dopt_hip_conv_pair_probe(0))
+    up = lambda v, m: (v + m - 1) // m * m
+    # 128-row tiles in both products (wherever 64-row tiles would not pad less) on images of 4 x 4 pixels and more
+    one_launch = Cin > 64 and up(Cin, 128) <= up(Cin, 64) and k >= 128 and up(k, 128) <= up(k, 64) and W >= 4
+    assert n.value == (1 if one_launch else 0)
+    if one_launch:
+        assert us.value > 0 and fl.value == 2 * 2.0 * N * H * W * k * Cin * 9
+    assert np.array_equal(dx.numpy(), dx_want) and np.array_equal(dw.numpy(), dw_want)
+    # open, closed by dopt_hip_split_sum_close
+    dx.set(np.full(xs, np.nan, np.float32)); dw.set(np.full((k, Cin, 3, 3), np.nan, np.float32))
+    o = capi.SplitSum()
+    capi.check(lib.dopt_hip_conv_bwd_pair_packed_open(C.byref(d), dy.ptr, packed.ptr, x.ptr, dx.ptr, dw.ptr, C.byref(o)))
+    assert o.value == dx.ptr
+    if xs == (8, 256, 4, 4):
+        assert o.splits > 1
+    if o.splits:
+        capi.check(lib.dopt_hip_split_sum_close(C.byref(o)))
+    assert np.array_equal(dx.numpy(), dx_want) and np.array_equal(dw.numpy(), dw_want)
+    # open, closed by the batch-norm gradient one layer down
+    inner = H * W
+    xin = ops.tensor(r.standard_normal(xs).astype(np.float32))
+    yrelu = ops.tensor(np.maximum(r.standard_normal(xs), 0).astype(np.float32))
+    sc = ops.tensor(r.uniform(0.5, 1.5, Cin).astype(np.float32))
+    g_want, db_want = ops.Tensor([int(np.prod(xs)) + 2 * Cin]), ops.Tensor([Cin])
+    capi.check(lib.dopt_hip_bn_grad_fused(N, Cin, inner, ops.tensor(dx_want).ptr, yrelu.ptr, xin.ptr, sc.ptr, g_want.ptr, db_want.ptr))
+    g_got, db_got = ops.Tensor([int(np.prod(xs)) + 2 * Cin]), ops.Tensor([Cin])
+    dw.set(np.full((k, Cin, 3, 3), np.nan, np.float32))
+    o = capi.SplitSum()
+    capi.check(lib.dopt_hip_conv_bwd_pair_packed_open(C.byref(d), dy.ptr, packed.ptr, x.ptr, dx.ptr, dw.ptr, C.byref(o)))
+    capi.check(lib.dopt_hip_bn_grad_open(N, Cin, inner, C.byref(o), 1, yrelu.ptr, xin.ptr, sc.ptr, g_got.ptr, db_got.ptr))
+    assert np.array_equal(g_got.numpy(), g_want.numpy()) and np.array_equal(db_got.numpy(), db_want.numpy())
+    assert np.array_equal(dx.numpy(), dx_want) and np.array_equal(dw.numpy(), dw_want)
+    ops.sync()
 
 
 @pytest.mark.parametrize("xs,k", [((8, 256, 4, 4), 512),     # split reduction: the result is left open
