@@ -28,7 +28,7 @@ class ConvDesc(C.Structure):
 class SplitSum(C.Structure):
     """dopt_hip_split_sum: a convolution result left as partial copies for its reader to add."""
     _fields_ = [("partial", C.c_void_p), ("splits", C.c_int), ("elems", C.c_size_t), ("C", C.c_size_t),
-                ("inner", C.c_size_t), ("bias", C.c_void_p), ("value", C.c_void_p)]
+                ("inner", C.c_size_t), ("bias", C.c_void_p), ("value", C.c_void_p), ("lanes", C.c_int)]
 
 
 class TensorRef(C.Structure):
@@ -87,7 +87,7 @@ PROTOTYPES = {
     "dopt_hip_conv_bwd_data_packed_open": [C.POINTER(ConvDesc), _vp, _vp, _vp, C.POINTER(SplitSum)],
     "dopt_hip_conv_pair_probe": [_i],
     "dopt_hip_conv_pair_probe_read": [C.POINTER(_i), C.POINTER(_d), C.POINTER(_d), C.POINTER(_d)],
-    "dopt_hip_conv_bwd_pair_packed_open": [C.POINTER(ConvDesc), _vp, _vp, _vp, _vp, _vp, C.POINTER(SplitSum)],
+    "dopt_hip_conv_bwd_pair_packed_open": [C.POINTER(ConvDesc), _vp, _vp, _vp, _vp, _vp, C.POINTER(SplitSum), C.POINTER(SplitSum)],
     "dopt_hip_split_sum_close": [C.POINTER(SplitSum)],
     "dopt_hip_conv_bwd_filter": [C.POINTER(ConvDesc), _vp, _vp, _vp],
     "dopt_hip_maxpool_fwd": [_sz, _sz, _sz, _sz, _sz, _sz, _vp, _vp],
@@ -111,6 +111,8 @@ PROTOTYPES = {
     "dopt_hip_bn_grad_pool": [_sz, _sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_bn_train_open": [_sz, _sz, _sz, _d, C.POINTER(SplitSum), _vp, _vp, _vp, _vp, _vp, _i],
     "dopt_hip_bn_grad_open": [_sz, _sz, _sz, C.POINTER(SplitSum), _i, _vp, _vp, _vp, _vp, _vp],
+    "dopt_hip_bn_grad_side": [_sz, _sz, _sz, _sz, _vp, C.POINTER(SplitSum), _i, _vp, C.POINTER(SplitSum), _vp, _vp, _vp, _vp, _vp,
+                              C.POINTER(SplitSum)],
     "dopt_hip_bn_wait_limit": [C.c_uint],
     "dopt_hip_bn_infer": [_sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp],
     "dopt_hip_optim_create": [_i, C.POINTER(TensorRef), C.POINTER(_vp)],

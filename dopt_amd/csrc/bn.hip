@@ -60,7 +60,41 @@ struct Pool {
     unsigned wq, wshift;  // quads per image row and its log2 (mode 1)
     float *pooled;        // forward: [N, C, H/2, W/2]
     const float *dpool;   // backward: gradient of that tensor
+    // backward, dsplits > 1: the gradient still lies in `dsplits` partial copies, `dstride` floats apart, the first
+    // at dpool; the kernel adds them in order as it routes them and writes the sum to dvalue unless that is null
+    unsigned dsplits;
+    size_t dstride;
+    float *dvalue;
 };
+
+// The value at `at` (in units of V) of a pooled gradient that may still lie in partial copies: copy 0 + copy 1 + ...
+// in that order, up to four loads in flight (indices clamped to the last copy, surplus values dropped).
+template <typename V>
+__device__ inline V pool_dvalue(const Pool &pl, size_t at, bool write)
+{
+    const V *src = (const V *)pl.dpool + at;
+    if (pl.dsplits <= 1) return *src;
+    const size_t stride = pl.dstride / (sizeof(V) / sizeof(float));
+    const unsigned last = pl.dsplits - 1;
+    V acc = src[0];
+    for (unsigned s = 1; s <= last; s += 4) {
+        const unsigned s1 = min(s + 1, last), s2 = min(s + 2, last), s3 = min(s + 3, last);
+        const V v0 = src[(size_t)s * stride], v1 = src[(size_t)s1 * stride], v2 = src[(size_t)s2 * stride], v3 = src[(size_t)s3 * stride];
+        if constexpr (sizeof(V) == sizeof(float)) {
+            acc += v0;
+            if (s + 1 <= last) acc += v1;
+            if (s + 2 <= last) acc += v2;
+            if (s + 3 <= last) acc += v3;
+        } else {
+            acc.x += v0.x; acc.y += v0.y;
+            if (s + 1 <= last) { acc.x += v1.x; acc.y += v1.y; }
+            if (s + 2 <= last) { acc.x += v2.x; acc.y += v2.y; }
+            if (s + 3 <= last) { acc.x += v3.x; acc.y += v3.y; }
+        }
+    }
+    if (write && pl.dvalue) ((V *)pl.dvalue)[at] = acc;
+    return acc;
+}
 
 __device__ inline float4 quad_xor(float4 v, unsigned lanes)
 {
@@ -92,14 +126,15 @@ __device__ inline float4 pool_grad(const Pool &pl, float4 y, unsigned idx)
     const bool present = idx != 0xffffffffu;
     float4 r;
     if (pl.mode == 2) {
-        const float g = present ? pl.dpool[idx] : 0.0f;
+        const float g = present ? pool_dvalue<float>(pl, idx, true) : 0.0f;
         route2x2(y.x, y.y, y.z, y.w, g, r.x, r.y, r.z, r.w);
         return r;
     }
     const float4 o = quad_xor(y, pl.wq);
     const unsigned row = present ? idx >> pl.wshift : 0u, cq = idx & (pl.wq - 1);
     const bool odd = row & 1;
-    const float2 g = present ? ((const float2 *)pl.dpool)[(size_t)(row >> 1) * pl.wq + cq] : make_float2(0.0f, 0.0f);
+    // both rows of a window read its gradient; the even row writes the finished sum of an open one
+    const float2 g = present ? pool_dvalue<float2>(pl, (size_t)(row >> 1) * pl.wq + cq, !odd) : make_float2(0.0f, 0.0f);
     const float4 top = odd ? o : y, bot = odd ? y : o;
     float4 t, b;
     route2x2(top.x, top.y, bot.x, bot.y, g.x, t.x, t.y, b.x, b.y);
@@ -487,6 +522,48 @@ __device__ __forceinline__ void open_add(const OpenSum &open, const unsigned (&a
     }
 }
 
+// A sum that rides along in a batch-norm launch: `splits` partial copies of n4 quads (stride n4), added by the
+// workgroups from `first` on in the order of the filter gradient's own finishing pass (split_sum_k in conv.hip:
+// `lanes` interleaved lanes, lane l folding copies l, l + lanes, ... in four chains that start from zero, lane
+// value (a0 + a1) + (a2 + a3), lanes added in lane order, a lane without copies contributing +0).  One thread
+// per quad walks the lanes one after the other with a lane's four chains in flight.
+struct SideSum {
+    const float4 *partial;
+    float4 *out;
+    unsigned n4, splits, lanes;
+    unsigned first;   // 0: nothing rides
+};
+
+__device__ inline void add4(float4 &a, const float4 v)
+{
+    a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w;
+}
+
+__device__ inline void side_sum(const SideSum &sd)
+{
+    const unsigned L = sd.lanes, S = sd.splits;
+    const size_t step = (size_t)(gridDim.x - sd.first) * blockDim.x;
+    for (size_t i = (size_t)(blockIdx.x - sd.first) * blockDim.x + threadIdx.x; i < sd.n4; i += step) {
+        const float4 *q = sd.partial + i;
+        float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (unsigned sl = 0; sl < L; sl++) {
+            float4 a0 = make_float4(0.f, 0.f, 0.f, 0.f), a1 = a0, a2 = a0, a3 = a0;
+            unsigned sp = sl;
+            for (; sp + 3 * L < S; sp += 4 * L) {
+                const float4 v0 = q[(size_t)sp * sd.n4], v1 = q[(size_t)(sp + L) * sd.n4];
+                const float4 v2 = q[(size_t)(sp + 2 * L) * sd.n4], v3 = q[(size_t)(sp + 3 * L) * sd.n4];
+                add4(a0, v0); add4(a1, v1); add4(a2, v2); add4(a3, v3);
+            }
+            for (; sp < S; sp += L) add4(a0, q[(size_t)sp * sd.n4]);
+            const float4 lane = make_float4((a0.x + a1.x) + (a2.x + a3.x), (a0.y + a1.y) + (a2.y + a3.y),
+                                            (a0.z + a1.z) + (a2.z + a3.z), (a0.w + a1.w) + (a2.w + a3.w));
+            if (sl == 0) r = lane;
+            else add4(r, lane);
+        }
+        sd.out[i] = r;
+    }
+}
+
 // kQ: float4 per thread (a thread of the open variant holds kQ quads of every copy at once, so it is
 // built for small channels only).
 template <bool kGrad, bool kOpen, int kQ>
@@ -494,9 +571,13 @@ __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, un
                                                        const float *x, const float *dy, const float *scale,
                                                        const float *bias, const float *run_mean, const float *run_var,
                                                        const float *ymask, int relu, float *out, float *out1, float *out2,
-                                                       float *dx_sum, OpenSum open, Pool pool)
+                                                       float *dx_sum, OpenSum open, Pool pool, SideSum side)
 {
     __shared__ float part[3][16];
+    if (side.first && blockIdx.x >= side.first) {   // a workgroup behind the channels': the sum that rides along
+        side_sum(side);
+        return;
+    }
     const unsigned c = blockIdx.x, T = blockDim.x, E4 = N * inner4;
     const float4 *x4 = (const float4 *)x, *g4 = (const float4 *)dy;
     float4 xv[kQ], gv[kQ];
@@ -689,11 +770,15 @@ __global__ __launch_bounds__(1024) void bn_cluster_k(unsigned N, unsigned C, uns
                                                       const float *scale, const float *bias, const float *run_mean,
                                                       const float *run_var, const float *ymask, int relu, float *out,
                                                       float *out1, float *out2, float *dx_sum, ClusterMem cm,
-                                                      unsigned spin_limit, Pool pool)
+                                                      unsigned spin_limit, Pool pool, SideSum side)
 {
     constexpr int kQ = kResQuads;
     __shared__ float part[3][16];
     __shared__ double comb[4];
+    if (side.first && blockIdx.x >= side.first) {   // behind every cluster: the sum that rides along (waits for no one)
+        side_sum(side);
+        return;
+    }
     const unsigned c = blockIdx.x / S, piece = blockIdx.x - c * S, T = blockDim.x, E4 = N * inner4;
     const unsigned q0 = piece * per;                                  // this block's quads: [q0, q0 + mine)
     const unsigned mine = E4 - q0 < per ? E4 - q0 : per;
@@ -1023,6 +1108,8 @@ struct PoolArg {
     size_t H, W;
     float *pooled;        // forward
     const float *dpool;   // backward
+    const dopt_hip_split_sum *dopen = nullptr;   // backward: dpool still lies in partial copies (or null)
+    bool keep = true;                            // ... and its finished value is wanted as well
 };
 
 bool pool_inline(const PoolArg *a, Pool *k)
@@ -1068,7 +1155,7 @@ int bn_train_impl(size_t N, size_t C, size_t inner, double momentum, const float
             hipLaunchKernelGGL((bn_resident_k<false, true, kOpenQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N, (unsigned)C,
                                (unsigned)(inner / 4), factor, eps, x, (const float *)nullptr, scale, bias, run_mean, run_var,
                                (const float *)nullptr, relu, packed, packed + total, packed + total + C, (float *)nullptr, os,
-                               pool_in ? pl : Pool{});
+                               pool_in ? pl : Pool{}, SideSum{});
             DOPT_LAUNCH_CHECK();
             return pool_in ? DOPT_HIP_OK : pooled_after();
         }
@@ -1082,7 +1169,7 @@ int bn_train_impl(size_t N, size_t C, size_t inner, double momentum, const float
         hipLaunchKernelGGL((bn_cluster_k<false>), dim3((unsigned)(C * S)), dim3(1024), 0, stream(), (unsigned)N, (unsigned)C,
                            (unsigned)(inner / 4), S, per, factor, eps, x, (const float *)nullptr, scale, bias, run_mean,
                            run_var, (const float *)nullptr, relu, packed, packed + total, packed + total + C,
-                           (float *)nullptr, cm, g_cluster_spin_limit, in ? pl : Pool{});
+                           (float *)nullptr, cm, g_cluster_spin_limit, in ? pl : Pool{}, SideSum{});
         DOPT_LAUNCH_CHECK();
         g_cluster_unchecked = true;
         return in ? DOPT_HIP_OK : pooled_after();
@@ -1093,12 +1180,12 @@ int bn_train_impl(size_t N, size_t C, size_t inner, double momentum, const float
             hipLaunchKernelGGL((bn_resident_k<false, false, kOpenQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N,
                                (unsigned)C, (unsigned)(inner / 4), factor, eps, x, (const float *)nullptr, scale, bias, run_mean,
                                run_var, (const float *)nullptr, relu, packed, packed + total, packed + total + C,
-                               (float *)nullptr, OpenSum{}, pool_in ? pl : Pool{});
+                               (float *)nullptr, OpenSum{}, pool_in ? pl : Pool{}, SideSum{});
         else
             hipLaunchKernelGGL((bn_resident_k<false, false, kResQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N,
                                (unsigned)C, (unsigned)(inner / 4), factor, eps, x, (const float *)nullptr, scale, bias, run_mean,
                                run_var, (const float *)nullptr, relu, packed, packed + total, packed + total + C,
-                               (float *)nullptr, OpenSum{}, pool_in ? pl : Pool{});
+                               (float *)nullptr, OpenSum{}, pool_in ? pl : Pool{}, SideSum{});
         DOPT_LAUNCH_CHECK();
         return pool_in ? DOPT_HIP_OK : pooled_after();
     }
@@ -1118,9 +1205,31 @@ int bn_train_impl(size_t N, size_t C, size_t inner, double momentum, const float
     return pooled_after();
 }
 
+// The kernel-side description of a sum that rides along, for a launch whose own workgroups are `own` of `T`
+// threads: false when `side` is null, complete or not of that kind (the caller closes it first).
+bool side_sum_arg(const dopt_hip_split_sum *side, unsigned own, unsigned T, SideSum *k, unsigned *blocks)
+{
+    *k = SideSum{};
+    *blocks = 0;
+    if (!side || side->splits < 2 || side->lanes <= 0 || !side->partial || !side->value || side->elems % 4 != 0 ||
+        !aligned16(side->partial) || !aligned16(side->value) || side->elems / 4 >= 0xffffffffull || own == 0 || T == 0)
+        return false;
+    k->partial = (const float4 *)side->partial;
+    k->out = (float4 *)side->value;
+    k->n4 = (unsigned)(side->elems / 4);
+    k->splits = (unsigned)side->splits;
+    k->lanes = (unsigned)side->lanes;
+    k->first = own;
+    // one quad per thread, at most 1024 threads' worth per compute unit (the loop strides beyond that)
+    const size_t want = ceil_div((size_t)k->n4, (size_t)T), cap = ceil_div((size_t)num_cus() * 1024, (size_t)T);
+    *blocks = (unsigned)(want < cap ? want : cap);
+    return true;
+}
+
 int bn_grad_impl(size_t N, size_t C, size_t inner, const float *dy, const float *ymask, const float *x,
                  const float *scale, float *packed, float *dx_sum, const char *who,
-                 const dopt_hip_split_sum *dy_open = nullptr, bool keep_dy = true, const PoolArg *pool = nullptr)
+                 const dopt_hip_split_sum *dy_open = nullptr, bool keep_dy = true, const PoolArg *pool = nullptr,
+                 const dopt_hip_split_sum *side = nullptr)
 {
     size_t total = N * C * inner;
     DOPT_REQUIRE(total > 0, "%s: empty input", who);
@@ -1129,14 +1238,50 @@ int bn_grad_impl(size_t N, size_t C, size_t inner, const float *dy, const float 
     DOPT_ENSURE_INIT();
     double eps = (double)1e-5f;  // cudnn7.d:634
     unsigned T = (!ymask || aligned16(ymask)) ? resident_threads(N, C, inner, x, dy, packed) : 0;
+    unsigned per = 0;
+    const unsigned clusterS = cluster_pieces(N, C, inner, x, pool ? nullptr : dy, ymask, packed, &per);
+    // A sum that rides along does so in the launch of a register-resident kernel; the other paths (which use the
+    // workspace its copies lie in) finish it first.
+    if (side && side->splits) {
+        DOPT_REQUIRE(side->splits > 1 && side->lanes > 0 && side->partial && side->value, "%s: malformed side sum", who);
+        SideSum probe;
+        unsigned nb;
+        if (!(clusterS || T) || !side_sum_arg(side, 1, 64, &probe, &nb)) {
+            if (int rc = dopt_hip_split_sum_close(side)) return rc;
+            side = nullptr;
+        }
+    } else {
+        side = nullptr;
+    }
+    SideSum sd{};
+    unsigned side_blocks = 0;
+    auto with_side = [&](unsigned own, unsigned threads) {   // grid of a launch whose own workgroups are `own`
+        if (side && side_sum_arg(side, own, threads, &sd, &side_blocks)) open_split_clear(side->partial);
+        return dim3(own + side_blocks);
+    };
     Pool pl{};
     if (pool) {
         // dy = maxpoolGrad(dpool, y): made inside a register-resident kernel where one will run, else by a pass
         // of its own into the output buffer, which every path below may read as dy while it writes dx (each
         // thread reads its elements before it writes them)
-        unsigned per = 0;
-        const unsigned S = cluster_pieces(N, C, inner, x, nullptr, ymask, packed, &per);
-        const bool in = pool_inline(pool, &pl) && (S ? (pl.mode == 2 || per % (2 * pl.wq) == 0) : T != 0);
+        const bool in = pool_inline(pool, &pl) && (clusterS ? (pl.mode == 2 || per % (2 * pl.wq) == 0) : T != 0);
+        const dopt_hip_split_sum *dopen = pool->dopen && pool->dopen->splits ? pool->dopen : nullptr;
+        if (dopen) {
+            // the kernel adds the copies itself where it routes the gradient anyway; else they are added first
+            const size_t pelems = total / 4;
+            const bool ok = in && dopen->splits > 1 && dopen->lanes == 0 && dopen->elems == pelems && !dopen->bias &&
+                            dopen->partial && dopen->value == pool->dpool && pelems % 4 == 0 && aligned16(dopen->partial) &&
+                            aligned16(dopen->value);
+            if (ok) {
+                open_split_clear(dopen->partial);
+                pl.dpool = dopen->partial;
+                pl.dsplits = (unsigned)dopen->splits;
+                pl.dstride = pelems;
+                pl.dvalue = pool->keep ? dopen->value : nullptr;
+            } else if (int rc = dopt_hip_split_sum_close(dopen)) {
+                return rc;
+            }
+        }
         if (!in) {
             pl = Pool{};
             if (int rc = dopt_hip_maxpool_bwd(N, C, pool->H, pool->W, 2, 2, pool->dpool, ymask, packed)) return rc;
@@ -1147,38 +1292,40 @@ int bn_grad_impl(size_t N, size_t C, size_t inner, const float *dy, const float 
         OpenSum os;
         if (T && N * (inner / 4) <= (size_t)kOpenQuads * T && open_sum(dy_open, total, C, inner, keep_dy, &os)) {
             open_split_clear(dy_open->partial);
-            hipLaunchKernelGGL((bn_resident_k<true, true, kOpenQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N, (unsigned)C,
+            const dim3 grid = with_side((unsigned)C, T);
+            hipLaunchKernelGGL((bn_resident_k<true, true, kOpenQuads>), grid, dim3(T), 0, stream(), (unsigned)N, (unsigned)C,
                                (unsigned)(inner / 4), 0.0, eps, x, dy, scale, (const float *)nullptr,
                                (const float *)nullptr, (const float *)nullptr, ymask, 0, packed, packed + total,
-                               packed + total + C, dx_sum, os, Pool{});
+                               packed + total + C, dx_sum, os, Pool{}, sd);
             DOPT_LAUNCH_CHECK();
             return DOPT_HIP_OK;
         }
         if (int rc = dopt_hip_split_sum_close(dy_open)) return rc;
     }
-    unsigned per = 0;
     if (const unsigned S = cluster_pieces(N, C, inner, x, dy, ymask, packed, &per)) {
         ClusterMem cm;
         if (int rc = cluster_mem(&cm)) return rc;
-        hipLaunchKernelGGL((bn_cluster_k<true>), dim3((unsigned)(C * S)), dim3(1024), 0, stream(), (unsigned)N, (unsigned)C,
+        const dim3 grid = with_side((unsigned)(C * S), 1024);
+        hipLaunchKernelGGL((bn_cluster_k<true>), grid, dim3(1024), 0, stream(), (unsigned)N, (unsigned)C,
                            (unsigned)(inner / 4), S, per, 0.0, eps, x, dy, scale, (const float *)nullptr,
                            (const float *)nullptr, (const float *)nullptr, ymask, 0, packed, packed + total,
-                           packed + total + C, dx_sum, cm, g_cluster_spin_limit, pl);
+                           packed + total + C, dx_sum, cm, g_cluster_spin_limit, pl, sd);
         DOPT_LAUNCH_CHECK();
         g_cluster_unchecked = true;
         return DOPT_HIP_OK;
     }
     if (T) {
+        const dim3 grid = with_side((unsigned)C, T);
         if (N * (inner / 4) <= (size_t)kOpenQuads * T)
-            hipLaunchKernelGGL((bn_resident_k<true, false, kOpenQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N,
+            hipLaunchKernelGGL((bn_resident_k<true, false, kOpenQuads>), grid, dim3(T), 0, stream(), (unsigned)N,
                                (unsigned)C, (unsigned)(inner / 4), 0.0, eps, x, dy, scale, (const float *)nullptr,
                                (const float *)nullptr, (const float *)nullptr, ymask, 0, packed, packed + total,
-                               packed + total + C, dx_sum, OpenSum{}, pl);
+                               packed + total + C, dx_sum, OpenSum{}, pl, sd);
         else
-            hipLaunchKernelGGL((bn_resident_k<true, false, kResQuads>), dim3((unsigned)C), dim3(T), 0, stream(), (unsigned)N,
+            hipLaunchKernelGGL((bn_resident_k<true, false, kResQuads>), grid, dim3(T), 0, stream(), (unsigned)N,
                                (unsigned)C, (unsigned)(inner / 4), 0.0, eps, x, dy, scale, (const float *)nullptr,
                                (const float *)nullptr, (const float *)nullptr, ymask, 0, packed, packed + total,
-                               packed + total + C, dx_sum, OpenSum{}, pl);
+                               packed + total + C, dx_sum, OpenSum{}, pl, sd);
         DOPT_LAUNCH_CHECK();
         return DOPT_HIP_OK;
     }
@@ -1308,6 +1455,30 @@ int dopt_hip_bn_grad_pool(size_t N, size_t C, size_t H, size_t W, const float *d
     DOPT_REQUIRE((H & 1) == 0 && (W & 1) == 0, "dopt_hip_bn_grad_pool: images of %zu x %zu do not split into 2 x 2 windows", H, W);
     const PoolArg pa{H, W, nullptr, dpooled};
     return bn_grad_impl(N, C, H * W, nullptr, y, x, scale, packed, dx_sum, "dopt_hip_bn_grad_pool", nullptr, true, &pa);
+}
+
+int dopt_hip_bn_grad_side(size_t N, size_t C, size_t H, size_t W, const float *dy, const dopt_hip_split_sum *dy_open,
+                          int keep_dy, const float *dpooled, const dopt_hip_split_sum *dpooled_open, const float *y,
+                          const float *x, const float *scale, float *packed, float *dx_sum, const dopt_hip_split_sum *side)
+{
+    const char *who = "dopt_hip_bn_grad_side";
+    DOPT_REQUIRE((dy != nullptr) + (dy_open != nullptr) + (dpooled != nullptr) == 1,
+                 "%s: exactly one of dy, dy_open and dpooled says where the incoming gradient is", who);
+    DOPT_REQUIRE(!dpooled_open || dpooled, "%s: dpooled_open without dpooled", who);
+    if (dpooled) {
+        DOPT_REQUIRE(y != nullptr, "%s: the pooled form needs y", who);
+        DOPT_REQUIRE((H & 1) == 0 && (W & 1) == 0, "%s: images of %zu x %zu do not split into 2 x 2 windows", who, H, W);
+        DOPT_REQUIRE(!dpooled_open || dpooled_open->value == dpooled, "%s: dpooled is not the open value", who);
+        PoolArg pa{H, W, nullptr, dpooled};
+        pa.dopen = dpooled_open;
+        pa.keep = keep_dy != 0;
+        return bn_grad_impl(N, C, H * W, nullptr, y, x, scale, packed, dx_sum, who, nullptr, true, &pa, side);
+    }
+    if (dy_open) {
+        DOPT_REQUIRE(dy_open->value != nullptr, "%s: null argument", who);
+        return bn_grad_impl(N, C, H * W, dy_open->value, y, x, scale, packed, dx_sum, who, dy_open, keep_dy != 0, nullptr, side);
+    }
+    return bn_grad_impl(N, C, H * W, dy, y, x, scale, packed, dx_sum, who, nullptr, true, nullptr, side);
 }
 
 int dopt_hip_bn_grad_fused(size_t N, size_t C, size_t inner, const float *dy, const float *y, const float *x,

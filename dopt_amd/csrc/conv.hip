@@ -1792,19 +1792,30 @@ WgradSetup wgrad_patch_setup(const dopt_hip_conv_desc *d, const float *dw)
     return u;
 }
 
+// Split lanes of the pass that adds a filter gradient's partial copies: enough blocks for small filters with
+// hundreds of splits means more split lanes per block.
+int wgrad_sum_lanes(size_t n4) { return n4 >= (size_t)64 * 512 ? 4 : 16; }
+
+// out = `splits` partial copies of n4 quads added in the order `lanes` fixes (split_sum_k)
+int launch_split_sum(size_t n4, int splits, int lanes, const float *partial, float *out)
+{
+    if (lanes == 4)
+        hipLaunchKernelGGL(split_sum_k<4>, dim3((unsigned)ceil_div(n4, (size_t)64)), dim3(256), 0, stream(), n4, splits, n4,
+                           (const float4 *)partial, (float4 *)out);
+    else if (lanes == 16)
+        hipLaunchKernelGGL(split_sum_k<16>, dim3((unsigned)ceil_div(n4, (size_t)16)), dim3(256), 0, stream(), n4, splits, n4,
+                           (const float4 *)partial, (float4 *)out);
+    else
+        return fail(DOPT_HIP_ERR_INVALID, "split sum: %d lanes (4 or 16)", lanes);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
 // dw = the partial filters added in split order
 int wgrad_split_sum(const WgradSetup &u, const float *partial, float *dw)
 {
-    // enough blocks for small filters with hundreds of splits: more split lanes per block
     const size_t n4 = u.out_elems / 4;
-    if (n4 >= (size_t)64 * 512)
-        hipLaunchKernelGGL(split_sum_k<4>, dim3((unsigned)ceil_div(n4, (size_t)64)), dim3(256), 0, stream(), n4, u.splits,
-                           n4, (const float4 *)partial, (float4 *)dw);
-    else
-        hipLaunchKernelGGL(split_sum_k<16>, dim3((unsigned)ceil_div(n4, (size_t)16)), dim3(256), 0, stream(), n4, u.splits,
-                           n4, (const float4 *)partial, (float4 *)dw);
-    DOPT_LAUNCH_CHECK();
-    return DOPT_HIP_OK;
+    return launch_split_sum(n4, u.splits, wgrad_sum_lanes(n4), partial, dw);
 }
 
 int run_wgrad_patch(const dopt_hip_conv_desc *d, const float *dy, const float *x, float *dw, bool *done)
@@ -1864,7 +1875,7 @@ struct PairProbe {
 PairProbe g_pair_probe;
 
 int run_bwd_pair(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *dy, const float *prepacked, const float *x,
-                 float *dx, float *dw, dopt_hip_split_sum *open, bool *done)
+                 float *dx, float *dw, dopt_hip_split_sum *open, dopt_hip_split_sum *open_dw, bool *done)
 {
     *done = false;
     PatchSetup a = patch_setup<true>(d, P, Q);
@@ -1916,8 +1927,16 @@ int run_bwd_pair(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *d
         probe.bytes += 4.0 * (2.0 * px * d->C + px * d->K + 2.0 * (double)d->K * d->C * 9.0);   // dy, x, dx, filter, dw once each
     }
     *done = true;
-    if (b.splits > 1)
+    if (b.splits > 1 && open_dw) {   // the caller's next call adds the copies
+        open_dw->partial = partial_b;
+        open_dw->splits = b.splits;
+        open_dw->elems = b.out_elems;
+        open_dw->value = dw;
+        open_dw->lanes = wgrad_sum_lanes(b.out_elems / 4);
+        open_split_set(partial_b);
+    } else if (b.splits > 1) {
         if (int rc2 = wgrad_split_sum(b, partial_b, dw)) return rc2;
+    }
     if (splits_a > 1 && open) {   // the caller's next call adds the copies
         open->partial = partial_a;
         open->splits = splits_a;
@@ -2071,7 +2090,7 @@ int dopt_hip_conv_bwd_data_packed(const dopt_hip_conv_desc *d, const float *dy, 
 }
 
 int dopt_hip_conv_bwd_pair_packed_open(const dopt_hip_conv_desc *d, const float *dy, const float *packed, const float *x,
-                                       float *dx, float *dw, dopt_hip_split_sum *open)
+                                       float *dx, float *dw, dopt_hip_split_sum *open, dopt_hip_split_sum *open_dw)
 {
     size_t P, Q;
     if (int rc = check_desc(d, &P, &Q, "dopt_hip_conv_bwd_pair_packed_open")) return rc;
@@ -2081,8 +2100,12 @@ int dopt_hip_conv_bwd_pair_packed_open(const dopt_hip_conv_desc *d, const float 
         *open = dopt_hip_split_sum{};
         open->value = dx;
     }
+    if (open_dw) {
+        *open_dw = dopt_hip_split_sum{};
+        open_dw->value = dw;
+    }
     bool done = false;
-    if (int rc = run_bwd_pair(d, P, Q, dy, packed, x, dx, dw, open, &done)) return rc;
+    if (int rc = run_bwd_pair(d, P, Q, dy, packed, x, dx, dw, open, open_dw, &done)) return rc;
     if (done) return DOPT_HIP_OK;
     // not a pair the one-launch kernel takes: filter gradient first (it may use the workspace), then backward-data,
     // which may leave its result open in it
@@ -2125,10 +2148,12 @@ int dopt_hip_split_sum_close(const dopt_hip_split_sum *open)
 {
     DOPT_REQUIRE(open != nullptr, "dopt_hip_split_sum_close: null argument");
     if (open->splits == 0) return DOPT_HIP_OK;
-    DOPT_REQUIRE(open->splits > 1 && open->partial && open->value && open->elems % 4 == 0 && open->C > 0 && open->inner > 0,
+    DOPT_REQUIRE(open->splits > 1 && open->partial && open->value && open->elems % 4 == 0 &&
+                     (open->lanes > 0 || (open->C > 0 && open->inner > 0)),
                  "dopt_hip_split_sum_close: malformed description");
     DOPT_ENSURE_INIT();
     open_split_clear(open->partial);
+    if (open->lanes > 0) return launch_split_sum(open->elems / 4, open->splits, open->lanes, open->partial, open->value);
     return launch_splitk_reduce(open->elems, open->splits, open->partial, open->value, open->bias, (unsigned)open->C,
                                 (unsigned)open->inner);
 }

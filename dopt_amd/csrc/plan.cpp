@@ -1290,7 +1290,7 @@ int HIPPlan::Builder::buildSteps()
                 float *dw = (float *)p->mResults[pairOf[id]];
                 k = make([=](const std::vector<const void *> &in, void *out) {
                     return dopt_hip_conv_bwd_pair_packed_open(&d, (const float *)in[0], packed, (const float *)in[1], (float *)out,
-                                                              dw, nullptr);
+                                                              dw, nullptr, nullptr);
                 });
                 label = "convolutionFeaturesGrad+convolutionFiltersGrad";
             } else if (pk.bwd) {
@@ -1392,16 +1392,25 @@ void HIPPlan::Builder::openSplitSums()
                 });
             }
         } else if (cs.bwd && bo.opType == "batchNormGrad" && bo.deps.size() == 3 &&
-                   ((fusedKind[b] == 3 && next.inputOps.size() == 4) || (fusedKind[b] == 0 && next.inputOps.size() == 3))) {
-            const bool relu = fusedKind[b] == 3;
+                   (((fusedKind[b] == 3 || fusedKind[b] == 8) && next.inputOps.size() == 4) ||
+                    (fusedKind[b] == 0 && next.inputOps.size() == 3))) {
+            // kind 8: the gradient arrives through a 2 x 2 max-pool and a relu (inputs [dpooled, y, x, scale]); kind 3:
+            // through a relu ([dy, y, x, scale]); kind 0: as it is ([dy, x, scale])
+            const int kind = fusedKind[b];
+            const bool has_y = kind != 0;
             void *extra = biasGradOf[b] >= 0 && needed[biasGradOf[b]] ? p->mResults[biasGradOf[b]] : nullptr;
-            nci(g.ops[bo.deps[1]].shape, &N, &C, &inner);
+            const auto &xs = g.ops[bo.deps[1]].shape;
+            if (kind == 8 && xs.size() != 4) continue;
+            nci(xs, &N, &C, &inner);
+            const size_t H = kind == 8 ? xs[2] : inner, W = kind == 8 ? xs[3] : 1;
             const int keep = uses[cs.op].size() == 1 && !isOutput(cs.op) ? 0 : 1;   // does anything else read dy?
+            // the filter gradient of a backward pair stays open as well: the gradient kernel's launch adds its copies
+            auto side = std::make_shared<dopt_hip_split_sum>();
             if (pairOf[cs.op] >= 0) {
                 float *dw = (float *)p->mResults[pairOf[cs.op]];
                 conv.kernel = make([=](const std::vector<const void *> &in, void *out) {
                     return dopt_hip_conv_bwd_pair_packed_open(&d, (const float *)in[0], packed, (const float *)in[1], (float *)out,
-                                                              dw, open.get());
+                                                              dw, open.get(), side.get());
                 });
             } else {
                 conv.kernel = make([=](const std::vector<const void *> &in, void *out) {
@@ -1410,9 +1419,13 @@ void HIPPlan::Builder::openSplitSums()
             }
             next.kernel = make([=](const std::vector<const void *> &in, void *out) {
                 if (open->value != in[0]) return fail(DOPT_HIP_ERR_RUNTIME, "plan: open convolution result is not the gradient's input");
-                const float *y = relu ? (const float *)in[1] : nullptr;
-                const float *x = (const float *)in[relu ? 2 : 1], *scale = (const float *)in[relu ? 3 : 2];
-                return dopt_hip_bn_grad_open(N, C, inner, open.get(), keep, y, x, scale, (float *)out, (float *)extra);
+                const float *y = has_y ? (const float *)in[1] : nullptr;
+                const float *x = (const float *)in[has_y ? 2 : 1], *scale = (const float *)in[has_y ? 3 : 2];
+                if (kind == 8)
+                    return dopt_hip_bn_grad_side(N, C, H, W, nullptr, nullptr, keep, (const float *)in[0], open.get(), y, x, scale,
+                                                 (float *)out, (float *)extra, side.get());
+                return dopt_hip_bn_grad_side(N, C, H, W, nullptr, open.get(), keep, nullptr, nullptr, y, x, scale, (float *)out,
+                                             (float *)extra, side.get());
             });
         }
     }

@@ -39,7 +39,7 @@ struct Runtime {
     void *ws[2] = {nullptr, nullptr};
     size_t ws_bytes[2] = {0, 0};
     unsigned long ws_generation = 0;   // bumped whenever a workspace moves: recorded graphs hold its address
-    const void *open_split[2] = {nullptr, nullptr};   // partial copies a convolution left in the workspace for its reader
+    const void *open_split[2][2] = {{nullptr, nullptr}, {nullptr, nullptr}};   // per queue: partial copies convolutions left in the workspace for their readers
 
     // rtc
     std::unordered_map<std::string, hipFunction_t> kernels;
@@ -127,22 +127,29 @@ bool capturing() { return rt().capturing; }
 int num_cus() { return rt().cus; }
 unsigned long workspace_generation() { return rt().ws_generation; }
 
-void open_split_set(const void *partial) { rt().open_split[rt().lane] = partial; }
+void open_split_set(const void *partial)
+{
+    Runtime &r = rt();
+    const void **slot = r.open_split[r.lane];
+    if (slot[0] == partial || slot[1] == partial) return;
+    slot[slot[0] ? 1 : 0] = partial;   // at most two are pending at once: a backward pair's dx and dw
+}
 void open_split_clear(const void *partial)
 {
     Runtime &r = rt();
-    if (r.open_split[r.lane] == partial) r.open_split[r.lane] = nullptr;
+    for (const void *&slot : r.open_split[r.lane])
+        if (slot == partial) slot = nullptr;
 }
 
 void *workspace(size_t bytes)
 {
     Runtime &r = rt();
     const int l = r.lane;
-    if (r.open_split[l]) {
+    if (r.open_split[l][0] || r.open_split[l][1]) {
         // the previous call left partial sums here for the NEXT call to add up; anything else would overwrite them
-        r.open_split[l] = nullptr;   // report once
+        r.open_split[l][0] = r.open_split[l][1] = nullptr;   // report once
         fail(DOPT_HIP_ERR_INVALID, "an open convolution result (dopt_hip_conv_*_packed_open) was not closed by the call "
-                                   "that followed it: dopt_hip_split_sum_close, dopt_hip_bn_train_open or dopt_hip_bn_grad_open");
+                                   "that followed it: dopt_hip_split_sum_close, dopt_hip_bn_train_open, dopt_hip_bn_grad_open or dopt_hip_bn_grad_side");
         return nullptr;
     }
     if (bytes <= r.ws_bytes[l]) return r.ws[l];

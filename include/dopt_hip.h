@@ -235,6 +235,11 @@ typedef struct dopt_hip_split_sum {
     size_t C, inner;      /* the value is [N, C, inner] */
     const float *bias;    /* per-channel addend of the finished sum, or null */
     float *value;         /* where the finished sum belongs */
+    int lanes;            /* 0: the copies are added one after the other (((c0 + c1) + c2) + ...).  L > 0 (an open filter
+                             gradient): L interleaved lanes, lane l folding copies l, l + L, l + 2L, ... in four chains
+                             (chain j takes every fourth of them, starting from zero), lane value = (ch0 + ch1) + (ch2 + ch3),
+                             and the lane values are added in lane order: the order of the filter gradient's own
+                             finishing pass.  C, inner and bias are not used then. */
 } dopt_hip_split_sum;
 int dopt_hip_conv_fwd_bias_packed_open(const dopt_hip_conv_desc *d, const float *x, const float *packed,
                                        const float *bias, float *y, dopt_hip_split_sum *open);
@@ -245,9 +250,14 @@ int dopt_hip_conv_bwd_data_packed_open(const dopt_hip_conv_desc *d, const float 
    cudnnConvolutionBackwardFilter (cudnn7.d:244) read the same dy and nothing of each other.  For 3x3 unit-stride
    layers of at least 128 input and output channels on rows of 8 .. 64 pixels or 4 x 4 images both run as ONE
    launch, the filter-gradient tiles starting on each compute unit as its backward-data tile ends; every other
-   shape runs the two entry points one after the other.  dx and dw are bit for bit what those write. */
+   shape runs the two entry points one after the other.  dx and dw are bit for bit what those write.
+   open_dw (may be null): where the one launch leaves the filter gradient as partial copies (it always splits its
+   pixels over the compute units), the pass that adds them is skipped and the copies are described there, to be
+   closed by the next call like an open dx: dopt_hip_split_sum_close, or dopt_hip_bn_grad_side, whose launch adds
+   them on compute units the batch norm leaves idle.  Both open and open_dw may be pending at once. */
 int dopt_hip_conv_bwd_pair_packed_open(const dopt_hip_conv_desc *d, const float *dy, const float *packed,
-                                       const float *x, float *dx, float *dw, dopt_hip_split_sum *open);
+                                       const float *x, float *dx, float *dw, dopt_hip_split_sum *open,
+                                       dopt_hip_split_sum *open_dw);
 /* Measurement aid (no counterpart in the reference; CUDAPlan.profiler, cuda/package.d:424-431, times whole kernel
    objects): while enabled, every one-launch pair above is bracketed by two events on the library's queue, so its
    device time is known apart from the split sums the same entry point runs.  probe(1) starts a fresh collection,
@@ -377,6 +387,20 @@ int dopt_hip_bn_train_pool(size_t N, size_t C, size_t H, size_t W, double moment
                            const float *run_mean, const float *run_var, float *packed, int relu, float *pooled);
 int dopt_hip_bn_grad_pool(size_t N, size_t C, size_t H, size_t W, const float *dpooled, const float *y,
                           const float *x, const float *scale, float *packed, float *dx_sum);
+/* Every form of the batch-norm gradient above in one entry point, plus a sum that rides along.  The tensor is
+   [N, C, H, W] (H * W = inner).  Exactly one of dy, dy_open and dpooled says where the incoming gradient is:
+   dy as in dopt_hip_bn_grad_fused; dy_open / keep_dy as in dopt_hip_bn_grad_open; dpooled as in
+   dopt_hip_bn_grad_pool (y is required then), and when dpooled_open is given as well, dpooled is its value and
+   still lies in partial copies, which the kernel adds as it routes them (keep_dy as for dy_open).
+   side (may be null, or complete: splits == 0) is a sum that has nothing to do with the batch norm: an open
+   filter gradient left by dopt_hip_conv_bwd_pair_packed_open.  Where a register-resident batch-norm kernel runs,
+   extra workgroups of the same launch add its copies (bit for bit what dopt_hip_split_sum_close writes); both
+   are short bandwidth-bound passes, and one launch costs less than two.  Elsewhere it is closed first by a launch
+   of its own.  No counterpart in the reference. */
+int dopt_hip_bn_grad_side(size_t N, size_t C, size_t H, size_t W, const float *dy, const dopt_hip_split_sum *dy_open,
+                          int keep_dy, const float *dpooled, const dopt_hip_split_sum *dpooled_open, const float *y,
+                          const float *x, const float *scale, float *packed, float *dx_sum,
+                          const dopt_hip_split_sum *side);
 /* Channels of more than 32768 values are normalised by a few workgroups each, which meet once inside the
    kernel; a workgroup polls for its partners at most `polls` times (about a microsecond each; default
    2^21) and then gives up: the kernel still ends, and the next dopt_hip_sync or dopt_hip_copy_d2h

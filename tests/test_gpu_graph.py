@@ -437,11 +437,12 @@ def test_backward_data_and_filter_gradient_as_one_call(xs, k):
     capi.check(lib.dopt_hip_conv_bwd_data_packed(C.byref(d), dy.ptr, packed.ptr, dx_want.ptr))
     capi.check(lib.dopt_hip_conv_bwd_filter(C.byref(d), dy.ptr, x.ptr, dw_want.ptr))
     dx_want, dw_want = dx_want.numpy(), dw_want.numpy()
+    dw_scratch = ops.Tensor((k, Cin, 3, 3))
     # closed
     dx, dw = ops.Tensor(xs), ops.Tensor((k, Cin, 3, 3))
     dx.set(np.full(xs, np.nan, np.float32)); dw.set(np.full((k, Cin, 3, 3), np.nan, np.float32))
     capi.check(lib.dopt_hip_conv_pair_probe(1))
-    capi.check(lib.dopt_hip_conv_bwd_pair_packed_open(C.byref(d), dy.ptr, packed.ptr, x.ptr, dx.ptr, dw.ptr, None))
+    capi.check(lib.dopt_hip_conv_bwd_pair_packed_open(C.byref(d), dy.ptr, packed.ptr, x.ptr, dx.ptr, dw.ptr, None, None))
     n, us, fl, by = C.c_int(), C.c_double(), C.c_double(), C.c_double()
     capi.check(lib.dopt_hip_conv_pair_probe_read(C.byref(n), C.byref(us), C.byref(fl), C.byref(by)))
     capi.check(lib.dopt_hip_conv_pair_probe(0))
@@ -455,10 +456,26 @@ def test_backward_data_and_filter_gradient_as_one_call(xs, k):
     # open, closed by dopt_hip_split_sum_close
     dx.set(np.full(xs, np.nan, np.float32)); dw.set(np.full((k, Cin, 3, 3), np.nan, np.float32))
     o = capi.SplitSum()
-    capi.check(lib.dopt_hip_conv_bwd_pair_packed_open(C.byref(d), dy.ptr, packed.ptr, x.ptr, dx.ptr, dw.ptr, C.byref(o)))
+    capi.check(lib.dopt_hip_conv_bwd_pair_packed_open(C.byref(d), dy.ptr, packed.ptr, x.ptr, dx.ptr, dw.ptr, C.byref(o), None))
     assert o.value == dx.ptr
     if xs == (8, 256, 4, 4):
         assert o.splits > 1
+    if o.splits:
+        capi.check(lib.dopt_hip_split_sum_close(C.byref(o)))
+    assert np.array_equal(dx.numpy(), dx_want) and np.array_equal(dw.numpy(), dw_want)
+    # both left open, both closed by dopt_hip_split_sum_close (the filter gradient first: either order is allowed)
+    dx.set(np.full(xs, np.nan, np.float32)); dw.set(np.full((k, Cin, 3, 3), np.nan, np.float32))
+    o, ow = capi.SplitSum(), capi.SplitSum()
+    capi.check(lib.dopt_hip_conv_bwd_pair_packed_open(C.byref(d), dy.ptr, packed.ptr, x.ptr, dx.ptr, dw.ptr, C.byref(o), C.byref(ow)))
+    assert ow.value == dw.ptr and (ow.splits == 0 or (one_launch and ow.splits > 1 and ow.lanes in (4, 16)))
+    if xs == (128, 128, 16, 16):
+        assert ow.splits > 1
+    if ow.splits:
+        # nothing else may take the workspace while the copies lie in it
+        assert lib.dopt_hip_conv_bwd_filter(C.byref(d), dy.ptr, x.ptr, dw_scratch.ptr) != 0
+        assert b"was not closed" in lib.dopt_hip_last_error()
+        # ... and that refusal drops the library's note of them: the copies themselves are still there
+        capi.check(lib.dopt_hip_split_sum_close(C.byref(ow)))
     if o.splits:
         capi.check(lib.dopt_hip_split_sum_close(C.byref(o)))
     assert np.array_equal(dx.numpy(), dx_want) and np.array_equal(dw.numpy(), dw_want)
@@ -472,10 +489,98 @@ def test_backward_data_and_filter_gradient_as_one_call(xs, k):
     g_got, db_got = ops.Tensor([int(np.prod(xs)) + 2 * Cin]), ops.Tensor([Cin])
     dw.set(np.full((k, Cin, 3, 3), np.nan, np.float32))
     o = capi.SplitSum()
-    capi.check(lib.dopt_hip_conv_bwd_pair_packed_open(C.byref(d), dy.ptr, packed.ptr, x.ptr, dx.ptr, dw.ptr, C.byref(o)))
+    capi.check(lib.dopt_hip_conv_bwd_pair_packed_open(C.byref(d), dy.ptr, packed.ptr, x.ptr, dx.ptr, dw.ptr, C.byref(o), None))
     capi.check(lib.dopt_hip_bn_grad_open(N, Cin, inner, C.byref(o), 1, yrelu.ptr, xin.ptr, sc.ptr, g_got.ptr, db_got.ptr))
     assert np.array_equal(g_got.numpy(), g_want.numpy()) and np.array_equal(db_got.numpy(), db_want.numpy())
     assert np.array_equal(dx.numpy(), dx_want) and np.array_equal(dw.numpy(), dw_want)
+    # both open, both closed by ONE batch-norm gradient launch: dx as it is loaded, dw by workgroups that ride along
+    g_got.set(np.full(g_got.shape, np.nan, np.float32))
+    dx.set(np.full(xs, np.nan, np.float32)); dw.set(np.full((k, Cin, 3, 3), np.nan, np.float32))
+    o, ow = capi.SplitSum(), capi.SplitSum()
+    capi.check(lib.dopt_hip_conv_bwd_pair_packed_open(C.byref(d), dy.ptr, packed.ptr, x.ptr, dx.ptr, dw.ptr, C.byref(o), C.byref(ow)))
+    capi.check(lib.dopt_hip_bn_grad_side(N, Cin, H, W, None, C.byref(o), 1, None, None, yrelu.ptr, xin.ptr, sc.ptr, g_got.ptr,
+                                         db_got.ptr, C.byref(ow)))
+    assert np.array_equal(g_got.numpy(), g_want.numpy()) and np.array_equal(db_got.numpy(), db_want.numpy())
+    assert np.array_equal(dx.numpy(), dx_want) and np.array_equal(dw.numpy(), dw_want)
+    # the workspace is free again
+    capi.check(lib.dopt_hip_conv_bwd_filter(C.byref(d), dy.ptr, x.ptr, dw_scratch.ptr))
+    ops.sync()
+
+
+@pytest.mark.parametrize("lanes,splits,n4", [(4, 16, 36864), (16, 37, 1000), (4, 3, 70000)])
+@pytest.mark.parametrize("shape,form", [
+    ((16, 32, 8, 8), "dy"),            # one workgroup per channel, two quads per lane
+    ((128, 16, 16, 16), "dy"),         # eight quads per lane
+    ((128, 8, 32, 32), "dy"),          # channels shared by clusters of workgroups
+    ((16, 32, 8, 8), "dy_open"),       # dy still in partial copies
+    ((16, 32, 8, 8), "pool"),          # dy routed from the gradient of a 2 x 2 max-pool
+    ((16, 32, 8, 8), "pool_open"),     # ... which still lies in partial copies
+    ((64, 24, 2, 2), "pool_open"),     # 2 x 2 images: a quad is a window
+    ((128, 8, 32, 32), "pool_open"),   # in the cluster kernel
+    ((16, 12, 8, 12), "pool_open"),    # rows of three quads: pooled by a pass of its own, copies added first
+    ((4, 6, 5, 5), "dy"),              # not a register-resident shape: the side sum gets a launch of its own
+])
+def test_batch_norm_gradient_with_a_sum_riding_along(shape, form, lanes, splits, n4):
+    """dopt_hip_bn_grad_side against the separate entry points: the gradient is what dopt_hip_bn_grad_fused /
+    dopt_hip_bn_grad_pool give on the finished operands, the side sum what dopt_hip_split_sum_close gives, all to the
+    last bit, whichever kernel the shape selects."""
+    import ctypes as C
+    from dopt_amd import capi
+    lib = capi.load()
+    r = np.random.default_rng(n4 + shape[1])
+    N, Cc, H, W = shape
+    x = ops.tensor(r.standard_normal(shape).astype(np.float32))
+    y = ops.tensor(np.maximum(r.standard_normal(shape), 0).astype(np.float32))
+    sc = ops.tensor(r.uniform(0.5, 1.5, Cc).astype(np.float32))
+    total = int(np.prod(shape))
+
+    def open_sum(value_shape, S):
+        part = ops.tensor(r.standard_normal((S,) + value_shape).astype(np.float32))
+        value = ops.Tensor(value_shape)
+        o = capi.SplitSum(part.ptr, S, int(np.prod(value_shape)), value_shape[1], int(np.prod(value_shape[2:])), None, value.ptr, 0)
+        return part, value, o
+
+    # the side sum and what closing it gives
+    side_part = ops.tensor(r.standard_normal((splits, n4 * 4)).astype(np.float32))
+    side_want, side_got = ops.Tensor([n4 * 4]), ops.Tensor([n4 * 4])
+    capi.check(lib.dopt_hip_split_sum_close(C.byref(capi.SplitSum(side_part.ptr, splits, n4 * 4, 0, 0, None, side_want.ptr, lanes))))
+    side = capi.SplitSum(side_part.ptr, splits, n4 * 4, 0, 0, None, side_got.ptr, lanes)
+    side_got.set(np.full(n4 * 4, np.nan, np.float32))
+
+    want, dbw = ops.Tensor([total + 2 * Cc]), ops.Tensor([Cc])
+    got, dbg = ops.Tensor([total + 2 * Cc]), ops.Tensor([Cc])
+    got.set(np.full(total + 2 * Cc, np.nan, np.float32))
+    if form == "dy":
+        dy = ops.tensor(r.standard_normal(shape).astype(np.float32))
+        capi.check(lib.dopt_hip_bn_grad_fused(N, Cc, H * W, dy.ptr, y.ptr, x.ptr, sc.ptr, want.ptr, dbw.ptr))
+        capi.check(lib.dopt_hip_bn_grad_side(N, Cc, H, W, dy.ptr, None, 1, None, None, y.ptr, x.ptr, sc.ptr, got.ptr, dbg.ptr,
+                                             C.byref(side)))
+    elif form == "dy_open":
+        part, dy, o = open_sum(shape, 3)
+        capi.check(lib.dopt_hip_split_sum_close(C.byref(o)))
+        closed = dy.numpy()
+        capi.check(lib.dopt_hip_bn_grad_fused(N, Cc, H * W, dy.ptr, y.ptr, x.ptr, sc.ptr, want.ptr, dbw.ptr))
+        dy.set(np.full(shape, np.nan, np.float32))
+        capi.check(lib.dopt_hip_bn_grad_side(N, Cc, H, W, None, C.byref(o), 1, None, None, y.ptr, x.ptr, sc.ptr, got.ptr, dbg.ptr,
+                                             C.byref(side)))
+        assert np.array_equal(dy.numpy(), closed)
+    else:
+        pshape = (N, Cc, H // 2, W // 2)
+        if form == "pool":
+            dp = ops.tensor(r.standard_normal(pshape).astype(np.float32))
+            o = None
+        else:
+            part, dp, o = open_sum(pshape, 4)
+            capi.check(lib.dopt_hip_split_sum_close(C.byref(o)))
+        closed = dp.numpy()
+        capi.check(lib.dopt_hip_bn_grad_pool(N, Cc, H, W, dp.ptr, y.ptr, x.ptr, sc.ptr, want.ptr, dbw.ptr))
+        if o is not None:
+            dp.set(np.full(pshape, np.nan, np.float32))
+        capi.check(lib.dopt_hip_bn_grad_side(N, Cc, H, W, None, None, 1, dp.ptr, C.byref(o) if o is not None else None, y.ptr,
+                                             x.ptr, sc.ptr, got.ptr, dbg.ptr, C.byref(side)))
+        assert np.array_equal(dp.numpy(), closed)
+    assert np.array_equal(got.numpy(), want.numpy()) and np.array_equal(dbg.numpy(), dbw.numpy())
+    assert np.array_equal(side_got.numpy(), side_want.numpy())
     ops.sync()
 
 
