@@ -508,15 +508,25 @@ __device__ __forceinline__ void open_add(const OpenSum &open, const unsigned (&a
                 sum[i] = make_float4(sum[i].x + v[sp][i].x, sum[i].y + v[sp][i].y, sum[i].z + v[sp][i].z, sum[i].w + v[sp][i].w);
         }
     } else {
-        for (int sp = 0; sp < open.splits; sp++) {
-            const float4 *src = open.partial + (size_t)sp * open.stride4;
-            float4 v[kQ];
+        // rounds of eight copies in flight (indices clamped to the last copy, surplus values dropped); the adds stay
+        // in ascending copy order
+        const int last = open.splits - 1;
+        for (int sp = 0; sp <= last; sp += 8) {
+            float4 v[8][kQ];
 #pragma unroll
-            for (int i = 0; i < kQ; i++) v[i] = src[at[i]];
+            for (int u = 0; u < 8; u++) {
+                const float4 *src = open.partial + (size_t)min(sp + u, last) * open.stride4;
 #pragma unroll
-            for (int i = 0; i < kQ; i++) {
-                if (sp == 0) sum[i] = v[i];
-                else sum[i] = make_float4(sum[i].x + v[i].x, sum[i].y + v[i].y, sum[i].z + v[i].z, sum[i].w + v[i].w);
+                for (int i = 0; i < kQ; i++) v[u][i] = src[at[i]];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                if (sp + u > last) break;
+#pragma unroll
+                for (int i = 0; i < kQ; i++) {
+                    if (sp + u == 0) sum[i] = v[u][i];
+                    else sum[i] = make_float4(sum[i].x + v[u][i].x, sum[i].y + v[u][i].y, sum[i].z + v[u][i].z, sum[i].w + v[u][i].w);
+                }
             }
         }
     }

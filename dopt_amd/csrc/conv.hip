@@ -1434,6 +1434,191 @@ int run_dense2x2(const dopt_hip_conv_desc *d, const float *in, const float *w, c
     return rc;
 }
 
+// ---- 2 x 2 images, straight from the filter ----------------------------------------------------
+// The product above needs the 16 MB matrix made first, and its 32 x 32-output blocks read their operands
+// with a handful of loads in flight per wavefront (one cache line per lane and step), which is what
+// bounds them.  This kernel keeps that decomposition - a block owns 32 images x 8 output channels x 4
+// pixels over the WHOLE reduction, so nothing is split and no partial copies are left for a reader
+// (whose 16-byte pieces per image and channel would be re-read once per copy) - but reads the taps from
+// the filter as it lies (no Wd) and streams both operands through LDS in bulk:
+//   * the eight wavefronts split the reduction channels (64 consecutive channels each, R % 64 == 0) and
+//     never share data, so each runs a pipeline of its own with no workgroup barrier: per step of 8
+//     channels it loads 32 images x 128 bytes of the batch (whole cache lines) and 8 runs of 8 x 9 taps,
+//     three steps ahead, passes them through a wavefront-private LDS tile and multiplies;
+//   * a batch row is read back as one 128-bit LDS read per eight reduction steps (lane half h takes
+//     steps 8g + 4h .. 8g + 4h + 3 on both operands), the four taps a lane needs per (channel, pixel
+//     pair) as four 4-byte reads: tap = {4,3,1,0}[input pixel] + {0,1,3,4}[output pixel] (see Wd above);
+//   * the eight partial 32 x 32 tiles are added through LDS in wavefront order (+ bias).
+// Forward (kBwd = false): in = x [N][C*4], columns (k, output pixel), a filter run = one output channel's
+// 8 reduction channels x 9 taps; backward-data: in = dy [N][K*4], columns (c, input pixel), a run = one
+// reduction channel k, its 8 output channels c x 9 taps.
+struct Direct2x2 {
+    const float *in;    // [N][R*4]
+    const float *w;     // [K][C][3][3]
+    const float *bias;  // [O] or null (forward)
+    float *out;         // [N][O*4]
+    int N, R, O, C;     // images, reduction channels, output channels, the filter's input channels (its pitch is C*9)
+};
+
+constexpr int kD2Rows = 32, kD2Chans = 8, kD2Step = 8, kD2Waves = 8, kD2Depth = 3;
+constexpr int kD2APitch = kD2Step * 4 + 4;   // 36 floats: 128-bit reads of 32 rows touch every bank once
+constexpr int kD2WPitch = kD2Step * 9 + 5;   // 77 floats per run of 8 x 9 taps
+constexpr int kD2WaveLds = 2 * (kD2Rows * kD2APitch + 8 * kD2WPitch);   // floats per wavefront, double buffered
+constexpr size_t kD2Lds = (size_t)kD2Waves * kD2WaveLds * sizeof(float);
+static_assert(kD2Waves * kD2WaveLds >= kD2Waves * 32 * 33, "the partial tiles reuse the staging area");
+
+template <bool kBwd>
+__global__ __launch_bounds__(64 * kD2Waves) void conv2x2_direct_k(Direct2x2 p)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, l32 = lane & 31, kh = lane >> 5;
+    const int o0 = blockIdx.x * kD2Chans, n0 = blockIdx.y * kD2Rows;
+    const int per_wave = p.R / kD2Waves, steps = per_wave / kD2Step, c_first = w * per_wave;
+    float *const mine = lds + w * kD2WaveLds;
+
+    // this lane's pieces of a step: 4 quads of the batch (row = idx / 8, quad idx % 8) and up to 3 of the taps
+    // (run = idx / 18, quad idx % 18)
+    const float *a_src[4];
+    bool a_ok[4];
+    int a_dst[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int idx = lane + 64 * i, row = idx >> 3, q = idx & 7;
+        a_ok[i] = n0 + row < p.N;
+        a_src[i] = p.in + ((size_t)(a_ok[i] ? n0 + row : 0) * p.R + c_first) * 4 + 4 * q;
+        a_dst[i] = row * kD2APitch + 4 * q;
+    }
+    const float *w_src[3];
+    bool w_ok[3];
+    int w_dst[3];
+#pragma unroll
+    for (int i = 0; i < 3; i++) {
+        const int idx = lane + 64 * i, run = min(idx / 18, 7), q = idx - (idx / 18) * 18;
+        w_ok[i] = idx < 8 * 18;
+        // forward: run = output channel, its 8 reduction channels of the step; backward: run = reduction channel of the
+        // step, the block's 8 output channels
+        w_src[i] = kBwd ? p.w + ((size_t)(c_first + run) * p.C + o0) * 9 + 4 * q : p.w + ((size_t)(o0 + run) * p.C + c_first) * 9 + 4 * q;
+        w_dst[i] = run * kD2WPitch + 4 * q;
+    }
+    const size_t w_step = kBwd ? (size_t)kD2Step * p.C * 9 : (size_t)kD2Step * 9;   // floats between steps
+    float4 ra[kD2Depth][4], rw[kD2Depth][3];
+    auto load = [&](int slot, int s) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            ra[slot][i] = a_ok[i] ? *(const float4 *)(a_src[i] + (size_t)s * kD2Step * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int i = 0; i < 3; i++)
+            rw[slot][i] = w_ok[i] ? *(const float4 *)(w_src[i] + (size_t)s * w_step) : make_float4(0.f, 0.f, 0.f, 0.f);
+    };
+    auto store = [&](int slot, float *buf) {
+        float *As = buf, *Ws = buf + kD2Rows * kD2APitch;
+#pragma unroll
+        for (int i = 0; i < 4; i++) *(float4 *)&As[a_dst[i]] = ra[slot][i];
+#pragma unroll
+        for (int i = 0; i < 3; i++)
+            if (w_ok[i]) {
+                float *dst = &Ws[w_dst[i]];
+                dst[0] = rw[slot][i].x; dst[1] = rw[slot][i].y; dst[2] = rw[slot][i].z; dst[3] = rw[slot][i].w;
+            }
+    };
+
+    const int pix = l32 & 3, oc = l32 >> 2;   // the column: output channel inside the block, and its pixel
+    const int lane_tap = kBwd ? (pix == 0 ? 4 : pix == 1 ? 3 : pix == 2 ? 1 : 0) : (pix == 0 ? 0 : pix == 1 ? 1 : pix == 2 ? 3 : 4);
+    const int a_frag = l32 * kD2APitch + 4 * kh;
+    const int b_frag = kD2Rows * kD2APitch + (kBwd ? kh * kD2WPitch + oc * 9 + lane_tap : oc * kD2WPitch + kh * 9 + lane_tap);
+    // two accumulators (even and odd channel pairs), so that consecutive matrix instructions do not wait for each other
+    v16f acc0, acc1;
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc0[v] = acc1[v] = 0.0f;
+
+#pragma unroll
+    for (int d = 0; d < kD2Depth; d++)
+        if (d < steps) load(d, d);
+    // steps in groups of kD2Depth so that the register slots are compile-time indices
+    for (int s0 = 0; s0 < steps; s0 += kD2Depth) {
+#pragma unroll
+        for (int d = 0; d < kD2Depth; d++) {
+            const int s = s0 + d;
+            if (s < steps) {
+                float *buf = mine + (s & 1) * (kD2WaveLds / 2);
+                store(d, buf);
+                __builtin_amdgcn_wave_barrier();   // the tile is read by other lanes of this wavefront: keep the order
+                if (s + kD2Depth < steps) load(d, s + kD2Depth);
+#pragma unroll
+                for (int g = 0; g < 4; g++) {   // reduction steps 8g .. 8g + 7 of the tile: channels 2g (lane half 0), 2g + 1
+                    const float4 a = *(const float4 *)(buf + a_frag + 8 * g);
+                    const float *src = buf + b_frag + (kBwd ? 2 * g * kD2WPitch : 2 * g * 9);
+                    float b0, b1, b2, b3;
+                    if (kBwd) { b0 = src[0]; b1 = src[1]; b2 = src[3]; b3 = src[4]; }
+                    else { b0 = src[4]; b1 = src[3]; b2 = src[1]; b3 = src[0]; }
+                    if (g & 1) {
+                        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b0, acc1, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b1, acc1, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b2, acc1, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b3, acc1, 0, 0, 0);
+                    } else {
+                        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b0, acc0, 0, 0, 0);
+                        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b1, acc0, 0, 0, 0);
+                        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b2, acc0, 0, 0, 0);
+                        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b3, acc0, 0, 0, 0);
+                    }
+                }
+            }
+        }
+    }
+
+    // ---- the eight partial tiles, added in wavefront order
+    __syncthreads();   // every wavefront is done with its staging tiles
+    float *red = lds;  // [8][32 * 33]
+#pragma unroll
+    for (int v = 0; v < 16; v++) red[w * (32 * 33) + acc_row(v, lane) * 33 + l32] = acc0[v] + acc1[v];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int idx = tid + i * 64 * kD2Waves, rr = idx >> 5, cc = idx & 31;
+        float sum = red[rr * 33 + cc];
+#pragma unroll
+        for (int k = 1; k < kD2Waves; k++) sum += red[k * (32 * 33) + rr * 33 + cc];
+        if (p.bias) sum += p.bias[o0 + (cc >> 2)];
+        if (n0 + rr < p.N) p.out[(size_t)(n0 + rr) * p.O * 4 + o0 * 4 + cc] = sum;
+    }
+}
+
+bool direct2x2_takes(const dopt_hip_conv_desc *d)
+{
+    return dense2x2_takes(d) && d->C % 64 == 0 && d->K % 64 == 0 && d->N * d->C * 4 < ((size_t)1 << 31) &&
+           d->N * d->K * 4 < ((size_t)1 << 31) && d->K * d->C * 9 < ((size_t)1 << 31) && ceil_div(d->N, (size_t)kD2Rows) < 65536;
+}
+
+// *done = false: not this kernel's shape (or operands it cannot read as quads).
+template <bool kBwd>
+int run_direct2x2(const dopt_hip_conv_desc *d, const float *in, const float *w, const float *bias, float *out, bool *done)
+{
+    *done = false;
+    if (!direct2x2_takes(d) || !aligned16(in) || !aligned16(w) || !aligned16(out)) return DOPT_HIP_OK;
+    Direct2x2 p{};
+    p.in = in;
+    p.w = w;
+    p.bias = bias;
+    p.out = out;
+    p.N = (int)d->N;
+    p.R = (int)(kBwd ? d->K : d->C);
+    p.O = (int)(kBwd ? d->C : d->K);
+    p.C = (int)d->C;
+    static bool raised[2] = {false, false};
+    if (!raised[kBwd]) {
+        DOPT_HIP_CHECK(hipFuncSetAttribute((const void *)conv2x2_direct_k<kBwd>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)kD2Lds));
+        raised[kBwd] = true;
+    }
+    // column tiles fastest: the blocks an XCD receives share an eighth of the filter and all of the batch
+    const dim3 grid((unsigned)(p.O / kD2Chans), (unsigned)ceil_div(d->N, (size_t)kD2Rows));
+    hipLaunchKernelGGL(conv2x2_direct_k<kBwd>, grid, dim3(64 * kD2Waves), kD2Lds, stream(), p);
+    DOPT_LAUNCH_CHECK();
+    *done = true;
+    return DOPT_HIP_OK;
+}
+
 // Filter gradient of the same layers: dWd = x^T * dy, [4C, N] x [N, 4K], is the gradient of the matrix
 // above; every filter tap collects the (input pixel, output pixel) pairs that read it - one pair for
 // a corner tap, two for an edge tap, four for the centre - in a fixed order.
@@ -1646,7 +1831,12 @@ int run_gather(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in,
         if (int rc = conv_smallc_fwd(d, in, w, bias, out, &done)) return rc;
         if (done) return DOPT_HIP_OK;
     }
-    if (dense2x2_takes(d)) return run_dense2x2<kBwd>(d, in, w, nullptr, bias, out);
+    if (dense2x2_takes(d)) {
+        bool done = false;
+        if (int rc = run_direct2x2<kBwd>(d, in, w, bias, out, &done)) return rc;
+        if (done) return DOPT_HIP_OK;
+        return run_dense2x2<kBwd>(d, in, w, nullptr, bias, out);
+    }
     {
         bool done = false;
         if (int rc = run_patch<kBwd>(d, P, Q, in, w, bias, out, &done)) return rc;
@@ -1992,6 +2182,7 @@ size_t dopt_hip_conv_packed_bytes(const dopt_hip_conv_desc *d, int bwd_data)
     size_t P, Q;
     if (check_desc(d, &P, &Q, "dopt_hip_conv_packed_bytes") || !ensure_init()) return 0;
     if (!bwd_data && conv_smallc_takes(d)) return 0;   // that forward kernel reads the filter as it is
+    if (direct2x2_takes(d)) return d->K * d->C * 9 * sizeof(float);   // the filter as it is
     if (dense2x2_takes(d)) return dense2x2_elems(d) * sizeof(float);
     const PatchSetup u = bwd_data ? patch_setup<true>(d, P, Q) : patch_setup<false>(d, P, Q);
     // PackJob keeps strides in 32 bits
@@ -2001,6 +2192,7 @@ size_t dopt_hip_conv_packed_bytes(const dopt_hip_conv_desc *d, int bwd_data)
 int dopt_hip_conv_packed_layout(const dopt_hip_conv_desc *d, int bwd_data)
 {
     if (dopt_hip_conv_packed_bytes(d, bwd_data) == 0) return -1;
+    if (direct2x2_takes(d)) return 3;  // the filter itself: such kernels read [K][C][3][3], and a caller may pass the filter
     if (dense2x2_takes(d)) return 2;   // the same matrix, read transposed by backward-data
     return bwd_data ? 1 : 0;
 }
@@ -2025,6 +2217,12 @@ int dopt_hip_conv_pack_batch(int n, const dopt_hip_conv_desc *descs, const int *
         size_t P, Q;
         if (int rc = check_desc(&descs[i], &P, &Q, "dopt_hip_conv_pack_batch")) return rc;
         DOPT_REQUIRE(w[i] && packed[i] && aligned16(packed[i]), "dopt_hip_conv_pack_batch: filter %d: null or unaligned pointer", i);
+        if (direct2x2_takes(&descs[i])) {   // "packed" is a plain copy (callers that know pass the filter itself instead)
+            if (int rc = flush()) return rc;
+            if (packed[i] != w[i])
+                if (int rc = dopt_hip_copy_d2d(packed[i], w[i], descs[i].K * descs[i].C * 9 * sizeof(float))) return rc;
+            continue;
+        }
         if (dense2x2_takes(&descs[i]) && !(!bwd_data[i] && conv_smallc_takes(&descs[i]))) {
             if (int rc = dense2x2_pack(&descs[i], w[i], packed[i])) return rc;   // a launch of its own: the matrix is large
             continue;
@@ -2053,6 +2251,12 @@ int dopt_hip_conv_fwd_bias_packed_open(const dopt_hip_conv_desc *d, const float 
     if (int rc = check_desc(d, &P, &Q, "dopt_hip_conv_fwd_bias_packed")) return rc;
     DOPT_REQUIRE(x && packed && y, "dopt_hip_conv_fwd_bias_packed: null argument");
     DOPT_ENSURE_INIT();
+    if (dopt_hip_conv_packed_layout(d, 0) == 3) {
+        bool done = false;
+        if (int rc = run_direct2x2<false>(d, x, packed, bias, y, &done)) return rc;
+        if (done) return DOPT_HIP_OK;
+        return run_dense2x2<false>(d, x, packed, nullptr, bias, y);   // operands it cannot read as quads: from the filter
+    }
     if (dopt_hip_conv_packed_layout(d, 0) == 2) return run_dense2x2<false>(d, x, nullptr, packed, bias, y);
     bool done = false;
     if (int rc = run_patch<false>(d, P, Q, x, nullptr, bias, y, &done, packed, open)) return rc;
@@ -2077,6 +2281,12 @@ int dopt_hip_conv_bwd_data_packed_open(const dopt_hip_conv_desc *d, const float 
     if (int rc = check_desc(d, &P, &Q, "dopt_hip_conv_bwd_data_packed")) return rc;
     DOPT_REQUIRE(dy && packed && dx, "dopt_hip_conv_bwd_data_packed: null argument");
     DOPT_ENSURE_INIT();
+    if (dopt_hip_conv_packed_layout(d, 1) == 3) {
+        bool done = false;
+        if (int rc = run_direct2x2<true>(d, dy, packed, nullptr, dx, &done)) return rc;
+        if (done) return DOPT_HIP_OK;
+        return run_dense2x2<true>(d, dy, packed, nullptr, nullptr, dx);
+    }
     if (dopt_hip_conv_packed_layout(d, 1) == 2) return run_dense2x2<true>(d, dy, nullptr, packed, nullptr, dx);
     bool done = false;
     if (int rc = run_patch<true>(d, P, Q, dy, nullptr, nullptr, dx, &done, packed, open)) return rc;

@@ -605,7 +605,7 @@ struct HIPPlan::Builder {
     struct MatmulInfo { bool valid = false; int a = -1, b = -1, tA = 0, tB = 0; size_t M = 0, N = 0, K = 0; };
     std::vector<MatmulInfo> mmInfo;
     // steps that run a convolution on a packed filter (candidates for leaving their result open)
-    struct ConvStep { size_t step; int op; int bwd; bool bias; dopt_hip_conv_desc d; const float *packed; };
+    struct ConvStep { size_t step; int op; int bwd; bool bias; dopt_hip_conv_desc d; const float *packed; int filterIn; };
     std::vector<ConvStep> convSteps;
 
     Builder(const Graph &graph, HIPPlan *plan, const std::vector<int> &outs, unsigned f)
@@ -1138,6 +1138,8 @@ int HIPPlan::Builder::prepackFilters()
                 if (other.owner && other.filter == k.filter && memcmp(&other.d, &k.d, sizeof(k.d)) == 0 &&
                     dopt_hip_conv_packed_layout(&other.d, other.bwd) == layout)
                     k.buf = other.buf;
+            if (layout == 3) k.buf = g.ops[k.filter].value;   // such kernels read the filter as it lies: nothing to pack (the
+                                                              // step reads the filter operand of each run, see buildSteps)
             k.owner = k.buf == nullptr;
             k.late = layout == 2;
             if (k.owner) {
@@ -1284,7 +1286,10 @@ int HIPPlan::Builder::buildSteps()
             const float *packed = (const float *)pk.buf;
             const dopt_hip_conv_desc d = pk.d;
             onPacked = true;
-            convSteps.push_back({0, id, pk.bwd, !pk.bwd && fusedKind[id] == 1, d, packed});
+            // layout 3: the kernel reads the filter itself, which is then one more input of the step (its last)
+            const bool asIs = dopt_hip_conv_packed_layout(&d, pk.bwd) == 3;
+            const int fi = !asIs ? -1 : pk.bwd ? 1 : fusedKind[id] == 1 ? 2 : 1;
+            convSteps.push_back({0, id, pk.bwd, !pk.bwd && fusedKind[id] == 1, d, packed, fi});
             if (pk.bwd && pairOf[id] >= 0) {
                 stepInputs = {op.deps[0], g.ops[pairOf[id]].deps[1]};
                 float *dw = (float *)p->mResults[pairOf[id]];
@@ -1295,19 +1300,25 @@ int HIPPlan::Builder::buildSteps()
                 label = "convolutionFeaturesGrad+convolutionFiltersGrad";
             } else if (pk.bwd) {
                 stepInputs = {op.deps[0]};
+                if (asIs) stepInputs.push_back(pk.filter);
                 k = make([=](const std::vector<const void *> &in, void *out) {
-                    return dopt_hip_conv_bwd_data_packed(&d, (const float *)in[0], packed, (float *)out);
+                    return dopt_hip_conv_bwd_data_packed(&d, (const float *)in[0], fi >= 0 ? (const float *)in[fi] : packed,
+                                                         (float *)out);
                 });
             } else if (fusedKind[id] == 1) {
                 stepInputs = {inputsOf[id][0], inputsOf[id][2]};
+                if (asIs) stepInputs.push_back(pk.filter);
                 k = make([=](const std::vector<const void *> &in, void *out) {
-                    return dopt_hip_conv_fwd_bias_packed(&d, (const float *)in[0], packed, (const float *)in[1], (float *)out);
+                    return dopt_hip_conv_fwd_bias_packed(&d, (const float *)in[0], fi >= 0 ? (const float *)in[fi] : packed,
+                                                         (const float *)in[1], (float *)out);
                 });
                 label = "convolution+addBias";
             } else {
                 stepInputs = {op.deps[0]};
+                if (asIs) stepInputs.push_back(pk.filter);
                 k = make([=](const std::vector<const void *> &in, void *out) {
-                    return dopt_hip_conv_fwd_bias_packed(&d, (const float *)in[0], packed, nullptr, (float *)out);
+                    return dopt_hip_conv_fwd_bias_packed(&d, (const float *)in[0], fi >= 0 ? (const float *)in[fi] : packed,
+                                                         nullptr, (float *)out);
                 });
             }
         } else if (prebuilt[id]) {
@@ -1368,6 +1379,7 @@ void HIPPlan::Builder::openSplitSums()
         auto open = std::make_shared<dopt_hip_split_sum>();
         const dopt_hip_conv_desc d = cs.d;
         const float *packed = cs.packed;
+        const int fi = cs.filterIn;   // >= 0: the kernel reads the filter operand itself
         size_t N, C, inner;
         if (!cs.bwd && bo.opType == "batchNormTrain" && bo.deps.size() == 5 && next.inputOps.size() == 5 &&
             (fusedKind[b] == 0 || fusedKind[b] == 2)) {
@@ -1378,8 +1390,8 @@ void HIPPlan::Builder::openSplitSums()
             nci(g.ops[bo.deps[0]].shape, &N, &C, &inner);
             const bool bias = cs.bias;
             conv.kernel = make([=](const std::vector<const void *> &in, void *out) {
-                return dopt_hip_conv_fwd_bias_packed_open(&d, (const float *)in[0], packed, bias ? (const float *)in[1] : nullptr,
-                                                          (float *)out, open.get());
+                return dopt_hip_conv_fwd_bias_packed_open(&d, (const float *)in[0], fi >= 0 ? (const float *)in[fi] : packed,
+                                                          bias ? (const float *)in[1] : nullptr, (float *)out, open.get());
             });
             if (poolOf[b] >= 0 && needed[poolOf[b]]) {
                 std::string unused;
@@ -1414,7 +1426,8 @@ void HIPPlan::Builder::openSplitSums()
                 });
             } else {
                 conv.kernel = make([=](const std::vector<const void *> &in, void *out) {
-                    return dopt_hip_conv_bwd_data_packed_open(&d, (const float *)in[0], packed, (float *)out, open.get());
+                    return dopt_hip_conv_bwd_data_packed_open(&d, (const float *)in[0], fi >= 0 ? (const float *)in[fi] : packed,
+                                                              (float *)out, open.get());
                 });
             }
             next.kernel = make([=](const std::vector<const void *> &in, void *out) {

@@ -211,7 +211,10 @@ int dopt_hip_conv_bwd_data(const dopt_hip_conv_desc *d, const float *dy, const f
    device, and is valid until the filter changes. */
 size_t dopt_hip_conv_packed_bytes(const dopt_hip_conv_desc *d, int bwd_data);
 /* Which layout that packed copy has, or -1 when there is none: two packed copies of the same filter
-   under the same descriptor and with equal layout ids are identical, so a caller needs only one. */
+   under the same descriptor and with equal layout ids are identical, so a caller needs only one.
+   Layout 3 is the filter itself, [K, C, R, S]: the kernel reads it as it lies, dopt_hip_conv_pack_batch
+   makes a plain copy, and a caller may skip that and pass the filter as `packed` (it must be 16-byte
+   aligned). */
 int dopt_hip_conv_packed_layout(const dopt_hip_conv_desc *d, int bwd_data);
 int dopt_hip_conv_pack_batch(int n, const dopt_hip_conv_desc *descs, const int *bwd_data,
                              const float *const *w, float *const *packed /* 16-byte aligned */);

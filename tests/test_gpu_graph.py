@@ -361,7 +361,7 @@ def test_packed_filter_entry_points_match_the_unpacked_ones():
     lib = capi.load()
     r = np.random.default_rng(0)
     cases = [((4, 16, 8, 8), 32), ((2, 64, 32, 32), 64), ((8, 128, 4, 4), 256), ((16, 48, 2, 2), 40), ((3, 3, 16, 16), 8),
-             ((2, 32, 16, 16), 96)]
+             ((2, 32, 16, 16), 96), ((20, 64, 2, 2), 128)]   # the last: 2 x 2 images read straight from the filter
     descs, flags, ws, packed, shapes = [], [], [], [], []
     for xs, k in cases:
         for bwd in (0, 1):
@@ -588,7 +588,9 @@ def test_batch_norm_gradient_with_a_sum_riding_along(shape, form, lanes, splits,
                                   ((16, 128, 8, 8), 256),
                                   ((2, 64, 32, 32), 64),
                                   ((48, 32, 32, 32), 32),    # channels too large for the resident batch norm: closed first
-                                  ((16, 48, 2, 2), 40)])     # dense 2x2 route: never open
+                                  ((16, 48, 2, 2), 40),      # dense 2x2 route: never open
+                                  ((24, 128, 2, 2), 64),     # 2 x 2 images straight from the filter: never open either
+                                  ((128, 512, 2, 2), 512)])  # ... at the benchmark shape
 def test_open_convolution_results_closed_by_batch_norm(xs, k):
     """The *_open convolutions followed by dopt_hip_bn_train_open / dopt_hip_bn_grad_open /
     dopt_hip_split_sum_close against the closed entry points (checked against the oracle elsewhere):
@@ -628,6 +630,8 @@ def test_open_convolution_results_closed_by_batch_norm(xs, k):
         if xs == (8, 256, 4, 4):
             assert o.splits > 1 and o.elems == np.prod(ys) and o.C == k and o.inner == inner
         if xs == (16, 48, 2, 2):
+            assert o.splits == 0
+        if xs[2:] == (2, 2):
             assert o.splits == 0
         if closer == "close":
             capi.check(lib.dopt_hip_split_sum_close(C.byref(o)))

@@ -338,6 +338,10 @@ CONV_CASES = [  # N, C, H, W, K, R, S, pad, stride
     # 2x2 images at sizes whose filter gradient is one launch (dense product with the fold in its
     # epilogue): the VGG shape, and one with a shorter batch and ragged edge tiles
     (128, 512, 2, 2, 512, 3, 3, (1, 1), (1, 1)),
+    # 2x2 images with channel counts in multiples of 64 read the filter itself (32 images x 8 channels per block, the
+    # reduction split over its wavefronts): ragged tiles of images, one and three steps per wavefront
+    (70, 64, 2, 2, 128, 3, 3, (1, 1), (1, 1)),
+    (5, 192, 2, 2, 64, 3, 3, (1, 1), (1, 1)),
     (100, 500, 2, 2, 520, 3, 3, (1, 1), (1, 1)),
     # at most three input channels, pad 1: the first-layer kernels (rows of 8 .. 128 pixels, one to
     # sixteen rows per sub-tile, output channels off the 32-row fragment, a single-channel image)
