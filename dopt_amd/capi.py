@@ -76,6 +76,7 @@ PROTOTYPES = {
     "dopt_hip_sgemm": [_sz, _sz, _sz, _vp, _vp, _vp],
     "dopt_hip_sgemm_t": [C.c_int, C.c_int, _sz, _sz, _sz, _vp, _vp, _vp],
     "dopt_hip_sgemm_rank1": [_i, _i, _sz, _sz, _sz, _vp, _vp, _vp, _vp, _i, _vp],
+    "dopt_hip_sgemm_relu_grad": [_i, _i, _sz, _sz, _sz, _vp, _vp, _vp, _vp],
     "dopt_hip_conv_fwd": [C.POINTER(ConvDesc), _vp, _vp, _vp],
     "dopt_hip_conv_fwd_bias": [C.POINTER(ConvDesc), _vp, _vp, _vp, _vp],
     "dopt_hip_conv_bwd_data": [C.POINTER(ConvDesc), _vp, _vp, _vp],

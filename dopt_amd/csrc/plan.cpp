@@ -634,6 +634,8 @@ struct HIPPlan::Builder {
     void fusePairs();
     void foldTransposes();
     void fuseDenseLayers();
+    void fuseDenseBackward();
+    bool plainProduct(int id, MatmulInfo *mi, bool sole_reader) const;
     void formChains();
     void absorbBiasGrads();
     void absorbPools();
@@ -844,23 +846,7 @@ void HIPPlan::Builder::foldTransposes()
 // and the relu becomes an alias of its output - the same arrangement as batch norm + relu above.
 void HIPPlan::Builder::fuseDenseLayers()
 {
-    auto plain_product = [&](int id, MatmulInfo *mi) {   // a matmul this pass may absorb: no other reader, not an output
-        if (alias[id].source >= 0 || isOutput(id) || uses[id].size() != 1 || g.ops[id].dtype != DOPT_HIP_F32 ||
-            g.ops[id].rank() != 2)
-            return false;
-        if (fusedKind[id] == 6 && mmInfo[id].valid) {
-            *mi = mmInfo[id];
-            return true;
-        }
-        const Operation &o = g.ops[id];
-        if (fusedKind[id] || o.opType != "matmul" || o.deps.size() != 2) return false;
-        const Operation &l = g.ops[o.deps[0]], &r = g.ops[o.deps[1]];
-        if (l.rank() != 2 || r.rank() != 2 || l.dtype != DOPT_HIP_F32 || r.dtype != DOPT_HIP_F32) return false;
-        mi->valid = true;
-        mi->a = o.deps[0]; mi->b = o.deps[1]; mi->tA = mi->tB = 0;
-        mi->M = o.shape[0]; mi->N = o.shape[1]; mi->K = l.shape[1];
-        return true;
-    };
+    auto plain_product = [&](int id, MatmulInfo *mi) { return plainProduct(id, mi, true); };   // a matmul this pass may absorb
     for (int id : p->mOps) {
         const Operation &op = g.ops[id];
         if (!live[id] || alias[id].source >= 0 || fusedKind[id] || op.opType != "add" || op.deps.size() != 2 ||
@@ -903,6 +889,58 @@ void HIPPlan::Builder::fuseDenseLayers()
                 alias[relu_op].offset = 0;
             }
             break;
+        }
+    }
+}
+
+// A rank-2 fp32 product as this pass may read it: what foldTransposes made of it, or the matmul as written.
+// sole_reader: only a product whose value has exactly one reader and is no plan output (it can be absorbed).
+bool HIPPlan::Builder::plainProduct(int id, MatmulInfo *mi, bool sole_reader) const
+{
+    if (alias[id].source >= 0 || g.ops[id].dtype != DOPT_HIP_F32 || g.ops[id].rank() != 2) return false;
+    if (sole_reader && (isOutput(id) || uses[id].size() != 1)) return false;
+    if (fusedKind[id] == 6 && mmInfo[id].valid) {
+        *mi = mmInfo[id];
+        return true;
+    }
+    const Operation &o = g.ops[id];
+    if (fusedKind[id] || o.opType != "matmul" || o.deps.size() != 2) return false;
+    const Operation &l = g.ops[o.deps[0]], &r = g.ops[o.deps[1]];
+    if (l.rank() != 2 || r.rank() != 2 || l.dtype != DOPT_HIP_F32 || r.dtype != DOPT_HIP_F32) return false;
+    mi->valid = true;
+    mi->a = o.deps[0]; mi->b = o.deps[1]; mi->tA = mi->tB = 0;
+    mi->M = o.shape[0]; mi->N = o.shape[1]; mi->K = l.shape[1];
+    return true;
+}
+
+// reluGrad(matmul(dz, W), y, x): the input gradient of a dense layer (nnet/layers/dense.d, differentiated by
+// core/ops/math.d:234-256) through the relu in front of it - a launch of its own for a few microseconds of work.
+// When the product has no other reader it runs with the mask in its epilogue (dopt_hip_sgemm_relu_grad); the values
+// do not change.  (The bias gradient next to it, matmul(ones, dz), could be summed by the weight-gradient product on
+// the way, but not in the order the ones-vector product adds it: that would make plans with and without the rewrites
+// differ in the last bit of every bias, so it stays a kernel of its own.)
+void HIPPlan::Builder::fuseDenseBackward()
+{
+    for (int id : p->mOps) {
+        const Operation &op = g.ops[id];
+        if (!live[id] || alias[id].source >= 0 || op.dtype != DOPT_HIP_F32 || op.volume() == 0) continue;
+        if (!fusedKind[id] && op.opType == "reluGrad" && op.deps.size() == 3 && op.rank() == 2) {
+            size_t off;
+            const int pid = root(op.deps[0], &off);
+            MatmulInfo mi;
+            if (off != 0 || !plainProduct(pid, &mi, true) || mi.K == 0 || mi.M != op.shape[0] || mi.N != op.shape[1] ||
+                g.ops[op.deps[2]].volume() != op.volume() || g.ops[op.deps[2]].dtype != DOPT_HIP_F32)
+                continue;
+            fusedKind[id] = 9;
+            inputsOf[id] = {mi.a, mi.b, op.deps[2]};
+            prebuilt[id] = make([=](const std::vector<const void *> &in, void *out) {
+                return dopt_hip_sgemm_relu_grad(mi.tA, mi.tB, mi.M, mi.N, mi.K, (const float *)in[0], (const float *)in[1],
+                                                (const float *)in[2], (float *)out);
+            });
+            prebuiltLabel[id] = "matmul+reluGrad";
+            prebuilt[pid].reset();   // the product no longer runs on its own
+            prebuiltLabel[pid].clear();
+            fusedKind[pid] = 0;
         }
     }
 }
@@ -1622,6 +1660,7 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         b.fusePairs();
         b.foldTransposes();
         b.fuseDenseLayers();
+        b.fuseDenseBackward();
         b.formChains();
         b.absorbBiasGrads();
         b.absorbPools();

@@ -197,7 +197,7 @@ template <bool kTA, bool kTB, bool kVec>
 __global__ __launch_bounds__(64 * kSmallWaves) void sgemm_small_k(int M, int N, int K, int lda, int ldb, int kslice,
                                                                    const float *A, const float *B, float *C,
                                                                    const float *colbias, int bias_shift,
-                                                                   const float *rowvec, int relu)
+                                                                   const float *rowvec, int relu, const float *mask)
 {
     __shared__ float red[kSmallWaves][32 * 33];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, r = lane & 31;
@@ -246,6 +246,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void sgemm_small_k(int M, int N, 
                 sum += add;
             }
             if (relu) sum = sum < 0.0f ? 0.0f : sum;
+            if (mask) sum = mask[(size_t)(m0 + rr) * N + n0 + cc] > 0.0f ? sum : 0.0f;   // reluGrad(product, ., mask)
             C[(size_t)(m0 + rr) * N + n0 + cc] = sum;
         }
     }
@@ -499,8 +500,13 @@ namespace dopt {
 
 // C = op(A) * op(B), plus colbias[col >> bias_shift] on every element when colbias is given.  Returns
 // *biased = false when the shape took a kernel without that epilogue (the caller adds the bias itself).
+// What may ride in a product's epilogue besides the bias forms: a reluGrad mask (C = mask > 0 ? product : 0).
+struct Extras {
+    const float *mask = nullptr;
+};
+
 int sgemm_epilogue(int transA, int transB, size_t M, size_t N, size_t K, const float *A, const float *B, float *C,
-                   const float *colbias, int bias_shift, const float *rowvec, int relu, bool *biased);
+                   const float *colbias, int bias_shift, const float *rowvec, int relu, bool *biased, const Extras &ex = Extras{});
 
 int sgemm_bias(int transA, int transB, size_t M, size_t N, size_t K, const float *A, const float *B, float *C,
                const float *colbias, int bias_shift, bool *biased)
@@ -511,7 +517,7 @@ int sgemm_bias(int transA, int transB, size_t M, size_t N, size_t K, const float
 // The products with an epilogue: + rowvec[row] * colbias[col >> bias_shift] (rowvec optional), then relu.
 // *biased says whether the kernel that ran applied it; if not, C holds the plain product.
 int sgemm_epilogue(int transA, int transB, size_t M, size_t N, size_t K, const float *A, const float *B, float *C,
-                   const float *colbias, int bias_shift, const float *rowvec, int relu, bool *biased)
+                   const float *colbias, int bias_shift, const float *rowvec, int relu, bool *biased, const Extras &ex)
 {
     *biased = false;
     if (M * N == 0) return DOPT_HIP_OK;
@@ -587,9 +593,9 @@ int sgemm_epilogue(int transA, int transB, size_t M, size_t N, size_t K, const f
 #define DOPT_SMALL(TA, TB)                                                                                             \
     do {                                                                                                               \
         if (vec) hipLaunchKernelGGL((sgemm_small_k<TA, TB, true>), grid, block, 0, stream(), (int)M, (int)N, (int)K, lda, \
-                                    ldb, kslice, A, B, C, colbias, bias_shift, rowvec, relu);                           \
+                                    ldb, kslice, A, B, C, colbias, bias_shift, rowvec, relu, ex.mask);                    \
         else hipLaunchKernelGGL((sgemm_small_k<TA, TB, false>), grid, block, 0, stream(), (int)M, (int)N, (int)K, lda,  \
-                                ldb, kslice, A, B, C, colbias, bias_shift, rowvec, relu);                               \
+                                ldb, kslice, A, B, C, colbias, bias_shift, rowvec, relu, ex.mask);                       \
     } while (0)
             if (transA && transB) DOPT_SMALL(true, true);
             else if (transA) DOPT_SMALL(true, false);
@@ -597,7 +603,7 @@ int sgemm_epilogue(int transA, int transB, size_t M, size_t N, size_t K, const f
             else DOPT_SMALL(false, false);
 #undef DOPT_SMALL
             DOPT_LAUNCH_CHECK();
-            *biased = true;   // whatever epilogue was asked for, this kernel applied it
+            *biased = true;   // whatever epilogue was asked for (the extras included), this kernel applied it
             return DOPT_HIP_OK;
         }
     }
@@ -683,6 +689,18 @@ int dopt_hip_sgemm_rank1(int transA, int transB, size_t M, size_t N, size_t K, c
     hipLaunchKernelGGL(rank1_epilogue_k, dim3(flat_grid(M * N)), dim3(256), 0, dopt::stream(), M, N, u, v, relu, C);
     DOPT_LAUNCH_CHECK();
     return DOPT_HIP_OK;
+}
+
+int dopt_hip_sgemm_relu_grad(int transA, int transB, size_t M, size_t N, size_t K, const float *A, const float *B,
+                             const float *x, float *C)
+{
+    DOPT_REQUIRE(x != nullptr || M * N == 0, "dopt_hip_sgemm_relu_grad: null argument");
+    dopt::Extras ex;
+    ex.mask = x;
+    bool applied = false;
+    if (int rc = dopt::sgemm_epilogue(transA, transB, M, N, K, A, B, C, nullptr, 0, nullptr, 0, &applied, ex)) return rc;
+    if (applied || M * N == 0) return DOPT_HIP_OK;
+    return dopt_hip_relu_bwd(M * N, C, x, C);   // in place: every element is read before it is written
 }
 
 int dopt_hip_sgemm_t(int transA, int transB, size_t M, size_t N, size_t K, const float *A, const float *B, float *C)

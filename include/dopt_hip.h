@@ -183,6 +183,13 @@ int dopt_hip_sgemm_t(int transA, int transB, size_t M, size_t N, size_t K, const
    DOPT_HIP_PLAN_FUSE. */
 int dopt_hip_sgemm_rank1(int transA, int transB, size_t M, size_t N, size_t K, const float *A,
                          const float *B, const float *u, const float *v, int relu, float *C);
+/* C = reluGrad(op(A) * op(B), ., x), i.e. the product where x[M,N] > 0 and zero elsewhere: the input gradient of a
+   dense layer (nnet/layers/dense.d:107, differentiated by core/ops/math.d:234-256) passed through the relu in front
+   of it (cudnnActivationBackward, cudnn7.d:470).  The mask is applied in the product's epilogue where the
+   small-output kernel runs it and by dopt_hip_relu_bwd in place behind it otherwise; either way the values are those
+   of dopt_hip_sgemm_t followed by dopt_hip_relu_bwd.  Used by plans compiled with DOPT_HIP_PLAN_FUSE. */
+int dopt_hip_sgemm_relu_grad(int transA, int transB, size_t M, size_t N, size_t K, const float *A,
+                             const float *B, const float *x, float *C);
 
 typedef struct {
     size_t N, C, H, W;       /* features [N,C,H,W] */

@@ -507,6 +507,56 @@ def test_backward_data_and_filter_gradient_as_one_call(xs, k):
     ops.sync()
 
 
+@pytest.mark.parametrize("M,N,K,ta,tb", [(128, 512, 512, 0, 0),     # the small-output kernel: the epilogue does it
+                                          (512, 512, 128, 1, 0),     # a weight gradient: dz stored [K][M]
+                                          (10, 512, 128, 1, 0),
+                                          (70, 33, 50, 0, 0),        # ragged tiles, scalar loads
+                                          (30, 40, 64, 1, 1),
+                                          (2048, 2048, 128, 1, 0),   # the LDS-resident panel kernel: separate launches behind it
+                                          (1500, 1200, 300, 0, 0),   # the tile engine
+                                          (1, 40, 64, 0, 0), (40, 1, 64, 1, 0), (8, 8, 1, 0, 0)])   # vector shapes
+def test_products_with_relu_gradient(M, N, K, ta, tb):
+    """dopt_hip_sgemm_relu_grad = dopt_hip_sgemm_t then dopt_hip_relu_bwd, bit for bit, whichever kernel runs the product."""
+    import ctypes as C
+    from dopt_amd import capi
+    lib = capi.load()
+    r = np.random.default_rng(M * 7 + N + K)
+    a = ops.tensor(r.standard_normal((K, M) if ta else (M, K)).astype(np.float32))
+    b = ops.tensor(r.standard_normal((N, K) if tb else (K, N)).astype(np.float32))
+    x = ops.tensor(r.standard_normal((M, N)).astype(np.float32))
+    prod = ops.matmul_t(a, b, bool(ta), bool(tb))
+    want = ops.relu_grad(prod, x).numpy()
+    got = ops.Tensor((M, N))
+    got.set(np.full((M, N), np.nan, np.float32))
+    capi.check(lib.dopt_hip_sgemm_relu_grad(ta, tb, M, N, K, a.ptr, b.ptr, x.ptr, got.ptr))
+    assert np.array_equal(got.numpy(), want)
+    ops.sync()
+
+
+def test_dense_backward_runs_inside_the_products():
+    """With the rewrites on, the relu gradient between two dense layers has no kernel of its own: the product in front of
+    it applies the mask.  Values as without the rewrites, bit for bit."""
+    r = np.random.default_rng(5)
+    X = r.random((64, 96)).astype(np.float32)
+    Y = np.zeros((64, 10), np.float32)
+    Y[np.arange(64), r.integers(0, 10, 64)] = 1
+    feats, labels = float32([64, 96]), float32([64, 10])
+    init = nnet.Init(6)
+    body = nnet.relu(nnet.dense(nnet.dataSource(feats), 128, init))
+    body = nnet.relu(nnet.dense(body, 80, init))
+    preds = nnet.softmax(nnet.dense(body, 10, init))
+    net = nnet.DAGNetwork([feats], [preds])
+    loss = nnet.crossEntropy(preds.trainOutput, labels) + net.paramLoss
+    outs = [loss] + core.grad(loss, net.params)
+    plan = core.compile(outs, core.PLAN_VIEWS | core.PLAN_FUSE | core.PLAN_TIMING)
+    fused = plan.execute({feats: X, labels: Y})
+    prof = plan.profile()
+    assert prof["matmul+reluGrad"][1] == 2 and "reluGrad" not in prof, prof
+    plain = core.compile(outs, core.PLAN_VIEWS).execute({feats: X, labels: Y})
+    for a, b in zip(plain, fused):
+        assert np.array_equal(a, b)
+
+
 @pytest.mark.parametrize("lanes,splits,n4", [(4, 16, 36864), (16, 37, 1000), (4, 3, 70000)])
 @pytest.mark.parametrize("shape,form", [
     ((16, 32, 8, 8), "dy"),            # one workgroup per channel, two quads per lane
