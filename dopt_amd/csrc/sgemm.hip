@@ -23,6 +23,7 @@ struct Gemm {
     int lda, ldb;  // row pitch of A and B as stored
     int mtiles, ntiles, slabs_total, slabs_per_split, splits;
     size_t out_elems;
+    bool quads_a, quads_b;  // sgemm_rows_k: the k-contiguous operand can be read in 16-byte pieces
 };
 
 // An operand tile is BR rows (of M or of N) by BK reduction steps, staged k-major in LDS:
@@ -152,6 +153,175 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_k(Gemm p)
 #pragma unroll
     for (int j = 0; j < 2; j++) {
         const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+        if (col >= p.N) continue;
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int m = m0 + wm * 64 + i * 32 + acc_row(v, lane);
+                if (m < p.M) outp[(size_t)m * p.N + col] = acc[i][j][v];
+            }
+    }
+}
+
+// The same product with row-major LDS tiles: Xs[r][k], 32 reduction steps per slab at a pitch of 36 floats, so that a
+// lane's operands for eight steps are ONE 128-bit LDS read (lane half h takes steps 8g + 4h .. 8g + 4h + 3 on both
+// operands - any pairing of steps works as long as A and B agree) instead of eight 32-bit reads: 16 LDS reads per
+// 64 matrix instructions where the k-major tiles above need 128.  Every instruction a wavefront issues besides the
+// matrix ones costs the matrix pipe about four cycles, which is what the large products lost.
+//   k-contiguous operand: a thread copies 16-byte pieces, eight lanes per 128-byte row segment (whole cache lines);
+//   r-contiguous operand: a thread gathers four reduction steps of one row with 4-byte loads (64 lanes = 256
+//     contiguous bytes per load) and stores them as one quad - the transposition happens in registers.
+// 128 x 128 tiles, four wavefronts of 64 x 64, two workgroups per CU.  It serves every product of more than 64 rows,
+// whatever the operands' alignment and however they are transposed, so that one (M, N, K) always adds its terms in
+// one order (a plan that reads a transposed operand in place gets the bits of the plan that copies it first).
+constexpr int BK2 = 32, kPitch2 = BK2 + 4;
+
+// Loads go through a buffer resource: an element outside the tile's rows or past the end of the reduction is fetched
+// from kOobOffset, where the hardware range check returns zero, so the loop holds no branch and every load of a slab is
+// in flight at once (guarded plain loads compile to one exec-masked region each, with waits in between).
+template <bool kKContig, bool kQuads>
+struct Stage2 {
+    float4 q[4];        // the staged quads: 128 rows x 8 quads over 256 threads
+    unsigned base[4];   // byte offset of quad i at reduction step 0, or kOobOffset when its row is outside the matrix
+    int kq[4];          // first reduction step of quad i inside a slab
+    unsigned step;      // bytes between consecutive reduction steps (r-contiguous: the row pitch)
+    __device__ void init(int ld, int r_base, int r_max, int tid)
+    {
+        step = kKContig ? 4u : (unsigned)ld * 4u;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            int row;
+            if (kKContig) {
+                const int idx = tid + 256 * i;
+                row = idx >> 3;
+                kq[i] = 4 * (idx & 7);
+            } else {
+                row = tid & 127;
+                kq[i] = 4 * ((tid >> 7) + 2 * i);
+            }
+            const int r = r_base + row;
+            const unsigned at = kKContig ? ((unsigned)r * (unsigned)ld + (unsigned)kq[i]) * 4u
+                                         : ((unsigned)kq[i] * (unsigned)ld + (unsigned)r) * 4u;
+            base[i] = r < r_max ? at : kOobOffset;
+        }
+    }
+    // kQuads: the rows of a k-contiguous operand are 16-byte addressable (pitch and the reduction's ends multiples of
+    // 4, aligned base); otherwise its pieces are fetched element by element - same values, same order of the sums.
+    // A slab wholly past the end of the reduction loads nothing (every offset out of range).
+    __device__ void load(__amdgpu_buffer_rsrc_t rs, int k0, int k_max)
+    {
+        const unsigned soff = (unsigned)k0 * step;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int k = k0 + kq[i];
+            if (kKContig && kQuads) {
+                q[i] = buffer_load_f32x4(rs, k < k_max ? base[i] : kOobOffset, soff);
+            } else {
+                q[i].x = buffer_load_f32(rs, k + 0 < k_max ? base[i] : kOobOffset, soff);
+                q[i].y = buffer_load_f32(rs, k + 1 < k_max ? base[i] + step : kOobOffset, soff);
+                q[i].z = buffer_load_f32(rs, k + 2 < k_max ? base[i] + 2u * step : kOobOffset, soff);
+                q[i].w = buffer_load_f32(rs, k + 3 < k_max ? base[i] + 3u * step : kOobOffset, soff);
+            }
+        }
+    }
+    __device__ void store(float *Xs, int tid) const
+    {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int row = kKContig ? (tid + 256 * i) >> 3 : tid & 127;
+            *(float4 *)&Xs[row * kPitch2 + kq[i]] = q[i];
+        }
+    }
+};
+
+template <bool kTA, bool kTB, bool kQA, bool kQB>
+__global__ __launch_bounds__(kGemmThreads, 2) void sgemm_rows_k(Gemm p)
+{
+    constexpr int BM = 128, BN = 128;
+    __shared__ __attribute__((aligned(16))) float As[2][BM * kPitch2];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BN * kPitch2];
+
+    unsigned L;
+    const unsigned tiles = (unsigned)(p.mtiles * p.ntiles);
+    if (!xcd_remap(blockIdx.x, tiles * (unsigned)p.splits, &L)) return;
+    const int split = (int)(L / tiles);
+    const unsigned tile = L - (unsigned)split * tiles;
+    const int mt = (int)(tile % (unsigned)p.mtiles), nt = (int)(tile / (unsigned)p.mtiles);
+    const int m0 = mt * BM, n0 = nt * BN;
+    // p.slabs_* count 16-step slabs (the other kernel's unit): two of them per slab here
+    const int k_begin = split * p.slabs_per_split * BK;
+    const int k_end = min(min(k_begin + p.slabs_per_split * BK, p.slabs_total * BK), p.K);
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, l32 = lane & 31, kh = lane >> 5;
+    const int wm = w >> 1, wn = w & 1;
+    const int a_frag = (wm * 64 + l32) * kPitch2 + 4 * kh, b_frag = (wn * 64 + l32) * kPitch2 + 4 * kh;
+
+    v16f acc[2][2];
+    zero_acc(acc);
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.A, (size_t)p.M * p.K * sizeof(float));
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.B, (size_t)p.K * p.N * sizeof(float));
+    // Two register sets: while slab s is multiplied out of LDS, slab s + 1 waits in one set to be stored behind it and
+    // slab s + 2 is on its way into the other, so a load has two slabs' worth of matrix work to arrive.  No branch
+    // inside the loop: loads behind the last slab fall out of range and fetch nothing, their stores fill a buffer
+    // nobody reads.
+    Stage2<!kTA, kQA> la[2];   // A as given is k-contiguous
+    Stage2<kTB, kQB> lb[2];    // B transposed is k-contiguous
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        la[u].init(p.lda, m0, p.M, tid);
+        lb[u].init(p.ldb, n0, p.N, tid);
+    }
+    la[0].load(ra, k_begin, k_end);
+    lb[0].load(rb, k_begin, k_end);
+    la[1].load(ra, k_begin + BK2, k_end);
+    lb[1].load(rb, k_begin + BK2, k_end);
+    la[0].store(As[0], tid);
+    lb[0].store(Bs[0], tid);
+    __syncthreads();
+    auto slab = [&](const float *as, const float *bs) {
+#pragma unroll
+        for (int g = 0; g < BK2 / 8; g++) {
+            float4 a[2], b[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++) a[i] = *(const float4 *)(as + i * 32 * kPitch2 + 8 * g);
+#pragma unroll
+            for (int j = 0; j < 2; j++) b[j] = *(const float4 *)(bs + j * 32 * kPitch2 + 8 * g);
+            // step by step over the four accumulators: consecutive matrix instructions never wait for each other
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
+                        const float av = e == 0 ? a[i].x : e == 1 ? a[i].y : e == 2 ? a[i].z : a[i].w;
+                        const float bv = e == 0 ? b[j].x : e == 1 ? b[j].y : e == 2 ? b[j].z : b[j].w;
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[i][j], 0, 0, 0);
+                    }
+        }
+    };
+    // iteration pair: slab k0 from buffer 0 (set 1 holds k0 + 32, set 0 is refilled with k0 + 64), then slab k0 + 32
+    // from buffer 1 (set 0 holds k0 + 64, set 1 is refilled with k0 + 96)
+    for (int k0 = k_begin; k0 < k_end; k0 += 2 * BK2) {
+        la[0].load(ra, k0 + 2 * BK2, k_end);
+        lb[0].load(rb, k0 + 2 * BK2, k_end);
+        slab(As[0] + a_frag, Bs[0] + b_frag);
+        la[1].store(As[1], tid);
+        lb[1].store(Bs[1], tid);
+        __syncthreads();
+        if (k0 + BK2 >= k_end) break;   // uniform
+        la[1].load(ra, k0 + 3 * BK2, k_end);
+        lb[1].load(rb, k0 + 3 * BK2, k_end);
+        slab(As[1] + a_frag, Bs[1] + b_frag);
+        la[0].store(As[0], tid);
+        lb[0].store(Bs[0], tid);
+        __syncthreads();
+    }
+
+    float *outp = p.C + (size_t)split * p.out_elems;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int col = n0 + wn * 64 + j * 32 + l32;
         if (col >= p.N) continue;
 #pragma unroll
         for (int i = 0; i < 2; i++)
@@ -652,7 +822,22 @@ int sgemm_epilogue(int transA, int transB, size_t M, size_t N, size_t K, const f
         else if (!transB) DOPT_SGEMM(BMV, true, false);     \
         else DOPT_SGEMM(BMV, true, true);                   \
     } while (0)
-    if (big) DOPT_SGEMM_T(128);
+    // more than 64 rows: row-major LDS tiles (sgemm_rows_k)
+    g.quads_a = g.lda % 4 == 0 && K % 4 == 0 && aligned16(A);
+    g.quads_b = g.ldb % 4 == 0 && K % 4 == 0 && aligned16(B);
+    if (big && M * K < ((size_t)1 << 29) && K * N < ((size_t)1 << 29)) {   // 32-bit byte offsets into either operand
+#define DOPT_ROWS(TA, TB, QA, QB) hipLaunchKernelGGL((sgemm_rows_k<TA, TB, QA, QB>), grid, dim3(kGemmThreads), 0, stream(), g)
+        const bool qa = g.quads_a, qb = g.quads_b;   // only a k-contiguous operand has the choice
+        if (!transA && !transB) { if (qa) DOPT_ROWS(false, false, true, false); else DOPT_ROWS(false, false, false, false); }
+        else if (!transA) {
+            if (qa && qb) DOPT_ROWS(false, true, true, true);
+            else if (qa) DOPT_ROWS(false, true, true, false);
+            else if (qb) DOPT_ROWS(false, true, false, true);
+            else DOPT_ROWS(false, true, false, false);
+        } else if (!transB) DOPT_ROWS(true, false, false, false);
+        else { if (qb) DOPT_ROWS(true, true, false, true); else DOPT_ROWS(true, true, false, false); }
+#undef DOPT_ROWS
+    } else if (big) DOPT_SGEMM_T(128);
     else DOPT_SGEMM_T(64);
 #undef DOPT_SGEMM_T
 #undef DOPT_SGEMM

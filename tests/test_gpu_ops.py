@@ -770,6 +770,32 @@ def test_sgemm_short_reduction_large_output(shape):
     assert_close(got.numpy(), O.matmul(a, b, f64=True), "sgemm_t panel", scale=np.sqrt(K))
 
 
+@pytest.mark.parametrize("shape", [(1024, 1024, 1024),   # 64 tiles, the reduction split over workgroups
+                                   (2100, 2050, 36),     # more tiles than the small-output kernel takes, ragged edges
+                                   (1100, 1030, 1026),   # a reduction that is no multiple of 4: element-wise loads
+                                   (4096, 640, 70)])
+def test_sgemm_large_products_all_operand_layouts(shape):
+    """Products of more than 64 rows that the small-output kernel does not take (sgemm_rows_k): against float64, and
+    every transposition - also with operands off the 16-byte grid - gives the product of the plain copies to the last
+    bit (one order of summation per shape)."""
+    M, N, K = shape
+    r = rng(M + N + K)
+    a = r.standard_normal((M, K)).astype(np.float32)
+    b = (r.standard_normal((K, N)) * np.sqrt(2.0 / K)).astype(np.float32)
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    plain = ops.matmul(T(a), T(b)).numpy()
+    assert_close(plain, want, "sgemm %dx%dx%d" % shape)
+    for ta in (False, True):
+        for tb in (False, True):
+            sa, sb = (np.ascontiguousarray(a.T) if ta else a), (np.ascontiguousarray(b.T) if tb else b)
+            assert np.array_equal(ops.matmul_t(T(sa), T(sb), ta, tb).numpy(), plain), (ta, tb)
+            # the same operands one float off the 16-byte grid
+            ba = T(np.concatenate([np.zeros(1, np.float32), sa.ravel()]))
+            bb = T(np.concatenate([np.zeros(1, np.float32), sb.ravel()]))
+            got = ops.matmul_t(ba.view(1, sa.shape), bb.view(1, sb.shape), ta, tb).numpy()
+            assert np.array_equal(got, plain), (ta, tb, "unaligned")
+
+
 @pytest.mark.parametrize("shape", [(128, 512, 512), (70, 33, 129), (130, 10, 512), (1, 300, 77), (200, 1, 64), (5, 7, 1),
                                    (256, 256, 40), (64, 260, 96)])
 @pytest.mark.parametrize("ta,tb", [(False, True), (True, False), (True, True)])
