@@ -125,16 +125,20 @@ __device__ inline float4 pool_grad(const Pool &pl, float4 y, unsigned idx)
 {
     const bool present = idx != 0xffffffffu;
     float4 r;
+    // an absent lane loads element 0 and drops it: a load under a lane mask would end in a wait of its own, and the
+    // loads of a thread's quads would go out one after the other instead of together
     if (pl.mode == 2) {
-        const float g = present ? pool_dvalue<float>(pl, idx, true) : 0.0f;
+        const float gl = pool_dvalue<float>(pl, present ? idx : 0u, present);
+        const float g = present ? gl : 0.0f;
         route2x2(y.x, y.y, y.z, y.w, g, r.x, r.y, r.z, r.w);
         return r;
     }
     const float4 o = quad_xor(y, pl.wq);
-    const unsigned row = present ? idx >> pl.wshift : 0u, cq = idx & (pl.wq - 1);
+    const unsigned row = present ? idx >> pl.wshift : 0u, cq = present ? idx & (pl.wq - 1) : 0u;
     const bool odd = row & 1;
     // both rows of a window read its gradient; the even row writes the finished sum of an open one
-    const float2 g = present ? pool_dvalue<float2>(pl, (size_t)(row >> 1) * pl.wq + cq, !odd) : make_float2(0.0f, 0.0f);
+    const float2 gl = pool_dvalue<float2>(pl, (size_t)(row >> 1) * pl.wq + cq, present && !odd);
+    const float2 g = present ? gl : make_float2(0.0f, 0.0f);
     const float4 top = odd ? o : y, bot = odd ? y : o;
     float4 t, b;
     route2x2(top.x, top.y, bot.x, bot.y, g.x, t.x, t.y, b.x, b.y);
@@ -591,34 +595,47 @@ __global__ __launch_bounds__(1024) void bn_resident_k(unsigned N, unsigned C, un
     const unsigned c = blockIdx.x, T = blockDim.x, E4 = N * inner4;
     const float4 *x4 = (const float4 *)x, *g4 = (const float4 *)dy;
     float4 xv[kQ], gv[kQ];
-    unsigned idx[kQ];
+    unsigned idx[kQ], at[kQ];
 #pragma unroll
     for (int i = 0; i < kQ; i++) {
         const unsigned q = i * T + threadIdx.x;
         const unsigned n = q / inner4, r = q - n * inner4;
         idx[i] = q < E4 ? (n * C + c) * inner4 + r : 0xffffffffu;
-        xv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-        gv[i] = xv[i];
-        if (q < E4) {
-            if (!(kOpen && !kGrad)) xv[i] = x4[idx[i]];
-            if (kGrad && !kOpen) {
-                if (pool.mode) gv[i] = ((const float4 *)ymask)[idx[i]];   // y for now; dy below
-                else {
-                    gv[i] = g4[idx[i]];
-                    if (ymask) gv[i] = masked4(gv[i], ((const float4 *)ymask)[idx[i]]);
-                }
+        at[i] = q < E4 ? idx[i] : c * inner4;   // an absent quad loads the channel's first one and drops it
+    }
+    // Loads are clamped, never branched, and grouped per operand: a load under a lane mask ends in a wait of its own,
+    // and a thread's quads would be fetched one after the other instead of all at once.
+    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int i = 0; i < kQ; i++) {
+        xv[i] = (kOpen && !kGrad) ? zero4 : x4[at[i]];
+        gv[i] = zero4;
+    }
+    if (kGrad && !kOpen) {
+        if (pool.mode) {
+#pragma unroll
+            for (int i = 0; i < kQ; i++) gv[i] = ((const float4 *)ymask)[at[i]];   // y for now; dy below
+        } else {
+#pragma unroll
+            for (int i = 0; i < kQ; i++) gv[i] = g4[at[i]];
+            if (ymask) {
+                float4 mv[kQ];
+#pragma unroll
+                for (int i = 0; i < kQ; i++) mv[i] = ((const float4 *)ymask)[at[i]];
+#pragma unroll
+                for (int i = 0; i < kQ; i++) gv[i] = masked4(gv[i], mv[i]);
             }
         }
     }
+#pragma unroll
+    for (int i = 0; i < kQ; i++)
+        if (idx[i] == 0xffffffffu) xv[i] = gv[i] = zero4;
     if (kGrad && !kOpen && pool.mode) {   // dy = reluGrad(maxpoolGrad(dpool, y), y)
 #pragma unroll
         for (int i = 0; i < kQ; i++) gv[i] = masked4(pool_grad(pool, gv[i], idx[i]), gv[i]);
     }
     if (kOpen) {
         float4 sum[kQ];
-        unsigned at[kQ];
-#pragma unroll
-        for (int i = 0; i < kQ; i++) at[i] = idx[i] == 0xffffffffu ? 0u : idx[i];   // clamped, not branched
         // two to four copies: every load of the thread is issued before the first add
         if (open.splits == 2) open_add<2, kQ>(open, at, sum);
         else if (open.splits == 3) open_add<3, kQ>(open, at, sum);
@@ -794,26 +811,41 @@ __global__ __launch_bounds__(1024) void bn_cluster_k(unsigned N, unsigned C, uns
     const unsigned mine = E4 - q0 < per ? E4 - q0 : per;
     const float4 *x4 = (const float4 *)x, *g4 = (const float4 *)dy;
     float4 xv[kQ], gv[kQ];
-    unsigned idx[kQ];
+    unsigned idx[kQ], at[kQ];
 #pragma unroll
     for (int i = 0; i < kQ; i++) {
         const unsigned l = i * T + threadIdx.x;
         const unsigned q = q0 + l;
         const unsigned n = q / inner4, r = q - n * inner4;
         idx[i] = l < mine ? (n * C + c) * inner4 + r : 0xffffffffu;
-        xv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-        gv[i] = xv[i];
-        if (l < mine) {
-            xv[i] = x4[idx[i]];
-            if (kGrad) {
-                if (pool.mode) gv[i] = ((const float4 *)ymask)[idx[i]];   // y for now; dy below
-                else {
-                    gv[i] = g4[idx[i]];
-                    if (ymask) gv[i] = masked4(gv[i], ((const float4 *)ymask)[idx[i]]);
-                }
+        at[i] = l < mine ? idx[i] : c * inner4;   // an absent quad loads the channel's first one and drops it
+    }
+    // clamped, never branched, grouped per operand: all of a thread's loads are in flight together (see bn_resident_k)
+    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int i = 0; i < kQ; i++) {
+        xv[i] = x4[at[i]];
+        gv[i] = zero4;
+    }
+    if (kGrad) {
+        if (pool.mode) {
+#pragma unroll
+            for (int i = 0; i < kQ; i++) gv[i] = ((const float4 *)ymask)[at[i]];   // y for now; dy below
+        } else {
+#pragma unroll
+            for (int i = 0; i < kQ; i++) gv[i] = g4[at[i]];
+            if (ymask) {
+                float4 mv[kQ];
+#pragma unroll
+                for (int i = 0; i < kQ; i++) mv[i] = ((const float4 *)ymask)[at[i]];
+#pragma unroll
+                for (int i = 0; i < kQ; i++) gv[i] = masked4(gv[i], mv[i]);
             }
         }
     }
+#pragma unroll
+    for (int i = 0; i < kQ; i++)
+        if (idx[i] == 0xffffffffu) xv[i] = gv[i] = zero4;
     if (kGrad && pool.mode) {   // dy = reluGrad(maxpoolGrad(dpool, y), y)
 #pragma unroll
         for (int i = 0; i < kQ; i++) gv[i] = masked4(pool_grad(pool, gv[i], idx[i]), gv[i]);
