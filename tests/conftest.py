@@ -27,14 +27,14 @@ def kats():
 
 
 def pytest_sessionfinish(session, exitstatus):
-    """The configuration tests record the largest error they saw per quantity; keep the table where a
-    GPU run's outputs are collected."""
+    """The configuration tests record the largest error they saw per quantity; the table is written to the directory
+    DOPT_TEST_REPORT_DIR names (nothing is written when it is not set)."""
     try:
         import util
     except ImportError:
         return
-    out_dir = os.path.join(ROOT, "gpurun_out")
-    if not util.ERROR_ROWS or not os.path.isdir(out_dir):
+    out_dir = os.environ.get("DOPT_TEST_REPORT_DIR", "")
+    if not util.ERROR_ROWS or not out_dir or not os.path.isdir(out_dir):
         return
     with open(os.path.join(out_dir, "parity_errors.txt"), "w") as f:
         f.write("%-34s %-40s %12s %14s %12s\n" % ("case", "quantity", "max|err|", "err/(a+r|w|)", "max|want|"))

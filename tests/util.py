@@ -32,7 +32,7 @@ def assert_close(got, want, what="", rtol=GEMM_RTOL, atol=GEMM_ATOL, scale=None)
 
 
 # Rows of (case, quantity, max |err|, max |err| / (atol + rtol |want|), max |want|) collected by the
-# configuration tests; conftest.py writes them to gpurun_out/parity_errors.txt at the end of a session.
+# configuration tests; conftest.py writes them to parity_errors.txt at the end of a session (see there).
 ERROR_ROWS = []
 
 
