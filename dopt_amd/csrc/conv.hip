@@ -290,12 +290,15 @@ __device__ __forceinline__ void conv_patch_body(const PatchConv &p, const unsign
     // ---- filter fragments: this lane's 8 channels (kh * 8 ..) of row l32 of each 32-row group
     const unsigned slab_bytes = (unsigned)p.Mp * CH * 4u;
     const unsigned fa_voff = (unsigned)((m0 + wm * (BM / T::WM) + l32) * CH + kh * 8) * 4u;   // m0 + row < Mp always
-    float4 fa_next[MI][2];
-    auto fa_load = [&](int slab) {   // past the last slab the range check returns zeros
+    // three sets of filter fragments: the tap being multiplied, the next one, and the one after it on its way (a tap
+    // lasts ~0.4 us per wavefront, less than a load from the L2 can take under load)
+    float4 fa_ring[3][MI][2];
+    auto fa_load = [&](auto slot_tag, int slab) {   // past the last slab the range check returns zeros
+        constexpr int slot = decltype(slot_tag)::value;
 #pragma unroll
         for (int i = 0; i < MI; i++) {
-            fa_next[i][0] = buffer_load_f32x4(rwp, fa_voff + (unsigned)(i * 32 * CH) * 4u, (unsigned)slab * slab_bytes);
-            fa_next[i][1] = buffer_load_f32x4(rwp, fa_voff + (unsigned)(i * 32 * CH) * 4u + 16u, (unsigned)slab * slab_bytes);
+            fa_ring[slot][i][0] = buffer_load_f32x4(rwp, fa_voff + (unsigned)(i * 32 * CH) * 4u, (unsigned)slab * slab_bytes);
+            fa_ring[slot][i][1] = buffer_load_f32x4(rwp, fa_voff + (unsigned)(i * 32 * CH) * 4u + 16u, (unsigned)slab * slab_bytes);
         }
     };
     int b_frag[NI];  // float offset inside a patch buffer of this lane's pixel, tap offset (0,0)
@@ -312,7 +315,8 @@ __device__ __forceinline__ void conv_patch_body(const PatchConv &p, const unsign
     // prologue: the first patch and the first filter slab
 #pragma unroll
     for (int i = 0; i < NPMAX; i++) patch_load(i, cb);
-    fa_load(cb * TAPS);
+    fa_load(StepTag<0>{}, cb * TAPS);
+    fa_load(StepTag<1>{}, cb * TAPS + 1);
 #pragma unroll
     for (int i = 0; i < NPMAX; i++) patch_store(i, Bp0);
     __syncthreads();
@@ -330,9 +334,9 @@ __device__ __forceinline__ void conv_patch_body(const PatchConv &p, const unsign
             const int tapoff = (p.flip ? (2 - tr) * p.PC + (2 - ts) : tr * p.PC + ts) * LDP;
             float4 fa[MI][2], fb[NI][2];
 #pragma unroll
-            for (int i = 0; i < MI; i++) {
-                fa[i][0] = fa_next[i][0];
-                fa[i][1] = fa_next[i][1];
+            for (int i = 0; i < MI; i++) {   // nine taps per chunk: the ring slot of a tap is the same in every chunk
+                fa[i][0] = fa_ring[t % 3][i][0];
+                fa[i][1] = fa_ring[t % 3][i][1];
             }
 #pragma unroll
             for (int j = 0; j < NI; j++) {
@@ -342,7 +346,7 @@ __device__ __forceinline__ void conv_patch_body(const PatchConv &p, const unsign
             static_for<0, 8>([&](auto stag) {
                 constexpr int ks = decltype(stag)::value;
                 // side work of this step
-                if constexpr (ks == 0) fa_load(sidx + 1);
+                if constexpr (ks == 0) fa_load(StepTag<(t + 2) % 3>{}, sidx + 2);
                 if constexpr (t < 4 && ks >= 1 && ks <= 6) {
                     // PER loads of tap t, dealt over steps 1..6
                     constexpr int first = t * PER + (ks - 1) * ((PER + 5) / 6);
