@@ -921,9 +921,20 @@ bool HIPPlan::Builder::plainProduct(int id, MatmulInfo *mi, bool sole_reader) co
 // differ in the last bit of every bias, so it stays a kernel of its own.)
 void HIPPlan::Builder::fuseDenseBackward()
 {
+    // Which values the kernels as rewritten so far still read: a reluGrad that a batch-norm gradient reads around
+    // (fusePairs) is dead, and the product in front of it now feeds that kernel - it must stay what it is.
+    std::vector<char> read((size_t)nops, 0);
+    for (int x : p->mOps) {
+        if (!live[x] || alias[x].source >= 0) continue;
+        for (int d : inputsOf[x]) {
+            size_t off;
+            read[root(d, &off)] = 1;
+        }
+    }
     for (int id : p->mOps) {
         const Operation &op = g.ops[id];
         if (!live[id] || alias[id].source >= 0 || op.dtype != DOPT_HIP_F32 || op.volume() == 0) continue;
+        if (!read[id] && !isOutput(id)) continue;
         if (!fusedKind[id] && op.opType == "reluGrad" && op.deps.size() == 3 && op.rank() == 2) {
             size_t off;
             const int pid = root(op.deps[0], &off);

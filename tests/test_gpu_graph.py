@@ -557,6 +557,37 @@ def test_dense_backward_runs_inside_the_products():
         assert np.array_equal(a, b)
 
 
+def test_dense_backward_keeps_a_product_that_a_batch_norm_gradient_reads():
+    """dense -> batch norm -> relu -> dense: the batch-norm gradient applies the relu mask itself and reads the product
+    behind the relu gradient, so that product has to stay a plain one - the relu gradient nobody reads any more must not
+    pull it into a masked product.  Values as without the rewrites."""
+    r = np.random.default_rng(8)
+    X = r.standard_normal((64, 48)).astype(np.float32)
+    Y = np.zeros((64, 10), np.float32)
+    Y[np.arange(64), r.integers(0, 10, 64)] = 1
+    feats, labels = float32([64, 48]), float32([64, 10])
+    init = nnet.Init(9)
+    body = nnet.dense(nnet.dataSource(feats), 32, init)
+    as_images = nnet.Layer([body], body.output.reshape([64, 32, 1, 1]), body.trainOutput.reshape([64, 32, 1, 1]), [])
+    normed = nnet.relu(nnet.batchNorm(as_images))
+    flat = nnet.Layer([normed], normed.output.reshape([64, 32]), normed.trainOutput.reshape([64, 32]), [])
+    body = nnet.relu(nnet.dense(flat, 40, init))
+    preds = nnet.softmax(nnet.dense(body, 10, init))
+    net = nnet.DAGNetwork([feats], [preds])
+    loss = nnet.crossEntropy(preds.trainOutput, labels) + net.paramLoss
+    outs = [loss] + core.grad(loss, net.params)
+    plan = core.compile(outs, core.PLAN_VIEWS | core.PLAN_FUSE | core.PLAN_TIMING)
+    fused = plan.execute({feats: X, labels: Y})
+    prof = plan.profile()
+    assert prof["matmul+reluGrad"][1] == 1 and "reluGrad" not in prof, prof   # the one between the last two dense layers
+    plain = core.compile(outs, core.PLAN_VIEWS).execute({feats: X, labels: Y})
+    for a, b in zip(plain, fused):
+        if a.ndim <= 1 or a.size == a.shape[0]:
+            np.testing.assert_allclose(a, b, rtol=2e-5, atol=1e-6)
+        else:
+            assert np.array_equal(a, b)
+
+
 @pytest.mark.parametrize("lanes,splits,n4", [(4, 16, 36864), (16, 37, 1000), (4, 3, 70000)])
 @pytest.mark.parametrize("shape,form", [
     ((16, 32, 8, 8), "dy"),            # one workgroup per channel, two quads per lane
