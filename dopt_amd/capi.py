@@ -126,6 +126,7 @@ _SPECIAL = {
     "dopt_hip_last_error": ([], C.c_char_p),
     "dopt_hip_stream": ([], _vp),
     "dopt_hip_conv_packed_bytes": ([C.POINTER(ConvDesc), _i], _sz),
+    "dopt_hip_sgemm_order": ([C.c_int, C.c_int, _sz, _sz, _sz], C.c_uint64),
 }
 
 _lib = None

@@ -779,7 +779,9 @@ void HIPPlan::Builder::foldTransposes()
 {
     // matmul reads a transposed operand in place instead of a copy made by `transpose`, and
     // transpose(matmul(A, B)) is computed as matmul(B^T, A^T); the transposes left without a
-    // reader drop out.
+    // reader drop out.  Only where the product as rewritten adds its terms in the order of the product
+    // as written (dopt_hip_sgemm_order): a flag or exchanged dimensions can select another kernel, and
+    // a plan with rewrites has to give the bits of the plan without.
     auto is_swap = [&](int t) {
         const Operation &o = g.ops[t];
         if (o.opType != "transpose" || o.deps.size() != 1 || o.rank() != 2 || alias[t].source >= 0) return false;
@@ -800,32 +802,46 @@ void HIPPlan::Builder::foldTransposes()
         return o.opType == "matmul" && o.deps.size() == 2 && o.rank() == 2 && o.dtype == DOPT_HIP_F32 &&
                alias[m].source < 0;
     };
+    struct Fold { int a, b; bool tA, tB; size_t M, N, K; bool same_order; };
+    auto fold_of = [&](int mm, bool outT) {   // the product `mm` (or its transpose) on the matrices behind the transposes
+        Fold f{};
+        f.a = through(g.ops[mm].deps[0], &f.tA);
+        f.b = through(g.ops[mm].deps[1], &f.tB);
+        f.M = g.ops[mm].shape[0];
+        f.N = g.ops[mm].shape[1];
+        f.K = g.ops[g.ops[mm].deps[0]].shape[1];
+        const uint64_t as_written = dopt_hip_sgemm_order(0, 0, f.M, f.N, f.K);
+        if (outT) {  // (A B)^T = B^T A^T
+            std::swap(f.a, f.b);
+            const bool na = !f.tB, nb = !f.tA;
+            f.tA = na;
+            f.tB = nb;
+            std::swap(f.M, f.N);
+        }
+        f.same_order = as_written != 0 && dopt_hip_sgemm_order(f.tA, f.tB, f.M, f.N, f.K) == as_written;
+        return f;
+    };
+    auto feeds_a_transpose_only = [&](int mm) {
+        return uses[mm].size() == 1 && is_swap(uses[mm][0].op) && !isOutput(mm);
+    };
     for (int id : p->mOps) {
         if (!live[id]) continue;
         int mm = id;
         bool outT = false;  // compute the transpose of the product
-        if (is_swap(id) && plain_matmul(g.ops[id].deps[0]) && uses[g.ops[id].deps[0]].size() == 1 &&
-            !isOutput(g.ops[id].deps[0])) {
+        if (is_swap(id) && plain_matmul(g.ops[id].deps[0]) && feeds_a_transpose_only(g.ops[id].deps[0])) {
             mm = g.ops[id].deps[0];
             outT = true;
         } else if (!plain_matmul(id)) {
             continue;
         }
         if (!outT && fusedKind[id]) continue;
-        bool tA, tB;
-        int a = through(g.ops[mm].deps[0], &tA), b = through(g.ops[mm].deps[1], &tB);
-        if (!outT && a == g.ops[mm].deps[0] && b == g.ops[mm].deps[1]) continue;  // nothing to fold
-        if (!outT && uses[mm].size() == 1 && is_swap(uses[mm][0].op) && !isOutput(mm)) continue;  // folded into its transpose
-        size_t M = g.ops[mm].shape[0], N = g.ops[mm].shape[1];
-        const Operation &ao = g.ops[g.ops[mm].deps[0]];
-        size_t K = ao.shape[1];
-        if (outT) {  // (A B)^T = B^T A^T
-            std::swap(a, b);
-            const bool na = !tB, nb = !tA;
-            tA = na;
-            tB = nb;
-            std::swap(M, N);
-        }
+        if (!outT && feeds_a_transpose_only(mm) && fold_of(mm, true).same_order) continue;  // folded into its transpose
+        const Fold f = fold_of(mm, outT);
+        if (!f.same_order) continue;
+        if (!outT && f.a == g.ops[mm].deps[0] && f.b == g.ops[mm].deps[1]) continue;  // nothing to fold
+        int a = f.a, b = f.b;
+        bool tA = f.tA, tB = f.tB;
+        size_t M = f.M, N = f.N, K = f.K;
         fusedKind[id] = 6;
         inputsOf[id] = {a, b};
         const int ta = tA, tb = tB;

@@ -680,12 +680,6 @@ int dopt_hip_reduce(const char *op, int dtype, const size_t *shape, int rank, co
     }
     if (vol == 0) return DOPT_HIP_OK;
     DOPT_ENSURE_INIT();
-    std::string key = std::string("red:") + op + (dtype == DOPT_HIP_F32 ? ":f32" : ":i32");
-    std::string src = reduce_source(is_sum, dtype);
-    hipFunction_t rows, rows4, cols;
-    if (int rc = rtc_get(key + ":rows", src, "red_rows", &rows)) return rc;
-    if (int rc = rtc_get(key + ":rows4", src, "red_rows4", &rows4)) return rc;
-    if (int rc = rtc_get(key + ":cols", src, "red_cols", &cols)) return rc;
 
     // Runs of adjacent reduced axes collapse into one (outer, R, inner) pass each, last run first.
     // The result is independent of the order in which axes are folded up to fp32 rounding.
@@ -707,6 +701,12 @@ int dopt_hip_reduce(const char *op, int dtype, const size_t *shape, int rank, co
         int crc = DOPT_HIP_OK;
         if (channel_sum(N, C, inner, (const float *)in, (float *)out, &crc)) return crc;
     }
+    std::string key = std::string("red:") + op + (dtype == DOPT_HIP_F32 ? ":f32" : ":i32");
+    std::string src = reduce_source(is_sum, dtype);
+    hipFunction_t rows, rows4, cols;
+    if (int rc = rtc_get(key + ":rows", src, "red_rows", &rows)) return rc;
+    if (int rc = rtc_get(key + ":rows4", src, "red_rows4", &rows4)) return rc;
+    if (int rc = rtc_get(key + ":cols", src, "red_cols", &cols)) return rc;
     const void *src_ptr = in;
     void *tmp_prev = nullptr;
     int rc = DOPT_HIP_OK;

@@ -636,11 +636,16 @@ unsigned flat_grid(size_t n)
 // The LDS-resident kernel wins where its 128 x 128 tiles give every CU one or two blocks and the
 // operands take 128-bit loads (2048 x 2048 x 128: 17 us against 22 us for the 32 x 32 tiles); with
 // fewer tiles CUs idle, with more the tile engine's two resident blocks per CU overlap better.
-bool panel_takes(size_t M, size_t N, size_t K, const float *A, const float *B)
+bool panel_shape(size_t M, size_t N, size_t K)
 {
     const size_t tiles = ceil_div(M, (size_t)kPanelTile) * ceil_div(N, (size_t)kPanelTile);
-    return K >= 1 && K <= (size_t)kPanelK && tiles >= (size_t)num_cus() && tiles <= (size_t)2 * num_cus() &&
-           aligned16(A) && aligned16(B) && M % 4 == 0 && N % 4 == 0;
+    return K >= 1 && K <= (size_t)kPanelK && tiles >= (size_t)num_cus() && tiles <= (size_t)2 * num_cus() && M % 4 == 0 &&
+           N % 4 == 0;
+}
+
+bool panel_takes(size_t M, size_t N, size_t K, const float *A, const float *B)
+{
+    return panel_shape(M, N, K) && aligned16(A) && aligned16(B);
 }
 
 int panel_launch(bool fold, size_t M, size_t N, size_t K, const float *A, const float *B, float *C)
@@ -684,6 +689,62 @@ int sgemm_bias(int transA, int transB, size_t M, size_t N, size_t K, const float
     return sgemm_epilogue(transA, transB, M, N, K, A, B, C, colbias, bias_shift, nullptr, 0, biased);
 }
 
+// Which kernel a product takes and how it cuts the reduction: everything that decides the order in which an
+// element's K terms are added.  It follows from the dimensions and the transposition flags alone - not from an epilogue
+// being asked for, which a kernel without one leaves to a pass behind it; operand alignment picks between variants of a
+// kernel that add in the same order (the LDS-resident kernel apart: panel_allowed = false is the route without it).
+struct Route {
+    enum Kind { kNone, kOuter, kGemvRows, kGemvColsShort, kGemvCols, kPanel, kSmall, kTile64, kTile128, kRows } kind;
+    size_t cuts;    // partial sums per element that a second pass adds (gemv slices, tile-engine splits)
+    size_t depth;   // reduction steps per partial sum (k per slice, slabs per split)
+};
+
+Route sgemm_route(int transA, int transB, size_t M, size_t N, size_t K, bool panel_allowed = true)
+{
+    Route r{Route::kNone, 1, K};
+    if (M * N == 0 || K == 0) return r;
+    if (K == 1) { r.kind = Route::kOuter; return r; }
+    // matrix-vector products: `rows` reads the matrix row by row (k contiguous), `cols` column-wise
+    if ((N == 1 && !transA) || (M == 1 && transB)) { r.kind = Route::kGemvRows; return r; }
+    if ((M == 1 && !transB) || (N == 1 && transA)) {
+        const size_t R = M == 1 ? N : M;
+        if (K <= 256 && R < ((size_t)1 << 30)) { r.kind = Route::kGemvColsShort; return r; }   // one launch, no partial sums
+        const size_t nblocks = ceil_div(R, (size_t)256);
+        size_t slices = ceil_div((size_t)num_cus() * 2, nblocks);
+        if (slices > ceil_div(K, (size_t)32)) slices = ceil_div(K, (size_t)32);
+        if (slices > 64) slices = 64;
+        if (slices < 1) slices = 1;
+        r.kind = Route::kGemvCols;
+        r.depth = ceil_div(K, slices);
+        r.cuts = ceil_div(K, r.depth);
+        return r;
+    }
+    // short reduction, both operands k-major, enough 128 x 128 tiles to fill the machine (alignment is checked at the
+    // launch: the plan's buffers and every tensor of the pool are aligned)
+    if (transA && !transB && panel_allowed && panel_shape(M, N, K)) { r.kind = Route::kPanel; return r; }
+    // small and medium outputs: one block per 32 x 32 tile, the reduction split over its wavefronts.
+    // Each tile reads its own 32 rows of A and 32 columns of B, so the operand traffic grows with the
+    // number of tiles: up to 256 MB of it (served by the L2) this beats the LDS-tiled engine below,
+    // whose 128-wide tiles leave most CUs with one four-wavefront block (1024 x 1024 x 256: 11 against
+    // 22 us; 2048 x 2048 x 128: 21 against 31 us); beyond that the tile engine's operand reuse wins.
+    const size_t tiles32 = ceil_div(M, (size_t)32) * ceil_div(N, (size_t)32);
+    if (tiles32 <= 4096 && tiles32 * 64 * K * sizeof(float) <= ((size_t)256 << 20)) { r.kind = Route::kSmall; return r; }
+    const bool big = M > 64;
+    const size_t BM = big ? 128 : 64, BN = big ? 128 : 256;
+    const size_t tiles = ceil_div(M, BM) * ceil_div(N, BN);
+    const size_t slabs_total = ceil_div(K, (size_t)BK);
+    size_t want = ((size_t)2 * num_cus() + tiles - 1) / tiles;
+    const size_t max_by_depth = slabs_total / 4 > 0 ? slabs_total / 4 : 1;
+    size_t splits = want < max_by_depth ? want : max_by_depth;
+    if (splits > 32) splits = 32;
+    if (splits < 1) splits = 1;
+    r.depth = (slabs_total + splits - 1) / splits;
+    r.cuts = (slabs_total + r.depth - 1) / r.depth;
+    // more than 64 rows: row-major LDS tiles (sgemm_rows_k) while byte offsets into either operand fit 32 bits
+    r.kind = !big ? Route::kTile64 : M * K < ((size_t)1 << 29) && K * N < ((size_t)1 << 29) ? Route::kRows : Route::kTile128;
+    return r;
+}
+
 // The products with an epilogue: + rowvec[row] * colbias[col >> bias_shift] (rowvec optional), then relu.
 // *biased says whether the kernel that ran applied it; if not, C holds the plain product.
 int sgemm_epilogue(int transA, int transB, size_t M, size_t N, size_t K, const float *A, const float *B, float *C,
@@ -699,37 +760,32 @@ int sgemm_epilogue(int transA, int transB, size_t M, size_t N, size_t K, const f
                      M * N < ((size_t)1 << 40),
                  "dopt_hip_sgemm: dimensions too large");
 
-    if (K == 1) {  // vectors: a transposed vector is the same memory
+    Route route = sgemm_route(transA, transB, M, N, K);
+    if (route.kind == Route::kPanel && !panel_takes(M, N, K, A, B))   // operands off the 16-byte grid: as if it were not there
+        route = sgemm_route(transA, transB, M, N, K, false);
+    const Route::Kind kind = route.kind;
+    if (kind == Route::kOuter) {  // vectors: a transposed vector is the same memory
         hipLaunchKernelGGL(outer_k, dim3(flat_grid(M * N)), dim3(256), 0, stream(), M, N, A, B, C);
         DOPT_LAUNCH_CHECK();
         return DOPT_HIP_OK;
     }
-    // matrix-vector products: `rows` reads the matrix row by row (k contiguous), `cols` column-wise
-    const bool mv_rows = (N == 1 && !transA) || (M == 1 && transB);
-    const bool mv_cols = (M == 1 && !transB) || (N == 1 && transA);
-    if (mv_rows) {
+    if (kind == Route::kGemvRows) {
         const size_t R = N == 1 ? M : N;
         const float *mat = N == 1 ? A : B, *vec = N == 1 ? B : A;
         hipLaunchKernelGGL(gemv_rows_k, dim3((unsigned)ceil_div(R, (size_t)4)), dim3(256), 0, stream(), R, K, mat, vec, C);
         DOPT_LAUNCH_CHECK();
         return DOPT_HIP_OK;
     }
-    if (mv_cols) {
+    if (kind == Route::kGemvColsShort || kind == Route::kGemvCols) {
         const size_t R = M == 1 ? N : M;
         const float *mat = M == 1 ? B : A, *vec = M == 1 ? A : B;
-        if (K <= 256 && R < ((size_t)1 << 30)) {   // one launch, no partial sums
+        if (kind == Route::kGemvColsShort) {
             hipLaunchKernelGGL(gemv_cols_short_k, dim3((unsigned)ceil_div(R, (size_t)64)), dim3(256), 0, stream(), (int)K, (int)R,
                                vec, mat, C);
             DOPT_LAUNCH_CHECK();
             return DOPT_HIP_OK;
         }
-        size_t nblocks = ceil_div(R, (size_t)256);
-        size_t slices = ceil_div((size_t)num_cus() * 2, nblocks);
-        if (slices > ceil_div(K, (size_t)32)) slices = ceil_div(K, (size_t)32);
-        if (slices > 64) slices = 64;
-        if (slices < 1) slices = 1;
-        size_t kslice = ceil_div(K, slices);
-        slices = ceil_div(K, kslice);
+        const size_t nblocks = ceil_div(R, (size_t)256), slices = route.cuts, kslice = route.depth;
         float *partial = C;
         if (slices > 1) {
             partial = (float *)workspace(slices * R * sizeof(float));
@@ -744,22 +800,12 @@ int sgemm_epilogue(int transA, int transB, size_t M, size_t N, size_t K, const f
         }
         return DOPT_HIP_OK;
     }
-
-    // short reduction, both operands k-major, enough 128 x 128 tiles to fill the machine
-    if (transA && !transB && !colbias && !relu && panel_takes(M, N, K, A, B)) return panel_launch(false, M, N, K, A, B, C);
-
-    // small and medium outputs: one block per 32 x 32 tile, the reduction split over its wavefronts.
-    // Each tile reads its own 32 rows of A and 32 columns of B, so the operand traffic grows with the
-    // number of tiles: up to 256 MB of it (served by the L2) this beats the LDS-tiled engine below,
-    // whose 128-wide tiles leave most CUs with one four-wavefront block (1024 x 1024 x 256: 11 against
-    // 22 us; 2048 x 2048 x 128: 21 against 31 us); beyond that the tile engine's operand reuse wins.
-    {
-        const size_t tiles = ceil_div(M, (size_t)32) * ceil_div(N, (size_t)32);
-        if (tiles <= 4096 && tiles * 64 * K * sizeof(float) <= ((size_t)256 << 20)) {
-            const int lda = (int)(transA ? M : K), ldb = (int)(transB ? K : N);
-            int kslice = (int)ceil_div(ceil_div(K, (size_t)kSmallWaves), (size_t)8) * 8;
-            const bool vec = aligned16(A) && aligned16(B) && lda % 4 == 0 && ldb % 4 == 0;
-            const dim3 grid((unsigned)ceil_div(N, (size_t)32), (unsigned)ceil_div(M, (size_t)32)), block(64 * kSmallWaves);
+    if (kind == Route::kPanel) return panel_launch(false, M, N, K, A, B, C);
+    if (kind == Route::kSmall) {
+        const int lda = (int)(transA ? M : K), ldb = (int)(transB ? K : N);
+        int kslice = (int)ceil_div(ceil_div(K, (size_t)kSmallWaves), (size_t)8) * 8;
+        const bool vec = aligned16(A) && aligned16(B) && lda % 4 == 0 && ldb % 4 == 0;
+        const dim3 grid((unsigned)ceil_div(N, (size_t)32), (unsigned)ceil_div(M, (size_t)32)), block(64 * kSmallWaves);
 #define DOPT_SMALL(TA, TB)                                                                                             \
     do {                                                                                                               \
         if (vec) hipLaunchKernelGGL((sgemm_small_k<TA, TB, true>), grid, block, 0, stream(), (int)M, (int)N, (int)K, lda, \
@@ -767,15 +813,14 @@ int sgemm_epilogue(int transA, int transB, size_t M, size_t N, size_t K, const f
         else hipLaunchKernelGGL((sgemm_small_k<TA, TB, false>), grid, block, 0, stream(), (int)M, (int)N, (int)K, lda,  \
                                 ldb, kslice, A, B, C, colbias, bias_shift, rowvec, relu, ex.mask);                       \
     } while (0)
-            if (transA && transB) DOPT_SMALL(true, true);
-            else if (transA) DOPT_SMALL(true, false);
-            else if (transB) DOPT_SMALL(false, true);
-            else DOPT_SMALL(false, false);
+        if (transA && transB) DOPT_SMALL(true, true);
+        else if (transA) DOPT_SMALL(true, false);
+        else if (transB) DOPT_SMALL(false, true);
+        else DOPT_SMALL(false, false);
 #undef DOPT_SMALL
-            DOPT_LAUNCH_CHECK();
-            *biased = true;   // whatever epilogue was asked for (the extras included), this kernel applied it
-            return DOPT_HIP_OK;
-        }
+        DOPT_LAUNCH_CHECK();
+        *biased = true;   // whatever epilogue was asked for (the extras included), this kernel applied it
+        return DOPT_HIP_OK;
     }
 
     Gemm g{};
@@ -788,18 +833,13 @@ int sgemm_epilogue(int transA, int transB, size_t M, size_t N, size_t K, const f
     g.ldb = (int)(transB ? K : N);
     g.out_elems = M * N;
     g.slabs_total = (int)ceil_div(K, (size_t)BK);
-    const bool big = M > 64;
+    const bool big = kind != Route::kTile64;
     const int BM = big ? 128 : 64, BN = big ? 128 : 256;
     g.mtiles = (int)ceil_div(M, (size_t)BM);
     g.ntiles = (int)ceil_div(N, (size_t)BN);
     const int tiles = g.mtiles * g.ntiles;
-    int want = (2 * num_cus() + tiles - 1) / tiles;
-    int max_by_depth = g.slabs_total / 4 > 0 ? g.slabs_total / 4 : 1;
-    int splits = want < max_by_depth ? want : max_by_depth;
-    if (splits > 32) splits = 32;
-    if (splits < 1) splits = 1;
-    g.slabs_per_split = (g.slabs_total + splits - 1) / splits;
-    splits = (g.slabs_total + g.slabs_per_split - 1) / g.slabs_per_split;
+    const int splits = (int)route.cuts;
+    g.slabs_per_split = (int)route.depth;
     g.splits = splits;
     float *partial = nullptr;
     if (splits > 1) {
@@ -825,7 +865,7 @@ int sgemm_epilogue(int transA, int transB, size_t M, size_t N, size_t K, const f
     // more than 64 rows: row-major LDS tiles (sgemm_rows_k)
     g.quads_a = g.lda % 4 == 0 && K % 4 == 0 && aligned16(A);
     g.quads_b = g.ldb % 4 == 0 && K % 4 == 0 && aligned16(B);
-    if (big && M * K < ((size_t)1 << 29) && K * N < ((size_t)1 << 29)) {   // 32-bit byte offsets into either operand
+    if (kind == Route::kRows) {
 #define DOPT_ROWS(TA, TB, QA, QB) hipLaunchKernelGGL((sgemm_rows_k<TA, TB, QA, QB>), grid, dim3(kGemmThreads), 0, stream(), g)
         const bool qa = g.quads_a, qb = g.quads_b;   // only a k-contiguous operand has the choice
         if (!transA && !transB) { if (qa) DOPT_ROWS(false, false, true, false); else DOPT_ROWS(false, false, false, false); }
@@ -886,6 +926,13 @@ int dopt_hip_sgemm_relu_grad(int transA, int transB, size_t M, size_t N, size_t 
     if (int rc = dopt::sgemm_epilogue(transA, transB, M, N, K, A, B, C, nullptr, 0, nullptr, 0, &applied, ex)) return rc;
     if (applied || M * N == 0) return DOPT_HIP_OK;
     return dopt_hip_relu_bwd(M * N, C, x, C);   // in place: every element is read before it is written
+}
+
+uint64_t dopt_hip_sgemm_order(int transA, int transB, size_t M, size_t N, size_t K)
+{
+    if (!dopt::ensure_init()) return 0;   // the cut of a reduction follows the device's size
+    const dopt::Route r = dopt::sgemm_route(transA, transB, M, N, K);
+    return (uint64_t)r.kind | (uint64_t)r.cuts << 8 | (uint64_t)r.depth << 24;
 }
 
 int dopt_hip_sgemm_t(int transA, int transB, size_t M, size_t N, size_t K, const float *A, const float *B, float *C)

@@ -39,6 +39,19 @@ def gemm_rows():
     return rows, keep
 
 
+_blocker = []
+
+
+def _hold_the_queue():
+    """Enqueues a product that lasts several milliseconds.  The calls timed behind it are enqueued while it runs, so
+    the device executes them back to back and the events measure kernels, not the host's call overhead (a Python call
+    into the library costs as much as a short kernel lasts)."""
+    if not _blocker:
+        a, b = _rand((8192, 8192), 21), _rand((8192, 8192), 22)
+        _blocker.extend([a, b, ops.matmul(a, b)])
+    ops.matmul(_blocker[0], _blocker[1], out=_blocker[2])
+
+
 def _time(fn, iters, warm=5):
     lib = capi.load()
     ev = [C.c_void_p(), C.c_void_p()]
@@ -46,6 +59,7 @@ def _time(fn, iters, warm=5):
         capi.check(lib.dopt_hip_event_create(C.byref(e)))
     for _ in range(warm):
         fn()
+    _hold_the_queue()
     capi.check(lib.dopt_hip_event_record(ev[0]))
     for _ in range(iters):
         fn()

@@ -174,6 +174,14 @@ int dopt_hip_sgemm(size_t M, size_t N, size_t K, const float *A, const float *B,
    the `transpose` kernels that only feed a matmul. */
 int dopt_hip_sgemm_t(int transA, int transB, size_t M, size_t N, size_t K, const float *A,
                      const float *B, float *C);
+/* Names the order in which dopt_hip_sgemm_t adds the K terms of an output element for these flags and dimensions
+   (which kernel runs, and where it cuts the reduction): two calls with equal values give equal bits for equal
+   operand values, also when one computes the transpose of the other's product, (A B)^T = B^T A^T with M and N
+   exchanged; calls with different values may differ in the last bits.  Operands are taken to lie on 16-byte
+   boundaries, as every buffer of this library does.  0: the device could not be initialised.  No counterpart in the
+   reference, whose plans never rewrite a product; plans compiled with DOPT_HIP_PLAN_FUSE read a transposed
+   operand in place only where this says that the values stay what the `transpose` copies would have given. */
+uint64_t dopt_hip_sgemm_order(int transA, int transB, size_t M, size_t N, size_t K);
 /* C = op(A) * op(B) + u[M,1] * v[1,N], then relu when relu != 0: a dense layer as the reference
    spells it -- matmul(x, W^T) (nnet/layers/dense.d:107) plus the bias broadcast over the rows, which
    is itself a matmul with a ones column (dense.d:143, core/ops/basic.d:370-381), then the relu

@@ -796,6 +796,43 @@ def test_sgemm_large_products_all_operand_layouts(shape):
             assert np.array_equal(got, plain), (ta, tb, "unaligned")
 
 
+@pytest.mark.parametrize("shape", [(12, 32768, 32), (32768, 12, 16), (12, 32768, 100), (64, 8192, 512), (8192, 64, 512),
+                                   (33, 70000, 40), (70000, 33, 40), (128, 2048, 2048), (2048, 128, 2048),
+                                   (256, 256, 8192), (1, 3000, 77), (3000, 1, 77), (1, 5000, 700), (5000, 1, 700),
+                                   (40, 48, 300), (4096, 512, 128), (2100, 2050, 36), (100, 9, 1)])
+def test_sgemm_order_names_what_gives_equal_bits(shape):
+    """dopt_hip_sgemm_order's promise, which the plan's transpose folding rests on: whatever the flags, and whether a
+    call computes the product or its transpose, calls with the same order value give the same bits.  At least the
+    plain product and its transposed form with both flags set always exist; the count of differing values is
+    printed by the assertion so that a shape whose every call stands alone is visible."""
+    from dopt_amd import capi
+    lib = capi.load()
+    M, N, K = shape
+    r = rng(M * 5 + N * 11 + K)
+    a = r.standard_normal((M, K)).astype(np.float32)
+    b = r.standard_normal((K, N)).astype(np.float32)
+    seen = {}
+    for out_t in (False, True):
+        for ta in (False, True):
+            for tb in (False, True):
+                sa, sb = (np.ascontiguousarray(a.T) if ta else a), (np.ascontiguousarray(b.T) if tb else b)
+                if out_t:   # (A B)^T = B^T A^T on the same memory: B as stored is B^T read transposed, and so on
+                    order = lib.dopt_hip_sgemm_order(int(not tb), int(not ta), N, M, K)
+                    got = ops.matmul_t(T(sb), T(sa), not tb, not ta).numpy().T
+                else:
+                    order = lib.dopt_hip_sgemm_order(int(ta), int(tb), M, N, K)
+                    got = ops.matmul_t(T(sa), T(sb), ta, tb).numpy()
+                assert order != 0
+                if order in seen:
+                    assert np.array_equal(got, seen[order][0]), (shape, (out_t, ta, tb), seen[order][1], hex(order))
+                else:
+                    seen[order] = (got, (out_t, ta, tb))
+    assert len(seen) <= 4, sorted(hex(k) for k in seen)
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    for got, which in seen.values():
+        assert_close(got, want, "sgemm %s %s" % (shape, which), scale=np.sqrt(K))
+
+
 @pytest.mark.parametrize("shape", [(128, 512, 512), (70, 33, 129), (130, 10, 512), (1, 300, 77), (200, 1, 64), (5, 7, 1),
                                    (256, 256, 40), (64, 260, 96)])
 @pytest.mark.parametrize("ta,tb", [(False, True), (True, False), (True, True)])
