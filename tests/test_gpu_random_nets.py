@@ -8,7 +8,7 @@ matches on the graph, and a pattern that fires on a neighbourhood it was not wri
 import numpy as np
 import pytest
 
-from dopt_amd import core, nnet, workloads
+from dopt_amd import core, nnet, online, workloads
 from dopt_amd.core import float32, grad
 from oracle import evaluator
 from util import assert_close
@@ -30,18 +30,28 @@ def _as_images(layer):
 def _random_net(r, feats, widths=(8, 16, 24, 32, 64)):
     init = nnet.Init(int(r.integers(1 << 30)))
     layer = nnet.dataSource(feats)
-    size = feats.shape[2]
+
+    def size():
+        return layer.output.shape[2]
+
+    def decay():
+        return float(r.choice([0.0, 0.0, 5e-4]))
+
     for _ in range(int(r.integers(2, 5))):
         channels = int(r.choice(widths))
         entry = layer
-        shape = int(r.integers(0, 8))
+        shape = int(r.integers(0, 10))
+        bias = bool(r.integers(0, 2))
         if shape == 0:
-            conv = nnet.conv2D(layer, channels, (1, 1), init, use_bias=bool(r.integers(0, 2)))
-        elif shape == 1 and size >= 8:
-            conv = nnet.conv2D(layer, channels, (3, 3), init, padding=(1, 1), stride=(2, 2), use_bias=bool(r.integers(0, 2)))
-            size //= 2
+            conv = nnet.conv2D(layer, channels, (1, 1), init, use_bias=bias, weight_decay=decay())
+        elif shape == 1 and size() >= 8:
+            conv = nnet.conv2D(layer, channels, (3, 3), init, padding=(1, 1), stride=(2, 2), use_bias=bias)
+        elif shape == 2 and size() >= 8:
+            conv = nnet.conv2D(layer, channels, (3, 3), init, use_bias=bias)                    # no padding: the image shrinks
+        elif shape == 3 and size() >= 8:
+            conv = nnet.conv2D(layer, channels, (5, 5), init, padding=(2, 2), use_bias=bias, weight_decay=decay())
         else:
-            conv = nnet.conv2D(layer, channels, (3, 3), init, padding=(1, 1), use_bias=bool(r.integers(0, 2)))
+            conv = nnet.conv2D(layer, channels, (3, 3), init, padding=(1, 1), use_bias=bias, weight_decay=decay())
         order = int(r.integers(0, 6))
         if order == 0:
             layer = nnet.relu(nnet.batchNorm(conv))
@@ -51,21 +61,20 @@ def _random_net(r, feats, widths=(8, 16, 24, 32, 64)):
             layer = nnet.batchNorm(conv)
         elif order == 3:
             layer = nnet.batchNorm(nnet.relu(conv))
-        elif order == 4:
+        elif order == 4 and entry.output.shape[2] % conv.output.shape[2] == 0:
             # a residual block: the entry reaches the sum through a 1x1 projection of the same stride
             stride = (entry.output.shape[2] // conv.output.shape[2],) * 2
             shortcut = nnet.conv2D(entry, channels, (1, 1), init, stride=stride, use_bias=False)
             layer = _residual(nnet.relu(nnet.batchNorm(conv)), shortcut)
         else:
             layer = conv
-        if size >= 4 and r.integers(0, 2):
+        if size() >= 4 and size() % 2 == 0 and r.integers(0, 2):
             layer = nnet.maxPool(layer, (2, 2))
-            size //= 2
             if r.integers(0, 3) == 0:
                 layer = nnet.relu(layer)
     for _ in range(int(r.integers(0, 3))):
         width = int(r.choice([12, 32, 40]))
-        dense = nnet.dense(layer, width, init, use_bias=bool(r.integers(0, 2)))
+        dense = nnet.dense(layer, width, init, use_bias=bool(r.integers(0, 2)), weight_decay=decay())
         head = int(r.integers(0, 4))
         if head == 0:
             layer = nnet.relu(nnet.batchNorm(_as_images(dense)))
@@ -120,7 +129,7 @@ def test_random_networks_match_the_cpu_evaluator_with_and_without_rewrites(seed)
         plan.cleanup()
 
 
-@pytest.mark.parametrize("seed", range(24))
+@pytest.mark.parametrize("seed", range(48))
 def test_random_wider_networks_give_the_same_values_with_the_rewrites(seed):
     """The same at sizes where the tiled convolution kernels, packed filters, one-launch backward pairs and results
     left as partial copies come into play (the small networks above mostly take the generic kernels): the plans with
@@ -152,3 +161,42 @@ def test_random_wider_networks_give_the_same_values_with_the_rewrites(seed):
                 else:
                     assert np.array_equal(g, p), what
         plan.cleanup()
+
+
+@pytest.mark.parametrize("seed", range(18))
+def test_random_networks_fused_updaters_follow_the_op_graph_updaters(seed):
+    """Two steps of SGD (plain, momentum, Nesterov), ADAM or AMSGrad on a random network: the fused update kernels
+    leave the parameters and report the losses the reference's op-graph update rules do, bit for bit, with and
+    without the plan rewrites."""
+    rule = seed % 3
+    after = []
+    for fused in (False, True):
+        for flags in (0, REWRITES):
+            r = np.random.default_rng(6000 + seed)
+            n, size, cin = int(r.choice([4, 8])), int(r.choice([8, 16])), int(r.choice([3, 16]))
+            X = r.standard_normal((n, cin, size, size)).astype(np.float32)
+            Y = workloads.one_hot(r.integers(0, 10, n))
+            feats, labels = float32([n, cin, size, size]), float32([n, 10])
+            preds = _random_net(r, feats)
+            net = nnet.DAGNetwork([feats], [preds])
+            loss = nnet.crossEntropy(preds.trainOutput, labels) + net.paramLoss
+            if rule == 0:
+                mu, nesterov = float(r.choice([0.0, 0.9])), bool(r.integers(0, 2))
+                if fused:
+                    up = online.fused_sgd([loss], net.params, net.paramProj, 0.05, mu, nesterov, flags=flags)
+                else:
+                    up = online.sgd([loss], net.params, net.paramProj, float32([], [0.05]), float32([], [mu]), nesterov, flags=flags)
+            elif rule == 1:
+                up = (online.fused_adam if fused else online.adam)([loss], net.params, net.paramProj, flags=flags)
+            else:
+                up = (online.fused_amsgrad if fused else online.amsgrad)([loss], net.params, net.paramProj, flags=flags)
+            losses = [up({feats: X, labels: Y})[0] for _ in range(2)]
+            after.append((fused, flags, losses, [p.value.copy() for p in net.params]))
+            del up
+    for flags in (0, REWRITES):
+        graph, fusedrun = [a for a in after if a[1] == flags]
+        assert not graph[0] and fusedrun[0]
+        assert np.isfinite(graph[2]).all() and graph[2][0] != graph[2][1], graph[2]
+        assert graph[2] == fusedrun[2], (seed, flags, graph[2], fusedrun[2])
+        for i, (a, b) in enumerate(zip(graph[3], fusedrun[3])):
+            assert np.array_equal(a, b), (seed, flags, i, a.shape)
