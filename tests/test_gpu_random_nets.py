@@ -72,6 +72,8 @@ def _random_net(r, feats, widths=(8, 16, 24, 32, 64)):
             layer = nnet.maxPool(layer, (2, 2))
             if r.integers(0, 3) == 0:
                 layer = nnet.relu(layer)
+    if r.integers(0, 4) == 0:
+        layer = nnet.meanPool(layer)           # the Wide-ResNet head: a row sum, which `sum` turns into a GEMV
     for _ in range(int(r.integers(0, 3))):
         width = int(r.choice([12, 32, 40]))
         dense = nnet.dense(layer, width, init, use_bias=bool(r.integers(0, 2)), weight_decay=decay())
