@@ -343,63 +343,80 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_rows_k(Gemm p)
 //
 // X is "k-contiguous" when element (r, k) sits at X[r * ld + k] (A as given, B transposed), else
 // "r-contiguous" at X[k * ld + r].
+//
+// Loads go through buffer resources (an element outside the matrix or past the end of the wavefront's share of K
+// comes from kOobOffset and reads as zero: no branch) and kSmallDepth steps are in flight per wavefront: with one
+// step of prefetch every step waited a full memory latency, eight of them in a row for a 512-deep reduction -
+// most of such a kernel's duration.  The order of the sums is that of the steps, whatever is in flight.
+constexpr int kSmallWaves = 8, kSmallDepth = 4;
+
+// The lane's four reductions kk .. kk + 3 of row / column r.  `base`: byte offset of (r, reduction 0), or kOobOffset
+// when r lies outside the matrix; `pitch`: bytes between consecutive reductions of an r-contiguous operand.
 template <bool kKContig, bool kVec>
-__device__ __forceinline__ void small_load(const float *X, int ld, int r, bool r_ok, int kk, int k_end, float (&v)[4])
+__device__ __forceinline__ void small_load(__amdgpu_buffer_rsrc_t rs, unsigned base, unsigned pitch, int kk, int k_end,
+                                           float (&v)[4])
 {
-    if (kKContig) {
-        const float *src = X + (size_t)r * ld + kk;
-        if (kVec && r_ok && kk + 3 < k_end) {
-            const float4 q = *(const float4 *)src;
-            v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
-        } else {
-#pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = (r_ok && kk + e < k_end) ? src[e] : 0.0f;
-        }
+    if (kKContig && kVec) {   // rows are whole quads: the end of the reduction never cuts one
+        const float4 q = buffer_load_f32x4(rs, kk < k_end ? base + (unsigned)kk * 4u : kOobOffset, 0);
+        v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
     } else {
+        const unsigned step = kKContig ? 4u : pitch;
 #pragma unroll
-        for (int e = 0; e < 4; e++) v[e] = (r_ok && kk + e < k_end) ? X[(size_t)(kk + e) * ld + r] : 0.0f;
+        for (int e = 0; e < 4; e++) v[e] = buffer_load_f32(rs, kk + e < k_end ? base + (unsigned)(kk + e) * step : kOobOffset, 0);
     }
 }
 
-constexpr int kSmallWaves = 8;
-
-template <bool kTA, bool kTB, bool kVec>
+// kVA / kVB: the rows of a k-contiguous A / B are 16-byte addressable (an r-contiguous operand has no use for the flag).
+template <bool kTA, bool kTB, bool kVA, bool kVB>
 __global__ __launch_bounds__(64 * kSmallWaves) void sgemm_small_k(int M, int N, int K, int lda, int ldb, int kslice,
                                                                    const float *A, const float *B, float *C,
                                                                    const float *colbias, int bias_shift,
                                                                    const float *rowvec, int relu, const float *mask)
 {
     __shared__ float red[kSmallWaves][32 * 33];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, r = lane & 31;
+    const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, r = lane & 31;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // the same in every lane: loop bounds stay scalar
     const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
     const int row = m0 + r, col = n0 + r;
-    const bool row_ok = row < M, col_ok = col < N;
     const int k_begin = wave * kslice, k_end = min(K, k_begin + kslice);
+    const __amdgpu_buffer_rsrc_t rsa = make_rsrc(A, (size_t)M * K * sizeof(float)), rsb = make_rsrc(B, (size_t)K * N * sizeof(float));
+    // A is k-contiguous as given, B when it is read transposed
+    const unsigned abase = row < M ? (kTA ? (unsigned)row * 4u : (unsigned)row * (unsigned)lda * 4u) : kOobOffset;
+    const unsigned bbase = col < N ? (kTB ? (unsigned)col * (unsigned)ldb * 4u : (unsigned)col * 4u) : kOobOffset;
+    const unsigned apitch = (unsigned)lda * 4u, bpitch = (unsigned)ldb * 4u;
 
     v16f acc;
 #pragma unroll
     for (int v = 0; v < 16; v++) acc[v] = 0.0f;
-    float a[4], b[4], an[4], bn[4];
-    if (k_begin < k_end) {
-        small_load<!kTA, kVec>(A, lda, row, row_ok, k_begin + 4 * half, k_end, a);
-        small_load<kTB, kVec>(B, ldb, col, col_ok, k_begin + 4 * half, k_end, b);
-    }
-    for (int k = k_begin; k < k_end; k += 8) {
-        const bool more = k + 8 < k_end;
-        if (more) {   // the next step's operands are in flight while this step multiplies
-            small_load<!kTA, kVec>(A, lda, row, row_ok, k + 8 + 4 * half, k_end, an);
-            small_load<kTB, kVec>(B, ldb, col, col_ok, k + 8 + 4 * half, k_end, bn);
-        }
+    float a[kSmallDepth][4], b[kSmallDepth][4];
+    const int nsteps = k_begin < k_end ? (k_end - k_begin + 7) / 8 : 0;
 #pragma unroll
-        for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], acc, 0, 0, 0);
-        if (more) {
+    for (int j = 0; j < kSmallDepth; j++) {   // steps past the end fetch nothing
+        small_load<!kTA, kVA>(rsa, abase, apitch, k_begin + 8 * j + 4 * half, k_end, a[j]);
+        small_load<kTB, kVB>(rsb, bbase, bpitch, k_begin + 8 * j + 4 * half, k_end, b[j]);
+        __builtin_amdgcn_sched_barrier(0);   // in this order: the first step's operands are waited for first
+    }
+    // Whole rounds of kSmallDepth steps without a branch inside (a branch per step made the compiler wait for every
+    // load in flight at the top of the loop), then the steps left over, whose operands are in their registers or on
+    // their way already.
+    const int whole = nsteps / kSmallDepth * kSmallDepth;
+    for (int s = 0; s < whole; s += kSmallDepth) {
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                a[e] = an[e];
-                b[e] = bn[e];
-            }
+        for (int j = 0; j < kSmallDepth; j++) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j][e], b[j][e], acc, 0, 0, 0);
+            const int kk = k_begin + 8 * (s + j + kSmallDepth) + 4 * half;   // this register set's next step
+            small_load<!kTA, kVA>(rsa, abase, apitch, kk, k_end, a[j]);
+            small_load<kTB, kVB>(rsb, bbase, bpitch, kk, k_end, b[j]);
+            __builtin_amdgcn_sched_barrier(0);   // keep each refill behind its own step: sunk to the loop's end, all of them are waited for at once
         }
     }
+#pragma unroll
+    for (int j = 0; j < kSmallDepth - 1; j++)
+        if (whole + j < nsteps) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j][e], b[j][e], acc, 0, 0, 0);
+        }
 #pragma unroll
     for (int v = 0; v < 16; v++) red[wave][acc_row(v, lane) * 33 + r] = acc[v];
     __syncthreads();
@@ -728,7 +745,11 @@ Route sgemm_route(int transA, int transB, size_t M, size_t N, size_t K, bool pan
     // whose 128-wide tiles leave most CUs with one four-wavefront block (1024 x 1024 x 256: 11 against
     // 22 us; 2048 x 2048 x 128: 21 against 31 us); beyond that the tile engine's operand reuse wins.
     const size_t tiles32 = ceil_div(M, (size_t)32) * ceil_div(N, (size_t)32);
-    if (tiles32 <= 4096 && tiles32 * 64 * K * sizeof(float) <= ((size_t)256 << 20)) { r.kind = Route::kSmall; return r; }
+    if (tiles32 <= 4096 && tiles32 * 64 * K * sizeof(float) <= ((size_t)256 << 20) && M * K < ((size_t)1 << 29) &&
+        K * N < ((size_t)1 << 29)) {   // (32-bit byte offsets into either operand)
+        r.kind = Route::kSmall;
+        return r;
+    }
     const bool big = M > 64;
     const size_t BM = big ? 128 : 64, BN = big ? 128 : 256;
     const size_t tiles = ceil_div(M, BM) * ceil_div(N, BN);
@@ -804,19 +825,20 @@ int sgemm_epilogue(int transA, int transB, size_t M, size_t N, size_t K, const f
     if (kind == Route::kSmall) {
         const int lda = (int)(transA ? M : K), ldb = (int)(transB ? K : N);
         int kslice = (int)ceil_div(ceil_div(K, (size_t)kSmallWaves), (size_t)8) * 8;
-        const bool vec = aligned16(A) && aligned16(B) && lda % 4 == 0 && ldb % 4 == 0;
+        // 128-bit loads for a k-contiguous operand whose rows start on 16-byte boundaries
+        const bool va = !transA && aligned16(A) && lda % 4 == 0, vb = transB && aligned16(B) && ldb % 4 == 0;
         const dim3 grid((unsigned)ceil_div(N, (size_t)32), (unsigned)ceil_div(M, (size_t)32)), block(64 * kSmallWaves);
-#define DOPT_SMALL(TA, TB)                                                                                             \
-    do {                                                                                                               \
-        if (vec) hipLaunchKernelGGL((sgemm_small_k<TA, TB, true>), grid, block, 0, stream(), (int)M, (int)N, (int)K, lda, \
-                                    ldb, kslice, A, B, C, colbias, bias_shift, rowvec, relu, ex.mask);                    \
-        else hipLaunchKernelGGL((sgemm_small_k<TA, TB, false>), grid, block, 0, stream(), (int)M, (int)N, (int)K, lda,  \
-                                ldb, kslice, A, B, C, colbias, bias_shift, rowvec, relu, ex.mask);                       \
-    } while (0)
-        if (transA && transB) DOPT_SMALL(true, true);
-        else if (transA) DOPT_SMALL(true, false);
-        else if (transB) DOPT_SMALL(false, true);
-        else DOPT_SMALL(false, false);
+#define DOPT_SMALL(TA, TB, VA, VB)                                                                                       \
+    hipLaunchKernelGGL((sgemm_small_k<TA, TB, VA, VB>), grid, block, 0, stream(), (int)M, (int)N, (int)K, lda, ldb, kslice, \
+                       A, B, C, colbias, bias_shift, rowvec, relu, ex.mask)
+        if (transA && transB) { if (vb) DOPT_SMALL(true, true, false, true); else DOPT_SMALL(true, true, false, false); }
+        else if (transA) DOPT_SMALL(true, false, false, false);
+        else if (transB) {
+            if (va && vb) DOPT_SMALL(false, true, true, true);
+            else if (va) DOPT_SMALL(false, true, true, false);
+            else if (vb) DOPT_SMALL(false, true, false, true);
+            else DOPT_SMALL(false, true, false, false);
+        } else { if (va) DOPT_SMALL(false, false, true, false); else DOPT_SMALL(false, false, false, false); }
 #undef DOPT_SMALL
         DOPT_LAUNCH_CHECK();
         *biased = true;   // whatever epilogue was asked for (the extras included), this kernel applied it
