@@ -147,8 +147,8 @@ def secondary(cfg, a):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", type=int, default=4, choices=[1, 2, 3, 4, 5])
     ap.add_argument("--unfused", action="store_true", help="run the reference's op-graph optimizer instead of the fused kernel")
     ap.add_argument("--no-views", action="store_true", help="disable the copy-eliding plan rewrites")
