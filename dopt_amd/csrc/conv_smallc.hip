@@ -101,15 +101,13 @@ __global__ __launch_bounds__(512) void smallc_fwd_k(SmallC p)
             if ((int)threadIdx.x + u * nthreads < count) ws[threadIdx.x + u * nthreads] = v[u];
     }
     load_patch<2>(p, n, p0, p.G * p.RT, nthreads, xs);
-    float bv[16];   // accumulators start at the bias of their row
-#pragma unroll
-    for (int v = 0; v < 16; v++) {
-        const int k = k0 + acc_row(v, lane);
-        bv[v] = p.bias ? p.bias[min(k, p.K - 1)] : 0.0f;
-    }
+    // Pixels are the rows of the MFMA tile and output channels its columns, so a lane ends up with four consecutive
+    // pixels of ONE channel in four consecutive accumulators: a 16-byte store (with channels as rows a lane held four
+    // channels of one pixel, sixteen 4-byte stores per column; the store unit takes as long for the one as for the other).
+    const float bv = p.bias ? p.bias[min(k0 + r32, p.K - 1)] : 0.0f;   // accumulators start at the bias of their channel
     __syncthreads();
 
-    // the filter as MFMA A operands: lane (i, half) holds w for row k0 + i, step kk = 2 t + half
+    // the filter as MFMA B operands: lane (i, half) holds w for channel k0 + i, step kk = 2 t + half
     float aw[kSteps];
     int koff[kSteps];
 #pragma unroll
@@ -125,21 +123,21 @@ __global__ __launch_bounds__(512) void smallc_fwd_k(SmallC p)
     // column drain while the next one multiplies (with all four columns multiplied first and stored last,
     // every wavefront of the chip computed at the same time and then wrote at the same time).
     const size_t plane = (size_t)p.H * p.W;
-    float *out = p.y + ((size_t)n * p.K + k0) * plane + (size_t)p0 * p.W + wave * kPix + r32;
+    float *out = p.y + ((size_t)n * p.K + k0 + r32) * plane + (size_t)p0 * p.W + wave * kPix + 4 * half;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const int px = wave * kPix + j * 32 + r32;
         const int poff = (px >> p.wshift) * (p.W + 2) + (px & (p.W - 1));
         v16f acc;
 #pragma unroll
-        for (int v = 0; v < 16; v++) acc[v] = bv[v];
+        for (int v = 0; v < 16; v++) acc[v] = bv;
 #pragma unroll
         for (int t = 0; t < kSteps; t++)
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(aw[t], xs[poff + koff[t]], acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xs[poff + koff[t]], aw[t], acc, 0, 0, 0);
+        if (r32 < krows) {
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const int kr = acc_row(v, lane);
-            if (kr < krows) out[(size_t)kr * plane + j * 32] = acc[v];
+            for (int g = 0; g < 4; g++)   // accumulators 4g .. 4g + 3: pixels 8g + 4 half .. + 3 of the column
+                *(float4 *)(out + j * 32 + 8 * g) = make_float4(acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]);
         }
     }
 }
