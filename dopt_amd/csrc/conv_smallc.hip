@@ -284,7 +284,7 @@ int conv_smallc_fwd(const dopt_hip_conv_desc *d, const float *x, const float *w,
 {
     SmallC p{};
     *done = false;
-    if (!smallc_setup(d, &p) || !aligned16(x)) return DOPT_HIP_OK;
+    if (!smallc_setup(d, &p) || !aligned16(x) || !aligned16(y)) return DOPT_HIP_OK;   // 16-byte loads of x, stores of y
     p.x = x; p.w = w; p.bias = bias; p.y = y;
     p.G = 1;
     for (int g = 2; g <= 8; g++)

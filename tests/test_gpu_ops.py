@@ -386,6 +386,43 @@ def test_convolution_all_three(case):
     assert_close(dw, O.conv_bwd_filter(dys, x, w.shape, pad, st), "conv bwd-filter, mean-loss gradient")
 
 
+@pytest.mark.parametrize("case", [(4, 3, 32, 32, 64), (4, 3, 16, 16, 16),      # first-layer kernels
+                                  (4, 64, 16, 16, 128), (8, 128, 8, 8, 128),  # patch kernels
+                                  (32, 128, 2, 2, 128), (3, 5, 7, 7, 6)])     # 2 x 2 images; the generic kernels
+def test_convolution_operands_off_the_16_byte_grid(case):
+    """Every operand and every result one float past a 16-byte boundary: kernels that load or store 128 bits at a
+    time have to step aside (or handle it), and nothing may write outside its result."""
+    N, C, H, W, K = case
+    r = rng(N + C + H + K)
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+    w = (r.standard_normal((K, C, 3, 3)) * np.sqrt(2.0 / (C * 9))).astype(np.float32)
+    dy = r.standard_normal((N, K, H, W)).astype(np.float32)
+    b = r.standard_normal(K).astype(np.float32)
+
+    def off(a):   # the array one element into a buffer, with a guard element on either side
+        t = T(np.concatenate([[7.0], a.ravel(), [7.0]]).astype(np.float32))
+        return t, t.view(1, a.shape)
+
+    def result(shape):
+        t = T(np.full(int(np.prod(shape)) + 2, 7.0, np.float32))
+        return t, t.view(1, shape)
+
+    (_, xo), (_, wo), (_, dyo), (_, bo) = off(x), off(w), off(dy), off(b)
+    pad, st = (1, 1), (1, 1)
+    for name, want, run in (
+            ("forward", O.convolution(x, w, pad, st), lambda o: ops.convolution(xo, wo, pad, st, out=o)),
+            ("forward + bias", O.convolution(x, w, pad, st) + b[None, :, None, None],
+             lambda o: ops.convolution_bias(xo, wo, bo, pad, st, out=o)),
+            ("backward-data", O.conv_bwd_data(dy, w, x.shape, pad, st), lambda o: ops.conv_bwd_data(dyo, wo, x.shape, pad, st, out=o)),
+            ("filter gradient", O.conv_bwd_filter(dy, x, w.shape, pad, st),
+             lambda o: ops.conv_bwd_filter(dyo, xo, w.shape, pad, st, out=o))):
+        whole, view = result(want.shape)
+        run(view)
+        got = whole.numpy()
+        assert got[0] == 7.0 and got[-1] == 7.0, name
+        assert_close(got[1:-1].reshape(want.shape), want, "%s %s" % (name, case), scale=np.sqrt(N * H * W) if "filter" in name else 1.0)
+
+
 def test_convolution_matches_reference_cpu_kernel_on_same_shapes():
     # the reference CPU kernel (fp32, its own loop order) is a valid oracle when out dims == in dims
     r = rng(41)
@@ -849,3 +886,57 @@ def test_sgemm_transposed_operands(shape, ta, tb):
     # matrix-vector kernels sum in a different order when the matrix is read the other way)
     if min(M, N, K) > 1:
         assert np.array_equal(got.numpy(), ops.matmul(T(a), T(b)).numpy())
+
+
+# ----------------------------------------------------------------------------- operands off the 16-byte grid
+def _off(a):
+    """(whole buffer, view one element in): the array with a guard element on either side."""
+    t = T(np.concatenate([[7.0], np.asarray(a, np.float32).ravel(), [7.0]]).astype(np.float32))
+    return t, t.view(1, np.shape(a))
+
+
+@pytest.mark.parametrize("shape", [(8, 16, 8, 8), (16, 64, 32, 32), (4, 6, 6, 10), (64, 128, 2, 2)])
+def test_entry_points_with_every_operand_off_the_16_byte_grid(shape):
+    """Each tensor one float past a 16-byte boundary: the 128-bit kernels have to step aside, results equal those of
+    the aligned call (to rounding where another kernel adds in another order), and nothing is written outside a result."""
+    r = rng(sum(shape))
+    N, Cc, H, W = shape
+    x = r.standard_normal(shape).astype(np.float32)
+    dy = r.standard_normal(shape).astype(np.float32)
+    sc, bi = r.uniform(0.5, 1.5, Cc).astype(np.float32), r.standard_normal(Cc).astype(np.float32)
+    rm, rv = r.standard_normal(Cc).astype(np.float32), r.uniform(0.5, 1.5, Cc).astype(np.float32)
+    dp = r.standard_normal((N, Cc, H // 2, W // 2)).astype(np.float32)
+    flat = x.reshape(N * Cc, H * W)
+    n = x.size
+    cases = [
+        ("relu", (n,), lambda t, o: ops.relu(t(x), out=o)),
+        ("reluGrad", (n,), lambda t, o: ops.relu_grad(t(dy), t(x), out=o)),
+        ("addBias", shape, lambda t, o: ops.add_bias(t(x), t(bi), out=o)),
+        ("addBiasGrad", (Cc,), lambda t, o: ops.add_bias_grad(t(dy), out=o)),
+        ("maxpool", dp.shape, lambda t, o: ops.maxpool(t(x), (2, 2), out=o)),
+        ("maxpoolGrad", shape, lambda t, o: ops.maxpool_grad(t(dp), t(x), (2, 2), out=o)),
+        ("softmax", flat.shape, lambda t, o: ops.softmax(t(flat), out=o)),
+        ("softmaxGrad", flat.shape, lambda t, o: ops.softmax_grad(t(dy.reshape(flat.shape)), t(np.abs(flat)), out=o)),
+        ("batchNormTrain", (n + 2 * Cc,), lambda t, o: ops.bn_train(t(x), t(sc), t(bi), t(rm), t(rv), 0.9, out=o)),
+        ("batchNormTrain+relu", (n + 2 * Cc,), lambda t, o: ops.bn_train_relu(t(x), t(sc), t(bi), t(rm), t(rv), 0.9, out=o)),
+        ("batchNormGrad", (n + 2 * Cc,), lambda t, o: ops.bn_grad(t(dy), t(x), t(sc), out=o)),
+        ("reluGrad+batchNormGrad", (n + 2 * Cc,), lambda t, o: ops.bn_grad_relu(t(dy), t(np.maximum(x, 0)), t(x), t(sc), out=o)),
+        ("batchNormInference", shape, lambda t, o: ops.bn_infer(t(x), t(sc), t(bi), t(rm), t(rv), out=o)),
+        ("sum over all", (), lambda t, o: ops.sum(t(x), None, out=o)),
+        ("sum over [0,2,3]", (Cc,), lambda t, o: ops.sum(t(x), [0, 2, 3], out=o)),
+        ("sum over [1]", (N, H, W), lambda t, o: ops.sum(t(x), [1], out=o)),
+        ("maxElement over [2,3]", (N, Cc), lambda t, o: ops.max_element(t(x), [2, 3], out=o)),
+        ("transpose", flat.shape[::-1], lambda t, o: ops.transpose(t(flat), out=o)),
+        ("slice", (N, Cc, H - 1, W - 1), lambda t, o: ops.slice(t(x), [0, 0, 1, 0], [N, Cc, H, W - 1], out=o)),
+        ("pad", (N, Cc, H + 1, W + 2), lambda t, o: ops.pad(t(x), [0, 0, 1, 1], [0, 0, 0, 1], out=o)),
+        ("repeat", (N, Cc, 2 * H, W), lambda t, o: ops.repeat(t(x), [1, 1, 2, 1], out=o)),
+        ("matmul", (N * Cc, N * Cc), lambda t, o: ops.matmul_t(t(flat), t(flat), False, True, out=o)),
+    ]
+    for name, oshape, run in cases:
+        want = run(lambda a: T(np.asarray(a, np.float32)), None).numpy()
+        size = int(np.prod(oshape)) if oshape != () else 1
+        whole = T(np.full(size + 2, 7.0, np.float32))
+        run(lambda a: _off(a)[1], whole.view(1, want.shape))
+        got = whole.numpy()
+        assert got[0] == 7.0 and got[-1] == 7.0, name
+        assert_close(got[1:-1].reshape(want.shape), want, "%s %s" % (name, shape), scale=max(1.0, float(np.abs(want).max())))
