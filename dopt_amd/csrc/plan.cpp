@@ -14,6 +14,7 @@
 #include "plan.h"
 
 #include <atomic>
+#include <cstdio>
 #include <cstdlib>
 #include <random>
 
@@ -1610,7 +1611,9 @@ int HIPPlan::Builder::assignQueues()
             int a = -1;
             for (int pr : producers[i]) {
                 int at = side[(size_t)pr] ? anchorOf[(size_t)pr] : pr;
-                if (!side[(size_t)pr] && glued[(size_t)pr]) at += 1;
+                // (the step behind a convolution stays with it only if it stays on the main queue itself: a relu
+                // that moves to the side queue is no anchor - what is placed behind it would never be emitted)
+                if (!side[(size_t)pr] && glued[(size_t)pr] && !side[(size_t)pr + 1]) at += 1;
                 a = std::max(a, at);
             }
             anchorOf[i] = a;
@@ -1634,6 +1637,7 @@ int HIPPlan::Builder::assignQueues()
                 ordered.push_back(std::move(st));
             }
         }
+        if (ordered.size() != n) return fail(DOPT_HIP_ERR_RUNTIME, "plan: %zu of %zu steps placed on the two queues", ordered.size(), n);
         p->mSteps = std::move(ordered);
         if (any) {
             p->mUsesSide = true;
@@ -1704,6 +1708,16 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
     if (flags & (DOPT_HIP_PLAN_OVERLAP | DOPT_HIP_PLAN_OVERLAP_LIGHT))
         if (int rc = b.assignQueues()) return rc;
     if (int rc = b.createEvents()) return rc;
+    if (const char *dump = std::getenv("DOPT_HIP_PLAN_DUMP")) {   // the steps as they will run: queue, label, operation, inputs
+        if (dump[0] && dump[0] != '0')
+            for (size_t i = 0; i < p->mSteps.size(); i++) {
+                const Step &st = p->mSteps[i];
+                std::fprintf(stderr, "plan step %3zu queue %d%s%s %-44s op %d <-", i, st.lane, st.fenceBefore ? " (waits)" : "",
+                             st.joinSide ? " (joins)" : "", st.label.c_str(), st.op);
+                for (int in : st.inputOps) std::fprintf(stderr, " %d", in);
+                std::fprintf(stderr, "\n");
+            }
+    }
     // Resolve aliases once against the variables' own values so that result() is meaningful before
     // the first execution (an alias of a variable that is later passed as an argument moves with it).
     if (int rc = p->resolve(0, nullptr, nullptr, nullptr)) return rc;

@@ -93,6 +93,9 @@ enum {
                                  it would otherwise follow one launch latency at a time. */
 };
 
+/* With DOPT_HIP_PLAN_DUMP=1 in the environment, dopt_hip_plan_create prints the plan's steps to stderr as they will
+   run: position, queue, profiler label, operation id and the operations whose buffers the kernel reads. */
+
 /* new CUDAPlan(outputs) (cuda/package.d:267-312): topological sort, one kernel object per
    operation (constructed through the registry), one zero-filled device buffer per operation
    (`reshape` aliases its dependency, `constant` is uploaded once). */
