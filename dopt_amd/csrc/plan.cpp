@@ -1590,8 +1590,12 @@ int HIPPlan::Builder::assignQueues()
         for (size_t i = n; i-- > 0;) {   // readers come later in the order, so they are decided first
             const Step &st = p->mSteps[i];
             if (st.op < 0 || biasGradOf[st.op] >= 0 || producers[i].empty()) continue;
+            // by label: a fused step carries the operation it ends in (convolution+addBias ends in an addBias), and a
+            // convolution must stay behind the step that packs its filter
             const std::string &t = g.ops[st.op].opType;
-            if (t.compare(0, 11, "convolution") == 0 || t.compare(0, 9, "batchNorm") == 0 || t == "uniform") continue;
+            if (st.label.find("convolution") != std::string::npos || st.label.find("batchNorm") != std::string::npos ||
+                t.compare(0, 11, "convolution") == 0 || t.compare(0, 9, "batchNorm") == 0 || t == "uniform")
+                continue;
             size_t bytes = g.ops[st.op].bytes();
             for (size_t b : st.inputBytes) bytes += b;
             bool off = bytes <= kLightBytes;

@@ -5,7 +5,8 @@ a batch norm in between).  Loss, predictions, every parameter gradient and the r
 with the CPU evaluator, and the plans with rewrites against the plan without them: the rewrites are pattern
 matches on the graph, and a pattern that fires on a neighbourhood it was not written for shows up here.
 (Found this way: a transpose folded into a product whose kernel then summed in another order; the steps behind a
-convolution without batch norm dropped from plans that move small steps to the second queue.)
+convolution without batch norm dropped from plans that move small steps to the second queue, and fused
+convolution + bias steps moved there ahead of the step that packs their filter.)
 """
 import numpy as np
 import pytest
@@ -206,3 +207,23 @@ def test_random_networks_fused_updaters_follow_the_op_graph_updaters(seed):
         assert graph[2] == fusedrun[2], (seed, flags, graph[2], fusedrun[2])
         for i, (a, b) in enumerate(zip(graph[3], fusedrun[3])):
             assert np.array_equal(a, b), (seed, flags, i, a.shape)
+
+
+@pytest.mark.parametrize("seed", range(150))
+def test_random_networks_inference_plans_in_every_mode(seed):
+    """The inference output alone: every step of such a plan leads to its one output, so the second-queue mode for small
+    steps moves whole tails of the network.  The FIRST execution is compared as well as later ones: a convolution that
+    ran ahead of the step packing its filter read an empty packed copy once and was right from then on."""
+    r = np.random.default_rng(9000 + seed)
+    n, size, cin = int(r.choice([4, 8, 16])), int(r.choice([8, 16])), int(r.choice([3, 16]))
+    X = r.standard_normal((n, cin, size, size)).astype(np.float32)
+    feats = float32([n, cin, size, size])
+    preds = _random_net(r, feats)
+    want = core.compile([preds.output], 0).execute({feats: X})[0]
+    assert np.isfinite(want).all()
+    for flags in (core.PLAN_VIEWS, REWRITES, REWRITES | core.PLAN_GRAPH, REWRITES | core.PLAN_OVERLAP_LIGHT,
+                  REWRITES | core.PLAN_OVERLAP, core.PLAN_OVERLAP_LIGHT):
+        plan = core.compile([preds.output], flags)
+        for rep in range(3):
+            assert np.array_equal(plan.execute({feats: X})[0], want), (seed, flags, rep)
+        plan.cleanup()
