@@ -420,12 +420,14 @@ int dopt_hip_pad(int rank, const size_t *in_shape, const size_t *out_shape, cons
                  const void *in, void *out)
 {
     DOPT_REQUIRE(rank >= 0 && rank <= kMaxRank, "dopt_hip_pad: rank %d not supported (max %d)", rank, kMaxRank);
-    DOPT_REQUIRE(in && out && (rank == 0 || (in_shape && out_shape && before)), "dopt_hip_pad: null argument");
+    DOPT_REQUIRE(rank == 0 || (in_shape && out_shape && before), "dopt_hip_pad: null argument");
     for (int i = 0; i < rank; i++)
         DOPT_REQUIRE(before[i] + in_shape[i] <= out_shape[i], "dopt_hip_pad: axis %d: input does not fit the output", i);
-    DOPT_ENSURE_INIT();
     size_t total = volume(out_shape, rank);
     if (total == 0) return DOPT_HIP_OK;
+    // (an empty input has no buffer: the result is all padding)
+    DOPT_REQUIRE(out && (in || volume(in_shape, rank) == 0), "dopt_hip_pad: null argument");
+    DOPT_ENSURE_INIT();
     if (rank == 0) return copy_contiguous((const uint32_t *)in, (uint32_t *)out, 1);
     if (int rc = try_map32<kPad>(rank, in_shape, out_shape, before, in, out); rc >= 0) return rc;
     NdDesc d{};
@@ -445,7 +447,8 @@ int dopt_hip_pad(int rank, const size_t *in_shape, const size_t *out_shape, cons
 int dopt_hip_repeat(int rank, const size_t *in_shape, const size_t *reps, const void *in, void *out)
 {
     DOPT_REQUIRE(rank >= 0 && rank <= kMaxRank, "dopt_hip_repeat: rank %d not supported (max %d)", rank, kMaxRank);
-    DOPT_REQUIRE(in && out && (rank == 0 || (in_shape && reps)), "dopt_hip_repeat: null argument");
+    DOPT_REQUIRE(rank == 0 || (in_shape && reps), "dopt_hip_repeat: null argument");
+    DOPT_REQUIRE((in && out) || volume(in_shape, rank) == 0, "dopt_hip_repeat: null argument");   // an empty tensor has no buffer
     DOPT_ENSURE_INIT();
     NdDesc d{};
     d.rank = rank;

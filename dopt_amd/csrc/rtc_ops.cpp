@@ -9,6 +9,7 @@
 #include <vector>
 
 #include "common.h"
+#include <limits>
 
 namespace {
 
@@ -561,9 +562,9 @@ int dopt_hip_pointwise(const char *op, int dtype, size_t n, const void *a, const
     const OpInfo *info = find_op(op);
     if (!info) return fail(DOPT_HIP_ERR_UNSUPPORTED, "dopt_hip_pointwise: unknown operation '%s'", op);
     if (int rc = check_dtype(dtype)) return rc;
+    if (n == 0) return DOPT_HIP_OK;   // empty tensors have no buffers: nothing to check them against
     DOPT_REQUIRE((info->arity == 2) == (b != nullptr), "dopt_hip_pointwise: '%s' takes %d operand(s)", op,
                  info->arity);
-    if (n == 0) return DOPT_HIP_OK;
     DOPT_REQUIRE(a && out, "dopt_hip_pointwise: null operand");
     DOPT_ENSURE_INIT();
     bool vec = aligned16(a) && aligned16(out) && (!b || aligned16(b));
@@ -661,7 +662,7 @@ int dopt_hip_pointwise_arity(const char *op)
 int dopt_hip_reduce(const char *op, int dtype, const size_t *shape, int rank, const size_t *axes, int naxes,
                     const void *in, void *out)
 {
-    DOPT_REQUIRE(op && shape && axes && in && out, "dopt_hip_reduce: null argument");
+    DOPT_REQUIRE(op && shape && axes, "dopt_hip_reduce: null argument");
     bool is_sum = !strcmp(op, "sum");
     if (!is_sum && strcmp(op, "maxElement"))
         return fail(DOPT_HIP_ERR_UNSUPPORTED, "dopt_hip_reduce: unknown reduction '%s'", op);
@@ -678,7 +679,23 @@ int dopt_hip_reduce(const char *op, int dtype, const size_t *shape, int rank, co
         cur[i] = shape[i];
         vol *= shape[i];
     }
-    if (vol == 0) return DOPT_HIP_OK;
+    if (vol == 0) {
+        // Nothing to fold.  Where only reduced axes are empty the result still has elements: the fold's start value
+        // (cpu/math.d:90-247 starts a sum at 0 and a maximum at -T.max).
+        size_t kept = 1;
+        for (int i = 0; i < rank; i++)
+            if (!reduced[i]) kept *= shape[i];
+        if (kept == 0) return DOPT_HIP_OK;
+        DOPT_REQUIRE(out != nullptr, "dopt_hip_reduce: null argument");
+        if (is_sum) return dopt_hip_memset(out, 0, kept * 4);
+        std::vector<uint32_t> start(kept);
+        const float lowest = -std::numeric_limits<float>::max();
+        uint32_t bits;
+        std::memcpy(&bits, &lowest, 4);
+        for (uint32_t &v : start) v = dtype == DOPT_HIP_F32 ? bits : (uint32_t)(-std::numeric_limits<int32_t>::max());
+        return dopt_hip_copy_h2d(out, start.data(), kept * 4);
+    }
+    DOPT_REQUIRE(in && out, "dopt_hip_reduce: null argument");
     DOPT_ENSURE_INIT();
 
     // Runs of adjacent reduced axes collapse into one (outer, R, inner) pass each, last run first.

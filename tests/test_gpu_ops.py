@@ -940,3 +940,26 @@ def test_entry_points_with_every_operand_off_the_16_byte_grid(shape):
         got = whole.numpy()
         assert got[0] == 7.0 and got[-1] == 7.0, name
         assert_close(got[1:-1].reshape(want.shape), want, "%s %s" % (name, shape), scale=max(1.0, float(np.abs(want).max())))
+
+
+def test_empty_tensors_are_no_ops_and_empty_folds_give_the_start_value():
+    """Tensors without elements have no buffer (a 0-byte allocation is a null pointer): entry points take them as
+    they are.  A reduction whose reduced axes are empty still fills its result, with the value the reference's fold
+    starts from (cpu/math.d:183-187: 0 for sum, -T.max for maxElement)."""
+    e = ops.Tensor((0, 4))
+    assert ops.pointwise("add", e, ops.Tensor((0, 4))).shape == (0, 4)
+    assert ops.relu(e).shape == (0, 4)
+    assert np.array_equal(ops.sum(e, [0]).numpy(), np.zeros(4, np.float32))
+    assert np.array_equal(ops.max_element(e, [0]).numpy(), np.full(4, -np.finfo(np.float32).max, np.float32))
+    ei = ops.Tensor((3, 0), np.int32)
+    assert np.array_equal(ops.sum(ei, [1]).numpy(), np.zeros(3, np.int32))
+    assert np.array_equal(ops.max_element(ei, [1]).numpy(), np.full(3, -np.iinfo(np.int32).max, np.int32))
+    assert ops.sum(e, [1]).shape == (0,)
+    assert np.array_equal(ops.pad(e, [1, 0], [1, 0]).numpy(), np.zeros((2, 4), np.float32))
+    assert ops.repeat(e, [2, 3]).shape == (0, 12)
+    assert ops.matmul(ops.Tensor((3, 0)), ops.Tensor((0, 5))).numpy().tolist() == np.zeros((3, 5)).tolist()
+    from dopt_amd import core
+    a, b = core.float32([0, 4]), core.float32([0, 4])
+    for flags in (0, core.PLAN_VIEWS | core.PLAN_FUSE):
+        got = core.compile([a + b, core.sum(a * b), core.sum(a + b, [0])], flags).execute()
+        assert got[0].shape == (0, 4) and got[1] == 0.0 and np.array_equal(got[2], np.zeros(4, np.float32))
