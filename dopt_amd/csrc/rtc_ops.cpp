@@ -480,7 +480,10 @@ std::string reduce_source(bool is_sum, int dtype)
         s += f ? "#define COMBINE a + b\n" : "#define COMBINE (int)((unsigned)a + (unsigned)b)\n";
         s += "#define IDENT 0\n";
     } else {
-        s += "#define COMBINE (a < b ? b : a)\n";
+        // The reference folds max(acc, element) = acc < element ? element : acc from -T.max, which passes over a NaN
+        // element (cpu/math.d:183-187).  Here elements also meet each other first (the four of a 128-bit load, the
+        // lanes of a wavefront), so a NaN on the left has to give way as well, or it would hide its partners.
+        s += "#define COMBINE (a < b || a != a ? b : a)\n";
         // identity -T.max (cpu/math.d:186): int32 starts at -INT_MAX, not INT_MIN
         s += f ? "#define IDENT -3.402823466e+38f\n" : "#define IDENT -2147483647\n";
     }

@@ -963,3 +963,23 @@ def test_empty_tensors_are_no_ops_and_empty_folds_give_the_start_value():
     for flags in (0, core.PLAN_VIEWS | core.PLAN_FUSE):
         got = core.compile([a + b, core.sum(a * b), core.sum(a + b, [0])], flags).execute()
         assert got[0].shape == (0, 4) and got[1] == 0.0 and np.array_equal(got[2], np.zeros(4, np.float32))
+
+
+@pytest.mark.parametrize("shape,axes", [((1000,), [0]), ((64, 300), [1]), ((64, 300), [0]), ((8, 16, 32), [0, 2]),
+                                        ((5, 7), [0, 1]), ((100000,), [0]), ((33, 4096), [1])])
+def test_max_element_passes_over_nans_like_the_reference_fold(shape, axes):
+    """max(acc, x) = acc < x ? x : acc started at -T.max never takes a NaN (cpu/math.d:183-187): the result is the
+    largest number, and -T.max where there is none.  In a tree of partial maxima a NaN must not hide the numbers
+    it was paired with."""
+    r = rng(len(shape) * 10 + axes[0])
+    x = r.standard_normal(shape).astype(np.float32)
+    x.ravel()[::7] = np.nan
+    x.ravel()[:3] = np.nan
+    want = O.max_element(x, axes)
+    assert not np.isnan(want).any()
+    assert np.array_equal(want, np.nanmax(x, axis=tuple(axes)))
+    assert np.array_equal(ops.max_element(T(x), axes).numpy(), want)
+    allnan = np.full(shape, np.nan, np.float32)
+    got = ops.max_element(T(allnan), axes).numpy()
+    assert np.array_equal(got, np.full(got.shape, -np.finfo(np.float32).max, np.float32))
+    assert np.array_equal(got, O.max_element(allnan, axes))
