@@ -84,7 +84,7 @@ private class FusedUpdater
             }
         }
 
-        mPlan = new NativeHIPPlan(outputs ~ grads ~ planProj, defaultPlanFlags);
+        mPlan = new HIPPlan(outputs ~ grads ~ planProj, defaultPlanFlags);
 
         //Outputs are copied out, gradients are read in place, projected statistics go straight over their variables
         mRets = outputs.map!(x => allocate(x.volume * x.elementType.sizeOf)).array();
@@ -93,7 +93,7 @@ private class FusedUpdater
 
         if(postProj.length != 0)
         {
-            mPostPlan = new NativeHIPPlan(postProj, defaultPlanFlags);
+            mPostPlan = new HIPPlan(postProj, defaultPlanFlags);
             mPostRets = postTarget.map!(x => x.value).array();
         }
 
@@ -181,7 +181,7 @@ private class FusedUpdater
     Operation[] mHyper;
     bool mNesterov;
     float mB1 = 1.0f, mB2 = 1.0f;   //the running products beta^t of online/adam.d:44-46
-    NativeHIPPlan mPlan, mPostPlan;
+    HIPPlan mPlan, mPostPlan;
     DeviceBuffer[] mRets, mPostRets;
     HIPBuffer[] mState;
     void *mHandle;

@@ -6,13 +6,12 @@
     $(D deregisterHIPKernel), $(D listHIPOperations).  Importing this module installs the backend as dopt's default
     evaluator, compiler and variable allocator, exactly as importing $(D dopt.cuda) does.
 
-    Two plans exist.  $(D HIPPlan) is the reference's loop: one kernel object per operation, built through the D
-    registry, executed in topological order (the kernel classes live in dopt.hip.basic / math / nnet / random and
-    each make one call into the kernel library).  $(D NativeHIPPlan) hands the whole graph to the planner inside
-    libdopthip.so (include/dopt_hip_plan.h), which runs the same kernels and can apply its result-preserving rewrites
-    (views, fused pairs, pointwise chains, graph replay); it is what $(D compile) returns unless
-    $(D useNativePlanner) is cleared.  Kernels registered from D work in both: the native planner calls them back
-    through a C trampoline.
+    There is one plan class.  $(D HIPPlan) hands the whole graph to the planner inside libdopthip.so
+    (include/dopt_hip_plan.h), which owns the topological order, the per-operation buffers and the kernel objects and
+    can apply its rewrites (views, fused pairs, pointwise chains, graph replay).  The kernel classes of
+    dopt.hip.basic / math / nnet / random each make one call into the kernel library; they exist so that D code can
+    construct and run a single kernel the way it does with $(D dopt.cuda), and so that the D registry lists every
+    operation.  Kernels registered from D take part in plans too: the planner calls them back through a C trampoline.
 
     Written where no D compiler exists (the library's build image has none): this package has never been compiled.
 
@@ -37,9 +36,6 @@ alias HIPKernelCtr = HIPKernel delegate(Operation op);
 
 /// Rewrites the native planner applies unless told otherwise; see include/dopt_hip_plan.h.
 __gshared uint defaultPlanFlags = DOPT_HIP_PLAN_VIEWS | DOPT_HIP_PLAN_FUSE;
-
-/// When set (the default), $(D compile) returns a $(D NativeHIPPlan); otherwise a $(D HIPPlan).
-__gshared bool useNativePlanner = true;
 
 /**
     Turns a status code of the library into the exception the reference raises with $(D enforce).
@@ -85,12 +81,7 @@ shared static this()
         defaultEvaluator = toDelegate(&evaluateHIP);
         defaultCompiler = (Operation[] ops)
         {
-            if(useNativePlanner)
-            {
-                return cast(Plan)new NativeHIPPlan(ops, defaultPlanFlags);
-            }
-
-            return cast(Plan)new HIPPlan(ops);
+            return cast(Plan)new HIPPlan(ops, defaultPlanFlags);
         };
         defaultVarAllocator = (size_t numBytes) { return cast(DeviceBuffer)HIPBuffer.create(numBytes); };
     }
@@ -235,168 +226,10 @@ class HIPBuffer : DeviceBuffer
 }
 
 /**
-    The reference's plan, kernel object by kernel object (cuda/source/dopt/cuda/package.d:261-433).
-*/
-class HIPPlan : Plan
-{
-    public
-    {
-        long[string] profiler;
-
-        this(Operation[] outputs)
-        {
-            import std.array : array;
-
-            super(outputs);
-
-            auto sortedOps = topologicalSort(outputs);
-
-            foreach(o; sortedOps)
-            {
-                if(o.opType == "variable" || o.opType == "reshape" || o.opType == "constant")
-                {
-                    continue;
-                }
-
-                auto k = o.opType in mKernelCtrs;
-
-                //Every operation has a device kernel; there is no round trip through the CPU evaluator
-                enforce(k !is null, "Could not construct a HIP kernel for operation of type '" ~ o.opType ~ "'");
-
-                mKernels[o] = (*k)(o);
-            }
-
-            mOps = sortedOps.array;
-
-            foreach(o; mOps)
-            {
-                if(o.opType == "reshape")
-                {
-                    mResults[o] = mResults[o.deps[0]];
-                }
-                else
-                {
-                    mResults[o] = HIPBuffer.create(o.volume * o.elementType.sizeOf);
-
-                    if(o.opType == "constant")
-                    {
-                        mResults[o].set(o.value);
-                    }
-                }
-            }
-
-            mResults.rehash();
-        }
-
-        ~this()
-        {
-            cleanup();
-        }
-
-        /**
-            Releases the device memory of this plan.
-        */
-        void cleanup()
-        {
-            if(mClean)
-            {
-                return;
-            }
-
-            foreach(o; mOps)
-            {
-                if(o.opType != "reshape")
-                {
-                    HIPBuffer.destroy(mResults[o]);
-                }
-            }
-
-            mClean = true;
-        }
-    }
-
-    protected
-    {
-        override void executeImpl(DeviceBuffer[Operation] args, DeviceBuffer[] rets)
-        {
-            import std.datetime.stopwatch : StopWatch;
-            StopWatch sw;
-
-            foreach(o; args.keys)
-            {
-                enforce(o.opType == "variable",
-                    "All assignments in args must be for Operations with an opType of 'variable'");
-            }
-
-            foreach(o; mOps)
-            {
-                if(o.opType == "variable" || o.opType == "constant")
-                {
-                    continue;
-                }
-
-                HIPBuffer[] inputs;
-                HIPBuffer output = mResults[o];
-
-                foreach(d; o.deps)
-                {
-                    if(d.opType == "variable")
-                    {
-                        DeviceBuffer given = (d in args) ? args[d] : d.value;
-                        auto hipbuf = cast(HIPBuffer)given;
-
-                        if(hipbuf is null)
-                        {
-                            hipbuf = mResults[d];
-                            hipbuf.set(given);
-                        }
-
-                        inputs ~= hipbuf;
-                    }
-                    else
-                    {
-                        inputs ~= mResults[d];
-                    }
-                }
-
-                if(o.opType == "reshape")
-                {
-                    mResults[o] = inputs[0];
-                }
-                else
-                {
-                    //Everything is enqueued on one in-order queue; the host does not wait per kernel, so this is
-                    //enqueue time. Device time per kernel comes from NativeHIPPlan with DOPT_HIP_PLAN_TIMING.
-                    sw.reset();
-                    sw.start();
-                    mKernels[o].execute(inputs, output);
-                    sw.stop();
-
-                    profiler[o.opType] = profiler.get(o.opType, 0) + sw.peek.split.usecs;
-                }
-            }
-
-            foreach(i, o; mOutputs)
-            {
-                rets[i].set(mResults[o]);
-            }
-        }
-    }
-
-    private
-    {
-        Operation[] mOps;
-        HIPKernel[Operation] mKernels;
-        HIPBuffer[Operation] mResults;
-        bool mClean = false;
-    }
-}
-
-/**
     A plan executed by the planner inside libdopthip.so: the graph is handed over once, operation by operation
     (type, judged output type, dependencies, attributes), and executions are one call each.
 */
-class NativeHIPPlan : Plan
+class HIPPlan : Plan
 {
     public
     {
@@ -632,6 +465,9 @@ class NativeHIPPlan : Plan
     }
 }
 
+/// Kept for code written against the earlier name of the plan class.
+alias NativeHIPPlan = HIPPlan;
+
 /**
     Used for performing a one-off evaluation of a set of operations.
 
@@ -644,7 +480,7 @@ class NativeHIPPlan : Plan
 */
 DeviceBuffer[] evaluateHIP(Operation[] ops, DeviceBuffer[Operation] args = null)
 {
-    Plan p = useNativePlanner ? cast(Plan)new NativeHIPPlan(ops, 0) : cast(Plan)new HIPPlan(ops);
+    Plan p = new HIPPlan(ops, 0);
 
     return p.execute(args);
 }
@@ -700,7 +536,7 @@ private
 {
     HIPKernelCtr[string] mKernelCtrs;
     HIPKernelCtr[] mUserCtrs;
-    NativeHIPPlan tlsBuilding;
+    HIPPlan tlsBuilding;
 
     //A D kernel object kept alive for the planner, and the buffers it is handed on each execution
     class Trampolined
