@@ -4,7 +4,7 @@ CIFAR-shape network with batch norm at batch 128 in fp32, on one MI355X, through
 kernel library.  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config N] [--unfused] [--no-views] [--no-fuse]
-                    [--graph] [--no-cpu] [--no-kernel-timing]
+                    [--graph] [--no-cpu] [--no-feed] [--no-kernel-timing]
 
 A step is one execution of the update plan on device-resident synthetic inputs (inputs are in HBM
 before the timed region starts).  W warm-up steps, then EXACTLY K timed steps between two device
@@ -89,23 +89,93 @@ def cpu_baseline(seconds_budget=20.0):
             if nb == b:
                 break
             b = nb
-    # configuration 1 on the CPU evaluator: graph outputs = loss, predictions, new W, new b, new momenta
+    # configuration 1 on the CPU evaluator: graph outputs = loss, predictions, new W, new b, new momenta.  Timed twice:
+    # every kernel on one thread, and threaded the way the reference's CPU backend is (matmul through BLAS at its
+    # default thread count, cpu/math.d:77-82; sum / maxElement / repeat parallel over the outer index,
+    # cpu/math.d:102,179, cpu/basic.d:166)
     s1 = configs.softmax_regression(flags=0, host_args=True)
     outs = s1.updater.plan.outputs
-    evaluator.evaluate(outs, s1.args)
-    n1, t0 = 0, time.perf_counter()
-    while n1 < 3 or (time.perf_counter() - t0 < 2.0 and n1 < 200):
-        evaluator.evaluate(outs, s1.args)
-        n1 += 1
-    cfg1_ms = (time.perf_counter() - t0) / n1 * 1e3
-    return {"value": round(b / t_total, 3), "unit": "images/s", "cores": 1, "host_cores": host_cores(), "kind": "port",
+
+    def time_config1(blas):
+        evaluator.evaluate(outs, s1.args, blas=blas)
+        n, t0 = 0, time.perf_counter()
+        while n < 3 or (time.perf_counter() - t0 < 2.0 and n < 200):
+            evaluator.evaluate(outs, s1.args, blas=blas)
+            n += 1
+        return (time.perf_counter() - t0) / n * 1e3, n
+
+    cfg1_ms, n1 = time_config1(False)
+    cores = host_cores()
+    O.set_threads(cores)
+    try:
+        cfg1_thr_ms, n1t = time_config1(True)
+    finally:
+        O.set_threads(1)
+    try:
+        from threadpoolctl import threadpool_info
+        blas_threads = max([p.get("num_threads", 1) for p in threadpool_info() if p.get("user_api") == "blas"] or [1])
+    except Exception:
+        blas_threads = None
+    return {"value": round(b / t_total, 3), "unit": "images/s", "cores": 1, "host_cores": cores, "kind": "port",
             "sample": "conv-forward only: the 13 VGG-16 3x3 convolutions at batch %d through the C restatement of "
-                      "the reference's single-threaded CPU kernel (%.1f s); the reference CPU backend implements no "
-                      "backward, bias, ReLU or batch-norm kernels, so a full CPU training step does not exist" % (
-                          b, t_total),
+                      "the reference's single-threaded CPU kernel (%.1f s; cpu/nnet.d:20-87 has no parallel loop); the "
+                      "reference CPU backend implements no backward, bias, ReLU or batch-norm kernels, so a full CPU "
+                      "training step does not exist" % (b, t_total),
             "config1_step_ms": round(cfg1_ms, 3),
             "config1_sample": "%d whole softmax-regression steps ([100,784] -> 10, forward + backward + SGD) through the "
-                              "CPU evaluator, one restated reference kernel per operation, 1 thread" % n1}
+                              "CPU evaluator, one restated reference kernel per operation, 1 thread" % n1,
+            "config1_threaded_step_ms": round(cfg1_thr_ms, 3),
+            "config1_threaded_cores": {"blas": blas_threads, "reductions_and_repeat": cores},
+            "config1_threaded_sample": "%d of the same steps with the reference's own threading: matmul through OpenBLAS "
+                                       "(numpy) at its default thread count, sum / maxElement / repeat parallel over "
+                                       "the outer index on %d threads" % (n1t, cores)}
+
+
+def host_feed_leg(step, steps, warmup):
+    """The same step fed from host memory, as the reference's training loop runs it (examples/cifar10.d:118-140 fills
+    float[] batches on the host; CUDAPlan.executeImpl uploads every host argument on each execution,
+    cuda/package.d:367-401): a shuffled host dataset, mirrored-pad / random-crop / flip augmentation (ImageTransformer
+    with 4, 4, true, false as in the example), page-locked staging and queued uploads through data.DeviceFeed, then the
+    step.  Reported beside the headline figure, never as it."""
+    from dopt_amd import data, ops, workloads
+    rng = np.random.default_rng(3)
+    n = 8 * BATCH
+    X = rng.standard_normal((n, 3, 32, 32)).astype(np.float32)
+    Y = workloads.one_hot(rng.integers(0, 10, n), 10)
+    it = data.SupervisedBatchIterator(X, Y, [[3, 32, 32], [10]], shuffle=True, seed=4)
+    feed = data.DeviceFeed(it, BATCH, 4, 4, True, False, seed=5)
+    feats, labels = step.extra["feats"], step.extra["labels"]
+
+    def run(k):
+        for _ in range(k):
+            if feed.finished():
+                feed.restart()
+            f, l = feed.next()
+            step.updater.step_async({feats: f, labels: l})
+
+    run(max(warmup, 2))
+    ops.sync()
+    t0 = time.perf_counter()
+    run(steps)
+    ops.sync()
+    sec = (time.perf_counter() - t0) / steps
+    # and the reference's own way: pageable host arrays handed to the plan, uploaded (blocking) inside every execution
+    xs, ys = X[:BATCH].copy(), Y[:BATCH].copy()
+    for _ in range(3):
+        step.updater.step_async({feats: xs, labels: ys})
+    ops.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step.updater.step_async({feats: xs, labels: ys})
+    ops.sync()
+    sec_plain = (time.perf_counter() - t0) / steps
+    return {"ms_per_step": round(sec * 1e3, 4), "images_per_s": round(BATCH / sec, 1),
+            "what": "the step with every batch coming from host memory: shuffled host dataset -> page-locked staging -> queued "
+                    "upload -> augmentation kernel (mirrored pad 4, random crop, horizontal flip) -> training step; host fill of "
+                    "batch k+1 overlaps the device work of batch k",
+            "pageable_args_ms_per_step": round(sec_plain * 1e3, 4),
+            "pageable_args_what": "the same step with pageable numpy arrays as plan arguments: the plan uploads them inside each "
+                                  "execution, as CUDAPlan.executeImpl does"}
 
 
 def secondary(cfg, a):
@@ -158,6 +228,7 @@ def main():
                     help="run only the small steps off the main chain (dense-layer gradients) on a second queue")
     ap.add_argument("--graph", action="store_true", help="replay the step's kernels as a recorded HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-feed", action="store_true", help="skip the host-fed variant of the step")
     ap.add_argument("--no-kernel-timing", action="store_true", help="skip the per-kernel event pass")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -202,6 +273,8 @@ def main():
     result.update(window_stats(win, a.steps))
     if not np.isfinite(loss):
         sys.exit("bench.py: the loss is not finite (%r)" % loss)
+    if not a.no_feed:
+        result["host_feed"] = host_feed_leg(step, a.steps, a.warmup)
 
     if not a.no_kernel_timing:
         # Same step, every kernel object bracketed by hipEvents on the library stream, keyed by operation

@@ -59,6 +59,7 @@ PROTOTYPES = {
     "dopt_hip_event_create": [C.POINTER(_vp)],
     "dopt_hip_event_record": [_vp],
     "dopt_hip_event_elapsed_ms": [_vp, _vp, C.POINTER(_f)],
+    "dopt_hip_event_sync": [_vp],
     "dopt_hip_event_destroy": [_vp],
     "dopt_hip_pointwise": [C.c_char_p, _i, _sz, _vp, _vp, _vp],
     "dopt_hip_pointwise_chain": [_i, _sz, _sz, _i, C.POINTER(_vp), C.POINTER(C.c_ubyte), _i, C.POINTER(C.c_char_p),

@@ -1022,25 +1022,17 @@ __global__ __launch_bounds__(1024) void bn_cluster_k(unsigned N, unsigned C, uns
 ClusterMem g_cluster_mem[64];
 bool g_cluster_ready[64];
 bool g_cluster_unchecked = false;
-unsigned g_cluster_spin_limit = 1u << 21;   // polls of ~1 us each before a block gives up
+unsigned g_cluster_spin_limit = 1u << 21;   // polls of ~1 us each (2 s in all) before a block gives up
 
+unsigned long g_cluster_launches = 0;
+
+// The addresses and the one-time fill are made by dopt_hip_init (bn_device_setup below); a call only looks them up.
 int cluster_mem(ClusterMem *out)
 {
     int dev = -1;
     DOPT_HIP_CHECK(hipGetDevice(&dev));
     DOPT_REQUIRE(dev >= 0 && dev < 64, "batch norm: device index %d out of range", dev);
-    if (!g_cluster_ready[dev]) {
-        ClusterMem m;
-        DOPT_HIP_CHECK(hipGetSymbolAddress((void **)&m.rec, HIP_SYMBOL(g_cl_rec)));
-        DOPT_HIP_CHECK(hipGetSymbolAddress((void **)&m.sdx, HIP_SYMBOL(g_cl_sdx)));
-        DOPT_HIP_CHECK(hipGetSymbolAddress((void **)&m.depart, HIP_SYMBOL(g_cl_depart)));
-        DOPT_HIP_CHECK(hipGetSymbolAddress((void **)&m.error, HIP_SYMBOL(g_cl_error)));
-        // "nothing there" is all-ones (the loader zero-fills); once per device, before the first launch
-        DOPT_HIP_CHECK(hipMemset(m.rec, 0xff, sizeof(unsigned long long) * kClusterRecs * 4));
-        DOPT_HIP_CHECK(hipDeviceSynchronize());
-        g_cluster_mem[dev] = m;
-        g_cluster_ready[dev] = true;
-    }
+    DOPT_REQUIRE(g_cluster_ready[dev], "batch norm: device %d was not set up by dopt_hip_init", dev);
     *out = g_cluster_mem[dev];
     return DOPT_HIP_OK;
 }
@@ -1214,6 +1206,7 @@ int bn_train_impl(size_t N, size_t C, size_t inner, double momentum, const float
                            (float *)nullptr, cm, g_cluster_spin_limit, in ? pl : Pool{}, SideSum{});
         DOPT_LAUNCH_CHECK();
         g_cluster_unchecked = true;
+        g_cluster_launches++;
         return in ? DOPT_HIP_OK : pooled_after();
     }
     if (T) {
@@ -1354,6 +1347,7 @@ int bn_grad_impl(size_t N, size_t C, size_t inner, const float *dy, const float 
                            packed + total + C, dx_sum, cm, g_cluster_spin_limit, pl, sd);
         DOPT_LAUNCH_CHECK();
         g_cluster_unchecked = true;
+        g_cluster_launches++;
         return DOPT_HIP_OK;
     }
     if (T) {
@@ -1425,6 +1419,29 @@ int bn_cluster_poll()
     DOPT_HIP_CHECK(hipMemset(cm.sdx, 0, kClusterRecs * sizeof(unsigned long long)));
     return fail(DOPT_HIP_ERR_RUNTIME, "batch norm: blocks sharing a channel did not meet within the wait limit; the "
                                       "results of batch-norm calls since the last synchronisation are invalid");
+}
+
+unsigned long bn_cluster_launches() { return g_cluster_launches; }
+void bn_cluster_mark_unchecked() { g_cluster_unchecked = true; }
+bool bn_cluster_pending() { return g_cluster_unchecked; }
+
+int bn_device_setup()
+{
+    int dev = -1;
+    DOPT_HIP_CHECK(hipGetDevice(&dev));
+    DOPT_REQUIRE(dev >= 0 && dev < 64, "batch norm: device index %d out of range", dev);
+    if (g_cluster_ready[dev]) return DOPT_HIP_OK;
+    ClusterMem m;
+    DOPT_HIP_CHECK(hipGetSymbolAddress((void **)&m.rec, HIP_SYMBOL(g_cl_rec)));
+    DOPT_HIP_CHECK(hipGetSymbolAddress((void **)&m.sdx, HIP_SYMBOL(g_cl_sdx)));
+    DOPT_HIP_CHECK(hipGetSymbolAddress((void **)&m.depart, HIP_SYMBOL(g_cl_depart)));
+    DOPT_HIP_CHECK(hipGetSymbolAddress((void **)&m.error, HIP_SYMBOL(g_cl_error)));
+    // "nothing there" is all-ones (the loader zero-fills); once per device, before any launch
+    DOPT_HIP_CHECK(hipMemset(m.rec, 0xff, sizeof(unsigned long long) * kClusterRecs * 4));
+    DOPT_HIP_CHECK(hipDeviceSynchronize());
+    g_cluster_mem[dev] = m;
+    g_cluster_ready[dev] = true;
+    return DOPT_HIP_OK;
 }
 
 }  // namespace dopt

@@ -60,6 +60,16 @@ bool channel_sum(size_t N, size_t C, size_t inner, const float *in, float *out, 
 hipStream_t lane_stream(int lane);
 // bn.hip: error report of the multi-block batch-norm kernels; call with the queues idle.
 int bn_cluster_poll();
+// bn.hip: how many such kernels have been enqueued so far (a plan samples it around a recording to learn whether the
+// recording holds one), and the note a replay of such a recording leaves for the next synchronisation point.
+unsigned long bn_cluster_launches();
+void bn_cluster_mark_unchecked();
+bool bn_cluster_pending();
+// Per-device set-up done inside dopt_hip_init, with the device current: addresses of the file-scope device arrays
+// (bn.hip: the records blocks of a channel exchange, filled with "absent"; nn.hip: the scratch of
+// dopt_hip_bias_bwd_noalloc), so that no later call has to load a code object, fill memory or wait for the device.
+int bn_device_setup();
+int nn_device_setup();
 
 // Number of compute units of the active device (256 on MI355X); used to size grids.
 int num_cus();

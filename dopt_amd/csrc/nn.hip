@@ -629,12 +629,13 @@ int dopt_hip_bias_bwd(size_t N, size_t C, size_t inner, const float *dy, float *
 
 // ---- the same sum for callers that must not allocate
 // The per-(channel, slice) partial sums live in this array instead of the library's grown-on-demand
-// workspace, and the call sets nothing up (no lazy initialisation).  Every device the library runs on
-// holds its own copy at its own address until the process ends; host code only ever uses the address
-// hipGetSymbolAddress reports for the current device.
+// workspace, and the call sets nothing up: the array's address on the device is taken by dopt_hip_init
+// (nn_device_setup), which is also what makes the runtime load this file's code object, array included.
+// Every device the library runs on holds its own copy at its own address until the process ends; host
+// code only ever uses the address hipGetSymbolAddress reported for that device.
 static constexpr size_t kBiasScratchFloats = 65536;   // 256 KiB
 static __device__ __align__(256) float scratch[kBiasScratchFloats];
-static float *g_scratch_ptr[kMaxDevices];             // per device; null until that device's first call
+static float *g_scratch_ptr[kMaxDevices];             // per device; set by dopt_hip_init
 
 int dopt_hip_bias_bwd_noalloc(size_t N, size_t C, size_t inner, const float *dy, float *db)
 {
@@ -659,12 +660,7 @@ int dopt_hip_bias_bwd_noalloc(size_t N, size_t C, size_t inner, const float *dy,
     int dev = -1;
     DOPT_HIP_CHECK(hipGetDevice(&dev));
     DOPT_REQUIRE(dev >= 0 && dev < kMaxDevices, "dopt_hip_bias_bwd_noalloc: device index %d out of range", dev);
-    if (!g_scratch_ptr[dev]) {   // once per device, with that device current
-        float *p = nullptr;
-        DOPT_HIP_CHECK(hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch)));
-        DOPT_REQUIRE(p != nullptr, "dopt_hip_bias_bwd_noalloc: the scratch array has no device address");
-        g_scratch_ptr[dev] = p;
-    }
+    DOPT_REQUIRE(g_scratch_ptr[dev] != nullptr, "dopt_hip_bias_bwd_noalloc: device %d was not set up by dopt_hip_init", dev);
     return chan_sum_launch(N, C, inner, S, dy, g_scratch_ptr[dev], db);
 }
 
@@ -790,6 +786,19 @@ bool channel_sum(size_t N, size_t C, size_t inner, const float *in, float *out, 
     float *partial = (float *)workspace(C * S * sizeof(float));
     *rc = partial ? chan_sum_launch(N, C, inner, S, in, partial, out) : DOPT_HIP_ERR_OOM;
     return true;
+}
+
+int nn_device_setup()
+{
+    int dev = -1;
+    DOPT_HIP_CHECK(hipGetDevice(&dev));
+    DOPT_REQUIRE(dev >= 0 && dev < kMaxDevices, "dopt_hip_init: device index %d out of range", dev);
+    if (g_scratch_ptr[dev]) return DOPT_HIP_OK;
+    float *p = nullptr;
+    DOPT_HIP_CHECK(hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch)));
+    DOPT_REQUIRE(p != nullptr, "dopt_hip_init: the scratch array of dopt_hip_bias_bwd_noalloc has no device address");
+    g_scratch_ptr[dev] = p;
+    return DOPT_HIP_OK;
 }
 
 }  // namespace dopt

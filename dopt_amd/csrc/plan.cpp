@@ -1229,8 +1229,8 @@ int HIPPlan::Builder::prepackFilters()
 
 // convolutionFeaturesGrad and convolutionFiltersGrad of one layer read the same dy and nothing of each other: where
 // the former runs on a packed filter they become one step (dopt_hip_conv_bwd_pair_packed_open), placed where the
-// earlier of the two stands in the order - every input of either is ready there, and every reader of either comes
-// after its own, later or equal, position.
+// earlier of the two stands in the order - checked below: every input of either is ready there - and every reader of
+// either comes after its own, later or equal, position.
 void HIPPlan::Builder::pairBackward()
 {
     if (!(flags & DOPT_HIP_PLAN_FUSE)) return;
@@ -1255,9 +1255,19 @@ void HIPPlan::Builder::pairBackward()
             const auto *pad2 = sizes_attr(fo, "padding"), *stride2 = sizes_attr(fo, "stride");
             if (!pad || !stride || !pad2 || !stride2 || *pad != *pad2 || *stride != *stride2) continue;
             if (fo.shape != g.ops[pk.filter].shape || g.ops[fo.deps[1]].shape != bo.shape) continue;
+            const int first = pos[bd] < pos[fg] ? bd : fg, second = first == bd ? fg : bd;
+            // The pair runs where `first` stands, so whatever else `second` reads (x of the filter gradient, a
+            // computed filter) must have been made before that place; a graph written by hand may compute it in
+            // between (gradient graphs never do: both read values of the forward pass).  Such a couple stays two steps.
+            bool ready = true;
+            for (int d : g.ops[second].deps) {
+                size_t o;
+                const int r = root(d, &o);
+                if (!is_leaf(g.ops[r]) && pos[r] > pos[first]) ready = false;
+            }
+            if (!ready) continue;
             pairOf[bd] = fg;
             taken[fg] = 1;
-            const int first = pos[bd] < pos[fg] ? bd : fg, second = first == bd ? fg : bd;
             pairLead[first] = bd;
             pairLater[second] = 1;
             break;
@@ -1871,6 +1881,7 @@ int HIPPlan::execute(int nargs, const int *argOps, const void *const *argPtrs, c
         if (run && run->exec) {
             mReplays++;
             DOPT_HIP_CHECK(hipGraphLaunch(run->exec, stream()));
+            if (run->clusterKernels) bn_cluster_mark_unchecked();   // the next synchronisation point reads their error word
             return DOPT_HIP_OK;
         }
         if (!run) {
@@ -1879,12 +1890,14 @@ int HIPPlan::execute(int nargs, const int *argOps, const void *const *argPtrs, c
                 if (mRuns.front().graph) (void)hipGraphDestroy(mRuns.front().graph);
                 mRuns.erase(mRuns.begin());
             }
-            mRuns.push_back(CapturedRun{key, nullptr, nullptr, 0});
+            mRuns.push_back(CapturedRun{key, nullptr, nullptr, 0, false});
         } else {
             if (int rc = resolve(nargs, argOps, argPtrs, argOnHost)) return rc;
             DOPT_HIP_CHECK(hipStreamBeginCapture(stream(), hipStreamCaptureModeRelaxed));
             set_capturing(true);
+            const unsigned long clusterBefore = bn_cluster_launches();
             const int rc = enqueue(nrets, rets);
+            run->clusterKernels = bn_cluster_launches() != clusterBefore;
             set_capturing(false);
             run->wsGeneration = workspace_generation();   // cannot change while recording: growth is refused
             hipGraph_t graph = nullptr;
@@ -1893,6 +1906,7 @@ int HIPPlan::execute(int nargs, const int *argOps, const void *const *argPtrs, c
                 hipGraphInstantiate(&run->exec, graph, nullptr, nullptr, 0) == hipSuccess) {
                 run->graph = graph;
                 DOPT_HIP_CHECK(hipGraphLaunch(run->exec, stream()));
+                if (run->clusterKernels) bn_cluster_mark_unchecked();
                 return DOPT_HIP_OK;
             }
             // something in this plan cannot be recorded (an allocation, a fill): nothing ran, run it directly from now on

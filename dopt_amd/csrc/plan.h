@@ -129,6 +129,7 @@ private:
         hipGraph_t graph;
         hipGraphExec_t exec;                     // null until the second execution with this key
         unsigned long wsGeneration;              // workspace_generation() when it was recorded
+        bool clusterKernels = false;             // holds a multi-block batch norm: every launch owes an error check
     };
     std::vector<CapturedRun> mRuns;
     bool mGraphOk = false;

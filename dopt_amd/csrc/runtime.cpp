@@ -89,6 +89,9 @@ int init_locked(int device)
                     r.arch.c_str());
     DOPT_HIP_CHECK(hipStreamCreateWithFlags(&r.stream, hipStreamNonBlocking));
     DOPT_HIP_CHECK(hipStreamCreateWithFlags(&r.side, hipStreamNonBlocking));   // same (default) priority
+    // addresses (and the one-time fill) of the file-scope device arrays: nothing is left for a first call to set up
+    if (int rc = bn_device_setup()) return rc;
+    if (int rc = nn_device_setup()) return rc;
     r.device = device;
     r.ready = true;
     return DOPT_HIP_OK;
@@ -440,6 +443,10 @@ int dopt_hip_copy_d2h(void *host_dst, const void *src, size_t bytes)
     DOPT_ENSURE_INIT();
     DOPT_HIP_CHECK(hipMemcpyAsync(host_dst, src, bytes, hipMemcpyDeviceToHost, stream()));
     DOPT_HIP_CHECK(hipStreamSynchronize(stream()));
+    if (!bn_cluster_pending()) return DOPT_HIP_OK;
+    // the report is read with both queues idle (a multi-block batch norm may still run on the other one)
+    DOPT_HIP_CHECK(hipStreamSynchronize(lane_stream(0)));
+    DOPT_HIP_CHECK(hipStreamSynchronize(lane_stream(1)));
     return bn_cluster_poll();
 }
 
@@ -484,6 +491,13 @@ int dopt_hip_event_elapsed_ms(void *start, void *stop, float *ms)
     DOPT_REQUIRE(start && stop && ms, "dopt_hip_event_elapsed_ms: null argument");
     DOPT_HIP_CHECK(hipEventSynchronize((hipEvent_t)stop));
     DOPT_HIP_CHECK(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_event_sync(void *event)
+{
+    DOPT_REQUIRE(event != nullptr, "dopt_hip_event_sync: event is null");
+    DOPT_HIP_CHECK(hipEventSynchronize((hipEvent_t)event));
     return DOPT_HIP_OK;
 }
 

@@ -137,8 +137,9 @@ class DeviceFeed:
 
     next() returns (features, labels) device tensors for one batch.  The host side of batch k+1
     (iterator fill, random draws, staging) overlaps the device side of batch k: each of the two slots
-    owns its staging memory and device buffers, and a slot is only refilled after the caller's work
-    on it was queued two batches ago and a sync has passed since."""
+    owns its staging memory and device buffers, and a slot is refilled only after the work the caller
+    queued on it two calls ago has finished - found through an event recorded on entry to the call in
+    between, so the host waits for that batch's step alone, not for the device to drain."""
 
     def __init__(self, dataset, batch_size, jitter_x=0, jitter_y=0, flip_x=False, flip_y=False, seed=0):
         self.dataset, self.batch = dataset, batch_size
@@ -155,6 +156,20 @@ class DeviceFeed:
                 "raw": ops.Tensor([batch_size] + list(fshape)), "f": ops.Tensor([batch_size] + list(fshape)),
                 "l": ops.Tensor([batch_size] + list(lshape)), "g": ops.Tensor([batch_size, 3], np.int32)})
         self._turn = 0
+        self._marks = []
+        for _ in range(2):
+            ev = C.c_void_p()
+            capi.check(capi.load().dopt_hip_event_create(C.byref(ev)))
+            self._marks.append(ev)
+        self._calls = 0
+
+    def __del__(self):
+        for ev in getattr(self, "_marks", []):
+            try:
+                capi.load().dopt_hip_event_destroy(ev)
+            except Exception:   # interpreter shutdown
+                pass
+        self._marks = []
 
     def finished(self):
         return self.dataset.finished()
@@ -165,8 +180,12 @@ class DeviceFeed:
     def next(self):
         s = self._slots[self._turn]
         self._turn ^= 1
-        if self._turn == 0:
-            ops.sync()        # both slots are in flight: wait before the first one is refilled
+        lib, j = capi.load(), self._calls
+        self._calls += 1
+        # the mark of the previous call lies behind everything queued before it, the step on this slot included
+        if j >= 1:
+            capi.check(lib.dopt_hip_event_sync(self._marks[(j - 1) & 1]))
+        capi.check(lib.dopt_hip_event_record(self._marks[j & 1]))
         self.dataset.getBatch([s["f_host"].array, s["l_host"].array])
         s["g_host"].array[:] = draw_geometry(self._rng, self.batch, self.jx, self.jy, self.fx, self.fy)
         s["f_host"].upload_async(s["raw"])

@@ -96,6 +96,9 @@ void *dopt_hip_stream(void);
 int dopt_hip_event_create(void **event);
 int dopt_hip_event_record(void *event);
 int dopt_hip_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for `stop` */
+/* Blocks the host until everything enqueued before the event's last record has finished: the per-buffer wait of a feed
+   loop, where the reference's blocking cuMemcpyHtoD per argument (cuda/package.d:367-401) waited for the whole device. */
+int dopt_hip_event_sync(void *event);
 int dopt_hip_event_destroy(void *event);
 
 /* ---------------------------------------------------------------------------------------

@@ -62,6 +62,17 @@ def _f32(a):
     return np.ascontiguousarray(a, dtype=np.float32)
 
 
+def set_threads(n):
+    """Threads for the loops the reference hands to std.parallelism (sum / maxElement over the outer index,
+    cpu/math.d:102,179; repeat over its blocks, cpu/basic.d:166).  Results do not depend on it; used by the
+    CPU-baseline timing only."""
+    lib().oracle_set_threads(int(n))
+
+
+def get_threads():
+    return int(lib().oracle_get_threads())
+
+
 BINARY = ("add", "sub", "mul", "div", "lt", "lte", "gt", "gte", "eq", "neq", "max", "min", "pow", "atan2")
 UNARY = ("neg", "abs", "sgn", "exp", "log", "sqrt", "sin", "cos", "tan", "asin", "acos", "atan",
          "sinh", "cosh", "tanh", "asinh", "acosh", "atanh")

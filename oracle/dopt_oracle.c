@@ -204,6 +204,14 @@ static size_t vol_of(const size_t *shape, int from, int to)
     return v;
 }
 
+/* Threads for the loops the reference hands to std.parallelism (`foreach(...; ....parallel)`: sum and maxElement over
+   the outer index, cpu/math.d:102,179; repeat over its blocks, cpu/basic.d:166).  Each output element is still
+   computed by one thread in the serial order, so results do not depend on the count.  1 unless the CPU-baseline
+   timing asks for more. */
+static int g_threads = 1;
+void oracle_set_threads(int n) { g_threads = n < 1 ? 1 : n; }
+int oracle_get_threads(void) { return g_threads; }
+
 #define DEFINE_REDUCE(NAME, T, INIT, COMBINE)                                                  \
     static int NAME(const size_t *shape0, int rank, const size_t *axes, int naxes,             \
                     const T *in, T *out)                                                       \
@@ -222,6 +230,7 @@ static size_t vol_of(const size_t *shape, int from, int to)
             size_t highstride = lowstride * shape[axis];                                       \
             outbuf = (T *)malloc(sizeof(T) * (newvol ? newvol : 1));                           \
             if (!outbuf) { free(owned_in); return 3; }                                         \
+            _Pragma("omp parallel for schedule(static) if (g_threads > 1) num_threads(g_threads)") \
             for (size_t o = 0; o < newvol / lowstride; o++) {                                  \
                 if (lowstride == 1) {                                                          \
                     T acc = INIT;                                                              \
@@ -402,8 +411,12 @@ int ref_repeat(int rank, const size_t *inShape, const size_t *reps, const void *
         vol *= inShape[ax];
         outbuf = (uint32_t *)malloc(4 * ((len * a) != 0 ? len * a : 1));
         if (!outbuf) { free(owned); return 3; }
-        for (size_t i = 0; i < len; i += vol)
+        /* cpu/basic.d:166: the blocks are handed to the task pool */
+#pragma omp parallel for schedule(static) if (g_threads > 1) num_threads(g_threads)
+        for (size_t b = 0; b < len / vol; b++) {
+            const size_t i = b * vol;
             for (size_t o = i * a; o < (i + vol) * a; o += vol) memcpy(outbuf + o, inbuf + i, vol * 4);
+        }
         vol *= a;
         len *= a;
         free(owned);

@@ -116,6 +116,11 @@ int ref_amsgrad_step(size_t n, float eta, float beta1, float beta2, float eps, c
 int ref_image_transform(size_t N, size_t C, size_t H, size_t W, size_t jx, size_t jy,
                         const int32_t *geom, float *batch, float *padded);
 
+/* Threads for the loops the reference runs through std.parallelism (sum, maxElement, repeat); default 1.
+   Results do not depend on it. */
+void oracle_set_threads(int n);
+int oracle_get_threads(void);
+
 #ifdef __cplusplus
 }
 #endif

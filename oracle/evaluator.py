@@ -45,14 +45,16 @@ def _transpose(x, order):
     raise NotImplementedError("transpose of rank %d" % x.ndim)
 
 
-def _kernel(op, d):
+def _kernel(op, d, blas=False):
     t, a = op.opType, op.attributes
     if t in O.BINARY and len(d) == 2:
         return O.pointwise(t, d[0], d[1])
     if t in O.UNARY:
         return O.pointwise(t, d[0])
     if t == "matmul":
-        return O.matmul(d[0], d[1])
+        # cpu/math.d:77-82 calls cblas gemm; `blas` times it that way (numpy's OpenBLAS at its default thread
+        # count), the checker uses the plain loop whose order of summation is known
+        return np.matmul(d[0], d[1]) if blas else O.matmul(d[0], d[1])
     if t == "sum":
         return O.sum(d[0], list(a["axes"]))
     if t == "maxElement":
@@ -111,14 +113,15 @@ def _kernel(op, d):
     raise NotImplementedError("no CPU kernel for operation '%s'" % t)
 
 
-def evaluate(outputs, args=None):
-    """Values of `outputs` (a list of graph nodes) as numpy arrays; args maps variables to arrays."""
+def evaluate(outputs, args=None, blas=False):
+    """Values of `outputs` (a list of graph nodes) as numpy arrays; args maps variables to arrays.  blas: matmul through
+    the BLAS numpy links, as the reference's CPU backend calls cblas (for timing; not the checker's path)."""
     given = {id(k): np.ascontiguousarray(v, dtype=k.dtype).reshape(k.shape) for k, v in (args or {}).items()}
     vals = {}
     for op in _topological(list(outputs)):
         if op.opType in ("variable", "constant"):
             vals[id(op)] = given[id(op)] if id(op) in given else np.ascontiguousarray(op.value)
             continue
-        out = _kernel(op, [vals[id(x)] for x in op.deps])
+        out = _kernel(op, [vals[id(x)] for x in op.deps], blas)
         vals[id(op)] = np.ascontiguousarray(out).reshape(op.shape)
     return [vals[id(o)] for o in outputs]

@@ -352,6 +352,42 @@ def test_pools_ride_in_the_batch_norm_kernels():
         assert np.array_equal(a, b) or (a.ndim == 1 and np.allclose(a, b, rtol=0, atol=2e-5))
 
 
+def test_backward_pair_waits_for_a_feature_operand_computed_in_between():
+    """A graph written by hand in which the x operand of the filter gradient is itself computed, and only the filter
+    gradient leads to it: in the plan's order it stands between backward-data and the filter gradient, so the two
+    must not share a step placed where backward-data stands (the step would read x before it exists).  With the
+    operand computed ahead of both, the same couple does share a step.  Values are those of the plain plan."""
+    r = np.random.default_rng(1259)
+    xs, k = (16, 128, 8, 8), 256
+    X = r.standard_normal(xs).astype(np.float32)
+    W = (r.standard_normal((k, xs[1], 3, 3)) * 0.05).astype(np.float32)
+    DY = r.standard_normal((xs[0], k, xs[2], xs[3])).astype(np.float32)
+    xv, wv, dyv = float32(list(xs)), float32(list(W.shape)), float32(list(DY.shape))
+    args = {xv: X, wv: W, dyv: DY}
+    flags = core.PLAN_VIEWS | core.PLAN_FUSE | core.PLAN_TIMING
+    # x computed between the two: two steps
+    xc = core.relu(xv)
+    dx = core.convolutionFeaturesGrad(dyv, wv, list(xs), [1, 1], [1, 1])
+    dw = core.convolutionFiltersGrad(dyv, xc, list(W.shape), [1, 1], [1, 1])
+    plan = core.compile([dx, dw], flags)
+    got = plan.execute(args)
+    prof = plan.profile()
+    assert "convolutionFeaturesGrad+convolutionFiltersGrad" not in prof, prof
+    want = core.compile([dx, dw], 0).execute(args)
+    assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
+    assert np.abs(want[1]).max() > 0
+    # the same operand reached first (it is also an output ahead of the two): one step
+    plan = core.compile([xc, dx, dw], flags)
+    got = plan.execute(args)
+    assert plan.profile()["convolutionFeaturesGrad+convolutionFiltersGrad"][1] == 1
+    assert np.array_equal(got[1], want[0]) and np.array_equal(got[2], want[1])
+    # the filter gradient first in the order: its step takes backward-data along (dy and the filter are ready)
+    plan = core.compile([dw, dx], flags)
+    got = plan.execute(args)
+    assert plan.profile()["convolutionFeaturesGrad+convolutionFiltersGrad"][1] == 1
+    assert np.array_equal(got[0], want[1]) and np.array_equal(got[1], want[0])
+
+
 def test_packed_filter_entry_points_match_the_unpacked_ones():
     """dopt_hip_conv_pack_batch + the *_packed entry points against dopt_hip_conv_fwd_bias /
     dopt_hip_conv_bwd_data (themselves checked against the oracle in test_gpu_ops.py): same kernels,
@@ -810,6 +846,41 @@ def test_overlapped_filter_gradients_change_nothing(maker):
     assert np.allclose(runs[0][0], runs[3][0], rtol=1e-4)
 
 
+def test_second_queue_beside_batch_norms_whose_blocks_share_a_channel():
+    """The first two layers of the benchmark network at batch 128 hold 131072 values per channel: their batch norms run
+    as four blocks per channel that wait for each other, sized for an otherwise idle device.  With a second queue live
+    (both overlap modes) other kernels run beside them; no batch norm is ever moved to that queue, so blocks that wait
+    only ever wait for blocks of their own launch, and the steps must stay what they are without the second queue -
+    and no launch may report blocks that did not meet."""
+    r = np.random.default_rng(5)
+    xs = ops.tensor(r.standard_normal((128, 3, 32, 32)).astype(np.float32))
+    ys = ops.tensor(np.eye(10, dtype=np.float32)[r.integers(0, 10, 128)])
+    base = core.PLAN_VIEWS | core.PLAN_FUSE
+
+    def network(seed):
+        init = nnet.Init(seed)
+        x, y = core.float32([128, 3, 32, 32]), core.float32([128, 10])
+        h = nnet.relu(nnet.batchNorm(nnet.conv2D(nnet.dataSource(x), 64, (3, 3), init, padding=(1, 1))))
+        h = nnet.maxPool(nnet.relu(nnet.batchNorm(nnet.conv2D(h, 64, (3, 3), init, padding=(1, 1)))), (2, 2))
+        h = nnet.maxPool(nnet.relu(nnet.batchNorm(nnet.conv2D(h, 128, (3, 3), init, padding=(1, 1)))), (2, 2))
+        h = nnet.maxPool(h, (2, 2))
+        top = nnet.softmax(nnet.dense(nnet.relu(nnet.dense(h, 64, init)), 10, init))
+        net = nnet.DAGNetwork([x], [top])
+        return x, y, net, nnet.crossEntropy(top.trainOutput, y) + net.paramLoss
+
+    runs = []
+    for flags in (base, base | core.PLAN_OVERLAP, base | core.PLAN_OVERLAP_LIGHT):
+        x, y, net, loss = network(6)
+        up = online.fused_sgd([loss], net.params, net.paramProj, flags=flags)
+        losses = [up({x: xs, y: ys})[0] for _ in range(4)]
+        ops.sync()                      # raises if a multi-block batch norm gave up waiting
+        runs.append((losses, [p.value for p in net.params]))
+    for other in runs[1:]:
+        assert runs[0][0] == other[0]
+        for a, b in zip(runs[0][1], other[1]):
+            assert np.array_equal(a, b)
+
+
 @pytest.mark.parametrize("maker", [online.fused_sgd, online.adam])
 def test_recorded_graph_replays_match_direct_execution(maker):
     """DOPT_HIP_PLAN_GRAPH: the first execution with a set of device pointers runs directly, the second
@@ -868,6 +939,50 @@ def test_recorded_graph_survives_a_workspace_move_and_pool_reuse():
         assert np.array_equal(a.value, b.value)
     for gd in guards:
         assert np.all(gd.numpy() == 3.25)
+
+
+def test_replayed_multi_block_batch_norm_still_reports_blocks_that_did_not_meet():
+    """A plan whose batch norm runs as blocks sharing a channel, replayed as a recorded graph: the error word such a
+    kernel raises when its blocks give up (here: the wait bound set to zero by the host, every block still exits) is
+    read at the next synchronisation point also when the kernel ran inside a replay, the exchange words are put
+    back, and the next replay is correct again."""
+    lib = capi.load()
+    r = np.random.default_rng(1873)
+    shape = (128, 64, 32, 32)                         # 131072 values per channel: four blocks per channel
+    X = ops.tensor(r.standard_normal(shape).astype(np.float32))
+    ones, zeros = np.ones(64, np.float32), np.zeros(64, np.float32)
+    xv = float32(list(shape))
+    y, _, _ = core.batchNormTrain(xv, float32([64], ones), float32([64], zeros), float32([64], zeros), float32([64], ones), 0.9)
+    plan = core.compile([y], core.PLAN_VIEWS | core.PLAN_GRAPH)
+    out = ops.Tensor(shape)
+    for _ in range(3):                                # direct, recorded, replayed
+        plan.execute({xv: X}, rets=[out])
+    ops.sync()
+    assert plan.recordings() == {"recorded": 1, "replays": 1}
+    want = out.numpy()
+    capi.check(lib.dopt_hip_bn_wait_limit(0))
+    try:
+        # the bound is a kernel argument of the recorded launch: record anew with the bound at zero
+        plan2 = core.compile([y], core.PLAN_VIEWS | core.PLAN_GRAPH)
+        out2 = ops.Tensor(shape)
+        plan2.execute({xv: X}, rets=[out2])           # direct
+        with pytest.raises(capi.HipError, match="did not meet"):
+            ops.sync()
+        plan2.execute({xv: X}, rets=[out2])           # recorded
+        with pytest.raises(capi.HipError, match="did not meet"):
+            ops.sync()
+        plan2.execute({xv: X}, rets=[out2])           # replayed
+        assert plan2.recordings() == {"recorded": 1, "replays": 1}
+        with pytest.raises(capi.HipError, match="did not meet"):
+            ops.sync()
+    finally:
+        capi.check(lib.dopt_hip_bn_wait_limit(1 << 21))
+    ops.sync()
+    plan.execute({xv: X}, rets=[out])                 # the first plan's recording: words were put back, result as before
+    ops.sync()
+    assert plan.recordings()["replays"] == 2
+    assert np.array_equal(out.numpy(), want)
+    assert_close(want.ravel(), O.bn_train(X.numpy(), ones, zeros, zeros, ones, 0.9)[:want.size], "replayed multi-block batch norm")
 
 
 def test_graph_flag_leaves_plans_with_caller_registered_kernels_direct():

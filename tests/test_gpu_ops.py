@@ -503,7 +503,11 @@ def test_bias(shape):
                                    (16, 16, 16, 16),
                                    (40, 4, 32, 32),     # channel too large for the register-resident path
                                    (128, 8, 16, 16),    # the largest channel that path takes (1024 threads)
-                                   (5, 7, 4, 3)])       # ragged tail in the resident path
+                                   (5, 7, 4, 3),        # ragged tail in the resident path
+                                   # two values per channel: xhat is +-1 up to eps, and dx is what is left of dy after
+                                   # both projections cancel - O(eps / var) of dy, far below the absolute tolerance, so
+                                   # a comparison relative to max|dx| reads large while the stated tolerance holds
+                                   (2, 8, 1, 1), (2, 128, 1, 1), (2, 3, 1, 1), (2, 17, 1, 1)])
 def test_batchnorm_train_grad_infer(shape):
     r = rng(61)
     C = shape[1]
