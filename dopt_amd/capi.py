@@ -76,6 +76,7 @@ PROTOTYPES = {
     "dopt_hip_transpose2d": [_sz, _sz, _vp, _vp],
     "dopt_hip_sgemm": [_sz, _sz, _sz, _vp, _vp, _vp],
     "dopt_hip_sgemm_t": [C.c_int, C.c_int, _sz, _sz, _sz, _vp, _vp, _vp],
+    "dopt_hip_sgemm_batch": [_i, C.POINTER(C.c_int), C.POINTER(C.c_int), _szp, _szp, _szp, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp)],
     "dopt_hip_sgemm_rank1": [_i, _i, _sz, _sz, _sz, _vp, _vp, _vp, _vp, _i, _vp],
     "dopt_hip_sgemm_relu_grad": [_i, _i, _sz, _sz, _sz, _vp, _vp, _vp, _vp],
     "dopt_hip_conv_fwd": [C.POINTER(ConvDesc), _vp, _vp, _vp],
@@ -92,6 +93,7 @@ PROTOTYPES = {
     "dopt_hip_conv_bwd_pair_packed_open": [C.POINTER(ConvDesc), _vp, _vp, _vp, _vp, _vp, C.POINTER(SplitSum), C.POINTER(SplitSum)],
     "dopt_hip_split_sum_close": [C.POINTER(SplitSum)],
     "dopt_hip_conv_bwd_filter": [C.POINTER(ConvDesc), _vp, _vp, _vp],
+    "dopt_hip_conv_bwd_filter_batch": [_i, C.POINTER(ConvDesc), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp)],
     "dopt_hip_maxpool_fwd": [_sz, _sz, _sz, _sz, _sz, _sz, _vp, _vp],
     "dopt_hip_maxpool_bwd": [_sz, _sz, _sz, _sz, _sz, _sz, _vp, _vp, _vp],
     "dopt_hip_softmax_fwd": [_sz, _sz, _sz, _vp, _vp],

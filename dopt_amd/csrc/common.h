@@ -50,6 +50,9 @@ int sgemm_bias(int transA, int transB, size_t M, size_t N, size_t K, const float
 // sgemm.hip: dw[K][C][3][3] = filter gradient of a 3x3, pad-1 convolution over 2x2 images, from x[N][4C]
 // and dy[N][4K] in one launch.  Returns false, with nothing launched, for shapes it does not take.
 bool sgemm_fold2x2(size_t C, size_t K, size_t N, const float *x, const float *dy, float *dw, int *rc);
+// The same for up to 8 layers in one launch; false, with nothing launched, unless every layer suits that kernel.
+bool sgemm_fold2x2_batch(int n, const size_t *C, const size_t *K, const size_t *N, const float *const *x,
+                         const float *const *dy, float *const *dw, int *rc);
 // conv_smallc.hip: 3x3 pad-1 unit-stride convolutions over at most three input channels.  `done`
 // stays false when the shape is not theirs (the caller then uses the general kernels).
 bool conv_smallc_takes(const dopt_hip_conv_desc *d);

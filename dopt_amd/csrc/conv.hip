@@ -2372,6 +2372,38 @@ int dopt_hip_split_sum_close(const dopt_hip_split_sum *open)
                                 (unsigned)open->inner);
 }
 
+int dopt_hip_conv_bwd_filter_batch(int n, const dopt_hip_conv_desc *descs, const float *const *dy, const float *const *x,
+                                   float *const *dw)
+{
+    DOPT_REQUIRE(n >= 0 && (n == 0 || (descs && dy && x && dw)), "dopt_hip_conv_bwd_filter_batch: null argument");
+    DOPT_ENSURE_INIT();
+    // the filter gradients of 2x2-image layers are one dense product each, all of the same kernel: up to 8 share a launch
+    int i = 0;
+    while (i < n) {
+        int m = 0;
+        size_t C[8], K[8], N[8];
+        while (i + m < n && m < 8) {
+            const dopt_hip_conv_desc *d = &descs[i + m];
+            size_t P, Q;
+            if (check_desc(d, &P, &Q, "dopt_hip_conv_bwd_filter_batch") || !dy[i + m] || !x[i + m] || !dw[i + m] ||
+                conv_smallc_takes(d) || !dense2x2_takes(d))
+                break;
+            C[m] = d->C; K[m] = d->K; N[m] = d->N;
+            m++;
+        }
+        clear_error();
+        int rc = DOPT_HIP_OK;
+        if (m >= 2 && sgemm_fold2x2_batch(m, C, K, N, x + i, dy + i, dw + i, &rc)) {
+            if (rc) return rc;
+            i += m;
+            continue;
+        }
+        if (int rc1 = dopt_hip_conv_bwd_filter(&descs[i], dy[i], x[i], dw[i])) return rc1;
+        i++;
+    }
+    return DOPT_HIP_OK;
+}
+
 int dopt_hip_conv_bwd_filter(const dopt_hip_conv_desc *d, const float *dy, const float *x, float *dw)
 {
     size_t P, Q;

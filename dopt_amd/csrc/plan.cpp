@@ -646,6 +646,7 @@ struct HIPPlan::Builder {
     int prepackFilters();
     int allocateBuffers();
     int buildSteps();
+    void batchIndependent();
     void openSplitSums();
     void rememberAliases();
     int assignQueues();
@@ -1435,6 +1436,115 @@ int HIPPlan::Builder::buildSteps()
     return DOPT_HIP_OK;
 }
 
+// Steps that nothing in the plan waits for - the weight and bias gradients of dense layers, the filter gradients of
+// layers whose backward-data runs apart from them - are each a launch of a few microseconds, and between two launches
+// of one queue the device idles about as long.  Those that read nothing but values made earlier and are read by nobody
+// (their values only leave the plan) can run in any order and all at once: the plain products of the plan become one
+// dopt_hip_sgemm_batch, the filter gradients of 2x2-image layers one dopt_hip_conv_bwd_filter_batch, each placed
+// where the last of its members stood (everything they read is older than that, and nothing was going to read them
+// before).  The members run the kernel bodies they would have run alone: no value changes (DOPT_HIP_PLAN_FUSE).
+void HIPPlan::Builder::batchIndependent()
+{
+    if (!(flags & DOPT_HIP_PLAN_FUSE)) return;
+    auto base_label = [](const std::string &l) { return l.substr(0, l.find('@')); };
+    struct Product { size_t step; MatmulInfo mi; };
+    struct Wgrad { size_t step; dopt_hip_conv_desc d; };
+    std::vector<Product> products;
+    std::vector<Wgrad> wgrads;
+    for (size_t i = 0; i < p->mSteps.size(); i++) {
+        const Step &st = p->mSteps[i];
+        const int id = st.op;
+        if (id < 0 || !uses[id].empty() || !dynamic_cast<FnKernel *>(st.kernel.get())) continue;
+        if (biasGradOf[id] >= 0 || poolOf[id] >= 0 || pairOf[id] >= 0 || pairLead[id] >= 0 || pairLater[id] || packOf[id] >= 0) continue;
+        const Operation &op = g.ops[id];
+        const std::string label = base_label(st.label);
+        MatmulInfo mi;
+        if ((label == "matmul" || label == "matmul+transpose") && (fusedKind[id] == 0 || fusedKind[id] == 6) &&
+            plainProduct(id, &mi, false) && st.inputOps.size() == 2 && st.inputOps[0] == mi.a && st.inputOps[1] == mi.b &&
+            products.size() < 64) {
+            products.push_back({i, mi});
+        } else if (label == "convolutionFiltersGrad" && op.opType == "convolutionFiltersGrad" && fusedKind[id] == 0 &&
+                   op.deps.size() == 2 && op.dtype == DOPT_HIP_F32 && st.inputOps == op.deps && wgrads.size() < 64) {
+            const auto *pad = sizes_attr(op, "padding"), *stride = sizes_attr(op, "stride");
+            const auto &x = g.ops[op.deps[1]].shape;
+            if (!pad || !stride || x.size() != 4 || op.shape.size() != 4 || x[2] != 2 || x[3] != 2) continue;
+            wgrads.push_back({i, conv_desc(x, op.shape, *pad, *stride)});
+        }
+    }
+    std::vector<char> drop(p->mSteps.size(), 0);
+    const bool shapes = (flags & DOPT_HIP_PLAN_TIMING_SHAPES) != 0;
+    if (products.size() >= 2) {
+        Step b;
+        b.op = -1;
+        b.label = "matmul*" + std::to_string(products.size()) + (shapes ? "@" : "");
+        std::vector<int> tA, tB;
+        std::vector<size_t> M, N, K;
+        std::vector<float *> outs;
+        for (const Product &c : products) {
+            tA.push_back(c.mi.tA); tB.push_back(c.mi.tB);
+            M.push_back(c.mi.M); N.push_back(c.mi.N); K.push_back(c.mi.K);
+            b.inputOps.push_back(c.mi.a);
+            b.inputOps.push_back(c.mi.b);
+            outs.push_back((float *)p->mResults[p->mSteps[c.step].op]);
+            drop[c.step] = 1;
+        }
+        const int n = (int)products.size();
+        b.kernel = make([=](const std::vector<const void *> &in, void *) {
+            std::vector<const float *> A((size_t)n), B((size_t)n);
+            for (int j = 0; j < n; j++) {
+                A[(size_t)j] = (const float *)in[(size_t)(2 * j)];
+                B[(size_t)j] = (const float *)in[(size_t)(2 * j + 1)];
+            }
+            return dopt_hip_sgemm_batch(n, tA.data(), tB.data(), M.data(), N.data(), K.data(), A.data(), B.data(), outs.data());
+        });
+        b.inputs.resize(b.inputOps.size());
+        b.inputBytes.resize(b.inputOps.size());
+        for (size_t i = 0; i < b.inputOps.size(); i++) b.inputBytes[i] = g.ops[b.inputOps[i]].bytes();
+        const size_t at = products.back().step;
+        drop[at] = 0;
+        p->mSteps[at] = std::move(b);
+    }
+    if (wgrads.size() >= 2) {
+        Step b;
+        b.op = -1;
+        b.label = "convolutionFiltersGrad*" + std::to_string(wgrads.size()) + (shapes ? "@" : "");
+        std::vector<dopt_hip_conv_desc> descs;
+        std::vector<float *> outs;
+        for (const Wgrad &c : wgrads) {
+            descs.push_back(c.d);
+            const Operation &op = g.ops[p->mSteps[c.step].op];
+            b.inputOps.push_back(op.deps[0]);
+            b.inputOps.push_back(op.deps[1]);
+            outs.push_back((float *)p->mResults[p->mSteps[c.step].op]);
+            drop[c.step] = 1;
+        }
+        const int n = (int)wgrads.size();
+        b.kernel = make([=](const std::vector<const void *> &in, void *) {
+            std::vector<const float *> dy((size_t)n), x((size_t)n);
+            for (int j = 0; j < n; j++) {
+                dy[(size_t)j] = (const float *)in[(size_t)(2 * j)];
+                x[(size_t)j] = (const float *)in[(size_t)(2 * j + 1)];
+            }
+            return dopt_hip_conv_bwd_filter_batch(n, descs.data(), dy.data(), x.data(), outs.data());
+        });
+        b.inputs.resize(b.inputOps.size());
+        b.inputBytes.resize(b.inputOps.size());
+        for (size_t i = 0; i < b.inputOps.size(); i++) b.inputBytes[i] = g.ops[b.inputOps[i]].bytes();
+        const size_t at = wgrads.back().step;
+        drop[at] = 0;
+        p->mSteps[at] = std::move(b);
+    }
+    // close the ranks; the convolution steps remembered for openSplitSums move with them
+    std::vector<size_t> moved(p->mSteps.size(), 0);
+    std::vector<Step> kept;
+    for (size_t i = 0; i < p->mSteps.size(); i++) {
+        moved[i] = kept.size();
+        if (!drop[i]) kept.push_back(std::move(p->mSteps[i]));
+    }
+    p->mSteps = std::move(kept);
+    for (ConvStep &cs : convSteps) cs.step = moved[cs.step];
+}
+
 // A convolution that splits its reduction normally ends with a pass that adds the partial copies.
 // When the step right behind it is the batch norm (forward) or batch-norm gradient (backward) that
 // reads the whole result anyway, the convolution leaves the result open and that step adds the
@@ -1717,6 +1827,7 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
     }
     if (int rc = b.allocateBuffers()) return rc;
     if (int rc = b.buildSteps()) return rc;
+    b.batchIndependent();
     b.openSplitSums();
     b.rememberAliases();
     if (flags & (DOPT_HIP_PLAN_OVERLAP | DOPT_HIP_PLAN_OVERLAP_LIGHT))

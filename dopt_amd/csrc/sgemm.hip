@@ -6,6 +6,8 @@
 // core/source/dopt/core/ops/package.d:96-103) and rank-2 row / column sums are products with a
 // ones vector too (core/source/dopt/core/ops/math.d:257-279).  Those degenerate shapes are
 // HBM-bound and get their own kernels here; everything else runs on the fp32 MFMA tile engine.
+#include <vector>
+
 #include "common.h"
 #include "mfma_core.h"
 
@@ -349,6 +351,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void sgemm_rows_k(Gemm p)
 // step of prefetch every step waited a full memory latency, eight of them in a row for a 512-deep reduction -
 // most of such a kernel's duration.  The order of the sums is that of the steps, whatever is in flight.
 constexpr int kSmallWaves = 8, kSmallDepth = 4;
+constexpr int kGroupJobs = 8;   // jobs one grouped launch may hold (its descriptions travel as kernel arguments)
 
 // The lane's four reductions kk .. kk + 3 of row / column r.  `base`: byte offset of (r, reduction 0), or kOobOffset
 // when r lies outside the matrix; `pitch`: bytes between consecutive reductions of an r-contiguous operand.
@@ -368,15 +371,14 @@ __device__ __forceinline__ void small_load(__amdgpu_buffer_rsrc_t rs, unsigned b
 
 // kVA / kVB: the rows of a k-contiguous A / B are 16-byte addressable (an r-contiguous operand has no use for the flag).
 template <bool kTA, bool kTB, bool kVA, bool kVB>
-__global__ __launch_bounds__(64 * kSmallWaves) void sgemm_small_k(int M, int N, int K, int lda, int ldb, int kslice,
-                                                                   const float *A, const float *B, float *C,
-                                                                   const float *colbias, int bias_shift,
-                                                                   const float *rowvec, int relu, const float *mask)
+__device__ __forceinline__ void sgemm_small_body(int M, int N, int K, int lda, int ldb, int kslice, const float *A,
+                                                 const float *B, float *C, const float *colbias, int bias_shift,
+                                                 const float *rowvec, int relu, const float *mask, int bx, int by,
+                                                 float (*red)[32 * 33])
 {
-    __shared__ float red[kSmallWaves][32 * 33];
     const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, r = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // the same in every lane: loop bounds stay scalar
-    const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+    const int m0 = by * 32, n0 = bx * 32;
     const int row = m0 + r, col = n0 + r;
     const int k_begin = wave * kslice, k_end = min(K, k_begin + kslice);
     const __amdgpu_buffer_rsrc_t rsa = make_rsrc(A, (size_t)M * K * sizeof(float)), rsb = make_rsrc(B, (size_t)K * N * sizeof(float));
@@ -439,6 +441,17 @@ __global__ __launch_bounds__(64 * kSmallWaves) void sgemm_small_k(int M, int N, 
     }
 }
 
+template <bool kTA, bool kTB, bool kVA, bool kVB>
+__global__ __launch_bounds__(64 * kSmallWaves) void sgemm_small_k(int M, int N, int K, int lda, int ldb, int kslice,
+                                                                   const float *A, const float *B, float *C,
+                                                                   const float *colbias, int bias_shift,
+                                                                   const float *rowvec, int relu, const float *mask)
+{
+    __shared__ float red[kSmallWaves][32 * 33];
+    sgemm_small_body<kTA, kTB, kVA, kVB>(M, N, K, lda, ldb, kslice, A, B, C, colbias, bias_shift, rowvec, relu, mask,
+                                         (int)blockIdx.x, (int)blockIdx.y, red);
+}
+
 // Short reductions over large outputs with both operands stored k-major (A as [K][M], B as [K][N]:
 // the product x^T * dy of a filter gradient).  With K <= 128 a 128 x 128 output tile needs 128 KB of
 // operands, which fit in LDS whole: every load of the block is issued before the first multiply, so
@@ -460,13 +473,13 @@ __device__ __forceinline__ float4 panel_load(const float *X, int ld, int k, int 
 // nine tap sums of every (k, c) pair to C[k][c][3][3] instead of the 4 x 4 block itself: tap (a, b)
 // collects the pixel pairs with 1 - iy + oy == a and 1 - ix + ox == b.
 template <bool kFold>
-__global__ __launch_bounds__(kPanelThreads) void sgemm_panel_k(int M, int N, int K, int mtiles, int ntiles, const float *A,
-                                                                const float *B, float *C)
+__device__ __forceinline__ void sgemm_panel_body(int M, int N, int K, int mtiles, int ntiles, const float *A, const float *B,
+                                                 float *C, unsigned bid)
 {
     extern __shared__ __attribute__((aligned(16))) float panel_lds[];
     float *As = panel_lds, *Bs = panel_lds + kPanelK * kPanelLd;
     unsigned L;
-    if (!xcd_remap(blockIdx.x, (unsigned)(mtiles * ntiles), &L)) return;
+    if (!xcd_remap(bid, (unsigned)(mtiles * ntiles), &L)) return;
     const int m0 = (int)(L % (unsigned)mtiles) * kPanelTile, n0 = (int)(L / (unsigned)mtiles) * kPanelTile;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, wm = w >> 2, wn = w & 3;
 
@@ -549,6 +562,36 @@ __global__ __launch_bounds__(kPanelThreads) void sgemm_panel_k(int M, int N, int
     }
 }
 
+template <bool kFold>
+__global__ __launch_bounds__(kPanelThreads) void sgemm_panel_k(int M, int N, int K, int mtiles, int ntiles, const float *A,
+                                                                const float *B, float *C)
+{
+    sgemm_panel_body<kFold>(M, N, K, mtiles, ntiles, A, B, C, blockIdx.x);
+}
+
+// Several such products in one launch (the filter gradients of consecutive 2x2-image layers wait for nothing but their
+// own dy): job j owns the blocks from first[j] on, a multiple of 8 each, so a block's place among the XCDs is what it
+// would be in a launch of its own.
+struct PanelJob {
+    int M, N, K, mtiles, ntiles;
+    unsigned first;
+    const float *A, *B;
+    float *C;
+};
+struct PanelGroup {
+    PanelJob j[kGroupJobs];
+    int n;
+};
+
+template <bool kFold>
+__global__ __launch_bounds__(kPanelThreads) void sgemm_panel_group_k(PanelGroup g)
+{
+    int j = 0;
+    while (j + 1 < g.n && blockIdx.x >= g.j[j + 1].first) j++;
+    const PanelJob &q = g.j[j];
+    sgemm_panel_body<kFold>(q.M, q.N, q.K, q.mtiles, q.ntiles, q.A, q.B, q.C, blockIdx.x - q.first);
+}
+
 __global__ __launch_bounds__(256) void splitk_reduce_k(size_t n, int splits, const float *partial, float *out)
 {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
@@ -606,27 +649,78 @@ __global__ __launch_bounds__(256) void gemv_cols_k(size_t K, size_t N, size_t ks
 // The same for a short reduction (K <= 256) in one launch: a block takes 64 columns, its four
 // groups of 64 threads take every fourth k, sixteen loads in flight per thread (clamped, not
 // branched), and the four sums are added in group order through LDS.
+// (`on`: false for the threads of a larger block that only keep the barrier company)
+__device__ __forceinline__ void gemv_cols_short_body(int K, int N, const float *a, const float *B, float *c, int bx, bool on,
+                                                     float (*part)[64])
+{
+    const int col = threadIdx.x & 63, kl = (threadIdx.x >> 6) & 3;
+    const int n = min(bx * 64 + col, N - 1);
+    float acc = 0.0f;
+    if (on) {
+        for (int k0 = kl; k0 < K; k0 += 64) {
+            float av[16], bv[16];
+#pragma unroll
+            for (int u = 0; u < 16; u++) {
+                const int k = min(k0 + 4 * u, K - 1);
+                av[u] = a[k];
+                bv[u] = B[(size_t)k * N + n];
+            }
+#pragma unroll
+            for (int u = 0; u < 16; u++)
+                if (k0 + 4 * u < K) acc += av[u] * bv[u];
+        }
+        part[kl][col] = acc;
+    }
+    __syncthreads();
+    if (on && kl == 0 && bx * 64 + col < N) c[n] = ((part[0][col] + part[1][col]) + part[2][col]) + part[3][col];
+}
+
 __global__ __launch_bounds__(256) void gemv_cols_short_k(int K, int N, const float *a, const float *B, float *c)
 {
     __shared__ float part[4][64];
-    const int col = threadIdx.x & 63, kl = threadIdx.x >> 6;
-    const int n = min((int)blockIdx.x * 64 + col, N - 1);
-    float acc = 0.0f;
-    for (int k0 = kl; k0 < K; k0 += 64) {
-        float av[16], bv[16];
-#pragma unroll
-        for (int u = 0; u < 16; u++) {
-            const int k = min(k0 + 4 * u, K - 1);
-            av[u] = a[k];
-            bv[u] = B[(size_t)k * N + n];
-        }
-#pragma unroll
-        for (int u = 0; u < 16; u++)
-            if (k0 + 4 * u < K) acc += av[u] * bv[u];
+    gemv_cols_short_body(K, N, a, B, c, (int)blockIdx.x, true, part);
+}
+
+// Several independent small products in ONE launch: the weight and bias gradients of a dense head are six kernels of a
+// few microseconds each that wait for nothing but the gradient in front of them, and a kernel boundary costs as much as
+// one of them runs.  A block finds its job by its index; each job runs the body of the kernel it would have run alone
+// (32 x 32-tile products of one template instance, and column sums of short reductions), so every value is what the
+// separate launches give.
+struct SmallJob {
+    int M, N, K, lda, ldb, kslice, nx, first;   // nx: tiles per row of tiles; first: the job's first block
+    const float *A, *B;
+    float *C;
+};
+struct GemvJob {
+    int K, N, first, pad;
+    const float *a, *B;
+    float *c;
+};
+struct SmallGroup {
+    SmallJob s[kGroupJobs];
+    GemvJob v[kGroupJobs];
+    int ns, nv;
+};
+
+template <bool kTA, bool kTB, bool kVA, bool kVB>
+__global__ __launch_bounds__(64 * kSmallWaves) void sgemm_small_group_k(SmallGroup g)
+{
+    __shared__ float red[kSmallWaves][32 * 33];
+    __shared__ float part[4][64];
+    const int b = (int)blockIdx.x;   // uniform: the scans below stay scalar
+    if (g.nv > 0 && b >= g.v[0].first) {
+        int j = 0;
+        while (j + 1 < g.nv && b >= g.v[j + 1].first) j++;
+        const GemvJob &q = g.v[j];
+        gemv_cols_short_body(q.K, q.N, q.a, q.B, q.c, b - q.first, threadIdx.x < 256, part);
+        return;
     }
-    part[kl][col] = acc;
-    __syncthreads();
-    if (kl == 0 && (int)blockIdx.x * 64 + col < N) c[n] = ((part[0][col] + part[1][col]) + part[2][col]) + part[3][col];
+    int j = 0;
+    while (j + 1 < g.ns && b >= g.s[j + 1].first) j++;
+    const SmallJob &q = g.s[j];
+    const int local = b - q.first;
+    sgemm_small_body<kTA, kTB, kVA, kVB>(q.M, q.N, q.K, q.lda, q.ldb, q.kslice, q.A, q.B, q.C, nullptr, 0, nullptr, 0, nullptr,
+                                         local % q.nx, local / q.nx, red);
 }
 
 // c[m][n] = relu?(c[m][n] + u[m] * v[n]): the epilogue of dopt_hip_sgemm_rank1 as a pass of its own, for the
@@ -673,12 +767,37 @@ int panel_launch(bool fold, size_t M, size_t N, size_t K, const float *A, const 
                                            (int)kPanelLds));
         DOPT_HIP_CHECK(hipFuncSetAttribute((const void *)sgemm_panel_k<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)kPanelLds));
+        DOPT_HIP_CHECK(hipFuncSetAttribute((const void *)sgemm_panel_group_k<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)kPanelLds));
         raised = true;
     }
+    if (M == 0) return DOPT_HIP_OK;   // called for the attributes only
     const int mt = (int)ceil_div(M, (size_t)kPanelTile), nt = (int)ceil_div(N, (size_t)kPanelTile);
     const dim3 grid(xcd_grid((unsigned)(mt * nt))), block(kPanelThreads);
     if (fold) hipLaunchKernelGGL(sgemm_panel_k<true>, grid, block, kPanelLds, stream(), (int)M, (int)N, (int)K, mt, nt, A, B, C);
     else hipLaunchKernelGGL(sgemm_panel_k<false>, grid, block, kPanelLds, stream(), (int)M, (int)N, (int)K, mt, nt, A, B, C);
+    DOPT_LAUNCH_CHECK();
+    return DOPT_HIP_OK;
+}
+
+// `n` folded filter-gradient products (all of them shapes panel_takes accepts) as one launch.
+int panel_fold_group_launch(int n, const size_t *M, const size_t *N, const size_t *K, const float *const *A,
+                            const float *const *B, float *const *C)
+{
+    if (int rc = panel_launch(true, 0, 0, 0, nullptr, nullptr, nullptr)) return rc;
+    PanelGroup g{};
+    unsigned blocks = 0;
+    for (int i = 0; i < n; i++) {
+        PanelJob &q = g.j[i];
+        q.M = (int)M[i]; q.N = (int)N[i]; q.K = (int)K[i];
+        q.mtiles = (int)ceil_div(M[i], (size_t)kPanelTile);
+        q.ntiles = (int)ceil_div(N[i], (size_t)kPanelTile);
+        q.first = blocks;
+        q.A = A[i]; q.B = B[i]; q.C = C[i];
+        blocks += xcd_grid((unsigned)(q.mtiles * q.ntiles));
+    }
+    g.n = n;
+    hipLaunchKernelGGL(sgemm_panel_group_k<true>, dim3(blocks), dim3(kPanelThreads), kPanelLds, stream(), g);
     DOPT_LAUNCH_CHECK();
     return DOPT_HIP_OK;
 }
@@ -922,9 +1041,107 @@ bool sgemm_fold2x2(size_t C, size_t K, size_t N, const float *x, const float *dy
     return true;
 }
 
+// The same for `n` layers at once (n <= 8): one launch when every layer suits the LDS-resident kernel, else false with
+// nothing launched.
+bool sgemm_fold2x2_batch(int n, const size_t *C, const size_t *K, const size_t *N, const float *const *x,
+                         const float *const *dy, float *const *dw, int *rc)
+{
+    if (n < 1 || n > kGroupJobs) return false;
+    size_t M4[kGroupJobs], N4[kGroupJobs];
+    for (int i = 0; i < n; i++) {
+        if (!panel_takes(4 * C[i], 4 * K[i], N[i], x[i], dy[i])) return false;
+        M4[i] = 4 * C[i];
+        N4[i] = 4 * K[i];
+    }
+    *rc = panel_fold_group_launch(n, M4, N4, N, x, dy, dw);
+    return true;
+}
+
 }  // namespace dopt
 
 extern "C" {
+
+int dopt_hip_sgemm_batch(int n, const int *transA, const int *transB, const size_t *M, const size_t *N, const size_t *K,
+                         const float *const *A, const float *const *B, float *const *C)
+{
+    using namespace dopt;
+    DOPT_REQUIRE(n >= 0 && (n == 0 || (transA && transB && M && N && K && A && B && C)), "dopt_hip_sgemm_batch: null argument");
+    DOPT_ENSURE_INIT();
+    // Products that take the 32 x 32-tile kernel (grouped per template instance) or the short column sum share launches;
+    // the others run one by one.  Outputs must not overlap any operand of the batch: the order inside it is not kept.
+    struct Inst { bool ta, tb, va, vb; SmallGroup g; unsigned blocks; bool used; };
+    std::vector<Inst> insts;
+    std::vector<GemvJob> gemvs;
+    std::vector<int> single;
+    for (int i = 0; i < n; i++) {
+        if (M[i] * N[i] == 0) continue;
+        const bool plain = K[i] > 0 && A[i] && B[i] && C[i] && M[i] < ((size_t)1 << 30) && N[i] < ((size_t)1 << 30) && K[i] < ((size_t)1 << 30);
+        const Route r = plain ? sgemm_route(transA[i], transB[i], M[i], N[i], K[i]) : Route{Route::kNone, 1, 0};
+        if (r.kind == Route::kGemvColsShort && gemvs.size() < (size_t)kGroupJobs) {
+            const size_t R = M[i] == 1 ? N[i] : M[i];
+            GemvJob q{};
+            q.K = (int)K[i]; q.N = (int)R;
+            q.a = M[i] == 1 ? A[i] : B[i];
+            q.B = M[i] == 1 ? B[i] : A[i];
+            q.c = C[i];
+            gemvs.push_back(q);
+        } else if (r.kind == Route::kSmall) {
+            const int lda = (int)(transA[i] ? M[i] : K[i]), ldb = (int)(transB[i] ? K[i] : N[i]);
+            const bool ta = transA[i] != 0, tb = transB[i] != 0;
+            const bool va = !ta && aligned16(A[i]) && lda % 4 == 0, vb = tb && aligned16(B[i]) && ldb % 4 == 0;
+            // the instance the product would take alone (flags an instance does not read are false there)
+            const bool iva = ta ? false : va, ivb = tb ? vb : false;
+            Inst *in = nullptr;
+            for (Inst &c : insts)
+                if (c.ta == ta && c.tb == tb && c.va == iva && c.vb == ivb && c.g.ns < kGroupJobs) in = &c;
+            if (!in) {
+                insts.push_back(Inst{ta, tb, iva, ivb, SmallGroup{}, 0, false});
+                in = &insts.back();
+            }
+            SmallJob &q = in->g.s[in->g.ns++];
+            q.M = (int)M[i]; q.N = (int)N[i]; q.K = (int)K[i]; q.lda = lda; q.ldb = ldb;
+            q.kslice = (int)ceil_div(ceil_div(K[i], (size_t)kSmallWaves), (size_t)8) * 8;
+            q.nx = (int)ceil_div(N[i], (size_t)32);
+            q.first = (int)in->blocks;
+            q.A = A[i]; q.B = B[i]; q.C = C[i];
+            in->blocks += (unsigned)(q.nx * ceil_div(M[i], (size_t)32));
+        } else {
+            single.push_back(i);
+        }
+    }
+    for (size_t k = 0; k < insts.size(); k++) {
+        Inst &in = insts[k];
+        if (k == 0) {   // the column sums ride in the first launch
+            for (const GemvJob &v : gemvs) {
+                GemvJob &q = in.g.v[in.g.nv++];
+                q = v;
+                q.first = (int)in.blocks;
+                in.blocks += (unsigned)ceil_div((size_t)v.N, (size_t)64);
+            }
+            gemvs.clear();
+        }
+        const dim3 grid(in.blocks), block(64 * kSmallWaves);
+#define DOPT_GROUP(TA, TB, VA, VB) hipLaunchKernelGGL((sgemm_small_group_k<TA, TB, VA, VB>), grid, block, 0, stream(), in.g)
+        if (in.ta && in.tb) { if (in.vb) DOPT_GROUP(true, true, false, true); else DOPT_GROUP(true, true, false, false); }
+        else if (in.ta) DOPT_GROUP(true, false, false, false);
+        else if (in.tb) {
+            if (in.va && in.vb) DOPT_GROUP(false, true, true, true);
+            else if (in.va) DOPT_GROUP(false, true, true, false);
+            else if (in.vb) DOPT_GROUP(false, true, false, true);
+            else DOPT_GROUP(false, true, false, false);
+        } else { if (in.va) DOPT_GROUP(false, false, true, false); else DOPT_GROUP(false, false, false, false); }
+#undef DOPT_GROUP
+        DOPT_LAUNCH_CHECK();
+    }
+    for (const GemvJob &v : gemvs) {   // no 32 x 32-tile launch to ride in
+        hipLaunchKernelGGL(gemv_cols_short_k, dim3((unsigned)ceil_div((size_t)v.N, (size_t)64)), dim3(256), 0, stream(), v.K, v.N,
+                           v.a, v.B, v.c);
+        DOPT_LAUNCH_CHECK();
+    }
+    for (int i : single)
+        if (int rc = dopt_hip_sgemm_t(transA[i], transB[i], M[i], N[i], K[i], A[i], B[i], C[i])) return rc;
+    return DOPT_HIP_OK;
+}
 
 int dopt_hip_sgemm_rank1(int transA, int transB, size_t M, size_t N, size_t K, const float *A, const float *B,
                          const float *u, const float *v, int relu, float *C)

@@ -177,6 +177,13 @@ int dopt_hip_sgemm(size_t M, size_t N, size_t K, const float *A, const float *B,
    the `transpose` kernels that only feed a matmul. */
 int dopt_hip_sgemm_t(int transA, int transB, size_t M, size_t N, size_t K, const float *A,
                      const float *B, float *C);
+/* `n` independent products in one call, each computed exactly as dopt_hip_sgemm_t computes it (same kernel body, same
+   order of summation).  The reference issues one cublasSgemm per matmul (cuda/math.d:234-235); the weight and bias
+   gradients of a dense head are products that wait for nothing but the gradient in front of them, and those among
+   them that take the small-output kernel or the short column sum share launches here.  No C may overlap an operand
+   of another job: the order inside the batch is not kept. */
+int dopt_hip_sgemm_batch(int n, const int *transA, const int *transB, const size_t *M, const size_t *N, const size_t *K,
+                         const float *const *A, const float *const *B, float *const *C);
 /* Names the order in which dopt_hip_sgemm_t adds the K terms of an output element for these flags and dimensions
    (which kernel runs, and where it cuts the reduction): two calls with equal values give equal bits for equal
    operand values, also when one computes the transpose of the other's product, (A B)^T = B^T A^T with M and N
@@ -291,6 +298,11 @@ int dopt_hip_conv_pair_probe_read(int *launches, double *total_us, double *flops
 int dopt_hip_split_sum_close(const dopt_hip_split_sum *open);
 /* `convolutionFiltersGrad`: cudnnConvolutionBackwardFilter, cudnn7.d:244. */
 int dopt_hip_conv_bwd_filter(const dopt_hip_conv_desc *d, const float *dy, const float *x, float *dw);
+/* `n` independent filter gradients in one call, each as dopt_hip_conv_bwd_filter computes it (the reference runs one
+   cudnnConvolutionBackwardFilter per layer, cudnn7.d:244; none of them reads another's result).  Runs of 2x2-image
+   layers share one launch; no dw may overlap another job's operands. */
+int dopt_hip_conv_bwd_filter_batch(int n, const dopt_hip_conv_desc *descs, const float *const *dy, const float *const *x,
+                                   float *const *dw);
 
 /* ---------------------------------------------------------------------------------------
  * Bandwidth-bound NN ops (fp32, NCHW; `inner` = product of the dims after the channel dim).

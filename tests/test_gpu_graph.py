@@ -543,6 +543,86 @@ def test_backward_data_and_filter_gradient_as_one_call(xs, k):
     ops.sync()
 
 
+def test_batched_products_and_filter_gradients_match_single_calls():
+    """dopt_hip_sgemm_batch / dopt_hip_conv_bwd_filter_batch against one dopt_hip_sgemm_t / dopt_hip_conv_bwd_filter per
+    job: the jobs that share a launch run the kernel body they would run alone, so every result is identical."""
+    lib = capi.load()
+    r = np.random.default_rng(70)
+    jobs = [(1, 0, 512, 512, 128),    # dense weight gradients: small-output kernel, A stored [K][M]
+            (1, 0, 10, 512, 128),
+            (1, 0, 512, 512, 128),
+            (0, 0, 1, 512, 128),      # bias gradients: short column sums
+            (0, 0, 1, 10, 128),
+            (1, 0, 37, 1, 100),       # ... of a transposed matrix
+            (0, 1, 128, 512, 512),    # small-output kernel, another instance (quads on both operands)
+            (0, 0, 70, 33, 50),       # ... and a third (scalar loads)
+            (0, 0, 300, 1, 77),       # a row-wise matrix-vector product: runs on its own
+            (1, 0, 2048, 2048, 128),  # the LDS-resident panel kernel: on its own
+            (0, 0, 16, 4, 1),         # K = 1
+            (0, 0, 8, 0, 5)]          # nothing to do
+    A, B, want, got = [], [], [], []
+    for ta, tb, M, N, K in jobs:
+        a = ops.tensor(r.standard_normal((K, M) if ta else (M, K)).astype(np.float32))
+        b = ops.tensor(r.standard_normal((N, K) if tb else (K, N)).astype(np.float32))
+        w, o = ops.Tensor((M, N)), ops.Tensor((M, N))
+        if M * N:
+            capi.check(lib.dopt_hip_sgemm_t(ta, tb, M, N, K, a.ptr, b.ptr, w.ptr))
+            o.set(np.full((M, N), np.nan, np.float32))
+        A.append(a); B.append(b); want.append(w); got.append(o)
+    n = len(jobs)
+    arr = lambda t, vals: (t * n)(*vals)
+    capi.check(lib.dopt_hip_sgemm_batch(n, arr(C.c_int, [j[0] for j in jobs]), arr(C.c_int, [j[1] for j in jobs]),
+                                        arr(C.c_size_t, [j[2] for j in jobs]), arr(C.c_size_t, [j[3] for j in jobs]),
+                                        arr(C.c_size_t, [j[4] for j in jobs]), arr(C.c_void_p, [t.ptr for t in A]),
+                                        arr(C.c_void_p, [t.ptr for t in B]), arr(C.c_void_p, [t.ptr for t in got])))
+    for j, w, o in zip(jobs, want, got):
+        if j[2] * j[3]:
+            assert np.array_equal(o.numpy(), w.numpy()), j
+    # filter gradients: three 2x2-image layers in a row share a launch, the 4x4 layer and the narrow one run as ever
+    shapes = [((128, 512, 2, 2), 512), ((128, 512, 2, 2), 512), ((128, 256, 2, 2), 512), ((8, 64, 4, 4), 32), ((128, 24, 2, 2), 40),
+              ((128, 512, 2, 2), 512)]
+    descs, dys, xs, want, got = [], [], [], [], []
+    for xshape, k in shapes:
+        d = ops.conv_desc(xshape, (k, xshape[1], 3, 3), (1, 1), (1, 1))
+        dy = ops.tensor(r.standard_normal((xshape[0], k, xshape[2], xshape[3])).astype(np.float32))
+        x = ops.tensor(r.standard_normal(xshape).astype(np.float32))
+        w, o = ops.Tensor((k, xshape[1], 3, 3)), ops.Tensor((k, xshape[1], 3, 3))
+        capi.check(lib.dopt_hip_conv_bwd_filter(C.byref(d), dy.ptr, x.ptr, w.ptr))
+        o.set(np.full(o.shape, np.nan, np.float32))
+        descs.append(d); dys.append(dy); xs.append(x); want.append(w); got.append(o)
+    n = len(shapes)
+    capi.check(lib.dopt_hip_conv_bwd_filter_batch(n, (type(descs[0]) * n)(*descs), (C.c_void_p * n)(*[t.ptr for t in dys]),
+                                                  (C.c_void_p * n)(*[t.ptr for t in xs]), (C.c_void_p * n)(*[t.ptr for t in got])))
+    for sh, w, o in zip(shapes, want, got):
+        assert np.array_equal(o.numpy(), w.numpy()), sh
+    ops.sync()
+
+
+def test_output_only_products_of_a_plan_share_a_launch():
+    """The weight and bias gradients of a dense head feed nothing but the plan's outputs: with the rewrites on they are
+    one step (`matmul*N`), and so are the filter gradients of consecutive 2x2-image layers; the values are those of the
+    plan without rewrites."""
+    r = np.random.default_rng(71)
+    X = r.standard_normal((128, 3, 8, 8)).astype(np.float32)
+    Y = np.eye(10, dtype=np.float32)[r.integers(0, 10, 128)]
+    feats, labels = float32([128, 3, 8, 8]), float32([128, 10])
+    init = nnet.Init(72)
+    body = nnet.vgg(feats, [64, -1, 128, -1, 128, 128], [64], init)     # the last two convolutions see 2x2 images
+    preds = nnet.softmax(nnet.dense(body, 10, init))
+    net = nnet.DAGNetwork([feats], [preds])
+    loss = nnet.crossEntropy(preds.trainOutput, labels) + net.paramLoss
+    outs = [loss] + core.grad(loss, net.params)
+    plan = core.compile(outs, core.PLAN_VIEWS | core.PLAN_FUSE | core.PLAN_TIMING)
+    fused = plan.execute({feats: X, labels: Y})
+    prof = plan.profile()
+    # (the product left over is the gradient that flows on into the convolutions: something reads it)
+    assert prof["matmul*4"][1] == 1 and prof["matmul"][1] == 1 and "matmul+transpose" not in prof, prof
+    assert prof["convolutionFiltersGrad*2"][1] == 1, prof
+    plain = core.compile(outs, core.PLAN_VIEWS).execute({feats: X, labels: Y})
+    for a, b in zip(plain, fused):
+        assert np.array_equal(a, b) or (a.ndim == 1 and np.allclose(a, b, rtol=0, atol=2e-5))
+
+
 @pytest.mark.parametrize("M,N,K,ta,tb", [(128, 512, 512, 0, 0),     # the small-output kernel: the epilogue does it
                                           (512, 512, 128, 1, 0),     # a weight gradient: dz stored [K][M]
                                           (10, 512, 128, 1, 0),
