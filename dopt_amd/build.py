@@ -13,9 +13,9 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(HERE, "libdopthip.so")
 
-SOURCES = ["runtime.cpp", "rtc_ops.cpp", "layout.hip", "nn.hip", "bn.hip", "optim.hip", "sgemm.hip", "conv.hip", "conv_smallc.hip",
+SOURCES = ["runtime.cpp", "rtc_ops.cpp", "layout.hip", "nn.hip", "bn.hip", "optim.hip", "sgemm.hip", "conv.hip", "conv_smallc.hip", "tiny.hip",
            "plan.cpp"]
-HEADERS = ["common.h", "mfma_core.h", "pool2x2.h", "plan.h", os.path.join("..", "..", "include", "dopt_hip.h"),
+HEADERS = ["common.h", "mfma_core.h", "pool2x2.h", "pw_ops.h", "plan.h", os.path.join("..", "..", "include", "dopt_hip.h"),
            os.path.join("..", "..", "include", "dopt_hip_plan.h")]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

@@ -20,6 +20,12 @@ class HipError(RuntimeError):
         self.code = code
 
 
+class TinyNode(C.Structure):
+    """dopt_hip_tiny_node of include/dopt_hip.h."""
+    _fields_ = [(n, C.c_int) for n in ("kind", "op", "dst", "a", "b", "a_kind", "b_kind", "n", "dst_offset", "a_offset",
+                                       "b_offset")] + [("dims", C.c_int * 4), ("reps", C.c_int * 4)]
+
+
 class ConvDesc(C.Structure):
     _fields_ = [(n, C.c_size_t) for n in
                 ("N", "C", "H", "W", "K", "R", "S", "padH", "padW", "strideH", "strideW")]
@@ -66,6 +72,8 @@ PROTOTYPES = {
                                  C.POINTER(_i), C.POINTER(_i), _vp],
     "dopt_hip_pointwise_chain_compile_only": [_i, _i, C.POINTER(C.c_ubyte), _i, C.POINTER(C.c_char_p), C.POINTER(_i),
                                               C.POINTER(_i), C.c_char_p],
+    "dopt_hip_pointwise_index": [C.c_char_p],
+    "dopt_hip_tiny_graph": [_i, C.POINTER(_vp), _i, C.POINTER(TinyNode)],
     "dopt_hip_pointwise_arity": [C.c_char_p],
     "dopt_hip_reduce": [C.c_char_p, _i, _szp, _i, _szp, _i, _vp, _vp],
     "dopt_hip_argmin": [_i, _szp, _i, _sz, _vp, _vp],

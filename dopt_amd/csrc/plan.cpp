@@ -596,6 +596,7 @@ struct HIPPlan::Builder {
     std::vector<int> pairLead;                  // the operation of such a pair that comes first in the order -> the backward-data op
     std::vector<char> pairLater;                // the operation of such a pair that comes second: no step of its own
     std::vector<char> absorbed;
+    std::vector<std::vector<int>> tinyWrites;   // last member of a run of tiny operations -> the other members
     std::vector<char> needed;
     // late: the copy is made right in front of its first reader instead of at the start of the run
     struct Prepack { int op, filter; int bwd; dopt_hip_conv_desc d; void *buf; bool owner, late; };
@@ -614,7 +615,7 @@ struct HIPPlan::Builder {
           inputsOf((size_t)nops), fusedKind((size_t)nops, 0), prebuilt((size_t)nops), prebuiltLabel((size_t)nops),
           live((size_t)nops, 0), uses((size_t)nops), exposed((size_t)nops), biasGradOf((size_t)nops, -1), poolOf((size_t)nops, -1), pairOf((size_t)nops, -1), pairLead((size_t)nops, -1),
           pairLater((size_t)nops, 0),
-          absorbed((size_t)nops, 0), needed((size_t)nops, 0), packOf((size_t)nops, -1), mmInfo((size_t)nops)
+          absorbed((size_t)nops, 0), tinyWrites((size_t)nops), needed((size_t)nops, 0), packOf((size_t)nops, -1), mmInfo((size_t)nops)
     {
     }
 
@@ -637,6 +638,7 @@ struct HIPPlan::Builder {
     void fuseDenseLayers();
     void fuseDenseBackward();
     bool plainProduct(int id, MatmulInfo *mi, bool sole_reader) const;
+    void formTinyRuns();
     void formChains();
     void absorbBiasGrads();
     void absorbPools();
@@ -972,6 +974,208 @@ void HIPPlan::Builder::fuseDenseBackward()
             fusedKind[pid] = 0;
         }
     }
+}
+
+// Runs of operations on tiny tensors (a softmax over ten classes, the loss behind it, the scalars of an update rule):
+// each would be a kernel that lasts as long as the gap between two kernels.  Walking the order, operations that
+// dopt_hip_tiny_graph can compute (every tensor involved of at most DOPT_HIP_TINY_ELEMS fp32 values) collect into a
+// run; an operation outside that reads a member ends it, so the run can stand where its last member stood: all it
+// reads is older, all that reads it comes later.  The run is one step; every member keeps its buffer and gets its
+// value there, computed as its own kernel computes it.
+void HIPPlan::Builder::formTinyRuns()
+{
+    const size_t cap = DOPT_HIP_TINY_ELEMS;
+    // operations whose values the plan as rewritten so far still computes (a product that a dense-layer kernel absorbed
+    // is read by nobody): reachable from the outputs through what each kernel reads.  A run's step stands where its last
+    // member does, so a member nobody needs must not be the one to carry it.
+    std::vector<char> read((size_t)nops, 0);
+    {
+        std::vector<int> work(outputs.begin(), outputs.end());
+        while (!work.empty()) {
+            const int id = work.back();
+            work.pop_back();
+            if (read[id]) continue;
+            read[id] = 1;
+            if (alias[id].source >= 0) work.push_back(alias[id].source);
+            else for (int d : inputsOf[id]) work.push_back(d);
+        }
+    }
+    auto small_f32 = [&](int id) { return g.ops[id].dtype == DOPT_HIP_F32 && g.ops[id].volume() >= 1 && g.ops[id].volume() <= cap; };
+    // what a member is to the kernel; false when it cannot be one
+    auto describe = [&](int id, dopt_hip_tiny_node *nd, int (&operands)[2]) -> bool {
+        const Operation &o = g.ops[id];
+        if (!live[id] || alias[id].source >= 0 || fusedKind[id] || prebuilt[id] || !small_f32(id)) return false;
+        if (!read[id]) return false;
+        for (int d : o.deps)
+            if (!small_f32(d)) return false;
+        *nd = dopt_hip_tiny_node{};
+        nd->n = (int)o.volume();
+        nd->b = -1;
+        operands[0] = operands[1] = -1;
+        if (o.opType == "reluGrad" && o.deps.size() == 3) {
+            for (const Use &u : uses[id])
+                if (fusedKind[u.op] == 3 || fusedKind[u.op] == 8) return false;   // that batchNormGrad reads dy and y itself
+            if (g.ops[o.deps[0]].volume() != o.volume() || g.ops[o.deps[2]].volume() != o.volume()) return false;
+            nd->kind = DOPT_HIP_TINY_POINTWISE;
+            nd->op = dopt_hip_pointwise_index("reluGrad");
+            operands[0] = o.deps[0];
+            operands[1] = o.deps[2];
+            return true;
+        }
+        if (o.opType == "matmul" && o.deps.size() == 2 && o.rank() == 2) {   // [m,1] x [1,n]: a column times a row
+            const Operation &l = g.ops[o.deps[0]], &r = g.ops[o.deps[1]];
+            if (l.rank() != 2 || r.rank() != 2 || l.shape[1] != 1 || r.shape[0] != 1) return false;
+            nd->kind = DOPT_HIP_TINY_POINTWISE;
+            nd->op = dopt_hip_pointwise_index("mul");
+            nd->a_kind = 2;
+            nd->b_kind = 3;
+            nd->dims[0] = (int)o.shape[1];
+            operands[0] = o.deps[0];
+            operands[1] = o.deps[1];
+            return true;
+        }
+        const int arity = o.opType == "relu" ? 1 : dopt_hip_pointwise_arity(o.opType.c_str());
+        if (arity > 0 && o.opType != "reluGrad") {
+            if (arity != (int)o.deps.size()) return false;
+            for (int d : o.deps)
+                if (g.ops[d].volume() != o.volume()) return false;
+            nd->kind = DOPT_HIP_TINY_POINTWISE;
+            nd->op = dopt_hip_pointwise_index(o.opType.c_str());
+            operands[0] = o.deps[0];
+            if (arity == 2) operands[1] = o.deps[1];
+            return nd->op >= 0;
+        }
+        if ((o.opType == "sum" || o.opType == "maxElement") && o.deps.size() == 1) {
+            const auto *axes = sizes_attr(o, "axes");
+            const auto &sh = g.ops[o.deps[0]].shape;
+            if (!axes || axes->empty() || sh.empty() || sh.size() > 16) return false;
+            std::vector<char> red(sh.size(), 0);
+            for (size_t a : *axes) {
+                if (a >= sh.size() || red[a]) return false;
+                red[a] = 1;
+            }
+            size_t first = sh.size(), last = 0;
+            for (size_t i = 0; i < sh.size(); i++)
+                if (red[i]) { first = std::min(first, i); last = i; }
+            for (size_t i = first; i <= last; i++)
+                if (!red[i]) return false;   // more than one run of reduced axes: passes with a temporary in between
+            size_t outer = 1, R = 1, inner = 1;
+            for (size_t i = 0; i < first; i++) outer *= sh[i];
+            for (size_t i = first; i <= last; i++) R *= sh[i];
+            for (size_t i = last + 1; i < sh.size(); i++) inner *= sh[i];
+            nd->kind = DOPT_HIP_TINY_REDUCE;
+            nd->op = o.opType == "sum" ? 0 : 1;
+            nd->dims[0] = (int)outer; nd->dims[1] = (int)R; nd->dims[2] = (int)inner;
+            operands[0] = o.deps[0];
+            return outer * inner == o.volume();
+        }
+        if ((o.opType == "softmax" && o.deps.size() == 1) || (o.opType == "softmaxGrad" && o.deps.size() == 2)) {
+            if (o.rank() < 2) return false;
+            size_t N, C, inner;
+            nci(o.shape, &N, &C, &inner);
+            if (inner == 1 && C >= 64) return false;   // such rows take the wavefront-per-row kernels
+            for (int d : o.deps)
+                if (g.ops[d].volume() != o.volume()) return false;
+            nd->kind = o.opType == "softmax" ? DOPT_HIP_TINY_SOFTMAX : DOPT_HIP_TINY_SOFTMAX_GRAD;
+            nd->dims[0] = (int)N; nd->dims[1] = (int)C; nd->dims[2] = (int)inner;
+            operands[0] = o.deps[0];
+            if (o.deps.size() == 2) operands[1] = o.deps[1];
+            return true;
+        }
+        if (o.opType == "repeat" && o.deps.size() == 1) {
+            const auto *reps = sizes_attr(o, "repetitions");
+            const auto &sh = g.ops[o.deps[0]].shape;
+            if (!reps || reps->size() != sh.size() || sh.size() > 4) return false;
+            nd->kind = DOPT_HIP_TINY_REPEAT;
+            for (int d = 0; d < 4; d++) nd->dims[d] = nd->reps[d] = 1;
+            const size_t lead = 4 - sh.size();
+            for (size_t i = 0; i < sh.size(); i++) {
+                nd->dims[lead + i] = (int)sh[i];
+                nd->reps[lead + i] = (int)(*reps)[i];
+            }
+            operands[0] = o.deps[0];
+            return true;
+        }
+        return false;
+    };
+    struct Member { int op; dopt_hip_tiny_node nd; int operands[2]; };
+    std::vector<Member> run;
+    std::vector<char> inRun((size_t)nops, 0);
+    auto close = [&]() {
+        if (run.size() >= 2) {
+            // buffers: the members' own, and whatever else they read (by owner of the buffer, with the byte offset in the node)
+            std::vector<int> slots;
+            auto slot_of = [&](int owner) {
+                for (size_t k = 0; k < slots.size(); k++)
+                    if (slots[k] == owner) return (int)k;
+                slots.push_back(owner);
+                return (int)slots.size() - 1;
+            };
+            std::vector<dopt_hip_tiny_node> nodes;
+            bool fits = true;
+            for (Member &m : run) {
+                dopt_hip_tiny_node nd = m.nd;
+                nd.dst = slot_of(m.op);
+                for (int k = 0; k < 2; k++) {
+                    if (m.operands[k] < 0) continue;
+                    size_t off;
+                    const int r = root(m.operands[k], &off);
+                    if (off > 0x7fffffffu) fits = false;
+                    (k == 0 ? nd.a : nd.b) = slot_of(r);
+                    (k == 0 ? nd.a_offset : nd.b_offset) = (int)off;
+                }
+                nodes.push_back(nd);
+            }
+            if (fits && slots.size() <= (size_t)DOPT_HIP_TINY_SLOTS && nodes.size() <= (size_t)DOPT_HIP_TINY_NODES) {
+                const int last = run.back().op;
+                for (const Member &m : run) {
+                    fusedKind[m.op] = 10;
+                    if (m.op != last) absorbed[m.op] = 1;   // keeps its buffer, filled by the run's kernel
+                }
+                // every buffer is an input of the step (the members' too: that is what keeps them allocated), except the
+                // last member's, which is the step's output
+                std::vector<int> ins;
+                std::vector<int> slotIn(slots.size(), -1);
+                for (size_t k = 0; k < slots.size(); k++)
+                    if (slots[k] != last) {
+                        slotIn[k] = (int)ins.size();
+                        ins.push_back(slots[k]);
+                    }
+                inputsOf[last] = ins;
+                tinyWrites[last].clear();
+                for (const Member &m : run)
+                    if (m.op != last) tinyWrites[last].push_back(m.op);
+                const int nslots = (int)slots.size();
+                prebuilt[last] = make([=](const std::vector<const void *> &in, void *out) {
+                    void *ptrs[DOPT_HIP_TINY_SLOTS];
+                    for (int k = 0; k < nslots; k++) ptrs[k] = slotIn[(size_t)k] >= 0 ? const_cast<void *>(in[(size_t)slotIn[(size_t)k]]) : out;
+                    return dopt_hip_tiny_graph(nslots, ptrs, (int)nodes.size(), nodes.data());
+                });
+                prebuiltLabel[last] = "tiny*" + std::to_string(nodes.size());
+            }
+        }
+        for (const Member &m : run) inRun[m.op] = 0;
+        run.clear();
+    };
+    for (int id : p->mOps) {
+        if (!live[id]) continue;
+        Member m{};
+        m.op = id;
+        if (describe(id, &m.nd, m.operands)) {
+            if (run.size() >= (size_t)DOPT_HIP_TINY_NODES || run.size() * 3 + 3 > (size_t)DOPT_HIP_TINY_SLOTS) close();
+            run.push_back(m);
+            inRun[id] = 1;
+            continue;
+        }
+        if (alias[id].source >= 0) continue;   // a view: its readers are looked at themselves
+        bool reads = false;
+        for (int d : inputsOf[id]) {
+            size_t off;
+            reads = reads || inRun[root(d, &off)];
+        }
+        if (reads) close();
+    }
+    close();
 }
 
 void HIPPlan::Builder::formChains()
@@ -1426,6 +1630,7 @@ int HIPPlan::Builder::buildSteps()
         s.op = id;
         s.label = label;
         s.inputOps = stepInputs;
+        s.writes = tinyWrites[id];
         s.kernel = std::move(k);
         s.inputs.resize(s.inputOps.size());
         s.inputBytes.resize(s.inputOps.size());
@@ -1666,6 +1871,7 @@ int HIPPlan::Builder::assignQueues()
                 st.lane = 1;
                 st.fenceBefore = true;
                 onSide[st.op] = 1;
+                for (int w : st.writes) onSide[w] = 1;
                 p->mUsesSide = true;
                 fences++;
             } else if (reads_side) {
@@ -1695,6 +1901,7 @@ int HIPPlan::Builder::assignQueues()
             if (biasGradOf[op] >= 0) stepOf[biasGradOf[op]] = (int)i;
             if (poolOf[op] >= 0) stepOf[poolOf[op]] = (int)i;
             if (pairOf[op] >= 0) stepOf[pairOf[op]] = (int)i;
+            for (int w : p->mSteps[i].writes) stepOf[w] = (int)i;
         }
         std::vector<std::vector<int>> readers(n), producers(n);
         for (size_t i = 0; i < n; i++)
@@ -1713,6 +1920,7 @@ int HIPPlan::Builder::assignQueues()
             // by label: a fused step carries the operation it ends in (convolution+addBias ends in an addBias), and a
             // convolution must stay behind the step that packs its filter
             const std::string &t = g.ops[st.op].opType;
+            if (!st.writes.empty()) continue;   // a run of tiny operations: some member may feed the main chain
             if (st.label.find("convolution") != std::string::npos || st.label.find("batchNorm") != std::string::npos ||
                 t.compare(0, 11, "convolution") == 0 || t.compare(0, 9, "batchNorm") == 0 || t == "uniform")
                 continue;
@@ -1816,6 +2024,7 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         b.foldTransposes();
         b.fuseDenseLayers();
         b.fuseDenseBackward();
+        b.formTinyRuns();
         b.formChains();
         b.absorbBiasGrads();
         b.absorbPools();

@@ -103,6 +103,7 @@ private:
         int op;
         std::string label;                       // profiler key: the opType, or "a+b" for a fused pair
         std::vector<int> inputOps;               // operations whose buffers are the kernel's inputs
+        std::vector<int> writes;                 // operations besides `op` whose buffers the kernel fills
         std::unique_ptr<HIPKernel> kernel;
         std::vector<const void *> inputs;
         std::vector<size_t> inputBytes;

@@ -9,6 +9,7 @@
 #include <vector>
 
 #include "common.h"
+#include "pw_ops.h"
 #include <limits>
 
 namespace {
@@ -22,45 +23,11 @@ struct OpInfo {
     const char *expr_i32;
 };
 
-// `a`, `b` are the operands of type T.  Integer arithmetic wraps (D semantics); every integer
-// unary op except neg goes through float and truncates back (cpu/math.d:418).
+// `a`, `b` are the operands of type T; the table is pw_ops.h, each expression as the text the run-time compiler gets.
 const OpInfo kOps[] = {
-    {"add", 2, "a + b", "(int)((unsigned)a + (unsigned)b)"},
-    {"sub", 2, "a - b", "(int)((unsigned)a - (unsigned)b)"},
-    {"mul", 2, "a * b", "(int)((unsigned)a * (unsigned)b)"},
-    {"div", 2, "a / b", "a / b"},
-    {"lt", 2, "(T)(a < b)", "(T)(a < b)"},
-    {"lte", 2, "(T)(a <= b)", "(T)(a <= b)"},
-    {"gt", 2, "(T)(a > b)", "(T)(a > b)"},
-    {"gte", 2, "(T)(a >= b)", "(T)(a >= b)"},
-    {"eq", 2, "(T)(a == b)", "(T)(a == b)"},
-    {"neq", 2, "(T)(a != b)", "(T)(a != b)"},
-    {"max", 2, "(a < b ? b : a)", "(a < b ? b : a)"},
-    {"min", 2, "(a < b ? a : b)", "(a < b ? a : b)"},
-    {"pow", 2, "powf(a, b)", "dopt_ipow(a, b)"},
-    {"atan2", 2, "atan2f(a, b)", "(int)atan2f((float)a, (float)b)"},
-    {"neg", 1, "-a", "(int)(0u - (unsigned)a)"},
-    {"abs", 1, "fabsf(a)", "(int)fabsf((float)a)"},
-    {"sgn", 1, "(T)((a > 0) - (a < 0))", "(int)(float)(((float)a > 0) - ((float)a < 0))"},
-    {"exp", 1, "expf(a)", "(int)expf((float)a)"},
-    {"log", 1, "logf(a)", "(int)logf((float)a)"},
-    {"sqrt", 1, "sqrtf(a)", "(int)sqrtf((float)a)"},
-    {"sin", 1, "sinf(a)", "(int)sinf((float)a)"},
-    {"cos", 1, "cosf(a)", "(int)cosf((float)a)"},
-    {"tan", 1, "tanf(a)", "(int)tanf((float)a)"},
-    {"asin", 1, "asinf(a)", "(int)asinf((float)a)"},
-    {"acos", 1, "acosf(a)", "(int)acosf((float)a)"},
-    {"atan", 1, "atanf(a)", "(int)atanf((float)a)"},
-    {"sinh", 1, "sinhf(a)", "(int)sinhf((float)a)"},
-    {"cosh", 1, "coshf(a)", "(int)coshf((float)a)"},
-    {"tanh", 1, "tanhf(a)", "(int)tanhf((float)a)"},
-    {"asinh", 1, "asinhf(a)", "(int)asinhf((float)a)"},
-    {"acosh", 1, "acoshf(a)", "(int)acoshf((float)a)"},
-    {"atanh", 1, "atanhf(a)", "(int)atanhf((float)a)"},
-    // the two activations of cuda/nnet/cudnn7.d:406-461 in the form nn.hip computes them (NaN passes through
-    // relu); reluGrad takes (dy, x).  They exist so that a plan can run them inside a pointwise chain.
-    {"relu", 1, "(a < 0 ? 0 : a)", "(a < 0 ? 0 : a)"},
-    {"reluGrad", 2, "(b > 0 ? a : 0)", "(b > 0 ? a : 0)"},
+#define DOPT_PW_ROW(name, arity, f32, i32) {#name, arity, #f32, #i32},
+    DOPT_PW_OPS(DOPT_PW_ROW)
+#undef DOPT_PW_ROW
 };
 
 const OpInfo *find_op(const char *name)
@@ -654,6 +621,17 @@ int dopt_hip_pointwise_chain_compile_only(int dtype, int nin, const unsigned cha
     std::string key, source;
     if (int rc = chain_prepare(dtype, nin, in_is_scalar, nnodes, node_op, node_lhs, node_rhs, &key, &source)) return rc;
     return rtc_compile_only(source, arch, nullptr);
+}
+
+int dopt_hip_pointwise_index(const char *op)
+{
+    if (!op) return -1;
+    int i = 0;
+    for (const OpInfo &o : kOps) {
+        if (!strcmp(o.name, op)) return i;
+        i++;
+    }
+    return -1;
 }
 
 int dopt_hip_pointwise_arity(const char *op)

@@ -130,6 +130,10 @@ def parse(text):
                 piece = piece.strip()
                 stars = piece.count("*")
                 nm = piece.replace("*", "").strip()
+                am = re.match(r"(\w+)\s*\[(\d+)\]$", nm)
+                if am:   # a fixed-size array member: `int dims[4]` is `int[4] dims` in D
+                    fields.append("%s[%s] %s" % (d_type(ctype + " " + "*" * stars, known), am.group(2), d_name(am.group(1))))
+                    continue
                 fields.append("%s %s" % (d_type(ctype + " " + "*" * stars, known), d_name(nm)))
         items.append(("struct", name, fields))
     for name, ret, plist in fptrs:

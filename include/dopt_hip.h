@@ -133,6 +133,47 @@ int dopt_hip_pointwise_chain_compile_only(int dtype, int nin, const unsigned cha
 /* 1 or 2 for the names dopt_hip_pointwise accepts, 0 otherwise. */
 int dopt_hip_pointwise_arity(const char *op);
 
+/* Position of a name dopt_hip_pointwise accepts (and of "relu", "reluGrad") in the library's table of pointwise
+   operations, or -1: the `op` of a pointwise node of dopt_hip_tiny_graph. */
+int dopt_hip_pointwise_index(const char *op);
+
+/* A run of operations on tiny fp32 tensors (at most DOPT_HIP_TINY_ELEMS elements each) as ONE launch of one workgroup,
+   node after node in the order given, with a workgroup barrier in between.  The reference runs each of them as a
+   kernel of its own (cuda/math.d:89-127 pointwise, cuda/package.d:81-119 the host round trip for sum / maxElement,
+   cudnn7.d:470-526 softmax and its gradient, cuda/basic.d:143-217 repeat); on a few hundred values each of those lasts
+   as long as the gap between two kernels.  Every node computes what its stand-alone entry point computes, in the same
+   order of operations, so the results are identical to calling those one by one.
+   slots: the buffers the nodes name (inputs, intermediate values and results alike; the caller owns them all).
+   A node writes n elements to slots[dst] + dst_offset bytes from operands at slots[a] + a_offset, slots[b] + b_offset:
+     POINTWISE     op = dopt_hip_pointwise_index(name); b = -1 for a unary operation; a_kind / b_kind: 0 the operand
+                   has n elements, 1 it has one element that every result reads, 2 one element per row and 3 one per
+                   column of the result seen as [n / dims[0], dims[0]] (the reference broadcasts a column or a row
+                   through a product [m,1] x [1,n], core/ops/basic.d:370-381: the node `mul` of kinds 2 and 3)
+     REDUCE        op = 0 sum, 1 maxElement; the operand is [dims[0], dims[1], dims[2]] and dims[1] is folded
+                   (n = dims[0] * dims[2]): one run of adjacent reduced axes, as dopt_hip_reduce folds it
+     SOFTMAX       the operand is [dims[0], dims[1], dims[2]] = [N, C, inner], normalised over C as dopt_hip_softmax_fwd
+                   does for rows of fewer than 64 classes (or inner > 1)
+     SOFTMAX_GRAD  a = dy, b = y, same layout, as dopt_hip_softmax_bwd
+     REPEAT        the operand has extents dims[0..3] (leading 1s for lower ranks) and is tiled reps[0..3] times */
+typedef enum { DOPT_HIP_TINY_SLOTS = 48, DOPT_HIP_TINY_NODES = 40, DOPT_HIP_TINY_ELEMS = 4096 } dopt_hip_tiny_limits;
+typedef enum {
+    DOPT_HIP_TINY_POINTWISE = 0,
+    DOPT_HIP_TINY_REDUCE = 1,
+    DOPT_HIP_TINY_SOFTMAX = 2,
+    DOPT_HIP_TINY_SOFTMAX_GRAD = 3,
+    DOPT_HIP_TINY_REPEAT = 4
+} dopt_hip_tiny_kind;
+typedef struct {
+    int kind, op;
+    int dst, a, b;
+    int a_kind, b_kind;
+    int n;
+    int dst_offset, a_offset, b_offset;
+    int dims[4];
+    int reps[4];
+} dopt_hip_tiny_node;
+int dopt_hip_tiny_graph(int nslots, void *const *slots, int nnodes, const dopt_hip_tiny_node *nodes);
+
 /* `sum` / `maxElement` (op = "sum" | "maxElement"): cpu/math.d:90-247, reached in the reference through
    the host fallback cuda/package.d:81-119.  Reduces `axes` (distinct, each < rank) of a dense
    tensor; out has the reduced axes removed (core/ops/math.d:162-175). */
