@@ -721,7 +721,8 @@ __global__ __launch_bounds__(256) void split_sum_k(size_t n4, int splits, size_t
 // Filter gradient of 3x3, unit-stride, pad-1 convolutions:
 //   dw[k][c][2-r][2-s] = sum over (n, p, q) of dy[n][k][p][q] * x[n][c][p-1+r][q-1+s].
 // The reduction runs over pixels.  A block owns BM output channels x BC input channels x all nine
-// taps and walks the pixels in chunks of 64.  Per chunk it stages dy[BM][64] and ONE zero-haloed
+// taps (BM x BC = 128 x 32, 64 x 64, or 160 x 32 for layers of 160 channels, which the other two would pad by
+// a fifth and more) and walks the pixels in chunks of 64.  Per chunk it stages dy[BM][64] and ONE zero-haloed
 // patch of x for its BC channels in LDS; the nine taps read that patch at nine offsets, so x is
 // fetched once, not nine times.  The twelve wavefronts are (32 rows of k) x (32 channels) x
 // (tap row r): a wavefront keeps the three taps s = 0..2 of its tap row in three 32x32
@@ -757,12 +758,12 @@ struct WgradPatch {
 template <int WM, int WC, int kGeo>
 __device__ __forceinline__ void conv_wgrad_patch_body(const WgradPatch &p, const unsigned block_id)
 {
-    constexpr int BM = 32 * WM, BC = 32 * WC, THREADS = 768, NPIX = 64, APITCH = NPIX + 4;
+    constexpr int BM = 32 * WM, BC = 32 * WC, THREADS = 64 * 3 * WM * WC, NPIX = 64, APITCH = NPIX + 4;
     constexpr int NAQ = (BM * NPIX / 4 + THREADS - 1) / THREADS;  // float4 slots of dy per thread
     // float4 slots of x per thread: geometry 0 up to 32*4*8 (W = 32) or 32*3*16 (W = 64) quads per 32
     // channels; geometries 1, 2 have 16 quads per channel
     constexpr int NBQ = kGeo == 0 ? (WC == 1 ? 2 : 3) : (BC * 16 + THREADS - 1) / THREADS;
-    static_assert(WM * WC == 4, "twelve wavefronts: 4 (row, channel) groups x 3 tap rows");
+    static_assert(WM * WC == 4 || WM * WC == 5, "twelve or fifteen wavefronts: 4 or 5 (row, channel) groups x 3 tap rows");
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int bsize = BC * p.cstride;
     float *const A0 = lds;                     // [2][BM * APITCH]
@@ -985,7 +986,7 @@ __device__ __forceinline__ void conv_wgrad_patch_body(const WgradPatch &p, const
             }
         }
         __syncthreads();
-        for (int r = w; r < 32; r += 12) {  // one wavefront per row
+        for (int r = w; r < 32; r += 3 * WM * WC) {  // one wavefront per row
             const int k = k0 + g * 32 + r;
             if (k >= p.K) continue;
             float *dst = outp + ((size_t)k * p.C + c0) * 9;
@@ -996,7 +997,7 @@ __device__ __forceinline__ void conv_wgrad_patch_body(const WgradPatch &p, const
 }
 
 template <int WM, int WC, int kGeo>
-__global__ __launch_bounds__(768, 1) void conv_wgrad_patch_k(WgradPatch p)
+__global__ __launch_bounds__(64 * 3 * WM * WC, 1) void conv_wgrad_patch_k(WgradPatch p)
 {
     conv_wgrad_patch_body<WM, WC, kGeo>(p, blockIdx.x);
 }
@@ -1160,6 +1161,7 @@ int launch_splitk_reduce(size_t elems, int splits, const float *partial, float *
 using GatherWide = Tile<64, 256, 1, 4>;     // few output channels, many pixels
 using GatherSquare = Tile<128, 128, 2, 2>;  // enough tiles for two workgroups per CU
 using GatherDeep = Tile<128, 128, 2, 4>;    // few tiles: 8 wavefronts per workgroup, one workgroup per CU
+using GatherTall = Tile<160, 128, 1, 4>;    // 160 output channels (and 480, ...): 64- and 128-row tiles would multiply a fifth more rows than there are
 
 unsigned div_magic(unsigned d) { return (unsigned)((((unsigned long long)1 << 32) / d) + 1); }
 
@@ -1186,13 +1188,24 @@ int launch_patch(const PatchConv &pc, bool c_full, dim3 grid, size_t lds_bytes)
 struct PatchSetup {
     bool ok;
     PatchConv pc;
-    int shape;            // 0 wide, 1 square, 2 deep
+    int shape;            // 0 wide, 1 square, 2 deep, 3 tall
     int BM, BN, blocks_wanted, tiles;
     size_t lds_bytes, wp_elems;
 };
 
 template <bool kBwd>
+PatchSetup patch_setup_as(const dopt_hip_conv_desc *d, size_t P, size_t Q, bool allow_tall);
+
+// (a layer the 160-row tiles do not take - its pixel tile does not fit their patch - is tried with the other heights)
+template <bool kBwd>
 PatchSetup patch_setup(const dopt_hip_conv_desc *d, size_t P, size_t Q)
+{
+    const PatchSetup u = patch_setup_as<kBwd>(d, P, Q, true);
+    return u.ok ? u : patch_setup_as<kBwd>(d, P, Q, false);
+}
+
+template <bool kBwd>
+PatchSetup patch_setup_as(const dopt_hip_conv_desc *d, size_t P, size_t Q, bool allow_tall)
 {
     PatchSetup u{};
     if (d->R != 3 || d->S != 3 || d->strideH != 1 || d->strideW != 1 || d->padH > 2 || d->padW > 2) return u;
@@ -1209,8 +1222,15 @@ PatchSetup patch_setup(const dopt_hip_conv_desc *d, size_t P, size_t Q)
     }
     pc.ncols = pc.N * pc.OH * pc.OW;
     int npmax, threads;
-    // 64-row tiles for up to 64 output channels, and wherever 128-row tiles would pad more (160 -> 192, not 256)
-    if (pc.Mout <= 64 || (pc.Mout + 63) / 64 * 64 < (pc.Mout + 127) / 128 * 128) {
+    // 160-row tiles where they pad less than both other heights (160 channels: 160 rows, not 192 or 256); 64-row tiles for
+    // up to 64 output channels, and wherever 128-row tiles would pad more
+    const int up64 = (pc.Mout + 63) / 64 * 64, up128 = (pc.Mout + 127) / 128 * 128, up160 = (pc.Mout + 159) / 160 * 160;
+    // (only where they still give every compute unit a tile: 480 channels on 8 x 8 images are 192 such tiles, and ran slower)
+    const long tall_tiles = (long)(up160 / 160) * ((pc.ncols + 127) / 128);
+    if (allow_tall && pc.Mout > 64 && up160 * 11 < up64 * 10 && up160 * 11 < up128 * 10 && tall_tiles >= num_cus() &&
+        std::getenv("DOPT_HIP_NO_TALL") == nullptr) {
+        u.shape = 3; u.BM = 160; u.BN = 128; u.blocks_wanted = num_cus(); npmax = 16; threads = 256;
+    } else if (pc.Mout <= 64 || up64 < up128) {
         u.shape = 0; u.BM = 64; u.BN = 256; u.blocks_wanted = 2 * num_cus(); npmax = 24; threads = 256;
     } else {
         u.BM = 128; u.BN = 128;
@@ -1340,6 +1360,7 @@ int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, 
     int rc;
     if (u.shape == 0) rc = launch_patch<GatherWide, 24>(pc, c_full, grid, u.lds_bytes);
     else if (u.shape == 1) rc = launch_patch<GatherSquare, 16>(pc, c_full, grid, u.lds_bytes);
+    else if (u.shape == 3) rc = launch_patch<GatherTall, 16>(pc, c_full, grid, u.lds_bytes);
     else rc = launch_patch<GatherDeep, 16>(pc, c_full, grid, u.lds_bytes);
     if (rc) return rc;
     *done = true;
@@ -1881,7 +1902,7 @@ int launch_wgrad_patch(const WgradPatch &wp, dim3 grid, size_t lds_bytes)
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         raised = true;
     }
-    hipLaunchKernelGGL((conv_wgrad_patch_k<WM, WC, kGeo>), grid, dim3(768), lds_bytes, stream(), wp);
+    hipLaunchKernelGGL((conv_wgrad_patch_k<WM, WC, kGeo>), grid, dim3(64 * 3 * WM * WC), lds_bytes, stream(), wp);
     DOPT_LAUNCH_CHECK();
     return DOPT_HIP_OK;
 }
@@ -1902,7 +1923,8 @@ int launch_wgrad_reduce(int K, int C, int Cp, int taps, int splits, size_t out_e
 struct WgradSetup {
     bool ok;
     WgradPatch wp;
-    bool tall;            // 128 rows x 32 channels per block, else 64 x 64
+    bool tall;            // 128 rows x 32 channels per block
+    int rows;             // output channels per block: 128 (tall), 160 (x 32 channels) or 64 (x 64 channels)
     int geo, tiles, splits;
     size_t out_elems, lds_bytes;
 };
@@ -1938,9 +1960,13 @@ WgradSetup wgrad_patch_setup(const dopt_hip_conv_desc *d, const float *dw)
     }
     while (wp.cstride % 8 != 4) wp.cstride += 4;  // 128-bit reads by 32 channels at this stride touch every LDS bank once
     // 128 rows x 32 channels, or 64 x 64 when that pads the output channels less (160 -> 192, not 256)
-    const bool tall = d->K >= 128 && (d->K + 127) / 128 * 128 <= (d->K + 63) / 64 * 64;
-    if (!tall && W == 64) return u;
-    const int BM = tall ? 128 : 64, BC = tall ? 32 : 64;
+    // ... or 160 x 32 where that pads them less than both (160 channels: 160 rows, not 192 or 256)
+    const int up64 = (int)((d->K + 63) / 64 * 64), up128 = (int)((d->K + 127) / 128 * 128), up160 = (int)((d->K + 159) / 160 * 160);
+    // (by a tenth at least: 480 channels are 512 rows of the 64-row tiles, and ran no faster as 3 x 160)
+    const bool rows160 = d->K > 64 && up160 * 11 < up64 * 10 && up160 * 11 < up128 * 10 && std::getenv("DOPT_HIP_NO_TALL") == nullptr;
+    const bool tall = !rows160 && d->K >= 128 && up128 <= up64;
+    if (!tall && !rows160 && W == 64) return u;
+    const int BM = rows160 ? 160 : tall ? 128 : 64, BC = BM == 64 ? 64 : 32;
     wp.N = (int)d->N; wp.C = (int)d->C; wp.K = (int)d->K; wp.H = H; wp.W = W;
     wp.quads_row = W / 4;
     wp.mtiles = (wp.K + BM - 1) / BM;
@@ -1981,7 +2007,7 @@ WgradSetup wgrad_patch_setup(const dopt_hip_conv_desc *d, const float *dw)
     u.lds_bytes = lds_main > lds_epi ? lds_main : lds_epi;
     if (u.lds_bytes > 160 * 1024) return u;
     wp.split_stride = out_elems;
-    u.tall = tall; u.geo = geo; u.tiles = tiles; u.splits = splits; u.out_elems = out_elems;
+    u.tall = tall; u.rows = BM; u.geo = geo; u.tiles = tiles; u.splits = splits; u.out_elems = out_elems;
     u.ok = true;
     return u;
 }
@@ -2028,7 +2054,10 @@ int run_wgrad_patch(const dopt_hip_conv_desc *d, const float *dy, const float *x
     const dim3 grid(xcd_grid((unsigned)(u.tiles * u.splits)));
     const int geo = u.geo;
     int rc;
-    if (u.tall) rc = geo == 0 ? launch_wgrad_patch<4, 1, 0>(wp, grid, u.lds_bytes)
+    if (u.rows == 160) rc = geo == 0 ? launch_wgrad_patch<5, 1, 0>(wp, grid, u.lds_bytes)
+                        : geo == 1 ? launch_wgrad_patch<5, 1, 1>(wp, grid, u.lds_bytes)
+                                   : launch_wgrad_patch<5, 1, 2>(wp, grid, u.lds_bytes);
+    else if (u.tall) rc = geo == 0 ? launch_wgrad_patch<4, 1, 0>(wp, grid, u.lds_bytes)
                    : geo == 1 ? launch_wgrad_patch<4, 1, 1>(wp, grid, u.lds_bytes)
                               : launch_wgrad_patch<4, 1, 2>(wp, grid, u.lds_bytes);
     else rc = geo == 0 ? launch_wgrad_patch<2, 2, 0>(wp, grid, u.lds_bytes)
