@@ -1222,12 +1222,14 @@ PatchSetup patch_setup_as(const dopt_hip_conv_desc *d, size_t P, size_t Q, bool 
     }
     pc.ncols = pc.N * pc.OH * pc.OW;
     int npmax, threads;
-    // 160-row tiles where they pad less than both other heights (160 channels: 160 rows, not 192 or 256); 64-row tiles for
-    // up to 64 output channels, and wherever 128-row tiles would pad more
+    // 160-row tiles where they pad no more than both other heights (160 channels: 160 rows, not 192 or 256; 320 and 640
+    // channels: two and four such tiles - on 8 x 8 images 640 channels are then exactly 256 tiles, one per compute unit
+    // with no split of the reduction, where 128-row tiles gave 320 and a four-way split); 64-row tiles for up to 64 output
+    // channels, and wherever 128-row tiles would pad more
     const int up64 = (pc.Mout + 63) / 64 * 64, up128 = (pc.Mout + 127) / 128 * 128, up160 = (pc.Mout + 159) / 160 * 160;
     // (only where they still give every compute unit a tile: 480 channels on 8 x 8 images are 192 such tiles, and ran slower)
     const long tall_tiles = (long)(up160 / 160) * ((pc.ncols + 127) / 128);
-    if (allow_tall && pc.Mout > 64 && up160 * 11 < up64 * 10 && up160 * 11 < up128 * 10 && tall_tiles >= num_cus() &&
+    if (allow_tall && pc.Mout > 64 && up160 <= up64 && up160 <= up128 && tall_tiles >= num_cus() &&
         std::getenv("DOPT_HIP_NO_TALL") == nullptr) {
         u.shape = 3; u.BM = 160; u.BN = 128; u.blocks_wanted = num_cus(); npmax = 16; threads = 256;
     } else if (pc.Mout <= 64 || up64 < up128) {
@@ -1963,6 +1965,7 @@ WgradSetup wgrad_patch_setup(const dopt_hip_conv_desc *d, const float *dw)
     // ... or 160 x 32 where that pads them less than both (160 channels: 160 rows, not 192 or 256)
     const int up64 = (int)((d->K + 63) / 64 * 64), up128 = (int)((d->K + 127) / 128 * 128), up160 = (int)((d->K + 159) / 160 * 160);
     // (by a tenth at least: 480 channels are 512 rows of the 64-row tiles, and ran no faster as 3 x 160)
+    // (320 and 640 channels, which the other heights do not pad either, ran slower this way: measured)
     const bool rows160 = d->K > 64 && up160 * 11 < up64 * 10 && up160 * 11 < up128 * 10 && std::getenv("DOPT_HIP_NO_TALL") == nullptr;
     const bool tall = !rows160 && d->K >= 128 && up128 <= up64;
     if (!tall && !rows160 && W == 64) return u;
