@@ -65,3 +65,35 @@ def test_convolution_block_graph_on_the_cpu_evaluator():
     assert np.allclose(got[2], O.add_bias_grad(dc), rtol=1e-5, atol=1e-6)
     assert np.allclose(got[3].reshape(-1), gp[c.size:c.size + 4], rtol=1e-5, atol=1e-6)
     assert np.allclose(got[4], gp[c.size + 4:], rtol=1e-5, atol=1e-6)
+
+
+def test_threaded_evaluator_equals_the_single_threaded_one_except_for_blas_products():
+    """The threaded CPU baseline: sum / maxElement / repeat parallel over their outer index (cpu/basic.d's
+    parallel foreach) add each output element's terms in the single-threaded order, so their values are
+    the same bits on any thread count; matmul through the host BLAS differs by rounding only."""
+    import oracle as O
+    r = np.random.default_rng(2)
+    a = r.standard_normal((37, 19, 11)).astype(np.float32)
+    before = O.get_threads()
+    try:
+        O.set_threads(1)
+        want = [O.sum(a, [0]), O.sum(a, [1, 2]), O.sum(a), O.max_element(a, [2]), O.repeat(a, [2, 1, 3])]
+        O.set_threads(4)
+        assert O.get_threads() == 4
+        got = [O.sum(a, [0]), O.sum(a, [1, 2]), O.sum(a), O.max_element(a, [2]), O.repeat(a, [2, 1, 3])]
+    finally:
+        O.set_threads(before)
+    for w, g in zip(want, got):
+        assert np.array_equal(w, g)
+
+    n, d, k = 16, 33, 5
+    x = r.random((n, d)).astype(np.float32)
+    f = float32([n, d])
+    W = float32([d, k], r.standard_normal((d, k)).astype(np.float32))
+    z = core.matmul(f, W)
+    loss = core.sum(z * z)
+    gW, = grad(loss, [W])
+    plain = evaluator.evaluate([z, loss, gW], {f: x})
+    blas = evaluator.evaluate([z, loss, gW], {f: x}, blas=True)
+    for p, b in zip(plain, blas):
+        assert np.allclose(p, b, rtol=1e-5, atol=1e-5)
