@@ -53,9 +53,10 @@ struct GatherConv {
     int out_plane, out_OW, out_sy, out_sx, out_oy, out_ox;
 };
 
-// kMode: 0 = forward, 1 = backward-data with unit stride (no divisions), 2 = backward-data, any stride
+// kMode: 0 = forward, 1 = backward-data with unit stride (no divisions), 2 = backward-data, any stride.
+// L: the workgroup's item among the problem's (split, tile) pairs, tile fastest.
 template <class T, int kMode>
-__global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_gather_k(GatherConv p)
+__device__ __forceinline__ void conv_gather_body(const GatherConv &p, unsigned L)
 {
     constexpr int BM = T::BM, BN = T::BN, LDA = T::LDA, LDB = T::LDB, THREADS = T::THREADS;
     constexpr int NA = BM * BK / 4 / THREADS;  // float4 loads of A per thread
@@ -65,11 +66,7 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_gather_k(Ga
     __shared__ __attribute__((aligned(16))) float As[2][BK * LDA];
     __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB];
 
-    // 1-D grid over (split, tile), tile fastest: the blocks an XCD receives work on neighbouring
-    // tiles of the same slice of the reduction, whatever the ratio of tiles to splits
-    unsigned L;
     const unsigned tiles = (unsigned)(p.mtiles * p.ntiles);
-    if (!xcd_remap(blockIdx.x, tiles * (unsigned)p.splits, &L)) return;
     const int split = (int)(L / tiles);
     const unsigned tile = L - (unsigned)split * tiles;
     const int mt = (int)(tile % (unsigned)p.mtiles), nt = (int)(tile / (unsigned)p.mtiles);
@@ -191,6 +188,43 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_gather_k(Ga
                 if (m < p.Mout) base[(size_t)m * p.out_plane] = acc[i][j][v];
             }
     }
+}
+
+template <class T, int kMode>
+__global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_gather_k(GatherConv p)
+{
+    // 1-D grid over (split, tile), tile fastest: the blocks an XCD receives work on neighbouring
+    // tiles of the same slice of the reduction, whatever the ratio of tiles to splits
+    unsigned L;
+    if (!xcd_remap(blockIdx.x, (unsigned)(p.mtiles * p.ntiles) * (unsigned)p.splits, &L)) return;
+    conv_gather_body<T, kMode>(p, L);
+}
+
+// Up to four problems that do not depend on each other in ONE launch (the residue classes of a strided backward-data
+// pass: same operands, different sub-filters, interleaved output pixels).  Every workgroup runs conv_gather_body on one
+// tile of one problem, so each problem's values are those of a launch of its own; what changes is that the chip is not
+// drained and refilled between problems that each fill only part of it.  An XCD takes the same share of every problem
+// (its tiles of a problem are neighbours, as in a single launch), longest problem first.
+constexpr int kGatherJobs = 4;
+struct GatherGroup {
+    GatherConv g[kGatherJobs];
+    unsigned per[kGatherJobs];   // workgroups of problem j on each XCD: ceil(tiles * splits / 8)
+    int n;
+};
+
+template <class T, int kMode>
+__global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_gather_group_k(GatherGroup gg)
+{
+    const unsigned xcd = blockIdx.x & 7u;
+    unsigned i = blockIdx.x >> 3;
+    int j = 0;
+    while (j < gg.n - 1 && i >= gg.per[j]) {
+        i -= gg.per[j];
+        j++;
+    }
+    const unsigned L = xcd * gg.per[j] + i;
+    if (i >= gg.per[j] || L >= (unsigned)(gg.g[j].mtiles * gg.g[j].ntiles) * (unsigned)gg.g[j].splits) return;
+    conv_gather_body<T, kMode>(gg.g[j], L);
 }
 
 // ------------------------------------------------------------------------------------ patch (3x3, unit stride)
@@ -1112,16 +1146,6 @@ __global__ __launch_bounds__(256) void pack_bwd_k(int K, int C, int taps, int KP
 
 int round_up(int v, int to) { return (v + to - 1) / to * to; }
 
-// Reduction splits so that about `blocks_wanted` workgroups exist, at least 4 slabs each.
-int pick_splits(int tiles, int slabs_total, int blocks_wanted, int cap)
-{
-    int want = (blocks_wanted + tiles - 1) / tiles;
-    int max_by_depth = slabs_total / 4 > 0 ? slabs_total / 4 : 1;
-    int s = want < max_by_depth ? want : max_by_depth;
-    if (s > cap) s = cap;
-    return s < 1 ? 1 : s;
-}
-
 int check_desc(const dopt_hip_conv_desc *d, size_t *P, size_t *Q, const char *who)
 {
     DOPT_REQUIRE(d != nullptr, "%s: descriptor is null", who);
@@ -1304,6 +1328,29 @@ int patch_splits(int tiles, int chunks, int slots, int BM, int BN, size_t out_el
         double cost = rounds * (per_block * t_chunk + 6.0);
         if (sp > 1) cost += 3.0 + (sp + 1.0) * out_elems * 4.0 / 4.5e6;       // partial tiles at ~4.5 TB/s
         if (sp == 1 || cost < best_cost * 0.97) {                    // a larger split must pay for itself clearly
+            best = sp;
+            best_cost = cost;
+        }
+    }
+    return best;
+}
+
+// The same estimate for the general kernels, whose unit is a slab of 16 reduction steps and whose main loops
+// sustain less (k-major LDS tiles, 32-bit fragment reads).
+int gather_splits(int tiles, int slabs, int slots, int BM, int BN, size_t out_elems, int cap = 64)
+{
+    const double cu_tflops = 0.33;
+    const double per_cu = (double)slots / num_cus();
+    const double t_slab = 2.0 * BM * BN * 16 / (cu_tflops * 1e6 / per_cu);
+    int best = 1;
+    double best_cost = 0.0;
+    for (int sp = 1; sp <= slabs && sp <= cap; sp++) {
+        const int per_block = (slabs + sp - 1) / sp;
+        if (sp > 1 && (slabs + per_block - 1) / per_block != sp) continue;
+        const double rounds = (double)(((long long)tiles * sp + slots - 1) / slots);
+        double cost = rounds * (per_block * t_slab + 6.0);
+        if (sp > 1) cost += 3.0 + (sp + 1.0) * out_elems * 4.0 / 4.5e6;
+        if (sp == 1 || cost < best_cost * 0.97) {
             best = sp;
             best_cost = cost;
         }
@@ -1726,7 +1773,7 @@ int gather_launch(GatherConv g, int mode, int K, int C, const float *in, const f
     g.mtiles = (g.Mout + BM - 1) / BM;
     g.ntiles = (g.ncols + BN - 1) / BN;
     const int tiles = g.mtiles * g.ntiles;
-    int splits = pick_splits(tiles, g.slabs_total, blocks_wanted, 64);
+    int splits = gather_splits(tiles, g.slabs_total, blocks_wanted, BM, BN, g.out_elems);
     // the split reduction works on float4 over a dense output
     if (g.out_elems % 4 != 0 || !aligned16(out) || !dense) splits = 1;
     g.slabs_per_split = (g.slabs_total + splits - 1) / splits;
@@ -1801,6 +1848,38 @@ __global__ __launch_bounds__(256) void subfilter_k(int KC, int R, int S, int R2,
     }
 }
 
+// The packed sub-filters of up to four classes in one launch: block (k, 64-channel chunk) stages w[k][c0 .. c0+64][*]
+// once and writes each class's taps as pack_bwd_k would write them from that class's sub-filter.
+struct SubFilter {
+    float *wp;            // [(tap * KPad + k)][Mp] of this class
+    int R2, S2, r0, s0;   // tap rows / columns of the class and its first tap offsets
+};
+struct SubFilters {
+    SubFilter f[kGatherJobs];
+    int n;
+};
+__global__ __launch_bounds__(256) void pack_bwd_classes_k(int K, int C, int R, int S, int sH, int sW, int KPad, int Mp,
+                                                           const float *w, SubFilters subs)
+{
+    extern __shared__ float stage[];  // 64 * R * S floats
+    const int k = blockIdx.x, c0 = blockIdx.y * 64, RS = R * S;
+    const int nc = min(64, C - c0);
+    const float *src = w + ((size_t)k * C + c0) * RS;
+    for (int i = threadIdx.x; i < nc * RS; i += 256) stage[i] = src[i];
+    __syncthreads();
+    for (int j = 0; j < subs.n; j++) {
+        const SubFilter f = subs.f[j];
+        const int taps = f.R2 * f.S2;
+        for (int i = threadIdx.x; i < nc * taps; i += 256) {
+            const int t = i / nc, c = i - t * nc, tr = t / f.S2, ts = t - tr * f.S2;
+            // stored tap (tr, ts) stands for offsets r = r0 + (R2 - 1 - tr) * sH, s likewise, and the element
+            // that multiplies offset (r, s) is the flipped one (see subfilter_k)
+            const int r = f.r0 + (f.R2 - 1 - tr) * sH, sc = f.s0 + (f.S2 - 1 - ts) * sW;
+            f.wp[(size_t)(t * KPad + k) * Mp + c0 + c] = stage[c * RS + (R - 1 - r) * S + (S - 1 - sc)];
+        }
+    }
+}
+
 int run_bwd_strided(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *dy, const float *w, float *dx)
 {
     const int sH = (int)d->strideH, sW = (int)d->strideW, R = (int)d->R, S = (int)d->S;
@@ -1819,6 +1898,84 @@ int run_bwd_strided(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float
     for (int b = 0; b < sW; b++) gaps = gaps || (cls(b, W, sW, padW, S).n > 0 && cls(b, W, sW, padW, S).taps == 0);
     if (gaps)
         if (int rc = dopt_hip_memset(dx, 0, d->N * d->C * d->H * d->W * sizeof(float))) return rc;
+    // Two to four classes with work (a 3 x 3 filter at stride 2 has four: 1, 2, 2 and 4 taps): one launch packs all
+    // their sub-filters and one launch multiplies all of them, instead of three dependent launches per class.
+    struct Job { Cls ch, cw; int a, b; };
+    Job jobs[kGatherJobs];
+    int njobs = 0;
+    bool fits = true;
+    for (int a = 0; a < sH; a++)
+        for (int b = 0; b < sW; b++) {
+            const Cls ch = cls(a, H, sH, padH, R), cw = cls(b, W, sW, padW, S);
+            if (ch.n == 0 || cw.n == 0 || ch.taps == 0 || cw.taps == 0) continue;
+            if (njobs == kGatherJobs) { fits = false; continue; }
+            jobs[njobs++] = Job{ch, cw, a, b};
+        }
+    if (fits && njobs >= 2) {
+        for (int i = 1; i < njobs; i++)   // most taps first (insertion sort, stable)
+            for (int j = i; j > 0 && jobs[j].ch.taps * jobs[j].cw.taps > jobs[j - 1].ch.taps * jobs[j - 1].cw.taps; j--)
+                std::swap(jobs[j], jobs[j - 1]);
+        const int K = (int)d->K, C = (int)d->C;
+        const int KPad = round_up(K, BK), Mp = round_up(C, 4);
+        size_t wp_off[kGatherJobs + 1] = {0};
+        for (int j = 0; j < njobs; j++) {
+            const size_t elems = (size_t)jobs[j].ch.taps * jobs[j].cw.taps * KPad * Mp;
+            wp_off[j + 1] = wp_off[j] + (elems * sizeof(float) + 255) / 256 * 256;
+        }
+        char *ws = (char *)workspace(wp_off[njobs]);
+        if (!ws) return DOPT_HIP_ERR_OOM;
+        if (KPad != K || Mp != C) {
+            if (capturing()) return fail(DOPT_HIP_ERR_UNSUPPORTED, "convolution: a fill cannot be recorded into a graph");
+            DOPT_HIP_CHECK(hipMemsetAsync(ws, 0, wp_off[njobs], stream()));
+        }
+        const bool wide = C <= 64 || (C + 63) / 64 * 64 < (C + 127) / 128 * 128;
+        const int BM = wide ? 64 : 128, BN = wide ? 256 : 128;
+        SubFilters subs{};
+        GatherGroup gg{};
+        subs.n = gg.n = njobs;
+        unsigned blocks = 0, tiles_all = 0;
+        for (int j = 0; j < njobs; j++) {
+            const Job &jb = jobs[j];
+            subs.f[j] = SubFilter{(float *)(ws + wp_off[j]), jb.ch.taps, jb.cw.taps, jb.ch.first, jb.cw.first};
+            GatherConv &g = gg.g[j];
+            g.N = (int)d->N;
+            g.R = jb.ch.taps; g.S = jb.cw.taps;
+            g.padH = jb.ch.pad; g.padW = jb.cw.pad;
+            g.strideH = g.strideW = 1;
+            g.Cin = K; g.IH = (int)P; g.IW = (int)Q;
+            g.Mout = C; g.OH = jb.ch.n; g.OW = jb.cw.n;
+            g.out_plane = H * W; g.out_OW = W;
+            g.out_sy = sH; g.out_sx = sW; g.out_oy = jb.a; g.out_ox = jb.b;
+            g.CinPad = KPad;
+            g.Mp = Mp;
+            g.ncols = g.N * g.OH * g.OW;
+            g.slabs_total = g.R * g.S * KPad / BK;
+            g.slabs_per_split = g.slabs_total;
+            g.splits = 1;   // a class's pixels are scattered over dx: nothing for a split sum to add in place
+            g.out_elems = (size_t)g.ncols * g.Mout;
+            g.mtiles = (g.Mout + BM - 1) / BM;
+            g.ntiles = (g.ncols + BN - 1) / BN;
+            g.in = dy;
+            g.wp = subs.f[j].wp;
+            g.out = dx;
+            g.in_bytes = (size_t)g.N * g.Cin * g.IH * g.IW * sizeof(float);
+            g.wp_bytes = (size_t)g.R * g.S * KPad * Mp * sizeof(float);
+            gg.per[j] = ((unsigned)(g.mtiles * g.ntiles) + 7u) / 8u;
+            blocks += 8u * gg.per[j];
+            tiles_all += (unsigned)(g.mtiles * g.ntiles);
+        }
+        hipLaunchKernelGGL(pack_bwd_classes_k, dim3((unsigned)K, (unsigned)((C + 63) / 64)), dim3(256),
+                           (size_t)64 * R * S * sizeof(float), stream(), K, C, R, S, sH, sW, KPad, Mp, w, subs);
+        DOPT_LAUNCH_CHECK();
+        if (wide)
+            hipLaunchKernelGGL((conv_gather_group_k<GatherWide, 1>), dim3(blocks), dim3(GatherWide::THREADS), 0, stream(), gg);
+        else if (tiles_all >= 2u * (unsigned)num_cus())
+            hipLaunchKernelGGL((conv_gather_group_k<GatherSquare, 1>), dim3(blocks), dim3(GatherSquare::THREADS), 0, stream(), gg);
+        else
+            hipLaunchKernelGGL((conv_gather_group_k<GatherDeep, 1>), dim3(blocks), dim3(GatherDeep::THREADS), 0, stream(), gg);
+        DOPT_LAUNCH_CHECK();
+        return DOPT_HIP_OK;
+    }
     void *sub = nullptr;
     if (int rc = scratch_alloc(&sub, d->K * d->C * d->R * d->S * sizeof(float))) return rc;
     int rc = DOPT_HIP_OK;
@@ -2470,7 +2627,7 @@ int dopt_hip_conv_bwd_filter(const dopt_hip_conv_desc *d, const float *dy, const
     f.ntiles = (f.ncols + BN - 1) / BN;
     const int tiles = f.mtiles * f.ntiles;
     // filter gradients are short and wide (small output, long pixel reduction): allow deep splits
-    int splits = pick_splits(tiles, f.slabs_total, 2 * num_cus(), 512);
+    int splits = gather_splits(tiles, f.slabs_total, 2 * num_cus(), BM, BN, f.out_elems, 512);
     f.slabs_per_split = (f.slabs_total + splits - 1) / splits;
     splits = (f.slabs_total + f.slabs_per_split - 1) / f.slabs_per_split;
     f.splits = splits;

@@ -531,7 +531,8 @@ int dopt_hip_tiny_graph(int nslots, void *const *slots, int nnodes, const dopt_h
         DOPT_REQUIRE(slots[nd.dst] && slots[nd.a] && (nd.b < 0 || slots[nd.b]), "dopt_hip_tiny_graph: node %d: null buffer", k);
         DOPT_REQUIRE(nd.n >= 0 && nd.n <= DOPT_HIP_TINY_ELEMS, "dopt_hip_tiny_graph: node %d has %d elements (at most %d)", k, nd.n,
                      DOPT_HIP_TINY_ELEMS);
-        DOPT_REQUIRE(nd.dst_offset % 4 == 0 && nd.a_offset % 4 == 0 && nd.b_offset % 4 == 0, "dopt_hip_tiny_graph: node %d: byte offsets must be multiples of 4", k);
+        DOPT_REQUIRE(nd.dst_offset >= 0 && nd.a_offset >= 0 && nd.b_offset >= 0 && nd.dst_offset % 4 == 0 && nd.a_offset % 4 == 0 && nd.b_offset % 4 == 0,
+                     "dopt_hip_tiny_graph: node %d: byte offsets must be non-negative multiples of 4", k);
         if (nd.kind == DOPT_HIP_TINY_POINTWISE) {
             DOPT_REQUIRE(nd.op >= 0 && nd.op < OP_count, "dopt_hip_tiny_graph: node %d: unknown pointwise operation %d", k, nd.op);
             DOPT_REQUIRE(nd.a_kind >= 0 && nd.a_kind <= 3 && nd.b_kind >= 0 && nd.b_kind <= 3, "dopt_hip_tiny_graph: node %d: unknown operand kind", k);

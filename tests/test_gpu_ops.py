@@ -361,6 +361,11 @@ CONV_CASES = [  # N, C, H, W, K, R, S, pad, stride
     (1, 3, 13, 12, 4, 5, 5, (2, 2), (2, 2)),
     (2, 8, 7, 9, 3, 3, 2, (2, 0), (1, 2)),
     (4, 20, 16, 16, 36, 3, 3, (1, 1), (2, 2)),
+    # the classes of a strided backward-data pass share one launch when there are two to four of them: 128-row tiles
+    # with few tiles (eight wavefronts) and with many (four), odd extents (classes of different sizes)
+    (2, 128, 8, 8, 64, 3, 3, (1, 1), (2, 2)),
+    (16, 128, 64, 64, 16, 3, 3, (1, 1), (2, 2)),
+    (3, 130, 9, 7, 24, 3, 3, (1, 1), (2, 2)),
 ]
 
 
