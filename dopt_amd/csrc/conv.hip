@@ -1146,6 +1146,13 @@ __global__ __launch_bounds__(256) void pack_bwd_k(int K, int C, int taps, int KP
 
 int round_up(int v, int to) { return (v + to - 1) / to * to; }
 
+// DOPT_HIP_NO_TALL=1 keeps the 160-row tiles out (for A/B measurements); read once.
+bool no_tall_tiles()
+{
+    static const bool off = std::getenv("DOPT_HIP_NO_TALL") != nullptr;
+    return off;
+}
+
 int check_desc(const dopt_hip_conv_desc *d, size_t *P, size_t *Q, const char *who)
 {
     DOPT_REQUIRE(d != nullptr, "%s: descriptor is null", who);
@@ -1254,7 +1261,7 @@ PatchSetup patch_setup_as(const dopt_hip_conv_desc *d, size_t P, size_t Q, bool 
     // (only where they still give every compute unit a tile: 480 channels on 8 x 8 images are 192 such tiles, and ran slower)
     const long tall_tiles = (long)(up160 / 160) * ((pc.ncols + 127) / 128);
     if (allow_tall && pc.Mout > 64 && up160 <= up64 && up160 <= up128 && tall_tiles >= num_cus() &&
-        std::getenv("DOPT_HIP_NO_TALL") == nullptr) {
+        !no_tall_tiles()) {
         u.shape = 3; u.BM = 160; u.BN = 128; u.blocks_wanted = num_cus(); npmax = 16; threads = 256;
     } else if (pc.Mout <= 64 || up64 < up128) {
         u.shape = 0; u.BM = 64; u.BN = 256; u.blocks_wanted = 2 * num_cus(); npmax = 24; threads = 256;
@@ -2123,7 +2130,7 @@ WgradSetup wgrad_patch_setup(const dopt_hip_conv_desc *d, const float *dw)
     const int up64 = (int)((d->K + 63) / 64 * 64), up128 = (int)((d->K + 127) / 128 * 128), up160 = (int)((d->K + 159) / 160 * 160);
     // (by a tenth at least: 480 channels are 512 rows of the 64-row tiles, and ran no faster as 3 x 160)
     // (320 and 640 channels, which the other heights do not pad either, ran slower this way: measured)
-    const bool rows160 = d->K > 64 && up160 * 11 < up64 * 10 && up160 * 11 < up128 * 10 && std::getenv("DOPT_HIP_NO_TALL") == nullptr;
+    const bool rows160 = d->K > 64 && up160 * 11 < up64 * 10 && up160 * 11 < up128 * 10 && !no_tall_tiles();
     const bool tall = !rows160 && d->K >= 128 && up128 <= up64;
     if (!tall && !rows160 && W == 64) return u;
     const int BM = rows160 ? 160 : tall ? 128 : 64, BC = BM == 64 ? 64 : 32;
