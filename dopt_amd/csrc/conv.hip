@@ -200,12 +200,12 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 128) void conv_gather_k(Ga
     conv_gather_body<T, kMode>(p, L);
 }
 
-// Up to four problems that do not depend on each other in ONE launch (the residue classes of a strided backward-data
-// pass: same operands, different sub-filters, interleaved output pixels).  Every workgroup runs conv_gather_body on one
+// Up to nine problems that do not depend on each other in ONE launch (the residue classes of a strided backward-data
+// pass - four at stride 2, nine at stride 3: same operands, different sub-filters, interleaved output pixels).  Every workgroup runs conv_gather_body on one
 // tile of one problem, so each problem's values are those of a launch of its own; what changes is that the chip is not
 // drained and refilled between problems that each fill only part of it.  An XCD takes the same share of every problem
 // (its tiles of a problem are neighbours, as in a single launch), longest problem first.
-constexpr int kGatherJobs = 4;
+constexpr int kGatherJobs = 9;
 struct GatherGroup {
     GatherConv g[kGatherJobs];
     unsigned per[kGatherJobs];   // workgroups of problem j on each XCD: ceil(tiles * splits / 8)
@@ -1855,7 +1855,7 @@ __global__ __launch_bounds__(256) void subfilter_k(int KC, int R, int S, int R2,
     }
 }
 
-// The packed sub-filters of up to four classes in one launch: block (k, 64-channel chunk) stages w[k][c0 .. c0+64][*]
+// The packed sub-filters of all classes in one launch: block (k, 64-channel chunk) stages w[k][c0 .. c0+64][*]
 // once and writes each class's taps as pack_bwd_k would write them from that class's sub-filter.
 struct SubFilter {
     float *wp;            // [(tap * KPad + k)][Mp] of this class
@@ -1905,7 +1905,7 @@ int run_bwd_strided(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float
     for (int b = 0; b < sW; b++) gaps = gaps || (cls(b, W, sW, padW, S).n > 0 && cls(b, W, sW, padW, S).taps == 0);
     if (gaps)
         if (int rc = dopt_hip_memset(dx, 0, d->N * d->C * d->H * d->W * sizeof(float))) return rc;
-    // Two to four classes with work (a 3 x 3 filter at stride 2 has four: 1, 2, 2 and 4 taps): one launch packs all
+    // Two to nine classes with work (a 3 x 3 filter at stride 2 has four: 1, 2, 2 and 4 taps): one launch packs all
     // their sub-filters and one launch multiplies all of them, instead of three dependent launches per class.
     struct Job { Cls ch, cw; int a, b; };
     Job jobs[kGatherJobs];

@@ -366,6 +366,8 @@ CONV_CASES = [  # N, C, H, W, K, R, S, pad, stride
     (2, 128, 8, 8, 64, 3, 3, (1, 1), (2, 2)),
     (16, 128, 64, 64, 16, 3, 3, (1, 1), (2, 2)),
     (3, 130, 9, 7, 24, 3, 3, (1, 1), (2, 2)),
+    (2, 7, 11, 13, 9, 5, 5, (2, 2), (3, 3)),      # nine classes with work in one launch
+    (1, 4, 9, 9, 5, 5, 5, (2, 2), (4, 4)),        # sixteen classes: one after the other
 ]
 
 
