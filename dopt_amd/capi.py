@@ -76,6 +76,7 @@ PROTOTYPES = {
     "dopt_hip_tiny_graph": [_i, C.POINTER(_vp), _i, C.POINTER(TinyNode)],
     "dopt_hip_pointwise_arity": [C.c_char_p],
     "dopt_hip_reduce": [C.c_char_p, _i, _szp, _i, _szp, _i, _vp, _vp],
+    "dopt_hip_reduce_squares": [_szp, _i, _szp, _i, _vp, _vp],
     "dopt_hip_argmin": [_i, _szp, _i, _sz, _vp, _vp],
     "dopt_hip_rtc_compile_only": [C.c_char_p, _i, C.c_char_p],
     "dopt_hip_slice": [_i, _szp, _szp, _szp, _vp, _vp],

@@ -580,7 +580,7 @@ struct HIPPlan::Builder {
     std::vector<Alias> alias;
     // inputsOf[id]: the operations whose buffers feed id's kernel (its deps, unless fused);
     // fusedKind[id]: 1 conv+bias, 2 bn+relu, 3 relugrad+bngrad, 6 matmul with transposes, 7 pointwise chain,
-    // 8 maxpoolgrad+relugrad+bngrad
+    // 8 maxpoolgrad+relugrad+bngrad, 9 matmul+relugrad, 10 member of a tiny run, 11 sum of squares
     std::vector<std::vector<int>> inputsOf;
     std::vector<int> fusedKind;
     std::vector<std::unique_ptr<HIPKernel>> prebuilt;
@@ -639,6 +639,7 @@ struct HIPPlan::Builder {
     void fuseDenseBackward();
     bool plainProduct(int id, MatmulInfo *mi, bool sole_reader) const;
     void formTinyRuns();
+    void fuseSquareSums();
     void formChains();
     void absorbBiasGrads();
     void absorbPools();
@@ -1176,6 +1177,50 @@ void HIPPlan::Builder::formTinyRuns()
         if (reads) close();
     }
     close();
+}
+
+// sum(mul(x, x)) - the L2 penalty of a parameter (`weightDecay * sum(filters * filters)`, nnet/layers/conv.d:117) and the
+// squared norms of nnet/lipschitz.d - where nothing else reads the product: one pass over x that squares on load
+// (dopt_hip_reduce_squares), the product rounded to fp32 before it is added and the sums in the reduction's own order,
+// so the value is the one the two kernels give; the product is never stored.  Tensors small enough for a tiny run have
+// been taken by one already (DOPT_HIP_PLAN_FUSE).
+void HIPPlan::Builder::fuseSquareSums()
+{
+    for (int id : p->mOps) {
+        const Operation &op = g.ops[id];
+        if (!live[id] || alias[id].source >= 0 || fusedKind[id] || prebuilt[id] || op.opType != "sum" || op.deps.size() != 1 ||
+            op.dtype != DOPT_HIP_F32 || op.volume() == 0)
+            continue;
+        const auto *axes = sizes_attr(op, "axes");
+        size_t off;
+        const int m = root(op.deps[0], &off);
+        const Operation &mo = g.ops[m];
+        if (!axes || off != 0 || mo.opType != "mul" || mo.deps.size() != 2 || mo.deps[0] != mo.deps[1] || mo.dtype != DOPT_HIP_F32 ||
+            !live[m] || fusedKind[m] || prebuilt[m] || isOutput(m) || uses[m].size() != 1 || uses[m][0].op != id ||
+            g.ops[mo.deps[0]].dtype != DOPT_HIP_F32 || g.ops[mo.deps[0]].volume() != mo.volume() ||
+            g.ops[op.deps[0]].volume() != mo.volume())
+            continue;
+        const std::vector<size_t> shape = g.ops[op.deps[0]].shape, ax = *axes;
+        // one run of adjacent reduced axes: the reduction is one pass (several runs go through temporaries or a kernel
+        // of their own, and gain nothing from squaring on load)
+        std::vector<char> red(shape.size(), 0);
+        bool valid = !ax.empty() && shape.size() <= 16;
+        for (size_t a : ax) {
+            if (a >= shape.size() || red[a]) { valid = false; break; }
+            red[a] = 1;
+        }
+        int runs = 0;
+        for (size_t i = 0; valid && i < shape.size(); i++)
+            if (red[i] && (i == 0 || !red[i - 1])) runs++;
+        if (!valid || runs != 1) continue;
+        fusedKind[id] = 11;
+        inputsOf[id] = {mo.deps[0]};
+        prebuilt[id] = make([=](const std::vector<const void *> &in, void *out) {
+            return dopt_hip_reduce_squares(shape.data(), (int)shape.size(), ax.data(), (int)ax.size(), (const float *)in[0],
+                                           (float *)out);
+        });
+        prebuiltLabel[id] = "mul+sum";
+    }
 }
 
 void HIPPlan::Builder::formChains()
@@ -2025,6 +2070,7 @@ int HIPPlan::create(Graph *graph, const std::vector<int> &outputs, unsigned flag
         b.fuseDenseLayers();
         b.fuseDenseBackward();
         b.formTinyRuns();
+        b.fuseSquareSums();
         b.formChains();
         b.absorbBiasGrads();
         b.absorbPools();

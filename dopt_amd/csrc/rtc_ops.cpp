@@ -237,6 +237,14 @@ const char *kReduceBody = R"SRC(
 
 __device__ inline T combine(T a, T b) { return (T)(COMBINE); }
 
+// what is folded is PRE(element): the element itself, or its square rounded to T (the value mul(x, x) would have stored)
+__device__ inline T4 pre4(T4 v)
+{
+    T4 r;
+    r.x = PRE(v.x); r.y = PRE(v.y); r.z = PRE(v.z); r.w = PRE(v.w);
+    return r;
+}
+
 __device__ inline T wave_reduce(T v)
 {
 #pragma unroll
@@ -272,13 +280,13 @@ extern "C" __global__ __launch_bounds__(BLOCK) void red_rows(const T *in, T *out
     T acc0 = (T)(IDENT), acc1 = (T)(IDENT), acc2 = (T)(IDENT), acc3 = (T)(IDENT);
     size_t i = start + threadIdx.x;
     for (; i + 3 * BLOCK < end; i += 4 * BLOCK) {
-        T v0 = row[i], v1 = row[i + BLOCK], v2 = row[i + 2 * BLOCK], v3 = row[i + 3 * BLOCK];
+        T v0 = PRE(row[i]), v1 = PRE(row[i + BLOCK]), v2 = PRE(row[i + 2 * BLOCK]), v3 = PRE(row[i + 3 * BLOCK]);
         acc0 = combine(acc0, v0);
         acc1 = combine(acc1, v1);
         acc2 = combine(acc2, v2);
         acc3 = combine(acc3, v3);
     }
-    for (; i < end; i += BLOCK) acc0 = combine(acc0, row[i]);
+    for (; i < end; i += BLOCK) acc0 = combine(acc0, PRE(row[i]));
     T acc = combine(combine(acc0, acc1), combine(acc2, acc3));
     acc = block_reduce(acc);
     if (threadIdx.x == 0) out[blockIdx.x] = acc;
@@ -297,14 +305,49 @@ extern "C" __global__ __launch_bounds__(BLOCK) void red_rows4(const T *in, T *ou
     T acc0 = (T)(IDENT), acc1 = (T)(IDENT), acc2 = (T)(IDENT), acc3 = (T)(IDENT);
     size_t i = q0 + threadIdx.x;
     for (; i + 3 * BLOCK < q1; i += 4 * BLOCK) {
-        T4 v0 = row[i], v1 = row[i + BLOCK], v2 = row[i + 2 * BLOCK], v3 = row[i + 3 * BLOCK];
+        T4 v0 = pre4(row[i]), v1 = pre4(row[i + BLOCK]), v2 = pre4(row[i + 2 * BLOCK]), v3 = pre4(row[i + 3 * BLOCK]);
         acc0 = combine(acc0, combine(combine(v0.x, v0.y), combine(v0.z, v0.w)));
         acc1 = combine(acc1, combine(combine(v1.x, v1.y), combine(v1.z, v1.w)));
         acc2 = combine(acc2, combine(combine(v2.x, v2.y), combine(v2.z, v2.w)));
         acc3 = combine(acc3, combine(combine(v3.x, v3.y), combine(v3.z, v3.w)));
     }
     for (; i < q1; i += BLOCK) {
-        T4 v0 = row[i];
+        T4 v0 = pre4(row[i]);
+        acc0 = combine(acc0, combine(combine(v0.x, v0.y), combine(v0.z, v0.w)));
+    }
+    T acc = combine(combine(acc0, acc1), combine(acc2, acc3));
+    acc = block_reduce(acc);
+    if (threadIdx.x == 0) out[blockIdx.x] = acc;
+}
+
+// The same order of sums from a buffer that is not 16-byte aligned (a view into a larger tensor): four 32-bit loads
+// per quad, so that a value does not depend on where its operand happens to start.
+__device__ inline T4 ld4(const T *p)
+{
+    T4 r;
+    r.x = PRE(p[0]); r.y = PRE(p[1]); r.z = PRE(p[2]); r.w = PRE(p[3]);
+    return r;
+}
+extern "C" __global__ __launch_bounds__(BLOCK) void red_rows4u(const T *in, T *out, size_t R, size_t chunk,
+                                                                size_t nchunks)
+{
+    const size_t o = blockIdx.x / nchunks, c = blockIdx.x % nchunks;
+    const size_t start = c * chunk;
+    size_t end = start + chunk;
+    if (end > R) end = R;
+    const T *row = in + o * R;
+    const size_t q0 = start / 4, q1 = end / 4;
+    T acc0 = (T)(IDENT), acc1 = (T)(IDENT), acc2 = (T)(IDENT), acc3 = (T)(IDENT);
+    size_t i = q0 + threadIdx.x;
+    for (; i + 3 * BLOCK < q1; i += 4 * BLOCK) {
+        T4 v0 = ld4(row + 4 * i), v1 = ld4(row + 4 * (i + BLOCK)), v2 = ld4(row + 4 * (i + 2 * BLOCK)), v3 = ld4(row + 4 * (i + 3 * BLOCK));
+        acc0 = combine(acc0, combine(combine(v0.x, v0.y), combine(v0.z, v0.w)));
+        acc1 = combine(acc1, combine(combine(v1.x, v1.y), combine(v1.z, v1.w)));
+        acc2 = combine(acc2, combine(combine(v2.x, v2.y), combine(v2.z, v2.w)));
+        acc3 = combine(acc3, combine(combine(v3.x, v3.y), combine(v3.z, v3.w)));
+    }
+    for (; i < q1; i += BLOCK) {
+        T4 v0 = ld4(row + 4 * i);
         acc0 = combine(acc0, combine(combine(v0.x, v0.y), combine(v0.z, v0.w)));
     }
     T acc = combine(combine(acc0, acc1), combine(acc2, acc3));
@@ -327,11 +370,11 @@ extern "C" __global__ __launch_bounds__(BLOCK) void red_cols(const T *in, T *out
         for (; r + 8 <= R; r += 8) {
             T v[8];
 #pragma unroll
-            for (int u = 0; u < 8; u++) v[u] = p[(r + u) * inner];
+            for (int u = 0; u < 8; u++) v[u] = PRE(p[(r + u) * inner]);
 #pragma unroll
             for (int u = 0; u < 8; u++) acc = combine(acc, v[u]);
         }
-        for (; r < R; r++) acc = combine(acc, p[r * inner]);
+        for (; r < R; r++) acc = combine(acc, PRE(p[r * inner]));
         out[idx] = acc;
     }
 }
@@ -438,7 +481,7 @@ extern "C" __global__ __launch_bounds__(BLOCK) void argmin_rows4_k(const T *in, 
 }
 )SRC";
 
-std::string reduce_source(bool is_sum, int dtype)
+std::string reduce_source(bool is_sum, int dtype, bool square = false)
 {
     std::string s;
     bool f = dtype == DOPT_HIP_F32;
@@ -454,6 +497,7 @@ std::string reduce_source(bool is_sum, int dtype)
         // identity -T.max (cpu/math.d:186): int32 starts at -INT_MAX, not INT_MIN
         s += f ? "#define IDENT -3.402823466e+38f\n" : "#define IDENT -2147483647\n";
     }
+    s += square ? "#define PRE(v) ((T)((v) * (v)))\n" : "#define PRE(v) (v)\n";
     s += kReduceBody;
     return s;
 }
@@ -484,9 +528,23 @@ int check_dtype(int dtype)
 }
 
 // One (outer, R, inner) reduction pass on the device.
-int reduce_pass(hipFunction_t rows, hipFunction_t rows4, hipFunction_t cols, const void *in, void *out, size_t outer,
-                size_t R, size_t inner, size_t esize)
+// `rows_plain` adds the partial results of a split row: the first stage may fold PRE(element), the second never does.
+struct ReduceKernels {
+    hipFunction_t rows, rows4, rows4u, cols;
+};
+int reduce_kernels(const std::string &key, const std::string &src, ReduceKernels *k)
 {
+    if (int rc = rtc_get(key + ":rows", src, "red_rows", &k->rows)) return rc;
+    if (int rc = rtc_get(key + ":rows4", src, "red_rows4", &k->rows4)) return rc;
+    if (int rc = rtc_get(key + ":rows4u", src, "red_rows4u", &k->rows4u)) return rc;
+    return rtc_get(key + ":cols", src, "red_cols", &k->cols);
+}
+
+int reduce_pass(const ReduceKernels &k, const void *in, void *out, size_t outer, size_t R, size_t inner, size_t esize,
+                hipFunction_t rows_plain = nullptr)
+{
+    const hipFunction_t rows = k.rows, rows4 = k.rows4, cols = k.cols;
+    if (!rows_plain) rows_plain = rows;
     if (outer * inner == 0) return DOPT_HIP_OK;
     if (inner > 1 || R <= 64) {
         unsigned grid = grid_for(256, outer * inner);
@@ -504,7 +562,7 @@ int reduce_pass(hipFunction_t rows, hipFunction_t rows4, hipFunction_t cols, con
     size_t chunk = ceil_div(R, nchunks);
     chunk = (chunk + 1023) / 1024 * 1024;
     nchunks = ceil_div(R, chunk);
-    hipFunction_t first = (R % 4 == 0 && aligned16(in)) ? rows4 : rows;
+    hipFunction_t first = R % 4 == 0 ? (aligned16(in) ? rows4 : k.rows4u) : rows;
     if (nchunks == 1) {
         void *args[] = {(void *)&in, (void *)&out, (void *)&R, (void *)&chunk, (void *)&nchunks};
         return rtc_launch(first, (unsigned)outer, 256, args);
@@ -519,7 +577,7 @@ int reduce_pass(hipFunction_t rows, hipFunction_t rows4, hipFunction_t cols, con
     size_t one = 1, r2 = nchunks, chunk2 = (nchunks + 255) / 256 * 256;
     const void *pin = partial;
     void *args[] = {(void *)&pin, (void *)&out, (void *)&r2, (void *)&chunk2, (void *)&one};
-    return rtc_launch(rows, (unsigned)outer, 256, args);
+    return rtc_launch(rows_plain, (unsigned)outer, 256, args);
 }
 
 }  // namespace
@@ -640,8 +698,13 @@ int dopt_hip_pointwise_arity(const char *op)
     return info ? info->arity : 0;
 }
 
-int dopt_hip_reduce(const char *op, int dtype, const size_t *shape, int rank, const size_t *axes, int naxes,
-                    const void *in, void *out)
+}  // extern "C"
+
+namespace {
+
+// `square`: what is folded is each element's square, rounded to fp32 before it is added (sum only).
+int reduce_impl(const char *op, int dtype, const size_t *shape, int rank, const size_t *axes, int naxes, const void *in,
+                void *out, bool square)
 {
     DOPT_REQUIRE(op && shape && axes, "dopt_hip_reduce: null argument");
     bool is_sum = !strcmp(op, "sum");
@@ -668,7 +731,7 @@ int dopt_hip_reduce(const char *op, int dtype, const size_t *shape, int rank, co
             if (!reduced[i]) kept *= shape[i];
         if (kept == 0) return DOPT_HIP_OK;
         DOPT_REQUIRE(out != nullptr, "dopt_hip_reduce: null argument");
-        if (is_sum) return dopt_hip_memset(out, 0, kept * 4);
+        if (is_sum) return dopt_hip_memset(out, 0, kept * 4);   // also the sum of no squares
         std::vector<uint32_t> start(kept);
         const float lowest = -std::numeric_limits<float>::max();
         uint32_t bits;
@@ -691,7 +754,7 @@ int dopt_hip_reduce(const char *op, int dtype, const size_t *shape, int rank, co
     }
     // fp32 sum over everything but one run of axes in the middle ([N, C, inner] -> [C], the shape of a
     // per-channel statistic): one launch instead of one pass per run of reduced axes
-    if (is_sum && dtype == DOPT_HIP_F32 && runs.size() == 2 && runs[0].first == 0 && runs[1].second == rank - 1) {
+    if (is_sum && !square && dtype == DOPT_HIP_F32 && runs.size() == 2 && runs[0].first == 0 && runs[1].second == rank - 1) {
         size_t N = 1, C = 1, inner = 1;
         for (int i = 0; i <= runs[0].second; i++) N *= cur[i];
         for (int i = runs[0].second + 1; i < runs[1].first; i++) C *= cur[i];
@@ -701,10 +764,10 @@ int dopt_hip_reduce(const char *op, int dtype, const size_t *shape, int rank, co
     }
     std::string key = std::string("red:") + op + (dtype == DOPT_HIP_F32 ? ":f32" : ":i32");
     std::string src = reduce_source(is_sum, dtype);
-    hipFunction_t rows, rows4, cols;
-    if (int rc = rtc_get(key + ":rows", src, "red_rows", &rows)) return rc;
-    if (int rc = rtc_get(key + ":rows4", src, "red_rows4", &rows4)) return rc;
-    if (int rc = rtc_get(key + ":cols", src, "red_cols", &cols)) return rc;
+    ReduceKernels plain{}, squares{};   // `squares`: the first pass of a sum of squares
+    if (int rc = reduce_kernels(key, src, &plain)) return rc;
+    if (square)
+        if (int rc = reduce_kernels("red:sumsq:f32", reduce_source(true, dtype, true), &squares)) return rc;
     const void *src_ptr = in;
     void *tmp_prev = nullptr;
     int rc = DOPT_HIP_OK;
@@ -721,13 +784,50 @@ int dopt_hip_reduce(const char *op, int dtype, const size_t *shape, int rank, co
             if (rc) break;
             dst = tmp;
         }
-        rc = reduce_pass(rows, rows4, cols, src_ptr, dst, outer, R, inner, 4);
+        const bool first = square && ri == (int)runs.size() - 1;   // only what is read from `in` is squared
+        rc = first ? reduce_pass(squares, src_ptr, dst, outer, R, inner, 4, plain.rows)
+                   : reduce_pass(plain, src_ptr, dst, outer, R, inner, 4);
         if (tmp_prev) dopt_hip_free(tmp_prev);
         tmp_prev = tmp;
         src_ptr = dst;
         for (int i = a0; i <= a1; i++) cur[i] = 1;
     }
     if (tmp_prev) dopt_hip_free(tmp_prev);
+    return rc;
+}
+
+}  // namespace
+
+extern "C" {
+
+int dopt_hip_reduce(const char *op, int dtype, const size_t *shape, int rank, const size_t *axes, int naxes,
+                    const void *in, void *out)
+{
+    return reduce_impl(op, dtype, shape, rank, axes, naxes, in, out, false);
+}
+
+int dopt_hip_reduce_squares(const size_t *shape, int rank, const size_t *axes, int naxes, const float *in, float *out)
+{
+    DOPT_REQUIRE(shape && axes, "dopt_hip_reduce_squares: null argument");
+    DOPT_REQUIRE(rank >= 1 && rank <= 16 && naxes >= 1 && naxes <= rank, "dopt_hip_reduce_squares: bad rank/axes count");
+    // One run of adjacent reduced axes is one pass that squares on load.  Several runs take dopt_hip_reduce's own route
+    // (which has a kernel of its own for sums around a kept run of axes), on the stored product: same value either way.
+    bool reduced[16] = {false};
+    for (int i = 0; i < naxes; i++)
+        if (axes[i] < (size_t)rank) reduced[axes[i]] = true;
+    int runs = 0;
+    size_t vol = 1;
+    for (int i = 0; i < rank; i++) {
+        vol *= shape[i];
+        if (reduced[i] && (i == 0 || !reduced[i - 1])) runs++;
+    }
+    if (runs <= 1 || vol == 0) return reduce_impl("sum", DOPT_HIP_F32, shape, rank, axes, naxes, in, out, true);
+    DOPT_REQUIRE(in && out, "dopt_hip_reduce_squares: null argument");
+    void *product = nullptr;
+    if (int rc = scratch_alloc(&product, vol * sizeof(float))) return rc;
+    int rc = dopt_hip_pointwise("mul", DOPT_HIP_F32, vol, in, in, product);
+    if (!rc) rc = reduce_impl("sum", DOPT_HIP_F32, shape, rank, axes, naxes, product, out, false);
+    dopt_hip_free(product);
     return rc;
 }
 
@@ -763,6 +863,8 @@ int dopt_hip_rtc_compile_only(const char *op, int dtype, const char *arch)
     std::string src;
     if (!strcmp(op, "sum") || !strcmp(op, "maxElement")) {
         src = reduce_source(!strcmp(op, "sum"), dtype);
+    } else if (!strcmp(op, "sumOfSquares")) {   // the first pass of dopt_hip_reduce_squares
+        src = reduce_source(true, DOPT_HIP_F32, true);
     } else if (!strcmp(op, "argmin")) {
         src = argmin_source(dtype);
     } else {

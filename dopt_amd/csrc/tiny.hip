@@ -186,7 +186,8 @@ __device__ __forceinline__ void reduce_node(const dopt_hip_tiny_node &nd, AP in,
         }
         return;
     }
-    const bool quads = R % 4 == 0 && in_aligned;   // dopt_hip_reduce's test, on the tensor as it lies in memory
+    (void)in_aligned;
+    const bool quads = R % 4 == 0;   // dopt_hip_reduce's test: the order does not depend on where the row starts in memory
     for (int o = 0; o < outer; o++) reduce_row<kSum, AP>(in + (size_t)o * R, R, quads, out ? out + o : nullptr, out2 ? out2 + o : nullptr, part);
 }
 

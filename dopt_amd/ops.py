@@ -150,6 +150,15 @@ def max_element(a, axes=None, out=None):
     return _reduce(b"maxElement", a, axes, out)
 
 
+def sum_of_squares(a, axes=None, out=None):
+    """sum(mul(a, a), axes) without storing the product: same value as the two operations."""
+    axes = list(range(len(a.shape))) if not axes else [int(x) for x in axes]
+    out = _out(out, [s for i, s in enumerate(a.shape) if i not in axes], a.dtype)
+    capi.check(capi.load().dopt_hip_reduce_squares(capi.sizes(a.shape), len(a.shape), capi.sizes(axes), len(axes),
+                                                   a.ptr, out.ptr))
+    return out
+
+
 def argmin(a, axis, out=None):
     oshape = list(a.shape)
     oshape[axis] = 1

@@ -179,6 +179,11 @@ int dopt_hip_tiny_graph(int nslots, void *const *slots, int nnodes, const dopt_h
    tensor; out has the reduced axes removed (core/ops/math.d:162-175). */
 int dopt_hip_reduce(const char *op, int dtype, const size_t *shape, int rank,
                     const size_t *axes, int naxes, const void *in, void *out);
+/* sum(mul(x, x)) over `axes` in one pass over x - the L2 penalty of a parameter as nnet/layers build it
+   (`weightDecay * sum(filters * filters)`, nnet/layers/conv.d:117; the norms of nnet/layers/conv.d:131-132, 184-187): every square is rounded to
+   fp32 before it is added and the sums run in dopt_hip_reduce's order, so the value is that of the two operations
+   run one after the other; the product is never stored.  fp32 only. */
+int dopt_hip_reduce_squares(const size_t *shape, int rank, const size_t *axes, int naxes, const float *in, float *out);
 /* `argmin`: cpu/math.d:249-310.  int32 output with the reduced axis kept as size 1
    (core/ops/math.d:185-191); the first minimum wins; a lane with no element below the
    type's maximum yields index 0. */

@@ -623,6 +623,31 @@ def test_output_only_products_of_a_plan_share_a_launch():
         assert np.array_equal(a, b) or (a.ndim == 1 and np.allclose(a, b, rtol=0, atol=2e-5))
 
 
+def test_weight_decay_terms_square_on_load():
+    """`weightDecay * sum(filters * filters)` (nnet/layers/conv.d:117): with the rewrites on the product is never stored
+    (`mul+sum`, one pass over the filter); loss and gradients are those of the plan without rewrites, bit for bit.
+    Filters of at most 4096 values go into a tiny run instead (here: the first layer's)."""
+    r = np.random.default_rng(81)
+    X = r.standard_normal((8, 3, 8, 8)).astype(np.float32)
+    Y = np.eye(10, dtype=np.float32)[r.integers(0, 10, 8)]
+    x, y = core.float32([8, 3, 8, 8]), core.float32([8, 10])
+    init = nnet.Init(82)
+    h = nnet.relu(nnet.conv2D(nnet.dataSource(x), 32, (3, 3), init, padding=(1, 1), weight_decay=1e-2))
+    h = nnet.relu(nnet.conv2D(h, 64, (3, 3), init, padding=(1, 1), weight_decay=1e-2))
+    h = nnet.relu(nnet.conv2D(h, 64, (3, 3), init, padding=(1, 1), stride=(2, 2), weight_decay=1e-2))
+    top = nnet.softmax(nnet.dense(h, 10, init))
+    net = nnet.DAGNetwork([x], [top])
+    loss = nnet.crossEntropy(top.trainOutput, y) + net.paramLoss
+    outs = [loss] + core.grad(loss, net.params)
+    plan = core.compile(outs, core.PLAN_VIEWS | core.PLAN_FUSE | core.PLAN_TIMING)
+    fused = plan.execute({x: X, y: Y})
+    prof = plan.profile()
+    assert prof["mul+sum"][1] == 2, prof
+    plain = core.compile(outs, core.PLAN_VIEWS).execute({x: X, y: Y})
+    for a, b in zip(plain, fused):
+        assert np.array_equal(a, b)
+
+
 @pytest.mark.parametrize("M,N,K,ta,tb", [(128, 512, 512, 0, 0),     # the small-output kernel: the epilogue does it
                                           (512, 512, 128, 1, 0),     # a weight gradient: dz stored [K][M]
                                           (10, 512, 128, 1, 0),

@@ -147,6 +147,31 @@ def test_sum_and_max(shape, axes):
     assert np.array_equal(ops.max_element(T(xi), axes).numpy(), O.max_element(xi, axes))
 
 
+@pytest.mark.parametrize("shape,axes", [
+    ((640, 640, 3, 3), None), ((320, 160, 1, 1), None), ((7,), None), ((3, 4, 5), (1,)), ((3, 4, 5), (0, 2)),
+    ((5, 70001), (1,)), ((2048, 33), (1,)), ((4, 6), (0,)), ((16, 8, 16, 32), (0, 2, 3)), ((2, 3, 100000), None),
+    ((0, 4), (0,)),
+])
+def test_sum_of_squares_is_the_sum_of_the_stored_product(shape, axes):
+    """dopt_hip_reduce_squares against mul followed by sum, bit for bit (one launch less and the product never stored),
+    and against float64 within the stated tolerance; also from a buffer off the 16-byte grid."""
+    r = rng(13)
+    x = r.standard_normal(shape).astype(np.float32)
+    got = ops.sum_of_squares(T(x), axes).numpy()
+    two = ops.sum(ops.pointwise("mul", T(x), T(x)), axes).numpy()
+    assert got.shape == two.shape and np.array_equal(got, two)
+    if x.size:
+        red = int(np.prod([shape[a] for a in (axes or range(len(shape)))]))
+        want = (x.astype(np.float64) ** 2).sum(axis=tuple(axes) if axes else None)
+        assert_close(got, want, "sum of squares", scale=np.sqrt(red))
+        # from a view one float off the 16-byte grid: the same bits (the order of the sums does not depend on alignment)
+        whole = T(np.concatenate([[3.0], x.ravel()]).astype(np.float32))
+        assert np.array_equal(ops.sum_of_squares(whole.view(1, shape), axes).numpy(), two)
+        ax = sorted(axes or range(len(shape)))
+        if ax == list(range(ax[0], ax[-1] + 1)):   # one run of adjacent axes: one pass (several runs have routes of their own)
+            assert np.array_equal(ops.sum(whole.view(1, shape), axes).numpy(), ops.sum(T(x), axes).numpy())
+
+
 def test_max_identity_is_minus_type_max():
     x = np.full((3, 5), -2**31, np.int32)
     assert np.array_equal(ops.max_element(T(x), (1,)).numpy(), O.max_element(x, (1,)))
