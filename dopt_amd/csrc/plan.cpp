@@ -1266,12 +1266,34 @@ void HIPPlan::Builder::formChains()
         if (!is_pw(id)) continue;
         int target = -1;
         bool joins = !isOutput(id) && !uses[id].empty();
-        for (const Use &u : uses[id]) {
-            if (!joins) break;
-            if (chainOf[u.op] < 0 || u.off != 0 || g.ops[u.op].volume() != g.ops[id].volume()) joins = false;
+        auto reader_joins = [&](const Use &u, size_t volume) {   // the reader is a member of the one chain, and reads all of it
+            if (chainOf[u.op] < 0 || u.off != 0 || g.ops[u.op].volume() != volume) joins = false;
             else if (g.ops[u.op].opType == "reluGrad" && u.slot == 1) joins = false;   // the y operand is not part of the node
             else if (target < 0) target = chainOf[u.op];
             else if (target != chainOf[u.op]) joins = false;
+        };
+        for (const Use &u : uses[id]) {
+            if (!joins) break;
+            // A one-element value that is only ever broadcast (repeat) into members of one chain - the scalar arithmetic
+            // of a loss term or an update rule in front of the tensor it scales - is a node of that chain too: every
+            // thread computes it again from the one-element operands, with the stand-alone kernel's expression.
+            const Operation &ro = g.ops[u.op];
+            if (g.ops[id].volume() == 1 && ro.opType == "repeat" && ro.deps.size() == 1 && u.off == 0 && u.slot == 0 &&
+                ro.volume() > 1 && alias[u.op].source < 0 && !isOutput(u.op) && live[u.op] && !fusedKind[u.op] && !uses[u.op].empty()) {
+                for (const Use &u2 : uses[u.op]) {
+                    if (!joins) break;
+                    reader_joins(u2, ro.volume());
+                }
+                continue;
+            }
+            // the same through the reference's other broadcast, the product with a ones vector ([n,1] x [1,1] or
+            // [1,1] x [1,n], core/ops/basic.d:370-381): the member reads the value as its one-element operand
+            if (g.ops[id].volume() == 1 && ro.volume() > 1 && outer_cols(u.op) && chainOf[u.op] >= 0 && u.off == 0 &&
+                ((u.slot == 1 && ro.shape[1] == 1) || (u.slot == 0 && ro.shape[0] == 1))) {
+                reader_joins(u, ro.volume());
+                continue;
+            }
+            reader_joins(u, g.ops[id].volume());
         }
         if (joins && chainOps[target].size() >= 48) joins = false;
         const size_t cols = outer_grid(id);
@@ -1304,8 +1326,13 @@ void HIPPlan::Builder::formChains()
             const Operation &ro = g.ops[r];
             size_t soff = 0;
             if (ro.opType == "repeat" && ro.deps.size() == 1 && off == 0 && alias[r].source < 0 &&
-                g.ops[ro.deps[0]].volume() == 1 && g.ops[root(ro.deps[0], &soff)].dtype == DOPT_HIP_F32)
+                g.ops[ro.deps[0]].volume() == 1 && g.ops[root(ro.deps[0], &soff)].dtype == DOPT_HIP_F32) {
+                const int sr = root(ro.deps[0], &soff);
+                if (chainOf[sr] == end && nodeOf[sr] >= 0 && soff == 0) return -2 - nodeOf[sr];   // a one-element member
                 return input_index(ro.deps[0], 1);
+            }
+            // the operands of a one-element member of a larger chain are single elements
+            if (g.ops[dep].volume() == 1 && g.ops[end].volume() > 1) return input_index(dep, 1);
             return input_index(dep, 0);
         };
         for (int id : members) {
@@ -1314,8 +1341,14 @@ void HIPPlan::Builder::formChains()
             if (outer_cols(id)) {
                 node.op = "mul";
                 const bool one_col = o.shape[1] == 1, one_row = o.shape[0] == 1;
-                node.lhs = input_index(o.deps[0], one_row ? 1 : (one_col ? 0 : 2));
-                node.rhs = input_index(o.deps[1], one_col ? 1 : (one_row ? 0 : 3));
+                auto element = [&](int dep, int kind) {   // a single element may be a one-element member of this chain
+                    size_t eoff;
+                    const int sr = root(dep, &eoff);
+                    if (kind == 1 && chainOf[sr] == end && nodeOf[sr] >= 0 && eoff == 0) return -2 - nodeOf[sr];
+                    return input_index(dep, kind);
+                };
+                node.lhs = element(o.deps[0], one_row ? 1 : (one_col ? 0 : 2));
+                node.rhs = element(o.deps[1], one_col ? 1 : (one_row ? 0 : 3));
             } else if (o.opType == "reluGrad") {
                 node.lhs = operand(o.deps[0]);
                 node.rhs = operand(o.deps[2]);

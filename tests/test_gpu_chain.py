@@ -130,6 +130,30 @@ def test_chain_keeps_values_that_something_else_reads():
         assert np.array_equal(g, w)
 
 
+def test_scalar_arithmetic_joins_the_chain_it_is_broadcast_into():
+    """`weightDecay * sum(...)` differentiated gives (one-element value) x (one-element value), broadcast over the filter
+    by the product with a ones vector (core/ops/basic.d:370-381): the one-element product has no kernel of its own, the
+    chain over the filter computes it; the same through a `repeat`.  Values as in the plan without rewrites."""
+    r = np.random.default_rng(5)
+    n = 6000                                     # above the tiny-run limit
+    w = core.float32([n], r.standard_normal(n).astype(np.float32))
+    g = core.float32([n], r.standard_normal(n).astype(np.float32))
+    u = core.float32([1], np.float32([0.37]))
+    s = core.sum(g)                              # a reduction: rank 0, not part of any chain
+    t = (s * 0.5) * 1.25                         # two one-element nodes, read only through the broadcast
+    out = w * t + g                              # rank 0 against rank 1: repeat(t, n) = ones[n,1] x t[1,1]
+    v = core.exp(u * 0.3)                        # one-element nodes again
+    out2 = core.repeat(v, [n]) * w - g           # ... broadcast by a repeat
+    outs = [out, out2]
+    plan = core.compile(outs, core.PLAN_VIEWS | core.PLAN_FUSE | core.PLAN_TIMING)
+    got = plan.execute()
+    prof = plan.profile()
+    assert "mul" not in prof and "exp" not in prof, prof
+    want = core.compile(outs).execute()
+    for a, b in zip(got, want):
+        assert np.array_equal(a, b)
+
+
 def _random_graph(r, n_leaves=4, n_ops=18, size=96):
     """A random DAG over [size]-vectors and [8, size/8] matrices: pointwise nodes, scalar broadcasts,
     reshapes, contiguous slices padded back, reductions as side consumers, a few outputs in the middle."""
