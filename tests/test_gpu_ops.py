@@ -846,6 +846,8 @@ def test_sgemm_short_reduction_large_output(shape):
 @pytest.mark.parametrize("shape", [(1024, 1024, 1024),   # 64 tiles, the reduction split over workgroups
                                    (2100, 2050, 36),     # more tiles than the small-output kernel takes, ragged edges
                                    (1100, 1030, 1026),   # a reduction that is no multiple of 4: element-wise loads
+                                   (900, 1300, 515),     # ragged edges on both sides, odd reduction length
+                                   (1600, 1500, 640),    # 128 x 128 tiles, the reduction split over workgroups
                                    (4096, 640, 70)])
 def test_sgemm_large_products_all_operand_layouts(shape):
     """Products of more than 64 rows that the small-output kernel does not take (sgemm_rows_k): against float64, and
