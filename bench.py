@@ -171,8 +171,8 @@ def host_feed_leg(step, steps, warmup):
     sec_plain = (time.perf_counter() - t0) / steps
     return {"ms_per_step": round(sec * 1e3, 4), "images_per_s": round(BATCH / sec, 1),
             "what": "the step with every batch coming from host memory: shuffled host dataset -> page-locked staging -> queued "
-                    "upload -> augmentation kernel (mirrored pad 4, random crop, horizontal flip) -> training step; host fill of "
-                    "batch k+1 overlaps the device work of batch k",
+                    "upload on the second queue -> augmentation kernel (mirrored pad 4, random crop, horizontal flip) -> "
+                    "training step; host fill and upload of batch k+1 overlap the device work of batch k",
             "pageable_args_ms_per_step": round(sec_plain * 1e3, 4),
             "pageable_args_what": "the same step with pageable numpy arrays as plan arguments: the plan uploads them inside each "
                                   "execution, as CUDAPlan.executeImpl does"}

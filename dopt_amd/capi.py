@@ -77,6 +77,8 @@ PROTOTYPES = {
     "dopt_hip_pointwise_arity": [C.c_char_p],
     "dopt_hip_reduce": [C.c_char_p, _i, _szp, _i, _szp, _i, _vp, _vp],
     "dopt_hip_reduce_squares": [_szp, _i, _szp, _i, _vp, _vp],
+    "dopt_hip_copy_h2d_beside": [_vp, _vp, _sz],
+    "dopt_hip_upload_join": [],
     "dopt_hip_argmin": [_i, _szp, _i, _sz, _vp, _vp],
     "dopt_hip_rtc_compile_only": [C.c_char_p, _i, C.c_char_p],
     "dopt_hip_slice": [_i, _szp, _szp, _szp, _vp, _vp],

@@ -25,6 +25,7 @@ struct Runtime {
     std::string arch = "gfx950";
     hipStream_t stream = nullptr;
     hipStream_t side = nullptr;     // second in-order queue for work a plan overlaps with its main chain
+    hipEvent_t uploads = nullptr;   // behind the uploads queued beside the main queue (dopt_hip_copy_h2d_beside)
     int lane = 0;                   // which of the two the entry points currently enqueue on
     bool capturing = false;         // a plan is recording its kernels into a HIP graph
 
@@ -89,6 +90,7 @@ int init_locked(int device)
                     r.arch.c_str());
     DOPT_HIP_CHECK(hipStreamCreateWithFlags(&r.stream, hipStreamNonBlocking));
     DOPT_HIP_CHECK(hipStreamCreateWithFlags(&r.side, hipStreamNonBlocking));   // same (default) priority
+    DOPT_HIP_CHECK(hipEventCreateWithFlags(&r.uploads, hipEventDisableTiming));
     // addresses (and the one-time fill) of the file-scope device arrays: nothing is left for a first call to set up
     if (int rc = bn_device_setup()) return rc;
     if (int rc = nn_device_setup()) return rc;
@@ -276,6 +278,8 @@ int dopt_hip_shutdown(void)
     for (hipModule_t m : r.modules) (void)hipModuleUnload(m);
     r.modules.clear();
     r.kernels.clear();
+    if (r.uploads) (void)hipEventDestroy(r.uploads);
+    r.uploads = nullptr;
     (void)hipStreamDestroy(r.stream);
     (void)hipStreamDestroy(r.side);
     r.stream = r.side = nullptr;
@@ -433,6 +437,25 @@ int dopt_hip_copy_h2d_async(void *dst, const void *pinned_src, size_t bytes)
     DOPT_REQUIRE(dst && pinned_src, "dopt_hip_copy_h2d_async: null pointer");
     DOPT_ENSURE_INIT();
     DOPT_HIP_CHECK(hipMemcpyAsync(dst, pinned_src, bytes, hipMemcpyHostToDevice, stream()));
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_copy_h2d_beside(void *dst, const void *pinned_src, size_t bytes)
+{
+    if (bytes == 0) return DOPT_HIP_OK;
+    DOPT_REQUIRE(dst && pinned_src, "dopt_hip_copy_h2d_beside: null pointer");
+    DOPT_ENSURE_INIT();
+    DOPT_REQUIRE(!rt().capturing, "dopt_hip_copy_h2d_beside: not while a plan records its kernels");
+    DOPT_HIP_CHECK(hipMemcpyAsync(dst, pinned_src, bytes, hipMemcpyHostToDevice, lane_stream(1)));
+    return DOPT_HIP_OK;
+}
+
+int dopt_hip_upload_join(void)
+{
+    DOPT_ENSURE_INIT();
+    DOPT_REQUIRE(!rt().capturing, "dopt_hip_upload_join: not while a plan records its kernels");
+    DOPT_HIP_CHECK(hipEventRecord(rt().uploads, lane_stream(1)));
+    DOPT_HIP_CHECK(hipStreamWaitEvent(lane_stream(0), rt().uploads, 0));
     return DOPT_HIP_OK;
 }
 

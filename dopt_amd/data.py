@@ -92,11 +92,13 @@ class PinnedArray:
         buf = (C.c_char * self.nbytes).from_address(self.ptr)
         self.array = np.frombuffer(buf, dtype=dtype).reshape(shape)
 
-    def upload_async(self, tensor):
-        """Queues the copy into `tensor`; the host must not refill this memory before the next sync."""
+    def upload_async(self, tensor, beside=False):
+        """Queues the copy into `tensor`; the host must not refill this memory before the next sync.  `beside`: on the
+        library's second queue, next to the work already queued instead of behind it (join with dopt_hip_upload_join)."""
         if tensor.nbytes != self.nbytes:
             raise capi.HipError(1, "Mismatch in buffer size")
-        capi.check(capi.load().dopt_hip_copy_h2d_async(tensor.ptr, self.ptr, self.nbytes))
+        lib = capi.load()
+        capi.check((lib.dopt_hip_copy_h2d_beside if beside else lib.dopt_hip_copy_h2d_async)(tensor.ptr, self.ptr, self.nbytes))
 
     def __del__(self):
         if getattr(self, "ptr", None):
@@ -188,8 +190,12 @@ class DeviceFeed:
         capi.check(lib.dopt_hip_event_record(self._marks[j & 1]))
         self.dataset.getBatch([s["f_host"].array, s["l_host"].array])
         s["g_host"].array[:] = draw_geometry(self._rng, self.batch, self.jx, self.jy, self.fx, self.fy)
-        s["f_host"].upload_async(s["raw"])
-        s["l_host"].upload_async(s["l"])
-        s["g_host"].upload_async(s["g"])
+        # The three uploads go to the second queue: the copy engine moves them while the first queue is still busy with
+        # the step on the previous batch (nothing on the device reads this slot's buffers any more: the wait above).
+        # The augmentation kernel, and whatever the caller queues next, waits for them.
+        s["f_host"].upload_async(s["raw"], beside=True)
+        s["l_host"].upload_async(s["l"], beside=True)
+        s["g_host"].upload_async(s["g"], beside=True)
+        capi.check(lib.dopt_hip_upload_join())
         image_transform(s["raw"], self.jx, self.jy, s["g"], out=s["f"])
         return s["f"], s["l"]

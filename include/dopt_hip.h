@@ -82,6 +82,13 @@ int dopt_hip_copy_d2d(void *dst, const void *src, size_t bytes);
 int dopt_hip_host_alloc(void **host_ptr, size_t bytes);
 int dopt_hip_host_free(void *host_ptr);
 int dopt_hip_copy_h2d_async(void *dst, const void *pinned_src, size_t bytes);
+/* The same upload on the library's second queue: it runs BESIDE whatever the first queue is doing (the training step
+   on the previous batch) instead of behind it - the copy engine moves the bytes, no compute unit is involved.
+   dopt_hip_upload_join makes everything enqueued on the first queue afterwards wait for the uploads queued so far.  The
+   caller must know that nothing still running reads `dst` (dopt_hip_event_sync on an event recorded behind its last
+   reader).  No counterpart in the reference, whose uploads block (cuda/package.d:172-176). */
+int dopt_hip_copy_h2d_beside(void *dst, const void *pinned_src, size_t bytes);
+int dopt_hip_upload_join(void);
 /* n device-to-device copies, in order; copies of at most 64 KiB share kernel launches.  Stands
    for the loop of cuMemcpy calls that hands a plan's outputs to the caller's buffers
    (cuda/package.d:419-422): most of them are a few hundred bytes of batch-norm statistics. */
