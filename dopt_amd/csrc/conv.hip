@@ -1379,6 +1379,18 @@ int patch_decide_splits(PatchSetup *u, const float *out)
 
 // `prepacked`: the filter already in the kernel's layout (dopt_hip_conv_pack_batch), or null to
 // pack it here first.
+// The launch of a filled-in patch setup: the tile shape picks the instance.
+int dispatch_patch(const PatchSetup &u, int splits)
+{
+    const PatchConv &pc = u.pc;
+    const dim3 grid(xcd_grid((unsigned)(u.tiles * splits)));
+    const bool c_full = pc.Cin % 16 == 0;
+    if (u.shape == 0) return launch_patch<GatherWide, 24>(pc, c_full, grid, u.lds_bytes);
+    if (u.shape == 1) return launch_patch<GatherSquare, 16>(pc, c_full, grid, u.lds_bytes);
+    if (u.shape == 3) return launch_patch<GatherTall, 16>(pc, c_full, grid, u.lds_bytes);
+    return launch_patch<GatherDeep, 16>(pc, c_full, grid, u.lds_bytes);
+}
+
 template <bool kBwd>
 int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, const float *w, const float *bias,
               float *out, bool *done, const float *prepacked = nullptr, dopt_hip_split_sum *open = nullptr)
@@ -1411,14 +1423,7 @@ int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, 
     pc.in_bytes = (size_t)pc.N * pc.Cin * pc.IH * pc.IW * sizeof(float);
     pc.wp_bytes = u.wp_elems * sizeof(float);
     pc.out = splits > 1 ? partial : out;
-    const dim3 grid(xcd_grid((unsigned)(tiles * splits)));
-    const bool c_full = pc.Cin % 16 == 0;
-    int rc;
-    if (u.shape == 0) rc = launch_patch<GatherWide, 24>(pc, c_full, grid, u.lds_bytes);
-    else if (u.shape == 1) rc = launch_patch<GatherSquare, 16>(pc, c_full, grid, u.lds_bytes);
-    else if (u.shape == 3) rc = launch_patch<GatherTall, 16>(pc, c_full, grid, u.lds_bytes);
-    else rc = launch_patch<GatherDeep, 16>(pc, c_full, grid, u.lds_bytes);
-    if (rc) return rc;
+    if (int rc = dispatch_patch(u, splits)) return rc;
     *done = true;
     if (splits > 1 && open) {   // the caller's next call adds the copies
         open->partial = partial;
@@ -2205,6 +2210,23 @@ int wgrad_split_sum(const WgradSetup &u, const float *partial, float *dw)
     return launch_split_sum(n4, u.splits, wgrad_sum_lanes(n4), partial, dw);
 }
 
+// The launch of a filled-in filter-gradient setup: tile height and pixel geometry pick the instance.
+int dispatch_wgrad_patch(const WgradSetup &u)
+{
+    const WgradPatch &wp = u.wp;
+    const dim3 grid(xcd_grid((unsigned)(u.tiles * u.splits)));
+    const int geo = u.geo;
+    if (u.rows == 160) return geo == 0 ? launch_wgrad_patch<5, 1, 0>(wp, grid, u.lds_bytes)
+                            : geo == 1 ? launch_wgrad_patch<5, 1, 1>(wp, grid, u.lds_bytes)
+                                       : launch_wgrad_patch<5, 1, 2>(wp, grid, u.lds_bytes);
+    if (u.tall) return geo == 0 ? launch_wgrad_patch<4, 1, 0>(wp, grid, u.lds_bytes)
+                     : geo == 1 ? launch_wgrad_patch<4, 1, 1>(wp, grid, u.lds_bytes)
+                                : launch_wgrad_patch<4, 1, 2>(wp, grid, u.lds_bytes);
+    return geo == 0 ? launch_wgrad_patch<2, 2, 0>(wp, grid, u.lds_bytes)
+         : geo == 1 ? launch_wgrad_patch<2, 2, 1>(wp, grid, u.lds_bytes)
+                    : launch_wgrad_patch<2, 2, 2>(wp, grid, u.lds_bytes);
+}
+
 int run_wgrad_patch(const dopt_hip_conv_desc *d, const float *dy, const float *x, float *dw, bool *done)
 {
     *done = false;
@@ -2218,19 +2240,7 @@ int run_wgrad_patch(const dopt_hip_conv_desc *d, const float *dy, const float *x
     }
     wp.dy = dy; wp.x = x;
     wp.out = u.splits > 1 ? partial : dw;
-    const dim3 grid(xcd_grid((unsigned)(u.tiles * u.splits)));
-    const int geo = u.geo;
-    int rc;
-    if (u.rows == 160) rc = geo == 0 ? launch_wgrad_patch<5, 1, 0>(wp, grid, u.lds_bytes)
-                        : geo == 1 ? launch_wgrad_patch<5, 1, 1>(wp, grid, u.lds_bytes)
-                                   : launch_wgrad_patch<5, 1, 2>(wp, grid, u.lds_bytes);
-    else if (u.tall) rc = geo == 0 ? launch_wgrad_patch<4, 1, 0>(wp, grid, u.lds_bytes)
-                   : geo == 1 ? launch_wgrad_patch<4, 1, 1>(wp, grid, u.lds_bytes)
-                              : launch_wgrad_patch<4, 1, 2>(wp, grid, u.lds_bytes);
-    else rc = geo == 0 ? launch_wgrad_patch<2, 2, 0>(wp, grid, u.lds_bytes)
-            : geo == 1 ? launch_wgrad_patch<2, 2, 1>(wp, grid, u.lds_bytes)
-                       : launch_wgrad_patch<2, 2, 2>(wp, grid, u.lds_bytes);
-    if (rc) return rc;
+    if (int rc = dispatch_wgrad_patch(u)) return rc;
     *done = true;
     if (u.splits > 1) return wgrad_split_sum(u, partial, dw);
     return DOPT_HIP_OK;
@@ -2276,6 +2286,10 @@ int run_bwd_pair(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *d
     // launch shaped for the filter gradient's 768 threads cannot hold), with 128 x 32 filter-gradient tiles on
     // rows of 8 .. 64 pixels or on 4 x 4 images.
     const int combo = a.shape == 2 && b.tall && b.geo == 0 ? 0 : a.shape == 2 && b.tall && b.geo == 1 ? 1 : -1;
+    // (Other pairs of patch-kernel shapes as two launches out of one workspace request, so that the filter gradient's
+    // split sum could ride in the batch-norm gradient behind them as well, were measured: the layers concerned are
+    // followed by the multi-block batch norm, whose workgroups fill every CU, so the riders only start when those have
+    // finished - 20 us per layer instead of the 7.6 us of the separate sum.)
     if (combo < 0) return DOPT_HIP_OK;
     PatchConv &pc = a.pc;
     WgradPatch &wp = b.wp;
