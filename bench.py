@@ -174,8 +174,9 @@ def host_feed_leg(step, steps, warmup):
                     "upload on the second queue -> augmentation kernel (mirrored pad 4, random crop, horizontal flip) -> "
                     "training step; host fill and upload of batch k+1 overlap the device work of batch k",
             "pageable_args_ms_per_step": round(sec_plain * 1e3, 4),
-            "pageable_args_what": "the same step with pageable numpy arrays as plan arguments: the plan uploads them inside each "
-                                  "execution, as CUDAPlan.executeImpl does"}
+            "pageable_args_what": "the same step with pageable numpy arrays as plan arguments, as examples/cifar10.d calls "
+                                  "plan.execute: the plan stages them in page-locked memory of its own and uploads them on the "
+                                  "second queue beside the previous execution (CUDAPlan.executeImpl uploads with a blocking copy)"}
 
 
 def secondary(cfg, a):

@@ -2145,8 +2145,16 @@ void HIPPlan::cleanup()
     if (mClean) return;
     for (void *b : mOwned) dopt_hip_free(b);
     mOwned.clear();
-    for (auto &kv : mArgStaging) dopt_hip_free(kv.second);
-    mArgStaging.clear();
+    for (int t = 0; t < 2; t++) {
+        for (auto &kv : mHostArgs[t]) {
+            if (kv.second.dev) dopt_hip_free(kv.second.dev);
+            if (kv.second.pinned) dopt_hip_host_free(kv.second.pinned);
+        }
+        mHostArgs[t].clear();
+        if (mArgDone[t]) (void)hipEventDestroy(mArgDone[t]);
+        mArgDone[t] = nullptr;
+        mArgUsed[t] = false;
+    }
     for (auto &ev : mEvents) {
         (void)hipEventDestroy(ev.first);
         (void)hipEventDestroy(ev.second);
@@ -2168,6 +2176,7 @@ int HIPPlan::resolve(int nargs, const int *argOps, const void *const *argPtrs, c
     // variables: argument buffer if given, else the variable's own value (package.d:367-401)
     for (int id : mOps)
         if (mNeeded[id] && is_leaf(g.ops[id])) mResults[id] = g.ops[id].value;
+    int slot = -1;   // the pair of copies this execution's host arguments go through
     for (int a = 0; a < nargs; a++) {
         const int id = argOps[a];
         if (id < 0 || id >= (int)g.ops.size() || g.ops[id].opType != "variable")
@@ -2175,14 +2184,31 @@ int HIPPlan::resolve(int nargs, const int *argOps, const void *const *argPtrs, c
                         "All assignments in args must be for Operations with an opType of 'variable'");
         if (!mNeeded[id]) continue;
         if (argOnHost && argOnHost[a]) {
-            void *&stage = mArgStaging[id];
-            if (!stage)
-                if (int rc = dopt_hip_malloc(&stage, g.ops[id].bytes())) return rc;
-            if (int rc = dopt_hip_copy_h2d(stage, argPtrs[a], g.ops[id].bytes())) return rc;  // once per execution
-            mResults[id] = stage;
+            const size_t bytes = g.ops[id].bytes();
+            if (slot < 0) {
+                slot = mArgTurn;
+                mArgTurn ^= 1;
+                // the execution before last read this slot's device copies, and its uploads read the staging memory
+                if (mArgUsed[slot]) DOPT_HIP_CHECK(hipEventSynchronize(mArgDone[slot]));
+            }
+            HostArg &h = mHostArgs[slot][id];
+            if (!h.dev && bytes)
+                if (int rc = dopt_hip_malloc(&h.dev, bytes)) return rc;
+            if (!h.pinned && bytes)
+                if (int rc = dopt_hip_host_alloc(&h.pinned, bytes)) return rc;
+            if (bytes) {
+                if (!argPtrs[a]) return fail(DOPT_HIP_ERR_INVALID, "Failed to set contents of HIP buffer: null pointer");
+                std::memcpy(h.pinned, argPtrs[a], bytes);   // once per execution; the caller's array is free again
+                if (int rc = dopt_hip_copy_h2d_beside(h.dev, h.pinned, bytes)) return rc;
+            }
+            mResults[id] = h.dev;
         } else {
             mResults[id] = const_cast<void *>(argPtrs[a]);
         }
+    }
+    if (slot >= 0) {
+        if (int rc = dopt_hip_upload_join()) return rc;   // the kernels queued from here on wait for the uploads
+        mArgPending = slot;
     }
     for (int id : mOps)
         if (mNeeded[id] && mAliasSource[id] >= 0)
@@ -2317,7 +2343,15 @@ int HIPPlan::execute(int nargs, const int *argOps, const void *const *argPtrs, c
         }
     }
     if (int rc = resolve(nargs, argOps, argPtrs, argOnHost)) return rc;
-    return enqueue(nrets, rets);
+    const int rc = enqueue(nrets, rets);
+    if (mArgPending >= 0) {   // behind everything that reads this execution's host arguments
+        const int slot = mArgPending;
+        mArgPending = -1;
+        if (!mArgDone[slot]) DOPT_HIP_CHECK(hipEventCreateWithFlags(&mArgDone[slot], hipEventDisableTiming));
+        DOPT_HIP_CHECK(hipEventRecord(mArgDone[slot], lane_stream(0)));
+        mArgUsed[slot] = true;
+    }
+    return rc;
 }
 
 int HIPPlan::result(int op, void **ptr, size_t *bytes) const

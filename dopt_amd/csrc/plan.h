@@ -118,7 +118,16 @@ private:
     std::vector<Step> mSteps;                    // kernels to run, in order
     std::unordered_map<int, void *> mResults;    // op -> buffer
     std::vector<void *> mOwned;                  // buffers to free in cleanup
-    std::unordered_map<int, void *> mArgStaging; // variable op -> plan-owned device copy for host args
+    // Arguments that arrive as host arrays (cuda/package.d:367-401 uploads them with a blocking copy on every
+    // execution): two slots per argument, each a page-locked staging copy and a device copy, used in turn.  The host
+    // array is copied into the staging memory before the call returns (the caller may change it at once, as after the
+    // reference's blocking copy), the upload runs on the second queue beside the previous execution's kernels, and a
+    // slot is reused only after the execution that read it has finished (mArgDone).
+    struct HostArg { void *pinned = nullptr; void *dev = nullptr; };
+    std::unordered_map<int, HostArg> mHostArgs[2];
+    hipEvent_t mArgDone[2] = {nullptr, nullptr};
+    bool mArgUsed[2] = {false, false};
+    int mArgTurn = 0, mArgPending = -1;
     std::vector<int> mAliasSource;               // per op: the op whose buffer it aliases, or -1
     std::vector<size_t> mAliasOffset;            // per op: byte offset into the aliased buffer
     std::vector<char> mNeeded;                   // per op: its result is consumed
