@@ -13,7 +13,7 @@ from util import assert_close
 pytestmark = pytest.mark.gpu
 
 from dopt_amd import core
-from dopt_amd import capi, nnet, online, ops  # noqa: E402
+from dopt_amd import capi, configs, nnet, online, ops, workloads  # noqa: E402
 from dopt_amd.core import (evaluate, float32, float32Constant, grad, int32)  # noqa: E402
 
 
@@ -621,6 +621,32 @@ def test_output_only_products_of_a_plan_share_a_launch():
     plain = core.compile(outs, core.PLAN_VIEWS).execute({feats: X, labels: Y})
     for a, b in zip(plain, fused):
         assert np.array_equal(a, b) or (a.ndim == 1 and np.allclose(a, b, rtol=0, atol=2e-5))
+
+
+def test_host_arguments_are_consumed_when_the_call_returns():
+    """A plan's host arguments (cuda/package.d:367-401 uploads them with a blocking copy) are copied into the plan's
+    own page-locked staging memory before the call returns and uploaded beside the kernels still queued, two copies
+    taking turns: the caller may overwrite its array at once, and back-to-back executions with different arrays each
+    see their own data.  Parameters after six steps equal those of a run that waits after every step."""
+    def run(hurry):
+        step = configs.softmax_regression(flags=configs.REWRITES)
+        feats, labels = step.extra["feats"], step.extra["labels"]
+        r = np.random.default_rng(9)
+        for k in range(6):
+            x = r.random((100, 784)).astype(np.float32)
+            y = workloads.one_hot(r.integers(0, 10, 100), 10)
+            step.updater.step_async({feats: x, labels: y})
+            if hurry:
+                x[:] = np.nan            # the call has returned: the arrays are the caller's again
+                y[:] = np.nan
+            else:
+                ops.sync()
+        ops.sync()
+        return [p.value.copy() for p in step.params]
+
+    a, b = run(True), run(False)
+    for u, v in zip(a, b):
+        assert np.all(np.isfinite(u)) and np.array_equal(u, v)
 
 
 def test_weight_decay_terms_square_on_load():
