@@ -102,8 +102,11 @@ enum {
 int dopt_hip_plan_create(void *graph, int noutputs, const int *outputs, unsigned flags, void **plan);
 /* CUDAPlan.executeImpl (cuda/package.d:343-423).  args: variable ids with the buffer to use in
    place of the variable's own value for this execution (host pointers are uploaded once per
-   execution, device pointers are used directly).  rets[i] (device) receives output i with a
-   device-to-device copy; a NULL entry skips the copy. */
+   execution, device pointers are used directly).  A host array is copied into page-locked memory
+   of the plan's own before the call returns - the caller may change it at once, as after the
+   reference's blocking cuMemcpyHtoD - and uploaded beside the kernels still queued; the plan keeps
+   two such copies (and two device copies) per host argument and uses them in turn.  rets[i]
+   (device) receives output i with a device-to-device copy; a NULL entry skips the copy. */
 int dopt_hip_plan_execute(void *plan, int nargs, const int *arg_ops, const void *const *arg_ptrs,
                           const int *arg_on_host, int nrets, void *const *rets);
 /* The plan-owned result buffer of an operation (valid until the plan is destroyed). */
