@@ -442,6 +442,280 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 256) void conv_patch_k(Pat
     conv_patch_body<T, NPMAX, kCFull>(p, blockIdx.x);
 }
 
+// ------------------------------------------------------------------------------------ Winograd F(2x2, 3x3)
+//
+// The same layers (3x3, unit stride, pad 1, even image sides, whole 16-channel chunks) with 16 instead of 36
+// multiplications per 2x2 output pixels (Lavin & Gray): Y = At [ (G g Gt) . (Bt d B) ] A, the element-wise product summed
+// over the channels - sixteen independent [rows x channels] . [channels x tiles] products, one per position xi of the
+// 4x4 transformed tile.  The direct kernels run at three quarters of the fp32 matrix peak, so what is left to remove is
+// arithmetic.
+//
+// A workgroup owns 128 rows x 32 tiles (the 128 pixels of the direct kernel's column tile: whole image rows or whole
+// images, so the input under them is the same rectangle, staged by the same loader, position-major with its zero halo).
+// Per 16-channel chunk: the raw patch goes to LDS; all 512 threads transform it - thread (i, tile, four channels)
+// forms row i of Bt d B for its tile from eight 128-bit reads and writes the four transformed values, four channels
+// each, to V[xi][tile][16 channels]; then wavefront (wk, wi) multiplies rows 32 wk .. + 31 with the eight positions
+// xi = 8 wi .. 8 wi + 7: per position two 128-bit reads of V (this lane's tile, its eight channels) and two 128-bit
+// loads of the transformed filter U[chunk][xi][row][16 channels] straight into operand registers, three positions
+// ahead, feed eight matrix instructions into the position's own accumulator (128 accumulator registers per
+// wavefront, two wavefronts per SIMD).
+//
+// At the end a lane holds M[xi][row][tile] for its eight positions - two rows i of the 4x4 grid, complete in j - so it
+// applies A along j in registers (z[i][b]), combines its two rows into its share of the four outputs, and the
+// wavefronts of a pair add their shares through LDS: y[a][b] = (At z)[a][b].  Output, split reductions and bias are
+// those of the direct kernel.
+//
+// What bounds it: the transformed filter is 16/9 the size of the packed one and a workgroup streams 128 KB of it per
+// chunk for 2.1 MFLOP - the rate at which a CU's L1 fills from the L2 (about 35 GB/s) and the matrix cores are
+// about equally busy.  128 rows x 64 tiles would halve that traffic and need 256 accumulator registers per wavefront.
+constexpr int kWinoXchg = 4 * 64 * 64;   // floats of the exchange area: four wavefront pairs x 64 values per lane
+
+template <int NPMAX>
+__global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
+{
+    constexpr int BM = 128, BN = 128, THREADS = 512, CH = 16, LDP = 20;
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int raw_floats = ((p.psz + 1) * LDP + 3) / 4 * 4;   // one spare position absorbs the stores of unused slots
+    float *const raw = lds;
+    float *const V = lds + raw_floats;                          // [16][32][LDP]
+
+    unsigned L;
+    const unsigned tiles = (unsigned)(p.mtiles * p.ntiles);
+    if (!xcd_remap(blockIdx.x, tiles * (unsigned)p.splits, &L)) return;
+    const int split = (int)(L / tiles);
+    const unsigned tile = L - (unsigned)split * tiles;
+    const int mt = (int)(tile % (unsigned)p.mtiles), nt = (int)(tile / (unsigned)p.mtiles);
+    const int m0 = mt * BM, n0 = nt * BN;
+    const int cb = split * p.chunks_per_split;
+    const int ce = min(cb + p.chunks_per_split, p.chunks_total);
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int wk = w >> 1, wi = w & 1;
+    const int kh = lane >> 5, l32 = lane & 31;
+    const int OHW = p.OH * p.OW;
+    const int chan_stride = p.IH * p.IW;
+    const __amdgpu_buffer_rsrc_t rin = make_rsrc(p.in, p.in_bytes);
+    const __amdgpu_buffer_rsrc_t rwp = make_rsrc(p.wp, p.wp_bytes);
+
+    // ---- patch slots of this thread, as in conv_patch_body
+    const int n_first = n0 / OHW, oh0 = (n0 - n_first * OHW) / p.OW;
+    unsigned p_voff[NPMAX];
+    int p_lds[NPMAX];
+#pragma unroll
+    for (int i = 0; i < NPMAX; i++) {
+        const unsigned e = (unsigned)(i * THREADS + tid);
+        const unsigned c = fast_div(e, p.magic_psz);
+        const unsigned pos = e - c * (unsigned)p.psz;
+        const unsigned img = fast_div(pos, p.magic_img);
+        const unsigned rem = pos - img * (unsigned)(p.PR * p.PC);
+        const unsigned pr = fast_div(rem, p.magic_pc);
+        const unsigned pc = rem - pr * (unsigned)p.PC;
+        const int n = n_first + (int)img, ih = oh0 + (int)pr - p.PT, iw = (int)pc - p.PL;
+        const int bad = (CH - 1 - (int)c) | (p.N - 1 - n) | ih | (p.IH - 1 - ih) | iw | (p.IW - 1 - iw);
+        p_voff[i] = bad < 0 ? kOobOffset : (unsigned)(((n * p.Cin + (int)c) * p.IH + ih) * p.IW + iw) * 4u;
+        p_lds[i] = c < (unsigned)CH ? (int)(pos * LDP + c) * 4 : (p.psz * LDP + (tid & 15)) * 4;
+    }
+    float preg[NPMAX];
+    auto patch_load = [&](int i, int chunk) {
+        preg[i] = buffer_load_f32(rin, p_voff[i], (unsigned)(chunk * CH * chan_stride) * 4u);
+    };
+    auto patch_store = [&](int i) { *(float *)((char *)raw + p_lds[i]) = preg[i]; };
+
+    // ---- the transform item of this thread: row ti of Bt d B for tile tau, channels 4 cq .. 4 cq + 3
+    const int ti = tid >> 7, tau_t = (tid & 127) >> 2, cq = tid & 3;
+    const int tcn = p.OW >> 1, tpi = (p.rows >> 1) * tcn;          // tiles per row of tiles, per image of the pixel tile
+    int t_in, t_out;
+    {
+        const int img = tau_t / tpi, tl = tau_t - img * tpi, r2 = tl / tcn, c2 = tl - r2 * tcn;
+        t_in = ((img * p.PR + 2 * r2) * p.PC + 2 * c2) * LDP + cq * 4;
+        t_out = ((ti * 4) * 32 + tau_t) * LDP + cq * 4;
+    }
+    // Bt = [1 0 -1 0; 0 1 1 0; 0 -1 1 0; 0 1 0 -1]: row ti is d[ra] + sg * d[rb]
+    const int ra = ti == 0 ? 0 : ti == 2 ? 2 : 1, rb = ti == 0 ? 2 : ti == 1 ? 2 : ti == 2 ? 1 : 3;
+    const float sg = ti == 1 ? 1.0f : -1.0f;
+    const int t_a = t_in + ra * p.PC * LDP, t_b = t_in + rb * p.PC * LDP;
+    auto transform = [&]() {
+        float4 t[4];
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            const float4 da = *(const float4 *)(raw + t_a + b * LDP), db = *(const float4 *)(raw + t_b + b * LDP);
+            t[b] = make_float4(da.x + sg * db.x, da.y + sg * db.y, da.z + sg * db.z, da.w + sg * db.w);
+        }
+        auto sub = [](float4 x, float4 y) { return make_float4(x.x - y.x, x.y - y.y, x.z - y.z, x.w - y.w); };
+        auto add = [](float4 x, float4 y) { return make_float4(x.x + y.x, x.y + y.y, x.z + y.z, x.w + y.w); };
+        *(float4 *)(V + t_out) = sub(t[0], t[2]);
+        *(float4 *)(V + t_out + 32 * LDP) = add(t[1], t[2]);
+        *(float4 *)(V + t_out + 2 * 32 * LDP) = sub(t[2], t[1]);
+        *(float4 *)(V + t_out + 3 * 32 * LDP) = sub(t[1], t[3]);
+    };
+
+    // ---- transformed-filter fragments: this lane's 8 channels (kh * 8 ..) of row m0 + 32 wk + l32
+    const unsigned slab_bytes = (unsigned)p.Mp * CH * 4u;
+    const unsigned fa_voff = (unsigned)((m0 + wk * 32 + l32) * CH + kh * 8) * 4u;
+    float4 fa_ring[4][2];
+    auto fa_load = [&](auto slot_tag, int slab) {   // past the last slab the range check returns zeros
+        constexpr int slot = decltype(slot_tag)::value;
+        fa_ring[slot][0] = buffer_load_f32x4(rwp, fa_voff, (unsigned)slab * slab_bytes);
+        fa_ring[slot][1] = buffer_load_f32x4(rwp, fa_voff + 16u, (unsigned)slab * slab_bytes);
+    };
+    const int b_frag = (wi * 8 * 32 + l32) * LDP + kh * 8;   // position 8 wi, this lane's tile and channels
+
+    v16f acc[8];
+#pragma unroll
+    for (int x = 0; x < 8; x++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[x][v] = 0.0f;
+
+    // prologue: the first patch, transformed, and the first three filter fragments
+#pragma unroll
+    for (int i = 0; i < NPMAX; i++) patch_load(i, cb);
+    fa_load(StepTag<0>{}, cb * 16 + wi * 8);
+    fa_load(StepTag<1>{}, cb * 16 + wi * 8 + 1);
+    fa_load(StepTag<2>{}, cb * 16 + wi * 8 + 2);
+#pragma unroll
+    for (int i = 0; i < NPMAX; i++) patch_store(i);
+    __syncthreads();
+    transform();
+    __syncthreads();
+
+    constexpr int PER = (NPMAX + 3) / 4;
+    for (int chunk = cb; chunk < ce; ++chunk) {
+        static_for<0, 8>([&](auto xtag) {
+            constexpr int xl = decltype(xtag)::value;
+            const float4 fb0 = *(const float4 *)(V + b_frag + xl * 32 * LDP);
+            const float4 fb1 = *(const float4 *)(V + b_frag + xl * 32 * LDP + 4);
+            const float4 fa0 = fa_ring[xl % 4][0], fa1 = fa_ring[xl % 4][1];
+            // three positions ahead (the slot of the position before this one)
+            fa_load(StepTag<(xl + 3) % 4>{}, (xl + 3 < 8 ? chunk * 16 : (chunk + 1) * 16 - 8) + wi * 8 + xl + 3);
+            // the next chunk's patch: loads during positions 0..3, LDS stores during 4..7 (nobody reads `raw` now)
+            if constexpr (xl < 4) {
+#pragma unroll
+                for (int i = xl * PER; i < (xl + 1) * PER && i < NPMAX; i++) patch_load(i, chunk + 1);
+            } else {
+#pragma unroll
+                for (int i = (xl - 4) * PER; i < (xl - 3) * PER && i < NPMAX; i++) patch_store(i);
+            }
+            static_for<0, 8>([&](auto stag) {
+                constexpr int ks = decltype(stag)::value;
+                const float4 av = ks < 4 ? fa0 : fa1, bv = ks < 4 ? fb0 : fb1;
+                const float a = ks % 4 == 0 ? av.x : ks % 4 == 1 ? av.y : ks % 4 == 2 ? av.z : av.w;
+                const float b = ks % 4 == 0 ? bv.x : ks % 4 == 1 ? bv.y : ks % 4 == 2 ? bv.z : bv.w;
+                acc[xl] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[xl], 0, 0, 0);
+            });
+        });
+        __syncthreads();              // every wavefront is done with V; the next patch is in `raw`
+        if (chunk + 1 < ce) transform();
+        __syncthreads();
+    }
+
+    // ---- inverse transform.  This wavefront's rows of the 4x4 grid are i = 2 wi, 2 wi + 1; acc[4 il + j] = M[i][j].
+    // At = [1 1 1 0; 0 1 -1 -1]:  z[i][0] = m0 + m1 + m2, z[i][1] = m1 - m2 - m3, then the same over i.
+    float *const xchg = lds;          // [wk][value 0..63][lane]: the main loop's LDS is free now
+    float *outp = p.out + (size_t)split * p.out_elems;
+    const bool add_bias = p.bias != nullptr && p.splits == 1;
+    float part[16][4];                // per accumulator row v: this wavefront's share of y[a][b], index 2 a + b
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        const float za0 = (acc[0][v] + acc[1][v]) + acc[2][v], za1 = (acc[1][v] - acc[2][v]) - acc[3][v];
+        const float zb0 = (acc[4][v] + acc[5][v]) + acc[6][v], zb1 = (acc[5][v] - acc[6][v]) - acc[7][v];
+        if (wi == 0) {                // rows 0, 1: y[0] += z0 + z1, y[1] += z1
+            part[v][0] = za0 + zb0; part[v][1] = za1 + zb1; part[v][2] = zb0; part[v][3] = zb1;
+        } else {                      // rows 2, 3: y[0] += z2, y[1] += -z2 - z3
+            part[v][0] = za0; part[v][1] = za1; part[v][2] = -za0 - zb0; part[v][3] = -za1 - zb1;
+        }
+    }
+    if (wi == 1) {
+#pragma unroll
+        for (int v = 0; v < 16; v++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) xchg[(wk * 64 + v * 4 + q) * 64 + lane] = part[v][q];
+    }
+    __syncthreads();
+    if (wi == 1) return;
+    {
+        const int tau = l32, img = tau / tpi, tl = tau - img * tpi, r2 = tl / tcn, c2 = tl - r2 * tcn;
+        const int n = n_first + img;
+        if (n >= p.N) return;
+        float *base = outp + ((size_t)n * p.Mout * p.OH + (oh0 + 2 * r2)) * p.OW + 2 * c2;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int m = m0 + wk * 32 + acc_row(v, lane);
+            if (m >= p.Mout) continue;
+            const float bias = add_bias ? p.bias[m] : 0.0f;
+            float y[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                y[q] = part[v][q] + xchg[(wk * 64 + v * 4 + q) * 64 + lane];
+                if (add_bias) y[q] += bias;
+            }
+            float *o = base + (size_t)m * OHW;
+            *(float2 *)o = make_float2(y[0], y[1]);
+            *(float2 *)(o + p.OW) = make_float2(y[2], y[3]);
+        }
+    }
+}
+
+// The transformed filter of the Winograd kernel: U[((chunk*16 + xi)*Mp + m)*16 + j] = (G g Gt)[xi] for row m and
+// channel chunk*16 + j, where g is the filter as the kernel applies it to the patch: g[r][s] multiplies patch offset
+// (r, s), i.e. the stored taps read backwards when the operation is a true convolution (`flip`).  Staged like
+// pack_tile (16 rows of one chunk); G = [1 0 0; .5 .5 .5; .5 -.5 .5; 0 0 1].
+template <bool kBwd>
+__device__ __forceinline__ void wino_pack_tile(int M, int Cred, int Mp, size_t sm, size_t sc, int flip, const float *w, float *wp,
+                                               int chunk, int m0, float *stage)
+{
+    constexpr int PITCH = kBwd ? 148 : 145;
+    float v[9];
+#pragma unroll
+    for (int i = 0; i < 9; i++) {
+        const int f = i * 256 + threadIdx.x;
+        const int run = f / 144, r = f - run * 144;
+        bool ok;
+        size_t src;
+        if (!kBwd) {
+            ok = m0 + run < M && chunk * 16 + r / 9 < Cred;
+            src = (size_t)(m0 + run) * sm + (size_t)chunk * 16 * sc + r;
+        } else {
+            ok = chunk * 16 + run < Cred && m0 + r / 9 < M;
+            src = (size_t)(chunk * 16 + run) * sc + (size_t)m0 * sm + r;
+        }
+        v[i] = ok ? w[src] : 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < 9; i++) {
+        const int f = i * 256 + threadIdx.x;
+        stage[(f / 144) * PITCH + f % 144] = v[i];
+    }
+    __syncthreads();
+    // one (row, channel) pair per thread: 16 x 16 pairs, sixteen values each
+    {
+        const int j = threadIdx.x & 15, ml = threadIdx.x >> 4;
+        const float *s = !kBwd ? stage + ml * PITCH + j * 9 : stage + j * PITCH + ml * 9;
+        float g[3][3];
+#pragma unroll
+        for (int r = 0; r < 3; r++)
+#pragma unroll
+            for (int c = 0; c < 3; c++) g[r][c] = flip ? s[(2 - r) * 3 + (2 - c)] : s[r * 3 + c];
+        float h[4][3];   // G g
+#pragma unroll
+        for (int c = 0; c < 3; c++) {
+            h[0][c] = g[0][c];
+            h[1][c] = ((g[0][c] + g[1][c]) + g[2][c]) * 0.5f;
+            h[2][c] = ((g[0][c] - g[1][c]) + g[2][c]) * 0.5f;
+            h[3][c] = g[2][c];
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const float u0 = h[r][0], u1 = ((h[r][0] + h[r][1]) + h[r][2]) * 0.5f, u2 = ((h[r][0] - h[r][1]) + h[r][2]) * 0.5f,
+                        u3 = h[r][2];
+            float *dst = wp + (((size_t)chunk * 16 + r * 4) * Mp + m0 + ml) * 16 + j;
+            dst[0] = u0;
+            dst[(size_t)Mp * 16] = u1;
+            dst[(size_t)2 * Mp * 16] = u2;
+            dst[(size_t)3 * Mp * 16] = u3;
+        }
+    }
+}
+
 // Packed filter of the patch kernel: wp[((chunk*9 + tap)*Mp + m)*16 + j] = w[m*sm + (chunk*16+j)*sc + tap]
 // (zero where m >= M or the channel is past the end).  Forward: m = output channel k (sm = C*9,
 // sc = 9); backward-data: m = input channel c (sm = 9, sc = C*9), reduction over k.
@@ -493,11 +767,12 @@ __device__ __forceinline__ void pack_tile(int M, int Cred, int Mp, size_t sm, si
 }
 
 template <bool kBwd>
-__global__ __launch_bounds__(256) void pack_patch_k(int M, int Cred, int Mp, size_t sm, size_t sc, const float *w,
-                                                     float *wp)
+__global__ __launch_bounds__(256) void pack_patch_k(int M, int Cred, int Mp, size_t sm, size_t sc, int wino, int flip,
+                                                     const float *w, float *wp)
 {
     __shared__ float stage[16 * 148];
-    pack_tile<kBwd>(M, Cred, Mp, sm, sc, w, wp, blockIdx.y, blockIdx.x * 16, stage);
+    if (wino) wino_pack_tile<kBwd>(M, Cred, Mp, sm, sc, flip, w, wp, blockIdx.y, blockIdx.x * 16, stage);
+    else pack_tile<kBwd>(M, Cred, Mp, sm, sc, w, wp, blockIdx.y, blockIdx.x * 16, stage);
 }
 
 // The filters of many layers in one launch (a training step packs each filter twice, once per
@@ -507,6 +782,7 @@ struct PackJob {
     const float *w;
     float *wp;
     int M, Cred, Mp, bwd;
+    int wino, flip;                  // wino: the Winograd kernel's transformed filter (16 positions per chunk instead of 9 taps)
     unsigned sm, sc;
     unsigned first_block, mblocks;   // blocks [first_block, next job's first_block): (chunk, row block) pairs
 };
@@ -523,7 +799,10 @@ __global__ __launch_bounds__(256) void pack_batch_k(PackBatch b)
     const PackJob &q = b.job[j];
     const unsigned local = blockIdx.x - q.first_block;
     const int chunk = (int)(local / q.mblocks), m0 = (int)(local % q.mblocks) * 16;
-    if (q.bwd) pack_tile<true>(q.M, q.Cred, q.Mp, q.sm, q.sc, q.w, q.wp, chunk, m0, stage);
+    if (q.wino) {
+        if (q.bwd) wino_pack_tile<true>(q.M, q.Cred, q.Mp, q.sm, q.sc, q.flip, q.w, q.wp, chunk, m0, stage);
+        else wino_pack_tile<false>(q.M, q.Cred, q.Mp, q.sm, q.sc, q.flip, q.w, q.wp, chunk, m0, stage);
+    } else if (q.bwd) pack_tile<true>(q.M, q.Cred, q.Mp, q.sm, q.sc, q.w, q.wp, chunk, m0, stage);
     else pack_tile<false>(q.M, q.Cred, q.Mp, q.sm, q.sc, q.w, q.wp, chunk, m0, stage);
 }
 
@@ -1219,24 +1498,35 @@ int launch_patch(const PatchConv &pc, bool c_full, dim3 grid, size_t lds_bytes)
 struct PatchSetup {
     bool ok;
     PatchConv pc;
-    int shape;            // 0 wide, 1 square, 2 deep, 3 tall
+    int shape;            // 0 wide, 1 square, 2 deep, 3 tall, 4 Winograd (128 rows x 32 tiles of 2x2 pixels)
     int BM, BN, blocks_wanted, tiles;
     size_t lds_bytes, wp_elems;
 };
 
 template <bool kBwd>
-PatchSetup patch_setup_as(const dopt_hip_conv_desc *d, size_t P, size_t Q, bool allow_tall);
+PatchSetup patch_setup_as(const dopt_hip_conv_desc *d, size_t P, size_t Q, bool allow_tall, bool wino = false);
+
+// DOPT_HIP_NO_WINO=1 keeps the Winograd kernel out (for A/B measurements); read once.
+bool no_wino()
+{
+    static const bool off = std::getenv("DOPT_HIP_NO_WINO") != nullptr;
+    return off;
+}
 
 // (a layer the 160-row tiles do not take - its pixel tile does not fit their patch - is tried with the other heights)
 template <bool kBwd>
 PatchSetup patch_setup(const dopt_hip_conv_desc *d, size_t P, size_t Q)
 {
+    if (!no_wino()) {
+        const PatchSetup v = patch_setup_as<kBwd>(d, P, Q, false, true);
+        if (v.ok) return v;
+    }
     const PatchSetup u = patch_setup_as<kBwd>(d, P, Q, true);
     return u.ok ? u : patch_setup_as<kBwd>(d, P, Q, false);
 }
 
 template <bool kBwd>
-PatchSetup patch_setup_as(const dopt_hip_conv_desc *d, size_t P, size_t Q, bool allow_tall)
+PatchSetup patch_setup_as(const dopt_hip_conv_desc *d, size_t P, size_t Q, bool allow_tall, bool wino)
 {
     PatchSetup u{};
     if (d->R != 3 || d->S != 3 || d->strideH != 1 || d->strideW != 1 || d->padH > 2 || d->padW > 2) return u;
@@ -1260,7 +1550,13 @@ PatchSetup patch_setup_as(const dopt_hip_conv_desc *d, size_t P, size_t Q, bool 
     const int up64 = (pc.Mout + 63) / 64 * 64, up128 = (pc.Mout + 127) / 128 * 128, up160 = (pc.Mout + 159) / 160 * 160;
     // (only where they still give every compute unit a tile: 480 channels on 8 x 8 images are 192 such tiles, and ran slower)
     const long tall_tiles = (long)(up160 / 160) * ((pc.ncols + 127) / 128);
-    if (allow_tall && pc.Mout > 64 && up160 <= up64 && up160 <= up128 && tall_tiles >= num_cus() &&
+    if (wino) {
+        // whole 16-channel chunks of a deep reduction, whole 128-row tiles, pad 1, 2 x 2 tiles
+        if (d->padH != 1 || d->padW != 1 || pc.Cin % 16 != 0 || pc.Cin < 64 || pc.Mout % 128 != 0 || pc.OH % 2 != 0 ||
+            pc.OW % 2 != 0 || pc.OH < 4 || pc.OW < 4)
+            return u;
+        u.shape = 4; u.BM = 128; u.BN = 128; u.blocks_wanted = num_cus(); npmax = 16; threads = 512;
+    } else if (allow_tall && pc.Mout > 64 && up160 <= up64 && up160 <= up128 && tall_tiles >= num_cus() &&
         !no_tall_tiles()) {
         u.shape = 3; u.BM = 160; u.BN = 128; u.blocks_wanted = num_cus(); npmax = 16; threads = 256;
     } else if (pc.Mout <= 64 || up64 < up128) {
@@ -1286,6 +1582,11 @@ PatchSetup patch_setup_as(const dopt_hip_conv_desc *d, size_t P, size_t Q, bool 
     pc.psz = pc.nimg * pc.PR * pc.PC;
     if ((size_t)pc.psz * 16 > (size_t)npmax * threads) return u;
     u.lds_bytes = (size_t)2 * (pc.psz + 1) * 20 * sizeof(float);
+    if (wino) {
+        if (pc.rows % 2 != 0) return u;   // a pixel tile is whole 2 x 2 tiles
+        const size_t floats = (size_t)(((pc.psz + 1) * 20 + 3) / 4 * 4) + 16 * 32 * 20;
+        u.lds_bytes = (floats > (size_t)kWinoXchg ? floats : (size_t)kWinoXchg) * sizeof(float);
+    }
     if (u.lds_bytes > 160 * 1024) return u;
     pc.magic_psz = div_magic((unsigned)pc.psz);
     pc.magic_img = div_magic((unsigned)(pc.PR * pc.PC));
@@ -1296,7 +1597,7 @@ PatchSetup patch_setup_as(const dopt_hip_conv_desc *d, size_t P, size_t Q, bool 
     pc.chunks_total = (pc.Cin + 15) / 16;
     pc.out_elems = (size_t)pc.ncols * pc.Mout;
     u.tiles = pc.mtiles * pc.ntiles;
-    u.wp_elems = (size_t)pc.chunks_total * 9 * pc.Mp * 16;
+    u.wp_elems = (size_t)pc.chunks_total * (wino ? 16 : 9) * pc.Mp * 16;
     u.ok = true;
     return u;
 }
@@ -1308,6 +1609,7 @@ PackJob pack_job(const dopt_hip_conv_desc *d, const PatchSetup &u, const float *
     PackJob j{};
     j.w = w; j.wp = wp;
     j.M = u.pc.Mout; j.Cred = u.pc.Cin; j.Mp = u.pc.Mp; j.bwd = kBwd;
+    j.wino = u.shape == 4; j.flip = u.pc.flip;
     j.sm = kBwd ? 9u : C9;
     j.sc = kBwd ? C9 : 9u;
     j.mblocks = (unsigned)(u.pc.Mp / 16);
@@ -1388,6 +1690,16 @@ int dispatch_patch(const PatchSetup &u, int splits)
     if (u.shape == 0) return launch_patch<GatherWide, 24>(pc, c_full, grid, u.lds_bytes);
     if (u.shape == 1) return launch_patch<GatherSquare, 16>(pc, c_full, grid, u.lds_bytes);
     if (u.shape == 3) return launch_patch<GatherTall, 16>(pc, c_full, grid, u.lds_bytes);
+    if (u.shape == 4) {
+        static bool raised = false;
+        if (!raised) {
+            DOPT_HIP_CHECK(hipFuncSetAttribute((const void *)conv_wino_k<16>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+            raised = true;
+        }
+        hipLaunchKernelGGL(conv_wino_k<16>, grid, dim3(512), u.lds_bytes, stream(), pc);
+        DOPT_LAUNCH_CHECK();
+        return DOPT_HIP_OK;
+    }
     return launch_patch<GatherDeep, 16>(pc, c_full, grid, u.lds_bytes);
 }
 
@@ -1411,9 +1723,9 @@ int run_patch(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *in, 
         const PackJob j = pack_job<kBwd>(d, u, w, (float *)ws);
         const dim3 pgrid(j.mblocks, (unsigned)pc.chunks_total);
         if (!kBwd) hipLaunchKernelGGL(pack_patch_k<false>, pgrid, dim3(256), 0, stream(), j.M, j.Cred, j.Mp, (size_t)j.sm,
-                                      (size_t)j.sc, w, j.wp);
+                                      (size_t)j.sc, j.wino, j.flip, w, j.wp);
         else hipLaunchKernelGGL(pack_patch_k<true>, pgrid, dim3(256), 0, stream(), j.M, j.Cred, j.Mp, (size_t)j.sm,
-                                (size_t)j.sc, w, j.wp);
+                                (size_t)j.sc, j.wino, j.flip, w, j.wp);
         DOPT_LAUNCH_CHECK();
         prepacked = j.wp;
     }
@@ -2285,6 +2597,7 @@ int run_bwd_pair(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *d
     // (the 64 x 256 tiles of layers with up to 64 input channels run two 256-thread workgroups per CU, which a
     // launch shaped for the filter gradient's 768 threads cannot hold), with 128 x 32 filter-gradient tiles on
     // rows of 8 .. 64 pixels or on 4 x 4 images.
+    // (a layer the Winograd kernel takes has its filter packed for that kernel: shape 4, not a pair)
     const int combo = a.shape == 2 && b.tall && b.geo == 0 ? 0 : a.shape == 2 && b.tall && b.geo == 1 ? 1 : -1;
     // (Other pairs of patch-kernel shapes as two launches out of one workspace request, so that the filter gradient's
     // split sum could ride in the batch-norm gradient behind them as well, were measured: the layers concerned are

@@ -442,9 +442,11 @@ def test_packed_filter_entry_points_match_the_unpacked_ones():
         capi.check(lib.dopt_hip_conv_fwd_bias_packed(C.byref(d5), x.ptr, scratch.ptr, None, y.ptr))
 
 
-@pytest.mark.parametrize("xs,k", [((8, 256, 4, 4), 512),     # one launch: 4 x 4 images, both reductions split
-                                  ((16, 128, 8, 8), 256),    # one launch: rows of 8 pixels
-                                  ((128, 128, 16, 16), 128), # one launch at a benchmark shape
+@pytest.mark.parametrize("xs,k", [((8, 256, 4, 4), 512),     # Winograd backward-data + filter gradient: 4 x 4 images, reductions split
+                                  ((16, 128, 8, 8), 256),    # the same on rows of 8 pixels
+                                  ((128, 128, 16, 16), 128), # ... at a benchmark shape
+                                  ((8, 250, 4, 4), 512),     # one launch: 4 x 4 images, both reductions split
+                                  ((16, 250, 8, 8), 256),    # one launch: rows of 8 pixels
                                   ((4, 200, 16, 16), 240),   # one launch, ragged: partial tiles in both products
                                   ((4, 160, 16, 16), 128),   # 160 input channels run as 64-row tiles: two launches
                                   ((2, 64, 32, 32), 64),     # 64-row tiles: the two kernels one after the other
@@ -483,8 +485,12 @@ def test_backward_data_and_filter_gradient_as_one_call(xs, k):
     capi.check(lib.dopt_hip_conv_pair_probe_read(C.byref(n), C.byref(us), C.byref(fl), C.byref(by)))
     capi.check(lib.dopt_hip_conv_pair_probe(0))
     up = lambda v, m: (v + m - 1) // m * m
-    # 128-row tiles in both products (wherever 64-row tiles would not pad less) on images of 4 x 4 pixels and more
-    one_launch = Cin > 64 and up(Cin, 128) <= up(Cin, 64) and k >= 128 and up(k, 128) <= up(k, 64) and W >= 4
+    # 128-row tiles in both products (wherever 64-row tiles would not pad less) on images of 4 x 4 pixels and more -
+    # unless backward-data is a Winograd layer (whole 128-row tiles of input channels, 64 and more output channels,
+    # even sides of at least 4): its filter is packed for that kernel and the two products are two launches
+    winograd = Cin % 128 == 0 and k % 16 == 0 and k >= 64 and H % 2 == 0 and W % 2 == 0 and H >= 4 and W >= 4 and \
+        (128 % W == 0) and ((128 // W) % 2 == 0)
+    one_launch = Cin > 64 and up(Cin, 128) <= up(Cin, 64) and k >= 128 and up(k, 128) <= up(k, 64) and W >= 4 and not winograd
     assert n.value == (1 if one_launch else 0)
     if one_launch:
         assert us.value > 0 and fl.value == 2 * 2.0 * N * H * W * k * Cin * 9
@@ -494,7 +500,7 @@ def test_backward_data_and_filter_gradient_as_one_call(xs, k):
     o = capi.SplitSum()
     capi.check(lib.dopt_hip_conv_bwd_pair_packed_open(C.byref(d), dy.ptr, packed.ptr, x.ptr, dx.ptr, dw.ptr, C.byref(o), None))
     assert o.value == dx.ptr
-    if xs == (8, 256, 4, 4):
+    if xs in ((8, 256, 4, 4), (8, 250, 4, 4)):
         assert o.splits > 1
     if o.splits:
         capi.check(lib.dopt_hip_split_sum_close(C.byref(o)))
@@ -504,7 +510,7 @@ def test_backward_data_and_filter_gradient_as_one_call(xs, k):
     o, ow = capi.SplitSum(), capi.SplitSum()
     capi.check(lib.dopt_hip_conv_bwd_pair_packed_open(C.byref(d), dy.ptr, packed.ptr, x.ptr, dx.ptr, dw.ptr, C.byref(o), C.byref(ow)))
     assert ow.value == dw.ptr and (ow.splits == 0 or (one_launch and ow.splits > 1 and ow.lanes in (4, 16)))
-    if xs == (128, 128, 16, 16):
+    if xs == (16, 250, 8, 8):
         assert ow.splits > 1
     if ow.splits:
         # nothing else may take the workspace while the copies lie in it

@@ -391,6 +391,15 @@ CONV_CASES = [  # N, C, H, W, K, R, S, pad, stride
     (2, 128, 8, 8, 64, 3, 3, (1, 1), (2, 2)),
     (16, 128, 64, 64, 16, 3, 3, (1, 1), (2, 2)),
     (3, 130, 9, 7, 24, 3, 3, (1, 1), (2, 2)),
+    # Winograd F(2x2, 3x3): 128-row tiles of 32 2x2-pixel tiles - half an image, two images, eight images per tile;
+    # a last tile with images missing; both directions (forward needs 128 k output channels, backward-data 128 k input
+    # channels); a reduction split over workgroups
+    (8, 128, 16, 16, 128, 3, 3, (1, 1), (1, 1)),
+    (8, 128, 8, 8, 256, 3, 3, (1, 1), (1, 1)),
+    (3, 64, 8, 8, 128, 3, 3, (1, 1), (1, 1)),
+    (21, 256, 4, 4, 128, 3, 3, (1, 1), (1, 1)),
+    (4, 128, 32, 32, 128, 3, 3, (1, 1), (1, 1)),
+    (2, 80, 8, 12, 128, 3, 3, (1, 1), (1, 1)),     # 12 columns: no whole tile rows in 128 pixels, the direct kernels
     (2, 7, 11, 13, 9, 5, 5, (2, 2), (3, 3)),      # nine classes with work in one launch
     (1, 4, 9, 9, 5, 5, 5, (2, 2), (4, 4)),        # sixteen classes: one after the other
 ]
