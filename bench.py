@@ -287,7 +287,7 @@ def main():
         before = tstep.updater.plan.profile()
         nsteps = max(3, min(a.steps, 10))
         lib = capi.load()
-        capi.check(lib.dopt_hip_conv_pair_probe(1))      # events around every conv_bwd_pair_k launch, on its own stream
+        capi.check(lib.dopt_hip_conv_pair_probe(2))      # events around every conv_wino_k launch, on its own stream
         tstep.run(nsteps)
         ops.sync()
         import ctypes as C
@@ -312,35 +312,39 @@ def main():
                         return int(line.split()[-1])
             return None
 
-        # The dominant kernel, by its share of the step: conv_bwd_pair_k, the backward-data convolution and the filter
-        # gradient of one layer in one launch (128 x 128 backward-data tiles first, 128 x 32 x 9 filter-gradient tiles
-        # behind them on the same compute units): layers 4-10 of the 13, 7 launches per step.  Timed by events recorded
-        # around each launch inside the library, on the stream the kernel runs on (the step around it also runs the split
-        # sum of the filter gradient, which is not part of this figure).  FLOPs are the executed ones: both products
-        # multiply every tap of every pixel, zero padding included.
+        # The dominant kernel, by its share of the step: conv_wino_k<16, 4, 1>, the Winograd F(2x2, 3x3) convolution on
+        # 128-row tiles that runs the forward pass of layers 3-10 and the backward-data pass of layers 4-10 (15 launches
+        # per step; the 64-row instantiation of layers 2-3 is not part of this figure).  Timed by events
+        # recorded around each launch inside the library, on the stream the kernel runs on (its steps may also run a
+        # split sum, which is not part of this figure).  `achieved` counts the layer's FLOPs by the direct algorithm,
+        # 2*N*K*C*R*S*P*Q - the algorithmic work of the operation, as the other figures of this file do; the kernel
+        # executes 16/36 of them on the matrix cores (`executed_*`), so `frac` above 1 is the algorithm's gain, not a
+        # measurement error.
         launches = pl.value / nsteps if nsteps else 0
         tflops = pfl.value / (pus.value * 1e-6) / 1e12 if pus.value else 0.0
         result["roofline"] = {
-            "kernel": "conv_bwd_pair_k<Tile<128,128,2,4>,16,4,1,*>: backward-data convolution (3x3 implicit GEMM on the packed "
-                      "filter) and filter gradient of one layer in one launch, layers 4-10 of the 13 (both template "
-                      "instances: rows of 8-16 pixels and 4x4 images); the other convolution kernels are listed under `kernels`",
+            "kernel": "conv_wino_k<16, 4, 1>: Winograd F(2x2, 3x3) convolution on the transformed filter, 128 rows x 32 tiles of 2x2 "
+                      "pixels per workgroup: forward of layers 3-10 and backward-data of layers 4-10 of the 13; the other "
+                      "convolution kernels are listed under `kernels`",
             "bound": "mfma", "achieved": round(tflops, 2), "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(tflops / MFMA_FP32_PEAK_TFLOPS, 4), "traffic": profile_line("traffic_bytes_per_launch conv_bwd_pair_k"),
+            "frac": round(tflops / MFMA_FP32_PEAK_TFLOPS, 4),
+            "executed_achieved": round(tflops * 16.0 / 36.0, 2), "executed_frac": round(tflops * 16.0 / 36.0 / MFMA_FP32_PEAK_TFLOPS, 4),
+            "traffic": profile_line("traffic_bytes_per_launch conv_wino_k"),
             "traffic_source": "profiles/conv_kernels_vgg16_b128_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of "
                               "the same %d launches per step; taken from that file, not measured in this run)" % round(launches),
             "algorithmic_bytes_per_launch": int(pby.value / pl.value) if pl.value else None,
-            "algorithmic_bytes_convention": "dy, x, dx, the filter and its gradient once each",
+            "algorithmic_bytes_convention": "input, output and the filter once each",
             "launches_per_step": int(round(launches)),
             "flops_per_launch": round(pfl.value / pl.value, 1) if pl.value else None,
-            "flops_convention": "2 x 2*N*K*C*R*S*P*Q per launch (backward-data + filter gradient) = what the kernel executes "
-                                "(it multiplies the taps that fall on zero padding too)",
+            "flops_convention": "2*N*K*C*R*S*P*Q per launch, the direct algorithm's count; the kernel's matrix instructions "
+                                "execute 16/36 of it (sixteen products per 2x2 outputs instead of thirty-six)",
             "avg_launch_us": round(pus.value / pl.value, 2) if pl.value else None,
             "timing": "HIP events around each launch on the library's stream, %d steps" % nsteps,
         }
 
-        # conv_patch_k with 128 x 128 tiles on its own: the forward convolutions of layers 3-10 (8 launches per step).
-        # Their steps hold nothing else (filters are packed by a step of their own; where a reduction is split the
-        # partial sums are added by the batch norm behind it).
+        # The forward convolutions of layers 3-10 on their own (8 launches per step, the Winograd kernel): their steps
+        # hold nothing else (filters are transformed by a step of their own; where a reduction is split the partial sums
+        # are added by the batch norm behind it).
         flops = us = n128 = bytes_alg = 0
         for i, (c, k, h) in enumerate(configs.VGG_CONVS):
             fwd_keys = [n for n in ("convolution+addBias", "convolution") if "%s@%dx%dx%dx%d" % (n, BATCH, k, h, h) in per_shape]
@@ -356,12 +360,12 @@ def main():
                     "convolutionFeaturesGrad+convolutionFiltersGrad", "filterPack")
         allconv_us = sum(per_op[k][0] for k in conv_ops if k in per_op)
         result["kernels"] = {
-            "conv_patch_k<Tile<128,128,2,4>,16,true> (forward convolutions of layers 3-10)": {
+            "forward convolutions of layers 3-10 (conv_wino_k; FLOPs by the direct algorithm's count)": {
                 "achieved_TFLOPs": round(flops / (us * 1e-6) / 1e12, 2) if us else None,
                 "frac_of_mfma_peak": round(flops / (us * 1e-6) / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4) if us else None,
                 "launches_per_step": n128, "avg_launch_us": round(us / n128, 2) if n128 else None,
                 "algorithmic_bytes_per_launch": int(bytes_alg / n128) if n128 else None,
-                "traffic": profile_line("traffic_bytes_per_launch conv_patch_k_128x128")},
+                "traffic": profile_line("traffic_bytes_per_launch conv_wino_k")},
             "all 38 convolution operations of the step incl. filter packing and split sums (2x2-image layers counted at the "
             "conventional 9-tap FLOPs although their dense route executes 4/9 of them)": {
                 "achieved_TFLOPs": round((2 * fwd + bwd_data) / (allconv_us * 1e-6) / 1e12, 2),

@@ -470,14 +470,18 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 256) void conv_patch_k(Pat
 // about equally busy.  128 rows x 64 tiles would halve that traffic and need 256 accumulator registers per wavefront.
 constexpr int kWinoXchg = 4 * 64 * 64;   // floats of the exchange area: four wavefront pairs x 64 values per lane
 
-template <int NPMAX>
+// WK x TH: the eight wavefronts are WK groups of 32 rows x TH groups of 32 tiles x the two halves of the 16 positions:
+// 4 x 1 (128 rows x 32 tiles = 128 pixels) for layers with whole 128-row tiles, 2 x 2 (64 rows x 64 tiles = 256 pixels)
+// for 64-row layers.
+template <int NPMAX, int WK, int TH>
 __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
 {
-    constexpr int BM = 128, BN = 128, THREADS = 512, CH = 16, LDP = 20;
+    static_assert(WK * TH == 4, "eight wavefronts");
+    constexpr int BM = 32 * WK, BN = 128 * TH, TT = 32 * TH, THREADS = 512, CH = 16, LDP = 20;
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int raw_floats = ((p.psz + 1) * LDP + 3) / 4 * 4;   // one spare position absorbs the stores of unused slots
     float *const raw = lds;
-    float *const V = lds + raw_floats;                          // [16][32][LDP]
+    float *const V = lds + raw_floats;                          // [16][TT][LDP]
 
     unsigned L;
     const unsigned tiles = (unsigned)(p.mtiles * p.ntiles);
@@ -490,7 +494,7 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
     const int ce = min(cb + p.chunks_per_split, p.chunks_total);
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-    const int wk = w >> 1, wi = w & 1;
+    const int wi = w & 1, wk = (w >> 1) % WK, th = (w >> 1) / WK;
     const int kh = lane >> 5, l32 = lane & 31;
     const int OHW = p.OH * p.OW;
     const int chan_stride = p.IH * p.IW;
@@ -521,32 +525,38 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
     };
     auto patch_store = [&](int i) { *(float *)((char *)raw + p_lds[i]) = preg[i]; };
 
-    // ---- the transform item of this thread: row ti of Bt d B for tile tau, channels 4 cq .. 4 cq + 3
-    const int ti = tid >> 7, tau_t = (tid & 127) >> 2, cq = tid & 3;
+    // ---- the transform items of this thread (TH of them): row ti of Bt d B for tile tau, channels 4 cq .. 4 cq + 3
     const int tcn = p.OW >> 1, tpi = (p.rows >> 1) * tcn;          // tiles per row of tiles, per image of the pixel tile
-    int t_in, t_out;
-    {
-        const int img = tau_t / tpi, tl = tau_t - img * tpi, r2 = tl / tcn, c2 = tl - r2 * tcn;
-        t_in = ((img * p.PR + 2 * r2) * p.PC + 2 * c2) * LDP + cq * 4;
-        t_out = ((ti * 4) * 32 + tau_t) * LDP + cq * 4;
-    }
     // Bt = [1 0 -1 0; 0 1 1 0; 0 -1 1 0; 0 1 0 -1]: row ti is d[ra] + sg * d[rb]
-    const int ra = ti == 0 ? 0 : ti == 2 ? 2 : 1, rb = ti == 0 ? 2 : ti == 1 ? 2 : ti == 2 ? 1 : 3;
-    const float sg = ti == 1 ? 1.0f : -1.0f;
-    const int t_a = t_in + ra * p.PC * LDP, t_b = t_in + rb * p.PC * LDP;
-    auto transform = [&]() {
-        float4 t[4];
+    int t_a[TH], t_b[TH], t_out[TH];
+    float sg[TH];
 #pragma unroll
-        for (int b = 0; b < 4; b++) {
-            const float4 da = *(const float4 *)(raw + t_a + b * LDP), db = *(const float4 *)(raw + t_b + b * LDP);
-            t[b] = make_float4(da.x + sg * db.x, da.y + sg * db.y, da.z + sg * db.z, da.w + sg * db.w);
-        }
+    for (int u = 0; u < TH; u++) {
+        const int item = u * THREADS + tid, ti = item / (TT * 4), tau_t = (item % (TT * 4)) >> 2, cq = item & 3;
+        const int img = tau_t / tpi, tl = tau_t - img * tpi, r2 = tl / tcn, c2 = tl - r2 * tcn;
+        const int t_in = ((img * p.PR + 2 * r2) * p.PC + 2 * c2) * LDP + cq * 4;
+        const int ra = ti == 0 ? 0 : ti == 2 ? 2 : 1, rb = ti == 0 ? 2 : ti == 1 ? 2 : ti == 2 ? 1 : 3;
+        t_a[u] = t_in + ra * p.PC * LDP;
+        t_b[u] = t_in + rb * p.PC * LDP;
+        t_out[u] = ((ti * 4) * TT + tau_t) * LDP + cq * 4;
+        sg[u] = ti == 1 ? 1.0f : -1.0f;
+    }
+    auto transform = [&]() {
         auto sub = [](float4 x, float4 y) { return make_float4(x.x - y.x, x.y - y.y, x.z - y.z, x.w - y.w); };
         auto add = [](float4 x, float4 y) { return make_float4(x.x + y.x, x.y + y.y, x.z + y.z, x.w + y.w); };
-        *(float4 *)(V + t_out) = sub(t[0], t[2]);
-        *(float4 *)(V + t_out + 32 * LDP) = add(t[1], t[2]);
-        *(float4 *)(V + t_out + 2 * 32 * LDP) = sub(t[2], t[1]);
-        *(float4 *)(V + t_out + 3 * 32 * LDP) = sub(t[1], t[3]);
+#pragma unroll
+        for (int u = 0; u < TH; u++) {
+            float4 t[4];
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const float4 da = *(const float4 *)(raw + t_a[u] + b * LDP), db = *(const float4 *)(raw + t_b[u] + b * LDP);
+                t[b] = make_float4(da.x + sg[u] * db.x, da.y + sg[u] * db.y, da.z + sg[u] * db.z, da.w + sg[u] * db.w);
+            }
+            *(float4 *)(V + t_out[u]) = sub(t[0], t[2]);
+            *(float4 *)(V + t_out[u] + TT * LDP) = add(t[1], t[2]);
+            *(float4 *)(V + t_out[u] + 2 * TT * LDP) = sub(t[2], t[1]);
+            *(float4 *)(V + t_out[u] + 3 * TT * LDP) = sub(t[1], t[3]);
+        }
     };
 
     // ---- transformed-filter fragments: this lane's 8 channels (kh * 8 ..) of row m0 + 32 wk + l32
@@ -558,7 +568,7 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
         fa_ring[slot][0] = buffer_load_f32x4(rwp, fa_voff, (unsigned)slab * slab_bytes);
         fa_ring[slot][1] = buffer_load_f32x4(rwp, fa_voff + 16u, (unsigned)slab * slab_bytes);
     };
-    const int b_frag = (wi * 8 * 32 + l32) * LDP + kh * 8;   // position 8 wi, this lane's tile and channels
+    const int b_frag = (wi * 8 * TT + th * 32 + l32) * LDP + kh * 8;   // position 8 wi, this lane's tile and channels
 
     v16f acc[8];
 #pragma unroll
@@ -582,8 +592,8 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
     for (int chunk = cb; chunk < ce; ++chunk) {
         static_for<0, 8>([&](auto xtag) {
             constexpr int xl = decltype(xtag)::value;
-            const float4 fb0 = *(const float4 *)(V + b_frag + xl * 32 * LDP);
-            const float4 fb1 = *(const float4 *)(V + b_frag + xl * 32 * LDP + 4);
+            const float4 fb0 = *(const float4 *)(V + b_frag + xl * TT * LDP);
+            const float4 fb1 = *(const float4 *)(V + b_frag + xl * TT * LDP + 4);
             const float4 fa0 = fa_ring[xl % 4][0], fa1 = fa_ring[xl % 4][1];
             // three positions ahead (the slot of the position before this one)
             fa_load(StepTag<(xl + 3) % 4>{}, (xl + 3 < 8 ? chunk * 16 : (chunk + 1) * 16 - 8) + wi * 8 + xl + 3);
@@ -628,12 +638,12 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
 #pragma unroll
         for (int v = 0; v < 16; v++)
 #pragma unroll
-            for (int q = 0; q < 4; q++) xchg[(wk * 64 + v * 4 + q) * 64 + lane] = part[v][q];
+            for (int q = 0; q < 4; q++) xchg[((w >> 1) * 64 + v * 4 + q) * 64 + lane] = part[v][q];
     }
     __syncthreads();
     if (wi == 1) return;
     {
-        const int tau = l32, img = tau / tpi, tl = tau - img * tpi, r2 = tl / tcn, c2 = tl - r2 * tcn;
+        const int tau = th * 32 + l32, img = tau / tpi, tl = tau - img * tpi, r2 = tl / tcn, c2 = tl - r2 * tcn;
         const int n = n_first + img;
         if (n >= p.N) return;
         float *base = outp + ((size_t)n * p.Mout * p.OH + (oh0 + 2 * r2)) * p.OW + 2 * c2;
@@ -645,7 +655,7 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
             float y[4];
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                y[q] = part[v][q] + xchg[(wk * 64 + v * 4 + q) * 64 + lane];
+                y[q] = part[v][q] + xchg[((w >> 1) * 64 + v * 4 + q) * 64 + lane];
                 if (add_bias) y[q] += bias;
             }
             float *o = base + (size_t)m * OHW;
@@ -1498,13 +1508,13 @@ int launch_patch(const PatchConv &pc, bool c_full, dim3 grid, size_t lds_bytes)
 struct PatchSetup {
     bool ok;
     PatchConv pc;
-    int shape;            // 0 wide, 1 square, 2 deep, 3 tall, 4 Winograd (128 rows x 32 tiles of 2x2 pixels)
+    int shape;            // 0 wide, 1 square, 2 deep, 3 tall, 4 Winograd (BM 128: 128 rows x 32 tiles of 2x2 pixels, BM 64: 64 rows x 64 tiles)
     int BM, BN, blocks_wanted, tiles;
     size_t lds_bytes, wp_elems;
 };
 
 template <bool kBwd>
-PatchSetup patch_setup_as(const dopt_hip_conv_desc *d, size_t P, size_t Q, bool allow_tall, bool wino = false);
+PatchSetup patch_setup_as(const dopt_hip_conv_desc *d, size_t P, size_t Q, bool allow_tall, int wino = 0);   // wino: rows of a Winograd tile, 0 none
 
 // DOPT_HIP_NO_WINO=1 keeps the Winograd kernel out (for A/B measurements); read once.
 bool no_wino()
@@ -1518,15 +1528,19 @@ template <bool kBwd>
 PatchSetup patch_setup(const dopt_hip_conv_desc *d, size_t P, size_t Q)
 {
     if (!no_wino()) {
-        const PatchSetup v = patch_setup_as<kBwd>(d, P, Q, false, true);
+        // 128-row tiles first: measured faster than 64-row tiles on every layer that has both (they read the input once
+        // per 128 rows and transform it once)
+        const PatchSetup v = patch_setup_as<kBwd>(d, P, Q, false, 128);
         if (v.ok) return v;
+        const PatchSetup v2 = patch_setup_as<kBwd>(d, P, Q, false, 64);
+        if (v2.ok) return v2;
     }
     const PatchSetup u = patch_setup_as<kBwd>(d, P, Q, true);
     return u.ok ? u : patch_setup_as<kBwd>(d, P, Q, false);
 }
 
 template <bool kBwd>
-PatchSetup patch_setup_as(const dopt_hip_conv_desc *d, size_t P, size_t Q, bool allow_tall, bool wino)
+PatchSetup patch_setup_as(const dopt_hip_conv_desc *d, size_t P, size_t Q, bool allow_tall, int wino)
 {
     PatchSetup u{};
     if (d->R != 3 || d->S != 3 || d->strideH != 1 || d->strideW != 1 || d->padH > 2 || d->padW > 2) return u;
@@ -1552,10 +1566,12 @@ PatchSetup patch_setup_as(const dopt_hip_conv_desc *d, size_t P, size_t Q, bool 
     const long tall_tiles = (long)(up160 / 160) * ((pc.ncols + 127) / 128);
     if (wino) {
         // whole 16-channel chunks of a deep reduction, whole 128-row tiles, pad 1, 2 x 2 tiles
-        if (d->padH != 1 || d->padW != 1 || pc.Cin % 16 != 0 || pc.Cin < 64 || pc.Mout % 128 != 0 || pc.OH % 2 != 0 ||
+        if (d->padH != 1 || d->padW != 1 || pc.Cin % 16 != 0 || pc.Cin < 64 || pc.Mout % wino != 0 || pc.OH % 2 != 0 ||
             pc.OW % 2 != 0 || pc.OH < 4 || pc.OW < 4)
             return u;
-        u.shape = 4; u.BM = 128; u.BN = 128; u.blocks_wanted = num_cus(); npmax = 16; threads = 512;
+        // whole 128-row tiles of 32 tiles (128 pixels), or whole 64-row tiles of 64 tiles (256 pixels)
+        u.shape = 4; u.BM = wino; u.BN = u.BM == 128 ? 128 : 256;
+        u.blocks_wanted = num_cus(); npmax = 16; threads = 512;
     } else if (allow_tall && pc.Mout > 64 && up160 <= up64 && up160 <= up128 && tall_tiles >= num_cus() &&
         !no_tall_tiles()) {
         u.shape = 3; u.BM = 160; u.BN = 128; u.blocks_wanted = num_cus(); npmax = 16; threads = 256;
@@ -1584,7 +1600,7 @@ PatchSetup patch_setup_as(const dopt_hip_conv_desc *d, size_t P, size_t Q, bool 
     u.lds_bytes = (size_t)2 * (pc.psz + 1) * 20 * sizeof(float);
     if (wino) {
         if (pc.rows % 2 != 0) return u;   // a pixel tile is whole 2 x 2 tiles
-        const size_t floats = (size_t)(((pc.psz + 1) * 20 + 3) / 4 * 4) + 16 * 32 * 20;
+        const size_t floats = (size_t)(((pc.psz + 1) * 20 + 3) / 4 * 4) + (size_t)16 * (u.BN / 4) * 20;
         u.lds_bytes = (floats > (size_t)kWinoXchg ? floats : (size_t)kWinoXchg) * sizeof(float);
     }
     if (u.lds_bytes > 160 * 1024) return u;
@@ -1681,6 +1697,29 @@ int patch_decide_splits(PatchSetup *u, const float *out)
 
 // `prepacked`: the filter already in the kernel's layout (dopt_hip_conv_pack_batch), or null to
 // pack it here first.
+// Device time of one kernel family alone (an entry point may also run split sums and packing): while the probe is on,
+// every launch of the family - 1: the one-launch backward pairs (conv_bwd_pair_k), 2: the Winograd kernel
+// (conv_wino_k) - is bracketed by two events on the stream it is launched on.
+struct PairProbe {
+    int on = 0;
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> events;   // kept for the process's lifetime, reused
+    size_t used = 0;
+    double flops = 0.0, bytes = 0.0;
+};
+PairProbe g_pair_probe;
+
+int probe_begin(PairProbe &probe)
+{
+    if (probe.used == probe.events.size()) {
+        hipEvent_t e0, e1;
+        DOPT_HIP_CHECK(hipEventCreate(&e0));
+        DOPT_HIP_CHECK(hipEventCreate(&e1));
+        probe.events.push_back({e0, e1});
+    }
+    DOPT_HIP_CHECK(hipEventRecord(probe.events[probe.used].first, stream()));
+    return DOPT_HIP_OK;
+}
+
 // The launch of a filled-in patch setup: the tile shape picks the instance.
 int dispatch_patch(const PatchSetup &u, int splits)
 {
@@ -1693,11 +1732,23 @@ int dispatch_patch(const PatchSetup &u, int splits)
     if (u.shape == 4) {
         static bool raised = false;
         if (!raised) {
-            DOPT_HIP_CHECK(hipFuncSetAttribute((const void *)conv_wino_k<16>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+            DOPT_HIP_CHECK(hipFuncSetAttribute((const void *)conv_wino_k<16, 4, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+            DOPT_HIP_CHECK(hipFuncSetAttribute((const void *)conv_wino_k<16, 2, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
             raised = true;
         }
-        hipLaunchKernelGGL(conv_wino_k<16>, grid, dim3(512), u.lds_bytes, stream(), pc);
+        PairProbe &probe = g_pair_probe;
+        const bool probing = probe.on == 2 && u.BM == 128 && !capturing();   // the 128-row instantiation only: one kernel, one average
+        if (probing)
+            if (int rc = probe_begin(probe)) return rc;
+        if (u.BM == 128) hipLaunchKernelGGL((conv_wino_k<16, 4, 1>), grid, dim3(512), u.lds_bytes, stream(), pc);
+        else hipLaunchKernelGGL((conv_wino_k<16, 2, 2>), grid, dim3(512), u.lds_bytes, stream(), pc);
         DOPT_LAUNCH_CHECK();
+        if (probing) {
+            DOPT_HIP_CHECK(hipEventRecord(probe.events[probe.used++].second, stream()));
+            // the direct algorithm's count (what the layer is, whatever the kernel multiplies): 2 N K C 9 P Q
+            probe.flops += 2.0 * (double)pc.ncols * pc.Mout * pc.Cin * 9.0;
+            probe.bytes += 4.0 * ((double)pc.N * pc.Cin * pc.IH * pc.IW + (double)pc.ncols * pc.Mout + (double)pc.Mout * pc.Cin * 9.0);
+        }
         return DOPT_HIP_OK;
     }
     return launch_patch<GatherDeep, 16>(pc, c_full, grid, u.lds_bytes);
@@ -2576,15 +2627,6 @@ int launch_bwd_pair(const PatchConv &pc, const WgradPatch &wp, unsigned grid_a, 
     return DOPT_HIP_OK;
 }
 
-// Device time of the one-launch pairs alone (their entry point also runs the split sums): while the probe is on,
-// every conv_bwd_pair_k launch is bracketed by two events on the stream it is launched on.
-struct PairProbe {
-    bool on = false;
-    std::vector<std::pair<hipEvent_t, hipEvent_t>> events;   // kept for the process's lifetime, reused
-    size_t used = 0;
-    double flops = 0.0, bytes = 0.0;
-};
-PairProbe g_pair_probe;
 
 int run_bwd_pair(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *dy, const float *prepacked, const float *x,
                  float *dx, float *dw, dopt_hip_split_sum *open, dopt_hip_split_sum *open_dw, bool *done)
@@ -2599,11 +2641,13 @@ int run_bwd_pair(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *d
     // rows of 8 .. 64 pixels or on 4 x 4 images.
     // (a layer the Winograd kernel takes has its filter packed for that kernel: shape 4, not a pair)
     const int combo = a.shape == 2 && b.tall && b.geo == 0 ? 0 : a.shape == 2 && b.tall && b.geo == 1 ? 1 : -1;
-    // (Other pairs of patch-kernel shapes as two launches out of one workspace request, so that the filter gradient's
-    // split sum could ride in the batch-norm gradient behind them as well, were measured: the layers concerned are
-    // followed by the multi-block batch norm, whose workgroups fill every CU, so the riders only start when those have
-    // finished - 20 us per layer instead of the 7.6 us of the separate sum.)
-    if (combo < 0) return DOPT_HIP_OK;
+    // A layer whose backward-data is the Winograd kernel: two launches, each as it would run alone, but out of ONE
+    // workspace request, so that both results can stay open for the launch behind them - the filter gradient's split
+    // sum rides in the batch-norm gradient there instead of being a launch of its own.  (The same for the 64-row layers
+    // was measured and does not pay: they are followed by the multi-block batch norm, whose workgroups fill every CU,
+    // so the riders only start when those have finished - 20 us per layer instead of the 7.6 us of the separate sum.)
+    const bool two = combo < 0 && a.shape == 4 && open_dw != nullptr && b.splits > 1;
+    if (combo < 0 && !two) return DOPT_HIP_OK;
     PatchConv &pc = a.pc;
     WgradPatch &wp = b.wp;
     const int splits_a = patch_decide_splits(&a, dx);
@@ -2623,18 +2667,14 @@ int run_bwd_pair(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *d
     const unsigned grid_a = xcd_grid((unsigned)(a.tiles * splits_a)), grid_b = xcd_grid((unsigned)(b.tiles * b.splits));
     const size_t lds_bytes = a.lds_bytes > b.lds_bytes ? a.lds_bytes : b.lds_bytes;
     PairProbe &probe = g_pair_probe;
-    const bool probing = probe.on && !capturing();
-    if (probing) {
-        if (probe.used == probe.events.size()) {
-            hipEvent_t e0, e1;
-            DOPT_HIP_CHECK(hipEventCreate(&e0));
-            DOPT_HIP_CHECK(hipEventCreate(&e1));
-            probe.events.push_back({e0, e1});
-        }
-        DOPT_HIP_CHECK(hipEventRecord(probe.events[probe.used].first, stream()));
-    }
+    const bool probing = probe.on == 1 && !capturing() && !two;
+    if (probing)
+        if (int rc2 = probe_begin(probe)) return rc2;
     int rc;
-    if (combo == 0) rc = launch_bwd_pair<GatherDeep, 16, 4, 1, 0>(pc, wp, grid_a, grid_b, lds_bytes);
+    if (two) {
+        rc = dispatch_wgrad_patch(b);
+        if (!rc) rc = dispatch_patch(a, splits_a);
+    } else if (combo == 0) rc = launch_bwd_pair<GatherDeep, 16, 4, 1, 0>(pc, wp, grid_a, grid_b, lds_bytes);
     else rc = launch_bwd_pair<GatherDeep, 16, 4, 1, 1>(pc, wp, grid_a, grid_b, lds_bytes);
     if (rc) return rc;
     if (probing) {
@@ -2854,7 +2894,8 @@ int dopt_hip_conv_bwd_pair_packed_open(const dopt_hip_conv_desc *d, const float 
 int dopt_hip_conv_pair_probe(int enable)
 {
     DOPT_ENSURE_INIT();
-    g_pair_probe.on = enable != 0;
+    DOPT_REQUIRE(enable >= 0 && enable <= 2, "dopt_hip_conv_pair_probe: 0 off, 1 one-launch backward pairs, 2 Winograd launches");
+    g_pair_probe.on = enable;
     if (enable) {
         g_pair_probe.used = 0;
         g_pair_probe.flops = g_pair_probe.bytes = 0.0;

@@ -340,11 +340,13 @@ int dopt_hip_conv_bwd_pair_packed_open(const dopt_hip_conv_desc *d, const float 
                                        const float *x, float *dx, float *dw, dopt_hip_split_sum *open,
                                        dopt_hip_split_sum *open_dw);
 /* Measurement aid (no counterpart in the reference; CUDAPlan.profiler, cuda/package.d:424-431, times whole kernel
-   objects): while enabled, every one-launch pair above is bracketed by two events on the library's queue, so its
-   device time is known apart from the split sums the same entry point runs.  probe(1) starts a fresh collection,
-   probe(0) stops it; read waits for the launches collected so far and returns their number, their summed
-   duration, the FLOPs they executed (both products, every tap) and their algorithmic bytes (dy, x, dx, filter,
-   dw once each).  Launches recorded into a HIP graph are not collected. */
+   objects): while enabled, every launch of one kernel family is bracketed by two events on the library's queue, so
+   its device time is known apart from the split sums and packing the same entry point runs.  probe(1) collects the
+   one-launch pairs above, probe(2) the launches of the Winograd kernel (forward and backward-data of 3x3 layers with
+   whole 128-row tiles); either starts a fresh collection, probe(0) stops it.  read waits for the launches collected so
+   far and returns their number, their summed duration, their FLOPs by the direct algorithm's count (2 N K C 9 P Q per
+   product, every tap: what a pair executes; the Winograd kernel executes 16/36 of it) and their algorithmic bytes
+   (every operand and result once).  Launches recorded into a HIP graph are not collected. */
 int dopt_hip_conv_pair_probe(int enable);
 int dopt_hip_conv_pair_probe_read(int *launches, double *total_us, double *flops, double *bytes);
 /* value = sum of the copies in order (+ bias): what the closed entry points do themselves. */

@@ -486,10 +486,20 @@ def test_backward_data_and_filter_gradient_as_one_call(xs, k):
     capi.check(lib.dopt_hip_conv_pair_probe(0))
     up = lambda v, m: (v + m - 1) // m * m
     # 128-row tiles in both products (wherever 64-row tiles would not pad less) on images of 4 x 4 pixels and more -
-    # unless backward-data is a Winograd layer (whole 128-row tiles of input channels, 64 and more output channels,
-    # even sides of at least 4): its filter is packed for that kernel and the two products are two launches
-    winograd = Cin % 128 == 0 and k % 16 == 0 and k >= 64 and H % 2 == 0 and W % 2 == 0 and H >= 4 and W >= 4 and \
-        (128 % W == 0) and ((128 // W) % 2 == 0)
+    # unless backward-data is a Winograd layer (whole 128-row or 64-row tiles of input channels with a pixel tile of
+    # whole 2 x 2 tiles, 64 and more output channels, even sides of at least 4): its filter is packed for that kernel
+    # and the two products are two launches
+    def winograd_tile(bm, bn):
+        if Cin % bm or bn % W:
+            return False
+        rows = bn // W
+        if rows <= H:
+            fits, psz = H % rows == 0 and rows % 2 == 0, (rows + 2) * (W + 2)
+        else:
+            fits, psz = rows % H == 0, (rows // H) * (H + 2) * (W + 2)
+        return fits and psz * 16 <= 16 * 512
+    winograd = k % 16 == 0 and k >= 64 and H % 2 == 0 and W % 2 == 0 and H >= 4 and W >= 4 and \
+        (winograd_tile(128, 128) or winograd_tile(64, 256))
     one_launch = Cin > 64 and up(Cin, 128) <= up(Cin, 64) and k >= 128 and up(k, 128) <= up(k, 64) and W >= 4 and not winograd
     assert n.value == (1 if one_launch else 0)
     if one_launch:
@@ -509,7 +519,8 @@ def test_backward_data_and_filter_gradient_as_one_call(xs, k):
     dx.set(np.full(xs, np.nan, np.float32)); dw.set(np.full((k, Cin, 3, 3), np.nan, np.float32))
     o, ow = capi.SplitSum(), capi.SplitSum()
     capi.check(lib.dopt_hip_conv_bwd_pair_packed_open(C.byref(d), dy.ptr, packed.ptr, x.ptr, dx.ptr, dw.ptr, C.byref(o), C.byref(ow)))
-    assert ow.value == dw.ptr and (ow.splits == 0 or (one_launch and ow.splits > 1 and ow.lanes in (4, 16)))
+    # (a Winograd backward-data and its filter gradient are two launches that leave a split filter gradient open too)
+    assert ow.value == dw.ptr and (ow.splits == 0 or ((one_launch or winograd) and ow.splits > 1 and ow.lanes in (4, 16)))
     if xs == (16, 250, 8, 8):
         assert ow.splits > 1
     if ow.splits:

@@ -399,6 +399,12 @@ CONV_CASES = [  # N, C, H, W, K, R, S, pad, stride
     (3, 64, 8, 8, 128, 3, 3, (1, 1), (1, 1)),
     (21, 256, 4, 4, 128, 3, 3, (1, 1), (1, 1)),
     (4, 128, 32, 32, 128, 3, 3, (1, 1), (1, 1)),
+    # ... and 64-row tiles of 64 2x2-pixel tiles where the rows are whole 64s but not whole 128s: a quarter of an image,
+    # one image, four images (the last tile with images missing), three row tiles
+    (4, 64, 32, 32, 64, 3, 3, (1, 1), (1, 1)),
+    (5, 128, 16, 16, 64, 3, 3, (1, 1), (1, 1)),
+    (7, 64, 8, 8, 192, 3, 3, (1, 1), (1, 1)),
+    (3, 192, 16, 16, 320, 3, 3, (1, 1), (1, 1)),
     (2, 80, 8, 12, 128, 3, 3, (1, 1), (1, 1)),     # 12 columns: no whole tile rows in 128 pixels, the direct kernels
     (2, 7, 11, 13, 9, 5, 5, (2, 2), (3, 3)),      # nine classes with work in one launch
     (1, 4, 9, 9, 5, 5, 5, (2, 2), (4, 4)),        # sixteen classes: one after the other
