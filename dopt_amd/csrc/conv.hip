@@ -2641,12 +2641,12 @@ int run_bwd_pair(const dopt_hip_conv_desc *d, size_t P, size_t Q, const float *d
     // rows of 8 .. 64 pixels or on 4 x 4 images.
     // (a layer the Winograd kernel takes has its filter packed for that kernel: shape 4, not a pair)
     const int combo = a.shape == 2 && b.tall && b.geo == 0 ? 0 : a.shape == 2 && b.tall && b.geo == 1 ? 1 : -1;
-    // A layer whose backward-data is the Winograd kernel: two launches, each as it would run alone, but out of ONE
+    // A layer whose backward-data is the Winograd kernel on 128-row tiles: two launches, each as it would run alone, but out of ONE
     // workspace request, so that both results can stay open for the launch behind them - the filter gradient's split
     // sum rides in the batch-norm gradient there instead of being a launch of its own.  (The same for the 64-row layers
     // was measured and does not pay: they are followed by the multi-block batch norm, whose workgroups fill every CU,
     // so the riders only start when those have finished - 20 us per layer instead of the 7.6 us of the separate sum.)
-    const bool two = combo < 0 && a.shape == 4 && open_dw != nullptr && b.splits > 1;
+    const bool two = combo < 0 && a.shape == 4 && a.BM == 128 && open_dw != nullptr && b.splits > 1;
     if (combo < 0 && !two) return DOPT_HIP_OK;
     PatchConv &pc = a.pc;
     WgradPatch &wp = b.wp;

@@ -498,8 +498,9 @@ def test_backward_data_and_filter_gradient_as_one_call(xs, k):
         else:
             fits, psz = rows % H == 0, (rows // H) * (H + 2) * (W + 2)
         return fits and psz * 16 <= 16 * 512
-    winograd = k % 16 == 0 and k >= 64 and H % 2 == 0 and W % 2 == 0 and H >= 4 and W >= 4 and \
-        (winograd_tile(128, 128) or winograd_tile(64, 256))
+    winograd_layer = k % 16 == 0 and k >= 64 and H % 2 == 0 and W % 2 == 0 and H >= 4 and W >= 4
+    winograd = winograd_layer and (winograd_tile(128, 128) or winograd_tile(64, 256))
+    winograd_open = winograd_layer and winograd_tile(128, 128)     # only the 128-row layers leave the filter gradient open
     one_launch = Cin > 64 and up(Cin, 128) <= up(Cin, 64) and k >= 128 and up(k, 128) <= up(k, 64) and W >= 4 and not winograd
     assert n.value == (1 if one_launch else 0)
     if one_launch:
@@ -519,8 +520,9 @@ def test_backward_data_and_filter_gradient_as_one_call(xs, k):
     dx.set(np.full(xs, np.nan, np.float32)); dw.set(np.full((k, Cin, 3, 3), np.nan, np.float32))
     o, ow = capi.SplitSum(), capi.SplitSum()
     capi.check(lib.dopt_hip_conv_bwd_pair_packed_open(C.byref(d), dy.ptr, packed.ptr, x.ptr, dx.ptr, dw.ptr, C.byref(o), C.byref(ow)))
-    # (a Winograd backward-data and its filter gradient are two launches that leave a split filter gradient open too)
-    assert ow.value == dw.ptr and (ow.splits == 0 or ((one_launch or winograd) and ow.splits > 1 and ow.lanes in (4, 16)))
+    # (a Winograd backward-data on 128-row tiles and its filter gradient are two launches that leave a split filter
+    # gradient open too)
+    assert ow.value == dw.ptr and (ow.splits == 0 or ((one_launch or winograd_open) and ow.splits > 1 and ow.lanes in (4, 16)))
     if xs == (16, 250, 8, 8):
         assert ow.splits > 1
     if ow.splits:
