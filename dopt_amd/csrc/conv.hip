@@ -1565,10 +1565,13 @@ PatchSetup patch_setup_as(const dopt_hip_conv_desc *d, size_t P, size_t Q, bool 
     // (only where they still give every compute unit a tile: 480 channels on 8 x 8 images are 192 such tiles, and ran slower)
     const long tall_tiles = (long)(up160 / 160) * ((pc.ncols + 127) / 128);
     if (wino) {
-        // whole 16-channel chunks of a deep reduction, whole 128-row tiles, pad 1, 2 x 2 tiles
-        if (d->padH != 1 || d->padW != 1 || pc.Cin % 16 != 0 || pc.Cin < 64 || pc.Mout % wino != 0 || pc.OH % 2 != 0 ||
-            pc.OW % 2 != 0 || pc.OH < 4 || pc.OW < 4)
+        // whole 16-channel chunks of a deep reduction, pad 1, 2 x 2 tiles
+        if (d->padH != 1 || d->padW != 1 || pc.Cin % 16 != 0 || pc.Cin < 64 || pc.OH % 2 != 0 || pc.OW % 2 != 0 || pc.OH < 4 ||
+            pc.OW < 4)
             return u;
+        // whole tiles of rows, or 64-row tiles padded by no more than a fifth (160 rows as 192: still 1.9 times fewer
+        // matrix instructions than the direct kernels execute)
+        if (pc.Mout % wino != 0 && !(wino == 64 && pc.Mout > 64 && up64 * 5 <= pc.Mout * 6)) return u;
         // whole 128-row tiles of 32 tiles (128 pixels), or whole 64-row tiles of 64 tiles (256 pixels)
         u.shape = 4; u.BM = wino; u.BN = u.BM == 128 ? 128 : 256;
         u.blocks_wanted = num_cus(); npmax = 16; threads = 512;
