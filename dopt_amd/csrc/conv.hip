@@ -493,7 +493,8 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
     const int cb = split * p.chunks_per_split;
     const int ce = min(cb + p.chunks_per_split, p.chunks_total);
 
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wavefront-uniform, and known to be: it enters scalar load offsets
     const int wi = w & 1, wk = (w >> 1) % WK, th = (w >> 1) / WK;
     const int kh = lane >> 5, l32 = lane & 31;
     const int OHW = p.OH * p.OW;
@@ -589,33 +590,45 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
     __syncthreads();
 
     constexpr int PER = (NPMAX + 3) / 4;
+    float4 fb_next[2];
+    fb_next[0] = *(const float4 *)(V + b_frag);
+    fb_next[1] = *(const float4 *)(V + b_frag + 4);
     for (int chunk = cb; chunk < ce; ++chunk) {
         static_for<0, 8>([&](auto xtag) {
             constexpr int xl = decltype(xtag)::value;
-            const float4 fb0 = *(const float4 *)(V + b_frag + xl * TT * LDP);
-            const float4 fb1 = *(const float4 *)(V + b_frag + xl * TT * LDP + 4);
+            const float4 fb0 = fb_next[0], fb1 = fb_next[1];
             const float4 fa0 = fa_ring[xl % 4][0], fa1 = fa_ring[xl % 4][1];
-            // three positions ahead (the slot of the position before this one)
-            fa_load(StepTag<(xl + 3) % 4>{}, (xl + 3 < 8 ? chunk * 16 : (chunk + 1) * 16 - 8) + wi * 8 + xl + 3);
-            // the next chunk's patch: loads during positions 0..3, LDS stores during 4..7 (nobody reads `raw` now)
-            if constexpr (xl < 4) {
-#pragma unroll
-                for (int i = xl * PER; i < (xl + 1) * PER && i < NPMAX; i++) patch_load(i, chunk + 1);
-            } else {
-#pragma unroll
-                for (int i = (xl - 4) * PER; i < (xl - 3) * PER && i < NPMAX; i++) patch_store(i);
-            }
             static_for<0, 8>([&](auto stag) {
                 constexpr int ks = decltype(stag)::value;
+                // side work of this step, pinned to it: left to itself the scheduler sinks every load to its first use
+                if constexpr (ks == 0) {
+                    // the filter fragments three positions ahead (into the slot of the position before this one)
+                    fa_load(StepTag<(xl + 3) % 4>{}, (xl + 3 < 8 ? chunk * 16 : (chunk + 1) * 16 - 8) + wi * 8 + xl + 3);
+                }
+                if constexpr (ks == 1 && xl < 7) {   // this lane's tile at the next position
+                    fb_next[0] = *(const float4 *)(V + b_frag + (xl + 1) * TT * LDP);
+                    fb_next[1] = *(const float4 *)(V + b_frag + (xl + 1) * TT * LDP + 4);
+                }
+                // the next chunk's patch: loads during positions 0..3, LDS stores during 4..7 (nobody reads `raw` now)
+                if constexpr (ks >= 2 && ks < 2 + PER) {
+                    constexpr int i = (xl % 4) * PER + ks - 2;
+                    if constexpr (i < NPMAX) {
+                        if constexpr (xl < 4) patch_load(i, chunk + 1);
+                        else patch_store(i);
+                    }
+                }
                 const float4 av = ks < 4 ? fa0 : fa1, bv = ks < 4 ? fb0 : fb1;
                 const float a = ks % 4 == 0 ? av.x : ks % 4 == 1 ? av.y : ks % 4 == 2 ? av.z : av.w;
                 const float b = ks % 4 == 0 ? bv.x : ks % 4 == 1 ? bv.y : ks % 4 == 2 ? bv.z : bv.w;
                 acc[xl] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[xl], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
             });
         });
         __syncthreads();              // every wavefront is done with V; the next patch is in `raw`
         if (chunk + 1 < ce) transform();
         __syncthreads();
+        fb_next[0] = *(const float4 *)(V + b_frag);
+        fb_next[1] = *(const float4 *)(V + b_frag + 4);
     }
 
     // ---- inverse transform.  This wavefront's rows of the 4x4 grid are i = 2 wi, 2 wi + 1; acc[4 il + j] = M[i][j].
