@@ -476,12 +476,16 @@ constexpr int kWinoXchg = 4 * 64 * 64;   // floats of the exchange area: four wa
 template <int NPMAX, int WK, int TH>
 __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
 {
-    static_assert(WK * TH == 4, "eight wavefronts");
-    constexpr int BM = 32 * WK, BN = 128 * TH, TT = 32 * TH, THREADS = 512, CH = 16, LDP = 20;
+    static_assert(WK * TH == 4 && NPMAX == 16, "eight wavefronts, sixteen channels per chunk");
+    constexpr int BM = 32 * WK, BN = 128 * TH, TT = 32 * TH, CH = 16, LDP = 20, VSZ = 16 * TT * LDP;
+    // 32 tiles per workgroup: V and the raw patch are double-buffered, the transform of the next chunk runs under this
+    // chunk's matrix instructions and the workgroup meets once per chunk.  64 tiles: one V (80 KB), transformed between
+    // two barriers.
+    constexpr bool DB = TH == 1;
     extern __shared__ __attribute__((aligned(16))) float lds[];
-    const int raw_floats = ((p.psz + 1) * LDP + 3) / 4 * 4;   // one spare position absorbs the stores of unused slots
-    float *const raw = lds;
-    float *const V = lds + raw_floats;                          // [16][TT][LDP]
+    const int raw_floats = ((p.psz + 1) * LDP + 3) / 4 * 4;   // one spare position absorbs the stores of idle threads
+    float *const raw0 = lds;
+    float *const V0 = lds + (DB ? 2 : 1) * raw_floats;          // [16][TT][LDP] (x 2)
 
     unsigned L;
     const unsigned tiles = (unsigned)(p.mtiles * p.ntiles);
@@ -492,6 +496,7 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
     const int m0 = mt * BM, n0 = nt * BN;
     const int cb = split * p.chunks_per_split;
     const int ce = min(cb + p.chunks_per_split, p.chunks_total);
+    const int nch = ce - cb;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wavefront-uniform, and known to be: it enters scalar load offsets
@@ -502,29 +507,33 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
     const __amdgpu_buffer_rsrc_t rin = make_rsrc(p.in, p.in_bytes);
     const __amdgpu_buffer_rsrc_t rwp = make_rsrc(p.wp, p.wp_bytes);
 
-    // ---- patch slots of this thread, as in conv_patch_body
+    // ---- the patch: a thread owns ONE position and loads `nslots` of the chunk's channels of it, so its sixteen
+    // addresses are one per-lane offset plus a wavefront-uniform channel offset (sixteen separate offsets and LDS
+    // addresses would hold 32 registers).  Up to 256 positions: wavefronts 4..7 take channels 8..15 of the same positions.
     const int n_first = n0 / OHW, oh0 = (n0 - n_first * OHW) / p.OW;
-    unsigned p_voff[NPMAX];
-    int p_lds[NPMAX];
-#pragma unroll
-    for (int i = 0; i < NPMAX; i++) {
-        const unsigned e = (unsigned)(i * THREADS + tid);
-        const unsigned c = fast_div(e, p.magic_psz);
-        const unsigned pos = e - c * (unsigned)p.psz;
-        const unsigned img = fast_div(pos, p.magic_img);
-        const unsigned rem = pos - img * (unsigned)(p.PR * p.PC);
+    const int nslots = p.psz <= 256 ? 8 : 16;
+    const int pos = p.psz <= 256 ? (tid & 255) : tid;
+    const int cbase = p.psz <= 256 ? (w >> 2) * 8 : 0;
+    unsigned p_voff;
+    int p_lds;
+    {
+        const unsigned ps = (unsigned)min(pos, p.psz - 1);
+        const unsigned img = fast_div(ps, p.magic_img);
+        const unsigned rem = ps - img * (unsigned)(p.PR * p.PC);
         const unsigned pr = fast_div(rem, p.magic_pc);
         const unsigned pc = rem - pr * (unsigned)p.PC;
         const int n = n_first + (int)img, ih = oh0 + (int)pr - p.PT, iw = (int)pc - p.PL;
-        const int bad = (CH - 1 - (int)c) | (p.N - 1 - n) | ih | (p.IH - 1 - ih) | iw | (p.IW - 1 - iw);
-        p_voff[i] = bad < 0 ? kOobOffset : (unsigned)(((n * p.Cin + (int)c) * p.IH + ih) * p.IW + iw) * 4u;
-        p_lds[i] = c < (unsigned)CH ? (int)(pos * LDP + c) * 4 : (p.psz * LDP + (tid & 15)) * 4;
+        const int bad = (p.psz - 1 - pos) | (p.N - 1 - n) | ih | (p.IH - 1 - ih) | iw | (p.IW - 1 - iw);
+        p_voff = bad < 0 ? kOobOffset : (unsigned)((n * p.Cin * p.IH + ih) * p.IW + iw) * 4u;
+        p_lds = (min(pos, p.psz) * LDP + cbase) * 4;
     }
     float preg[NPMAX];
     auto patch_load = [&](int i, int chunk) {
-        preg[i] = buffer_load_f32(rin, p_voff[i], (unsigned)(chunk * CH * chan_stride) * 4u);
+        if (i < nslots) preg[i] = buffer_load_f32(rin, p_voff, (unsigned)((chunk * CH + cbase + i) * chan_stride) * 4u);
     };
-    auto patch_store = [&](int i) { *(float *)((char *)raw + p_lds[i]) = preg[i]; };
+    auto patch_store = [&](int i, float *rawb) {
+        if (i < nslots) *(float *)((char *)rawb + p_lds + i * 4) = preg[i];
+    };
 
     // ---- the transform items of this thread (TH of them): row ti of Bt d B for tile tau, channels 4 cq .. 4 cq + 3
     const int tcn = p.OW >> 1, tpi = (p.rows >> 1) * tcn;          // tiles per row of tiles, per image of the pixel tile
@@ -533,7 +542,7 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
     float sg[TH];
 #pragma unroll
     for (int u = 0; u < TH; u++) {
-        const int item = u * THREADS + tid, ti = item / (TT * 4), tau_t = (item % (TT * 4)) >> 2, cq = item & 3;
+        const int item = u * 512 + tid, ti = item / (TT * 4), tau_t = (item % (TT * 4)) >> 2, cq = item & 3;
         const int img = tau_t / tpi, tl = tau_t - img * tpi, r2 = tl / tcn, c2 = tl - r2 * tcn;
         const int t_in = ((img * p.PR + 2 * r2) * p.PC + 2 * c2) * LDP + cq * 4;
         const int ra = ti == 0 ? 0 : ti == 2 ? 2 : 1, rb = ti == 0 ? 2 : ti == 1 ? 2 : ti == 2 ? 1 : 3;
@@ -542,21 +551,23 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
         t_out[u] = ((ti * 4) * TT + tau_t) * LDP + cq * 4;
         sg[u] = ti == 1 ? 1.0f : -1.0f;
     }
-    auto transform = [&]() {
+    float4 tt[TH][4];
+    auto transform_read = [&](int b, const float *rawb) {       // column b of the thread's row of Bt d
+#pragma unroll
+        for (int u = 0; u < TH; u++) {
+            const float4 da = *(const float4 *)(rawb + t_a[u] + b * LDP), db = *(const float4 *)(rawb + t_b[u] + b * LDP);
+            tt[u][b] = make_float4(da.x + sg[u] * db.x, da.y + sg[u] * db.y, da.z + sg[u] * db.z, da.w + sg[u] * db.w);
+        }
+    };
+    auto transform_write = [&](float *Vb) {                      // ... times B: four positions, four channels each
         auto sub = [](float4 x, float4 y) { return make_float4(x.x - y.x, x.y - y.y, x.z - y.z, x.w - y.w); };
         auto add = [](float4 x, float4 y) { return make_float4(x.x + y.x, x.y + y.y, x.z + y.z, x.w + y.w); };
 #pragma unroll
         for (int u = 0; u < TH; u++) {
-            float4 t[4];
-#pragma unroll
-            for (int b = 0; b < 4; b++) {
-                const float4 da = *(const float4 *)(raw + t_a[u] + b * LDP), db = *(const float4 *)(raw + t_b[u] + b * LDP);
-                t[b] = make_float4(da.x + sg[u] * db.x, da.y + sg[u] * db.y, da.z + sg[u] * db.z, da.w + sg[u] * db.w);
-            }
-            *(float4 *)(V + t_out[u]) = sub(t[0], t[2]);
-            *(float4 *)(V + t_out[u] + TT * LDP) = add(t[1], t[2]);
-            *(float4 *)(V + t_out[u] + 2 * TT * LDP) = sub(t[2], t[1]);
-            *(float4 *)(V + t_out[u] + 3 * TT * LDP) = sub(t[1], t[3]);
+            *(float4 *)(Vb + t_out[u]) = sub(tt[u][0], tt[u][2]);
+            *(float4 *)(Vb + t_out[u] + TT * LDP) = add(tt[u][1], tt[u][2]);
+            *(float4 *)(Vb + t_out[u] + 2 * TT * LDP) = sub(tt[u][2], tt[u][1]);
+            *(float4 *)(Vb + t_out[u] + 3 * TT * LDP) = sub(tt[u][1], tt[u][3]);
         }
     };
 
@@ -577,23 +588,42 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
 #pragma unroll
         for (int v = 0; v < 16; v++) acc[x][v] = 0.0f;
 
-    // prologue: the first patch, transformed, and the first three filter fragments
+    // prologue: the first patch (and, double-buffered, the second), the first transform, the first three filter fragments
 #pragma unroll
     for (int i = 0; i < NPMAX; i++) patch_load(i, cb);
     fa_load(StepTag<0>{}, cb * 16 + wi * 8);
     fa_load(StepTag<1>{}, cb * 16 + wi * 8 + 1);
     fa_load(StepTag<2>{}, cb * 16 + wi * 8 + 2);
 #pragma unroll
-    for (int i = 0; i < NPMAX; i++) patch_store(i);
+    for (int i = 0; i < NPMAX; i++) patch_store(i, raw0);
+    if constexpr (DB) {
+        if (nch > 1) {
+#pragma unroll
+            for (int i = 0; i < NPMAX; i++) patch_load(i, cb + 1);
+#pragma unroll
+            for (int i = 0; i < NPMAX; i++) patch_store(i, raw0 + raw_floats);
+        }
+    }
     __syncthreads();
-    transform();
+#pragma unroll
+    for (int b = 0; b < 4; b++) transform_read(b, raw0);
+    transform_write(V0);
     __syncthreads();
 
-    constexpr int PER = (NPMAX + 3) / 4;
+    constexpr int PER = NPMAX / 4;
     float4 fb_next[2];
-    fb_next[0] = *(const float4 *)(V + b_frag);
-    fb_next[1] = *(const float4 *)(V + b_frag + 4);
-    for (int chunk = cb; chunk < ce; ++chunk) {
+    fb_next[0] = *(const float4 *)(V0 + b_frag);
+    fb_next[1] = *(const float4 *)(V0 + b_frag + 4);
+    for (int it = 0; it < nch; ++it) {
+        const int chunk = cb + it;
+        // double-buffered: V of this chunk, raw patch and V of the next one, raw patch of the one after (into the buffer
+        // this chunk's patch left when it was transformed)
+        const float *const Vc = V0 + (DB ? (it & 1) * VSZ : 0);
+        float *const Vn = V0 + (DB ? ((it + 1) & 1) * VSZ : 0);
+        const float *const rawn = raw0 + (DB ? ((it + 1) & 1) * raw_floats : 0);
+        float *const raww = raw0 + (DB ? (it & 1) * raw_floats : 0);
+        const int ahead = DB ? 2 : 1;
+        const bool more = it + 1 < nch, fetch = it + ahead < nch;
         static_for<0, 8>([&](auto xtag) {
             constexpr int xl = decltype(xtag)::value;
             const float4 fb0 = fb_next[0], fb1 = fb_next[1];
@@ -606,15 +636,21 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
                     fa_load(StepTag<(xl + 3) % 4>{}, (xl + 3 < 8 ? chunk * 16 : (chunk + 1) * 16 - 8) + wi * 8 + xl + 3);
                 }
                 if constexpr (ks == 1 && xl < 7) {   // this lane's tile at the next position
-                    fb_next[0] = *(const float4 *)(V + b_frag + (xl + 1) * TT * LDP);
-                    fb_next[1] = *(const float4 *)(V + b_frag + (xl + 1) * TT * LDP + 4);
+                    fb_next[0] = *(const float4 *)(Vc + b_frag + (xl + 1) * TT * LDP);
+                    fb_next[1] = *(const float4 *)(Vc + b_frag + (xl + 1) * TT * LDP + 4);
                 }
-                // the next chunk's patch: loads during positions 0..3, LDS stores during 4..7 (nobody reads `raw` now)
+                // the patch `ahead` chunks on: loads during positions 0..3, LDS stores during 4..7
                 if constexpr (ks >= 2 && ks < 2 + PER) {
                     constexpr int i = (xl % 4) * PER + ks - 2;
-                    if constexpr (i < NPMAX) {
-                        if constexpr (xl < 4) patch_load(i, chunk + 1);
-                        else patch_store(i);
+                    if (fetch) {
+                        if constexpr (xl < 4) patch_load(i, chunk + ahead);
+                        else patch_store(i, raww);
+                    }
+                }
+                if constexpr (DB && ks == 6) {       // the next chunk's transform: a column per position, then the products
+                    if (more) {
+                        if constexpr (xl < 4) transform_read(xl, rawn);
+                        if constexpr (xl == 4) transform_write(Vn);
                     }
                 }
                 const float4 av = ks < 4 ? fa0 : fa1, bv = ks < 4 ? fb0 : fb1;
@@ -624,11 +660,17 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
                 __builtin_amdgcn_sched_barrier(0);
             });
         });
-        __syncthreads();              // every wavefront is done with V; the next patch is in `raw`
-        if (chunk + 1 < ce) transform();
-        __syncthreads();
-        fb_next[0] = *(const float4 *)(V + b_frag);
-        fb_next[1] = *(const float4 *)(V + b_frag + 4);
+        __syncthreads();              // every wavefront is done with V of this chunk; the next patch is in place
+        if constexpr (!DB) {
+            if (more) {
+#pragma unroll
+                for (int b = 0; b < 4; b++) transform_read(b, raw0);
+                transform_write(V0);
+            }
+            __syncthreads();
+        }
+        fb_next[0] = *(const float4 *)(Vn + b_frag);
+        fb_next[1] = *(const float4 *)(Vn + b_frag + 4);
     }
 
     // ---- inverse transform.  This wavefront's rows of the 4x4 grid are i = 2 wi, 2 wi + 1; acc[4 il + j] = M[i][j].
@@ -1616,7 +1658,8 @@ PatchSetup patch_setup_as(const dopt_hip_conv_desc *d, size_t P, size_t Q, bool 
     u.lds_bytes = (size_t)2 * (pc.psz + 1) * 20 * sizeof(float);
     if (wino) {
         if (pc.rows % 2 != 0) return u;   // a pixel tile is whole 2 x 2 tiles
-        const size_t floats = (size_t)(((pc.psz + 1) * 20 + 3) / 4 * 4) + (size_t)16 * (u.BN / 4) * 20;
+        const size_t buffers = u.BM == 128 ? 2 : 1;   // 32 tiles: raw patch and V are double-buffered
+        const size_t floats = buffers * ((size_t)(((pc.psz + 1) * 20 + 3) / 4 * 4) + (size_t)16 * (u.BN / 4) * 20);
         u.lds_bytes = (floats > (size_t)kWinoXchg ? floats : (size_t)kWinoXchg) * sizeof(float);
     }
     if (u.lds_bytes > 160 * 1024) return u;
