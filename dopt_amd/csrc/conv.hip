@@ -531,8 +531,9 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
     auto patch_load = [&](int i, int chunk) {
         if (i < nslots) preg[i] = buffer_load_f32(rin, p_voff, (unsigned)((chunk * CH + cbase + i) * chan_stride) * 4u);
     };
-    auto patch_store = [&](int i, float *rawb) {
-        if (i < nslots) *(float *)((char *)rawb + p_lds + i * 4) = preg[i];
+    auto patch_store = [&](int g, float *rawb) {   // channels 4 g .. 4 g + 3 of the position: one 128-bit store
+        if (4 * g < nslots)
+            *(float4 *)((char *)rawb + p_lds + g * 16) = make_float4(preg[4 * g], preg[4 * g + 1], preg[4 * g + 2], preg[4 * g + 3]);
     };
 
     // ---- the transform items of this thread (TH of them): row ti of Bt d B for tile tau, channels 4 cq .. 4 cq + 3
@@ -556,7 +557,9 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
 #pragma unroll
         for (int u = 0; u < TH; u++) {
             const float4 da = *(const float4 *)(rawb + t_a[u] + b * LDP), db = *(const float4 *)(rawb + t_b[u] + b * LDP);
-            tt[u][b] = make_float4(da.x + sg[u] * db.x, da.y + sg[u] * db.y, da.z + sg[u] * db.z, da.w + sg[u] * db.w);
+            // sg is +-1: the fused form rounds once, like the sum or difference it stands for
+            tt[u][b] = make_float4(__builtin_fmaf(sg[u], db.x, da.x), __builtin_fmaf(sg[u], db.y, da.y),
+                                   __builtin_fmaf(sg[u], db.z, da.z), __builtin_fmaf(sg[u], db.w, da.w));
         }
     };
     auto transform_write = [&](float *Vb) {                      // ... times B: four positions, four channels each
@@ -588,21 +591,31 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
 #pragma unroll
         for (int v = 0; v < 16; v++) acc[x][v] = 0.0f;
 
-    // prologue: the first patch (and, double-buffered, the second), the first transform, the first three filter fragments
+    // prologue: the first patch (and, double-buffered, the second: both in flight together), the first transform, the
+    // first three filter fragments
 #pragma unroll
     for (int i = 0; i < NPMAX; i++) patch_load(i, cb);
-    fa_load(StepTag<0>{}, cb * 16 + wi * 8);
-    fa_load(StepTag<1>{}, cb * 16 + wi * 8 + 1);
-    fa_load(StepTag<2>{}, cb * 16 + wi * 8 + 2);
-#pragma unroll
-    for (int i = 0; i < NPMAX; i++) patch_store(i, raw0);
     if constexpr (DB) {
-        if (nch > 1) {
+        float second[NPMAX];
 #pragma unroll
-            for (int i = 0; i < NPMAX; i++) patch_load(i, cb + 1);
+        for (int i = 0; i < NPMAX; i++)
+            second[i] = i < nslots && nch > 1 ? buffer_load_f32(rin, p_voff, (unsigned)(((cb + 1) * CH + cbase + i) * chan_stride) * 4u) : 0.0f;
+        fa_load(StepTag<0>{}, cb * 16 + wi * 8);
+        fa_load(StepTag<1>{}, cb * 16 + wi * 8 + 1);
+        fa_load(StepTag<2>{}, cb * 16 + wi * 8 + 2);
 #pragma unroll
-            for (int i = 0; i < NPMAX; i++) patch_store(i, raw0 + raw_floats);
-        }
+        for (int g = 0; g < NPMAX / 4; g++) patch_store(g, raw0);
+#pragma unroll
+        for (int g = 0; g < NPMAX / 4; g++)
+            if (4 * g < nslots)
+                *(float4 *)((char *)(raw0 + raw_floats) + p_lds + g * 16) =
+                    make_float4(second[4 * g], second[4 * g + 1], second[4 * g + 2], second[4 * g + 3]);
+    } else {
+        fa_load(StepTag<0>{}, cb * 16 + wi * 8);
+        fa_load(StepTag<1>{}, cb * 16 + wi * 8 + 1);
+        fa_load(StepTag<2>{}, cb * 16 + wi * 8 + 2);
+#pragma unroll
+        for (int g = 0; g < NPMAX / 4; g++) patch_store(g, raw0);
     }
     __syncthreads();
 #pragma unroll
@@ -640,12 +653,11 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
                     fb_next[1] = *(const float4 *)(Vc + b_frag + (xl + 1) * TT * LDP + 4);
                 }
                 // the patch `ahead` chunks on: loads during positions 0..3, LDS stores during 4..7
-                if constexpr (ks >= 2 && ks < 2 + PER) {
-                    constexpr int i = (xl % 4) * PER + ks - 2;
-                    if (fetch) {
-                        if constexpr (xl < 4) patch_load(i, chunk + ahead);
-                        else patch_store(i, raww);
-                    }
+                if constexpr (xl < 4 && ks >= 2 && ks < 2 + PER) {
+                    if (fetch) patch_load(xl * PER + ks - 2, chunk + ahead);
+                }
+                if constexpr (xl >= 4 && ks == 2) {
+                    if (fetch) patch_store(xl - 4, raww);
                 }
                 if constexpr (DB && ks == 6) {       // the next chunk's transform: a column per position, then the products
                     if (more) {
