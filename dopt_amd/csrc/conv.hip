@@ -1308,32 +1308,65 @@ __device__ __forceinline__ void conv_wgrad_patch_body(const WgradPatch &p, const
     typedef __attribute__((address_space(3))) float lds_float_t;
     // Fetching runs one chunk ahead and also past the end of this block's range: those loads are
     // range-checked and their data lands in the LDS buffer that is not read again.
-    for (int chunk = cb; chunk < ce; ++chunk) {
-        const float *A = A0 + cur * (BM * APITCH) + a_frag;
+    // The fragments of a step are read one step ahead (the first step's after the barrier that releases the chunk), so
+    // that their LDS latency passes under the previous step's matrix instructions - with twelve wavefronts; fifteen have
+    // 128 registers each and no room for a second set.
+    constexpr bool AHEAD = WM * WC == 4;
+    struct Frag {
+        float4 a_lo, a_hi, q[4];
+        float e[4];
+    };
+    auto read_frag = [&](int buf, int s_) {
+        Frag f;
+        const float *A = A0 + buf * (BM * APITCH) + a_frag;
         // float4 indexing keeps the 16-byte alignment of the patch reads visible to the compiler
-        const float4 *B = (const float4 *)B0 + cur * (bsize / 4);
+        const float4 *bq = (const float4 *)B0 + buf * (bsize / 4) + b_frag[s_];
+        // The edge-column reads are volatile so that the compiler does not fuse a whole window
+        // into one run starting at the unaligned edge (it would then read it in 2-dword pieces).
+        const volatile lds_float_t *be = (const volatile lds_float_t *)bq;
+        f.a_lo = *(const float4 *)(A + s_ * 16);
+        f.a_hi = *(const float4 *)(A + s_ * 16 + 4);
+        if constexpr (kGeo == 0) {
+            f.q[0] = bq[0]; f.q[1] = bq[1];
+            f.e[0] = be[-1]; f.e[1] = be[8];
+        } else if constexpr (kGeo == 1) {
+            f.q[0] = bq[0]; f.q[1] = bq[3];   // the next patch row is 12 floats on
+            f.e[0] = be[-1]; f.e[1] = be[4]; f.e[2] = be[11]; f.e[3] = be[16];
+        } else {
+            // (image, row) quads: image 0 rows 0, 1 then image 1 rows 0, 1
+            f.q[0] = bq[0]; f.q[1] = bq[1]; f.q[2] = bq[4]; f.q[3] = bq[5];
+        }
+        return f;
+    };
+    Frag nxt;
+    if constexpr (AHEAD) nxt = read_frag(0, 0);
+    for (int chunk = cb; chunk < ce; ++chunk) {
         static_for<0, 4>([&](auto stag) {
             constexpr int s = decltype(stag)::value;
             if constexpr (s == 0) fetch();
-            const float4 a_lo = *(const float4 *)(A + s * 16), a_hi = *(const float4 *)(A + s * 16 + 4);
-            const float a8[8] = {a_lo.x, a_lo.y, a_lo.z, a_lo.w, a_hi.x, a_hi.y, a_hi.z, a_hi.w};
-            const float4 *bq = B + b_frag[s];
-            // The edge-column reads are volatile so that the compiler does not fuse a whole window
-            // into one run starting at the unaligned edge (it would then read it in 2-dword pieces).
-            const volatile lds_float_t *be = (const volatile lds_float_t *)bq;
+            Frag f;
+            if constexpr (AHEAD) {
+                f = nxt;
+                if constexpr (s < 3) {
+                    nxt = read_frag(cur, s + 1);
+                    __builtin_amdgcn_sched_barrier(0);   // issued here, not where they are first used
+                }
+            } else {
+                f = read_frag(cur, s);
+            }
+            const float a8[8] = {f.a_lo.x, f.a_lo.y, f.a_lo.z, f.a_lo.w, f.a_hi.x, f.a_hi.y, f.a_hi.z, f.a_hi.w};
             if constexpr (kGeo == 0) {
-                const float4 b_lo = bq[0], b_hi = bq[1];
-                const float e_lo = be[-1], e_hi = be[8];
-                const float win[10] = {e_lo, b_lo.x, b_lo.y, b_lo.z, b_lo.w, b_hi.x, b_hi.y, b_hi.z, b_hi.w, e_hi};
+                const float4 b_lo = f.q[0], b_hi = f.q[1];
+                const float win[10] = {f.e[0], b_lo.x, b_lo.y, b_lo.z, b_lo.w, b_hi.x, b_hi.y, b_hi.z, b_hi.w, f.e[1]};
 #pragma unroll
                 for (int ks = 0; ks < 8; ks++)
 #pragma unroll
                     for (int ds = 0; ds < 3; ds++)
                         acc[ds] = __builtin_amdgcn_mfma_f32_32x32x2f32(a8[ks], win[ks + ds], acc[ds], 0, 0, 0);
             } else if constexpr (kGeo == 1) {
-                const float4 r0 = bq[0], r1 = bq[3];  // the next patch row is 12 floats on
-                const float w0[6] = {be[-1], r0.x, r0.y, r0.z, r0.w, be[4]};
-                const float w1[6] = {be[11], r1.x, r1.y, r1.z, r1.w, be[16]};
+                const float4 r0 = f.q[0], r1 = f.q[1];
+                const float w0[6] = {f.e[0], r0.x, r0.y, r0.z, r0.w, f.e[1]};
+                const float w1[6] = {f.e[2], r1.x, r1.y, r1.z, r1.w, f.e[3]};
 #pragma unroll
                 for (int ks = 0; ks < 8; ks++)
 #pragma unroll
@@ -1341,9 +1374,8 @@ __device__ __forceinline__ void conv_wgrad_patch_body(const WgradPatch &p, const
                         acc[ds] = __builtin_amdgcn_mfma_f32_32x32x2f32(a8[ks], ks < 4 ? w0[ks + ds] : w1[ks - 4 + ds],
                                                                        acc[ds], 0, 0, 0);
             } else {
-                // (image, row) quads: image 0 rows 0, 1 then image 1 rows 0, 1; pixel (row, col) of tap
-                // column ds reads element col + ds of the quad of patch row row + dr
-                const float4 q00 = bq[0], q01 = bq[1], q10 = bq[4], q11 = bq[5];
+                // pixel (row, col) of tap column ds reads element col + ds of the quad of patch row row + dr
+                const float4 q00 = f.q[0], q01 = f.q[1], q10 = f.q[2], q11 = f.q[3];
                 const float win[4][4] = {{q00.x, q00.y, q00.z, q00.w}, {q01.x, q01.y, q01.z, q01.w},
                                          {q10.x, q10.y, q10.z, q10.w}, {q11.x, q11.y, q11.z, q11.w}};
 #pragma unroll
@@ -1356,6 +1388,7 @@ __device__ __forceinline__ void conv_wgrad_patch_body(const WgradPatch &p, const
         });
         __syncthreads();
         cur ^= 1;
+        if constexpr (AHEAD) nxt = read_frag(cur, 0);   // (past the last chunk: the buffer the final, unused prefetch was stored to)
     }
 
     // Epilogue: the accumulators leave through LDS so that every output row -- the BC*9 values
