@@ -687,7 +687,7 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
 
     // ---- inverse transform.  This wavefront's rows of the 4x4 grid are i = 2 wi, 2 wi + 1; acc[4 il + j] = M[i][j].
     // At = [1 1 1 0; 0 1 -1 -1]:  z[i][0] = m0 + m1 + m2, z[i][1] = m1 - m2 - m3, then the same over i.
-    float *const xchg = lds;          // [wk][value 0..63][lane]: the main loop's LDS is free now
+    float *const xchg = lds;          // [wavefront pair][accumulator row][lane][4]: the main loop's LDS is free now
     float *outp = p.out + (size_t)split * p.out_elems;
     const bool add_bias = p.bias != nullptr && p.splits == 1;
     float part[16][4];                // per accumulator row v: this wavefront's share of y[a][b], index 2 a + b
@@ -701,11 +701,10 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
             part[v][0] = za0; part[v][1] = za1; part[v][2] = -za0 - zb0; part[v][3] = -za1 - zb1;
         }
     }
-    if (wi == 1) {
+    if (wi == 1) {   // a lane's four shares of one accumulator row are one 128-bit store
 #pragma unroll
         for (int v = 0; v < 16; v++)
-#pragma unroll
-            for (int q = 0; q < 4; q++) xchg[((w >> 1) * 64 + v * 4 + q) * 64 + lane] = part[v][q];
+            *(float4 *)(xchg + (((w >> 1) * 16 + v) * 64 + lane) * 4) = make_float4(part[v][0], part[v][1], part[v][2], part[v][3]);
     }
     __syncthreads();
     if (wi == 1) return;
@@ -719,11 +718,11 @@ __global__ __launch_bounds__(512, 1) void conv_wino_k(PatchConv p)
             const int m = m0 + wk * 32 + acc_row(v, lane);
             if (m >= p.Mout) continue;
             const float bias = add_bias ? p.bias[m] : 0.0f;
-            float y[4];
+            const float4 other = *(const float4 *)(xchg + (((w >> 1) * 16 + v) * 64 + lane) * 4);
+            float y[4] = {part[v][0] + other.x, part[v][1] + other.y, part[v][2] + other.z, part[v][3] + other.w};
+            if (add_bias) {
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
-                y[q] = part[v][q] + xchg[((w >> 1) * 64 + v * 4 + q) * 64 + lane];
-                if (add_bias) y[q] += bias;
+                for (int q = 0; q < 4; q++) y[q] += bias;
             }
             float *o = base + (size_t)m * OHW;
             *(float2 *)o = make_float2(y[0], y[1]);
