@@ -312,6 +312,15 @@ def main():
                         return int(line.split()[-1])
             return None
 
+        def profile_kernel_avg(name):
+            """Average duration (us) of a kernel in the committed rocprofv3 kernel-stats summary: NOT measured in this run."""
+            spath = os.path.join(ROOT, "profiles", "vgg16_b128_train_step_kernel_stats.txt")
+            if os.path.exists(spath):
+                for line in open(spath):
+                    if line.startswith(name + " "):
+                        return float(line[len(name):].split()[2])
+            return None
+
         # The dominant kernel, by its share of the step: conv_wino_k<16, 4, 1>, the Winograd F(2x2, 3x3) convolution on
         # 128-row tiles that runs the forward pass of layers 3-10 and the backward-data pass of layers 4-10 (15 launches
         # per step; the 64-row instantiation of layers 2-3 is not part of this figure).  Timed by events
@@ -339,7 +348,11 @@ def main():
             "flops_convention": "2*N*K*C*R*S*P*Q per launch, the direct algorithm's count; the kernel's matrix instructions "
                                 "execute 16/36 of it (sixteen products per 2x2 outputs instead of thirty-six)",
             "avg_launch_us": round(pus.value / pl.value, 2) if pl.value else None,
-            "timing": "HIP events around each launch on the library's stream, %d steps" % nsteps,
+            "timing": "HIP events around each launch on the library's stream, %d steps; an event pair also sees the "
+                      "boundary to the kernel in front (3-4 us), which the profiler's kernel durations do not" % nsteps,
+            "profile_avg_launch_us": profile_kernel_avg("conv_wino_k<16, 4, 1>"),
+            "profile_source": "profiles/vgg16_b128_train_step_kernel_stats.txt (rocprofv3 --kernel-trace --stats of this "
+                              "command; taken from that file, not measured in this run)",
         }
 
         # The forward convolutions of layers 3-10 on their own (8 launches per step, the Winograd kernel): their steps

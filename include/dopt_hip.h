@@ -286,7 +286,9 @@ int dopt_hip_conv_bwd_data(const dopt_hip_conv_desc *d, const float *dy, const f
    dopt_hip_conv_packed_bytes: size of the packed copy for the forward (bwd_data = 0) or the
    backward-data (1) direction, or 0 when that convolution does not take one (the caller then uses
    the unpacked entry points).  A packed copy depends on the descriptor, the direction and the
-   device, and is valid until the filter changes. */
+   device, and is valid until the filter changes.  Layers that run the Winograd F(2x2, 3x3) kernel (pad 1, even
+   image sides of 4 and more, whole 16-channel chunks and at least 64 reduction channels, rows in whole 128s or
+   in 64s padded by at most a fifth) get the transformed filter G g Gt as their packed copy, 16/9 the size. */
 size_t dopt_hip_conv_packed_bytes(const dopt_hip_conv_desc *d, int bwd_data);
 /* Which layout that packed copy has, or -1 when there is none: two packed copies of the same filter
    under the same descriptor and with equal layout ids are identical, so a caller needs only one.
@@ -329,10 +331,12 @@ int dopt_hip_conv_bwd_data_packed_open(const dopt_hip_conv_desc *d, const float 
 /* Backward-data (on a packed filter, as dopt_hip_conv_bwd_data_packed_open; open may be null) and filter gradient
    (as dopt_hip_conv_bwd_filter) of one convolution in one call: cudnnConvolutionBackwardData (cudnn7.d:195) and
    cudnnConvolutionBackwardFilter (cudnn7.d:244) read the same dy and nothing of each other.  For 3x3 unit-stride
-   layers of at least 128 input and output channels on rows of 8 .. 64 pixels or 4 x 4 images both run as ONE
-   launch, the filter-gradient tiles starting on each compute unit as its backward-data tile ends; every other
-   shape runs the two entry points one after the other.  dx and dw are bit for bit what those write.
-   open_dw (may be null): where the one launch leaves the filter gradient as partial copies (it always splits its
+   layers of at least 128 input and output channels on rows of 8 .. 64 pixels or 4 x 4 images whose backward-data is
+   not a Winograd layer both run as ONE launch, the filter-gradient tiles starting on each compute unit as its
+   backward-data tile ends; every other shape runs the two entry points one after the other (a Winograd
+   backward-data on 128-row tiles and its filter gradient out of one workspace request, so that both can stay
+   open).  dx and dw are bit for bit what the two entry points write.
+   open_dw (may be null): where the filter gradient is left as partial copies (the one launch always splits its
    pixels over the compute units), the pass that adds them is skipped and the copies are described there, to be
    closed by the next call like an open dx: dopt_hip_split_sum_close, or dopt_hip_bn_grad_side, whose launch adds
    them on compute units the batch norm leaves idle.  Both open and open_dw may be pending at once. */
