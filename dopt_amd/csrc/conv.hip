@@ -451,23 +451,27 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 256) void conv_patch_k(Pat
 // arithmetic.
 //
 // A workgroup owns 128 rows x 32 tiles (the 128 pixels of the direct kernel's column tile: whole image rows or whole
-// images, so the input under them is the same rectangle, staged by the same loader, position-major with its zero halo).
-// Per 16-channel chunk: the raw patch goes to LDS; all 512 threads transform it - thread (i, tile, four channels)
-// forms row i of Bt d B for its tile from eight 128-bit reads and writes the four transformed values, four channels
-// each, to V[xi][tile][16 channels]; then wavefront (wk, wi) multiplies rows 32 wk .. + 31 with the eight positions
-// xi = 8 wi .. 8 wi + 7: per position two 128-bit reads of V (this lane's tile, its eight channels) and two 128-bit
-// loads of the transformed filter U[chunk][xi][row][16 channels] straight into operand registers, three positions
-// ahead, feed eight matrix instructions into the position's own accumulator (128 accumulator registers per
-// wavefront, two wavefronts per SIMD).
+// images, so the input under them is the same rectangle with the same zero halo) or 64 rows x 64 tiles.
+// Per 16-channel chunk: the raw patch goes to LDS position-major (a thread owns one position and stores its channels
+// as 128-bit pieces); all 512 threads transform it - thread (i, tile, four channels) forms row i of Bt d B for its tile
+// from eight 128-bit reads and writes the four transformed values, four channels each, to V[xi][tile][16 channels];
+// wavefront (wk, wi) multiplies rows 32 wk .. + 31 with the eight positions xi = 8 wi .. 8 wi + 7: per position two
+// 128-bit reads of V (this lane's tile, its eight channels; one position ahead) and two 128-bit loads of the
+// transformed filter U[chunk][xi][row][16 channels] straight into operand registers, three positions ahead, feed
+// eight matrix instructions into the position's own accumulator (128 accumulator registers per wavefront, two
+// wavefronts per SIMD).  With 32 tiles, patch and V are double-buffered and the next chunk's transform runs under
+// this chunk's matrix instructions; every piece of side work is pinned to a matrix step (sched_barrier), or the
+// scheduler sinks the prefetches to their first use.
 //
 // At the end a lane holds M[xi][row][tile] for its eight positions - two rows i of the 4x4 grid, complete in j - so it
 // applies A along j in registers (z[i][b]), combines its two rows into its share of the four outputs, and the
 // wavefronts of a pair add their shares through LDS: y[a][b] = (At z)[a][b].  Output, split reductions and bias are
 // those of the direct kernel.
 //
-// What bounds it: the transformed filter is 16/9 the size of the packed one and a workgroup streams 128 KB of it per
-// chunk for 2.1 MFLOP - the rate at which a CU's L1 fills from the L2 (about 35 GB/s) and the matrix cores are
-// about equally busy.  128 rows x 64 tiles would halve that traffic and need 256 accumulator registers per wavefront.
+// What bounds it: a chunk is 3.4 us of matrix time per workgroup and takes 4.65 - the filter loads (128 KB per chunk
+// and workgroup, 16/9 the direct kernel's), the V reads, the patch and the transform each add their share, roughly in
+// proportion to their instruction counts (loops without one of them: -0.5, -0.2, -0.3, -0.4 us).  128 rows x 64 tiles
+// would halve filter traffic and fragment loads per matrix instruction and need 256 accumulator registers per wavefront.
 constexpr int kWinoXchg = 4 * 64 * 64;   // floats of the exchange area: four wavefront pairs x 64 values per lane
 
 // WK x TH: the eight wavefronts are WK groups of 32 rows x TH groups of 32 tiles x the two halves of the 16 positions:
