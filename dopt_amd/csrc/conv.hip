@@ -468,7 +468,8 @@ __global__ __launch_bounds__(T::THREADS, T::THREADS / 256) void conv_patch_k(Pat
 // wavefronts of a pair add their shares through LDS: y[a][b] = (At z)[a][b].  Output, split reductions and bias are
 // those of the direct kernel.
 //
-// What bounds it: a chunk is 3.4 us of matrix time per workgroup and takes 4.65 - the filter loads (128 KB per chunk
+// What bounds it: a chunk is 3.4 us of matrix time per workgroup at the nominal rate, 3.95 in a build of this loop with
+// nothing but its matrix instructions, and takes 4.6 .. 5.0 - the filter loads (128 KB per chunk
 // and workgroup, 16/9 the direct kernel's), the V reads, the patch and the transform each add their share, roughly in
 // proportion to their instruction counts (loops without one of them: -0.5, -0.2, -0.3, -0.4 us).  128 rows x 64 tiles
 // would halve filter traffic and fragment loads per matrix instruction and need 256 accumulator registers per wavefront.
