@@ -406,6 +406,10 @@ CONV_CASES = [  # N, C, H, W, K, R, S, pad, stride
     (7, 64, 8, 8, 192, 3, 3, (1, 1), (1, 1)),
     (3, 192, 16, 16, 320, 3, 3, (1, 1), (1, 1)),
     (3, 160, 16, 16, 160, 3, 3, (1, 1), (1, 1)),   # 160 rows as three 64-row tiles, the last half empty
+    (1, 80, 4, 4, 128, 3, 3, (1, 1), (1, 1)),      # one image in a tile of eight; five chunks (an odd count through two buffers)
+    (5, 64, 8, 4, 128, 3, 3, (1, 1), (1, 1)),      # rows of four pixels, four images per tile
+    (1, 64, 64, 64, 64, 3, 3, (1, 1), (1, 1)),     # 64-row tiles on rows of 64 pixels
+    (2, 112, 16, 32, 128, 3, 3, (1, 1), (1, 1)),   # seven chunks, rows of 32 pixels
     (2, 80, 8, 12, 128, 3, 3, (1, 1), (1, 1)),     # 12 columns: no whole tile rows in 128 pixels, the direct kernels
     (2, 7, 11, 13, 9, 5, 5, (2, 2), (3, 3)),      # nine classes with work in one launch
     (1, 4, 9, 9, 5, 5, 5, (2, 2), (4, 4)),        # sixteen classes: one after the other
